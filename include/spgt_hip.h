@@ -1,0 +1,101 @@
+/* C ABI of libspgt_hip.so: the gfx950 (MI355X) kernels behind SpGT's operator API.
+ *
+ * Conventions
+ *   - every pointer is a device pointer to fp32 data unless stated otherwise;
+ *     complex64 tensors are passed as float pairs (re, im);
+ *   - the caller owns all memory: outputs and workspaces are passed in, the
+ *     library allocates nothing and keeps no state between calls;
+ *   - kernels are enqueued on `stream` (0 = the null stream) of the current
+ *     device and the call returns without synchronising;
+ *   - the return value is SPGT_OK or a negative SPGT_ERR_* code, in which case
+ *     nothing was launched and spgt_last_error() describes the problem;
+ *   - `*_workspace_bytes` functions return the scratch size the matching call
+ *     needs for the same shape arguments (0 for invalid shapes).
+ *
+ * Each entry point names the interface of the reference (Bloonow/SpGT) that a
+ * binding would replace with it.
+ */
+#ifndef SPGT_HIP_H
+#define SPGT_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct ihipStream_t* spgt_stream_t; /* == hipStream_t */
+
+enum {
+    SPGT_OK = 0,
+    SPGT_ERR_INVALID_ARGUMENT = -1,
+    SPGT_ERR_WORKSPACE = -2,
+    SPGT_ERR_LAUNCH = -3
+};
+
+/* Operand orders of the reference's batched GEMMs (extension/utils/gemm_utils.cu:3-12):
+ * letter k of the name is the storage order (R row-major, C column-major) of A, B, C. */
+enum {
+    SPGT_ORDER_RRR = 0, SPGT_ORDER_RRC = 1, SPGT_ORDER_RCR = 2, SPGT_ORDER_RCC = 3,
+    SPGT_ORDER_CRR = 4, SPGT_ORDER_CRC = 5, SPGT_ORDER_CCR = 6, SPGT_ORDER_CCC = 7
+};
+
+/* Library version as major*10000 + minor*100 + patch. */
+int spgt_version(void);
+
+/* Message of the last failed call on the calling thread ("" if none). */
+const char* spgt_last_error(void);
+
+/* ---- Galerkin attention ------------------------------------------------ */
+
+/* Replaces multihead_galerkin_attention_cccr_forward
+ * (extension/bind/galerkin_attention.cu:104-124).
+ *   Q, K, V : [batch, num_head, d_posk, seqlen]  (feature-major, seqlen contiguous)
+ *   out     : [batch, num_head, seqlen, d_posk]
+ *   out[b,h,s,j] = sum_i Q[b,h,i,s] * ( sum_t K[b,h,i,t] V[b,h,j,t] / seqlen )
+ * d_posk must be 32 or 34.  The seqlen reduction is split over workgroups and
+ * finished by a fixed-order second stage, so results are run-to-run identical. */
+size_t spgt_galerkin_attention_cccr_workspace_bytes(int batch, int num_head, int d_posk, int seqlen);
+int spgt_galerkin_attention_cccr_forward(const float* Q, const float* K, const float* V, float* out,
+                                         void* workspace, size_t workspace_bytes, int batch,
+                                         int num_head, int d_posk, int seqlen, spgt_stream_t stream);
+
+/* Replaces batched_skinny_gemm (extension/bind/galerkin_attention.cu:175-198) and the
+ * launcher under it, sgemm_32x32_4x8_SplitK::sgemm_cuda
+ * (extension/native/sgemm_32x32_splitk.cu:662-705):
+ *   C[b] = alpha * A[b] * B[b],  A: M x K, B: K x N, C: M x N, small M, N and long K,
+ * with batch strides a_stride, b_stride, c_stride (in floats) and any of the eight
+ * operand orders.  Two-stage deterministic split-K. */
+size_t spgt_batched_skinny_gemm_workspace_bytes(int M, int N, int K, int batch_count);
+int spgt_batched_skinny_gemm(const float* A, const float* B, float* C, float alpha, int M, int N,
+                             int K, int64_t a_stride, int64_t b_stride, int64_t c_stride, int order,
+                             int batch_count, void* workspace, size_t workspace_bytes,
+                             spgt_stream_t stream);
+
+/* One-call fused attention core on token-major operands.  No single reference
+ * function corresponds to it: it computes what Sp_GalerkinAttention.forward
+ * (network/sp_layer.py:64-72) obtains from the LayerNorm epilogue of
+ * multihead_projection_layernorm_with_position_rrc_forward followed by
+ * multihead_galerkin_attention_cccr_forward, i.e. GalerkinAttention's
+ * layer_norm + concat + matmuls (network/layer.py:130-152), starting from the
+ * plain projections x@W+b.
+ *   Q, K, V  : [B, S, H*32] with row stride ld_in floats (>= H*32, multiple of 4)
+ *   position : [B, S, 2] (dp == 2) or NULL (dp == 0)
+ *   ln_*     : [H, 32] LayerNorm affine of K and of V; eps as in F.layer_norm
+ *   out      : [B, S, H*(dp+32)]  (per head: dp position channels, then 32 features)
+ *   ktv      : [B, H, dp+32, dp+32] row-major, receives K'^T V' / S */
+size_t spgt_galerkin_attention_fused_workspace_bytes(int B, int S, int H, int dp);
+int spgt_galerkin_attention_fused_forward(const float* Q, const float* K, const float* V,
+                                          int64_t ld_in, const float* position,
+                                          const float* ln_weight_K, const float* ln_bias_K,
+                                          const float* ln_weight_V, const float* ln_bias_V,
+                                          float norm_eps, float* out, float* ktv, void* workspace,
+                                          size_t workspace_bytes, int B, int S, int H, int dp,
+                                          spgt_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* SPGT_HIP_H */

@@ -1,0 +1,93 @@
+"""ctypes binding of libspgt_hip.so (the C ABI declared in include/spgt_hip.h).
+
+There is no fallback: if the library has not been built, or a call is made
+with tensors that do not live on a GPU, an exception is raised.
+"""
+import ctypes
+import os
+import threading
+
+import torch
+
+PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(PKG_DIR, "libspgt_hip.so")
+
+_c_float_p = ctypes.c_void_p  # device pointers travel as integers
+_i = ctypes.c_int
+_i64 = ctypes.c_int64
+_sz = ctypes.c_size_t
+_f = ctypes.c_float
+_p = ctypes.c_void_p
+
+# name -> (restype, argtypes); must list every function of include/spgt_hip.h
+SIGNATURES = {
+    "spgt_version": (_i, []),
+    "spgt_last_error": (ctypes.c_char_p, []),
+    "spgt_galerkin_attention_cccr_workspace_bytes": (_sz, [_i, _i, _i, _i]),
+    "spgt_galerkin_attention_cccr_forward": (_i, [_p, _p, _p, _p, _p, _sz, _i, _i, _i, _i, _p]),
+    "spgt_batched_skinny_gemm_workspace_bytes": (_sz, [_i, _i, _i, _i]),
+    "spgt_batched_skinny_gemm": (_i, [_p, _p, _p, _f, _i, _i, _i, _i64, _i64, _i64, _i, _i, _p, _sz, _p]),
+    "spgt_galerkin_attention_fused_workspace_bytes": (_sz, [_i, _i, _i, _i]),
+    "spgt_galerkin_attention_fused_forward": (
+        _i, [_p, _p, _p, _i64, _p, _p, _p, _p, _p, _f, _p, _p, _p, _sz, _i, _i, _i, _i, _p]),
+}
+
+_lock = threading.Lock()
+_lib = None
+
+
+class SpgtError(RuntimeError):
+    """A libspgt_hip.so entry point rejected its arguments or failed to launch."""
+
+
+def load():
+    """Returns the loaded library, loading it on first use."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is None:
+            if not os.path.exists(LIB_PATH):
+                raise SpgtError(
+                    f"{LIB_PATH} is missing: build it with `python -m spgt_amd.build` "
+                    "(there is no non-HIP implementation of these operators)")
+            lib = ctypes.CDLL(LIB_PATH)
+            for name, (restype, argtypes) in SIGNATURES.items():
+                fn = getattr(lib, name)
+                fn.restype = restype
+                fn.argtypes = argtypes
+            _lib = lib
+    return _lib
+
+
+def last_error() -> str:
+    return load().spgt_last_error().decode("utf-8", "replace")
+
+
+def check(rc: int) -> None:
+    if rc != 0:
+        raise SpgtError(f"libspgt_hip error {rc}: {last_error()}")
+
+
+def require_gpu_f32(name: str, t: torch.Tensor, dtype=torch.float32) -> None:
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name} must be a torch.Tensor")
+    if not t.is_cuda:
+        raise SpgtError(f"{name} must live on a GPU (got device {t.device}); there is no CPU implementation")
+    if t.dtype != dtype:
+        raise TypeError(f"{name} must have dtype {dtype} (got {t.dtype})")
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")
+
+
+def ptr(t: torch.Tensor):
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def stream_of(t: torch.Tensor):
+    return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def workspace(nbytes: int, like: torch.Tensor) -> torch.Tensor:
+    """Scratch from torch's caching allocator on `like`'s device (at least 16 bytes)."""
+    return torch.empty(max(int(nbytes), 16), dtype=torch.uint8, device=like.device)

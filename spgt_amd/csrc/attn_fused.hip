@@ -1,0 +1,453 @@
+// Fused softmax-free Galerkin attention core on token-major operands.
+//
+//   Q, K, V : [B, S, H*32] fp32 (rows may be strided: one x@[Wq|Wk|Wv] GEMM
+//             output serves all three), optional position [B, S, 2]
+//   out     : [B, S, H*(dp+32)]
+//
+// Semantics follow the reference's plain PyTorch path
+// (network/layer.py:114-152): K and V are LayerNorm'ed per token and per head
+// over the 32 head features (biased variance, eps inside the square root,
+// per-head affine), the position channels are prepended to every head, then
+// M = K'^T V' / S and out = Q' M.
+//
+// Three launches:
+//   1. ktv_ln_partial_tm  - one pass over K and V: LayerNorm in registers
+//      (16 lanes share a token, DPP row reductions), partial d x d tiles
+//      accumulated on the fp32 matrix cores, one tile per (chunk, head).
+//   2. tile_reduce        - deterministic fixed-order sum of the partial tiles,
+//      scaled by 1/S.
+//   3. qm_apply_tm        - streams Q once, keeps the head's d x d matrix in
+//      registers as the MFMA A operand, writes out once.
+#include "spgt_device.h"
+#include "spgt_host.h"
+
+namespace spgt {
+
+namespace {
+
+template <int DP>
+struct KtvUnit {
+    float2 k, v, p;
+};
+
+// LayerNorm of the two features this lane holds; the other 30 features of the
+// token live in the other 15 lanes of the DPP row.
+__device__ __forceinline__ float2 ln_pair(float2 x, float g0, float g1, float b0, float b1, float eps) {
+    const float mean = row16_allsum(x.x + x.y) * (1.0f / 32.0f);
+    const float d0 = x.x - mean;
+    const float d1 = x.y - mean;
+    const float ss = row16_allsum(fmaf(d1, d1, d0 * d0));
+    const float rstd = rsqrtf(fmaf(ss, 1.0f / 32.0f, eps));
+    float2 y;
+    y.x = fmaf(d0 * rstd, g0, b0);
+    y.y = fmaf(d1 * rstd, g1, b1);
+    return y;
+}
+
+}  // namespace
+
+// grid (nchunk, H/4, B), block 256: wave w handles head 4*blockIdx.y + w.
+// Lane l of a wave: token slot t = l/16, feature pair p = l%16 (features 2p, 2p+1).
+template <int DP, int U>
+__global__ __launch_bounds__(256) void ktv_ln_partial_tm(
+    const float* __restrict__ K, const float* __restrict__ V, const float* __restrict__ pos,
+    const float* __restrict__ lnwK, const float* __restrict__ lnbK,
+    const float* __restrict__ lnwV, const float* __restrict__ lnbV, float eps,
+    float* __restrict__ partial, int S, int H, int64_t ld, int tokens_per_chunk) {
+    constexpr int D = DP + 32;
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int h = blockIdx.y * 4 + wave;
+    const int b = blockIdx.z;
+    const int chunk = blockIdx.x;
+    const int nchunk = gridDim.x;
+    const int t = lane >> 4;
+    const int p = lane & 15;
+
+    const int s0 = chunk * tokens_per_chunk;
+    const int s1 = min(S, s0 + tokens_per_chunk);
+
+    const int f = h * 32 + 2 * p;
+    const float gK0 = lnwK[f], gK1 = lnwK[f + 1], bK0 = lnbK[f], bK1 = lnbK[f + 1];
+    const float gV0 = lnwV[f], gV1 = lnwV[f + 1], bV0 = lnbV[f], bV1 = lnbV[f + 1];
+
+    const float* kbase = K + (int64_t)b * S * ld + f;
+    const float* vbase = V + (int64_t)b * S * ld + f;
+    const float* pbase = pos + (int64_t)b * S * 2;
+
+    v4f acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
+    float kp[2][2] = {{0.f, 0.f}, {0.f, 0.f}};  // sum yK[ta] * pos[a]
+    float pv[2][2] = {{0.f, 0.f}, {0.f, 0.f}};  // sum pos[a] * yV[tb]
+    float pp[3] = {0.f, 0.f, 0.f};              // sum p0p0, p0p1, p1p1
+
+    auto load_unit = [&](int s) {
+        KtvUnit<DP> u;
+        u.k = *reinterpret_cast<const float2*>(kbase + (int64_t)s * ld);
+        u.v = *reinterpret_cast<const float2*>(vbase + (int64_t)s * ld);
+        if (DP == 2) u.p = *reinterpret_cast<const float2*>(pbase + (int64_t)s * 2);
+        return u;
+    };
+    auto compute_unit = [&](const KtvUnit<DP>& u, bool valid) {
+        float2 yk = ln_pair(u.k, gK0, gK1, bK0, bK1, eps);
+        const float2 yv = ln_pair(u.v, gV0, gV1, bV0, bV1, eps);
+        float2 pz = u.p;
+        if (!valid) {
+            yk.x = 0.f;
+            yk.y = 0.f;
+            if (DP == 2) { pz.x = 0.f; pz.y = 0.f; }
+        }
+        acc[0][0] = mfma16(yk.x, yv.x, acc[0][0]);
+        acc[0][1] = mfma16(yk.x, yv.y, acc[0][1]);
+        acc[1][0] = mfma16(yk.y, yv.x, acc[1][0]);
+        acc[1][1] = mfma16(yk.y, yv.y, acc[1][1]);
+        if (DP == 2) {
+            kp[0][0] = fmaf(yk.x, u.p.x, kp[0][0]);
+            kp[0][1] = fmaf(yk.x, u.p.y, kp[0][1]);
+            kp[1][0] = fmaf(yk.y, u.p.x, kp[1][0]);
+            kp[1][1] = fmaf(yk.y, u.p.y, kp[1][1]);
+            pv[0][0] = fmaf(pz.x, yv.x, pv[0][0]);
+            pv[0][1] = fmaf(pz.x, yv.y, pv[0][1]);
+            pv[1][0] = fmaf(pz.y, yv.x, pv[1][0]);
+            pv[1][1] = fmaf(pz.y, yv.y, pv[1][1]);
+            pp[0] = fmaf(pz.x, pz.x, pp[0]);
+            pp[1] = fmaf(pz.x, pz.y, pp[1]);
+            pp[2] = fmaf(pz.y, pz.y, pp[2]);
+        }
+    };
+
+    constexpr int G = 4 * U;  // tokens per unrolled group
+    const int ngroups = (s1 - s0) / G;
+    if (ngroups > 0) {
+        KtvUnit<DP> cur[U], nxt[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) cur[u] = load_unit(s0 + 4 * u + t);
+        for (int g = 0; g < ngroups; ++g) {
+            if (g + 1 < ngroups) {
+                const int sn = s0 + (g + 1) * G + t;
+#pragma unroll
+                for (int u = 0; u < U; ++u) nxt[u] = load_unit(sn + 4 * u);
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) compute_unit(cur[u], true);
+#pragma unroll
+            for (int u = 0; u < U; ++u) cur[u] = nxt[u];
+        }
+    }
+    // Ragged tail of the chunk (< G tokens): clamp the address, mask the value.
+    for (int s = s0 + ngroups * G; s < s1; s += 4) {
+        const bool valid = (s + t) < s1;
+        const KtvUnit<DP> u = load_unit(valid ? s + t : s1 - 1);
+        compute_unit(u, valid);
+    }
+
+    // acc[ta][tb][r] = M[2*(4t+r)+ta][2p+tb]
+    float* tile = partial + (((int64_t)b * H + h) * nchunk + chunk) * (D * D);
+#pragma unroll
+    for (int ta = 0; ta < 2; ++ta)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int i = DP + 8 * t + 2 * r + ta;
+            float2 o;
+            o.x = acc[ta][0][r];
+            o.y = acc[ta][1][r];
+            *reinterpret_cast<float2*>(tile + i * D + DP + 2 * p) = o;
+        }
+    if (DP == 2) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                kp[i][j] = rows4_allsum(kp[i][j]);
+                pv[i][j] = rows4_allsum(pv[i][j]);
+            }
+#pragma unroll
+        for (int i = 0; i < 3; ++i) pp[i] = rows4_allsum(pp[i]);
+        if (t == 0) {
+#pragma unroll
+            for (int ta = 0; ta < 2; ++ta) {
+                float2 o;
+                o.x = kp[ta][0];
+                o.y = kp[ta][1];
+                *reinterpret_cast<float2*>(tile + (DP + 2 * p + ta) * D) = o;
+            }
+#pragma unroll
+            for (int a = 0; a < 2; ++a) {
+                float2 o;
+                o.x = pv[a][0];
+                o.y = pv[a][1];
+                *reinterpret_cast<float2*>(tile + a * D + DP + 2 * p) = o;
+            }
+            if (p == 0) {
+                tile[0] = pp[0];
+                tile[1] = pp[1];
+                tile[D] = pp[1];
+                tile[D + 1] = pp[2];
+            }
+        }
+    }
+}
+
+// out[bh][e] = scale * sum_c partial[bh][c][e], summed in a fixed order:
+// four interleaved chains (c = q, q+4, ...) combined as ((c0+c1)+(c2+c3)).
+// grid (ceil(E/256), BH), block 256 = 64 element-quads x 4 chains.
+__global__ __launch_bounds__(256) void tile_reduce(
+    const float* __restrict__ partial, float* __restrict__ out, int E, int nchunk, float scale) {
+    __shared__ float4 sm[4][64];
+    const int q = threadIdx.x >> 6;
+    const int e4 = threadIdx.x & 63;
+    const int e = (blockIdx.x * 64 + e4) * 4;
+    const int64_t bh = blockIdx.y;
+    float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (e < E) {
+        const float* src = partial + bh * nchunk * (int64_t)E + e;
+#pragma unroll 8
+        for (int c = q; c < nchunk; c += 4) {
+            const float4 v = *reinterpret_cast<const float4*>(src + (int64_t)c * E);
+            s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+        }
+    }
+    sm[q][e4] = s;
+    __syncthreads();
+    if (q == 0 && e < E) {
+        const float4 a = sm[0][e4], b2 = sm[1][e4], c2 = sm[2][e4], d2 = sm[3][e4];
+        float4 r;
+        r.x = ((a.x + b2.x) + (c2.x + d2.x)) * scale;
+        r.y = ((a.y + b2.y) + (c2.y + d2.y)) * scale;
+        r.z = ((a.z + b2.z) + (c2.z + d2.z)) * scale;
+        r.w = ((a.w + b2.w) + (c2.w + d2.w)) * scale;
+        *reinterpret_cast<float4*>(out + bh * E + e) = r;
+    }
+}
+
+// grid (nchunk, H/4, B), block 256: wave w handles head 4*blockIdx.y + w.
+// Lane l: token slot tk = l%16, feature group g = l/16; the lane loads
+// Q[s][4g..4g+3] and Q[s][16+4g..16+4g+3] of its token.  MFMA step kk contracts
+// the four features {i(kk, g) : g = 0..3}, i(kk,g) = 4g+kk (kk<4) or 16+4g+kk-4.
+template <int DP, int U>
+__global__ __launch_bounds__(256) void qm_apply_tm(
+    const float* __restrict__ Q, const float* __restrict__ pos, const float* __restrict__ M,
+    float* __restrict__ out, int S, int H, int64_t ld, int tokens_per_chunk) {
+    constexpr int D = DP + 32;
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int h = blockIdx.y * 4 + wave;
+    const int b = blockIdx.z;
+    const int tk = lane & 15;
+    const int g = lane >> 4;
+    const int s0 = blockIdx.x * tokens_per_chunk;
+    const int s1 = min(S, s0 + tokens_per_chunk);
+    const int64_t ldo = (int64_t)H * D;
+
+    const float* m = M + ((int64_t)b * H + h) * (D * D);
+    float mreg[8][2];
+#pragma unroll
+    for (int kk = 0; kk < 8; ++kk) {
+        const int i = (kk < 4) ? (4 * g + kk) : (16 + 4 * g + kk - 4);
+#pragma unroll
+        for (int jb = 0; jb < 2; ++jb) mreg[kk][jb] = m[(DP + i) * D + DP + jb * 16 + tk];
+    }
+    // DP == 2 only: rows 0,1 of M for this lane's output features, and
+    // columns 0,1 of M for this lane's input features.
+    float mrow[2][2][4];
+    float mcol[8][2];
+    float mpp[2][2];
+    if (DP == 2) {
+#pragma unroll
+        for (int a = 0; a < 2; ++a)
+#pragma unroll
+            for (int jb = 0; jb < 2; ++jb)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) mrow[a][jb][r] = m[a * D + DP + jb * 16 + 4 * g + r];
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk) {
+            const int i = (kk < 4) ? (4 * g + kk) : (16 + 4 * g + kk - 4);
+            mcol[kk][0] = m[(DP + i) * D + 0];
+            mcol[kk][1] = m[(DP + i) * D + 1];
+        }
+        mpp[0][0] = m[0]; mpp[0][1] = m[1]; mpp[1][0] = m[D]; mpp[1][1] = m[D + 1];
+    }
+
+    const float* qbase = Q + (int64_t)b * S * ld + h * 32 + 4 * g;
+    const float* pbase = pos + (int64_t)b * S * 2;
+    float* obase = out + (int64_t)b * S * ldo + h * D;
+
+    struct Unit { float4 q0, q1; float2 p; };
+    auto load_unit = [&](int s) {
+        Unit u;
+        const float* qp = qbase + (int64_t)s * ld;
+        u.q0 = *reinterpret_cast<const float4*>(qp);
+        u.q1 = *reinterpret_cast<const float4*>(qp + 16);
+        if (DP == 2) u.p = *reinterpret_cast<const float2*>(pbase + (int64_t)s * 2);
+        return u;
+    };
+    auto compute_unit = [&](const Unit& u, int s, bool valid) {
+        const float q[8] = {u.q0.x, u.q0.y, u.q0.z, u.q0.w, u.q1.x, u.q1.y, u.q1.z, u.q1.w};
+        v4f acc[2];
+#pragma unroll
+        for (int jb = 0; jb < 2; ++jb) {
+            if (DP == 2) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    acc[jb][r] = fmaf(u.p.y, mrow[1][jb][r], u.p.x * mrow[0][jb][r]);
+            } else {
+                acc[jb] = v4f{0.f, 0.f, 0.f, 0.f};
+            }
+        }
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk) {
+            acc[0] = mfma16(mreg[kk][0], q[kk], acc[0]);
+            acc[1] = mfma16(mreg[kk][1], q[kk], acc[1]);
+        }
+        float* op = obase + (int64_t)s * ldo;
+        if (DP == 2) {
+            float c0 = 0.f, c1 = 0.f;
+#pragma unroll
+            for (int kk = 0; kk < 8; ++kk) {
+                c0 = fmaf(q[kk], mcol[kk][0], c0);
+                c1 = fmaf(q[kk], mcol[kk][1], c1);
+            }
+            c0 = rows4_allsum(c0);
+            c1 = rows4_allsum(c1);
+            if (valid) {
+                if (g == 0) {
+                    float2 o;
+                    o.x = fmaf(u.p.y, mpp[1][0], fmaf(u.p.x, mpp[0][0], c0));
+                    o.y = fmaf(u.p.y, mpp[1][1], fmaf(u.p.x, mpp[0][1], c1));
+                    *reinterpret_cast<float2*>(op) = o;
+                }
+#pragma unroll
+                for (int jb = 0; jb < 2; ++jb) {
+                    float* o = op + DP + jb * 16 + 4 * g;
+                    *reinterpret_cast<float2*>(o) = make_float2(acc[jb][0], acc[jb][1]);
+                    *reinterpret_cast<float2*>(o + 2) = make_float2(acc[jb][2], acc[jb][3]);
+                }
+            }
+        } else if (valid) {
+#pragma unroll
+            for (int jb = 0; jb < 2; ++jb)
+                *reinterpret_cast<float4*>(op + jb * 16 + 4 * g) =
+                    make_float4(acc[jb][0], acc[jb][1], acc[jb][2], acc[jb][3]);
+        }
+    };
+
+    constexpr int G = 16 * U;
+    const int ngroups = (s1 - s0) / G;
+    if (ngroups > 0) {
+        Unit cur[U], nxt[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) cur[u] = load_unit(s0 + 16 * u + tk);
+        for (int gi = 0; gi < ngroups; ++gi) {
+            const int sc = s0 + gi * G + tk;
+            if (gi + 1 < ngroups) {
+#pragma unroll
+                for (int u = 0; u < U; ++u) nxt[u] = load_unit(sc + G + 16 * u);
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) compute_unit(cur[u], sc + 16 * u, true);
+#pragma unroll
+            for (int u = 0; u < U; ++u) cur[u] = nxt[u];
+        }
+    }
+    for (int s = s0 + ngroups * G; s < s1; s += 16) {
+        const bool valid = (s + tk) < s1;
+        const int sl = valid ? s + tk : s1 - 1;
+        const Unit u = load_unit(sl);
+        compute_unit(u, sl, valid);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------
+
+namespace {
+
+struct FusedPlan {
+    int tpc1, nchunk1;  // K^T V pass
+    int tpc2, nchunk2;  // Q M pass
+};
+
+constexpr int kU1 = 4;  // 16 tokens per unrolled group in pass 1
+constexpr int kU2 = 2;  // 32 tokens per unrolled group in pass 2
+
+FusedPlan make_plan(int B, int S, int H) {
+    // Aim at ~4 resident workgroups per CU (256 CUs); chunks are whole
+    // unrolled groups so that only the last chunk of a batch has a ragged tail.
+    const int target_wg = 1024;
+    const int per_bh = std::max(1, target_wg / std::max(1, B * (H / 4)));
+    FusedPlan p;
+    const int g1 = 4 * kU1, g2 = 16 * kU2;
+    p.tpc1 = std::max(g1, ceil_div(ceil_div(S, per_bh), g1) * g1);
+    p.nchunk1 = ceil_div(S, p.tpc1);
+    p.tpc2 = std::max(g2, ceil_div(ceil_div(S, per_bh), g2) * g2);
+    p.nchunk2 = ceil_div(S, p.tpc2);
+    return p;
+}
+
+}  // namespace
+
+}  // namespace spgt
+
+using namespace spgt;
+
+extern "C" size_t spgt_galerkin_attention_fused_workspace_bytes(int B, int S, int H, int dp) {
+    if (B <= 0 || S <= 0 || H <= 0 || (dp != 0 && dp != 2)) return 0;
+    const FusedPlan p = make_plan(B, S, H);
+    const size_t D = dp + 32;
+    return (size_t)B * H * p.nchunk1 * D * D * sizeof(float);
+}
+
+extern "C" int spgt_galerkin_attention_fused_forward(
+    const float* Q, const float* K, const float* V, int64_t ld_in, const float* position,
+    const float* ln_weight_K, const float* ln_bias_K, const float* ln_weight_V,
+    const float* ln_bias_V, float norm_eps, float* out, float* ktv, void* workspace,
+    size_t workspace_bytes, int B, int S, int H, int dp, hipStream_t stream) {
+    if (!Q || !K || !V || !out || !ktv || !ln_weight_K || !ln_bias_K || !ln_weight_V || !ln_bias_V)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "galerkin_attention_fused: null pointer argument");
+    if (B <= 0 || S <= 0 || H <= 0)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "galerkin_attention_fused: B, S, H must be positive");
+    if (H % 4 != 0)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "galerkin_attention_fused: num_head must be a multiple of 4");
+    if (dp != 0 && dp != 2)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "galerkin_attention_fused: dim_position must be 0 or 2");
+    if (dp == 2 && !position)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "galerkin_attention_fused: position is null with dim_position 2");
+    if (ld_in < (int64_t)H * 32 || (ld_in % 4) != 0)
+        return fail(SPGT_ERR_INVALID_ARGUMENT,
+                    "galerkin_attention_fused: row stride must be >= H*32 and a multiple of 4 floats");
+    if (!aligned16(Q) || !aligned16(K) || !aligned16(V) || !aligned16(out) || !aligned16(ktv) ||
+        (position && !aligned8(position)))
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "galerkin_attention_fused: operands must be 16-byte aligned");
+    if (B > 65535 || H / 4 > 65535)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "galerkin_attention_fused: batch or head count exceeds the grid limit");
+    const size_t need = spgt_galerkin_attention_fused_workspace_bytes(B, S, H, dp);
+    if (!workspace || workspace_bytes < need || !aligned16(workspace))
+        return fail(SPGT_ERR_WORKSPACE, "galerkin_attention_fused: workspace missing, misaligned or too small");
+
+    const FusedPlan p = make_plan(B, S, H);
+    const int D = dp + 32;
+    float* partial = static_cast<float*>(workspace);
+    const dim3 block(256);
+    const dim3 grid1(p.nchunk1, H / 4, B);
+    const dim3 grid2(p.nchunk2, H / 4, B);
+    const dim3 gridr(ceil_div(D * D, 256), B * H);
+    const float* pos = position ? position : Q;  // never dereferenced when dp == 0
+    if (dp == 0) {
+        hipLaunchKernelGGL((ktv_ln_partial_tm<0, kU1>), grid1, block, 0, stream, K, V, pos, ln_weight_K,
+                           ln_bias_K, ln_weight_V, ln_bias_V, norm_eps, partial, S, H, ld_in, p.tpc1);
+    } else {
+        hipLaunchKernelGGL((ktv_ln_partial_tm<2, kU1>), grid1, block, 0, stream, K, V, pos, ln_weight_K,
+                           ln_bias_K, ln_weight_V, ln_bias_V, norm_eps, partial, S, H, ld_in, p.tpc1);
+    }
+    hipLaunchKernelGGL(tile_reduce, gridr, block, 0, stream, partial, ktv, D * D, p.nchunk1, 1.0f / (float)S);
+    if (dp == 0) {
+        hipLaunchKernelGGL((qm_apply_tm<0, kU2>), grid2, block, 0, stream, Q, pos, ktv, out, S, H, ld_in, p.tpc2);
+    } else {
+        hipLaunchKernelGGL((qm_apply_tm<2, kU2>), grid2, block, 0, stream, Q, pos, ktv, out, S, H, ld_in, p.tpc2);
+    }
+    return check_launch("galerkin_attention_fused");
+}

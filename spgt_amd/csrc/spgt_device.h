@@ -1,0 +1,72 @@
+// Device-side helpers shared by the gfx950 kernels of this library.
+//
+// Everything here assumes wave64 (CDNA) and is only ever compiled for gfx950.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace spgt {
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+// 4-byte aligned vector views: rows of a [d, S] tensor with odd S start at
+// arbitrary 4-byte offsets, and the hardware handles unaligned dwordx2/x4
+// global accesses, so the compiler is told only what is true.
+struct __attribute__((packed, aligned(4))) f2u { float x, y; };
+struct __attribute__((packed, aligned(4))) f4u { float x, y, z, w; };
+
+// DPP controls (a DPP row = 16 consecutive lanes).
+#define SPGT_DPP_QUAD_XOR1 0xB1         // quad_perm:[1,0,3,2]
+#define SPGT_DPP_QUAD_XOR2 0x4E         // quad_perm:[2,3,0,1]
+#define SPGT_DPP_ROW_HALF_MIRROR 0x141  // lane i <-> 7-i inside each 8 lanes
+#define SPGT_DPP_ROW_MIRROR 0x140       // lane i <-> 15-i inside each 16 lanes
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+    return __builtin_bit_cast(
+        float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+
+// Sum over the 16 lanes of a DPP row; every lane of the row receives the same
+// bit pattern (each step adds a value to its mirror image, and fp add commutes).
+__device__ __forceinline__ float row16_allsum(float v) {
+    v += dpp_move<SPGT_DPP_QUAD_XOR1>(v);
+    v += dpp_move<SPGT_DPP_QUAD_XOR2>(v);
+    v += dpp_move<SPGT_DPP_ROW_HALF_MIRROR>(v);
+    v += dpp_move<SPGT_DPP_ROW_MIRROR>(v);
+    return v;
+}
+
+// Sum over groups of 8 consecutive lanes (same guarantee as above).
+__device__ __forceinline__ float row8_allsum(float v) {
+    v += dpp_move<SPGT_DPP_QUAD_XOR1>(v);
+    v += dpp_move<SPGT_DPP_QUAD_XOR2>(v);
+    v += dpp_move<SPGT_DPP_ROW_HALF_MIRROR>(v);
+    return v;
+}
+
+// Sum of one value over the four 16-lane rows of a wave (lanes l, l^16, l^32, l^48).
+__device__ __forceinline__ float rows4_allsum(float v) {
+    v += __shfl_xor(v, 16, 64);
+    v += __shfl_xor(v, 32, 64);
+    return v;
+}
+
+// D(16x16) += A(16x4) * B(4x16), fp32.
+//   lane l supplies A[l%16][l/16] and B[l/16][l%16];
+//   lane l, element r of the result holds D[4*(l/16)+r][l%16].
+__device__ __forceinline__ v4f mfma16(float a, float b, v4f c) {
+    return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
+}
+
+// D(32x32) += A(32x2) * B(2x32), fp32.
+//   lane l supplies A[l%32][l/32] and B[l/32][l%32];
+//   lane l, element r holds D[8*(r/4) + 4*(l/32) + r%4][l%32].
+__device__ __forceinline__ v16f mfma32(float a, float b, v16f c) {
+    return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
+}
+
+__host__ __device__ __forceinline__ int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+}  // namespace spgt

@@ -1,0 +1,29 @@
+// Error state and version of the C ABI.
+#include "spgt_host.h"
+
+#include <stdio.h>
+#include <string.h>
+
+namespace spgt {
+
+namespace {
+thread_local char g_last_error[512] = "";
+}
+
+int fail(int code, const char* msg) {
+    snprintf(g_last_error, sizeof(g_last_error), "%s", msg);
+    return code;
+}
+
+int check_launch(const char* what) {
+    const hipError_t e = hipGetLastError();
+    if (e == hipSuccess) return SPGT_OK;
+    snprintf(g_last_error, sizeof(g_last_error), "%s: kernel launch failed: %s", what, hipGetErrorString(e));
+    return SPGT_ERR_LAUNCH;
+}
+
+}  // namespace spgt
+
+extern "C" int spgt_version(void) { return 100; }
+
+extern "C" const char* spgt_last_error(void) { return spgt::g_last_error; }

@@ -1,0 +1,23 @@
+// Host-side helpers of the C ABI: error reporting and argument checks.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <algorithm>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "../../include/spgt_hip.h"
+
+namespace spgt {
+
+// Records `msg` as the calling thread's last error and returns `code`.
+int fail(int code, const char* msg);
+
+// Returns SPGT_OK, or SPGT_ERR_LAUNCH (with the HIP error string recorded) if
+// a kernel launch issued by `what` since the last check was rejected.
+int check_launch(const char* what);
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+inline bool aligned8(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 7u) == 0; }
+inline bool aligned4(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 3u) == 0; }
+
+}  // namespace spgt

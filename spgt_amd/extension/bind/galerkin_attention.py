@@ -1,0 +1,159 @@
+"""Operator API of the Galerkin attention path, backed by libspgt_hip.so.
+
+Same function names, argument order and result layouts as the reference's
+extension/bind/galerkin_attention.py:87-107 (python surface) and
+extension/bind/galerkin_attention.cu:200-226 (the `gexts` module surface).
+Tensors must be fp32, contiguous and on a GPU; anything else raises.
+"""
+from types import SimpleNamespace
+from typing import Any
+
+import torch
+from torch import Tensor
+
+from ... import _lib
+from ..._lib import check, ptr, require_gpu_f32, stream_of, workspace
+
+GEMM_ORDER = {"RRR": 0, "RRC": 1, "RCR": 2, "RCC": 3, "CRR": 4, "CRC": 5, "CCR": 6, "CCC": 7}
+
+
+# --------------------------------------------------------------------------- #
+# `gexts` surface: plain functions on tensors, no autograd
+# --------------------------------------------------------------------------- #
+
+def _attention_cccr_forward(Q: Tensor, K: Tensor, V: Tensor, batch: int, num_head: int, d_posk: int,
+                            seqlen: int) -> Tensor:
+    """Q, K, V [batch, num_head, d_posk, seqlen] -> [batch, num_head, seqlen, d_posk]
+    (reference: extension/bind/galerkin_attention.cu:104-124)."""
+    for name, t in (("Q", Q), ("K", K), ("V", V)):
+        require_gpu_f32(name, t)
+        if tuple(t.shape) != (batch, num_head, d_posk, seqlen):
+            raise ValueError(f"{name} has shape {tuple(t.shape)}, expected {(batch, num_head, d_posk, seqlen)}")
+    lib = _lib.load()
+    out = torch.empty((batch, num_head, seqlen, d_posk), dtype=Q.dtype, device=Q.device)
+    nbytes = lib.spgt_galerkin_attention_cccr_workspace_bytes(batch, num_head, d_posk, seqlen)
+    if nbytes == 0:
+        raise ValueError(f"unsupported attention shape: batch={batch} num_head={num_head} d_posk={d_posk} "
+                         f"seqlen={seqlen} (d_posk must be 32 or 34)")
+    ws = workspace(nbytes, Q)
+    with torch.cuda.device(Q.device):
+        check(lib.spgt_galerkin_attention_cccr_forward(
+            ptr(Q), ptr(K), ptr(V), ptr(out), ptr(ws), ws.numel(), batch, num_head, d_posk, seqlen, stream_of(Q)))
+    return out
+
+
+def _batched_skinny_gemm(A: Tensor, B: Tensor, alpha: float) -> Tensor:
+    """A [..., M, K] @ B [..., K, N] * alpha, all row-major
+    (reference: extension/bind/galerkin_attention.cu:175-198)."""
+    require_gpu_f32("A", A)
+    require_gpu_f32("B", B)
+    if A.dim() < 2 or A.dim() != B.dim() or A.shape[:-2] != B.shape[:-2] or A.shape[-1] != B.shape[-2]:
+        raise ValueError(f"incompatible shapes {tuple(A.shape)} and {tuple(B.shape)}")
+    M, K = A.shape[-2], A.shape[-1]
+    N = B.shape[-1]
+    lead = tuple(A.shape[:-2])
+    batch = 1
+    for n in lead:
+        batch *= n
+    C = torch.empty(lead + (M, N), dtype=A.dtype, device=A.device)
+    if batch == 0 or M == 0 or N == 0:
+        return C
+    if K == 0:
+        return C.zero_()
+    lib = _lib.load()
+    ws = workspace(lib.spgt_batched_skinny_gemm_workspace_bytes(M, N, K, batch), A)
+    with torch.cuda.device(A.device):
+        check(lib.spgt_batched_skinny_gemm(
+            ptr(A), ptr(B), ptr(C), float(alpha), M, N, K, M * K, K * N, M * N, GEMM_ORDER["RRR"], batch,
+            ptr(ws), ws.numel(), stream_of(A)))
+    return C
+
+
+def _attention_fused_forward(QKV_or_Q, K, V, position, ln_weight_K, ln_bias_K, ln_weight_V, ln_bias_V,
+                             norm_eps: float, num_head: int, dim_position: int, return_ktv: bool = False):
+    """Token-major fused attention core (no reference counterpart as one call).
+
+    Either pass Q, K, V as three [B, S, H*32] tensors (contiguous, or equal-stride
+    column slices of one [B, S, 3*H*32] projection output), position [B, S, dp].
+    Returns out [B, S, H*(dp+32)] (and K'^T V'/S [B, H, d, d] if return_ktv).
+    """
+    Q = QKV_or_Q
+    H = num_head
+    for name, t in (("Q", Q), ("K", K), ("V", V)):
+        if not t.is_cuda:
+            raise _lib.SpgtError(f"{name} must live on a GPU; there is no CPU implementation")
+        if t.dtype != torch.float32:
+            raise TypeError(f"{name} must be float32")
+        if t.dim() != 3 or t.shape[-1] != H * 32 or t.stride(-1) != 1:
+            raise ValueError(f"{name} must be [B, S, {H * 32}] with unit stride on the last axis")
+    B, S, _ = Q.shape
+    ld = Q.stride(1)
+    for name, t in (("Q", Q), ("K", K), ("V", V)):
+        if tuple(t.shape) != (B, S, H * 32) or t.stride(1) != ld or (B > 1 and t.stride(0) != S * ld):
+            raise ValueError(f"{name}: all of Q, K, V must share shape and strides [S*ld, ld, 1]")
+    for name, t in (("ln_weight_K", ln_weight_K), ("ln_bias_K", ln_bias_K), ("ln_weight_V", ln_weight_V),
+                    ("ln_bias_V", ln_bias_V)):
+        require_gpu_f32(name, t)
+        if t.numel() != H * 32:
+            raise ValueError(f"{name} must have {H * 32} elements")
+    if dim_position not in (0, 2):
+        raise ValueError("dim_position must be 0 or 2")
+    if dim_position == 2:
+        require_gpu_f32("position", position)
+        if tuple(position.shape) != (B, S, 2):
+            raise ValueError(f"position must be [{B}, {S}, 2]")
+    D = dim_position + 32
+    lib = _lib.load()
+    out = torch.empty((B, S, H * D), dtype=torch.float32, device=Q.device)
+    ktv = torch.empty((B, H, D, D), dtype=torch.float32, device=Q.device)
+    ws = workspace(lib.spgt_galerkin_attention_fused_workspace_bytes(B, S, H, dim_position), Q)
+    pos_ptr = ptr(position) if dim_position == 2 else None
+    with torch.cuda.device(Q.device):
+        check(lib.spgt_galerkin_attention_fused_forward(
+            ptr(Q), ptr(K), ptr(V), ld, pos_ptr, ptr(ln_weight_K), ptr(ln_bias_K), ptr(ln_weight_V),
+            ptr(ln_bias_V), float(norm_eps), ptr(out), ptr(ktv), ptr(ws), ws.numel(), B, S, H, dim_position,
+            stream_of(Q)))
+    return (out, ktv) if return_ktv else out
+
+
+gexts = SimpleNamespace(
+    multihead_galerkin_attention_cccr_forward=_attention_cccr_forward,
+    batched_skinny_gemm=_batched_skinny_gemm,
+    galerkin_attention_fused_forward=_attention_fused_forward,
+)
+
+
+# --------------------------------------------------------------------------- #
+# python surface
+# --------------------------------------------------------------------------- #
+
+class Multihead_Galerkin_Attention_cccr_Function(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx: Any, Q: Tensor, K: Tensor, V: Tensor):
+        batch, num_head, d_posk, seqlen = Q.size()
+        Attn = gexts.multihead_galerkin_attention_cccr_forward(Q, K, V, batch, num_head, d_posk, seqlen)
+        ctx.save_for_backward(Q, K, V)
+        return Attn
+
+    @staticmethod
+    def backward(ctx: Any, grad_Attn):
+        raise NotImplementedError("backward of multihead_galerkin_attention_cccr_cuda is not built yet")
+
+
+def multihead_galerkin_attention_cccr_cuda(Q: Tensor, K: Tensor, V: Tensor) -> Tensor:
+    """Q, K, V [B, H, d, S] -> Q^T (K V^T / S) laid out [B, H, S, d]."""
+    return Multihead_Galerkin_Attention_cccr_Function.apply(Q, K, V)
+
+
+def batched_skinny_gemm(A: Tensor, B: Tensor, alpha: float = 1.0) -> Tensor:
+    return gexts.batched_skinny_gemm(A, B, alpha)
+
+
+def galerkin_attention_fused(Q: Tensor, K: Tensor, V: Tensor, position, ln_weight_K: Tensor, ln_bias_K: Tensor,
+                             ln_weight_V: Tensor, ln_bias_V: Tensor, norm_eps: float, num_head: int,
+                             dim_position: int, return_ktv: bool = False):
+    """LayerNorm(K), LayerNorm(V), K'^T V'/S and Q' (K'^T V'/S) in one call on
+    token-major projections (inference only: no autograd graph is recorded)."""
+    return gexts.galerkin_attention_fused_forward(
+        Q, K, V, position, ln_weight_K, ln_bias_K, ln_weight_V, ln_bias_V, norm_eps, num_head, dim_position,
+        return_ktv)

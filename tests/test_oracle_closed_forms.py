@@ -1,0 +1,196 @@
+"""Oracle functions against what the mathematics fixes: brute-force loops on
+tiny inputs, special cases with textbook answers, library identities."""
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import spgt_oracle as O
+
+
+def rnd(*shape, seed=0, dtype=torch.float64):
+    return torch.randn(*shape, generator=torch.Generator().manual_seed(seed), dtype=dtype)
+
+
+def test_attention_bruteforce():
+    B, H, S, d = 2, 2, 7, 5
+    Q, K, V = rnd(B, H, S, d, seed=1), rnd(B, H, S, d, seed=2), rnd(B, H, S, d, seed=3)
+    want = np.zeros((B, H, S, d))
+    q, k, v = Q.numpy(), K.numpy(), V.numpy()
+    for b in range(B):
+        for h in range(H):
+            M = np.zeros((d, d))
+            for s in range(S):
+                for i in range(d):
+                    for j in range(d):
+                        M[i, j] += k[b, h, s, i] * v[b, h, s, j]
+            M /= S
+            for s in range(S):
+                for j in range(d):
+                    want[b, h, s, j] = sum(q[b, h, s, i] * M[i, j] for i in range(d))
+    np.testing.assert_allclose(O.galerkin_attention(Q, K, V).numpy(), want, rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(
+        O.op_attention_cccr(Q.transpose(-2, -1).contiguous(), K.transpose(-2, -1).contiguous(),
+                            V.transpose(-2, -1).contiguous()).numpy(), want, rtol=1e-12, atol=1e-12)
+
+
+def test_attention_special_cases():
+    S, d = 64, 32
+    # orthonormal columns: K = V with K^T K = I  =>  out = Q / S
+    Kq, _ = torch.linalg.qr(rnd(S, d, seed=4))
+    Q = rnd(1, 1, S, d, seed=5)
+    K = Kq[None, None]
+    torch.testing.assert_close(O.galerkin_attention(Q, K, K), Q / S, rtol=1e-10, atol=1e-12)
+    # all ones: K^T V / S is all ones, every output equals d
+    ones = torch.ones(1, 1, S, d, dtype=torch.float64)
+    assert torch.equal(O.galerkin_attention(ones, ones, ones), torch.full((1, 1, S, d), float(d), dtype=torch.float64))
+    # not symmetric in K and V: a transposed operand must show
+    Kr, Vr = rnd(1, 1, S, d, seed=6), rnd(1, 1, S, d, seed=7)
+    assert not torch.allclose(O.galerkin_attention(Q, Kr, Vr), O.galerkin_attention(Q, Vr, Kr))
+
+
+def test_projection_layout_and_invariants():
+    B, S, H, dh, dp = 2, 5, 4, 32, 2
+    x, pos = rnd(B, S, H * dh, seed=8), rnd(B, S, dp, seed=9)
+    W, b = rnd(H * dh, H * dh, seed=10), rnd(H * dh, seed=11)
+    y = O.project_heads(x, W, b, pos, H, dh)
+    assert y.shape == (B, H, S, dp + dh)
+    for h in range(H):
+        assert torch.equal(y[:, h, :, :dp], pos)  # position first, copied bit-exactly
+    # brute force one entry: feature j of head h is column h*dh+j of x W^T + b
+    bb, hh, ss, jj = 1, 2, 3, 7
+    want = sum(x[bb, ss, k] * W[hh * dh + jj, k] for k in range(H * dh)) + b[hh * dh + jj]
+    assert abs(y[bb, hh, ss, dp + jj] - want) < 1e-10
+    # identity weights: features are x itself
+    eye = torch.eye(H * dh, dtype=torch.float64)
+    y = O.project_heads(x, eye, torch.zeros(H * dh, dtype=torch.float64), pos, H, dh)
+    assert torch.equal(y[:, 1, :, dp:], x[:, :, dh:2 * dh])
+    # operator-level: x @ W (no transpose), feature-major
+    z = O.op_projection_rrc(x, W, b, pos, H, dh)
+    assert z.shape == (B, H, dp + dh, S)
+    want = sum(x[bb, ss, k] * W[k, hh * dh + jj] for k in range(H * dh)) + b[hh * dh + jj]
+    assert abs(z[bb, hh, dp + jj, ss] - want) < 1e-10
+
+
+def test_layernorm_closed_form():
+    B, S, H, dh = 2, 6, 4, 32
+    x = rnd(B, S, H * dh, seed=12)
+    eye = torch.eye(H * dh, dtype=torch.float64)
+    zero = torch.zeros(H * dh, dtype=torch.float64)
+    pos = torch.zeros(B, S, 0, dtype=torch.float64)
+    g, be = rnd(H, dh, seed=13), rnd(H, dh, seed=14)
+    eps = 1e-6
+    y = O.project_layernorm_heads(x, eye, zero, g, be, pos, eps, H, dh)
+    xh = x.reshape(B, S, H, dh).permute(0, 2, 1, 3)
+    mu = xh.mean(-1, keepdim=True)
+    var = ((xh - mu) ** 2).mean(-1, keepdim=True)  # biased
+    want = (xh - mu) / torch.sqrt(var + eps) * g[None, :, None, :] + be[None, :, None, :]
+    torch.testing.assert_close(y, want, rtol=1e-10, atol=1e-12)
+    # unit affine: mean 0, variance var/(var+eps)
+    y1 = O.project_layernorm_heads(x, eye, zero, torch.ones(H, dh, dtype=torch.float64),
+                                   torch.zeros(H, dh, dtype=torch.float64), pos, eps, H, dh)
+    assert y1.mean(-1).abs().max() < 1e-12
+    torch.testing.assert_close((y1 ** 2).mean(-1, keepdim=True), var / (var + eps), rtol=1e-9, atol=1e-12)
+    # constant rows: output is the bias (rstd finite thanks to eps)
+    yc = O.project_layernorm_heads(torch.full_like(x, 3.0), eye, zero, g, be, pos, eps, H, dh)
+    torch.testing.assert_close(yc, be[None, :, None, :].expand(B, H, S, dh), rtol=0, atol=1e-9)
+    # operator-level invsigma
+    _, inv = O.op_projection_layernorm_rrc(x, eye, zero, g, be, pos, eps, H, dh)
+    torch.testing.assert_close(inv, 1 / torch.sqrt(var[..., 0] + eps), rtol=1e-10, atol=0)
+
+
+def test_complex_mode_product_bruteforce():
+    N, I, Oc, h, w = 2, 3, 4, 2, 3
+    x, wt = rnd(N, I, h, w, 2, seed=15), rnd(I, Oc, h, w, 2, seed=16)
+    xc, wc = torch.view_as_complex(x), torch.view_as_complex(wt)
+    want = torch.zeros(N, Oc, h, w, dtype=torch.complex128)
+    for n in range(N):
+        for o in range(Oc):
+            for a in range(h):
+                for b in range(w):
+                    want[n, o, a, b] = sum(xc[n, i, a, b] * wc[i, o, a, b] for i in range(I))
+    got = torch.view_as_complex(O.complex_mode_product(x, wt).contiguous())
+    torch.testing.assert_close(got, want, rtol=1e-12, atol=1e-12)
+
+
+def test_spectral_identity_weights():
+    N, r, C = 1, 8, 3
+    x = rnd(N, r, r, C, seed=17)
+    zeros = {"residual_layer.weight": torch.zeros(C, C, dtype=torch.float64),
+             "residual_layer.bias": torch.zeros(C, dtype=torch.float64)}
+    # identity per mode and m covering the whole half spectrum: irfft2(rfft2(x)) = x
+    m = r // 2 + 1  # rows [:m] and [r-m:] overlap and together cover all r rows
+    wid = torch.zeros(C, C, m, m, 2, dtype=torch.float64)
+    for c in range(C):
+        wid[c, c, :, :, 0] = 1.0
+    p = dict(zeros, **{"fourier_weight.0": wid, "fourier_weight.1": wid})
+    y = O.spectral_conv2d(p, x, m, "relu")
+    torch.testing.assert_close(y, F.relu(x), rtol=1e-10, atol=1e-12)
+    # small m: a low-pass filter = zero all other modes by hand
+    m = 2
+    p = dict(zeros, **{"fourier_weight.0": wid[:, :, :m, :m].contiguous(),
+                       "fourier_weight.1": wid[:, :, :m, :m].contiguous()})
+    xf = torch.fft.rfft2(x.permute(0, 3, 1, 2), norm="ortho")
+    mask = torch.zeros_like(xf)
+    mask[..., :m, :m] = 1
+    mask[..., r - m:, :m] = 1
+    want = torch.fft.irfft2(xf * mask, s=(r, r), norm="ortho").permute(0, 2, 3, 1)
+    torch.testing.assert_close(O.spectral_conv2d(p, x, m, "relu"), F.relu(want), rtol=1e-10, atol=1e-12)
+
+
+def test_bilinear_explicit_vs_library():
+    x = rnd(2, 3, 7, 9, seed=18)
+    for size in [(7, 9), (4, 5), (13, 17), (1, 1), (2, 3)]:
+        got = O.bilinear_align_corners(x, size)
+        want = F.interpolate(x, size=size, mode="bilinear", align_corners=True)
+        torch.testing.assert_close(got, want, rtol=1e-12, atol=1e-12)
+    # corners map exactly; affine images are reproduced
+    y = O.bilinear_align_corners(x, (13, 17))
+    assert torch.equal(y[..., 0, 0], x[..., 0, 0]) and torch.allclose(y[..., -1, -1], x[..., -1, -1])
+    ii, jj = torch.meshgrid(torch.linspace(0, 1, 7, dtype=torch.float64), torch.linspace(0, 1, 9, dtype=torch.float64),
+                            indexing="ij")
+    plane = (2 * ii - 3 * jj + 0.5)[None, None]
+    i2, j2 = torch.meshgrid(torch.linspace(0, 1, 5, dtype=torch.float64), torch.linspace(0, 1, 4, dtype=torch.float64),
+                            indexing="ij")
+    torch.testing.assert_close(O.bilinear_align_corners(plane, (5, 4))[0, 0], 2 * i2 - 3 * j2 + 0.5, rtol=1e-12,
+                               atol=1e-12)
+
+
+@pytest.mark.parametrize("r_large,r_small,r_mid", [
+    (211, 71, 122), (141, 71, 99), (421, 71, 172), (512, 256, 363), (256, 128, 181), (128, 64, 90), (64, 32, 44),
+    (32, 16, 22)])
+def test_resolution_sizes_known_answers(r_large, r_small, r_mid):
+    rs = O.resolution_sizes(r_large, r_small)
+    assert rs == ((r_large,) * 2, (r_mid,) * 2, (r_small,) * 2, (r_mid,) * 2, (r_large,) * 2)
+
+
+def test_datamove_ops():
+    x = rnd(2, 3, 4, 5, seed=19)
+    y = O.op_batched_transpose(x, [2], [3, 4], [5])
+    assert y.shape == (2, 5, 3, 4)
+    for b in range(2):
+        for i in range(3):
+            for j in range(4):
+                for c in range(5):
+                    assert y[b, c, i, j] == x[b, i, j, c]
+    src = torch.view_as_complex(rnd(2, 3, 6, 4, 2, seed=20))
+    g1, g2 = O.op_transpose_gather_dual(src, [2, 3], 6, 4, 2, 3, 0, 0, 4, 1)
+    assert g1.shape == (2, 3, 2, 3)
+    for hh in range(2):
+        for ww in range(3):
+            for n in range(2):
+                for c in range(3):
+                    assert g1[hh, ww, n, c] == src[n, c, hh, ww]
+                    assert g2[hh, ww, n, c] == src[n, c, 4 + hh, 1 + ww]
+    back = O.op_transpose_scatter_dual(g1, g2, [2, 3], 6, 4, 2, 3, 0, 0, 4, 1)
+    mask = torch.zeros(6, 4, dtype=torch.bool)
+    mask[0:2, 0:3] = True
+    mask[4:6, 1:4] = True
+    assert torch.equal(back[..., mask], src[..., mask])
+    assert (back[..., ~mask] == 0).all()
+
+
+def test_skinny_gemm_oracle():
+    A, B = rnd(3, 4, 50, seed=21), rnd(3, 50, 5, seed=22)
+    want = torch.einsum("bmk,bkn->bmn", A, B) * 0.25
+    torch.testing.assert_close(O.op_batched_skinny_gemm(A, B, 0.25), want, rtol=1e-12, atol=1e-12)
