@@ -21,6 +21,22 @@
 #include "spgt_device.h"
 #include "spgt_host.h"
 
+// Cache policy of the three touch-once streams (K/V reads, Q reads, out
+// writes).  Measured on MI355X at B=8, S=44521 over all eight combinations:
+// non-temporal K/V loads and out stores with plain Q loads is the fastest
+// (146 us per call against 174 us with plain accesses everywhere); the
+// non-temporal out stores keep 182 MB of dirty lines from draining under the
+// next call's K/V pass.
+#ifndef SPGT_NT_P1LD
+#define SPGT_NT_P1LD true
+#endif
+#ifndef SPGT_NT_P2LD
+#define SPGT_NT_P2LD false
+#endif
+#ifndef SPGT_NT_P2ST
+#define SPGT_NT_P2ST true
+#endif
+
 namespace spgt {
 
 namespace {
@@ -37,7 +53,7 @@ __device__ __forceinline__ float2 ln_pair(float2 x, float g0, float g1, float b0
     const float d0 = x.x - mean;
     const float d1 = x.y - mean;
     const float ss = row16_allsum(fmaf(d1, d1, d0 * d0));
-    const float rstd = rsqrtf(fmaf(ss, 1.0f / 32.0f, eps));
+    const float rstd = __builtin_amdgcn_rsqf(fmaf(ss, 1.0f / 32.0f, eps));  // v_rsq_f32, 1 ulp
     float2 y;
     y.x = fmaf(d0 * rstd, g0, b0);
     y.y = fmaf(d1 * rstd, g1, b1);
@@ -71,9 +87,12 @@ __global__ __launch_bounds__(256) void ktv_ln_partial_tm(
     const float gK0 = lnwK[f], gK1 = lnwK[f + 1], bK0 = lnbK[f], bK1 = lnbK[f + 1];
     const float gV0 = lnwV[f], gV1 = lnwV[f + 1], bV0 = lnbV[f], bV1 = lnbV[f + 1];
 
-    const float* kbase = K + (int64_t)b * S * ld + f;
-    const float* vbase = V + (int64_t)b * S * ld + f;
-    const float* pbase = pos + (int64_t)b * S * 2;
+    // Wave-uniform chunk bases; per-lane offsets stay 32-bit so that loads
+    // use the scalar-base + vector-offset addressing form.
+    const float* kchunk = K + ((int64_t)b * S + s0) * ld;
+    const float* vchunk = V + ((int64_t)b * S + s0) * ld;
+    const float* pchunk = pos + ((int64_t)b * S + s0) * 2;
+    const uint32_t uld = (uint32_t)ld;
 
     v4f acc[2][2];
 #pragma unroll
@@ -84,11 +103,14 @@ __global__ __launch_bounds__(256) void ktv_ln_partial_tm(
     float pv[2][2] = {{0.f, 0.f}, {0.f, 0.f}};  // sum pos[a] * yV[tb]
     float pp[3] = {0.f, 0.f, 0.f};              // sum p0p0, p0p1, p1p1
 
-    auto load_unit = [&](int s) {
+    // `rel` is the token index relative to the chunk start.
+    auto load_unit = [&](const float* kg, const float* vg, const float* pg, uint32_t rel) {
         KtvUnit<DP> u;
-        u.k = *reinterpret_cast<const float2*>(kbase + (int64_t)s * ld);
-        u.v = *reinterpret_cast<const float2*>(vbase + (int64_t)s * ld);
-        if (DP == 2) u.p = *reinterpret_cast<const float2*>(pbase + (int64_t)s * 2);
+        const uint32_t off = rel * uld + (uint32_t)f;
+        u.k = ld_stream<SPGT_NT_P1LD>(reinterpret_cast<const float2*>(kg + off));
+        u.v = ld_stream<SPGT_NT_P1LD>(reinterpret_cast<const float2*>(vg + off));
+        if (DP == 2) u.p = *reinterpret_cast<const float2*>(pg + rel * 2u);
+        else u.p = make_float2(0.f, 0.f);
         return u;
     };
     auto compute_unit = [&](const KtvUnit<DP>& u, bool valid) {
@@ -119,29 +141,48 @@ __global__ __launch_bounds__(256) void ktv_ln_partial_tm(
         }
     };
 
-    constexpr int G = 4 * U;  // tokens per unrolled group
-    const int ngroups = (s1 - s0) / G;
-    if (ngroups > 0) {
-        KtvUnit<DP> cur[U], nxt[U];
+    // Software pipeline over full groups of G = 4*U tokens with two register
+    // buffers (no buffer-to-buffer copies inside the loop: a copy of a value
+    // still in flight would force a wait for every outstanding load).  The
+    // ragged remainder of the chunk is one extra clamped and masked group.
+    constexpr int G = 4 * U;
+    const int len = s1 - s0;
+    const int nfull = len / G;
+    KtvUnit<DP> bufA[U], bufB[U];
+    auto load_group = [&](KtvUnit<DP>(&buf)[U], int g) {  // g is clamped to the full groups
+        const int64_t go = (int64_t)min(g, nfull - 1) * G;
+        const float* kg = kchunk + go * ld;
+        const float* vg = vchunk + go * ld;
+        const float* pg = pchunk + go * 2;
 #pragma unroll
-        for (int u = 0; u < U; ++u) cur[u] = load_unit(s0 + 4 * u + t);
-        for (int g = 0; g < ngroups; ++g) {
-            if (g + 1 < ngroups) {
-                const int sn = s0 + (g + 1) * G + t;
+        for (int u = 0; u < U; ++u) buf[u] = load_unit(kg, vg, pg, (uint32_t)(4 * u + t));
+    };
+    auto compute_full = [&](const KtvUnit<DP>(&buf)[U]) {
 #pragma unroll
-                for (int u = 0; u < U; ++u) nxt[u] = load_unit(sn + 4 * u);
-            }
-#pragma unroll
-            for (int u = 0; u < U; ++u) compute_unit(cur[u], true);
-#pragma unroll
-            for (int u = 0; u < U; ++u) cur[u] = nxt[u];
+        for (int u = 0; u < U; ++u) compute_unit(buf[u], true);
+    };
+    if (nfull > 0) {
+        load_group(bufA, 0);
+        int g = 0;
+        for (; g + 2 <= nfull; g += 2) {
+            load_group(bufB, g + 1);
+            __builtin_amdgcn_sched_barrier(0);  // keep the prefetch ahead of the arithmetic
+            compute_full(bufA);
+            __builtin_amdgcn_sched_barrier(0);
+            load_group(bufA, g + 2);
+            __builtin_amdgcn_sched_barrier(0);
+            compute_full(bufB);
+            __builtin_amdgcn_sched_barrier(0);
         }
+        if (g < nfull) compute_full(bufA);
     }
-    // Ragged tail of the chunk (< G tokens): clamp the address, mask the value.
-    for (int s = s0 + ngroups * G; s < s1; s += 4) {
-        const bool valid = (s + t) < s1;
-        const KtvUnit<DP> u = load_unit(valid ? s + t : s1 - 1);
-        compute_unit(u, valid);
+    if (nfull * G < len) {
+        const int rel0 = nfull * G + t;
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            bufA[u] = load_unit(kchunk, vchunk, pchunk, (uint32_t)min(rel0 + 4 * u, len - 1));
+#pragma unroll
+        for (int u = 0; u < U; ++u) compute_unit(bufA[u], (rel0 + 4 * u) < len);
     }
 
     // acc[ta][tb][r] = M[2*(4t+r)+ta][2p+tb]
@@ -279,8 +320,8 @@ __global__ __launch_bounds__(256) void qm_apply_tm(
     auto load_unit = [&](int s) {
         Unit u;
         const float* qp = qbase + (int64_t)s * ld;
-        u.q0 = *reinterpret_cast<const float4*>(qp);
-        u.q1 = *reinterpret_cast<const float4*>(qp + 16);
+        u.q0 = ld_stream<SPGT_NT_P2LD>(reinterpret_cast<const float4*>(qp));
+        u.q1 = ld_stream<SPGT_NT_P2LD>(reinterpret_cast<const float4*>(qp + 16));
         if (DP == 2) u.p = *reinterpret_cast<const float2*>(pbase + (int64_t)s * 2);
         return u;
     };
@@ -329,34 +370,53 @@ __global__ __launch_bounds__(256) void qm_apply_tm(
         } else if (valid) {
 #pragma unroll
             for (int jb = 0; jb < 2; ++jb)
-                *reinterpret_cast<float4*>(op + jb * 16 + 4 * g) =
-                    make_float4(acc[jb][0], acc[jb][1], acc[jb][2], acc[jb][3]);
+                st_stream<SPGT_NT_P2ST>(reinterpret_cast<float4*>(op + jb * 16 + 4 * g),
+                          make_float4(acc[jb][0], acc[jb][1], acc[jb][2], acc[jb][3]));
         }
     };
 
+    // Same two-buffer software pipeline as in ktv_ln_partial_tm.
     constexpr int G = 16 * U;
-    const int ngroups = (s1 - s0) / G;
-    if (ngroups > 0) {
-        Unit cur[U], nxt[U];
+    const int len = s1 - s0;
+    const int nfull = len / G;
+    const int ntot = (len + G - 1) / G;
+    Unit bufA[U], bufB[U];
+    auto load_group = [&](Unit(&buf)[U], int gi) {
+        const int sg = s0 + min(gi, ntot - 1) * G + tk;
 #pragma unroll
-        for (int u = 0; u < U; ++u) cur[u] = load_unit(s0 + 16 * u + tk);
-        for (int gi = 0; gi < ngroups; ++gi) {
-            const int sc = s0 + gi * G + tk;
-            if (gi + 1 < ngroups) {
+        for (int u = 0; u < U; ++u) buf[u] = load_unit(min(sg + 16 * u, s1 - 1));
+    };
+    auto compute_group = [&](const Unit(&buf)[U], int gi) {
+        const int sg = s0 + gi * G + tk;
 #pragma unroll
-                for (int u = 0; u < U; ++u) nxt[u] = load_unit(sc + G + 16 * u);
-            }
-#pragma unroll
-            for (int u = 0; u < U; ++u) compute_unit(cur[u], sc + 16 * u, true);
-#pragma unroll
-            for (int u = 0; u < U; ++u) cur[u] = nxt[u];
-        }
+        for (int u = 0; u < U; ++u) compute_unit(buf[u], sg + 16 * u, true);
+    };
+    load_group(bufA, 0);
+    int gi = 0;
+    for (; gi + 2 <= nfull; gi += 2) {
+        load_group(bufB, gi + 1);
+        __builtin_amdgcn_sched_barrier(0);  // keep the prefetch ahead of the arithmetic
+        compute_group(bufA, gi);
+        __builtin_amdgcn_sched_barrier(0);
+        load_group(bufA, gi + 2);
+        __builtin_amdgcn_sched_barrier(0);
+        compute_group(bufB, gi + 1);
+        __builtin_amdgcn_sched_barrier(0);
     }
-    for (int s = s0 + ngroups * G; s < s1; s += 16) {
-        const bool valid = (s + tk) < s1;
-        const int sl = valid ? s + tk : s1 - 1;
-        const Unit u = load_unit(sl);
-        compute_unit(u, sl, valid);
+    if (gi < nfull) {
+        load_group(bufB, gi + 1);
+        compute_group(bufA, gi);
+#pragma unroll
+        for (int u = 0; u < U; ++u) bufA[u] = bufB[u];
+        ++gi;
+    }
+    if (gi < ntot) {
+        const int sg = s0 + gi * G + tk;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int sl = sg + 16 * u;
+            compute_unit(bufA[u], min(sl, s1 - 1), sl < s1);
+        }
     }
 }
 

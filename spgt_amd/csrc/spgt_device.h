@@ -7,6 +7,7 @@
 
 namespace spgt {
 
+typedef float v2f __attribute__((ext_vector_type(2)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 
@@ -65,6 +66,38 @@ __device__ __forceinline__ v4f mfma16(float a, float b, v4f c) {
 //   lane l, element r holds D[8*(r/4) + 4*(l/32) + r%4][l%32].
 __device__ __forceinline__ v16f mfma32(float a, float b, v16f c) {
     return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
+}
+
+// Streaming (touch-once) global accesses: NT selects the non-temporal form.
+template <bool NT>
+__device__ __forceinline__ float2 ld_stream(const float2* p) {
+    if (NT) {
+        const v2f v = __builtin_nontemporal_load(reinterpret_cast<const v2f*>(p));
+        return make_float2(v.x, v.y);
+    }
+    return *p;
+}
+template <bool NT>
+__device__ __forceinline__ float4 ld_stream(const float4* p) {
+    if (NT) {
+        const v4f v = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(p));
+        return make_float4(v.x, v.y, v.z, v.w);
+    }
+    return *p;
+}
+template <bool NT>
+__device__ __forceinline__ void st_stream(float2* p, float2 v) {
+    if (NT)
+        __builtin_nontemporal_store(v2f{v.x, v.y}, reinterpret_cast<v2f*>(p));
+    else
+        *p = v;
+}
+template <bool NT>
+__device__ __forceinline__ void st_stream(float4* p, float4 v) {
+    if (NT)
+        __builtin_nontemporal_store(v4f{v.x, v.y, v.z, v.w}, reinterpret_cast<v4f*>(p));
+    else
+        *p = v;
 }
 
 __host__ __device__ __forceinline__ int ceil_div(int a, int b) { return (a + b - 1) / b; }
