@@ -1,0 +1,154 @@
+#!/usr/bin/env python3
+"""Benchmark of the hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one pass of the fused Galerkin attention core (LayerNorm of K and V,
+K^T V / S, Q (K^T V / S)) over one synthetic batch at the shape the metric is
+quoted on: B=8, S=44521 (211 x 211 grid points), d_model=128, 4 heads, fp32,
+inputs resident in HBM.  `value` is algorithmic bytes per second,
+4*B*H*32*S*4 bytes (Q, K, V read once, out written once) per step.
+
+One JSON line is printed.  Beside the contract keys it carries
+  roofline      the dominant kernel (K/V pass) against 8 TB/s, timed with HIP
+                events around the launch on its stream;
+  cpu_baseline  the CPU oracle (restatement of the reference's plain PyTorch
+                path) timed on this host's cores on the same shape;
+  extra         secondary measurements (feature-major op, config-2 split-K GEMM).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+
+
+def cpu_baseline(B, S, H, seed, budget_s=20.0):
+    """Oracle attention core on the host at the benchmark shape (fp32, all cores)."""
+    import torch
+    from oracle import spgt_oracle as O
+
+    g = torch.Generator().manual_seed(seed)
+    q, k, v = (torch.randn(B, S, H * 32, generator=g) for _ in range(3))
+    pos = torch.zeros(B, S, 0)
+    one, zero = torch.ones(H, 32), torch.zeros(H, 32)
+    run = lambda: O.attention_core_token_major(q, k, v, pos, one, zero, one, zero, 1e-6, H)
+    with torch.no_grad():
+        run()  # warm-up
+        times = []
+        t_start = time.perf_counter()
+        while len(times) < 5 or (time.perf_counter() - t_start < budget_s and len(times) < 15):
+            t0 = time.perf_counter()
+            run()
+            times.append(time.perf_counter() - t0)
+            if time.perf_counter() - t_start > 3 * budget_s:
+                break
+    times.sort()
+    med = times[len(times) // 2]
+    nbytes = 4 * B * H * 32 * S * 4
+    return {
+        "value": round(nbytes / med / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+        "sample": f"oracle attention core (per-head layer_norm + stack + cat + 2 matmuls + head merge), fp32, "
+                  f"full shape B={B} S={S} H={H}, median of {len(times)} runs, {med * 1e3:.1f} ms each",
+        "ms_per_step": round(med * 1e3, 3),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extra", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+
+    import torch
+    from spgt_amd.extension.bind import galerkin_attention as ga
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU (the HIP path has no CPU fallback)")
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    B, S, H, dp = 8, 44521, 4, 0
+    g = torch.Generator(device=dev).manual_seed(0)
+    q, k, v = (torch.randn(B, S, H * 32, device=dev, generator=g) for _ in range(3))
+    one, zero = torch.ones(H, 32, device=dev), torch.zeros(H, 32, device=dev)
+    step = lambda: ga.galerkin_attention_fused(q, k, v, None, one, zero, one, zero, 1e-6, H, dp)
+    nbytes = 4 * B * H * 32 * S * 4
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed / args.steps * 1e3
+    value = nbytes / (elapsed / args.steps) / 1e9
+
+    # dominant kernel: the K/V pass, HIP events around its launch on the launch stream
+    stage_ms = ga.gexts.galerkin_attention_fused_profile(q, k, v, None, one, zero, one, zero, 1e-6, H, dp, 30)
+    kv_bytes = 2 * B * H * 32 * S * 4  # K and V read once; partial tiles are not counted
+    achieved = kv_bytes / (stage_ms[0] * 1e-3) / 1e9
+    roofline = {
+        "bound": "hbm", "kernel": "ktv_ln_partial_tm<0,4>", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
+        "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+        "kernel_us": round(stage_ms[0] * 1e3, 2), "algorithmic_bytes": kv_bytes,
+        "stages_us": {"kv_pass": round(stage_ms[0] * 1e3, 2), "tile_reduce": round(stage_ms[1] * 1e3, 2),
+                      "q_pass": round(stage_ms[2] * 1e3, 2)},
+    }
+
+    extra = {}
+    if not args.no_extra:
+        def timed(fn, n=50, warm=5):
+            for _ in range(warm):
+                fn()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(n):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) / n
+
+        Qf, Kf, Vf = (torch.randn(B, H, 32, S, device=dev, generator=g) for _ in range(3))
+        ms = timed(lambda: ga.multihead_galerkin_attention_cccr_cuda(Qf, Kf, Vf))
+        extra["attention_cccr_d32"] = {"ms": round(ms, 4), "GB/s": round(nbytes / ms / 1e6, 1)}
+        del Qf, Kf, Vf
+        g1 = torch.Generator(device=dev).manual_seed(1)
+        A = torch.randn(32, 32, S, device=dev, generator=g1)
+        Bm = torch.randn(32, S, 32, device=dev, generator=g1)
+        c2_bytes = 2 * 32 * 32 * S * 4 + 32 * 32 * 32 * 4
+        ms = timed(lambda: ga.batched_skinny_gemm(A, Bm, 1.0))
+        extra["config2_split_k_gemm"] = {"ms": round(ms, 4), "GB/s": round(c2_bytes / ms / 1e6, 1)}
+        ms = timed(lambda: torch.matmul(A, Bm))
+        extra["config2_torch_matmul"] = {"ms": round(ms, 4), "GB/s": round(c2_bytes / ms / 1e6, 1)}
+
+    result = {
+        "metric": "galerkin_attn_hbm_gbps", "value": round(value, 1), "unit": "GB/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "fused Galerkin attention core (LayerNorm K,V + K^T V/S + Q(K^T V/S)), "
+                               "B=8 S=44521 d_model=128 heads=4 dp=0, token-major projections resident in HBM",
+                   "algorithmic_bytes_per_step": nbytes, "hbm_frac_of_8TBps": round(value / HBM_PEAK_GBPS, 4)},
+        "roofline": roofline,
+        "cpu_baseline": None if args.no_cpu_baseline else cpu_baseline(B, S, H, 0),
+        "extra": extra,
+    }
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

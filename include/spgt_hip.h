@@ -94,6 +94,23 @@ int spgt_galerkin_attention_fused_forward(const float* Q, const float* K, const 
                                           size_t workspace_bytes, int B, int S, int H, int dp,
                                           spgt_stream_t stream);
 
+
+/* Instrumented variant of spgt_galerkin_attention_fused_forward for benchmarks
+ * (no reference counterpart): runs the call `iterations` times, synchronising
+ * after each, with HIP events recorded on `stream` around each of its three
+ * launches, and writes the mean duration in milliseconds of
+ *   stage_ms[0]  K/V pass (LayerNorm + partial K'^T V' tiles)
+ *   stage_ms[1]  fixed-order reduction of the partial tiles
+ *   stage_ms[2]  Q pass (out = Q' M)
+ * to host memory. */
+int spgt_galerkin_attention_fused_profile(const float* Q, const float* K, const float* V,
+                                          int64_t ld_in, const float* position,
+                                          const float* ln_weight_K, const float* ln_bias_K,
+                                          const float* ln_weight_V, const float* ln_bias_V,
+                                          float norm_eps, float* out, float* ktv, void* workspace,
+                                          size_t workspace_bytes, int B, int S, int H, int dp,
+                                          spgt_stream_t stream, int iterations, float* stage_ms);
+
 #ifdef __cplusplus
 }
 #endif

@@ -16,6 +16,7 @@ Reference lines followed (paths relative to the reference checkout):
   project_layernorm_heads ...... network/layer.py:114-141
   galerkin_attention ........... network/layer.py:143-152
   attention_module ............. network/layer.py:67-93
+  attention_core_token_major ... network/layer.py:108-111, 128-140, 149-151, 89
   feed_forward ................. network/layer.py:165-174
   encoder_layer ................ network/layer.py:190-200
   complex_mode_product ......... network/layer.py:249-261
@@ -91,6 +92,23 @@ def galerkin_attention(Q, K, V):
 def attention_ktv(K, V):
     """The d x d matrices K^T V / S, [B, H, d, d]."""
     return (K.transpose(-2, -1) @ V) / K.shape[-2]
+
+
+def attention_core_token_major(q, k, v, position, ln_weight_K, ln_bias_K, ln_weight_V, ln_bias_V, eps, num_head):
+    """The part of GalerkinAttention.forward between the three Linear projections
+    and fc_layer (network/layer.py:108-111, 128-140, 149-151, 89), on projected
+    q, k, v [B, S, H*32]: split heads, per-head LayerNorm of k and v, position
+    channels first, Q (K^T V / S), heads merged back to [B, S, H*(dp+32)]."""
+    B, S, C = q.shape
+    dh = C // num_head
+    heads = lambda t: t.reshape(B, S, num_head, dh).permute(0, 2, 1, 3)
+    ln = lambda t, w, b: torch.stack(
+        [F.layer_norm(t[:, h], (dh,), w[h], b[h], eps) for h in range(num_head)], dim=1)
+    Q = _with_position(heads(q), position, num_head)
+    K = _with_position(ln(heads(k), ln_weight_K, ln_bias_K), position, num_head)
+    V = _with_position(ln(heads(v), ln_weight_V, ln_bias_V), position, num_head)
+    A = galerkin_attention(Q, K, V)
+    return A.permute(0, 2, 1, 3).contiguous().reshape(B, S, -1)
 
 
 def attention_module(p, xq, xk, xv, position, num_head, eps, prefix=""):

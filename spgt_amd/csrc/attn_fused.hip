@@ -461,11 +461,15 @@ extern "C" size_t spgt_galerkin_attention_fused_workspace_bytes(int B, int S, in
     return (size_t)B * H * p.nchunk1 * D * D * sizeof(float);
 }
 
-extern "C" int spgt_galerkin_attention_fused_forward(
+namespace {
+
+// Validates, then enqueues the three launches.  With `ev` (4 events) an event
+// is recorded before the first launch and after each launch.
+int fused_forward_impl(
     const float* Q, const float* K, const float* V, int64_t ld_in, const float* position,
     const float* ln_weight_K, const float* ln_bias_K, const float* ln_weight_V,
     const float* ln_bias_V, float norm_eps, float* out, float* ktv, void* workspace,
-    size_t workspace_bytes, int B, int S, int H, int dp, hipStream_t stream) {
+    size_t workspace_bytes, int B, int S, int H, int dp, hipStream_t stream, hipEvent_t* ev) {
     if (!Q || !K || !V || !out || !ktv || !ln_weight_K || !ln_bias_K || !ln_weight_V || !ln_bias_V)
         return fail(SPGT_ERR_INVALID_ARGUMENT, "galerkin_attention_fused: null pointer argument");
     if (B <= 0 || S <= 0 || H <= 0)
@@ -496,6 +500,7 @@ extern "C" int spgt_galerkin_attention_fused_forward(
     const dim3 grid2(p.nchunk2, H / 4, B);
     const dim3 gridr(ceil_div(D * D, 256), B * H);
     const float* pos = position ? position : Q;  // never dereferenced when dp == 0
+    if (ev) (void)hipEventRecord(ev[0], stream);
     if (dp == 0) {
         hipLaunchKernelGGL((ktv_ln_partial_tm<0, kU1>), grid1, block, 0, stream, K, V, pos, ln_weight_K,
                            ln_bias_K, ln_weight_V, ln_bias_V, norm_eps, partial, S, H, ld_in, p.tpc1);
@@ -503,11 +508,61 @@ extern "C" int spgt_galerkin_attention_fused_forward(
         hipLaunchKernelGGL((ktv_ln_partial_tm<2, kU1>), grid1, block, 0, stream, K, V, pos, ln_weight_K,
                            ln_bias_K, ln_weight_V, ln_bias_V, norm_eps, partial, S, H, ld_in, p.tpc1);
     }
+    if (ev) (void)hipEventRecord(ev[1], stream);
     hipLaunchKernelGGL(tile_reduce, gridr, block, 0, stream, partial, ktv, D * D, p.nchunk1, 1.0f / (float)S);
+    if (ev) (void)hipEventRecord(ev[2], stream);
     if (dp == 0) {
         hipLaunchKernelGGL((qm_apply_tm<0, kU2>), grid2, block, 0, stream, Q, pos, ktv, out, S, H, ld_in, p.tpc2);
     } else {
         hipLaunchKernelGGL((qm_apply_tm<2, kU2>), grid2, block, 0, stream, Q, pos, ktv, out, S, H, ld_in, p.tpc2);
     }
+    if (ev) (void)hipEventRecord(ev[3], stream);
     return check_launch("galerkin_attention_fused");
+}
+
+}  // namespace
+
+extern "C" int spgt_galerkin_attention_fused_forward(
+    const float* Q, const float* K, const float* V, int64_t ld_in, const float* position,
+    const float* ln_weight_K, const float* ln_bias_K, const float* ln_weight_V,
+    const float* ln_bias_V, float norm_eps, float* out, float* ktv, void* workspace,
+    size_t workspace_bytes, int B, int S, int H, int dp, hipStream_t stream) {
+    return fused_forward_impl(Q, K, V, ld_in, position, ln_weight_K, ln_bias_K, ln_weight_V, ln_bias_V, norm_eps,
+                              out, ktv, workspace, workspace_bytes, B, S, H, dp, stream, nullptr);
+}
+
+extern "C" int spgt_galerkin_attention_fused_profile(
+    const float* Q, const float* K, const float* V, int64_t ld_in, const float* position,
+    const float* ln_weight_K, const float* ln_bias_K, const float* ln_weight_V,
+    const float* ln_bias_V, float norm_eps, float* out, float* ktv, void* workspace,
+    size_t workspace_bytes, int B, int S, int H, int dp, hipStream_t stream, int iterations,
+    float* stage_ms) {
+    if (iterations <= 0 || !stage_ms)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "galerkin_attention_fused_profile: iterations and stage_ms required");
+    hipEvent_t ev[4];
+    for (int i = 0; i < 4; ++i)
+        if (hipEventCreate(&ev[i]) != hipSuccess) {
+            for (int j = 0; j < i; ++j) (void)hipEventDestroy(ev[j]);
+            return fail(SPGT_ERR_LAUNCH, "galerkin_attention_fused_profile: hipEventCreate failed");
+        }
+    double acc[3] = {0.0, 0.0, 0.0};
+    int rc = SPGT_OK;
+    for (int it = 0; it < iterations && rc == SPGT_OK; ++it) {
+        rc = fused_forward_impl(Q, K, V, ld_in, position, ln_weight_K, ln_bias_K, ln_weight_V, ln_bias_V,
+                                norm_eps, out, ktv, workspace, workspace_bytes, B, S, H, dp, stream, ev);
+        if (rc != SPGT_OK) break;
+        if (hipEventSynchronize(ev[3]) != hipSuccess) {
+            rc = fail(SPGT_ERR_LAUNCH, "galerkin_attention_fused_profile: hipEventSynchronize failed");
+            break;
+        }
+        for (int k = 0; k < 3; ++k) {
+            float ms = 0.f;
+            (void)hipEventElapsedTime(&ms, ev[k], ev[k + 1]);
+            acc[k] += ms;
+        }
+    }
+    for (int i = 0; i < 4; ++i) (void)hipEventDestroy(ev[i]);
+    if (rc == SPGT_OK)
+        for (int k = 0; k < 3; ++k) stage_ms[k] = (float)(acc[k] / iterations);
+    return rc;
 }

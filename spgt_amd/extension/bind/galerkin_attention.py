@@ -116,7 +116,28 @@ def _attention_fused_forward(QKV_or_Q, K, V, position, ln_weight_K, ln_bias_K, l
     return (out, ktv) if return_ktv else out
 
 
+def _attention_fused_profile(Q, K, V, position, ln_weight_K, ln_bias_K, ln_weight_V, ln_bias_V, norm_eps: float,
+                             num_head: int, dim_position: int, iterations: int):
+    """Mean milliseconds of the three launches of the fused attention core
+    (K/V pass, tile reduction, Q pass), measured with HIP events on the current stream."""
+    import ctypes
+    B, S, _ = Q.shape
+    H, D = num_head, dim_position + 32
+    lib = _lib.load()
+    out = torch.empty((B, S, H * D), dtype=torch.float32, device=Q.device)
+    ktv = torch.empty((B, H, D, D), dtype=torch.float32, device=Q.device)
+    ws = workspace(lib.spgt_galerkin_attention_fused_workspace_bytes(B, S, H, dim_position), Q)
+    stage = (ctypes.c_float * 3)()
+    with torch.cuda.device(Q.device):
+        check(lib.spgt_galerkin_attention_fused_profile(
+            ptr(Q), ptr(K), ptr(V), Q.stride(1), ptr(position) if dim_position == 2 else None, ptr(ln_weight_K),
+            ptr(ln_bias_K), ptr(ln_weight_V), ptr(ln_bias_V), float(norm_eps), ptr(out), ptr(ktv), ptr(ws),
+            ws.numel(), B, S, H, dim_position, stream_of(Q), int(iterations), stage))
+    return [float(x) for x in stage]
+
+
 gexts = SimpleNamespace(
+    galerkin_attention_fused_profile=_attention_fused_profile,
     multihead_galerkin_attention_cccr_forward=_attention_cccr_forward,
     batched_skinny_gemm=_batched_skinny_gemm,
     galerkin_attention_fused_forward=_attention_fused_forward,
