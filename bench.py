@@ -67,6 +67,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 256 MiB device copy (a kernel of known traffic, for scaling "
+                         "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -110,6 +113,14 @@ def main():
     }
 
     extra = {}
+    if args.calibrate_copy:
+        src = torch.empty(256 * 1024 * 1024 // 4, device=dev).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)  # vectorized elementwise copy kernel: reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        extra["calibrate_copy_bytes_each_way"] = src.numel() * 4
+        del src, dst
     if not args.no_extra:
         def timed(fn, n=50, warm=5):
             for _ in range(warm):
