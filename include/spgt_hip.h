@@ -94,6 +94,44 @@ int spgt_galerkin_attention_fused_forward(const float* Q, const float* K, const 
                                           size_t workspace_bytes, int B, int S, int H, int dp,
                                           spgt_stream_t stream);
 
+/* ---- FNO2d data movement and spectral contraction --------------------------- */
+
+/* Replaces batched_transpose (extension/bind/datamove.cu:8-23):
+ * src [batch_count, M, N] -> dst [batch_count, N, M], 32-bit words moved bit-exactly. */
+int spgt_batched_transpose(const float* src, float* dst, int batch_count, int M, int N,
+                           spgt_stream_t stream);
+
+/* Replaces transpose_gather_dual (extension/bind/datamove.cu:25-44).  src is complex64
+ * [dim, H_all, W_all]; out_k [H_low, W_low, dim] receives the window whose top-left
+ * corner is (H_base_k, W_base_k), transposed.  64-bit words moved bit-exactly. */
+int spgt_transpose_gather_dual(const float* src, float* out1, float* out2, int dim, int H_all,
+                               int W_all, int H_low, int W_low, int H_base_1, int W_base_1,
+                               int H_base_2, int W_base_2, spgt_stream_t stream);
+
+/* Replaces transpose_scatter_dual (extension/bind/datamove.cu:46-64), including its
+ * torch::zeros: out [dim, H_all, W_all] complex64 is written completely, zero outside
+ * the two windows; where the windows overlap the second source wins. */
+int spgt_transpose_scatter_dual(const float* src1, const float* src2, float* out, int dim, int H_all,
+                                int W_all, int H_low, int W_low, int H_base_1, int W_base_1,
+                                int H_base_2, int W_base_2, spgt_stream_t stream);
+
+/* The spectral part of Sp_SpectralConv2D.forward between rfft2 and irfft2 in one call
+ * (network/sp_layer.py:139-148: transpose_gather_dual, two complex `@`, and
+ * transpose_scatter_dual; the arithmetic is complex_matmul_2D of network/layer.py:249-261):
+ *   Out_ft[n, o, hb_k+h, wb_k+w] = sum_i X_ft[n, i, hb_k+h, wb_k+w] * weight_k[h, w, i, o]
+ * X_ft [N, Cin, H_all, W_all] complex64, weight_k [H_low, W_low, Cin, Cout] complex64
+ * (the accelerated module's parameter layout, sp_layer.py:119-121),
+ * Out_ft [N, Cout, H_all, W_all] complex64, written completely (zero outside the windows). */
+int spgt_spectral_mode_contract(const float* X_ft, const float* weight_1, const float* weight_2,
+                                float* Out_ft, int N, int Cin, int Cout, int H_all, int W_all,
+                                int H_low, int W_low, int H_base_1, int W_base_1, int H_base_2,
+                                int W_base_2, spgt_stream_t stream);
+
+/* Replaces F.interpolate(x, size, mode='bilinear', align_corners=True) as used by
+ * DownScaler2D / UpScaler2D (network/model.py:30, 36, 59, 63):
+ * src [planes, H_in, W_in] -> dst [planes, H_out, W_out]. */
+int spgt_bilinear_align_corners(const float* src, float* dst, int planes, int H_in, int W_in,
+                                int H_out, int W_out, spgt_stream_t stream);
 
 /* Instrumented variant of spgt_galerkin_attention_fused_forward for benchmarks
  * (no reference counterpart): runs the call `iterations` times, synchronising

@@ -30,6 +30,11 @@ SIGNATURES = {
     "spgt_galerkin_attention_fused_workspace_bytes": (_sz, [_i, _i, _i, _i]),
     "spgt_galerkin_attention_fused_forward": (
         _i, [_p, _p, _p, _i64, _p, _p, _p, _p, _p, _f, _p, _p, _p, _sz, _i, _i, _i, _i, _p]),
+    "spgt_batched_transpose": (_i, [_p, _p, _i, _i, _i, _p]),
+    "spgt_transpose_gather_dual": (_i, [_p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p]),
+    "spgt_transpose_scatter_dual": (_i, [_p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p]),
+    "spgt_spectral_mode_contract": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p]),
+    "spgt_bilinear_align_corners": (_i, [_p, _p, _i, _i, _i, _i, _i, _p]),
     "spgt_galerkin_attention_fused_profile": (
         _i, [_p, _p, _p, _i64, _p, _p, _p, _p, _p, _f, _p, _p, _p, _sz, _i, _i, _i, _i, _p, _i,
              ctypes.POINTER(ctypes.c_float)]),

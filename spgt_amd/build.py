@@ -16,6 +16,8 @@ SOURCES = [
     "spgt_host.cpp",
     "attn_fused.hip",
     "attn_cccr.hip",
+    "datamove.hip",
+    "spectral.hip",
 ]
 
 # Packed fp32 VALU forms (v_pk_*_f32) are switched off for all device code.

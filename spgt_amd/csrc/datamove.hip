@@ -1,0 +1,185 @@
+// Pure data-movement kernels of the FNO path: batched 2-D transpose, and the
+// corner-window gather / scatter (with transposition) of a half spectrum.
+// Every kernel copies 32-bit or 64-bit words unchanged, so results are
+// bit-exact whatever the payload (NaN payloads, -0.0, ...).
+//
+// Reference behaviour restated here:
+//   batched_transpose       extension/bind/datamove.cu:8-23,  native/datamove.cu:8-32, 92-99
+//   transpose_gather_dual   extension/bind/datamove.cu:25-44, native/datamove.cu:34-61, 102-109
+//   transpose_scatter_dual  extension/bind/datamove.cu:46-64, native/datamove.cu:63-89, 112-119
+#include "spgt_device.h"
+#include "spgt_host.h"
+
+namespace spgt {
+
+// [batch, M, N] -> [batch, N, M], 32-bit words.  grid (tiles_n, tiles_m, batch), block 256.
+// A 64x64 tile goes through LDS (pitch 65: conflict-free both ways); global
+// reads and writes are 256-byte runs per wave.
+__global__ __launch_bounds__(256) void batched_transpose_64(const uint32_t* __restrict__ src,
+                                                            uint32_t* __restrict__ dst, int M, int N) {
+    __shared__ uint32_t tile[64 * 65];
+    const int tx = threadIdx.x & 63;
+    const int ty = threadIdx.x >> 6;
+    const int n0 = blockIdx.x * 64;
+    const int m0 = blockIdx.y * 64;
+    const int64_t base = (int64_t)blockIdx.z * M * N;
+    const uint32_t* s = src + base;
+    uint32_t* d = dst + base;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const int m = m0 + 4 * i + ty;
+        const int n = n0 + tx;
+        if (m < M && n < N) tile[(4 * i + ty) * 65 + tx] = s[(int64_t)m * N + n];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const int n = n0 + 4 * i + ty;
+        const int m = m0 + tx;
+        if (m < M && n < N) d[(int64_t)n * M + m] = tile[tx * 65 + 4 * i + ty];
+    }
+}
+
+struct Windows {
+    int h_base[2];
+    int w_base[2];
+};
+
+// src [dim, H_all, W_all] (64-bit words) -> out_k [H_low, W_low, dim] for the two windows.
+// grid (ceil(dim/64), H_low, 2), block 256: a block moves 64 values of `dim` for one window row.
+__global__ __launch_bounds__(256) void transpose_gather_dual_k(const uint64_t* __restrict__ src,
+                                                               uint64_t* __restrict__ out1,
+                                                               uint64_t* __restrict__ out2, int dim, int H_all,
+                                                               int W_all, int H_low, int W_low, Windows win) {
+    extern __shared__ uint64_t gtile[];  // [W_low][65]
+    const int d0 = blockIdx.x * 64;
+    const int h = blockIdx.y;
+    const int k = blockIdx.z;
+    uint64_t* out = k == 0 ? out1 : out2;
+    const int64_t plane = (int64_t)H_all * W_all;
+    const uint64_t* row = src + (int64_t)(win.h_base[k] + h) * W_all + win.w_base[k];
+    // read: consecutive threads walk along w (contiguous in src), then along dim
+    for (int e = threadIdx.x; e < 64 * W_low; e += 256) {
+        const int w = e % W_low;
+        const int dd = e / W_low;
+        if (d0 + dd < dim) gtile[w * 65 + dd] = row[(int64_t)(d0 + dd) * plane + w];
+    }
+    __syncthreads();
+    // write: consecutive threads walk along dim (contiguous in out)
+    for (int e = threadIdx.x; e < 64 * W_low; e += 256) {
+        const int dd = e & 63;
+        const int w = e >> 6;
+        if (d0 + dd < dim) out[((int64_t)h * W_low + w) * dim + d0 + dd] = gtile[w * 65 + dd];
+    }
+}
+
+// out [dim, H_all, W_all] (64-bit words): zero everywhere except the two windows,
+// which receive src_k [H_low, W_low, dim] transposed.  Where the windows overlap the
+// second one wins (the reference scatters window 1, then window 2).
+// grid (ceil(dim/64), H_all), block 256: a block writes row h of 64 planes.
+__global__ __launch_bounds__(256) void transpose_scatter_dual_k(const uint64_t* __restrict__ src1,
+                                                                const uint64_t* __restrict__ src2,
+                                                                uint64_t* __restrict__ out, int dim, int H_all,
+                                                                int W_all, int H_low, int W_low, Windows win) {
+    extern __shared__ uint64_t stile[];  // [2][W_low][65]
+    const int d0 = blockIdx.x * 64;
+    const int h = blockIdx.y;
+    bool in_win[2];
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+        in_win[k] = h >= win.h_base[k] && h < win.h_base[k] + H_low;
+        if (in_win[k]) {
+            const uint64_t* s = (k == 0 ? src1 : src2) + (int64_t)(h - win.h_base[k]) * W_low * dim;
+            uint64_t* t = stile + k * W_low * 65;
+            for (int e = threadIdx.x; e < 64 * W_low; e += 256) {
+                const int dd = e & 63;
+                const int w = e >> 6;
+                if (d0 + dd < dim) t[w * 65 + dd] = s[(int64_t)w * dim + d0 + dd];
+            }
+        }
+    }
+    __syncthreads();
+    const int64_t plane = (int64_t)H_all * W_all;
+    for (int e = threadIdx.x; e < 64 * W_all; e += 256) {
+        const int w = e % W_all;
+        const int dd = e / W_all;
+        if (d0 + dd >= dim) continue;
+        uint64_t v = 0;
+        if (in_win[1] && w >= win.w_base[1] && w < win.w_base[1] + W_low)
+            v = stile[(W_low + w - win.w_base[1]) * 65 + dd];
+        else if (in_win[0] && w >= win.w_base[0] && w < win.w_base[0] + W_low)
+            v = stile[(w - win.w_base[0]) * 65 + dd];
+        out[(int64_t)(d0 + dd) * plane + (int64_t)h * W_all + w] = v;
+    }
+}
+
+namespace {
+
+int check_windows(const char* who, int dim, int H_all, int W_all, int H_low, int W_low, int hb1, int wb1, int hb2,
+                  int wb2) {
+    if (dim <= 0 || H_all <= 0 || W_all <= 0 || H_low <= 0 || W_low <= 0)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "transpose_gather/scatter_dual: sizes must be positive");
+    if (hb1 < 0 || hb2 < 0 || wb1 < 0 || wb2 < 0 || hb1 + H_low > H_all || hb2 + H_low > H_all ||
+        wb1 + W_low > W_all || wb2 + W_low > W_all)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "transpose_gather/scatter_dual: a window leaves the [H_all, W_all] plane");
+    if ((size_t)W_low * 65 * 8 * 2 > 64 * 1024)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "transpose_gather/scatter_dual: W_low above 63 is not supported");
+    if (H_all > 65535 || H_low > 65535)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "transpose_gather/scatter_dual: H_all exceeds 65535");
+    (void)who;
+    return SPGT_OK;
+}
+
+}  // namespace
+
+}  // namespace spgt
+
+using namespace spgt;
+
+extern "C" int spgt_batched_transpose(const float* src, float* dst, int batch_count, int M, int N,
+                                      hipStream_t stream) {
+    if (!src || !dst) return fail(SPGT_ERR_INVALID_ARGUMENT, "batched_transpose: null pointer argument");
+    if (batch_count <= 0 || M <= 0 || N <= 0)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "batched_transpose: batch_count, M, N must be positive");
+    if (src == dst) return fail(SPGT_ERR_INVALID_ARGUMENT, "batched_transpose: in-place transposition is not supported");
+    if (batch_count > 65535 || ceil_div(M, 64) > 65535)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "batched_transpose: batch_count or M/64 exceeds 65535");
+    if (!aligned4(src) || !aligned4(dst))
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "batched_transpose: operands must be 4-byte aligned");
+    const dim3 grid(ceil_div(N, 64), ceil_div(M, 64), batch_count);
+    hipLaunchKernelGGL(batched_transpose_64, grid, dim3(256), 0, stream, reinterpret_cast<const uint32_t*>(src),
+                       reinterpret_cast<uint32_t*>(dst), M, N);
+    return check_launch("batched_transpose");
+}
+
+extern "C" int spgt_transpose_gather_dual(const float* src, float* out1, float* out2, int dim, int H_all, int W_all,
+                                          int H_low, int W_low, int H_base_1, int W_base_1, int H_base_2,
+                                          int W_base_2, hipStream_t stream) {
+    if (!src || !out1 || !out2) return fail(SPGT_ERR_INVALID_ARGUMENT, "transpose_gather_dual: null pointer argument");
+    const int rc = check_windows("gather", dim, H_all, W_all, H_low, W_low, H_base_1, W_base_1, H_base_2, W_base_2);
+    if (rc != SPGT_OK) return rc;
+    if (!aligned8(src) || !aligned8(out1) || !aligned8(out2))
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "transpose_gather_dual: complex operands must be 8-byte aligned");
+    Windows win{{H_base_1, H_base_2}, {W_base_1, W_base_2}};
+    const dim3 grid(ceil_div(dim, 64), H_low, 2);
+    hipLaunchKernelGGL(transpose_gather_dual_k, grid, dim3(256), (size_t)W_low * 65 * 8, stream,
+                       reinterpret_cast<const uint64_t*>(src), reinterpret_cast<uint64_t*>(out1),
+                       reinterpret_cast<uint64_t*>(out2), dim, H_all, W_all, H_low, W_low, win);
+    return check_launch("transpose_gather_dual");
+}
+
+extern "C" int spgt_transpose_scatter_dual(const float* src1, const float* src2, float* out, int dim, int H_all,
+                                           int W_all, int H_low, int W_low, int H_base_1, int W_base_1,
+                                           int H_base_2, int W_base_2, hipStream_t stream) {
+    if (!src1 || !src2 || !out) return fail(SPGT_ERR_INVALID_ARGUMENT, "transpose_scatter_dual: null pointer argument");
+    const int rc = check_windows("scatter", dim, H_all, W_all, H_low, W_low, H_base_1, W_base_1, H_base_2, W_base_2);
+    if (rc != SPGT_OK) return rc;
+    if (!aligned8(src1) || !aligned8(src2) || !aligned8(out))
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "transpose_scatter_dual: complex operands must be 8-byte aligned");
+    Windows win{{H_base_1, H_base_2}, {W_base_1, W_base_2}};
+    const dim3 grid(ceil_div(dim, 64), H_all);
+    hipLaunchKernelGGL(transpose_scatter_dual_k, grid, dim3(256), (size_t)W_low * 65 * 8 * 2, stream,
+                       reinterpret_cast<const uint64_t*>(src1), reinterpret_cast<const uint64_t*>(src2),
+                       reinterpret_cast<uint64_t*>(out), dim, H_all, W_all, H_low, W_low, win);
+    return check_launch("transpose_scatter_dual");
+}

@@ -1,0 +1,177 @@
+// FNO2d spectral-mode complex channel contraction, fused with the gather of the
+// two retained corner windows and the scatter into a zero-filled output
+// spectrum, and bilinear (align_corners) resampling.
+//
+// Reference behaviour restated here:
+//   Sp_SpectralConv2D.forward, the part between rfft2 and irfft2
+//       network/sp_layer.py:139-148 (gather_dual, two complex matmuls, scatter_dual)
+//   SpectralConv2D.complex_matmul_2D      network/layer.py:249-261
+//   F.interpolate(mode='bilinear', align_corners=True) in DownScaler2D / UpScaler2D
+//       network/model.py:30, 36, 59, 63
+#include "spgt_device.h"
+#include "spgt_host.h"
+
+namespace spgt {
+
+struct SpecWindows {
+    int h_base[2];
+    int w_base[2];
+};
+
+// out[n, o, hb_k + hh, wb_k + ww] = sum_i X[n, i, hb_k + hh, wb_k + ww] * W_k[hh, ww, i, o]   (complex)
+// grid (m_h * m_w, 2, ceil(Cout/64)), block 256 = 64 output channels x 4 batch groups.
+// One workgroup per mode: the mode's input column X[:, :, h, w] is staged in LDS
+// (NB batch entries at a time), the mode's weight block [Cin, 64] is streamed
+// once per batch group with 512-byte coalesced rows.
+constexpr int kSpecNB = 16;
+
+__global__ __launch_bounds__(256) void spectral_mode_contract_k(
+    const float2* __restrict__ X, const float2* __restrict__ W0, const float2* __restrict__ W1,
+    float2* __restrict__ out, int N, int Cin, int Cout, int H_all, int W_all, int m_h, int m_w,
+    SpecWindows win) {
+    extern __shared__ float2 xs[];  // [kSpecNB][Cin]
+    const int mode = blockIdx.x;
+    const int k = blockIdx.y;
+    const int hh = mode / m_w;
+    const int ww = mode % m_w;
+    const int h = win.h_base[k] + hh;
+    const int w = win.w_base[k] + ww;
+    // Where the windows overlap the second one wins (the reference assigns it last).
+    if (k == 0 && h >= win.h_base[1] && h < win.h_base[1] + m_h && w >= win.w_base[1] && w < win.w_base[1] + m_w)
+        return;
+    const int o = blockIdx.z * 64 + (threadIdx.x & 63);
+    const int ng = threadIdx.x >> 6;
+    const float2* Wm = (k == 0 ? W0 : W1) + (int64_t)mode * Cin * Cout;
+    const int64_t plane = (int64_t)H_all * W_all;
+    const int64_t pix = (int64_t)h * W_all + w;
+
+    for (int n0 = 0; n0 < N; n0 += kSpecNB) {
+        const int nb = min(kSpecNB, N - n0);
+        __syncthreads();
+        for (int e = threadIdx.x; e < nb * Cin; e += 256) {
+            const int n = e / Cin;
+            const int i = e - n * Cin;
+            xs[e] = X[((int64_t)(n0 + n) * Cin + i) * plane + pix];
+        }
+        __syncthreads();
+        float2 acc[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[j] = make_float2(0.f, 0.f);
+        if (o < Cout) {
+            for (int i = 0; i < Cin; ++i) {
+                const float2 wv = Wm[(int64_t)i * Cout + o];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int n = ng + 4 * j;
+                    if (n < nb) {
+                        const float2 xv = xs[n * Cin + i];
+                        acc[j].x = fmaf(xv.x, wv.x, acc[j].x);
+                        acc[j].x = fmaf(-xv.y, wv.y, acc[j].x);
+                        acc[j].y = fmaf(xv.y, wv.x, acc[j].y);
+                        acc[j].y = fmaf(xv.x, wv.y, acc[j].y);
+                    }
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int n = ng + 4 * j;
+                if (n < nb) out[((int64_t)(n0 + n) * Cout + o) * plane + pix] = acc[j];
+            }
+        }
+    }
+}
+
+// Zeros every element of out [planes, H_all, W_all] (complex) outside the two windows.
+__global__ __launch_bounds__(256) void spectrum_zero_outside_k(float2* __restrict__ out, int64_t total, int H_all,
+                                                               int W_all, int m_h, int m_w, SpecWindows win) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < total; e += stride) {
+        const int w = (int)(e % W_all);
+        const int h = (int)((e / W_all) % H_all);
+        const bool in0 = h >= win.h_base[0] && h < win.h_base[0] + m_h && w >= win.w_base[0] && w < win.w_base[0] + m_w;
+        const bool in1 = h >= win.h_base[1] && h < win.h_base[1] + m_h && w >= win.w_base[1] && w < win.w_base[1] + m_w;
+        if (!in0 && !in1) out[e] = make_float2(0.f, 0.f);
+    }
+}
+
+// Bilinear resampling with align_corners=True of [planes, Hin, Win] -> [planes, Hout, Wout].
+// Same arithmetic as torch's upsample_bilinear2d: scale = (in-1)/(out-1) in fp32
+// (0 when out == 1), source coordinate scale*dst, weights (1-l, l), rows blended last.
+// grid (ceil(Wout/64), ceil(Hout/4), planes), block (64, 4).
+__global__ __launch_bounds__(256) void bilinear_align_corners_k(const float* __restrict__ src,
+                                                                float* __restrict__ dst, int planes, int Hin,
+                                                                int Win, int Hout, int Wout, float hscale,
+                                                                float wscale) {
+    const int ox = blockIdx.x * 64 + threadIdx.x;
+    const int oy = blockIdx.y * 4 + threadIdx.y;
+    if (ox >= Wout || oy >= Hout) return;
+    const float hr = hscale * (float)oy;
+    const int h1 = (int)hr;
+    const int hp = (h1 < Hin - 1) ? 1 : 0;
+    const float h1l = hr - (float)h1;
+    const float h0l = 1.0f - h1l;
+    const float wr = wscale * (float)ox;
+    const int w1 = (int)wr;
+    const int wp = (w1 < Win - 1) ? 1 : 0;
+    const float w1l = wr - (float)w1;
+    const float w0l = 1.0f - w1l;
+    for (int64_t pl = blockIdx.z; pl < planes; pl += gridDim.z) {
+        const float* r0 = src + pl * Hin * Win + (int64_t)h1 * Win + w1;
+        const float* r1 = r0 + (int64_t)hp * Win;
+        const float top = w0l * r0[0] + w1l * r0[wp];
+        const float bot = w0l * r1[0] + w1l * r1[wp];
+        dst[(pl * Hout + oy) * Wout + ox] = h0l * top + h1l * bot;
+    }
+}
+
+}  // namespace spgt
+
+using namespace spgt;
+
+extern "C" int spgt_spectral_mode_contract(const float* X_ft, const float* weight_1, const float* weight_2,
+                                           float* Out_ft, int N, int Cin, int Cout, int H_all, int W_all,
+                                           int H_low, int W_low, int H_base_1, int W_base_1, int H_base_2,
+                                           int W_base_2, hipStream_t stream) {
+    if (!X_ft || !weight_1 || !weight_2 || !Out_ft)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "spectral_mode_contract: null pointer argument");
+    if (N <= 0 || Cin <= 0 || Cout <= 0 || H_all <= 0 || W_all <= 0 || H_low <= 0 || W_low <= 0)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "spectral_mode_contract: sizes must be positive");
+    if (H_base_1 < 0 || H_base_2 < 0 || W_base_1 < 0 || W_base_2 < 0 || H_base_1 + H_low > H_all ||
+        H_base_2 + H_low > H_all || W_base_1 + W_low > W_all || W_base_2 + W_low > W_all)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "spectral_mode_contract: a window leaves the [H_all, W_all] plane");
+    if ((size_t)kSpecNB * Cin * sizeof(float2) > 64 * 1024)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "spectral_mode_contract: Cin above 512 is not supported");
+    if (ceil_div(Cout, 64) > 65535)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "spectral_mode_contract: Cout too large");
+    if (X_ft == Out_ft) return fail(SPGT_ERR_INVALID_ARGUMENT, "spectral_mode_contract: in-place call is not supported");
+    if (!aligned8(X_ft) || !aligned8(weight_1) || !aligned8(weight_2) || !aligned8(Out_ft))
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "spectral_mode_contract: complex operands must be 8-byte aligned");
+    SpecWindows win{{H_base_1, H_base_2}, {W_base_1, W_base_2}};
+    const int64_t total = (int64_t)N * Cout * H_all * W_all;
+    const int fill_blocks = (int)std::min<int64_t>((total + 255) / 256, 256 * 32);
+    hipLaunchKernelGGL(spectrum_zero_outside_k, dim3(fill_blocks), dim3(256), 0, stream,
+                       reinterpret_cast<float2*>(Out_ft), total, H_all, W_all, H_low, W_low, win);
+    const dim3 grid(H_low * W_low, 2, ceil_div(Cout, 64));
+    hipLaunchKernelGGL(spectral_mode_contract_k, grid, dim3(256), (size_t)kSpecNB * Cin * sizeof(float2), stream,
+                       reinterpret_cast<const float2*>(X_ft), reinterpret_cast<const float2*>(weight_1),
+                       reinterpret_cast<const float2*>(weight_2), reinterpret_cast<float2*>(Out_ft), N, Cin, Cout,
+                       H_all, W_all, H_low, W_low, win);
+    return check_launch("spectral_mode_contract");
+}
+
+extern "C" int spgt_bilinear_align_corners(const float* src, float* dst, int planes, int H_in, int W_in, int H_out,
+                                           int W_out, hipStream_t stream) {
+    if (!src || !dst) return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear_align_corners: null pointer argument");
+    if (planes <= 0 || H_in <= 0 || W_in <= 0 || H_out <= 0 || W_out <= 0)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear_align_corners: sizes must be positive");
+    if (ceil_div(H_out, 4) > 65535)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear_align_corners: H_out/4 exceeds 65535");
+    if (!aligned4(src) || !aligned4(dst))
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear_align_corners: operands must be 4-byte aligned");
+    const float hscale = H_out > 1 ? (float)(H_in - 1) / (float)(H_out - 1) : 0.f;
+    const float wscale = W_out > 1 ? (float)(W_in - 1) / (float)(W_out - 1) : 0.f;
+    const dim3 grid(ceil_div(W_out, 64), ceil_div(H_out, 4), std::min(planes, 65535));
+    hipLaunchKernelGGL(bilinear_align_corners_k, grid, dim3(64, 4), 0, stream, src, dst, planes, H_in, W_in, H_out,
+                       W_out, hscale, wscale);
+    return check_launch("bilinear_align_corners");
+}

@@ -1,0 +1,196 @@
+"""Operator API of the FNO data-movement path, backed by libspgt_hip.so.
+
+Same function names, argument order and result layouts as the reference's
+extension/bind/datamove.py:68-87 (python surface) and
+extension/bind/datamove.cu:66-70 (the `dexts` module surface), plus two
+operators the reference leaves to library calls: the fused spectral-mode
+contraction and bilinear resampling.  Tensors must be contiguous and on a GPU.
+"""
+from math import prod
+from types import SimpleNamespace
+from typing import Any, List, Tuple
+
+import torch
+from torch import Tensor
+
+from ... import _lib
+from ..._lib import check, ptr, require_gpu_f32, stream_of
+
+
+# --------------------------------------------------------------------------- #
+# `dexts` surface: plain functions on tensors, no autograd
+# --------------------------------------------------------------------------- #
+
+def _batched_transpose(src: Tensor, batch_list: List[int], M_list: List[int], N_list: List[int]) -> Tensor:
+    """src viewed as [prod(batch), prod(M), prod(N)] -> shape batch_list + N_list + M_list
+    (reference: extension/bind/datamove.cu:8-23)."""
+    require_gpu_f32("src", src)
+    b, M, N = prod(batch_list), prod(M_list), prod(N_list)
+    if src.numel() != b * M * N:
+        raise ValueError(f"src has {src.numel()} elements, the lists describe {b}x{M}x{N}")
+    out = torch.empty(list(batch_list) + list(N_list) + list(M_list), dtype=src.dtype, device=src.device)
+    if src.numel() == 0:
+        return out
+    with torch.cuda.device(src.device):
+        check(_lib.load().spgt_batched_transpose(ptr(src), ptr(out), b, M, N, stream_of(src)))
+    return out
+
+
+def _transpose_gather_dual(src: Tensor, dim_list: List[int], H_all: int, W_all: int, H_low: int, W_low: int,
+                           H_base_1: int, W_base_1: int, H_base_2: int, W_base_2: int) -> Tuple[Tensor, Tensor]:
+    """src complex64 [*dim_list, H_all, W_all] -> two [H_low, W_low, *dim_list] windows
+    (reference: extension/bind/datamove.cu:25-44)."""
+    require_gpu_f32("src", src, torch.complex64)
+    dim = prod(dim_list)
+    if src.numel() != dim * H_all * W_all:
+        raise ValueError(f"src has {src.numel()} elements, expected {dim}x{H_all}x{W_all}")
+    shape = [H_low, W_low] + list(dim_list)
+    out1 = torch.empty(shape, dtype=src.dtype, device=src.device)
+    out2 = torch.empty(shape, dtype=src.dtype, device=src.device)
+    with torch.cuda.device(src.device):
+        check(_lib.load().spgt_transpose_gather_dual(
+            ptr(src), ptr(out1), ptr(out2), dim, H_all, W_all, H_low, W_low, H_base_1, W_base_1, H_base_2, W_base_2,
+            stream_of(src)))
+    return out1, out2
+
+
+def _transpose_scatter_dual(src1: Tensor, src2: Tensor, dim_list: List[int], H_all: int, W_all: int, H_low: int,
+                            W_low: int, H_base_1: int, W_base_1: int, H_base_2: int, W_base_2: int) -> Tensor:
+    """Inverse of the gather into a zero-filled complex64 [*dim_list, H_all, W_all]
+    (reference: extension/bind/datamove.cu:46-64)."""
+    require_gpu_f32("src1", src1, torch.complex64)
+    require_gpu_f32("src2", src2, torch.complex64)
+    dim = prod(dim_list)
+    for name, t in (("src1", src1), ("src2", src2)):
+        if t.numel() != H_low * W_low * dim:
+            raise ValueError(f"{name} has {t.numel()} elements, expected {H_low}x{W_low}x{dim}")
+    out = torch.empty(list(dim_list) + [H_all, W_all], dtype=src1.dtype, device=src1.device)
+    with torch.cuda.device(src1.device):
+        check(_lib.load().spgt_transpose_scatter_dual(
+            ptr(src1), ptr(src2), ptr(out), dim, H_all, W_all, H_low, W_low, H_base_1, W_base_1, H_base_2, W_base_2,
+            stream_of(src1)))
+    return out
+
+
+def _spectral_mode_contract(X_ft: Tensor, weight_1: Tensor, weight_2: Tensor, H_low: int, W_low: int, H_base_1: int,
+                            W_base_1: int, H_base_2: int, W_base_2: int) -> Tensor:
+    """X_ft complex64 [N, Cin, H_all, W_all]; weight_k fp32 [H_low, W_low, Cin, Cout, 2] (or complex64
+    [H_low, W_low, Cin, Cout]) -> complex64 [N, Cout, H_all, W_all], zero outside the two windows."""
+    require_gpu_f32("X_ft", X_ft, torch.complex64)
+    if X_ft.dim() != 4:
+        raise ValueError("X_ft must be [N, Cin, H_all, W_all]")
+    N, Cin, H_all, W_all = X_ft.shape
+    ws = []
+    for name, w in (("weight_1", weight_1), ("weight_2", weight_2)):
+        if w.is_complex():
+            w = torch.view_as_real(w)
+        require_gpu_f32(name, w)
+        if w.dim() != 5 or tuple(w.shape[:3]) != (H_low, W_low, Cin) or w.shape[-1] != 2:
+            raise ValueError(f"{name} must be [{H_low}, {W_low}, {Cin}, Cout, 2], got {tuple(w.shape)}")
+        ws.append(w)
+    Cout = ws[0].shape[3]
+    if ws[1].shape[3] != Cout:
+        raise ValueError("weight_1 and weight_2 disagree on Cout")
+    out = torch.empty((N, Cout, H_all, W_all), dtype=torch.complex64, device=X_ft.device)
+    with torch.cuda.device(X_ft.device):
+        check(_lib.load().spgt_spectral_mode_contract(
+            ptr(X_ft), ptr(ws[0]), ptr(ws[1]), ptr(out), N, Cin, Cout, H_all, W_all, H_low, W_low, H_base_1,
+            W_base_1, H_base_2, W_base_2, stream_of(X_ft)))
+    return out
+
+
+def _bilinear_align_corners(X: Tensor, size) -> Tensor:
+    """X [..., H_in, W_in] -> [..., H_out, W_out], F.interpolate(mode='bilinear', align_corners=True)."""
+    require_gpu_f32("X", X)
+    if X.dim() < 2:
+        raise ValueError("X needs at least two dimensions")
+    H_out, W_out = (size, size) if isinstance(size, int) else tuple(size)
+    lead = tuple(X.shape[:-2])
+    H_in, W_in = X.shape[-2:]
+    out = torch.empty(lead + (H_out, W_out), dtype=X.dtype, device=X.device)
+    planes = prod(lead)
+    if planes == 0:
+        return out
+    with torch.cuda.device(X.device):
+        check(_lib.load().spgt_bilinear_align_corners(ptr(X), ptr(out), planes, H_in, W_in, H_out, W_out,
+                                                       stream_of(X)))
+    return out
+
+
+dexts = SimpleNamespace(
+    batched_transpose=_batched_transpose,
+    transpose_gather_dual=_transpose_gather_dual,
+    transpose_scatter_dual=_transpose_scatter_dual,
+    spectral_mode_contract=_spectral_mode_contract,
+    bilinear_align_corners=_bilinear_align_corners,
+)
+
+
+# --------------------------------------------------------------------------- #
+# python surface (autograd-aware; each backward is another of these operators)
+# --------------------------------------------------------------------------- #
+
+class Batched_Transpose_Function(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx: Any, X: Tensor, batch_list: List[int], M_list: List[int], N_list: List[int]):
+        ctx.extras_shape = [batch_list, M_list, N_list]
+        return dexts.batched_transpose(X, batch_list, M_list, N_list)
+
+    @staticmethod
+    def backward(ctx: Any, grad_out: Tensor):
+        batch_list, M_list, N_list = ctx.extras_shape
+        return dexts.batched_transpose(grad_out.contiguous(), batch_list, N_list, M_list), None, None, None
+
+
+class Transpose_Gather_Dual_Function(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx: Any, src: Tensor, dim_list, H_all, W_all, H_low, W_low, H_base_1, W_base_1, H_base_2, W_base_2):
+        ctx.extras_shape = [dim_list, H_all, W_all, H_low, W_low, H_base_1, W_base_1, H_base_2, W_base_2]
+        return dexts.transpose_gather_dual(src, *ctx.extras_shape)
+
+    @staticmethod
+    def backward(ctx: Any, grad_out1: Tensor, grad_out2: Tensor):
+        grad_src = dexts.transpose_scatter_dual(grad_out1.contiguous(), grad_out2.contiguous(), *ctx.extras_shape)
+        return (grad_src,) + (None,) * 9
+
+
+class Transpose_Scatter_Dual_Function(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx: Any, src1: Tensor, src2: Tensor, dim_list, H_all, W_all, H_low, W_low, H_base_1, W_base_1,
+                H_base_2, W_base_2):
+        ctx.extras_shape = [dim_list, H_all, W_all, H_low, W_low, H_base_1, W_base_1, H_base_2, W_base_2]
+        return dexts.transpose_scatter_dual(src1, src2, *ctx.extras_shape)
+
+    @staticmethod
+    def backward(ctx: Any, grad_out: Tensor):
+        g1, g2 = dexts.transpose_gather_dual(grad_out.contiguous(), *ctx.extras_shape)
+        return (g1, g2) + (None,) * 9
+
+
+def batched_transpose(X: Tensor, batch_list: List[int], M_list: List[int], N_list: List[int]) -> Tensor:
+    return Batched_Transpose_Function.apply(X, batch_list, M_list, N_list)
+
+
+def transpose_gather_dual(src: Tensor, dim_list: List[int], H_all, W_all, H_low, W_low, H_base_1, W_base_1, H_base_2,
+                          W_base_2) -> Tuple[Tensor, Tensor]:
+    return Transpose_Gather_Dual_Function.apply(src, dim_list, H_all, W_all, H_low, W_low, H_base_1, W_base_1,
+                                                H_base_2, W_base_2)
+
+
+def transpose_scatter_dual(src1: Tensor, src2: Tensor, dim_list: List[int], H_all, W_all, H_low, W_low, H_base_1,
+                           W_base_1, H_base_2, W_base_2) -> Tensor:
+    return Transpose_Scatter_Dual_Function.apply(src1, src2, dim_list, H_all, W_all, H_low, W_low, H_base_1, W_base_1,
+                                                 H_base_2, W_base_2)
+
+
+def spectral_mode_contract(X_ft: Tensor, weight_1: Tensor, weight_2: Tensor, H_low: int, W_low: int, H_base_1: int,
+                           W_base_1: int, H_base_2: int, W_base_2: int) -> Tensor:
+    """Gather of the two corner windows, per-mode complex channel contraction and scatter
+    into a zero-filled spectrum, in one call (inference only: no autograd graph is recorded)."""
+    return dexts.spectral_mode_contract(X_ft.detach(), weight_1.detach(), weight_2.detach(), H_low, W_low, H_base_1,
+                                        W_base_1, H_base_2, W_base_2)
+
+
+def bilinear_align_corners(X: Tensor, size) -> Tensor:
+    """F.interpolate(X, size, mode='bilinear', align_corners=True) (inference only)."""
+    return dexts.bilinear_align_corners(X.detach(), size)

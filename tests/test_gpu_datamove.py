@@ -1,0 +1,168 @@
+"""Bit-exact parity of the data-movement kernels, and tolerance parity of the
+spectral contraction and bilinear resampling, against the CPU oracle."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from conftest import load_golden, max_rel
+from oracle import spgt_oracle as O
+from spgt_amd import _lib
+from spgt_amd.extension.bind import datamove as dm
+
+pytestmark = pytest.mark.gpu
+
+
+def rnd(*shape, seed=0):
+    return torch.randn(*shape, generator=torch.Generator().manual_seed(seed), dtype=torch.float32)
+
+
+def bits_equal(a, b):
+    ia = torch.view_as_real(a).contiguous().view(torch.int32) if a.is_complex() else a.contiguous().view(torch.int32)
+    ib = torch.view_as_real(b).contiguous().view(torch.int32) if b.is_complex() else b.contiguous().view(torch.int32)
+    return a.shape == b.shape and torch.equal(ia, ib)
+
+
+def special_values(x):
+    """Sprinkles NaN payloads, infinities, -0.0 and denormals into a float tensor."""
+    flat = x.view(-1).view(torch.int32)
+    # quiet NaN with payload, signalling-range NaN, -inf, -0.0, smallest denormal, +inf
+    pats = torch.tensor([0x7FC00001, 0x7FA00000, -0x800000, -0x80000000, 0x00000001, 0x7F800000],
+                        dtype=torch.int64).to(torch.int32)
+    idx = torch.arange(0, flat.numel(), max(1, flat.numel() // 97))
+    flat[idx] = pats[torch.arange(idx.numel()) % pats.numel()]
+    return x
+
+
+@pytest.mark.parametrize("batch,M,N", [([1], [1], [1]), ([2], [3, 5], [7]), ([3], [64], [64]), ([2], [65], [63]),
+                                       ([2, 2], [9, 9], [6]), ([1], [141, 141], [64]), ([4], [64], [71, 71]),
+                                       ([1], [1], [1000]), ([1], [1000], [1])])
+def test_batched_transpose_bit_exact(gpu, batch, M, N):
+    x = special_values(rnd(*batch, *M, *N, seed=1))
+    want = O.op_batched_transpose(x, batch, M, N)
+    got = dm.batched_transpose(x.to(gpu), batch, M, N)
+    assert bits_equal(got.cpu(), want)
+    back = dm.batched_transpose(got, batch, N, M)
+    assert bits_equal(back.cpu(), x)
+
+
+GATHER_CASES = [
+    # dim_list, H_all, W_all, H_low, W_low, hb1, wb1, hb2, wb2
+    ([1], 1, 1, 1, 1, 0, 0, 0, 0),
+    ([2, 3], 6, 4, 2, 3, 0, 0, 4, 1),
+    ([2, 6], 9, 5, 3, 3, 0, 0, 6, 0),
+    ([8, 64], 141, 71, 12, 12, 0, 0, 129, 0),
+    ([3, 65], 20, 11, 5, 7, 2, 1, 15, 4),
+    ([4, 32], 8, 5, 5, 5, 0, 0, 3, 0),  # overlapping windows
+]
+
+
+@pytest.mark.parametrize("case", GATHER_CASES)
+def test_gather_scatter_bit_exact(gpu, case):
+    dim_list, H_all, W_all, H_low, W_low, hb1, wb1, hb2, wb2 = case
+    src = torch.view_as_complex(special_values(rnd(*dim_list, H_all, W_all, 2, seed=2)))
+    w1, w2 = O.op_transpose_gather_dual(src, dim_list, H_all, W_all, H_low, W_low, hb1, wb1, hb2, wb2)
+    g1, g2 = dm.transpose_gather_dual(src.to(gpu), dim_list, H_all, W_all, H_low, W_low, hb1, wb1, hb2, wb2)
+    assert bits_equal(g1.cpu(), w1) and bits_equal(g2.cpu(), w2)
+    a = torch.view_as_complex(special_values(rnd(H_low, W_low, *dim_list, 2, seed=3)))
+    b = torch.view_as_complex(special_values(rnd(H_low, W_low, *dim_list, 2, seed=4)))
+    want = O.op_transpose_scatter_dual(a, b, dim_list, H_all, W_all, H_low, W_low, hb1, wb1, hb2, wb2)
+    got = dm.transpose_scatter_dual(a.to(gpu), b.to(gpu), dim_list, H_all, W_all, H_low, W_low, hb1, wb1, hb2, wb2)
+    assert bits_equal(got.cpu(), want)
+
+
+def test_scatter_of_gather_is_masked_identity(gpu):
+    N, C, r, m = 8, 64, 141, 12
+    src = torch.view_as_complex(rnd(N, C, r, r // 2 + 1, 2, seed=5)).to(gpu)
+    g1, g2 = dm.transpose_gather_dual(src, [N, C], r, r // 2 + 1, m, m, 0, 0, r - m, 0)
+    back = dm.transpose_scatter_dual(g1, g2, [N, C], r, r // 2 + 1, m, m, 0, 0, r - m, 0)
+    mask = torch.zeros(r, r // 2 + 1, dtype=torch.bool, device=gpu)
+    mask[:m, :m] = True
+    mask[r - m:, :m] = True
+    assert torch.equal(torch.view_as_real(back[..., mask]), torch.view_as_real(src[..., mask]))
+    assert (torch.view_as_real(back[..., ~mask]) == 0).all()
+
+
+def test_datamove_autograd(gpu):
+    x = rnd(2, 6, 5, seed=6).to(gpu).requires_grad_(True)
+    y = dm.batched_transpose(x, [2], [6], [5])
+    gy = rnd(2, 5, 6, seed=7).to(gpu)
+    y.backward(gy)
+    assert torch.equal(x.grad, gy.transpose(1, 2))
+    src = torch.view_as_complex(rnd(3, 6, 4, 2, seed=8)).to(gpu).requires_grad_(True)
+    a, b = dm.transpose_gather_dual(src, [3], 6, 4, 2, 3, 0, 0, 4, 1)
+    ga, gb = torch.view_as_complex(rnd(2, 3, 3, 2, seed=9)).to(gpu), torch.view_as_complex(rnd(2, 3, 3, 2, seed=10)).to(gpu)
+    torch.autograd.backward([a, b], [ga, gb])
+    want = O.op_transpose_scatter_dual(ga.cpu(), gb.cpu(), [3], 6, 4, 2, 3, 0, 0, 4, 1)
+    assert bits_equal(src.grad.cpu(), want)
+
+
+@pytest.mark.parametrize("N,Cin,Cout,r,m", [(1, 1, 1, 4, 1), (2, 6, 4, 9, 3), (8, 64, 64, 141, 12), (3, 32, 32, 33, 6),
+                                             (17, 20, 70, 16, 4), (2, 8, 8, 8, 5)])
+def test_spectral_mode_contract_vs_oracle(gpu, N, Cin, Cout, r, m):
+    W_all = r // 2 + 1
+    xf = torch.view_as_complex(rnd(N, Cin, r, W_all, 2, seed=11))
+    w1, w2 = rnd(m, m, Cin, Cout, 2, seed=12) / Cin, rnd(m, m, Cin, Cout, 2, seed=13) / Cin
+    # oracle: the reference's gather -> complex matmul -> scatter sequence, in complex128
+    g1, g2 = O.op_transpose_gather_dual(xf.to(torch.complex128), [N, Cin], r, W_all, m, m, 0, 0, r - m, 0)
+    c = lambda w: torch.view_as_complex(w.double().contiguous())
+    want = O.op_transpose_scatter_dual(g1 @ c(w1), g2 @ c(w2), [N, Cout], r, W_all, m, m, 0, 0, r - m, 0)
+    got = dm.spectral_mode_contract(xf.to(gpu), w1.to(gpu), w2.to(gpu), m, m, 0, 0, r - m, 0)
+    assert got.shape == (N, Cout, r, W_all)
+    inside = want != 0
+    assert (torch.view_as_real(got.cpu())[~inside] == 0).all()
+    assert max_rel(torch.view_as_real(got.cpu()).double(), torch.view_as_real(want)) < 1e-5
+    # and the three-operator sequence on the GPU gives the same numbers
+    a, b = dm.transpose_gather_dual(xf.to(gpu), [N, Cin], r, W_all, m, m, 0, 0, r - m, 0)
+    seq = dm.transpose_scatter_dual(a @ torch.view_as_complex(w1.to(gpu)), b @ torch.view_as_complex(w2.to(gpu)),
+                                    [N, Cout], r, W_all, m, m, 0, 0, r - m, 0)
+    assert max_rel(torch.view_as_real(seq.cpu()).double(), torch.view_as_real(want)) < 1e-5
+
+
+def test_spectral_mode_contract_golden(gpu):
+    """Reference SpectralConv2D fixture: rfft2 / irfft2 by torch on the GPU, the middle by the fused kernel."""
+    p, i, want, meta = load_golden("spectral_conv2d")
+    m = int(meta["mode"])
+    x = i["x"].to(gpu)
+    N, r, _, cin = x.shape
+    w = [p[f"fourier_weight.{k}"].permute(2, 3, 0, 1, 4).contiguous().to(gpu) for k in (0, 1)]  # GT -> Sp layout
+    res = F.linear(x, p["residual_layer.weight"].to(gpu), p["residual_layer.bias"].to(gpu))
+    xt = dm.batched_transpose(x, [N], [r, r], [cin])
+    of = dm.spectral_mode_contract(torch.fft.rfft2(xt, s=(r, r), norm="ortho"), w[0], w[1], m, m, 0, 0, r - m, 0)
+    y = torch.fft.irfft2(of, s=(r, r), norm="ortho")
+    y = dm.batched_transpose(y, [N], [w[0].shape[3]], [r, r])
+    got = F.silu(y + res)
+    assert max_rel(got.cpu(), want) < 1e-4
+
+
+@pytest.mark.parametrize("shape,size", [((2, 3, 7, 9), (7, 9)), ((2, 3, 7, 9), (4, 5)), ((2, 3, 7, 9), (13, 17)),
+                                        ((1, 1, 5, 5), (1, 1)), ((1, 2, 1, 1), (3, 4)), ((4, 128, 211, 211), (122, 122)),
+                                        ((2, 128, 71, 71), (122, 122)), ((1, 3, 2, 300), (5, 301))])
+def test_bilinear_vs_oracle(gpu, shape, size):
+    x = rnd(*shape, seed=14)
+    want = O.bilinear_align_corners(x.double(), size)
+    got = dm.bilinear_align_corners(x.to(gpu), size)
+    assert got.shape == want.shape
+    assert max_rel(got.cpu().double(), want) < 1e-5
+    # torch's own fp32 kernel rounds the source coordinates differently; both sit within
+    # ~1e-5 of the fp64 result, so they are compared at the path's stated 1e-4 tolerance
+    lib = F.interpolate(x, size=size, mode="bilinear", align_corners=True)
+    assert max_rel(got.cpu(), lib) < 1e-4
+
+
+def test_bilinear_closed_forms(gpu):
+    x = rnd(2, 3, 7, 9, seed=15).to(gpu)
+    assert torch.equal(dm.bilinear_align_corners(x, (7, 9)), x)  # identity when sizes agree
+    y = dm.bilinear_align_corners(x, (13, 17))
+    assert torch.equal(y[..., 0, 0], x[..., 0, 0])
+    assert torch.allclose(y[..., -1, -1], x[..., -1, -1], rtol=1e-6)
+
+
+def test_datamove_argument_validation(gpu):
+    lib = _lib.load()
+    x = torch.zeros(4, 4, device=gpu)
+    assert lib.spgt_batched_transpose(_lib.ptr(x), _lib.ptr(x), 1, 4, 4, None) == -1
+    c = torch.zeros(2, 4, 4, dtype=torch.complex64, device=gpu)
+    with pytest.raises(_lib.SpgtError):
+        dm.transpose_gather_dual(c, [2], 4, 4, 3, 3, 0, 0, 2, 0)  # second window leaves the plane
+    with pytest.raises(TypeError):
+        dm.batched_transpose(x.double(), [1], [4], [4])
