@@ -49,6 +49,27 @@ const char* spgt_last_error(void);
 
 /* ---- Galerkin attention ------------------------------------------------ */
 
+/* Replaces multihead_projection_with_position_rrc_forward
+ * (extension/bind/galerkin_attention.cu:9-24; same argument order, output passed in).
+ *   input [batch, seqlen, dim_hidden], weight [dim_hidden, dim_hidden] used as stored
+ *   (x @ W), bias [dim_hidden], position [batch, seqlen, dim_position] or NULL,
+ *   out [batch, num_head, dim_position + dim_head, seqlen].
+ * dim_head must be 32, dim_hidden 128 or 256, dim_position 0 or 2. */
+int spgt_multihead_projection_with_position_rrc_forward(
+    const float* input, const float* weight, const float* bias, const float* position, float* out,
+    int seqlen, int dim_hidden, int num_head, int dim_head, int dim_position, int batch,
+    spgt_stream_t stream);
+
+/* Replaces multihead_projection_layernorm_with_position_rrc_forward
+ * (extension/bind/galerkin_attention.cu:50-68): the projection above followed, per token
+ * and head, by LayerNorm over the 32 head features with affine ln_weight/ln_bias
+ * [num_head, 32]; also writes invsigma [batch, num_head, seqlen] = 1/sqrt(var + eps). */
+int spgt_multihead_projection_layernorm_with_position_rrc_forward(
+    const float* input, const float* weight, const float* bias, const float* ln_weight,
+    const float* ln_bias, float norm_eps, const float* position, float* out, float* invsigma,
+    int seqlen, int dim_hidden, int num_head, int dim_head, int dim_position, int batch,
+    spgt_stream_t stream);
+
 /* Replaces multihead_galerkin_attention_cccr_forward
  * (extension/bind/galerkin_attention.cu:104-124).
  *   Q, K, V : [batch, num_head, d_posk, seqlen]  (feature-major, seqlen contiguous)

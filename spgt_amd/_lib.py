@@ -23,6 +23,9 @@ _p = ctypes.c_void_p
 SIGNATURES = {
     "spgt_version": (_i, []),
     "spgt_last_error": (ctypes.c_char_p, []),
+    "spgt_multihead_projection_with_position_rrc_forward": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p]),
+    "spgt_multihead_projection_layernorm_with_position_rrc_forward": (
+        _i, [_p, _p, _p, _p, _p, _f, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p]),
     "spgt_galerkin_attention_cccr_workspace_bytes": (_sz, [_i, _i, _i, _i]),
     "spgt_galerkin_attention_cccr_forward": (_i, [_p, _p, _p, _p, _p, _sz, _i, _i, _i, _i, _p]),
     "spgt_batched_skinny_gemm_workspace_bytes": (_sz, [_i, _i, _i, _i]),

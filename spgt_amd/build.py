@@ -16,6 +16,7 @@ SOURCES = [
     "spgt_host.cpp",
     "attn_fused.hip",
     "attn_cccr.hip",
+    "projection.hip",
     "datamove.hip",
     "spectral.hip",
 ]

@@ -1,0 +1,210 @@
+// Multi-head projection with bias, optional per-head LayerNorm and position
+// rows, written feature-major:
+//   out[b, h, dp + j, s] = sum_k x[b, s, k] * W[k, h*32 + j] + bias[h*32 + j]
+//   out[b, h, 0:dp, s]   = position[b, s, 0:dp]
+// and, for the LayerNorm variant, each (b, h, s) column of 32 features is
+// normalised (biased variance, eps under the root) and scaled by the head's
+// affine before it is stored; invsigma[b, h, s] = 1 / sqrt(var + eps).
+//
+// Reference behaviour restated here:
+//   multihead_projection_with_position_rrc_forward            extension/bind/galerkin_attention.cu:9-24
+//   multihead_projection_layernorm_with_position_rrc_forward  extension/bind/galerkin_attention.cu:50-68
+//   mh32::sgemm_rrc_cuda and its kernels                      extension/native/multihead_dim32.cu:6-146, 490-599
+// The weight is used as stored, x @ W (multihead_dim32.cu:343-344).
+//
+// One wave owns one head.  Its 32 weight columns W[:, h*32 .. h*32+31] stay in
+// registers for the whole kernel as the MFMA A operand (feature x k), token
+// tiles of x go through LDS once (coalesced 512-byte rows in, k-strided reads
+// out as the B operand), so the 32x32 accumulator holds features along rows
+// and 32 consecutive tokens along lanes: stores run along the contiguous
+// sequence axis, and a token's 32 features sit in two lanes x 16 registers,
+// which makes the LayerNorm statistics an in-register sum plus one lane swap.
+#include "spgt_device.h"
+#include "spgt_host.h"
+
+namespace spgt {
+
+// grid (nchunk, H/4, B), block 256.  KC = dim_hidden / 128.
+template <int KC, int DP, bool LN>
+__global__ __launch_bounds__(256) void projection_rrc_k(
+    const float* __restrict__ x, const float* __restrict__ W, const float* __restrict__ bias,
+    const float* __restrict__ lnw, const float* __restrict__ lnb, const float* __restrict__ pos,
+    float* __restrict__ out, float* __restrict__ invsigma, int S, int H, float eps, int tokens_per_chunk) {
+    constexpr int K = 128 * KC;
+    constexpr int D = DP + 32;
+    constexpr int PITCH = K + 1;
+    extern __shared__ float xs[];  // [64][PITCH]
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int h = blockIdx.y * 4 + wave;
+    const int b = blockIdx.z;
+    const int tk = lane & 31;
+    const int kh = lane >> 5;
+    const int s_begin = blockIdx.x * tokens_per_chunk;
+    const int s_end = min(S, s_begin + tokens_per_chunk);
+
+    // A operand: W[2kk + kh][h*32 + tk]
+    float wreg[K / 2];
+#pragma unroll
+    for (int kk = 0; kk < K / 2; ++kk) wreg[kk] = W[(int64_t)(2 * kk + kh) * K + h * 32 + tk];
+    // accumulator element r holds feature i(r) = 8*(r/4) + 4*kh + r%4
+    float breg[16], greg[16], oreg[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const int i = 8 * (r >> 2) + 4 * kh + (r & 3);
+        breg[r] = bias[h * 32 + i];
+        if (LN) {
+            greg[r] = lnw[h * 32 + i];
+            oreg[r] = lnb[h * 32 + i];
+        }
+    }
+
+    const float* xb = x + (int64_t)b * S * K;
+    float* ob = out + ((int64_t)b * H + h) * D * S;
+    constexpr int NLD = K / 16;  // float4 loads per thread per tile (64*K/4 / 256)
+    float4 stage[NLD];
+    auto load_tile = [&](int s0) {
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) {
+            const int e = threadIdx.x + 256 * i;
+            const int row = e / (K / 4);
+            const int c4 = e % (K / 4);
+            const int s = s0 + row;
+            stage[i] = (s < s_end) ? *reinterpret_cast<const float4*>(xb + (int64_t)s * K + 4 * c4)
+                                   : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    };
+    auto store_tile = [&]() {
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) {
+            const int e = threadIdx.x + 256 * i;
+            const int row = e / (K / 4);
+            const int c4 = e % (K / 4);
+            float* d = xs + row * PITCH + 4 * c4;
+            d[0] = stage[i].x; d[1] = stage[i].y; d[2] = stage[i].z; d[3] = stage[i].w;
+        }
+    };
+
+    if (s_begin < s_end) load_tile(s_begin);
+    for (int s0 = s_begin; s0 < s_end; s0 += 64) {
+        __syncthreads();  // previous tile fully consumed
+        store_tile();
+        __syncthreads();
+        if (s0 + 64 < s_end) load_tile(s0 + 64);
+#pragma unroll
+        for (int tb = 0; tb < 2; ++tb) {
+            v16f acc;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+            const float* xr = xs + (tb * 32 + tk) * PITCH + kh;
+#pragma unroll
+            for (int kk = 0; kk < K / 2; ++kk) acc = mfma32(wreg[kk], xr[2 * kk], acc);
+            const int s = s0 + tb * 32 + tk;
+            float y[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) y[r] = acc[r] + breg[r];
+            if (LN) {
+                float sum = 0.f;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) sum += y[r];
+                sum += __shfl_xor(sum, 32, 64);
+                const float mean = sum * (1.0f / 32.0f);
+                float ss = 0.f;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    y[r] -= mean;
+                    ss = fmaf(y[r], y[r], ss);
+                }
+                ss += __shfl_xor(ss, 32, 64);
+                const float rstd = __builtin_amdgcn_rsqf(fmaf(ss, 1.0f / 32.0f, eps));
+#pragma unroll
+                for (int r = 0; r < 16; ++r) y[r] = fmaf(y[r] * rstd, greg[r], oreg[r]);
+                if (kh == 0 && s < s_end) invsigma[((int64_t)b * H + h) * S + s] = rstd;
+            }
+            if (s < s_end) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int i = 8 * (r >> 2) + 4 * kh + (r & 3);
+                    ob[(int64_t)(DP + i) * S + s] = y[r];
+                }
+                if (DP == 2) ob[(int64_t)kh * S + s] = pos[((int64_t)b * S + s) * 2 + kh];
+            }
+        }
+    }
+}
+
+namespace {
+
+template <int KC, int DP, bool LN>
+void launch_projection(const float* x, const float* W, const float* bias, const float* lnw, const float* lnb,
+                       const float* pos, float* out, float* invsigma, int B, int S, int H, float eps,
+                       hipStream_t stream) {
+    constexpr int K = 128 * KC;
+    const size_t lds = (size_t)64 * (K + 1) * sizeof(float);
+    // about two workgroups per CU; chunks are whole 64-token tiles
+    const int per_b = std::max(1, 512 / std::max(1, B * (H / 4)));
+    const int tpc = std::max(64, ceil_div(ceil_div(S, per_b), 64) * 64);
+    const dim3 grid(ceil_div(S, tpc), H / 4, B);
+    auto kernel = projection_rrc_k<KC, DP, LN>;
+    if (lds > 64 * 1024)
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  (int)lds);
+    hipLaunchKernelGGL(kernel, grid, dim3(256), lds, stream, x, W, bias, lnw, lnb, pos, out, invsigma, S, H, eps, tpc);
+}
+
+int projection_common(const char* who, const float* input, const float* weight, const float* bias,
+                      const float* ln_weight, const float* ln_bias, float norm_eps, const float* position, float* out,
+                      float* invsigma, int batch, int seqlen, int dim_hidden, int num_head, int dim_head,
+                      int dim_position, bool ln, hipStream_t stream) {
+    if (!input || !weight || !bias || !out || (ln && (!ln_weight || !ln_bias || !invsigma)))
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "multihead_projection: null pointer argument");
+    if (batch <= 0 || seqlen <= 0) return fail(SPGT_ERR_INVALID_ARGUMENT, "multihead_projection: batch and seqlen must be positive");
+    if (dim_head != 32 || num_head * dim_head != dim_hidden)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "multihead_projection: dim_head must be 32 and num_head*32 == dim_hidden");
+    if (dim_hidden != 128 && dim_hidden != 256)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "multihead_projection: dim_hidden must be 128 or 256");
+    if (dim_position != 0 && dim_position != 2)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "multihead_projection: dim_position must be 0 or 2");
+    if (dim_position == 2 && !position)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "multihead_projection: position is null with dim_position 2");
+    if (batch > 65535) return fail(SPGT_ERR_INVALID_ARGUMENT, "multihead_projection: batch exceeds 65535");
+    if (!aligned16(input) || !aligned4(weight) || !aligned4(bias) || !aligned4(out))
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "multihead_projection: input must be 16-byte aligned");
+    const float* pos = position ? position : input;
+    const int kc = dim_hidden / 128;
+#define SPGT_PROJ(KC, DP, LNF)                                                                                   \
+    launch_projection<KC, DP, LNF>(input, weight, bias, ln_weight, ln_bias, pos, out, invsigma, batch, seqlen, \
+                                   num_head, norm_eps, stream)
+    if (kc == 1) {
+        if (ln) { if (dim_position) SPGT_PROJ(1, 2, true); else SPGT_PROJ(1, 0, true); }
+        else    { if (dim_position) SPGT_PROJ(1, 2, false); else SPGT_PROJ(1, 0, false); }
+    } else {
+        if (ln) { if (dim_position) SPGT_PROJ(2, 2, true); else SPGT_PROJ(2, 0, true); }
+        else    { if (dim_position) SPGT_PROJ(2, 2, false); else SPGT_PROJ(2, 0, false); }
+    }
+#undef SPGT_PROJ
+    return check_launch(who);
+}
+
+}  // namespace
+
+}  // namespace spgt
+
+using namespace spgt;
+
+extern "C" int spgt_multihead_projection_with_position_rrc_forward(
+    const float* input, const float* weight, const float* bias, const float* position, float* out, int seqlen,
+    int dim_hidden, int num_head, int dim_head, int dim_position, int batch, hipStream_t stream) {
+    return projection_common("multihead_projection_with_position_rrc_forward", input, weight, bias, nullptr, nullptr,
+                             0.f, position, out, nullptr, batch, seqlen, dim_hidden, num_head, dim_head, dim_position,
+                             false, stream);
+}
+
+extern "C" int spgt_multihead_projection_layernorm_with_position_rrc_forward(
+    const float* input, const float* weight, const float* bias, const float* ln_weight, const float* ln_bias,
+    float norm_eps, const float* position, float* out, float* invsigma, int seqlen, int dim_hidden, int num_head,
+    int dim_head, int dim_position, int batch, hipStream_t stream) {
+    return projection_common("multihead_projection_layernorm_with_position_rrc_forward", input, weight, bias,
+                             ln_weight, ln_bias, norm_eps, position, out, invsigma, batch, seqlen, dim_hidden, num_head,
+                             dim_head, dim_position, true, stream);
+}

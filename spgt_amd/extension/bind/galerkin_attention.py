@@ -21,6 +21,55 @@ GEMM_ORDER = {"RRR": 0, "RRC": 1, "RCR": 2, "RCC": 3, "CRR": 4, "CRC": 5, "CCR":
 # `gexts` surface: plain functions on tensors, no autograd
 # --------------------------------------------------------------------------- #
 
+def _check_projection_args(input, weight, bias, position, seqlen, dim_hidden, num_head, dim_head, dim_position, batch):
+    require_gpu_f32("input", input)
+    require_gpu_f32("weight", weight)
+    require_gpu_f32("bias", bias)
+    if tuple(input.shape) != (batch, seqlen, dim_hidden):
+        raise ValueError(f"input has shape {tuple(input.shape)}, expected {(batch, seqlen, dim_hidden)}")
+    if tuple(weight.shape) != (dim_hidden, dim_hidden) or bias.numel() != dim_hidden:
+        raise ValueError("weight must be [dim_hidden, dim_hidden] and bias [dim_hidden]")
+    if num_head * dim_head != dim_hidden:
+        raise ValueError("num_head * dim_head must equal dim_hidden")
+    if dim_position:
+        require_gpu_f32("position", position)
+        if tuple(position.shape) != (batch, seqlen, dim_position):
+            raise ValueError(f"position has shape {tuple(position.shape)}, expected {(batch, seqlen, dim_position)}")
+
+
+def _projection_forward(input: Tensor, weight: Tensor, bias: Tensor, position: Tensor, seqlen: int, dim_hidden: int,
+                        num_head: int, dim_head: int, dim_position: int, batch: int) -> Tensor:
+    """x @ W + b split into heads, position rows first -> [batch, num_head, dim_position + dim_head, seqlen]
+    (reference: extension/bind/galerkin_attention.cu:9-24)."""
+    _check_projection_args(input, weight, bias, position, seqlen, dim_hidden, num_head, dim_head, dim_position, batch)
+    out = torch.empty((batch, num_head, dim_position + dim_head, seqlen), dtype=input.dtype, device=input.device)
+    with torch.cuda.device(input.device):
+        check(_lib.load().spgt_multihead_projection_with_position_rrc_forward(
+            ptr(input), ptr(weight), ptr(bias), ptr(position) if dim_position else None, ptr(out), seqlen, dim_hidden,
+            num_head, dim_head, dim_position, batch, stream_of(input)))
+    return out
+
+
+def _projection_layernorm_forward(input: Tensor, weight: Tensor, bias: Tensor, lnw: Tensor, lnb: Tensor,
+                                  norm_eps: float, position: Tensor, seqlen: int, dim_hidden: int, num_head: int,
+                                  dim_head: int, dim_position: int, batch: int):
+    """As above with per-head LayerNorm; returns (hat_ln, invsigma [batch, num_head, seqlen])
+    (reference: extension/bind/galerkin_attention.cu:50-68)."""
+    _check_projection_args(input, weight, bias, position, seqlen, dim_hidden, num_head, dim_head, dim_position, batch)
+    require_gpu_f32("lnw", lnw)
+    require_gpu_f32("lnb", lnb)
+    if lnw.numel() != dim_hidden or lnb.numel() != dim_hidden:
+        raise ValueError("LayerNorm weight and bias must be [num_head, dim_head]")
+    hat_ln = torch.empty((batch, num_head, dim_position + dim_head, seqlen), dtype=input.dtype, device=input.device)
+    invsigma = torch.empty((batch, num_head, seqlen), dtype=input.dtype, device=input.device)
+    with torch.cuda.device(input.device):
+        check(_lib.load().spgt_multihead_projection_layernorm_with_position_rrc_forward(
+            ptr(input), ptr(weight), ptr(bias), ptr(lnw), ptr(lnb), float(norm_eps),
+            ptr(position) if dim_position else None, ptr(hat_ln), ptr(invsigma), seqlen, dim_hidden, num_head,
+            dim_head, dim_position, batch, stream_of(input)))
+    return hat_ln, invsigma
+
+
 def _attention_cccr_forward(Q: Tensor, K: Tensor, V: Tensor, batch: int, num_head: int, d_posk: int,
                             seqlen: int) -> Tensor:
     """Q, K, V [batch, num_head, d_posk, seqlen] -> [batch, num_head, seqlen, d_posk]
@@ -137,6 +186,8 @@ def _attention_fused_profile(Q, K, V, position, ln_weight_K, ln_bias_K, ln_weigh
 
 
 gexts = SimpleNamespace(
+    multihead_projection_with_position_rrc_forward=_projection_forward,
+    multihead_projection_layernorm_with_position_rrc_forward=_projection_layernorm_forward,
     galerkin_attention_fused_profile=_attention_fused_profile,
     multihead_galerkin_attention_cccr_forward=_attention_cccr_forward,
     batched_skinny_gemm=_batched_skinny_gemm,
@@ -147,6 +198,40 @@ gexts = SimpleNamespace(
 # --------------------------------------------------------------------------- #
 # python surface
 # --------------------------------------------------------------------------- #
+
+class Multihead_Porjection_with_Position_Function(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx: Any, input: Tensor, weight: Tensor, bias: Tensor, position: Tensor, num_head, dim_head,
+                dim_position):
+        batch, seqlen, d_model = input.size()
+        out = gexts.multihead_projection_with_position_rrc_forward(
+            input, weight, bias, position, seqlen, d_model, num_head, dim_head, dim_position, batch)
+        ctx.save_for_backward(input, weight)
+        ctx.shape_kwargs = [num_head, dim_head, dim_position]
+        return out
+
+    @staticmethod
+    def backward(ctx: Any, grad_out: Tensor):
+        raise NotImplementedError("backward of multihead_projection_with_position_rrc_cuda is not built yet")
+
+
+class Multihead_Porjection_Layernorm_with_Position_Function(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx: Any, input: Tensor, weight: Tensor, bias: Tensor, lnw: Tensor, lnb: Tensor, position: Tensor,
+                norm_eps: float, num_head, dim_head, dim_position):
+        batch, seqlen, d_model = input.size()
+        hat_ln, invsigma = gexts.multihead_projection_layernorm_with_position_rrc_forward(
+            input, weight, bias, lnw, lnb, norm_eps, position, seqlen, d_model, num_head, dim_head, dim_position,
+            batch)
+        ctx.save_for_backward(input, weight, hat_ln, invsigma, lnw, lnb)
+        ctx.shape_kwargs = [num_head, dim_head, dim_position]
+        return hat_ln
+
+    @staticmethod
+    def backward(ctx: Any, grad_ln: Tensor):
+        raise NotImplementedError(
+            "backward of multihead_projection_layernorm_with_position_rrc_cuda is not built yet")
+
 
 class Multihead_Galerkin_Attention_cccr_Function(torch.autograd.Function):
     @staticmethod
@@ -159,6 +244,21 @@ class Multihead_Galerkin_Attention_cccr_Function(torch.autograd.Function):
     @staticmethod
     def backward(ctx: Any, grad_Attn):
         raise NotImplementedError("backward of multihead_galerkin_attention_cccr_cuda is not built yet")
+
+
+def multihead_projection_with_position_rrc_cuda(input: Tensor, weight: Tensor, bias: Tensor, position: Tensor,
+                                                num_head, dim_head, dim_position) -> Tensor:
+    """[B, S, Dm] -> [B, H, dim_position + dim_head, S]: (x @ W + b) per head, position rows first."""
+    return Multihead_Porjection_with_Position_Function.apply(input, weight, bias, position, num_head, dim_head,
+                                                             dim_position)
+
+
+def multihead_projection_layernorm_with_position_rrc_cuda(input: Tensor, weight: Tensor, bias: Tensor,
+                                                          ln_weight: Tensor, ln_bias: Tensor, position: Tensor,
+                                                          norm_eps, num_head, dim_head, dim_position) -> Tensor:
+    """As above with each head LayerNorm'ed over its dim_head features."""
+    return Multihead_Porjection_Layernorm_with_Position_Function.apply(
+        input, weight, bias, ln_weight, ln_bias, position, norm_eps, num_head, dim_head, dim_position)
 
 
 def multihead_galerkin_attention_cccr_cuda(Q: Tensor, K: Tensor, V: Tensor) -> Tensor:

@@ -1,0 +1,60 @@
+"""Down- and up-scalers around the encoder: 3x3 convolutions (library) with
+bilinear align_corners resampling (this package's HIP kernel when no autograd
+graph is needed).  Structure, parameter names and shapes follow the
+reference's network/model.py:7-39 (DownScaler2D) and :42-65 (UpScaler2D).
+"""
+import torch
+import torch.nn.functional as F
+from torch import Tensor, nn
+
+from ..extension.bind.datamove import bilinear_align_corners
+from .layer import ConvResBlock2D, always_dropout, make_activation
+
+
+def resample(X: Tensor, size) -> Tensor:
+    """Bilinear, align_corners=True, on [N, C, H, W]."""
+    if torch.is_grad_enabled() and X.requires_grad:
+        return F.interpolate(X, size=tuple(size), mode="bilinear", align_corners=True)
+    return bilinear_align_corners(X.contiguous(), tuple(size))
+
+
+class DownScaler2D(nn.Module):
+    """[N, r, r, in_dim] -> [N, r_attn, r_attn, out_dim] in two resampling steps; the three
+    stacked convolutions after the first step are concatenated along channels."""
+
+    def __init__(self, resolution_size, in_dim, out_dim, droprate, activation) -> None:
+        super().__init__()
+        self.resolution_size = resolution_size
+        d1 = d2 = out_dim // 3
+        d3 = out_dim - d1 - d2
+        self.conv0 = ConvResBlock2D(in_dim, out_dim, 3, 1, droprate, activation)
+        self.conv1 = ConvResBlock2D(out_dim, d1, 3, 1, droprate, activation)
+        self.conv2 = ConvResBlock2D(d1, d2, 3, 1, droprate, activation)
+        self.conv3 = ConvResBlock2D(d2, d3, 3, 1, droprate, activation)
+        self.activation_layer = make_activation(activation)
+
+    def forward(self, X: Tensor) -> Tensor:
+        X = self.conv0(X.permute(0, 3, 1, 2))
+        X = self.activation_layer(resample(X, self.resolution_size[1]))
+        X1 = self.conv1(X)
+        X2 = self.conv2(X1)
+        X3 = self.conv3(X2)
+        X = self.activation_layer(resample(torch.cat([X1, X2, X3], dim=1), self.resolution_size[2]))
+        return X.permute(0, 2, 3, 1)
+
+
+class UpScaler2D(nn.Module):
+    """[N, r_attn, r_attn, in_dim] -> [N, r, r, out_dim]: resample, conv block, activation (again), resample."""
+
+    def __init__(self, resolution_size, in_dim, out_dim, droprate, activation) -> None:
+        super().__init__()
+        self.resolution_size = resolution_size
+        self.droprate = droprate
+        self.conv = ConvResBlock2D(in_dim, out_dim, 3, 1, droprate, activation)
+        self.activation_layer = make_activation(activation)
+
+    def forward(self, X: Tensor) -> Tensor:
+        X = resample(X.permute(0, 3, 1, 2), self.resolution_size[3])
+        X = self.activation_layer(always_dropout(self.conv(X), self.droprate))
+        X = resample(X, self.resolution_size[4])
+        return X.permute(0, 2, 3, 1)

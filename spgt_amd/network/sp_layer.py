@@ -1,0 +1,173 @@
+"""Accelerated layers: Galerkin attention, encoder layer, FNO spectral
+convolution.  Class names, constructor arguments, parameter names and shapes
+follow the reference's network/sp_layer.py (Sp_GalerkinAttention :12-78,
+Sp_EncoderLayer :81-104, Sp_SpectralConv2D :107-156), so a checkpoint of the
+reference's accelerated model loads unchanged and gives the same outputs.
+
+Two conventions of the reference are kept on purpose:
+  * the projections multiply by the weight as stored, x @ W + b (its CUDA
+    kernel, extension/native/multihead_dim32.cu:343-344), whereas the plain
+    PyTorch model computes x @ W^T + b; `convert_gt_state_dict` maps a
+    checkpoint of the plain model onto these modules;
+  * F.dropout runs with training=True whenever a drop rate is non-zero.
+
+Without autograd (inference) the layers take the fused kernels: one GEMM for
+the three projections, then LayerNorm + K^T V / S + Q (K^T V / S) in one call
+on token-major data; the spectral layer contracts the retained modes straight
+out of and into the full spectrum.  With autograd they run the reference's
+operator sequence.
+"""
+import math
+from typing import Dict
+
+import torch
+import torch.nn.functional as F
+from torch import Tensor, nn
+
+from ..extension.bind.datamove import (batched_transpose, spectral_mode_contract, transpose_gather_dual,
+                                       transpose_scatter_dual)
+from ..extension.bind.galerkin_attention import (galerkin_attention_fused, multihead_galerkin_attention_cccr_cuda,
+                                                 multihead_projection_layernorm_with_position_rrc_cuda,
+                                                 multihead_projection_with_position_rrc_cuda)
+from .layer import FeedForward, always_dropout, make_activation
+
+
+class Sp_GalerkinAttention(nn.Module):
+    def __init__(self, dim_hidden, num_head, dim_position, norm_eps, attn_droprate, fc_droprate, xavier, diagonal,
+                 symmetric) -> None:
+        super().__init__()
+        assert dim_hidden % 128 == 0 and dim_hidden // num_head == 32
+        self.dim_hidden = dim_hidden
+        self.num_head = num_head
+        self.dim_head = dim_hidden // num_head
+        self.dim_position = dim_position
+        self.norm_eps = norm_eps
+        self.attn_droprate = attn_droprate  # accepted and, as in the reference's accelerated layer, unused
+        self.fc_droprate = fc_droprate
+        for n in "QKV":
+            setattr(self, f"weight_{n}", nn.Parameter(torch.empty(dim_hidden, dim_hidden)))
+        for n in "QKV":
+            setattr(self, f"bias_{n}", nn.Parameter(torch.empty(dim_hidden)))
+        for kind in ("weight", "bias"):
+            for n in "KV":
+                setattr(self, f"ln_{kind}_{n}", nn.Parameter(torch.empty(num_head, self.dim_head)))
+        self.fc_layer = nn.Linear(dim_hidden + dim_position * num_head, dim_hidden)
+        self._reset_parameters(xavier, diagonal, symmetric)
+        self._qkv_cache = None
+
+    def _reset_parameters(self, xavier, diagonal, symmetric) -> None:
+        with torch.no_grad():
+            for w in (self.weight_Q, self.weight_K, self.weight_V):
+                nn.init.xavier_uniform_(w, gain=xavier)
+                if diagonal > 0:
+                    w += diagonal * torch.eye(w.size(-1))
+                if symmetric:
+                    w += w.T.clone()
+            for b in (self.bias_Q, self.bias_K, self.bias_V, self.ln_bias_K, self.ln_bias_V):
+                b.zero_()
+            for g in (self.ln_weight_K, self.ln_weight_V):
+                g.fill_(1.0)
+
+    def _packed_qkv(self):
+        """[W_Q | W_K | W_V] (dim_hidden x 3 dim_hidden) and the packed bias, rebuilt when a parameter changes."""
+        ps = (self.weight_Q, self.weight_K, self.weight_V, self.bias_Q, self.bias_K, self.bias_V)
+        key = tuple((p.data_ptr(), p._version) for p in ps)
+        if self._qkv_cache is None or self._qkv_cache[0] != key:
+            with torch.no_grad():
+                self._qkv_cache = (key, torch.cat(ps[:3], dim=1).contiguous(), torch.cat(ps[3:]).contiguous())
+        return self._qkv_cache[1], self._qkv_cache[2]
+
+    def _needs_graph(self, *tensors) -> bool:
+        return torch.is_grad_enabled() and (any(t.requires_grad for t in tensors) or
+                                            any(p.requires_grad for p in self.parameters()))
+
+    def forward(self, Q: Tensor, K: Tensor, V: Tensor, position: Tensor) -> Tensor:
+        """Q, K, V [N, seqlen, dim_hidden], position [N, seqlen, dim_position] -> [N, seqlen, dim_hidden]."""
+        N, seqlen, C = Q.size()
+        H, dp = self.num_head, self.dim_position
+        if self._needs_graph(Q, K, V):
+            q = multihead_projection_with_position_rrc_cuda(Q, self.weight_Q, self.bias_Q, position, H, self.dim_head, dp)
+            k = multihead_projection_layernorm_with_position_rrc_cuda(
+                K, self.weight_K, self.bias_K, self.ln_weight_K, self.ln_bias_K, position, self.norm_eps, H,
+                self.dim_head, dp)
+            v = multihead_projection_layernorm_with_position_rrc_cuda(
+                V, self.weight_V, self.bias_V, self.ln_weight_V, self.ln_bias_V, position, self.norm_eps, H,
+                self.dim_head, dp)
+            X = multihead_galerkin_attention_cccr_cuda(q, k, v)
+            X = X.transpose(1, 2).contiguous().view(N, seqlen, H * (dp + self.dim_head))
+        else:
+            if Q is K and K is V:
+                w, b = self._packed_qkv()
+                qkv = torch.addmm(b, Q.reshape(N * seqlen, C), w).view(N, seqlen, 3 * C)
+                q, k, v = qkv[..., :C], qkv[..., C:2 * C], qkv[..., 2 * C:]
+            else:
+                proj = lambda x, w, b: torch.addmm(b, x.reshape(N * seqlen, C), w).view(N, seqlen, C)
+                q, k, v = (proj(Q, self.weight_Q, self.bias_Q), proj(K, self.weight_K, self.bias_K),
+                           proj(V, self.weight_V, self.bias_V))
+            pos = position.contiguous() if dp else None
+            X = galerkin_attention_fused(q, k, v, pos, self.ln_weight_K.detach(), self.ln_bias_K.detach(),
+                                         self.ln_weight_V.detach(), self.ln_bias_V.detach(), self.norm_eps, H, dp)
+        return always_dropout(self.fc_layer(X), self.fc_droprate)
+
+
+class Sp_EncoderLayer(nn.Module):
+    """x + attention(x); then x + ffn(x).  No normalisation on the residual stream."""
+
+    def __init__(self, dim_hidden, num_head, dim_position, norm_eps, attn_droprate, fc_droprate, xavier, diagonal,
+                 symmetric, ffn_dim_hidden, ffn_droprate, ffn_activation) -> None:
+        super().__init__()
+        self.attention_layer = Sp_GalerkinAttention(dim_hidden, num_head, dim_position, norm_eps, attn_droprate,
+                                                    fc_droprate, xavier, diagonal, symmetric)
+        self.ffn_layer = FeedForward(dim_hidden, dim_hidden, ffn_dim_hidden, ffn_droprate, ffn_activation)
+
+    def forward(self, X: Tensor, position: Tensor) -> Tensor:
+        X = X + self.attention_layer(X, X, X, position)
+        return X + self.ffn_layer(X)
+
+
+class Sp_SpectralConv2D(nn.Module):
+    def __init__(self, in_dim, out_dim, mode, droprate, activation) -> None:
+        super().__init__()
+        self.in_dim, self.out_dim, self.mode, self.droprate = in_dim, out_dim, mode, droprate
+        self.activation_layer = make_activation(activation)
+        self.residual_layer = nn.Linear(in_dim, out_dim)
+        # real pairs rather than complex64 (the reference's choice: its collective backend lacks complex types)
+        self.fourier_weight = nn.ParameterList(
+            [nn.Parameter(torch.empty(mode, mode, in_dim, out_dim, 2)) for _ in range(2)])
+        for w in self.fourier_weight:
+            nn.init.xavier_normal_(w, gain=1.0 / (in_dim * out_dim) * math.sqrt(in_dim + out_dim))
+
+    def forward(self, X: Tensor) -> Tensor:
+        """[N, r, r, in_dim] -> [N, r, r, out_dim]."""
+        N, r, _, cin = X.size()
+        m, cout = self.mode, self.out_dim
+        res = self.residual_layer(X)
+        X = always_dropout(X, self.droprate)
+        X = batched_transpose(X, [N], [r, r], [cin])  # -> [N, in_dim, r, r]
+        X_ft = torch.fft.rfft2(X, s=(r, r), norm="ortho")
+        w_all = r // 2 + 1
+        if torch.is_grad_enabled() and (X.requires_grad or self.fourier_weight[0].requires_grad):
+            g0, g1 = transpose_gather_dual(X_ft, [N, cin], r, w_all, m, m, 0, 0, r - m, 0)
+            o0 = g0 @ torch.view_as_complex(self.fourier_weight[0])
+            o1 = g1 @ torch.view_as_complex(self.fourier_weight[1])
+            Out_ft = transpose_scatter_dual(o0, o1, [N, cout], r, w_all, m, m, 0, 0, r - m, 0)
+        else:
+            Out_ft = spectral_mode_contract(X_ft, self.fourier_weight[0], self.fourier_weight[1], m, m, 0, 0, r - m, 0)
+        X = torch.fft.irfft2(Out_ft, s=(r, r), norm="ortho")
+        X = batched_transpose(X, [N], [cout], [r, r])  # -> [N, r, r, out_dim]
+        return self.activation_layer(X + res)
+
+
+def convert_gt_state_dict(state_dict: Dict[str, Tensor]) -> Dict[str, Tensor]:
+    """Maps a state_dict of the reference's plain-PyTorch model (or of any of its sub-modules) onto the
+    accelerated modules: projection weights are transposed (x @ W^T there, x @ W here) and Fourier weights
+    go from [Cin, Cout, m, m, 2] (network/layer.py:214-216) to [m, m, Cin, Cout, 2] (network/sp_layer.py:119-121)."""
+    out = {}
+    for k, v in state_dict.items():
+        leaf = k.rsplit(".", 1)[-1]
+        if leaf in ("weight_Q", "weight_K", "weight_V"):
+            v = v.t().contiguous()
+        elif ".fourier_weight." in "." + k and v.dim() == 5:
+            v = v.permute(2, 3, 0, 1, 4).contiguous()
+        out[k] = v
+    return out

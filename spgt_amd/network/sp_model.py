@@ -1,0 +1,94 @@
+"""Accelerated Galerkin Transformer for 2-D problems: DownScaler2D ->
+Sp_EncoderMixer -> UpScaler2D -> Sp_DecoderRegressor.  Class names,
+constructor arguments and parameter names follow the reference's
+network/sp_model.py (Sp_EncoderMixer :9-36, Sp_DecoderRegressor :39-64,
+Sp_GalerkinTransformer2D :67-113).
+"""
+import torch
+import torch.nn.functional as F
+from torch import Tensor, nn
+
+from .layer import FeedForward, always_dropout
+from .model import DownScaler2D, UpScaler2D
+from .sp_layer import Sp_EncoderLayer, Sp_SpectralConv2D
+
+
+class UnitNormalizer:
+    """The reference's GaussNormalizer fitted on nothing (dataset/darcy_dataset.py:12-31): mean 0, std 1, eps 1e-5."""
+
+    def __init__(self, mean=0.0, std=1.0, eps=1.0e-5) -> None:
+        self.mean, self.std, self.eps = mean, std, eps
+
+    def transform(self, X):
+        return (X - self.mean) / (self.std + self.eps)
+
+    def inverse_transform(self, X):
+        return X * (self.std + self.eps) + self.mean
+
+
+class Sp_EncoderMixer(nn.Module):
+    def __init__(self, num_layer, dim_hidden, num_head, dim_position, norm_eps, attn_droprate, fc_droprate, xavier,
+                 diagonal, symmetric, ffn_dim_hidden, ffn_droprate, ffn_activation) -> None:
+        super().__init__()
+        self.layers = nn.ModuleList([
+            Sp_EncoderLayer(dim_hidden, num_head, dim_position, norm_eps, attn_droprate, fc_droprate, xavier, diagonal,
+                            symmetric, ffn_dim_hidden, ffn_droprate, ffn_activation) for _ in range(num_layer)])
+
+    def forward(self, X: Tensor, position: Tensor) -> Tensor:
+        """X [N, ra, ra, dim_hidden], position [N, ra, ra, dim_position] -> [N, ra, ra, dim_hidden]."""
+        N, ra, _, C = X.size()
+        X = X.reshape(N, ra * ra, C)
+        position = position.reshape(N, ra * ra, position.size(-1))
+        for layer in self.layers:
+            X = layer(X, position)
+        return X.view(N, ra, ra, C)
+
+
+class Sp_DecoderRegressor(nn.Module):
+    def __init__(self, num_layer, in_dim, out_dim, dim_position, dim_spatial_hidden, mode, droprate,
+                 activation) -> None:
+        super().__init__()
+        self.spatial_fc_layer = nn.Linear(in_dim + dim_position, dim_spatial_hidden)
+        self.layers = nn.ModuleList([
+            Sp_SpectralConv2D(dim_spatial_hidden, dim_spatial_hidden, mode, droprate, activation)
+            for _ in range(num_layer)])
+        self.ffn_layer = FeedForward(dim_spatial_hidden, out_dim, 2 * dim_position * dim_spatial_hidden, droprate,
+                                     activation)
+
+    def forward(self, X: Tensor, grid: Tensor = None) -> Tensor:
+        """X [N, r, r, dim_hidden], grid [N, r, r, dim_position] -> [N, r, r, dim_target]."""
+        X = self.spatial_fc_layer(torch.cat([X, grid], dim=-1))
+        for layer in self.layers:
+            X = layer(X)
+        return self.ffn_layer(X)
+
+
+class Sp_GalerkinTransformer2D(nn.Module):
+    def __init__(self, cfg) -> None:
+        super().__init__()
+        self.droprate = cfg["drop_module"]
+        self.boundary_condition = cfg["boundary_condition"]
+        self.normalizer = cfg["target_normalizer"]
+        self.down_scaler = DownScaler2D(cfg["resolution_size"], cfg["dim_node"], cfg["dim_hidden"],
+                                        cfg["drop_downscaler"], cfg["acti_downscaler"])
+        self.encoder_mixer = Sp_EncoderMixer(
+            cfg["num_encoder_layer"], cfg["dim_hidden"], cfg["num_head"], cfg["dim_position"], cfg["attn_norm_eps"],
+            cfg["drop_encoder_attn"], cfg["drop_encoder_attn_fc"], cfg["attn_xavier"], cfg["attn_diagonal"],
+            cfg["attn_symmetric"], cfg["dim_encoder_ffn"], cfg["drop_encoder_ffn"], cfg["acti_encoder_ffn"])
+        self.up_scaler = UpScaler2D(cfg["resolution_size"], cfg["dim_hidden"], cfg["dim_hidden"], cfg["drop_upscaler"],
+                                    cfg["acti_upscaler"])
+        self.decoder_regressor = Sp_DecoderRegressor(
+            cfg["num_decoder_layer"], cfg["dim_hidden"], cfg["dim_target"], cfg["dim_position"],
+            cfg["dim_spatial_hidden"], cfg["num_frequence_mode"], cfg["drop_decoder_layer"], cfg["acti_decoder_layer"])
+
+    def forward(self, X: Tensor, position: Tensor, grid: Tensor) -> Tensor:
+        """X [N, r, r, dim_node], position [N, ra, ra, dim_position], grid [N, r, r, dim_position]
+        -> [N, r, r, dim_target] (de-normalised; zero on the boundary for the Dirichlet condition)."""
+        X = always_dropout(self.down_scaler(X), self.droprate)
+        X = self.encoder_mixer(X, position)
+        X = always_dropout(self.up_scaler(X), self.droprate)
+        X = self.decoder_regressor(X, grid)
+        X = self.normalizer.inverse_transform(X)
+        if self.boundary_condition == "dirichlet":
+            X = F.pad(X[:, 1:-1, 1:-1], (0, 0, 1, 1, 1, 1), "constant", 0.0)
+        return X
