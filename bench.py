@@ -14,7 +14,9 @@ One JSON line is printed.  Beside the contract keys it carries
                 events around the launch on its stream;
   cpu_baseline  the CPU oracle (restatement of the reference's plain PyTorch
                 path) timed on this host's cores on the same shape;
-  extra         secondary measurements (feature-major op, config-2 split-K GEMM).
+  extra         secondary measurements: the feature-major attention operator, the
+                config-2 split-K GEMM, and end-to-end Darcy inference (samples/s, with
+                the CPU oracle of the same model timed beside it).
 """
 import argparse
 import json
@@ -58,6 +60,86 @@ def cpu_baseline(B, S, H, seed, budget_s=20.0):
                   f"full shape B={B} S={S} H={H}, median of {len(times)} runs, {med * 1e3:.1f} ms each",
         "ms_per_step": round(med * 1e3, 3),
     }
+
+
+def darcy_inputs(B, r, r_attn, seed):
+    """Synthetic Darcy batch: a = 12 where a Gaussian random field with covariance (-Laplace + 9 I)^-2
+    is >= 0 and 3 elsewhere (the reference's dataset/darcy_generate recipe: alpha 2, tau 3, cosine
+    basis, zero mean), plus the normalised coordinate grids at the fine and the attention resolution."""
+    import numpy as np
+    import torch
+    from scipy.fft import idctn
+
+    rng = np.random.default_rng(seed)
+    k1, k2 = np.meshgrid(np.arange(r), np.arange(r), indexing="ij")
+    coef = 3.0 * (np.pi ** 2 * (k1 ** 2 + k2 ** 2) + 9.0) ** (-1.0)  # tau^(alpha-1) (pi^2 |k|^2 + tau^2)^(-alpha/2)
+    fields = []
+    for _ in range(B):
+        xi = rng.standard_normal((r, r))
+        L = r * coef * xi
+        L[0, 0] = 0.0
+        g = idctn(L, type=2, norm="ortho")
+        fields.append(np.where(g >= 0, 12.0, 3.0))
+    a = torch.tensor(np.stack(fields), dtype=torch.float32)[..., None]
+    lin = lambda n: torch.linspace(0, 1, n)
+    mesh = lambda n: torch.stack(torch.meshgrid(lin(n), lin(n), indexing="ij"), dim=-1)[None].repeat(B, 1, 1, 1)
+    return a, mesh(r_attn), mesh(r)
+
+
+def darcy_config():
+    """End-to-end configuration: reference architecture, sizes 211 -> 122 -> 71 -> 122 -> 211,
+    4 encoder layers, FNO width 64, 12 modes, all drop rates 0."""
+    return dict(
+        drop_module=0.0, boundary_condition="dirichlet", resolution_size=((211, 211), (122, 122), (71, 71),
+                                                                           (122, 122), (211, 211)),
+        dim_node=1, dim_hidden=128, drop_downscaler=0.0, acti_downscaler="relu", num_encoder_layer=4, num_head=4,
+        dim_position=2, attn_norm_eps=1e-6, drop_encoder_attn=0.0, drop_encoder_attn_fc=0.0, attn_xavier=0.01,
+        attn_diagonal=0.01, attn_symmetric=False, dim_encoder_ffn=256, drop_encoder_ffn=0.0, acti_encoder_ffn="relu",
+        drop_upscaler=0.0, acti_upscaler="silu", num_decoder_layer=2, dim_target=1, dim_spatial_hidden=64,
+        num_frequence_mode=12, drop_decoder_layer=0.0, acti_decoder_layer="silu")
+
+
+def darcy_bench(dev, with_cpu, steps=30):
+    """End-to-end Darcy inference, B=4, random init: samples/s on the GPU and, beside it, the CPU oracle."""
+    import torch
+    from spgt_amd.network import sp_model as SM
+
+    B = 4
+    cfg = darcy_config()
+    torch.manual_seed(0)
+    model = SM.Sp_GalerkinTransformer2D(dict(cfg, target_normalizer=SM.UnitNormalizer()))
+    a, pos, grid = darcy_inputs(B, 211, 71, seed=0)
+    sd = {k: v.clone() for k, v in model.state_dict().items()}
+    model = model.to(dev).eval()
+    ad, pd, gd = a.to(dev), pos.to(dev), grid.to(dev)
+    with torch.no_grad():
+        for _ in range(5):
+            out = model(ad, pd, gd)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            out = model(ad, pd, gd)
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) / steps * 1e3
+    res = {"ms_per_forward": round(ms, 3), "samples_per_s": round(B / ms * 1e3, 1), "batch": B,
+           "config": "r=211 -> 122 -> 71, 4 encoder layers (d_model 128, 4 heads, dp 2, FFN 256), "
+                     "2 FNO blocks (width 64, 12 modes), random init, drop rates 0"}
+    if with_cpu:
+        from oracle import spgt_oracle as O
+        po = {k: (v.t() if k.rsplit(".", 1)[-1] in ("weight_Q", "weight_K", "weight_V") else v) for k, v in sd.items()}
+        with torch.no_grad():
+            want = O.galerkin_transformer_2d(po, cfg, a, pos, grid, weight_layout="sp")  # warm-up + parity
+            times = []
+            for _ in range(3):
+                t0 = time.perf_counter()
+                O.galerkin_transformer_2d(po, cfg, a, pos, grid, weight_layout="sp")
+                times.append(time.perf_counter() - t0)
+        cpu_ms = sorted(times)[1] * 1e3
+        res["cpu_oracle_ms_per_forward"] = round(cpu_ms, 1)
+        res["cpu_oracle_samples_per_s"] = round(B / cpu_ms * 1e3, 2)
+        res["cpu_cores"] = torch.get_num_threads()
+        res["rel_l2_vs_cpu_oracle"] = float(((out.cpu() - want).norm() / want.norm()).item())
+    return res
 
 
 def main():
@@ -146,6 +228,8 @@ def main():
         extra["config2_split_k_gemm"] = {"ms": round(ms, 4), "GB/s": round(c2_bytes / ms / 1e6, 1)}
         ms = timed(lambda: torch.matmul(A, Bm))
         extra["config2_torch_matmul"] = {"ms": round(ms, 4), "GB/s": round(c2_bytes / ms / 1e6, 1)}
+        del A, Bm
+        extra["darcy_inference"] = darcy_bench(dev, with_cpu=not args.no_cpu_baseline)
 
     result = {
         "metric": "galerkin_attn_hbm_gbps", "value": round(value, 1), "unit": "GB/s", "n_gpus": 1,
