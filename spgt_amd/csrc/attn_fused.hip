@@ -233,11 +233,16 @@ __global__ __launch_bounds__(256) void ktv_ln_partial_tm(
 }
 
 // out[bh][e] = scale * sum_c partial[bh][c][e], summed in a fixed order:
-// four interleaved chains (c = q, q+4, ...) combined as ((c0+c1)+(c2+c3)).
-// grid (ceil(E/256), BH), block 256 = 64 element-quads x 4 chains.
-__global__ __launch_bounds__(256) void tile_reduce(
+// sixteen interleaved chains (c = q, q+16, ...), each summed in increasing c,
+// then combined by a fixed binary tree.  All loads of a chain are issued before
+// the first add, so the kernel costs about one memory round trip.
+// grid (ceil(E/256), BH), block 1024 = 64 element-quads x 16 chains.
+constexpr int kReduceChains = 16;
+constexpr int kReduceMaxPerChain = 16;  // nchunk <= 256
+
+__global__ __launch_bounds__(1024) void tile_reduce(
     const float* __restrict__ partial, float* __restrict__ out, int E, int nchunk, float scale) {
-    __shared__ float4 sm[4][64];
+    __shared__ float4 sm[kReduceChains][64];
     const int q = threadIdx.x >> 6;
     const int e4 = threadIdx.x & 63;
     const int e = (blockIdx.x * 64 + e4) * 4;
@@ -245,22 +250,32 @@ __global__ __launch_bounds__(256) void tile_reduce(
     float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
     if (e < E) {
         const float* src = partial + bh * nchunk * (int64_t)E + e;
-#pragma unroll 8
-        for (int c = q; c < nchunk; c += 4) {
-            const float4 v = *reinterpret_cast<const float4*>(src + (int64_t)c * E);
-            s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+        float4 v[kReduceMaxPerChain];
+#pragma unroll
+        for (int i = 0; i < kReduceMaxPerChain; ++i) {
+            const int c = q + kReduceChains * i;
+            v[i] = (c < nchunk) ? *reinterpret_cast<const float4*>(src + (int64_t)c * E)
+                                : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+#pragma unroll
+        for (int i = 0; i < kReduceMaxPerChain; ++i) {
+            s.x += v[i].x; s.y += v[i].y; s.z += v[i].z; s.w += v[i].w;
         }
     }
     sm[q][e4] = s;
     __syncthreads();
     if (q == 0 && e < E) {
-        const float4 a = sm[0][e4], b2 = sm[1][e4], c2 = sm[2][e4], d2 = sm[3][e4];
-        float4 r;
-        r.x = ((a.x + b2.x) + (c2.x + d2.x)) * scale;
-        r.y = ((a.y + b2.y) + (c2.y + d2.y)) * scale;
-        r.z = ((a.z + b2.z) + (c2.z + d2.z)) * scale;
-        r.w = ((a.w + b2.w) + (c2.w + d2.w)) * scale;
-        *reinterpret_cast<float4*>(out + bh * E + e) = r;
+        float4 t[kReduceChains];
+#pragma unroll
+        for (int i = 0; i < kReduceChains; ++i) t[i] = sm[i][e4];
+#pragma unroll
+        for (int w = kReduceChains / 2; w >= 1; w /= 2)
+#pragma unroll
+            for (int i = 0; i < w; ++i) {
+                t[i].x += t[i + w].x; t[i].y += t[i + w].y; t[i].z += t[i + w].z; t[i].w += t[i + w].w;
+            }
+        *reinterpret_cast<float4*>(out + bh * E + e) =
+            make_float4(t[0].x * scale, t[0].y * scale, t[0].z * scale, t[0].w * scale);
     }
 }
 
@@ -325,7 +340,10 @@ __global__ __launch_bounds__(256) void qm_apply_tm(
         if (DP == 2) u.p = *reinterpret_cast<const float2*>(pbase + (int64_t)s * 2);
         return u;
     };
-    auto compute_unit = [&](const Unit& u, int s, bool valid) {
+    // `sb` is the first token of the unit (this lane's token is sb + tk, clamped loads aside).
+    auto compute_unit = [&](const Unit& u, int sb) {
+        const int s = sb + tk;
+        const bool valid = s < s1;
         const float q[8] = {u.q0.x, u.q0.y, u.q0.z, u.q0.w, u.q1.x, u.q1.y, u.q1.z, u.q1.w};
         v4f acc[2];
 #pragma unroll
@@ -343,7 +361,7 @@ __global__ __launch_bounds__(256) void qm_apply_tm(
             acc[0] = mfma16(mreg[kk][0], q[kk], acc[0]);
             acc[1] = mfma16(mreg[kk][1], q[kk], acc[1]);
         }
-        float* op = obase + (int64_t)s * ldo;
+        float* op = obase + (int64_t)min(s, s1 - 1) * ldo;
         if (DP == 2) {
             float c0 = 0.f, c1 = 0.f;
 #pragma unroll
@@ -367,11 +385,32 @@ __global__ __launch_bounds__(256) void qm_apply_tm(
                     *reinterpret_cast<float2*>(o + 2) = make_float2(acc[jb][2], acc[jb][3]);
                 }
             }
-        } else if (valid) {
+        } else {
+            // Lanes tk and tk^8 swap halves so that one store instruction writes
+            // whole 128-byte head rows of 8 tokens (non-temporal stores of partial
+            // lines cost extra HBM write traffic).
+            const bool lo = tk < 8;
+            // cross-lane moves first, with every lane active; selects afterwards
+            float o0[4], o1[4];
 #pragma unroll
-            for (int jb = 0; jb < 2; ++jb)
-                st_stream<SPGT_NT_P2ST>(reinterpret_cast<float4*>(op + jb * 16 + 4 * g),
-                          make_float4(acc[jb][0], acc[jb][1], acc[jb][2], acc[jb][3]));
+            for (int r = 0; r < 4; ++r) {
+                o0[r] = dpp_move<SPGT_DPP_ROW_ROR8>(acc[0][r]);
+                o1[r] = dpp_move<SPGT_DPP_ROW_ROR8>(acc[1][r]);
+            }
+            float4 x, y;
+            x.x = lo ? acc[0][0] : o1[0];
+            x.y = lo ? acc[0][1] : o1[1];
+            x.z = lo ? acc[0][2] : o1[2];
+            x.w = lo ? acc[0][3] : o1[3];
+            y.x = lo ? o0[0] : acc[1][0];
+            y.y = lo ? o0[1] : acc[1][1];
+            y.z = lo ? o0[2] : acc[1][2];
+            y.w = lo ? o0[3] : acc[1][3];
+            const int fo = (lo ? 0 : 16) + 4 * g;
+            const int sx = sb + (tk & 7);
+            const int sy = sx + 8;
+            if (sx < s1) st_stream<SPGT_NT_P2ST>(reinterpret_cast<float4*>(obase + (int64_t)sx * ldo + fo), x);
+            if (sy < s1) st_stream<SPGT_NT_P2ST>(reinterpret_cast<float4*>(obase + (int64_t)sy * ldo + fo), y);
         }
     };
 
@@ -387,9 +426,9 @@ __global__ __launch_bounds__(256) void qm_apply_tm(
         for (int u = 0; u < U; ++u) buf[u] = load_unit(min(sg + 16 * u, s1 - 1));
     };
     auto compute_group = [&](const Unit(&buf)[U], int gi) {
-        const int sg = s0 + gi * G + tk;
+        const int sg = s0 + gi * G;
 #pragma unroll
-        for (int u = 0; u < U; ++u) compute_unit(buf[u], sg + 16 * u, true);
+        for (int u = 0; u < U; ++u) compute_unit(buf[u], sg + 16 * u);
     };
     load_group(bufA, 0);
     int gi = 0;
@@ -411,12 +450,9 @@ __global__ __launch_bounds__(256) void qm_apply_tm(
         ++gi;
     }
     if (gi < ntot) {
-        const int sg = s0 + gi * G + tk;
+        const int sg = s0 + gi * G;
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int sl = sg + 16 * u;
-            compute_unit(bufA[u], min(sl, s1 - 1), sl < s1);
-        }
+        for (int u = 0; u < U; ++u) compute_unit(bufA[u], sg + 16 * u);
     }
 }
 
@@ -434,16 +470,29 @@ struct FusedPlan {
 constexpr int kU1 = 4;  // 16 tokens per unrolled group in pass 1
 constexpr int kU2 = 2;  // 32 tokens per unrolled group in pass 2
 
+// Workgroups per pass: three per compute unit.  Measured on MI355X (256 CUs) at
+// B=8, S=44521: counts that are whole multiples of the CU count (512, 768, 1024)
+// beat those in between by 3-10 %, and 768 is the fastest of them.
+#ifdef SPGT_TUNING
+int g_target_wg1 = 0, g_target_wg2 = 0;
+#else
+constexpr int g_target_wg1 = 0, g_target_wg2 = 0;
+#endif
+
 FusedPlan make_plan(int B, int S, int H) {
-    // Aim at ~4 resident workgroups per CU (256 CUs); chunks are whole
-    // unrolled groups so that only the last chunk of a batch has a ragged tail.
-    const int target_wg = 1024;
-    const int per_bh = std::max(1, target_wg / std::max(1, B * (H / 4)));
+    // Chunks are whole unrolled groups so that only the last chunk of a batch has a ragged tail.
+    // The K/V pass never uses more chunks than tile_reduce can sum.
+    const int bg = std::max(1, B * (H / 4));
+    const int dflt = 3 * device_cu_count();
+    const int t1 = g_target_wg1 > 0 ? g_target_wg1 : dflt;
+    const int t2 = g_target_wg2 > 0 ? g_target_wg2 : dflt;
+    const int per_bh1 = std::min(kReduceChains * kReduceMaxPerChain, std::max(1, t1 / bg));
+    const int per_bh2 = std::max(1, t2 / bg);
     FusedPlan p;
     const int g1 = 4 * kU1, g2 = 16 * kU2;
-    p.tpc1 = std::max(g1, ceil_div(ceil_div(S, per_bh), g1) * g1);
+    p.tpc1 = std::max(g1, ceil_div(ceil_div(S, per_bh1), g1) * g1);
     p.nchunk1 = ceil_div(S, p.tpc1);
-    p.tpc2 = std::max(g2, ceil_div(ceil_div(S, per_bh), g2) * g2);
+    p.tpc2 = std::max(g2, ceil_div(ceil_div(S, per_bh2), g2) * g2);
     p.nchunk2 = ceil_div(S, p.tpc2);
     return p;
 }
@@ -499,6 +548,7 @@ int fused_forward_impl(
     const dim3 grid1(p.nchunk1, H / 4, B);
     const dim3 grid2(p.nchunk2, H / 4, B);
     const dim3 gridr(ceil_div(D * D, 256), B * H);
+    const dim3 blockr(1024);
     const float* pos = position ? position : Q;  // never dereferenced when dp == 0
     if (ev) (void)hipEventRecord(ev[0], stream);
     if (dp == 0) {
@@ -509,7 +559,7 @@ int fused_forward_impl(
                            ln_bias_K, ln_weight_V, ln_bias_V, norm_eps, partial, S, H, ld_in, p.tpc1);
     }
     if (ev) (void)hipEventRecord(ev[1], stream);
-    hipLaunchKernelGGL(tile_reduce, gridr, block, 0, stream, partial, ktv, D * D, p.nchunk1, 1.0f / (float)S);
+    hipLaunchKernelGGL(tile_reduce, gridr, blockr, 0, stream, partial, ktv, D * D, p.nchunk1, 1.0f / (float)S);
     if (ev) (void)hipEventRecord(ev[2], stream);
     if (dp == 0) {
         hipLaunchKernelGGL((qm_apply_tm<0, kU2>), grid2, block, 0, stream, Q, pos, ktv, out, S, H, ld_in, p.tpc2);

@@ -22,6 +22,7 @@ struct __attribute__((packed, aligned(4))) f4u { float x, y, z, w; };
 #define SPGT_DPP_QUAD_XOR2 0x4E         // quad_perm:[2,3,0,1]
 #define SPGT_DPP_ROW_HALF_MIRROR 0x141  // lane i <-> 7-i inside each 8 lanes
 #define SPGT_DPP_ROW_MIRROR 0x140       // lane i <-> 15-i inside each 16 lanes
+#define SPGT_DPP_ROW_ROR8 0x128         // rotate by 8 inside each 16 lanes: lane i <-> i^8
 
 template <int CTRL>
 __device__ __forceinline__ float dpp_move(float v) {

@@ -1,6 +1,7 @@
 // Error state and version of the C ABI.
 #include "spgt_host.h"
 
+#include <atomic>
 #include <stdio.h>
 #include <string.h>
 
@@ -20,6 +21,18 @@ int check_launch(const char* what) {
     if (e == hipSuccess) return SPGT_OK;
     snprintf(g_last_error, sizeof(g_last_error), "%s: kernel launch failed: %s", what, hipGetErrorString(e));
     return SPGT_ERR_LAUNCH;
+}
+
+int device_cu_count() {
+    static std::atomic<int> cached[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    int n = cached[dev].load(std::memory_order_relaxed);
+    if (n == 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cached[dev].store(n, std::memory_order_relaxed);
+    }
+    return n;
 }
 
 }  // namespace spgt

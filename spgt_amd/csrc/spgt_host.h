@@ -16,6 +16,9 @@ int fail(int code, const char* msg);
 // a kernel launch issued by `what` since the last check was rejected.
 int check_launch(const char* what);
 
+// Compute units of the current device (cached per device; 256 if the query fails).
+int device_cu_count();
+
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 inline bool aligned8(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 7u) == 0; }
 inline bool aligned4(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 3u) == 0; }
