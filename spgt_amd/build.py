@@ -15,7 +15,8 @@ LIB_PATH = os.path.join(PKG_DIR, "libspgt_hip.so")
 SOURCES = [
     "spgt_host.cpp",
     "attn_fused.hip",
-    "attn_cccr.hip",
+    "attn_fm.hip",
+    "splitk_gemm.hip",
     "projection.hip",
     "datamove.hip",
     "spectral.hip",

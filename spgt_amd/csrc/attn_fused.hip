@@ -20,6 +20,7 @@
 //      registers as the MFMA A operand, writes out once.
 #include "spgt_device.h"
 #include "spgt_host.h"
+#include "spgt_kernels.h"
 
 // Cache policy of the three touch-once streams (K/V reads, Q reads, out
 // writes).  Measured on MI355X at B=8, S=44521 over all eight combinations:
@@ -237,9 +238,6 @@ __global__ __launch_bounds__(256) void ktv_ln_partial_tm(
 // then combined by a fixed binary tree.  All loads of a chain are issued before
 // the first add, so the kernel costs about one memory round trip.
 // grid (ceil(E/256), BH), block 1024 = 64 element-quads x 16 chains.
-constexpr int kReduceChains = 16;
-constexpr int kReduceMaxPerChain = 16;  // nchunk <= 256
-
 __global__ __launch_bounds__(1024) void tile_reduce(
     const float* __restrict__ partial, float* __restrict__ out, int E, int nchunk, float scale) {
     __shared__ float4 sm[kReduceChains][64];

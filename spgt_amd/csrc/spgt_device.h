@@ -10,6 +10,9 @@ namespace spgt {
 typedef float v2f __attribute__((ext_vector_type(2)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef float v16f __attribute__((ext_vector_type(16)));
+// 4-byte aligned vector types for rows of [d, S] tensors with odd S (see f2u / f4u below)
+typedef v2f v2f_a4 __attribute__((aligned(4)));
+typedef v4f v4f_a4 __attribute__((aligned(4)));
 
 // 4-byte aligned vector views: rows of a [d, S] tensor with odd S start at
 // arbitrary 4-byte offsets, and the hardware handles unaligned dwordx2/x4

@@ -1,11 +1,9 @@
 // Batched skinny GEMM (small M, N; long K) with a deterministic two-stage
-// split-K reduction, and the feature-major Galerkin attention op built on it.
+// split-K reduction, for all eight operand storage orders.
 //
 // Reference behaviour restated here:
 //   sgemm_32x32_4x8_SplitK::sgemm_cuda   extension/native/sgemm_32x32_splitk.cu:662-705
-//   sgemm_32x32_4x4::sgemm_cuda (CCR)    extension/native/sgemm_32x32.cu:683-710
-//   multihead_galerkin_attention_cccr_forward / batched_skinny_gemm
-//                                        extension/bind/galerkin_attention.cu:104-124, 175-198
+//   batched_skinny_gemm                  extension/bind/galerkin_attention.cu:175-198
 //
 // Stage 1 (splitk_partial): a workgroup owns one 32x32 output tile and one
 // contiguous K range.  Operand tiles are staged through LDS so that global
@@ -191,93 +189,6 @@ __global__ __launch_bounds__(256) void splitk_reduce_store(
     }
 }
 
-// out[bh][s][j] = sum_i Q[bh][i][s] * Mt[bh][j*D + i]   (Mt = column-major K^T V / S)
-// grid (nchunk, BH), block 256; a wave owns runs of 32 tokens.
-// Lane l: token l%32, contraction half kh = l/32 (features 2kk+kh).
-template <int D, int U>
-__global__ __launch_bounds__(256) void qm_apply_fm(
-    const float* __restrict__ Q, const float* __restrict__ Mt, float* __restrict__ out, int S,
-    int tokens_per_chunk) {
-    constexpr int NK = D / 2;
-    const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
-    const int tk = lane & 31;
-    const int kh = lane >> 5;
-    const int64_t bh = blockIdx.y;
-    const int s0 = blockIdx.x * tokens_per_chunk;
-    const int s1 = min(S, s0 + tokens_per_chunk);
-
-    const float* m = Mt + bh * (D * D);
-    float mreg[NK];
-#pragma unroll
-    for (int kk = 0; kk < NK; ++kk) mreg[kk] = m[tk * D + 2 * kk + kh];  // M[2kk+kh][j = tk]
-    float mcol[NK][2];
-    if (D == 34) {
-#pragma unroll
-        for (int kk = 0; kk < NK; ++kk) {
-            mcol[kk][0] = m[32 * D + 2 * kk + kh];
-            mcol[kk][1] = m[33 * D + 2 * kk + kh];
-        }
-    }
-
-    const float* qb = Q + bh * D * (int64_t)S + (int64_t)kh * S;
-    float* ob = out + bh * (int64_t)S * D;
-
-    auto load_unit = [&](int s, float (&q)[NK]) {
-#pragma unroll
-        for (int kk = 0; kk < NK; ++kk) q[kk] = qb[(int64_t)(2 * kk) * S + s];
-    };
-    auto compute_unit = [&](const float (&q)[NK], int s, bool valid) {
-        v16f acc;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[r] = 0.f;
-#pragma unroll
-        for (int kk = 0; kk < NK; ++kk) acc = mfma32(mreg[kk], q[kk], acc);
-        float* op = ob + (int64_t)s * D;
-        if (D == 34) {
-            float c0 = 0.f, c1 = 0.f;
-#pragma unroll
-            for (int kk = 0; kk < NK; ++kk) {
-                c0 = fmaf(q[kk], mcol[kk][0], c0);
-                c1 = fmaf(q[kk], mcol[kk][1], c1);
-            }
-            c0 += __shfl_xor(c0, 32, 64);
-            c1 += __shfl_xor(c1, 32, 64);
-            if (valid) {
-#pragma unroll
-                for (int qd = 0; qd < 4; ++qd) {
-                    float* o = op + 8 * qd + 4 * kh;
-                    *reinterpret_cast<float2*>(o) = make_float2(acc[4 * qd], acc[4 * qd + 1]);
-                    *reinterpret_cast<float2*>(o + 2) = make_float2(acc[4 * qd + 2], acc[4 * qd + 3]);
-                }
-                if (kh == 0) *reinterpret_cast<float2*>(op + 32) = make_float2(c0, c1);
-            }
-        } else if (valid) {
-#pragma unroll
-            for (int qd = 0; qd < 4; ++qd)
-                *reinterpret_cast<float4*>(op + 8 * qd + 4 * kh) =
-                    make_float4(acc[4 * qd], acc[4 * qd + 1], acc[4 * qd + 2], acc[4 * qd + 3]);
-        }
-    };
-
-    // Waves interleave runs of 32*U tokens inside the chunk.
-    constexpr int G = 32 * U;
-    for (int sg = s0 + wave * G; sg < s1; sg += 4 * G) {
-        float q[U][NK];
-        int sl[U];
-        bool valid[U];
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int s = sg + 32 * u + tk;
-            valid[u] = s < s1;
-            sl[u] = valid[u] ? s : s1 - 1;
-            load_unit(sl[u], q[u]);
-        }
-#pragma unroll
-        for (int u = 0; u < U; ++u) compute_unit(q[u], sl[u], valid[u]);
-    }
-}
-
 namespace {
 
 struct SplitPlan {
@@ -332,8 +243,6 @@ size_t splitk_partial_bytes(int M, int N, int K, int batch_count) {
     return (size_t)batch_count * p.ntile * p.nsplit * 1024 * sizeof(float);
 }
 
-size_t round256(size_t x) { return (x + 255) & ~(size_t)255; }
-
 }  // namespace
 
 }  // namespace spgt
@@ -362,46 +271,4 @@ extern "C" int spgt_batched_skinny_gemm(const float* A, const float* B, float* C
     launch_splitk(A, B, C, alpha, M, N, K, a_stride, b_stride, c_stride, order, batch_count,
                   static_cast<float*>(workspace), stream);
     return check_launch("batched_skinny_gemm");
-}
-
-extern "C" size_t spgt_galerkin_attention_cccr_workspace_bytes(int batch, int num_head, int d_posk, int seqlen) {
-    if (batch <= 0 || num_head <= 0 || seqlen <= 0 || (d_posk != 32 && d_posk != 34)) return 0;
-    const int bh = batch * num_head;
-    // [K^T V / S, column-major, per (batch, head)] followed by the split-K partial tiles
-    return round256((size_t)bh * d_posk * d_posk * sizeof(float)) + splitk_partial_bytes(d_posk, d_posk, seqlen, bh);
-}
-
-extern "C" int spgt_galerkin_attention_cccr_forward(const float* Q, const float* K, const float* V, float* out,
-                                                    void* workspace, size_t workspace_bytes, int batch,
-                                                    int num_head, int d_posk, int seqlen, hipStream_t stream) {
-    if (!Q || !K || !V || !out) return fail(SPGT_ERR_INVALID_ARGUMENT, "galerkin_attention_cccr: null pointer argument");
-    if (batch <= 0 || num_head <= 0 || seqlen <= 0)
-        return fail(SPGT_ERR_INVALID_ARGUMENT, "galerkin_attention_cccr: batch, num_head, seqlen must be positive");
-    if (d_posk != 32 && d_posk != 34)
-        return fail(SPGT_ERR_INVALID_ARGUMENT, "galerkin_attention_cccr: d_posk must be 32 or 34");
-    const int64_t bh64 = (int64_t)batch * num_head;
-    if (bh64 > 65535) return fail(SPGT_ERR_INVALID_ARGUMENT, "galerkin_attention_cccr: batch*num_head exceeds 65535");
-    if (!aligned4(Q) || !aligned4(K) || !aligned4(V) || !aligned16(out))
-        return fail(SPGT_ERR_INVALID_ARGUMENT, "galerkin_attention_cccr: inputs must be 4-byte, out 16-byte aligned");
-    const size_t need = spgt_galerkin_attention_cccr_workspace_bytes(batch, num_head, d_posk, seqlen);
-    if (!workspace || workspace_bytes < need || !aligned16(workspace))
-        return fail(SPGT_ERR_WORKSPACE, "galerkin_attention_cccr: workspace missing, misaligned or too small");
-    const int bh = (int)bh64;
-    const int D = d_posk;
-    float* mt = static_cast<float*>(workspace);
-    float* partial = reinterpret_cast<float*>(static_cast<char*>(workspace) +
-                                              round256((size_t)bh * D * D * sizeof(float)));
-    const int64_t qs = (int64_t)D * seqlen;
-    launch_splitk(K, V, mt, 1.0f / (float)seqlen, D, D, seqlen, qs, qs, (int64_t)D * D, SPGT_ORDER_RCC, bh,
-                  partial, stream);
-    constexpr int U = 2;
-    const int per_bh = std::max(1, 2048 / bh);
-    const int g = 4 * 32 * U;
-    const int tpc = std::max(g, ceil_div(ceil_div(seqlen, per_bh), g) * g);
-    const dim3 grid(ceil_div(seqlen, tpc), bh);
-    if (D == 32)
-        hipLaunchKernelGGL((qm_apply_fm<32, U>), grid, dim3(256), 0, stream, Q, mt, out, seqlen, tpc);
-    else
-        hipLaunchKernelGGL((qm_apply_fm<34, U>), grid, dim3(256), 0, stream, Q, mt, out, seqlen, tpc);
-    return check_launch("galerkin_attention_cccr");
 }
