@@ -115,6 +115,32 @@ int spgt_galerkin_attention_fused_forward(const float* Q, const float* K, const 
                                           size_t workspace_bytes, int B, int S, int H, int dp,
                                           spgt_stream_t stream);
 
+/* ---- backward of the attention operators ------------------------------------ */
+
+/* Replaces multihead_galerkin_attention_cccr_backward (extension/bind/galerkin_attention.cu:126-173).
+ *   grad_out [batch, num_head, seqlen, d_posk]; Q, K, V, grad_Q, grad_K, grad_V [batch, num_head, d_posk, seqlen]. */
+size_t spgt_galerkin_attention_cccr_backward_workspace_bytes(int batch, int num_head, int d_posk, int seqlen);
+int spgt_galerkin_attention_cccr_backward(const float* grad_out, const float* Q, const float* K,
+                                          const float* V, float* grad_Q, float* grad_K, float* grad_V,
+                                          void* workspace, size_t workspace_bytes, int batch, int num_head,
+                                          int d_posk, int seqlen, spgt_stream_t stream);
+
+/* Replaces datamove::batched_transpose_gather (extension/native/datamove.cu:121-163), the first step of
+ * both projection backwards (extension/bind/galerkin_attention.cu:34-39):
+ *   src [batch, num_head, dim_position + dim_head, seqlen], rows dim_position.. of every head
+ *   -> dst [batch, seqlen, num_head * dim_head]. */
+int spgt_heads_feature_to_token_major(const float* src, float* dst, int batch, int num_head,
+                                      int dim_position, int dim_head, int seqlen, spgt_stream_t stream);
+
+/* Replaces mh32::lnorm_grad_ccc_cuda (extension/native/multihead_dim32.cu:148-271, 601-618), on token-major
+ * data and from the pre-LayerNorm projection instead of (y - beta) / gamma:
+ *   pre_ln, grad_ln, grad_pre_ln [tokens, num_head*32]; ln_weight, grad_ln_weight, grad_ln_bias [num_head, 32]. */
+size_t spgt_layernorm_heads_backward_workspace_bytes(int64_t tokens, int num_head);
+int spgt_layernorm_heads_backward(const float* pre_ln, const float* grad_ln, const float* ln_weight,
+                                  float norm_eps, float* grad_pre_ln, float* grad_ln_weight,
+                                  float* grad_ln_bias, void* workspace, size_t workspace_bytes,
+                                  int64_t tokens, int num_head, spgt_stream_t stream);
+
 /* ---- FNO2d data movement and spectral contraction --------------------------- */
 
 /* Replaces batched_transpose (extension/bind/datamove.cu:8-23):

@@ -16,6 +16,7 @@ SOURCES = [
     "spgt_host.cpp",
     "attn_fused.hip",
     "attn_fm.hip",
+    "attn_backward.hip",
     "splitk_gemm.hip",
     "projection.hip",
     "datamove.hip",

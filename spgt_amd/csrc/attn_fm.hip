@@ -332,6 +332,25 @@ __global__ __launch_bounds__(256) void qm_apply_fm(const float* __restrict__ Q, 
 
 }  // namespace spgt
 
+namespace spgt {
+
+// K V^T / S of every (batch, head) into m [bh, D, D] row-major: the K/V pass followed by the tile
+// reduction, with `partial` holding bh * nchunk * D*D floats.  Shared with the backward operator.
+size_t ktv_fm_partial_bytes(int bh, int D, int nchunk) { return (size_t)bh * nchunk * D * D * sizeof(float); }
+
+int launch_ktv_fm(const float* K, const float* V, float* m, float* partial, int bh, int D, int S, int tpc,
+                  int nchunk, hipStream_t stream) {
+    const dim3 grid1(nchunk, bh), gridr(ceil_div(D * D, 256), bh);
+    if (D == 32)
+        hipLaunchKernelGGL((ktv_partial_fm<32>), grid1, dim3(256), 0, stream, K, V, partial, S, tpc);
+    else
+        hipLaunchKernelGGL((ktv_partial_fm<34>), grid1, dim3(256), 0, stream, K, V, partial, S, tpc);
+    hipLaunchKernelGGL(tile_reduce, gridr, dim3(1024), 0, stream, partial, m, D * D, nchunk, 1.0f / (float)S);
+    return SPGT_OK;
+}
+
+}  // namespace spgt
+
 using namespace spgt;
 
 namespace {
@@ -386,15 +405,11 @@ extern "C" int spgt_galerkin_attention_cccr_forward(const float* Q, const float*
     float* mt = static_cast<float*>(workspace);
     float* partial = reinterpret_cast<float*>(static_cast<char*>(workspace) +
                                               round256((size_t)bh * D * D * sizeof(float)));
-    const dim3 grid1(p.nchunk1, bh), grid2(p.nchunk2, bh), gridr(ceil_div(D * D, 256), bh);
-    if (D == 32) {
-        hipLaunchKernelGGL((ktv_partial_fm<32>), grid1, dim3(256), 0, stream, K, V, partial, seqlen, p.tpc1);
-        hipLaunchKernelGGL(tile_reduce, gridr, dim3(1024), 0, stream, partial, mt, D * D, p.nchunk1, 1.0f / (float)seqlen);
+    const dim3 grid2(p.nchunk2, bh);
+    launch_ktv_fm(K, V, mt, partial, bh, D, seqlen, p.tpc1, p.nchunk1, stream);
+    if (D == 32)
         hipLaunchKernelGGL((qm_apply_fm<32>), grid2, dim3(256), 0, stream, Q, mt, out, seqlen, p.tpc2);
-    } else {
-        hipLaunchKernelGGL((ktv_partial_fm<34>), grid1, dim3(256), 0, stream, K, V, partial, seqlen, p.tpc1);
-        hipLaunchKernelGGL(tile_reduce, gridr, dim3(1024), 0, stream, partial, mt, D * D, p.nchunk1, 1.0f / (float)seqlen);
+    else
         hipLaunchKernelGGL((qm_apply_fm<34>), grid2, dim3(256), 0, stream, Q, mt, out, seqlen, p.tpc2);
-    }
     return check_launch("galerkin_attention_cccr");
 }

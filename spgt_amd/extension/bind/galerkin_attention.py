@@ -91,6 +91,88 @@ def _attention_cccr_forward(Q: Tensor, K: Tensor, V: Tensor, batch: int, num_hea
     return out
 
 
+def _attention_cccr_backward(grad_out: Tensor, Q: Tensor, K: Tensor, V: Tensor, batch: int, num_head: int,
+                             d_posk: int, seqlen: int):
+    """grad_out [batch, num_head, seqlen, d_posk] -> (dQ, dK, dV), each [batch, num_head, d_posk, seqlen]
+    (reference: extension/bind/galerkin_attention.cu:126-173)."""
+    grad_out = grad_out.contiguous()
+    require_gpu_f32("grad_out", grad_out)
+    if tuple(grad_out.shape) != (batch, num_head, seqlen, d_posk):
+        raise ValueError(f"grad_out has shape {tuple(grad_out.shape)}, expected {(batch, num_head, seqlen, d_posk)}")
+    for name, t in (("Q", Q), ("K", K), ("V", V)):
+        require_gpu_f32(name, t)
+        if tuple(t.shape) != (batch, num_head, d_posk, seqlen):
+            raise ValueError(f"{name} has shape {tuple(t.shape)}, expected {(batch, num_head, d_posk, seqlen)}")
+    lib = _lib.load()
+    dQ, dK, dV = torch.empty_like(Q), torch.empty_like(K), torch.empty_like(V)
+    nbytes = lib.spgt_galerkin_attention_cccr_backward_workspace_bytes(batch, num_head, d_posk, seqlen)
+    if nbytes == 0:
+        raise ValueError("unsupported attention shape (d_posk must be 32 or 34)")
+    ws = workspace(nbytes, Q)
+    with torch.cuda.device(Q.device):
+        check(lib.spgt_galerkin_attention_cccr_backward(
+            ptr(grad_out), ptr(Q), ptr(K), ptr(V), ptr(dQ), ptr(dK), ptr(dV), ptr(ws), ws.numel(), batch, num_head,
+            d_posk, seqlen, stream_of(Q)))
+    return dQ, dK, dV
+
+
+def _heads_feature_to_token_major(src: Tensor, batch: int, num_head: int, dim_position: int, dim_head: int,
+                                  seqlen: int) -> Tensor:
+    """[batch, num_head, dim_position + dim_head, seqlen] -> [batch, seqlen, num_head * dim_head]
+    (reference: datamove::batched_transpose_gather, extension/native/datamove.cu:121-163)."""
+    src = src.contiguous()
+    require_gpu_f32("src", src)
+    if tuple(src.shape) != (batch, num_head, dim_position + dim_head, seqlen):
+        raise ValueError(f"src has shape {tuple(src.shape)}")
+    dst = torch.empty((batch, seqlen, num_head * dim_head), dtype=src.dtype, device=src.device)
+    with torch.cuda.device(src.device):
+        check(_lib.load().spgt_heads_feature_to_token_major(ptr(src), ptr(dst), batch, num_head, dim_position,
+                                                            dim_head, seqlen, stream_of(src)))
+    return dst
+
+
+def _linear_backward(grad_tm: Tensor, input: Tensor, weight: Tensor):
+    """Gradients of y = x @ W + b given dL/dy token-major: library GEMMs, as in the reference's
+    extension/bind/galerkin_attention.cu:41-46."""
+    dm = weight.shape[0]
+    grad_input = torch.matmul(grad_tm, weight.t())
+    grad_bias = grad_tm.sum(dim=(0, 1))
+    grad_weight = torch.matmul(input.reshape(-1, dm).t(), grad_tm.reshape(-1, dm))
+    return grad_input, grad_weight, grad_bias
+
+
+def _projection_backward(grad_out: Tensor, input: Tensor, weight: Tensor, seqlen: int, dim_hidden: int, num_head: int,
+                         dim_head: int, dim_position: int, batch: int):
+    """-> (dX, dW, db) (reference: extension/bind/galerkin_attention.cu:26-48)."""
+    g = _heads_feature_to_token_major(grad_out, batch, num_head, dim_position, dim_head, seqlen)
+    return _linear_backward(g, input, weight)
+
+
+def _projection_layernorm_backward(grad_ln: Tensor, input: Tensor, weight: Tensor, bias: Tensor, lnw: Tensor,
+                                   norm_eps: float, seqlen: int, dim_hidden: int, num_head: int, dim_head: int,
+                                   dim_position: int, batch: int):
+    """-> (dX, dW, db, dgamma, dbeta) (reference: extension/bind/galerkin_attention.cu:70-102).
+
+    Unlike the reference, which recovers x_hat from the saved LayerNorm output as (y - beta) / gamma and
+    therefore fails when a gamma is zero, the pre-LayerNorm projection is recomputed from input, weight
+    and bias; that is why `bias` and `norm_eps` are arguments here and hat_ln / invsigma are not."""
+    require_gpu_f32("lnw", lnw)
+    g = _heads_feature_to_token_major(grad_ln, batch, num_head, dim_position, dim_head, seqlen)
+    pre = torch.addmm(bias, input.reshape(-1, dim_hidden), weight)
+    lib = _lib.load()
+    tokens = batch * seqlen
+    grad_pre = torch.empty_like(pre)
+    grad_lnw = torch.empty((num_head, dim_head), dtype=pre.dtype, device=pre.device)
+    grad_lnb = torch.empty((num_head, dim_head), dtype=pre.dtype, device=pre.device)
+    ws = workspace(lib.spgt_layernorm_heads_backward_workspace_bytes(tokens, num_head), pre)
+    with torch.cuda.device(pre.device):
+        check(lib.spgt_layernorm_heads_backward(
+            ptr(pre), ptr(g), ptr(lnw), float(norm_eps), ptr(grad_pre), ptr(grad_lnw), ptr(grad_lnb), ptr(ws),
+            ws.numel(), tokens, num_head, stream_of(pre)))
+    grad_input, grad_weight, grad_bias = _linear_backward(grad_pre.view(batch, seqlen, dim_hidden), input, weight)
+    return grad_input, grad_weight, grad_bias, grad_lnw, grad_lnb
+
+
 def _batched_skinny_gemm(A: Tensor, B: Tensor, alpha: float) -> Tensor:
     """A [..., M, K] @ B [..., K, N] * alpha, all row-major
     (reference: extension/bind/galerkin_attention.cu:175-198)."""
@@ -187,7 +269,11 @@ def _attention_fused_profile(Q, K, V, position, ln_weight_K, ln_bias_K, ln_weigh
 
 gexts = SimpleNamespace(
     multihead_projection_with_position_rrc_forward=_projection_forward,
+    multihead_projection_with_position_rrc_backward=_projection_backward,
     multihead_projection_layernorm_with_position_rrc_forward=_projection_layernorm_forward,
+    multihead_projection_layernorm_with_position_rrc_backward=_projection_layernorm_backward,
+    multihead_galerkin_attention_cccr_backward=_attention_cccr_backward,
+    heads_feature_to_token_major=_heads_feature_to_token_major,
     galerkin_attention_fused_profile=_attention_fused_profile,
     multihead_galerkin_attention_cccr_forward=_attention_cccr_forward,
     batched_skinny_gemm=_batched_skinny_gemm,
@@ -212,7 +298,12 @@ class Multihead_Porjection_with_Position_Function(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx: Any, grad_out: Tensor):
-        raise NotImplementedError("backward of multihead_projection_with_position_rrc_cuda is not built yet")
+        input, weight = ctx.saved_tensors
+        num_head, dim_head, dim_position = ctx.shape_kwargs
+        batch, seqlen, d_model = input.size()
+        grad_input, grad_weight, grad_bias = gexts.multihead_projection_with_position_rrc_backward(
+            grad_out, input, weight, seqlen, d_model, num_head, dim_head, dim_position, batch)
+        return grad_input, grad_weight, grad_bias, None, None, None, None
 
 
 class Multihead_Porjection_Layernorm_with_Position_Function(torch.autograd.Function):
@@ -223,14 +314,19 @@ class Multihead_Porjection_Layernorm_with_Position_Function(torch.autograd.Funct
         hat_ln, invsigma = gexts.multihead_projection_layernorm_with_position_rrc_forward(
             input, weight, bias, lnw, lnb, norm_eps, position, seqlen, d_model, num_head, dim_head, dim_position,
             batch)
-        ctx.save_for_backward(input, weight, hat_ln, invsigma, lnw, lnb)
+        ctx.save_for_backward(input, weight, bias, lnw)
         ctx.shape_kwargs = [num_head, dim_head, dim_position]
+        ctx.norm_eps = norm_eps
         return hat_ln
 
     @staticmethod
     def backward(ctx: Any, grad_ln: Tensor):
-        raise NotImplementedError(
-            "backward of multihead_projection_layernorm_with_position_rrc_cuda is not built yet")
+        input, weight, bias, lnw = ctx.saved_tensors
+        num_head, dim_head, dim_position = ctx.shape_kwargs
+        batch, seqlen, d_model = input.size()
+        grads = gexts.multihead_projection_layernorm_with_position_rrc_backward(
+            grad_ln, input, weight, bias, lnw, ctx.norm_eps, seqlen, d_model, num_head, dim_head, dim_position, batch)
+        return (*grads, None, None, None, None, None)
 
 
 class Multihead_Galerkin_Attention_cccr_Function(torch.autograd.Function):
@@ -243,7 +339,9 @@ class Multihead_Galerkin_Attention_cccr_Function(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx: Any, grad_Attn):
-        raise NotImplementedError("backward of multihead_galerkin_attention_cccr_cuda is not built yet")
+        Q, K, V = ctx.saved_tensors
+        batch, num_head, d_posk, seqlen = Q.size()
+        return gexts.multihead_galerkin_attention_cccr_backward(grad_Attn, Q, K, V, batch, num_head, d_posk, seqlen)
 
 
 def multihead_projection_with_position_rrc_cuda(input: Tensor, weight: Tensor, bias: Tensor, position: Tensor,
