@@ -161,8 +161,13 @@ template <int D>
 __global__ __launch_bounds__(256) void qm_apply_fm(const float* __restrict__ Q, const float* __restrict__ M,
                                                    float* __restrict__ out, int S, int tokens_per_chunk) {
     constexpr int DP = D - 32;
+    // D == 34: a wave stages the 64 x 34 output rows of a unit in its own LDS slice and writes them
+    // out as one contiguous 8704-byte run (rows of 136 bytes would otherwise go out in 8-byte pieces).
+    constexpr int kStagePitch = 36;
+    __shared__ __attribute__((aligned(16))) float stage_all[DP == 2 ? 4 * 64 * kStagePitch : 4];
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
+    float* stage = stage_all + (DP == 2 ? wave * 64 * kStagePitch : 0);
     const int tk = lane & 15;
     const int g = lane >> 4;
     const int64_t bh = blockIdx.y;
@@ -270,18 +275,15 @@ __global__ __launch_bounds__(256) void qm_apply_fm(const float* __restrict__ Q, 
                 }
                 c0 = rows4_allsum(c0);
                 c1 = rows4_allsum(c1);
-                const int s = sb + 4 * tk + j;
-                if (s < s1) {
-                    float* op = ob + (int64_t)s * D;
-                    if (g == 0)
-                        *reinterpret_cast<float2*>(op) = make_float2(fmaf(p1, mpp[1][0], fmaf(p0, mpp[0][0], c0)),
-                                                                     fmaf(p1, mpp[1][1], fmaf(p0, mpp[0][1], c1)));
+                float* row = stage + (4 * tk + j) * kStagePitch;
+                if (g == 0)
+                    *reinterpret_cast<float2*>(row) = make_float2(fmaf(p1, mpp[1][0], fmaf(p0, mpp[0][0], c0)),
+                                                                  fmaf(p1, mpp[1][1], fmaf(p0, mpp[0][1], c1)));
 #pragma unroll
-                    for (int jb = 0; jb < 2; ++jb) {
-                        float* o = op + DP + jb * 16 + 4 * g;
-                        *reinterpret_cast<float2*>(o) = make_float2(acc[jb][0], acc[jb][1]);
-                        *reinterpret_cast<float2*>(o + 2) = make_float2(acc[jb][2], acc[jb][3]);
-                    }
+                for (int jb = 0; jb < 2; ++jb) {
+                    float* o = row + DP + jb * 16 + 4 * g;
+                    *reinterpret_cast<float2*>(o) = make_float2(acc[jb][0], acc[jb][1]);
+                    *reinterpret_cast<float2*>(o + 2) = make_float2(acc[jb][2], acc[jb][3]);
                 }
             } else {
                 // lanes tk and tk^8 swap halves: each store writes whole 128-byte rows of 8 tokens
@@ -301,6 +303,18 @@ __global__ __launch_bounds__(256) void qm_apply_fm(const float* __restrict__ Q, 
                 const int sy = sx + 32;
                 if (sx < s1) st_stream<true>(reinterpret_cast<float4*>(ob + (int64_t)sx * D + fo), x);
                 if (sy < s1) st_stream<true>(reinterpret_cast<float4*>(ob + (int64_t)sy * D + fo), y);
+            }
+        }
+        if (DP == 2) {
+            // the wave's own LDS slice: program order is enough, no barrier
+            const int ntok = min(64, s1 - sb);
+            float* dst = ob + (int64_t)sb * D;
+            constexpr int R2 = D / 2;  // float2 per token row
+            for (int e = lane; e < ntok * R2; e += 64) {
+                const int tok = e / R2;
+                const int c2 = e - tok * R2;
+                const float2 v = *reinterpret_cast<const float2*>(stage + tok * kStagePitch + 2 * c2);
+                st_stream<true>(reinterpret_cast<float2*>(dst + (int64_t)tok * D + 2 * c2), v);
             }
         }
     };

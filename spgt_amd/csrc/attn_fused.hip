@@ -286,6 +286,11 @@ __global__ __launch_bounds__(256) void qm_apply_tm(
     const float* __restrict__ Q, const float* __restrict__ pos, const float* __restrict__ M,
     float* __restrict__ out, int S, int H, int64_t ld, int tokens_per_chunk) {
     constexpr int D = DP + 32;
+    // DP == 2: output rows of 4 heads x 34 floats are staged in LDS per group of U units and
+    // written out by the whole workgroup as one contiguous run (two buffers, one barrier per group).
+    constexpr int kStagePitch = 4 * D + 4;  // floats per token row in LDS (padding spreads the banks)
+    __shared__ __attribute__((aligned(16))) float stage[DP == 2 ? 2 * U * 16 * kStagePitch : 4];
+    int stage_parity = 0;
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int h = blockIdx.y * 4 + wave;
@@ -339,7 +344,7 @@ __global__ __launch_bounds__(256) void qm_apply_tm(
         return u;
     };
     // `sb` is the first token of the unit (this lane's token is sb + tk, clamped loads aside).
-    auto compute_unit = [&](const Unit& u, int sb) {
+    auto compute_unit = [&](const Unit& u, int sb, int slot) {
         const int s = sb + tk;
         const bool valid = s < s1;
         const float q[8] = {u.q0.x, u.q0.y, u.q0.z, u.q0.w, u.q1.x, u.q1.y, u.q1.z, u.q1.w};
@@ -359,7 +364,6 @@ __global__ __launch_bounds__(256) void qm_apply_tm(
             acc[0] = mfma16(mreg[kk][0], q[kk], acc[0]);
             acc[1] = mfma16(mreg[kk][1], q[kk], acc[1]);
         }
-        float* op = obase + (int64_t)min(s, s1 - 1) * ldo;
         if (DP == 2) {
             float c0 = 0.f, c1 = 0.f;
 #pragma unroll
@@ -369,20 +373,20 @@ __global__ __launch_bounds__(256) void qm_apply_tm(
             }
             c0 = rows4_allsum(c0);
             c1 = rows4_allsum(c1);
-            if (valid) {
-                if (g == 0) {
-                    float2 o;
-                    o.x = fmaf(u.p.y, mpp[1][0], fmaf(u.p.x, mpp[0][0], c0));
-                    o.y = fmaf(u.p.y, mpp[1][1], fmaf(u.p.x, mpp[0][1], c1));
-                    *reinterpret_cast<float2*>(op) = o;
-                }
-#pragma unroll
-                for (int jb = 0; jb < 2; ++jb) {
-                    float* o = op + DP + jb * 16 + 4 * g;
-                    *reinterpret_cast<float2*>(o) = make_float2(acc[jb][0], acc[jb][1]);
-                    *reinterpret_cast<float2*>(o + 2) = make_float2(acc[jb][2], acc[jb][3]);
-                }
+            float* row = stage + ((stage_parity * U + slot) * 16 + tk) * kStagePitch + (h & 3) * D;
+            if (g == 0) {
+                float2 o;
+                o.x = fmaf(u.p.y, mpp[1][0], fmaf(u.p.x, mpp[0][0], c0));
+                o.y = fmaf(u.p.y, mpp[1][1], fmaf(u.p.x, mpp[0][1], c1));
+                *reinterpret_cast<float2*>(row) = o;
             }
+#pragma unroll
+            for (int jb = 0; jb < 2; ++jb) {
+                float* o = row + DP + jb * 16 + 4 * g;
+                *reinterpret_cast<float2*>(o) = make_float2(acc[jb][0], acc[jb][1]);
+                *reinterpret_cast<float2*>(o + 2) = make_float2(acc[jb][2], acc[jb][3]);
+            }
+            (void)valid;
         } else {
             // Lanes tk and tk^8 swap halves so that one store instruction writes
             // whole 128-byte head rows of 8 tokens (non-temporal stores of partial
@@ -423,10 +427,28 @@ __global__ __launch_bounds__(256) void qm_apply_tm(
 #pragma unroll
         for (int u = 0; u < U; ++u) buf[u] = load_unit(min(sg + 16 * u, s1 - 1));
     };
+    // DP == 2: after the group's units are staged, the workgroup copies min(G, s1 - sg) token rows
+    // of 4*D floats (one contiguous run in `out`) with 16-byte stores.
+    auto flush_group = [&](int sg) {
+        if (DP != 2) return;
+        __syncthreads();
+        const int ntok = min(G, s1 - sg);
+        const float* src = stage + stage_parity * U * 16 * kStagePitch;
+        float* dst = out + ((int64_t)b * S + sg) * ldo + (int64_t)(blockIdx.y * 4) * D;
+        constexpr int R4 = D;  // float4 per token row (4 heads x D floats)
+        for (int e = threadIdx.x; e < ntok * R4; e += 256) {
+            const int tok = e / R4;
+            const int c4 = e - tok * R4;
+            const float4 v = *reinterpret_cast<const float4*>(src + tok * kStagePitch + 4 * c4);
+            st_stream<SPGT_NT_P2ST>(reinterpret_cast<float4*>(dst + (int64_t)tok * ldo + 4 * c4), v);
+        }
+        stage_parity ^= 1;
+    };
     auto compute_group = [&](const Unit(&buf)[U], int gi) {
         const int sg = s0 + gi * G;
 #pragma unroll
-        for (int u = 0; u < U; ++u) compute_unit(buf[u], sg + 16 * u);
+        for (int u = 0; u < U; ++u) compute_unit(buf[u], sg + 16 * u, u);
+        flush_group(sg);
     };
     load_group(bufA, 0);
     int gi = 0;
@@ -447,11 +469,7 @@ __global__ __launch_bounds__(256) void qm_apply_tm(
         for (int u = 0; u < U; ++u) bufA[u] = bufB[u];
         ++gi;
     }
-    if (gi < ntot) {
-        const int sg = s0 + gi * G;
-#pragma unroll
-        for (int u = 0; u < U; ++u) compute_unit(bufA[u], sg + 16 * u);
-    }
+    if (gi < ntot) compute_group(bufA, gi);
 }
 
 // ---------------------------------------------------------------------------
