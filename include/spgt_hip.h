@@ -174,6 +174,13 @@ int spgt_spectral_mode_contract(const float* X_ft, const float* weight_1, const 
                                 int H_low, int W_low, int H_base_1, int W_base_1, int H_base_2,
                                 int W_base_2, spgt_stream_t stream);
 
+/* The same contraction on compact operands that hold only the retained modes (for a spectral layer
+ * that obtains them by truncated DFTs instead of full FFTs; no reference counterpart):
+ *   O[n, k*H_low + h, o, w] = sum_i Z[n, k*H_low + h, i, w] * weight_k[h, w, i, o],  k = 0, 1
+ * Z [N, 2*H_low, Cin, W_low], O [N, 2*H_low, Cout, W_low] complex64. */
+int spgt_spectral_modes_compact(const float* Z, const float* weight_1, const float* weight_2, float* O,
+                                int N, int Cin, int Cout, int H_low, int W_low, spgt_stream_t stream);
+
 /* Replaces F.interpolate(x, size, mode='bilinear', align_corners=True) as used by
  * DownScaler2D / UpScaler2D (network/model.py:30, 36, 59, 63):
  * src [planes, H_in, W_in] -> dst [planes, H_out, W_out]. */

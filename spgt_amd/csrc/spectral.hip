@@ -18,6 +18,15 @@ struct SpecWindows {
     int w_base[2];
 };
 
+// Element strides (in complex elements) of the spectrum operands: element (n, c, h, w) of X sits at
+// n*x_n + c*x_c + h*x_h + w*x_w, likewise for the output.  `compact` operands hold only the two
+// windows, stacked along h: row index k*m_h + hh instead of h_base[k] + hh, column ww.
+struct SpecLayout {
+    int64_t x_n, x_c, x_h, x_w;
+    int64_t o_n, o_c, o_h, o_w;
+    int compact;
+};
+
 // out[n, o, hb_k + hh, wb_k + ww] = sum_i X[n, i, hb_k + hh, wb_k + ww] * W_k[hh, ww, i, o]   (complex)
 // grid (m_h * m_w, 2, ceil(Cout/64)), block 256 = 64 output channels x 4 batch groups.
 // One workgroup per mode: the mode's input column X[:, :, h, w] is staged in LDS
@@ -27,8 +36,7 @@ constexpr int kSpecNB = 16;
 
 __global__ __launch_bounds__(256) void spectral_mode_contract_k(
     const float2* __restrict__ X, const float2* __restrict__ W0, const float2* __restrict__ W1,
-    float2* __restrict__ out, int N, int Cin, int Cout, int H_all, int W_all, int m_h, int m_w,
-    SpecWindows win) {
+    float2* __restrict__ out, int N, int Cin, int Cout, int m_h, int m_w, SpecWindows win, SpecLayout lay) {
     extern __shared__ float2 xs[];  // [kSpecNB][Cin]
     const int mode = blockIdx.x;
     const int k = blockIdx.y;
@@ -37,13 +45,16 @@ __global__ __launch_bounds__(256) void spectral_mode_contract_k(
     const int h = win.h_base[k] + hh;
     const int w = win.w_base[k] + ww;
     // Where the windows overlap the second one wins (the reference assigns it last).
-    if (k == 0 && h >= win.h_base[1] && h < win.h_base[1] + m_h && w >= win.w_base[1] && w < win.w_base[1] + m_w)
+    if (!lay.compact && k == 0 && h >= win.h_base[1] && h < win.h_base[1] + m_h && w >= win.w_base[1] &&
+        w < win.w_base[1] + m_w)
         return;
     const int o = blockIdx.z * 64 + (threadIdx.x & 63);
     const int ng = threadIdx.x >> 6;
     const float2* Wm = (k == 0 ? W0 : W1) + (int64_t)mode * Cin * Cout;
-    const int64_t plane = (int64_t)H_all * W_all;
-    const int64_t pix = (int64_t)h * W_all + w;
+    const int he = lay.compact ? k * m_h + hh : h;
+    const int we = lay.compact ? ww : w;
+    const int64_t xpix = he * lay.x_h + we * lay.x_w;
+    const int64_t opix = he * lay.o_h + we * lay.o_w;
 
     for (int n0 = 0; n0 < N; n0 += kSpecNB) {
         const int nb = min(kSpecNB, N - n0);
@@ -51,13 +62,14 @@ __global__ __launch_bounds__(256) void spectral_mode_contract_k(
         for (int e = threadIdx.x; e < nb * Cin; e += 256) {
             const int n = e / Cin;
             const int i = e - n * Cin;
-            xs[e] = X[((int64_t)(n0 + n) * Cin + i) * plane + pix];
+            xs[e] = X[(n0 + n) * lay.x_n + i * lay.x_c + xpix];
         }
         __syncthreads();
         float2 acc[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[j] = make_float2(0.f, 0.f);
         if (o < Cout) {
+#pragma unroll 8
             for (int i = 0; i < Cin; ++i) {
                 const float2 wv = Wm[(int64_t)i * Cout + o];
 #pragma unroll
@@ -75,7 +87,7 @@ __global__ __launch_bounds__(256) void spectral_mode_contract_k(
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const int n = ng + 4 * j;
-                if (n < nb) out[((int64_t)(n0 + n) * Cout + o) * plane + pix] = acc[j];
+                if (n < nb) out[(n0 + n) * lay.o_n + o * lay.o_c + opix] = acc[j];
             }
         }
     }
@@ -152,11 +164,36 @@ extern "C" int spgt_spectral_mode_contract(const float* X_ft, const float* weigh
     hipLaunchKernelGGL(spectrum_zero_outside_k, dim3(fill_blocks), dim3(256), 0, stream,
                        reinterpret_cast<float2*>(Out_ft), total, H_all, W_all, H_low, W_low, win);
     const dim3 grid(H_low * W_low, 2, ceil_div(Cout, 64));
+    const int64_t plane = (int64_t)H_all * W_all;
+    const SpecLayout lay{Cin * plane, plane, W_all, 1, Cout * plane, plane, W_all, 1, 0};
     hipLaunchKernelGGL(spectral_mode_contract_k, grid, dim3(256), (size_t)kSpecNB * Cin * sizeof(float2), stream,
                        reinterpret_cast<const float2*>(X_ft), reinterpret_cast<const float2*>(weight_1),
                        reinterpret_cast<const float2*>(weight_2), reinterpret_cast<float2*>(Out_ft), N, Cin, Cout,
-                       H_all, W_all, H_low, W_low, win);
+                       H_low, W_low, win, lay);
     return check_launch("spectral_mode_contract");
+}
+
+extern "C" int spgt_spectral_modes_compact(const float* Z, const float* weight_1, const float* weight_2, float* O,
+                                           int N, int Cin, int Cout, int H_low, int W_low, hipStream_t stream) {
+    if (!Z || !weight_1 || !weight_2 || !O)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "spectral_modes_compact: null pointer argument");
+    if (N <= 0 || Cin <= 0 || Cout <= 0 || H_low <= 0 || W_low <= 0)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "spectral_modes_compact: sizes must be positive");
+    if ((size_t)kSpecNB * Cin * sizeof(float2) > 64 * 1024)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "spectral_modes_compact: Cin above 512 is not supported");
+    if (Z == O) return fail(SPGT_ERR_INVALID_ARGUMENT, "spectral_modes_compact: in-place call is not supported");
+    if (!aligned8(Z) || !aligned8(weight_1) || !aligned8(weight_2) || !aligned8(O))
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "spectral_modes_compact: complex operands must be 8-byte aligned");
+    // Z [N, 2*H_low, Cin, W_low], O [N, 2*H_low, Cout, W_low]
+    const SpecWindows win{{0, 0}, {0, 0}};
+    const SpecLayout lay{(int64_t)2 * H_low * Cin * W_low, W_low, (int64_t)Cin * W_low, 1,
+                         (int64_t)2 * H_low * Cout * W_low, W_low, (int64_t)Cout * W_low, 1, 1};
+    const dim3 grid(H_low * W_low, 2, ceil_div(Cout, 64));
+    hipLaunchKernelGGL(spectral_mode_contract_k, grid, dim3(256), (size_t)kSpecNB * Cin * sizeof(float2), stream,
+                       reinterpret_cast<const float2*>(Z), reinterpret_cast<const float2*>(weight_1),
+                       reinterpret_cast<const float2*>(weight_2), reinterpret_cast<float2*>(O), N, Cin, Cout, H_low,
+                       W_low, win, lay);
+    return check_launch("spectral_modes_compact");
 }
 
 extern "C" int spgt_bilinear_align_corners(const float* src, float* dst, int planes, int H_in, int W_in, int H_out,

@@ -99,6 +99,29 @@ def _spectral_mode_contract(X_ft: Tensor, weight_1: Tensor, weight_2: Tensor, H_
     return out
 
 
+def _spectral_modes_compact(Z: Tensor, weight_1: Tensor, weight_2: Tensor) -> Tensor:
+    """Z complex64 [N, 2*m_h, Cin, m_w] (the two retained windows stacked along the second axis);
+    weight_k fp32 [m_h, m_w, Cin, Cout, 2] -> complex64 [N, 2*m_h, Cout, m_w]."""
+    require_gpu_f32("Z", Z, torch.complex64)
+    ws = []
+    for name, w in (("weight_1", weight_1), ("weight_2", weight_2)):
+        if w.is_complex():
+            w = torch.view_as_real(w)
+        require_gpu_f32(name, w)
+        ws.append(w)
+    m_h, m_w, Cin, Cout, _ = ws[0].shape
+    if tuple(ws[1].shape) != tuple(ws[0].shape):
+        raise ValueError("weight_1 and weight_2 must have the same shape")
+    N = Z.shape[0]
+    if tuple(Z.shape) != (N, 2 * m_h, Cin, m_w):
+        raise ValueError(f"Z has shape {tuple(Z.shape)}, expected {(N, 2 * m_h, Cin, m_w)}")
+    out = torch.empty((N, 2 * m_h, Cout, m_w), dtype=torch.complex64, device=Z.device)
+    with torch.cuda.device(Z.device):
+        check(_lib.load().spgt_spectral_modes_compact(ptr(Z), ptr(ws[0]), ptr(ws[1]), ptr(out), N, Cin, Cout, m_h,
+                                                      m_w, stream_of(Z)))
+    return out
+
+
 def _bilinear_align_corners(X: Tensor, size) -> Tensor:
     """X [..., H_in, W_in] -> [..., H_out, W_out], F.interpolate(mode='bilinear', align_corners=True)."""
     require_gpu_f32("X", X)
@@ -122,6 +145,7 @@ dexts = SimpleNamespace(
     transpose_gather_dual=_transpose_gather_dual,
     transpose_scatter_dual=_transpose_scatter_dual,
     spectral_mode_contract=_spectral_mode_contract,
+    spectral_modes_compact=_spectral_modes_compact,
     bilinear_align_corners=_bilinear_align_corners,
 )
 
@@ -189,6 +213,11 @@ def spectral_mode_contract(X_ft: Tensor, weight_1: Tensor, weight_2: Tensor, H_l
     into a zero-filled spectrum, in one call (inference only: no autograd graph is recorded)."""
     return dexts.spectral_mode_contract(X_ft.detach(), weight_1.detach(), weight_2.detach(), H_low, W_low, H_base_1,
                                         W_base_1, H_base_2, W_base_2)
+
+
+def spectral_modes_compact(Z: Tensor, weight_1: Tensor, weight_2: Tensor) -> Tensor:
+    """Per-mode complex channel contraction on operands that hold only the retained modes (inference only)."""
+    return dexts.spectral_modes_compact(Z.detach(), weight_1.detach(), weight_2.detach())
 
 
 def bilinear_align_corners(X: Tensor, size) -> Tensor:

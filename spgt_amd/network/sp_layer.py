@@ -29,6 +29,7 @@ from ..extension.bind.datamove import (batched_transpose, spectral_mode_contract
 from ..extension.bind.galerkin_attention import (galerkin_attention_fused, multihead_galerkin_attention_cccr_cuda,
                                                  multihead_projection_layernorm_with_position_rrc_cuda,
                                                  multihead_projection_with_position_rrc_cuda)
+from . import truncated_dft
 from .layer import FeedForward, always_dropout, make_activation
 
 
@@ -132,6 +133,9 @@ class Sp_EncoderLayer(nn.Module):
 
 
 class Sp_SpectralConv2D(nn.Module):
+    # inference path: truncated DFTs as matrix products instead of rfft2 / irfft2 (see truncated_dft.py)
+    use_truncated_dft = True
+
     def __init__(self, in_dim, out_dim, mode, droprate, activation) -> None:
         super().__init__()
         self.in_dim, self.out_dim, self.mode, self.droprate = in_dim, out_dim, mode, droprate
@@ -149,10 +153,15 @@ class Sp_SpectralConv2D(nn.Module):
         m, cout = self.mode, self.out_dim
         res = self.residual_layer(X)
         X = always_dropout(X, self.droprate)
+        needs_graph = torch.is_grad_enabled() and (X.requires_grad or self.fourier_weight[0].requires_grad)
+        if self.use_truncated_dft and not needs_graph and truncated_dft.supported(r, m):
+            # only the retained modes are ever computed: no FFT, no transposes, no full-size spectrum
+            Y = truncated_dft.spectral_modes_apply(X.contiguous(), self.fourier_weight[0], self.fourier_weight[1], m)
+            return self.activation_layer(Y + res)
         X = batched_transpose(X, [N], [r, r], [cin])  # -> [N, in_dim, r, r]
         X_ft = torch.fft.rfft2(X, s=(r, r), norm="ortho")
         w_all = r // 2 + 1
-        if torch.is_grad_enabled() and (X.requires_grad or self.fourier_weight[0].requires_grad):
+        if needs_graph:
             g0, g1 = transpose_gather_dual(X_ft, [N, cin], r, w_all, m, m, 0, 0, r - m, 0)
             o0 = g0 @ torch.view_as_complex(self.fourier_weight[0])
             o1 = g1 @ torch.view_as_complex(self.fourier_weight[1])

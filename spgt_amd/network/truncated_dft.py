@@ -1,0 +1,72 @@
+"""Truncated 2-D DFTs for the spectral layer.
+
+Sp_SpectralConv2D keeps only the modes kh in [0, m) and [r-m, r), kw in [0, m) of rfft2(x) and feeds
+irfft2 a spectrum that is zero everywhere else (reference: network/sp_layer.py:138-150).  Computing
+exactly those modes as two small matrix products per direction,
+
+    forward   Y[n,h,c,kw]  = sum_w x[n,h,w,c] e^{-2 pi i kw w / r} / sqrt(r)
+              Z[n,kh,c,kw] = sum_h Y[n,h,c,kw] e^{-2 pi i kh h / r} / sqrt(r)
+    inverse   U[n,h,o,kw]  = sum_kh O[n,kh,o,kw] e^{+2 pi i kh h / r} / sqrt(r)
+              y[n,h,w,o]   = Re sum_kw c_kw U[n,h,o,kw] e^{+2 pi i kw w / r} / sqrt(r),   c_0 = 1, c_kw = 2
+                             (c = 1 as well for the Nyquist column of an even r),
+
+gives the same result as the FFT route up to fp32 rounding (the real part in the last line is what the
+complex-to-real transform of irfft2 computes from a half spectrum), works directly on the [N, r, r, C]
+layout of the module - both full-tensor transposes, the full-size spectra, the corner gather/scatter and
+the zero fill disappear - and does not depend on r having small prime factors (r = 211 is prime).
+The four products are library GEMMs; the per-mode channel contraction between them is the HIP kernel
+behind `spectral_modes_compact`.
+"""
+import math
+from typing import Dict, Tuple
+
+import torch
+from torch import Tensor
+
+from ..extension.bind.datamove import spectral_modes_compact
+
+_TABLES: Dict[Tuple[int, int, str], Tuple[Tensor, Tensor, Tensor, Tensor]] = {}
+
+
+def dft_tables(r: int, m: int, device) -> Tuple[Tensor, Tensor, Tensor, Tensor]:
+    """(Fw [r, 2m] real, Gh [2m, r] complex, Ghi [r, 2m] complex, Fwi [r, 2m] real), built in fp64."""
+    key = (r, m, str(device))
+    if key not in _TABLES:
+        idx = torch.arange(r, dtype=torch.float64)
+        kw = torch.arange(m, dtype=torch.float64)
+        kh = torch.cat([torch.arange(m), torch.arange(r - m, r)]).to(torch.float64)
+        s = 1.0 / math.sqrt(r)
+        ang_w = 2.0 * math.pi * idx[:, None] * kw[None, :] / r                  # [r, m]
+        fw = torch.stack([torch.cos(ang_w), -torch.sin(ang_w)], dim=-1) * s      # columns (kw, re|im)
+        c = torch.full((m,), 2.0, dtype=torch.float64)
+        c[0] = 1.0
+        if r % 2 == 0 and m - 1 == r // 2:
+            c[-1] = 1.0
+        fwi = torch.stack([torch.cos(ang_w) * c, -torch.sin(ang_w) * c], dim=-1) * s
+        ang_h = 2.0 * math.pi * kh[:, None] * idx[None, :] / r                  # [2m, r]
+        gh = torch.complex(torch.cos(ang_h), -torch.sin(ang_h)) * s
+        ghi = torch.complex(torch.cos(ang_h), torch.sin(ang_h)).t() * s
+        _TABLES[key] = (fw.reshape(r, 2 * m).float().to(device).contiguous(),
+                        gh.to(torch.complex64).to(device).contiguous(),
+                        ghi.to(torch.complex64).to(device).contiguous(),
+                        fwi.reshape(r, 2 * m).float().to(device).contiguous())
+    return _TABLES[key]
+
+
+def supported(r: int, m: int) -> bool:
+    """The two retained row windows must not overlap."""
+    return 2 * m <= r
+
+
+def spectral_modes_apply(x: Tensor, weight_1: Tensor, weight_2: Tensor, m: int) -> Tensor:
+    """x [N, r, r, Cin] -> irfft2(W . truncate(rfft2(x))) as [N, r, r, Cout] (norm='ortho')."""
+    N, r, _, cin = x.shape
+    cout = weight_1.shape[3]
+    fw, gh, ghi, fwi = dft_tables(r, m, x.device)
+    y = torch.matmul(x.reshape(N * r, r, cin).transpose(1, 2), fw)                       # [N r, Cin, 2m]
+    yc = torch.view_as_complex(y.view(N, r, cin, m, 2)).reshape(N, r, cin * m)
+    z = torch.matmul(gh, yc).view(N, 2 * m, cin, m)                                      # [N, 2m, Cin, m]
+    o = spectral_modes_compact(z, weight_1, weight_2)                                    # [N, 2m, Cout, m]
+    u = torch.matmul(ghi, o.view(N, 2 * m, cout * m))                                    # [N, r, Cout m]
+    ur = torch.view_as_real(u).view(N * r, cout, 2 * m)
+    return torch.matmul(fwi, ur.transpose(1, 2)).view(N, r, r, cout)

@@ -166,3 +166,39 @@ def test_datamove_argument_validation(gpu):
         dm.transpose_gather_dual(c, [2], 4, 4, 3, 3, 0, 0, 2, 0)  # second window leaves the plane
     with pytest.raises(TypeError):
         dm.batched_transpose(x.double(), [1], [4], [4])
+
+
+@pytest.mark.parametrize("N,Cin,Cout,m", [(1, 1, 1, 1), (2, 6, 4, 3), (8, 64, 64, 12), (17, 20, 70, 4)])
+def test_spectral_modes_compact_vs_einsum(gpu, N, Cin, Cout, m):
+    z = torch.view_as_complex(rnd(N, 2 * m, Cin, m, 2, seed=21))
+    w1, w2 = rnd(m, m, Cin, Cout, 2, seed=22) / Cin, rnd(m, m, Cin, Cout, 2, seed=23) / Cin
+    wc = torch.cat([torch.view_as_complex(w1.double()), torch.view_as_complex(w2.double())], 0)  # [2m, m, Cin, Cout]
+    want = torch.einsum("nhiw,hwio->nhow", z.to(torch.complex128), wc)
+    got = dm.spectral_modes_compact(z.to(gpu), w1.to(gpu), w2.to(gpu))
+    assert got.shape == (N, 2 * m, Cout, m)
+    assert max_rel(torch.view_as_real(got.cpu()).double(), torch.view_as_real(want)) < 1e-5
+
+
+@pytest.mark.parametrize("N,r,Cin,Cout,m", [(2, 9, 6, 4, 3), (8, 141, 64, 64, 12), (4, 211, 64, 64, 12), (3, 16, 8, 8, 8),
+                                             (2, 30, 5, 7, 15)])
+def test_truncated_dft_spectral_layer_vs_oracle(gpu, N, r, Cin, Cout, m):
+    """The DFT-as-matrix-product route of the spectral layer against the oracle's rfft2 / irfft2 route (fp64)."""
+    from spgt_amd.network import truncated_dft as T
+    x = rnd(N, r, r, Cin, seed=24)
+    w1, w2 = rnd(m, m, Cin, Cout, 2, seed=25) / Cin, rnd(m, m, Cin, Cout, 2, seed=26) / Cin
+    p = {"residual_layer.weight": torch.zeros(Cout, Cin, dtype=torch.float64),
+         "residual_layer.bias": torch.zeros(Cout, dtype=torch.float64),
+         "fourier_weight.0": w1.double(), "fourier_weight.1": w2.double()}
+
+    xf = torch.fft.rfft2(x.double().permute(0, 3, 1, 2), s=(r, r), norm="ortho")
+    of = torch.zeros(N, Cout, r, r // 2 + 1, dtype=torch.complex128)
+    of[:, :, :m, :m] = torch.einsum("nihw,hwio->nohw", xf[:, :, :m, :m], torch.view_as_complex(w1.double()))
+    of[:, :, r - m:, :m] = torch.einsum("nihw,hwio->nohw", xf[:, :, r - m:, :m], torch.view_as_complex(w2.double()))
+    want = torch.fft.irfft2(of, s=(r, r), norm="ortho").permute(0, 2, 3, 1)
+    assert T.supported(r, m)
+    got = T.spectral_modes_apply(x.to(gpu), w1.to(gpu), w2.to(gpu), m)
+    assert got.shape == (N, r, r, Cout)
+    assert max_rel(got.cpu().double(), want) < 1e-5
+    # and the oracle's own module function agrees with the hand-written FFT reference above
+    relu_want = O.spectral_conv2d(p, x.double(), m, "relu", weight_layout="sp")
+    assert max_rel(relu_want, torch.relu(want)) < 1e-10

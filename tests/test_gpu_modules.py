@@ -52,6 +52,10 @@ def test_spectral_conv_golden(gpu):
     assert max_rel(got.cpu(), want) < TOL
     graph_path = m(i["x"].to(gpu))  # autograd enabled: gather, complex matmul, scatter
     assert max_rel(graph_path.detach().cpu(), want) < TOL
+    m.use_truncated_dft = False  # inference through rfft2 / irfft2 and the full-spectrum contraction kernel
+    with torch.no_grad():
+        fft_path = m(i["x"].to(gpu))
+    assert max_rel(fft_path.cpu(), want) < TOL
 
 
 def test_scalers_golden(gpu):
