@@ -187,6 +187,11 @@ int spgt_spectral_modes_compact(const float* Z, const float* weight_1, const flo
 int spgt_bilinear_align_corners(const float* src, float* dst, int planes, int H_in, int W_in,
                                 int H_out, int W_out, spgt_stream_t stream);
 
+/* The same resampling fused with the NCHW -> NHWC permute that follows it in UpScaler2D.forward
+ * (network/model.py:63-64): src [N, C, H_in, W_in] -> dst [N, H_out, W_out, C]. */
+int spgt_bilinear_align_corners_nhwc(const float* src, float* dst, int N, int C, int H_in, int W_in,
+                                     int H_out, int W_out, spgt_stream_t stream);
+
 /* Instrumented variant of spgt_galerkin_attention_fused_forward for benchmarks
  * (no reference counterpart): runs the call `iterations` times, synchronising
  * after each, with HIP events recorded on `stream` around each of its three

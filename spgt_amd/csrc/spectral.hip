@@ -136,6 +136,58 @@ __global__ __launch_bounds__(256) void bilinear_align_corners_k(const float* __r
     }
 }
 
+// The same resampling with a channels-last result: src [N, C, Hin, Win] -> dst [N, Hout, Wout, C].
+// grid (ceil(Wout/32), Hout, N), block 256 = 32 output columns x 8 channel lanes.  Reads run along the
+// source rows of one channel, a 32 x 32 (channel x column) tile is turned in LDS, writes run along C.
+__global__ __launch_bounds__(256) void bilinear_align_corners_nhwc_k(const float* __restrict__ src,
+                                                                     float* __restrict__ dst, int C, int Hin,
+                                                                     int Win, int Hout, int Wout, float hscale,
+                                                                     float wscale) {
+    __shared__ float tile[32 * 33];
+    const int tx = threadIdx.x & 31;
+    const int ty = threadIdx.x >> 5;
+    const int ox = blockIdx.x * 32 + tx;
+    const int oy = blockIdx.y;
+    const int64_t n = blockIdx.z;
+    const float hr = hscale * (float)oy;
+    const int h1 = (int)hr;
+    const int hp = (h1 < Hin - 1) ? 1 : 0;
+    const float h1l = hr - (float)h1;
+    const float h0l = 1.0f - h1l;
+    const int oxc = min(ox, Wout - 1);
+    const float wr = wscale * (float)oxc;
+    const int w1 = (int)wr;
+    const int wp = (w1 < Win - 1) ? 1 : 0;
+    const float w1l = wr - (float)w1;
+    const float w0l = 1.0f - w1l;
+    const int64_t plane = (int64_t)Hin * Win;
+    const float* base = src + n * C * plane + (int64_t)h1 * Win + w1;
+    float* drow = dst + ((n * Hout + oy) * (int64_t)Wout) * C;
+    for (int c0 = 0; c0 < C; c0 += 32) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int cl = 8 * i + ty;
+            float v = 0.f;
+            if (c0 + cl < C) {
+                const float* r0 = base + (int64_t)(c0 + cl) * plane;
+                const float* r1 = r0 + (int64_t)hp * Win;
+                const float top = w0l * r0[0] + w1l * r0[wp];
+                const float bot = w0l * r1[0] + w1l * r1[wp];
+                v = h0l * top + h1l * bot;
+            }
+            tile[cl * 33 + tx] = v;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int xl = 8 * i + ty;
+            const int x = blockIdx.x * 32 + xl;
+            if (x < Wout && c0 + tx < C) drow[(int64_t)x * C + c0 + tx] = tile[tx * 33 + xl];
+        }
+        __syncthreads();
+    }
+}
+
 }  // namespace spgt
 
 using namespace spgt;
@@ -211,4 +263,21 @@ extern "C" int spgt_bilinear_align_corners(const float* src, float* dst, int pla
     hipLaunchKernelGGL(bilinear_align_corners_k, grid, dim3(64, 4), 0, stream, src, dst, planes, H_in, W_in, H_out,
                        W_out, hscale, wscale);
     return check_launch("bilinear_align_corners");
+}
+
+extern "C" int spgt_bilinear_align_corners_nhwc(const float* src, float* dst, int N, int C, int H_in, int W_in,
+                                                int H_out, int W_out, hipStream_t stream) {
+    if (!src || !dst) return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear_align_corners_nhwc: null pointer argument");
+    if (N <= 0 || C <= 0 || H_in <= 0 || W_in <= 0 || H_out <= 0 || W_out <= 0)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear_align_corners_nhwc: sizes must be positive");
+    if (H_out > 65535 || N > 65535)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear_align_corners_nhwc: N or H_out exceeds 65535");
+    if (!aligned4(src) || !aligned4(dst))
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear_align_corners_nhwc: operands must be 4-byte aligned");
+    const float hscale = H_out > 1 ? (float)(H_in - 1) / (float)(H_out - 1) : 0.f;
+    const float wscale = W_out > 1 ? (float)(W_in - 1) / (float)(W_out - 1) : 0.f;
+    const dim3 grid(ceil_div(W_out, 32), H_out, N);
+    hipLaunchKernelGGL(bilinear_align_corners_nhwc_k, grid, dim3(256), 0, stream, src, dst, C, H_in, W_in, H_out,
+                       W_out, hscale, wscale);
+    return check_launch("bilinear_align_corners_nhwc");
 }

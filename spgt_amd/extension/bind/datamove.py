@@ -140,7 +140,24 @@ def _bilinear_align_corners(X: Tensor, size) -> Tensor:
     return out
 
 
+def _bilinear_align_corners_nhwc(X: Tensor, size) -> Tensor:
+    """X [N, C, H_in, W_in] -> [N, H_out, W_out, C]: the resampling and the permute to channels-last in one pass."""
+    require_gpu_f32("X", X)
+    if X.dim() != 4:
+        raise ValueError("X must be [N, C, H, W]")
+    H_out, W_out = (size, size) if isinstance(size, int) else tuple(size)
+    N, C, H_in, W_in = X.shape
+    out = torch.empty((N, H_out, W_out, C), dtype=X.dtype, device=X.device)
+    if out.numel() == 0:
+        return out
+    with torch.cuda.device(X.device):
+        check(_lib.load().spgt_bilinear_align_corners_nhwc(ptr(X), ptr(out), N, C, H_in, W_in, H_out, W_out,
+                                                            stream_of(X)))
+    return out
+
+
 dexts = SimpleNamespace(
+    bilinear_align_corners_nhwc=_bilinear_align_corners_nhwc,
     batched_transpose=_batched_transpose,
     transpose_gather_dual=_transpose_gather_dual,
     transpose_scatter_dual=_transpose_scatter_dual,
@@ -223,3 +240,8 @@ def spectral_modes_compact(Z: Tensor, weight_1: Tensor, weight_2: Tensor) -> Ten
 def bilinear_align_corners(X: Tensor, size) -> Tensor:
     """F.interpolate(X, size, mode='bilinear', align_corners=True) (inference only)."""
     return dexts.bilinear_align_corners(X.detach(), size)
+
+
+def bilinear_align_corners_nhwc(X: Tensor, size) -> Tensor:
+    """F.interpolate(X, size, mode='bilinear', align_corners=True).permute(0, 2, 3, 1), contiguous (inference only)."""
+    return dexts.bilinear_align_corners_nhwc(X.detach(), size)

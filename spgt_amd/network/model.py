@@ -7,7 +7,7 @@ import torch
 import torch.nn.functional as F
 from torch import Tensor, nn
 
-from ..extension.bind.datamove import bilinear_align_corners
+from ..extension.bind.datamove import bilinear_align_corners, bilinear_align_corners_nhwc
 from .layer import ConvResBlock2D, always_dropout, make_activation
 
 
@@ -16,6 +16,21 @@ def resample(X: Tensor, size) -> Tensor:
     if torch.is_grad_enabled() and X.requires_grad:
         return F.interpolate(X, size=tuple(size), mode="bilinear", align_corners=True)
     return bilinear_align_corners(X.contiguous(), tuple(size))
+
+
+def resample_to_nhwc(X: Tensor, size) -> Tensor:
+    """Bilinear, align_corners=True, [N, C, H, W] -> [N, H', W', C] (contiguous)."""
+    if torch.is_grad_enabled() and X.requires_grad:
+        return F.interpolate(X, size=tuple(size), mode="bilinear", align_corners=True).permute(0, 2, 3, 1)
+    return bilinear_align_corners_nhwc(X.contiguous(), tuple(size))
+
+
+def nhwc_to_nchw(X: Tensor) -> Tensor:
+    """[N, H, W, C] -> [N, C, H, W] with plain row-major strides.  For C == 1 the permuted view is already
+    dense but its strides look channels-last, which makes the convolution library answer in channels-last."""
+    N, H, W, C = X.shape
+    X = X.permute(0, 3, 1, 2).contiguous()
+    return X.as_strided((N, C, H, W), (C * H * W, H * W, W, 1))
 
 
 class DownScaler2D(nn.Module):
@@ -34,13 +49,13 @@ class DownScaler2D(nn.Module):
         self.activation_layer = make_activation(activation)
 
     def forward(self, X: Tensor) -> Tensor:
-        X = self.conv0(X.permute(0, 3, 1, 2))
+        X = self.conv0(nhwc_to_nchw(X))
         X = self.activation_layer(resample(X, self.resolution_size[1]))
         X1 = self.conv1(X)
         X2 = self.conv2(X1)
         X3 = self.conv3(X2)
-        X = self.activation_layer(resample(torch.cat([X1, X2, X3], dim=1), self.resolution_size[2]))
-        return X.permute(0, 2, 3, 1)
+        # the activation commutes with the permute, so the second resampling can write channels-last directly
+        return self.activation_layer(resample_to_nhwc(torch.cat([X1, X2, X3], dim=1), self.resolution_size[2]))
 
 
 class UpScaler2D(nn.Module):
@@ -56,5 +71,4 @@ class UpScaler2D(nn.Module):
     def forward(self, X: Tensor) -> Tensor:
         X = resample(X.permute(0, 3, 1, 2), self.resolution_size[3])
         X = self.activation_layer(always_dropout(self.conv(X), self.droprate))
-        X = resample(X, self.resolution_size[4])
-        return X.permute(0, 2, 3, 1)
+        return resample_to_nhwc(X, self.resolution_size[4])

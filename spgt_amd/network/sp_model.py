@@ -37,7 +37,7 @@ class Sp_EncoderMixer(nn.Module):
     def forward(self, X: Tensor, position: Tensor) -> Tensor:
         """X [N, ra, ra, dim_hidden], position [N, ra, ra, dim_position] -> [N, ra, ra, dim_hidden]."""
         N, ra, _, C = X.size()
-        X = X.reshape(N, ra * ra, C)
+        X = X.reshape(N, ra * ra, C).contiguous()  # a strided residual stream would be re-copied by every Linear
         position = position.reshape(N, ra * ra, position.size(-1))
         for layer in self.layers:
             X = layer(X, position)
@@ -57,7 +57,9 @@ class Sp_DecoderRegressor(nn.Module):
 
     def forward(self, X: Tensor, grid: Tensor = None) -> Tensor:
         """X [N, r, r, dim_hidden], grid [N, r, r, dim_position] -> [N, r, r, dim_target]."""
-        X = self.spatial_fc_layer(torch.cat([X, grid], dim=-1))
+        # Linear(cat([X, grid])) without materialising the concatenation: W = [W_x | W_grid]
+        W, dim_x = self.spatial_fc_layer.weight, X.size(-1)
+        X = F.linear(X, W[:, :dim_x], self.spatial_fc_layer.bias) + F.linear(grid, W[:, dim_x:])
         for layer in self.layers:
             X = layer(X)
         return self.ffn_layer(X)

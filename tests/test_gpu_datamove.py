@@ -202,3 +202,14 @@ def test_truncated_dft_spectral_layer_vs_oracle(gpu, N, r, Cin, Cout, m):
     # and the oracle's own module function agrees with the hand-written FFT reference above
     relu_want = O.spectral_conv2d(p, x.double(), m, "relu", weight_layout="sp")
     assert max_rel(relu_want, torch.relu(want)) < 1e-10
+
+
+@pytest.mark.parametrize("shape,size", [((2, 3, 7, 9), (7, 9)), ((2, 3, 7, 9), (4, 5)), ((1, 128, 122, 122), (211, 211)),
+                                        ((2, 130, 16, 33), (40, 65)), ((1, 1, 5, 5), (1, 1)), ((3, 40, 9, 9), (9, 70))])
+def test_bilinear_nhwc_matches_nchw_kernel(gpu, shape, size):
+    """The channels-last variant is the planar kernel followed by a permute, value for value."""
+    x = rnd(*shape, seed=30).to(gpu)
+    want = dm.bilinear_align_corners(x, size).permute(0, 2, 3, 1)
+    got = dm.bilinear_align_corners_nhwc(x, size)
+    assert got.is_contiguous() and got.shape == want.shape
+    assert torch.equal(got, want)
