@@ -158,9 +158,58 @@ __global__ __launch_bounds__(256) void ktv_ln_partial_tm(
 #pragma unroll
         for (int u = 0; u < U; ++u) buf[u] = load_unit(kg, vg, pg, (uint32_t)(4 * u + t));
     };
+    // A full group normalises its 2*U (token, tensor) pairs in lock-step; each
+    // value sees the same operations in the same order as in ln_pair.
     auto compute_full = [&](const KtvUnit<DP>(&buf)[U]) {
+        constexpr int N = 2 * U;
+        float x0[N], x1[N], red[N];
 #pragma unroll
-        for (int u = 0; u < U; ++u) compute_unit(buf[u], true);
+        for (int u = 0; u < U; ++u) {
+            x0[2 * u] = buf[u].k.x;
+            x1[2 * u] = buf[u].k.y;
+            x0[2 * u + 1] = buf[u].v.x;
+            x1[2 * u + 1] = buf[u].v.y;
+        }
+#pragma unroll
+        for (int i = 0; i < N; ++i) red[i] = x0[i] + x1[i];
+        row16_allsum_n(red);
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
+            const float mean = red[i] * (1.0f / 32.0f);
+            x0[i] -= mean;
+            x1[i] -= mean;
+            red[i] = fmaf(x1[i], x1[i], x0[i] * x0[i]);
+        }
+        row16_allsum_n(red);
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
+            const float rstd = __builtin_amdgcn_rsqf(fmaf(red[i], 1.0f / 32.0f, eps));
+            const bool isv = i & 1;
+            x0[i] = fmaf(x0[i] * rstd, isv ? gV0 : gK0, isv ? bV0 : bK0);
+            x1[i] = fmaf(x1[i] * rstd, isv ? gV1 : gK1, isv ? bV1 : bK1);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const float yk0 = x0[2 * u], yk1 = x1[2 * u], yv0 = x0[2 * u + 1], yv1 = x1[2 * u + 1];
+            acc[0][0] = mfma16(yk0, yv0, acc[0][0]);
+            acc[0][1] = mfma16(yk0, yv1, acc[0][1]);
+            acc[1][0] = mfma16(yk1, yv0, acc[1][0]);
+            acc[1][1] = mfma16(yk1, yv1, acc[1][1]);
+            if (DP == 2) {
+                const float2 pz = buf[u].p;
+                kp[0][0] = fmaf(yk0, pz.x, kp[0][0]);
+                kp[0][1] = fmaf(yk0, pz.y, kp[0][1]);
+                kp[1][0] = fmaf(yk1, pz.x, kp[1][0]);
+                kp[1][1] = fmaf(yk1, pz.y, kp[1][1]);
+                pv[0][0] = fmaf(pz.x, yv0, pv[0][0]);
+                pv[0][1] = fmaf(pz.x, yv1, pv[0][1]);
+                pv[1][0] = fmaf(pz.y, yv0, pv[1][0]);
+                pv[1][1] = fmaf(pz.y, yv1, pv[1][1]);
+                pp[0] = fmaf(pz.x, pz.x, pp[0]);
+                pp[1] = fmaf(pz.x, pz.y, pp[1]);
+                pp[2] = fmaf(pz.y, pz.y, pp[2]);
+            }
+        }
     };
     if (nfull > 0) {
         load_group(bufA, 0);

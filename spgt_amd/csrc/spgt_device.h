@@ -43,6 +43,21 @@ __device__ __forceinline__ float row16_allsum(float v) {
     return v;
 }
 
+// The same sum for N independent values, one DPP step at a time across all of
+// them: a DPP result needs two wait states before its consumer, and stepping the
+// values in lock-step fills those slots with the neighbours' steps.
+template <int N>
+__device__ __forceinline__ void row16_allsum_n(float (&v)[N]) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) v[i] += dpp_move<SPGT_DPP_QUAD_XOR1>(v[i]);
+#pragma unroll
+    for (int i = 0; i < N; ++i) v[i] += dpp_move<SPGT_DPP_QUAD_XOR2>(v[i]);
+#pragma unroll
+    for (int i = 0; i < N; ++i) v[i] += dpp_move<SPGT_DPP_ROW_HALF_MIRROR>(v[i]);
+#pragma unroll
+    for (int i = 0; i < N; ++i) v[i] += dpp_move<SPGT_DPP_ROW_MIRROR>(v[i]);
+}
+
 // Sum over groups of 8 consecutive lanes (same guarantee as above).
 __device__ __forceinline__ float row8_allsum(float v) {
     v += dpp_move<SPGT_DPP_QUAD_XOR1>(v);
