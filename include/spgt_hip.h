@@ -192,6 +192,28 @@ int spgt_bilinear_align_corners(const float* src, float* dst, int planes, int H_
 int spgt_bilinear_align_corners_nhwc(const float* src, float* dst, int N, int C, int H_in, int W_in,
                                      int H_out, int W_out, spgt_stream_t stream);
 
+/* Activation and residual placement for spgt_linear_forward. */
+enum { SPGT_ACT_NONE = 0, SPGT_ACT_RELU = 1, SPGT_ACT_SILU = 2 };
+enum { SPGT_RES_NONE = 0, SPGT_RES_BEFORE_ACT = 1, SPGT_RES_AFTER_ACT = 2 };
+
+/* 1 when spgt_linear_forward has a kernel for this shape (in_features 64, 128, 136 or 256;
+ * out_features a multiple of 32), else 0. */
+int spgt_linear_supported(int in_features, int out_features);
+
+/* Replaces an nn.Linear call together with the elementwise kernels that follow it in the
+ * modules either side of the attention: FeedForward (network/layer.py:36-47: Linear ->
+ * activation -> Linear), the attention's fc_layer and the encoder's residual adds
+ * (network/sp_layer.py:58-117), Sp_SpectralConv2D's residual_layer + activation
+ * (network/sp_layer.py:119-160) and the decoder's Linear layers (network/sp_model.py).
+ *   y = x[tokens, in_features] @ weight_kn[in_features, out_features] + bias
+ *   out = act(y + residual) | act(y) + residual | act(y)      (residual_mode 1 | 2 | 0)
+ * weight_kn is the transpose of nn.Linear.weight, contiguous.  x, residual and out are
+ * row-major with row strides ldx, ldr, ldo (in floats, multiples of 4, 16-byte aligned
+ * bases); bias may be null; residual may alias out, x may not. */
+int spgt_linear_forward(const float* x, int64_t ldx, const float* weight_kn, const float* bias,
+                        const float* residual, int64_t ldr, int residual_mode, int activation, float* out,
+                        int64_t ldo, int64_t tokens, int in_features, int out_features, spgt_stream_t stream);
+
 /* Instrumented variant of spgt_galerkin_attention_fused_forward for benchmarks
  * (no reference counterpart): runs the call `iterations` times, synchronising
  * after each, with HIP events recorded on `stream` around each of its three

@@ -45,6 +45,8 @@ SIGNATURES = {
     "spgt_spectral_modes_compact": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _i, _p]),
     "spgt_bilinear_align_corners": (_i, [_p, _p, _i, _i, _i, _i, _i, _p]),
     "spgt_bilinear_align_corners_nhwc": (_i, [_p, _p, _i, _i, _i, _i, _i, _i, _p]),
+    "spgt_linear_supported": (_i, [_i, _i]),
+    "spgt_linear_forward": (_i, [_p, _i64, _p, _p, _p, _i64, _i, _i, _p, _i64, _i64, _i, _i, _p]),
     "spgt_galerkin_attention_fused_profile": (
         _i, [_p, _p, _p, _i64, _p, _p, _p, _p, _p, _f, _p, _p, _p, _sz, _i, _i, _i, _i, _p, _i,
              ctypes.POINTER(ctypes.c_float)]),
@@ -87,14 +89,14 @@ def check(rc: int) -> None:
         raise SpgtError(f"libspgt_hip error {rc}: {last_error()}")
 
 
-def require_gpu_f32(name: str, t: torch.Tensor, dtype=torch.float32) -> None:
+def require_gpu_f32(name: str, t: torch.Tensor, dtype=torch.float32, contiguous: bool = True) -> None:
     if not isinstance(t, torch.Tensor):
         raise TypeError(f"{name} must be a torch.Tensor")
     if not t.is_cuda:
         raise SpgtError(f"{name} must live on a GPU (got device {t.device}); there is no CPU implementation")
     if t.dtype != dtype:
         raise TypeError(f"{name} must have dtype {dtype} (got {t.dtype})")
-    if not t.is_contiguous():
+    if contiguous and not t.is_contiguous():
         raise ValueError(f"{name} must be contiguous")
 
 

@@ -1,0 +1,220 @@
+// Token-major fused linear layer for the modules either side of the attention:
+//   y[t, n]  = sum_k x[t, k] * W[k, n] + bias[n]
+//   out[t,n] = act(y + res)          (residual_mode 1)
+//            = act(y) + res          (residual_mode 2)
+//            = act(y)                (residual_mode 0)
+// with act in {identity, ReLU, SiLU}.  It stands in for the nn.Linear calls and
+// the elementwise kernels that follow them in the reference's modules:
+//   FeedForward.forward                      network/layer.py:36-47
+//   Sp_GalerkinAttention fc_layer, residuals network/sp_layer.py:58-117
+//   Sp_SpectralConv2D residual_layer + act   network/sp_layer.py:119-160
+//   Sp_DecoderRegressor                      network/sp_model.py (spatial_fc_layer, ffn_layer)
+//
+// One wave owns 32 output columns: its W[:, n0 .. n0+31] stays in registers for
+// the whole kernel as the MFMA A operand (column x k).  Token tiles of x go
+// through LDS once (coalesced rows in, one k-strided word per lane out as the
+// B operand).  The 32x32 accumulator then has output columns along registers
+// and tokens along lanes, so a lane stores four 16-byte pieces of its token's
+// row.  LDS reads for the next batch of MFMAs are issued before the current
+// batch so that their latency hides behind the matrix pipe.
+#include "spgt_device.h"
+#include "spgt_host.h"
+
+namespace spgt {
+
+namespace {
+
+__device__ __forceinline__ float activate(float v, int act) {
+    if (act == SPGT_ACT_RELU) return fmaxf(v, 0.f);
+    if (act == SPGT_ACT_SILU) return v / (1.f + __expf(-v));
+    return v;
+}
+
+}  // namespace
+
+// grid (workgroups, column groups), block 256.  NCB column blocks of 32 per
+// workgroup; the 4/NCB waves that share a column block take different 32-token
+// sub-tiles of the workgroup's TT = 32*(4/NCB)-token tile.
+template <int K, int NCB>
+__global__ __launch_bounds__(256) void linear_tm_k(
+    const float* __restrict__ x, int64_t ldx, const float* __restrict__ W, int ldw,
+    const float* __restrict__ bias, const float* res, int64_t ldr, int res_mode, int act,
+    float* out, int64_t ldo, int64_t T, int tiles_per_wg) {
+    constexpr int KH = K / 2;
+    constexpr int PITCH = K + 1;
+    constexpr int TT = 32 * (4 / NCB);
+    constexpr int BK = 16;  // MFMAs per LDS read batch
+    constexpr int NB = (KH + BK - 1) / BK;
+    constexpr int NVEC = TT * K / 4;  // float4 pieces of an x tile
+    constexpr int NLD = (NVEC + 255) / 256;
+    extern __shared__ float xs[];  // [TT][PITCH]
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int tk = lane & 31;
+    const int kh = lane >> 5;
+    const int n0 = (blockIdx.y * NCB + wave % NCB) * 32;
+    const int sub = wave / NCB;
+
+    // A operand: W[2kk + kh][n0 + tk]
+    float wreg[KH];
+#pragma unroll
+    for (int kk = 0; kk < KH; ++kk) wreg[kk] = W[(int64_t)(2 * kk + kh) * ldw + n0 + tk];
+    // accumulator element r holds column n0 + 8*(r/4) + 4*kh + r%4
+    float breg[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) breg[r] = bias ? bias[n0 + 8 * (r >> 2) + 4 * kh + (r & 3)] : 0.f;
+
+    const int64_t t_begin = (int64_t)blockIdx.x * tiles_per_wg * TT;
+    const int64_t t_end = min(T, t_begin + (int64_t)tiles_per_wg * TT);
+    float4 stage[NLD];
+    auto load_tile = [&](int64_t t0) {
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) {
+            const int e = threadIdx.x + 256 * i;
+            const int row = e / (K / 4);
+            const int c4 = e % (K / 4);
+            const int64_t t = t0 + row;
+            stage[i] = (e < NVEC && t < t_end) ? *reinterpret_cast<const float4*>(x + t * ldx + 4 * c4)
+                                               : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    };
+    auto store_tile = [&]() {
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) {
+            const int e = threadIdx.x + 256 * i;
+            if (e < NVEC) {
+                const int row = e / (K / 4);
+                const int c4 = e % (K / 4);
+                float* d = xs + row * PITCH + 4 * c4;
+                d[0] = stage[i].x; d[1] = stage[i].y; d[2] = stage[i].z; d[3] = stage[i].w;
+            }
+        }
+    };
+
+    if (t_begin < t_end) load_tile(t_begin);
+    for (int64_t t0 = t_begin; t0 < t_end; t0 += TT) {
+        __syncthreads();  // previous tile fully consumed
+        store_tile();
+        __syncthreads();
+        if (t0 + TT < t_end) load_tile(t0 + TT);
+
+        const float* xr = xs + (sub * 32 + tk) * PITCH + kh;
+        float xv[2][BK];
+        auto lds_batch = [&](int bt) {
+#pragma unroll
+            for (int j = 0; j < BK; ++j)
+                if (bt * BK + j < KH) xv[bt & 1][j] = xr[2 * (bt * BK + j)];
+        };
+        lds_batch(0);
+        v16f acc;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+#pragma unroll
+        for (int bt = 0; bt < NB; ++bt) {
+            if (bt + 1 < NB) lds_batch(bt + 1);
+            __builtin_amdgcn_sched_barrier(0);  // keep the next batch's reads ahead of this batch's MFMAs
+#pragma unroll
+            for (int j = 0; j < BK; ++j)
+                if (bt * BK + j < KH) acc = mfma32(wreg[bt * BK + j], xv[bt & 1][j], acc);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+
+        const int64_t t = t0 + sub * 32 + tk;
+        if (t < t_end) {
+            float* orow = out + t * ldo + n0 + 4 * kh;
+            const float* rrow = res_mode ? res + t * ldr + n0 + 4 * kh : nullptr;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                float4 r4 = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (res_mode) r4 = *reinterpret_cast<const float4*>(rrow + 8 * q);
+                float4 y;
+                y.x = acc[4 * q + 0] + breg[4 * q + 0];
+                y.y = acc[4 * q + 1] + breg[4 * q + 1];
+                y.z = acc[4 * q + 2] + breg[4 * q + 2];
+                y.w = acc[4 * q + 3] + breg[4 * q + 3];
+                if (res_mode == SPGT_RES_BEFORE_ACT) { y.x += r4.x; y.y += r4.y; y.z += r4.z; y.w += r4.w; }
+                y.x = activate(y.x, act); y.y = activate(y.y, act);
+                y.z = activate(y.z, act); y.w = activate(y.w, act);
+                if (res_mode == SPGT_RES_AFTER_ACT) { y.x += r4.x; y.y += r4.y; y.z += r4.z; y.w += r4.w; }
+                *reinterpret_cast<float4*>(orow + 8 * q) = y;
+            }
+        }
+    }
+}
+
+namespace {
+
+template <int K, int NCB>
+void launch_linear(const float* x, int64_t ldx, const float* W, const float* bias, const float* res, int64_t ldr,
+                   int res_mode, int act, float* out, int64_t ldo, int64_t T, int N, hipStream_t stream) {
+    constexpr int TT = 32 * (4 / NCB);
+    const size_t lds = (size_t)TT * (K + 1) * sizeof(float);
+    const int gy = N / (32 * NCB);
+    const int64_t tiles = ceil_div(T, (int64_t)TT);
+    // about three workgroups per CU, each with the same number of whole tiles
+    const int64_t target = std::max<int64_t>(1, (int64_t)3 * device_cu_count() / gy);
+    const int tpw = (int)ceil_div(tiles, std::min(tiles, target));
+    const dim3 grid((unsigned)ceil_div(tiles, (int64_t)tpw), gy);
+    auto kernel = linear_tm_k<K, NCB>;
+    if (lds > 64 * 1024)
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  (int)lds);
+    hipLaunchKernelGGL(kernel, grid, dim3(256), lds, stream, x, ldx, W, N, bias, res, ldr, res_mode, act, out, ldo, T,
+                       tpw);
+}
+
+template <int K>
+void launch_linear_k(int ncb, const float* x, int64_t ldx, const float* W, const float* bias, const float* res,
+                     int64_t ldr, int res_mode, int act, float* out, int64_t ldo, int64_t T, int N,
+                     hipStream_t stream) {
+    if (ncb == 4) launch_linear<K, 4>(x, ldx, W, bias, res, ldr, res_mode, act, out, ldo, T, N, stream);
+    else if (ncb == 2) launch_linear<K, 2>(x, ldx, W, bias, res, ldr, res_mode, act, out, ldo, T, N, stream);
+    else launch_linear<K, 1>(x, ldx, W, bias, res, ldr, res_mode, act, out, ldo, T, N, stream);
+}
+
+}  // namespace
+
+}  // namespace spgt
+
+using namespace spgt;
+
+extern "C" int spgt_linear_supported(int in_features, int out_features) {
+    const bool k_ok = in_features == 64 || in_features == 128 || in_features == 136 || in_features == 256;
+    return (k_ok && out_features > 0 && out_features % 32 == 0 && out_features <= 65535 * 32) ? 1 : 0;
+}
+
+extern "C" int spgt_linear_forward(const float* x, int64_t ldx, const float* weight_kn, const float* bias,
+                                   const float* residual, int64_t ldr, int residual_mode, int activation, float* out,
+                                   int64_t ldo, int64_t tokens, int in_features, int out_features,
+                                   hipStream_t stream) {
+    if (!x || !weight_kn || !out) return fail(SPGT_ERR_INVALID_ARGUMENT, "linear_forward: null pointer argument");
+    if (tokens < 0) return fail(SPGT_ERR_INVALID_ARGUMENT, "linear_forward: negative token count");
+    if (!spgt_linear_supported(in_features, out_features))
+        return fail(SPGT_ERR_INVALID_ARGUMENT,
+                    "linear_forward: in_features must be 64, 128, 136 or 256 and out_features a multiple of 32");
+    if (activation != SPGT_ACT_NONE && activation != SPGT_ACT_RELU && activation != SPGT_ACT_SILU)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "linear_forward: unknown activation");
+    if (residual_mode != SPGT_RES_NONE && residual_mode != SPGT_RES_BEFORE_ACT && residual_mode != SPGT_RES_AFTER_ACT)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "linear_forward: unknown residual_mode");
+    if (residual_mode != SPGT_RES_NONE && !residual)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "linear_forward: residual is null with a residual_mode");
+    if (ldx < in_features || ldo < out_features || (residual_mode && ldr < out_features))
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "linear_forward: a row stride is smaller than its row");
+    if ((ldx & 3) || (ldo & 3) || (residual_mode && (ldr & 3)) || !aligned16(x) || !aligned16(out) ||
+        (residual_mode && !aligned16(residual)) || !aligned4(weight_kn) || (bias && !aligned4(bias)))
+        return fail(SPGT_ERR_INVALID_ARGUMENT,
+                    "linear_forward: x, residual and out must be 16-byte aligned with row strides that are multiples of 4");
+    if (tokens == 0) return SPGT_OK;
+    const int ncb = out_features % 128 == 0 ? 4 : (out_features % 64 == 0 ? 2 : 1);
+    const float* res = residual_mode ? residual : nullptr;
+#define SPGT_LIN(KV) \
+    launch_linear_k<KV>(ncb, x, ldx, weight_kn, bias, res, ldr, residual_mode, activation, out, ldo, tokens, out_features, stream)
+    switch (in_features) {
+        case 64: SPGT_LIN(64); break;
+        case 128: SPGT_LIN(128); break;
+        case 136: SPGT_LIN(136); break;
+        default: SPGT_LIN(256); break;
+    }
+#undef SPGT_LIN
+    return check_launch("linear_forward");
+}

@@ -1,0 +1,71 @@
+"""Fused token-major linear layer, backed by libspgt_hip.so (inference only).
+
+The reference's modules call nn.Linear and then separate elementwise kernels for
+the activation and the residual add (network/layer.py:36-47,
+network/sp_layer.py:58-117 and 119-160, network/sp_model.py); here the three
+are one kernel.  There is no autograd: modules use it under torch.no_grad() and
+fall back to their nn.Linear graph when gradients are required.
+"""
+from typing import Optional
+
+import torch
+from torch import Tensor
+
+from ... import _lib
+from ..._lib import check, ptr, require_gpu_f32, stream_of
+
+ACTIVATIONS = {"none": 0, "relu": 1, "silu": 2}
+RES_NONE, RES_BEFORE_ACT, RES_AFTER_ACT = 0, 1, 2
+
+
+def linear_supported(in_features: int, out_features: int) -> bool:
+    """True when fused_linear has a kernel for this shape."""
+    return bool(_lib.load().spgt_linear_supported(int(in_features), int(out_features)))
+
+
+def _rows(name: str, t: Tensor, width: int):
+    """View `t` [..., width] as rows with one stride; returns (tensor to keep alive, row count, row stride)."""
+    require_gpu_f32(name, t, contiguous=False)
+    if t.shape[-1] != width:
+        raise ValueError(f"{name} has last dimension {t.shape[-1]}, expected {width}")
+    if t.stride(-1) == 1 and t.dim() == 2 and t.stride(0) >= width and t.stride(0) % 4 == 0 and t.data_ptr() % 16 == 0:
+        return t, t.shape[0], t.stride(0)
+    t = t.contiguous()
+    return t, t.numel() // max(width, 1), width
+
+
+def fused_linear(x: Tensor, weight_kn: Tensor, bias: Optional[Tensor] = None, activation: str = "none",
+                 residual: Optional[Tensor] = None, residual_after_activation: bool = False) -> Tensor:
+    """act(x @ weight_kn + bias [+ residual]) or act(x @ weight_kn + bias) + residual.
+
+    x [..., K] (a 2-D x may have a row stride larger than K), weight_kn [K, N] contiguous
+    (the transpose of nn.Linear.weight), bias [N] or None, residual [..., N] or None.
+    Returns a new contiguous [..., N] tensor.
+    """
+    if activation not in ACTIVATIONS:
+        raise ValueError(f"activation must be one of {sorted(ACTIVATIONS)}")
+    require_gpu_f32("weight_kn", weight_kn)
+    K, N = weight_kn.shape
+    xr, T, ldx = _rows("x", x, K)
+    lead = list(x.shape[:-1])
+    if bias is not None:
+        require_gpu_f32("bias", bias)
+        if bias.numel() != N:
+            raise ValueError(f"bias has {bias.numel()} elements, expected {N}")
+    out = torch.empty(lead + [N], dtype=x.dtype, device=x.device)
+    mode, rr, ldr = RES_NONE, None, 0
+    if residual is not None:
+        if list(residual.shape[:-1]) != lead and residual.numel() != T * N:
+            raise ValueError("residual must have the shape of the output")
+        rr, Tr, ldr = _rows("residual", residual if residual.dim() == 2 else residual.reshape(-1, N), N)
+        if Tr != T:
+            raise ValueError("residual must have the shape of the output")
+        mode = RES_AFTER_ACT if residual_after_activation else RES_BEFORE_ACT
+    if T == 0:
+        return out
+    with torch.cuda.device(x.device):
+        check(_lib.load().spgt_linear_forward(
+            ptr(xr), ldx, ptr(weight_kn), ptr(bias) if bias is not None else None,
+            ptr(rr) if rr is not None else None, ldr, mode, ACTIVATIONS[activation], ptr(out), N, T, K, N,
+            stream_of(x)))
+    return out

@@ -1,0 +1,100 @@
+"""Fused linear kernel (C-ABI spgt_linear_forward) against a float64 CPU product.
+
+The expected values are a plain float64 matmul + bias + activation + residual, the
+definition of nn.Linear followed by the elementwise steps of network/layer.py:36-47;
+tolerance 1e-5 of the output scale (fp32 accumulation over at most 256 terms).
+"""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _expected(x, w_kn, b, act, res, after):
+    y = x.double() @ w_kn.double()
+    if b is not None:
+        y = y + b.double()
+    if res is not None and not after:
+        y = y + res.double()
+    if act == "relu":
+        y = torch.relu(y)
+    elif act == "silu":
+        y = y * torch.sigmoid(y)
+    if res is not None and after:
+        y = y + res.double()
+    return y
+
+
+@pytest.mark.parametrize("K,N", [(128, 128), (128, 256), (128, 384), (256, 128), (136, 128), (64, 64), (64, 256),
+                                 (128, 64), (64, 32), (128, 96)])
+@pytest.mark.parametrize("T", [1, 31, 1000, 20164])
+def test_linear_shapes(gpu, K, N, T):
+    from spgt_amd.extension.bind.linear import fused_linear, linear_supported
+    assert linear_supported(K, N)
+    g = torch.Generator().manual_seed(K * 1000 + N + T)
+    x = torch.randn(T, K, generator=g)
+    w = torch.randn(K, N, generator=g) / K ** 0.5
+    b = torch.randn(N, generator=g)
+    got = fused_linear(x.to(gpu), w.to(gpu), b.to(gpu)).cpu()
+    want = _expected(x, w, b, "none", None, False)
+    assert got.shape == (T, N)
+    assert (got.double() - want).abs().max().item() <= 1e-5 * max(1.0, want.abs().max().item())
+
+
+@pytest.mark.parametrize("act", ["none", "relu", "silu"])
+@pytest.mark.parametrize("res_mode", [None, "before", "after"])
+@pytest.mark.parametrize("use_bias", [True, False])
+def test_linear_epilogues(gpu, act, res_mode, use_bias):
+    from spgt_amd.extension.bind.linear import fused_linear
+    T, K, N = 777, 128, 256
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(3, 259, K, generator=g)  # leading dims are flattened
+    w = torch.randn(K, N, generator=g) / K ** 0.5
+    b = torch.randn(N, generator=g) if use_bias else None
+    res = torch.randn(3, 259, N, generator=g) if res_mode else None
+    got = fused_linear(x.to(gpu), w.to(gpu), b.to(gpu) if use_bias else None, act,
+                       res.to(gpu) if res_mode else None, res_mode == "after").cpu()
+    want = _expected(x, w, b, act, res, res_mode == "after")
+    assert got.shape == (3, 259, N)
+    assert (got.double() - want).abs().max().item() <= 1e-5 * max(1.0, want.abs().max().item())
+
+
+def test_linear_strided_rows(gpu):
+    """x taken as a column slice of a packed [T, 384] tensor (row stride 384)."""
+    from spgt_amd.extension.bind.linear import fused_linear
+    g = torch.Generator().manual_seed(9)
+    packed = torch.randn(500, 384, generator=g)
+    w = torch.randn(128, 128, generator=g) / 128 ** 0.5
+    pd = packed.to(gpu)
+    got = fused_linear(pd[:, 128:256], w.to(gpu)).cpu()
+    want = packed[:, 128:256].double() @ w.double()
+    assert (got.double() - want).abs().max().item() <= 1e-5 * want.abs().max().item()
+
+
+def test_linear_matches_nn_linear(gpu):
+    """Same result as torch's own Linear on the device, to fp32 rounding."""
+    from spgt_amd.extension.bind.linear import fused_linear
+    torch.manual_seed(3)
+    lin = torch.nn.Linear(136, 128).to(gpu)
+    x = torch.randn(4, 1001, 136, device=gpu)
+    with torch.no_grad():
+        want = torch.nn.functional.silu(lin(x))
+        got = fused_linear(x, lin.weight.t().contiguous(), lin.bias, "silu")
+    assert (got - want).abs().max().item() <= 1e-5 * want.abs().max().item()
+
+
+def test_linear_errors(gpu):
+    from spgt_amd._lib import SpgtError
+    from spgt_amd.extension.bind.linear import fused_linear, linear_supported
+    assert not linear_supported(100, 128)
+    assert not linear_supported(128, 1)
+    x = torch.randn(8, 100, device=gpu)
+    w = torch.randn(100, 128, device=gpu)
+    with pytest.raises(SpgtError):
+        fused_linear(x, w)
+    with pytest.raises(ValueError):
+        fused_linear(torch.randn(8, 128, device=gpu), torch.randn(128, 128, device=gpu), activation="tanh")
+    with pytest.raises(SpgtError):
+        fused_linear(torch.randn(8, 128), torch.randn(128, 128, device=gpu))
+    out = fused_linear(torch.empty(0, 128, device=gpu), torch.randn(128, 128, device=gpu))
+    assert out.shape == (0, 128)
