@@ -201,18 +201,23 @@ enum { SPGT_RES_NONE = 0, SPGT_RES_BEFORE_ACT = 1, SPGT_RES_AFTER_ACT = 2 };
 int spgt_linear_supported(int in_features, int out_features);
 
 /* Replaces an nn.Linear call together with the elementwise kernels that follow it in the
- * modules either side of the attention: FeedForward (network/layer.py:36-47: Linear ->
+ * modules either side of the attention: FeedForward (network/layer.py:155-174: Linear ->
  * activation -> Linear), the attention's fc_layer and the encoder's residual adds
- * (network/sp_layer.py:58-117), Sp_SpectralConv2D's residual_layer + activation
- * (network/sp_layer.py:119-160) and the decoder's Linear layers (network/sp_model.py).
+ * (network/sp_layer.py:75, 97-103), Sp_SpectralConv2D's residual_layer + activation
+ * (network/sp_layer.py:132, 155) and the decoder's Linear layers (network/sp_model.py:60, 63).
  *   y = x[tokens, in_features] @ weight_kn[in_features, out_features] + bias
  *   out = act(y + residual) | act(y) + residual | act(y)      (residual_mode 1 | 2 | 0)
  * weight_kn is the transpose of nn.Linear.weight, contiguous.  x, residual and out are
  * row-major with row strides ldx, ldr, ldo (in floats, multiples of 4, 16-byte aligned
- * bases); bias may be null; residual may alias out, x may not. */
+ * bases); bias may be null; residual may alias out, x may not.
+ * The output columns may be split into planes of out_plane_cols columns (a multiple of 32
+ * that divides out_features; 0 = one plane): column n of token t is written to
+ * out[(n / out_plane_cols) * out_plane_stride + t * ldo + n % out_plane_cols], which lets one
+ * call with the packed [W_Q | W_K | W_V] produce three contiguous projections. */
 int spgt_linear_forward(const float* x, int64_t ldx, const float* weight_kn, const float* bias,
                         const float* residual, int64_t ldr, int residual_mode, int activation, float* out,
-                        int64_t ldo, int64_t tokens, int in_features, int out_features, spgt_stream_t stream);
+                        int64_t ldo, int out_plane_cols, int64_t out_plane_stride, int64_t tokens,
+                        int in_features, int out_features, spgt_stream_t stream);
 
 /* Instrumented variant of spgt_galerkin_attention_fused_forward for benchmarks
  * (no reference counterpart): runs the call `iterations` times, synchronising

@@ -5,10 +5,10 @@
 //            = act(y)                (residual_mode 0)
 // with act in {identity, ReLU, SiLU}.  It stands in for the nn.Linear calls and
 // the elementwise kernels that follow them in the reference's modules:
-//   FeedForward.forward                      network/layer.py:36-47
-//   Sp_GalerkinAttention fc_layer, residuals network/sp_layer.py:58-117
-//   Sp_SpectralConv2D residual_layer + act   network/sp_layer.py:119-160
-//   Sp_DecoderRegressor                      network/sp_model.py (spatial_fc_layer, ffn_layer)
+//   FeedForward.forward                      network/layer.py:155-174
+//   Sp_GalerkinAttention fc_layer, residuals network/sp_layer.py:75, 97-103
+//   Sp_SpectralConv2D residual_layer + act   network/sp_layer.py:132, 155
+//   Sp_DecoderRegressor                      network/sp_model.py:60, 63
 //
 // One wave owns 32 output columns: its W[:, n0 .. n0+31] stays in registers for
 // the whole kernel as the MFMA A operand (column x k).  Token tiles of x go
@@ -39,7 +39,7 @@ template <int K, int NCB>
 __global__ __launch_bounds__(256) void linear_tm_k(
     const float* __restrict__ x, int64_t ldx, const float* __restrict__ W, int ldw,
     const float* __restrict__ bias, const float* res, int64_t ldr, int res_mode, int act,
-    float* out, int64_t ldo, int64_t T, int tiles_per_wg) {
+    float* out, int64_t ldo, int plane_cols, int64_t plane_stride, int64_t T, int tiles_per_wg) {
     constexpr int KH = K / 2;
     constexpr int PITCH = K + 1;
     constexpr int TT = 32 * (4 / NCB);
@@ -121,7 +121,8 @@ __global__ __launch_bounds__(256) void linear_tm_k(
 
         const int64_t t = t0 + sub * 32 + tk;
         if (t < t_end) {
-            float* orow = out + t * ldo + n0 + 4 * kh;
+            // output column n lives in plane n / plane_cols at column n % plane_cols
+            float* orow = out + (n0 / plane_cols) * plane_stride + t * ldo + n0 % plane_cols + 4 * kh;
             const float* rrow = res_mode ? res + t * ldr + n0 + 4 * kh : nullptr;
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
@@ -144,32 +145,56 @@ __global__ __launch_bounds__(256) void linear_tm_k(
 
 namespace {
 
+// Tiles per workgroup.  With every workgroup resident at once, the time is set by the
+// CU with the most work, ceil(workgroups / CUs) * tiles_per_wg tile-times; among the
+// choices with the least such work, two workgroups per CU hide each other's load
+// latency best (one has nothing to overlap with, more re-read W more often).
+inline int pick_tiles_per_wg(int64_t tiles, int gy, int cus) {
+    int best = 1;
+    int64_t best_cost = INT64_MAX;
+    double best_dist = 0;
+    for (int tpw = 1; tpw <= 64; ++tpw) {
+        const int64_t wgs = ceil_div(tiles, (int64_t)tpw) * gy;
+        const int64_t per_cu = ceil_div(wgs, (int64_t)cus);
+        const int64_t cost = per_cu * tpw;
+        const double dist = per_cu >= 2 ? (double)per_cu / 2 : 2.5;  // 2 -> 1, 3 -> 1.5, 4 -> 2, 1 -> 2.5
+        if (cost < best_cost || (cost == best_cost && dist < best_dist)) {
+            best = tpw;
+            best_cost = cost;
+            best_dist = dist;
+        }
+        if (wgs <= gy) break;
+    }
+    return best;
+}
+
 template <int K, int NCB>
 void launch_linear(const float* x, int64_t ldx, const float* W, const float* bias, const float* res, int64_t ldr,
-                   int res_mode, int act, float* out, int64_t ldo, int64_t T, int N, hipStream_t stream) {
+                   int res_mode, int act, float* out, int64_t ldo, int plane_cols, int64_t plane_stride, int64_t T,
+                   int N, hipStream_t stream) {
     constexpr int TT = 32 * (4 / NCB);
     const size_t lds = (size_t)TT * (K + 1) * sizeof(float);
     const int gy = N / (32 * NCB);
     const int64_t tiles = ceil_div(T, (int64_t)TT);
-    // about three workgroups per CU, each with the same number of whole tiles
-    const int64_t target = std::max<int64_t>(1, (int64_t)3 * device_cu_count() / gy);
-    const int tpw = (int)ceil_div(tiles, std::min(tiles, target));
+    const int tpw = pick_tiles_per_wg(tiles, gy, device_cu_count());
     const dim3 grid((unsigned)ceil_div(tiles, (int64_t)tpw), gy);
     auto kernel = linear_tm_k<K, NCB>;
     if (lds > 64 * 1024)
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                   (int)lds);
-    hipLaunchKernelGGL(kernel, grid, dim3(256), lds, stream, x, ldx, W, N, bias, res, ldr, res_mode, act, out, ldo, T,
-                       tpw);
+    hipLaunchKernelGGL(kernel, grid, dim3(256), lds, stream, x, ldx, W, N, bias, res, ldr, res_mode, act, out, ldo,
+                       plane_cols, plane_stride, T, tpw);
 }
 
 template <int K>
 void launch_linear_k(int ncb, const float* x, int64_t ldx, const float* W, const float* bias, const float* res,
-                     int64_t ldr, int res_mode, int act, float* out, int64_t ldo, int64_t T, int N,
-                     hipStream_t stream) {
-    if (ncb == 4) launch_linear<K, 4>(x, ldx, W, bias, res, ldr, res_mode, act, out, ldo, T, N, stream);
-    else if (ncb == 2) launch_linear<K, 2>(x, ldx, W, bias, res, ldr, res_mode, act, out, ldo, T, N, stream);
-    else launch_linear<K, 1>(x, ldx, W, bias, res, ldr, res_mode, act, out, ldo, T, N, stream);
+                     int64_t ldr, int res_mode, int act, float* out, int64_t ldo, int plane_cols, int64_t plane_stride,
+                     int64_t T, int N, hipStream_t stream) {
+#define SPGT_ARGS x, ldx, W, bias, res, ldr, res_mode, act, out, ldo, plane_cols, plane_stride, T, N, stream
+    if (ncb == 4) launch_linear<K, 4>(SPGT_ARGS);
+    else if (ncb == 2) launch_linear<K, 2>(SPGT_ARGS);
+    else launch_linear<K, 1>(SPGT_ARGS);
+#undef SPGT_ARGS
 }
 
 }  // namespace
@@ -185,8 +210,8 @@ extern "C" int spgt_linear_supported(int in_features, int out_features) {
 
 extern "C" int spgt_linear_forward(const float* x, int64_t ldx, const float* weight_kn, const float* bias,
                                    const float* residual, int64_t ldr, int residual_mode, int activation, float* out,
-                                   int64_t ldo, int64_t tokens, int in_features, int out_features,
-                                   hipStream_t stream) {
+                                   int64_t ldo, int out_plane_cols, int64_t out_plane_stride, int64_t tokens,
+                                   int in_features, int out_features, hipStream_t stream) {
     if (!x || !weight_kn || !out) return fail(SPGT_ERR_INVALID_ARGUMENT, "linear_forward: null pointer argument");
     if (tokens < 0) return fail(SPGT_ERR_INVALID_ARGUMENT, "linear_forward: negative token count");
     if (!spgt_linear_supported(in_features, out_features))
@@ -198,7 +223,13 @@ extern "C" int spgt_linear_forward(const float* x, int64_t ldx, const float* wei
         return fail(SPGT_ERR_INVALID_ARGUMENT, "linear_forward: unknown residual_mode");
     if (residual_mode != SPGT_RES_NONE && !residual)
         return fail(SPGT_ERR_INVALID_ARGUMENT, "linear_forward: residual is null with a residual_mode");
-    if (ldx < in_features || ldo < out_features || (residual_mode && ldr < out_features))
+    if (out_plane_cols <= 0 || out_plane_cols > out_features) out_plane_cols = out_features;
+    if (out_plane_cols % 32 != 0 || out_features % out_plane_cols != 0)
+        return fail(SPGT_ERR_INVALID_ARGUMENT,
+                    "linear_forward: out_plane_cols must be a multiple of 32 that divides out_features");
+    if (out_plane_cols < out_features && (out_plane_stride & 3))
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "linear_forward: out_plane_stride must be a multiple of 4");
+    if (ldx < in_features || ldo < out_plane_cols || (residual_mode && ldr < out_features))
         return fail(SPGT_ERR_INVALID_ARGUMENT, "linear_forward: a row stride is smaller than its row");
     if ((ldx & 3) || (ldo & 3) || (residual_mode && (ldr & 3)) || !aligned16(x) || !aligned16(out) ||
         (residual_mode && !aligned16(residual)) || !aligned4(weight_kn) || (bias && !aligned4(bias)))
@@ -208,7 +239,8 @@ extern "C" int spgt_linear_forward(const float* x, int64_t ldx, const float* wei
     const int ncb = out_features % 128 == 0 ? 4 : (out_features % 64 == 0 ? 2 : 1);
     const float* res = residual_mode ? residual : nullptr;
 #define SPGT_LIN(KV) \
-    launch_linear_k<KV>(ncb, x, ldx, weight_kn, bias, res, ldr, residual_mode, activation, out, ldo, tokens, out_features, stream)
+    launch_linear_k<KV>(ncb, x, ldx, weight_kn, bias, res, ldr, residual_mode, activation, out, ldo, out_plane_cols, \
+                        out_plane_stride, tokens, out_features, stream)
     switch (in_features) {
         case 64: SPGT_LIN(64); break;
         case 128: SPGT_LIN(128); break;

@@ -1,8 +1,8 @@
 """Fused token-major linear layer, backed by libspgt_hip.so (inference only).
 
 The reference's modules call nn.Linear and then separate elementwise kernels for
-the activation and the residual add (network/layer.py:36-47,
-network/sp_layer.py:58-117 and 119-160, network/sp_model.py); here the three
+the activation and the residual add (network/layer.py:155-174,
+network/sp_layer.py:75, 97-103 and 132, 155, network/sp_model.py:60, 63); here the three
 are one kernel.  There is no autograd: modules use it under torch.no_grad() and
 fall back to their nn.Linear graph when gradients are required.
 """
@@ -35,12 +35,14 @@ def _rows(name: str, t: Tensor, width: int):
 
 
 def fused_linear(x: Tensor, weight_kn: Tensor, bias: Optional[Tensor] = None, activation: str = "none",
-                 residual: Optional[Tensor] = None, residual_after_activation: bool = False) -> Tensor:
+                 residual: Optional[Tensor] = None, residual_after_activation: bool = False,
+                 planes: int = 1) -> Tensor:
     """act(x @ weight_kn + bias [+ residual]) or act(x @ weight_kn + bias) + residual.
 
     x [..., K] (a 2-D x may have a row stride larger than K), weight_kn [K, N] contiguous
     (the transpose of nn.Linear.weight), bias [N] or None, residual [..., N] or None.
-    Returns a new contiguous [..., N] tensor.
+    Returns a new contiguous [..., N] tensor, or with planes > 1 a [planes, ..., N / planes] tensor whose
+    plane p holds output columns p*N/planes .. (p+1)*N/planes - 1.
     """
     if activation not in ACTIVATIONS:
         raise ValueError(f"activation must be one of {sorted(ACTIVATIONS)}")
@@ -52,7 +54,10 @@ def fused_linear(x: Tensor, weight_kn: Tensor, bias: Optional[Tensor] = None, ac
         require_gpu_f32("bias", bias)
         if bias.numel() != N:
             raise ValueError(f"bias has {bias.numel()} elements, expected {N}")
-    out = torch.empty(lead + [N], dtype=x.dtype, device=x.device)
+    if planes < 1 or N % planes or (N // planes) % 32:
+        raise ValueError("planes must divide the output width into multiples of 32 columns")
+    pc = N // planes
+    out = torch.empty(([planes] if planes > 1 else []) + lead + [pc], dtype=x.dtype, device=x.device)
     mode, rr, ldr = RES_NONE, None, 0
     if residual is not None:
         if list(residual.shape[:-1]) != lead and residual.numel() != T * N:
@@ -66,6 +71,6 @@ def fused_linear(x: Tensor, weight_kn: Tensor, bias: Optional[Tensor] = None, ac
     with torch.cuda.device(x.device):
         check(_lib.load().spgt_linear_forward(
             ptr(xr), ldx, ptr(weight_kn), ptr(bias) if bias is not None else None,
-            ptr(rr) if rr is not None else None, ldr, mode, ACTIVATIONS[activation], ptr(out), N, T, K, N,
+            ptr(rr) if rr is not None else None, ldr, mode, ACTIVATIONS[activation], ptr(out), pc, pc, T * pc, T, K, N,
             stream_of(x)))
     return out

@@ -11,9 +11,39 @@ import torch
 import torch.nn.functional as F
 from torch import Tensor, nn
 
+from ..extension.bind.linear import fused_linear, linear_supported
+
 
 def make_activation(name: str) -> nn.Module:
     return nn.SiLU() if name == "silu" else nn.ReLU()
+
+
+def activation_name(module: nn.Module) -> str:
+    return "silu" if isinstance(module, nn.SiLU) else "relu"
+
+
+def linear_weight_kn(lin: nn.Linear) -> Tensor:
+    """lin.weight transposed to [in_features, out_features], contiguous; rebuilt when the parameter changes."""
+    w = lin.weight
+    key = (w.data_ptr(), w._version, w.device)
+    cache = getattr(lin, "_spgt_weight_kn", None)
+    if cache is None or cache[0] != key:
+        cache = (key, w.detach().t().contiguous())
+        lin._spgt_weight_kn = cache
+    return cache[1]
+
+
+def gpu_inference(X: Tensor, *params: Tensor) -> bool:
+    """fp32 on a GPU with nothing to differentiate: the case the fused inference kernels serve."""
+    if not X.is_cuda or X.dtype != torch.float32:
+        return False
+    return not (torch.is_grad_enabled() and (X.requires_grad or any(p.requires_grad for p in params)))
+
+
+def fused_linear_usable(X: Tensor, *linears: nn.Linear) -> bool:
+    """gpu_inference, and the fused linear kernel has a variant for every layer's shape."""
+    return (gpu_inference(X, *[p for l in linears for p in l.parameters()]) and
+            all(linear_supported(l.in_features, l.out_features) for l in linears))
 
 
 def always_dropout(X: Tensor, p: float) -> Tensor:
@@ -43,5 +73,12 @@ class FeedForward(nn.Module):
         self.layer2 = nn.Linear(dim_hidden, out_dim)
         self.activation_layer = make_activation(activation)
 
-    def forward(self, X: Tensor) -> Tensor:
-        return always_dropout(self.layer2(self.activation_layer(self.layer1(X))), self.droprate)
+    def forward(self, X: Tensor, residual: Tensor = None) -> Tensor:
+        """ffn(X), or residual + ffn(X) when a residual is given."""
+        if fused_linear_usable(X, self.layer1, self.layer2) and (residual is None or self.droprate == 0):
+            # inference: bias + activation and bias + residual ride in the two GEMMs' epilogues
+            H = fused_linear(X, linear_weight_kn(self.layer1), self.layer1.bias, activation_name(self.activation_layer))
+            Y = fused_linear(H, linear_weight_kn(self.layer2), self.layer2.bias, "none", residual)
+            return always_dropout(Y, self.droprate)
+        Y = always_dropout(self.layer2(self.activation_layer(self.layer1(X))), self.droprate)
+        return Y if residual is None else residual + Y

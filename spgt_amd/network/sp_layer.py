@@ -30,12 +30,12 @@ from ..extension.bind.galerkin_attention import (galerkin_attention_fused, multi
                                                  multihead_projection_layernorm_with_position_rrc_cuda,
                                                  multihead_projection_with_position_rrc_cuda)
 from . import truncated_dft
-from .layer import FeedForward, always_dropout, make_activation
+from ..extension.bind.linear import fused_linear
+from .layer import (FeedForward, activation_name, always_dropout, fused_linear_usable, linear_weight_kn,
+                    make_activation)
 
 
 class Sp_GalerkinAttention(nn.Module):
-    PACKED_QKV_MAX_TOKENS = 65536
-
     def __init__(self, dim_hidden, num_head, dim_position, norm_eps, attn_droprate, fc_droprate, xavier, diagonal,
                  symmetric) -> None:
         super().__init__()
@@ -84,8 +84,9 @@ class Sp_GalerkinAttention(nn.Module):
         return torch.is_grad_enabled() and (any(t.requires_grad for t in tensors) or
                                             any(p.requires_grad for p in self.parameters()))
 
-    def forward(self, Q: Tensor, K: Tensor, V: Tensor, position: Tensor) -> Tensor:
-        """Q, K, V [N, seqlen, dim_hidden], position [N, seqlen, dim_position] -> [N, seqlen, dim_hidden]."""
+    def forward(self, Q: Tensor, K: Tensor, V: Tensor, position: Tensor, residual: Tensor = None) -> Tensor:
+        """Q, K, V [N, seqlen, dim_hidden], position [N, seqlen, dim_position] -> [N, seqlen, dim_hidden];
+        with `residual` the result is residual + attention(Q, K, V)."""
         N, seqlen, C = Q.size()
         H, dp = self.num_head, self.dim_position
         if self._needs_graph(Q, K, V):
@@ -99,22 +100,23 @@ class Sp_GalerkinAttention(nn.Module):
             X = multihead_galerkin_attention_cccr_cuda(q, k, v)
             X = X.transpose(1, 2).contiguous().view(N, seqlen, H * (dp + self.dim_head))
         else:
-            if Q is K and K is V and N * seqlen < self.PACKED_QKV_MAX_TOKENS:
-                # short sequences are launch-bound: one GEMM, Q/K/V as column slices of its output
+            if Q is K and K is V:
+                # one launch over [W_Q | W_K | W_V] with the bias in its epilogue; the three projections land
+                # in contiguous planes (the attention passes run 15 % faster on unit-stride rows)
                 w, b = self._packed_qkv()
-                qkv = torch.addmm(b, Q.reshape(N * seqlen, C), w).view(N, seqlen, 3 * C)
-                q, k, v = qkv[..., :C], qkv[..., C:2 * C], qkv[..., 2 * C:]
+                q, k, v = fused_linear(Q.reshape(N * seqlen, C), w, b, planes=3).view(3, N, seqlen, C).unbind(0)
             else:
-                # long sequences: three GEMMs into contiguous planes (measured on MI355X at
-                # 356k tokens: 384 us against 438 us packed, and the attention passes run
-                # 15 % faster on unit-stride rows than on a 3x strided buffer)
-                proj = lambda x, w, b: torch.addmm(b, x.reshape(N * seqlen, C), w).view(N, seqlen, C)
+                proj = lambda x, w, b: fused_linear(x.reshape(N * seqlen, C), w.detach(), b.detach()).view(N, seqlen, C)
                 q, k, v = (proj(Q, self.weight_Q, self.bias_Q), proj(K, self.weight_K, self.bias_K),
                            proj(V, self.weight_V, self.bias_V))
             pos = position.contiguous() if dp else None
             X = galerkin_attention_fused(q, k, v, pos, self.ln_weight_K.detach(), self.ln_bias_K.detach(),
                                          self.ln_weight_V.detach(), self.ln_bias_V.detach(), self.norm_eps, H, dp)
-        return always_dropout(self.fc_layer(X), self.fc_droprate)
+        if fused_linear_usable(X, self.fc_layer) and (residual is None or self.fc_droprate == 0):
+            Y = fused_linear(X, linear_weight_kn(self.fc_layer), self.fc_layer.bias, "none", residual)
+            return always_dropout(Y, self.fc_droprate)
+        Y = always_dropout(self.fc_layer(X), self.fc_droprate)
+        return Y if residual is None else residual + Y
 
 
 class Sp_EncoderLayer(nn.Module):
@@ -128,8 +130,8 @@ class Sp_EncoderLayer(nn.Module):
         self.ffn_layer = FeedForward(dim_hidden, dim_hidden, ffn_dim_hidden, ffn_droprate, ffn_activation)
 
     def forward(self, X: Tensor, position: Tensor) -> Tensor:
-        X = X + self.attention_layer(X, X, X, position)
-        return X + self.ffn_layer(X)
+        X = self.attention_layer(X, X, X, position, residual=X)
+        return self.ffn_layer(X, residual=X)
 
 
 class Sp_SpectralConv2D(nn.Module):
@@ -151,11 +153,19 @@ class Sp_SpectralConv2D(nn.Module):
         """[N, r, r, in_dim] -> [N, r, r, out_dim]."""
         N, r, _, cin = X.size()
         m, cout = self.mode, self.out_dim
+        needs_graph = torch.is_grad_enabled() and (X.requires_grad or self.fourier_weight[0].requires_grad)
+        if (self.use_truncated_dft and not needs_graph and truncated_dft.supported(r, m) and
+                fused_linear_usable(X, self.residual_layer)):
+            # only the retained modes are ever computed: no FFT, no transposes, no full-size spectrum;
+            # the residual Linear, the add and the activation are one kernel
+            X0 = X.contiguous()
+            Y = truncated_dft.spectral_modes_apply(always_dropout(X0, self.droprate), self.fourier_weight[0],
+                                                   self.fourier_weight[1], m)
+            return fused_linear(X0, linear_weight_kn(self.residual_layer), self.residual_layer.bias,
+                                activation_name(self.activation_layer), Y)
         res = self.residual_layer(X)
         X = always_dropout(X, self.droprate)
-        needs_graph = torch.is_grad_enabled() and (X.requires_grad or self.fourier_weight[0].requires_grad)
         if self.use_truncated_dft and not needs_graph and truncated_dft.supported(r, m):
-            # only the retained modes are ever computed: no FFT, no transposes, no full-size spectrum
             Y = truncated_dft.spectral_modes_apply(X.contiguous(), self.fourier_weight[0], self.fourier_weight[1], m)
             return self.activation_layer(Y + res)
         X = batched_transpose(X, [N], [r, r], [cin])  # -> [N, in_dim, r, r]

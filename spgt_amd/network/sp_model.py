@@ -8,7 +8,8 @@ import torch
 import torch.nn.functional as F
 from torch import Tensor, nn
 
-from .layer import FeedForward, always_dropout
+from ..extension.bind.linear import fused_linear, linear_supported
+from .layer import FeedForward, always_dropout, gpu_inference
 from .model import DownScaler2D, UpScaler2D
 from .sp_layer import Sp_EncoderLayer, Sp_SpectralConv2D
 
@@ -55,11 +56,27 @@ class Sp_DecoderRegressor(nn.Module):
         self.ffn_layer = FeedForward(dim_spatial_hidden, out_dim, 2 * dim_position * dim_spatial_hidden, droprate,
                                      activation)
 
+    def _weight_x_kn(self, dim_x: int) -> Tensor:
+        """The hidden-feature columns of spatial_fc_layer.weight as [dim_x, C], rebuilt when the parameter changes."""
+        w = self.spatial_fc_layer.weight
+        key = (w.data_ptr(), w._version, w.device, dim_x)
+        cache = getattr(self, "_spgt_weight_x_kn", None)
+        if cache is None or cache[0] != key:
+            cache = (key, w.detach()[:, :dim_x].t().contiguous())
+            self._spgt_weight_x_kn = cache
+        return cache[1]
+
     def forward(self, X: Tensor, grid: Tensor = None) -> Tensor:
         """X [N, r, r, dim_hidden], grid [N, r, r, dim_position] -> [N, r, r, dim_target]."""
         # Linear(cat([X, grid])) without materialising the concatenation: W = [W_x | W_grid]
         W, dim_x = self.spatial_fc_layer.weight, X.size(-1)
-        X = F.linear(X, W[:, :dim_x], self.spatial_fc_layer.bias) + F.linear(grid, W[:, dim_x:])
+        if gpu_inference(X, W, self.spatial_fc_layer.bias) and linear_supported(dim_x, W.size(0)):
+            # the grid columns first (a [T, dim_position] x [dim_position, C] product); the GEMM over the
+            # hidden features adds it in its epilogue
+            X = fused_linear(X, self._weight_x_kn(dim_x), self.spatial_fc_layer.bias, "none",
+                             F.linear(grid, W[:, dim_x:]))
+        else:
+            X = F.linear(X, W[:, :dim_x], self.spatial_fc_layer.bias) + F.linear(grid, W[:, dim_x:])
         for layer in self.layers:
             X = layer(X)
         return self.ffn_layer(X)

@@ -1,7 +1,7 @@
 """Fused linear kernel (C-ABI spgt_linear_forward) against a float64 CPU product.
 
 The expected values are a plain float64 matmul + bias + activation + residual, the
-definition of nn.Linear followed by the elementwise steps of network/layer.py:36-47;
+definition of nn.Linear followed by the elementwise steps of network/layer.py:155-174;
 tolerance 1e-5 of the output scale (fp32 accumulation over at most 256 terms).
 """
 import pytest
@@ -69,6 +69,21 @@ def test_linear_strided_rows(gpu):
     got = fused_linear(pd[:, 128:256], w.to(gpu)).cpu()
     want = packed[:, 128:256].double() @ w.double()
     assert (got.double() - want).abs().max().item() <= 1e-5 * want.abs().max().item()
+
+
+def test_linear_output_planes(gpu):
+    """planes=3: the packed projection's column thirds come back as three contiguous tensors."""
+    from spgt_amd.extension.bind.linear import fused_linear
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(2, 333, 128, generator=g)
+    w = torch.randn(128, 384, generator=g) / 128 ** 0.5
+    b = torch.randn(384, generator=g)
+    got = fused_linear(x.to(gpu), w.to(gpu), b.to(gpu), planes=3)
+    assert got.shape == (3, 2, 333, 128) and got.is_contiguous()
+    want = (x.double() @ w.double() + b.double()).view(2, 333, 3, 128).permute(2, 0, 1, 3)
+    assert (got.cpu().double() - want).abs().max().item() <= 1e-5 * want.abs().max().item()
+    with pytest.raises(ValueError):
+        fused_linear(x.to(gpu), w.to(gpu), b.to(gpu), planes=5)
 
 
 def test_linear_matches_nn_linear(gpu):
