@@ -219,6 +219,20 @@ int spgt_linear_forward(const float* x, int64_t ldx, const float* weight_kn, con
                         int64_t ldo, int out_plane_cols, int64_t out_plane_stride, int64_t tokens,
                         int in_features, int out_features, spgt_stream_t stream);
 
+/* 1 when spgt_ffn_scalar_forward has a kernel for this shape (in_features 64 or 128,
+ * hidden_features 128 or 256), else 0. */
+int spgt_ffn_scalar_supported(int in_features, int hidden_features);
+
+/* Replaces FeedForward (network/layer.py:155-174) when its out_dim is 1, the regression
+ * head of Sp_DecoderRegressor (network/sp_model.py:51, 63), in one kernel:
+ *   out[t] = sum_n act(x[t, :] . weight1_kn[:, n] + bias1[n]) * weight2[n] + bias2[0]
+ * weight1_kn [in_features, hidden_features] is the transpose of layer1.weight, weight2
+ * [hidden_features] is layer2.weight's single row; bias1 and bias2 (one element, on the
+ * device) may be null.  x is row-major with row stride ldx (floats, a multiple of 4). */
+int spgt_ffn_scalar_forward(const float* x, int64_t ldx, const float* weight1_kn, const float* bias1,
+                            const float* weight2, const float* bias2, int activation, float* out,
+                            int64_t tokens, int in_features, int hidden_features, spgt_stream_t stream);
+
 /* Instrumented variant of spgt_galerkin_attention_fused_forward for benchmarks
  * (no reference counterpart): runs the call `iterations` times, synchronising
  * after each, with HIP events recorded on `stream` around each of its three

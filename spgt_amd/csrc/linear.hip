@@ -143,6 +143,121 @@ __global__ __launch_bounds__(256) void linear_tm_k(
     }
 }
 
+// Two-layer feed-forward net with a single output feature:
+//   out[t] = sum_n act(x[t, :] . W1[:, n] + b1[n]) * w2[n] + b2
+// (FeedForward with out_dim 1, the regression head of network/sp_model.py:51, 63).
+// The hidden activations never leave registers.  grid (workgroups), block 256;
+// wave w owns hidden columns 32*(w + 4c) .. +31 for c < CBW; HID = 128*CBW.
+template <int K, int CBW>
+__global__ __launch_bounds__(256) void ffn_scalar_k(
+    const float* __restrict__ x, int64_t ldx, const float* __restrict__ W1, const float* __restrict__ b1,
+    const float* __restrict__ w2, const float* __restrict__ b2, int act, float* __restrict__ out, int64_t T,
+    int tiles_per_wg) {
+    constexpr int KH = K / 2;
+    constexpr int PITCH = K + 1;
+    constexpr int TT = 32;
+    constexpr int HID = 128 * CBW;
+    constexpr int BK = 16;
+    constexpr int NB = (KH + BK - 1) / BK;
+    constexpr int NVEC = TT * K / 4;
+    constexpr int NLD = (NVEC + 255) / 256;
+    __shared__ float xs[TT * PITCH];
+    __shared__ float red[4][32];
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int tk = lane & 31;
+    const int kh = lane >> 5;
+
+    float wreg[CBW][KH], breg[CBW][16], vreg[CBW][16];
+#pragma unroll
+    for (int c = 0; c < CBW; ++c) {
+        const int n0 = 32 * (wave + 4 * c);
+#pragma unroll
+        for (int kk = 0; kk < KH; ++kk) wreg[c][kk] = W1[(int64_t)(2 * kk + kh) * HID + n0 + tk];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int n = n0 + 8 * (r >> 2) + 4 * kh + (r & 3);
+            breg[c][r] = b1 ? b1[n] : 0.f;
+            vreg[c][r] = w2[n];
+        }
+    }
+    const float bias2 = b2 ? b2[0] : 0.f;
+
+    const int64_t t_begin = (int64_t)blockIdx.x * tiles_per_wg * TT;
+    const int64_t t_end = min(T, t_begin + (int64_t)tiles_per_wg * TT);
+    float4 stage[NLD];
+    auto load_tile = [&](int64_t t0) {
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) {
+            const int e = threadIdx.x + 256 * i;
+            const int row = e / (K / 4);
+            const int c4 = e % (K / 4);
+            const int64_t t = t0 + row;
+            stage[i] = (e < NVEC && t < t_end) ? *reinterpret_cast<const float4*>(x + t * ldx + 4 * c4)
+                                               : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    };
+    auto store_tile = [&]() {
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) {
+            const int e = threadIdx.x + 256 * i;
+            if (e < NVEC) {
+                const int row = e / (K / 4);
+                const int c4 = e % (K / 4);
+                float* d = xs + row * PITCH + 4 * c4;
+                d[0] = stage[i].x; d[1] = stage[i].y; d[2] = stage[i].z; d[3] = stage[i].w;
+            }
+        }
+    };
+
+    if (t_begin < t_end) load_tile(t_begin);
+    for (int64_t t0 = t_begin; t0 < t_end; t0 += TT) {
+        __syncthreads();  // previous tile and its partial sums fully consumed
+        store_tile();
+        __syncthreads();
+        if (t0 + TT < t_end) load_tile(t0 + TT);
+
+        const float* xr = xs + tk * PITCH + kh;
+        float xv[2][BK];
+        auto lds_batch = [&](int bt) {
+#pragma unroll
+            for (int j = 0; j < BK; ++j)
+                if (bt * BK + j < KH) xv[bt & 1][j] = xr[2 * (bt * BK + j)];
+        };
+        lds_batch(0);
+        v16f acc[CBW];
+#pragma unroll
+        for (int c = 0; c < CBW; ++c)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[c][r] = 0.f;
+#pragma unroll
+        for (int bt = 0; bt < NB; ++bt) {
+            if (bt + 1 < NB) lds_batch(bt + 1);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int j = 0; j < BK; ++j)
+                if (bt * BK + j < KH) {
+#pragma unroll
+                    for (int c = 0; c < CBW; ++c) acc[c] = mfma32(wreg[c][bt * BK + j], xv[bt & 1][j], acc[c]);
+                }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // this lane's share of token t0 + tk: 16*CBW hidden columns
+        float part = 0.f;
+#pragma unroll
+        for (int c = 0; c < CBW; ++c)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) part = fmaf(activate(acc[c][r] + breg[c][r], act), vreg[c][r], part);
+        part += __shfl_xor(part, 32, 64);
+        if (kh == 0) red[wave][tk] = part;
+        __syncthreads();
+        if (wave == 0 && kh == 0) {
+            const int64_t t = t0 + tk;
+            if (t < t_end) out[t] = ((red[0][tk] + red[1][tk]) + (red[2][tk] + red[3][tk])) + bias2;
+        }
+    }
+}
+
 namespace {
 
 // Tiles per workgroup.  With every workgroup resident at once, the time is set by the
@@ -197,6 +312,15 @@ void launch_linear_k(int ncb, const float* x, int64_t ldx, const float* W, const
 #undef SPGT_ARGS
 }
 
+template <int K, int CBW>
+void launch_ffn_scalar(const float* x, int64_t ldx, const float* W1, const float* b1, const float* w2, const float* b2,
+                       int act, float* out, int64_t T, hipStream_t stream) {
+    const int64_t tiles = ceil_div(T, (int64_t)32);
+    const int tpw = pick_tiles_per_wg(tiles, 1, device_cu_count());
+    hipLaunchKernelGGL((ffn_scalar_k<K, CBW>), dim3((unsigned)ceil_div(tiles, (int64_t)tpw)), dim3(256), 0, stream, x,
+                       ldx, W1, b1, w2, b2, act, out, T, tpw);
+}
+
 }  // namespace
 
 }  // namespace spgt
@@ -249,4 +373,32 @@ extern "C" int spgt_linear_forward(const float* x, int64_t ldx, const float* wei
     }
 #undef SPGT_LIN
     return check_launch("linear_forward");
+}
+
+extern "C" int spgt_ffn_scalar_supported(int in_features, int hidden_features) {
+    return ((in_features == 64 || in_features == 128) && (hidden_features == 128 || hidden_features == 256)) ? 1 : 0;
+}
+
+extern "C" int spgt_ffn_scalar_forward(const float* x, int64_t ldx, const float* weight1_kn, const float* bias1,
+                                       const float* weight2, const float* bias2, int activation, float* out,
+                                       int64_t tokens, int in_features, int hidden_features, hipStream_t stream) {
+    if (!x || !weight1_kn || !weight2 || !out)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "ffn_scalar_forward: null pointer argument");
+    if (tokens < 0) return fail(SPGT_ERR_INVALID_ARGUMENT, "ffn_scalar_forward: negative token count");
+    if (!spgt_ffn_scalar_supported(in_features, hidden_features))
+        return fail(SPGT_ERR_INVALID_ARGUMENT,
+                    "ffn_scalar_forward: in_features must be 64 or 128 and hidden_features 128 or 256");
+    if (activation != SPGT_ACT_NONE && activation != SPGT_ACT_RELU && activation != SPGT_ACT_SILU)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "ffn_scalar_forward: unknown activation");
+    if (ldx < in_features || (ldx & 3) || !aligned16(x) || !aligned4(out) || !aligned4(weight1_kn) ||
+        !aligned4(weight2))
+        return fail(SPGT_ERR_INVALID_ARGUMENT,
+                    "ffn_scalar_forward: x must be 16-byte aligned with a row stride that is a multiple of 4");
+    if (tokens == 0) return SPGT_OK;
+#define SPGT_FFN(KV, CB) \
+    launch_ffn_scalar<KV, CB>(x, ldx, weight1_kn, bias1, weight2, bias2, activation, out, tokens, stream)
+    if (in_features == 64) { if (hidden_features == 128) SPGT_FFN(64, 1); else SPGT_FFN(64, 2); }
+    else                   { if (hidden_features == 128) SPGT_FFN(128, 1); else SPGT_FFN(128, 2); }
+#undef SPGT_FFN
+    return check_launch("ffn_scalar_forward");
 }

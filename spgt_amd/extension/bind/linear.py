@@ -74,3 +74,37 @@ def fused_linear(x: Tensor, weight_kn: Tensor, bias: Optional[Tensor] = None, ac
             ptr(rr) if rr is not None else None, ldr, mode, ACTIVATIONS[activation], ptr(out), pc, pc, T * pc, T, K, N,
             stream_of(x)))
     return out
+
+
+def ffn_scalar_supported(in_features: int, hidden_features: int) -> bool:
+    """True when fused_ffn_scalar has a kernel for this shape."""
+    return bool(_lib.load().spgt_ffn_scalar_supported(int(in_features), int(hidden_features)))
+
+
+def fused_ffn_scalar(x: Tensor, weight1_kn: Tensor, bias1: Optional[Tensor], weight2: Tensor,
+                     bias2: Optional[Tensor], activation: str) -> Tensor:
+    """act(x @ weight1_kn + bias1) @ weight2 + bias2 for a single output feature, in one kernel.
+
+    x [..., K], weight1_kn [K, HID] contiguous, weight2 [HID] (or [1, HID]), bias2 [1] -> [..., 1].
+    """
+    if activation not in ACTIVATIONS:
+        raise ValueError(f"activation must be one of {sorted(ACTIVATIONS)}")
+    require_gpu_f32("weight1_kn", weight1_kn)
+    require_gpu_f32("weight2", weight2)
+    K, HID = weight1_kn.shape
+    if weight2.numel() != HID:
+        raise ValueError(f"weight2 has {weight2.numel()} elements, expected {HID}")
+    for name, b, n in (("bias1", bias1, HID), ("bias2", bias2, 1)):
+        if b is not None:
+            require_gpu_f32(name, b)
+            if b.numel() != n:
+                raise ValueError(f"{name} has {b.numel()} elements, expected {n}")
+    xr, T, ldx = _rows("x", x, K)
+    out = torch.empty(list(x.shape[:-1]) + [1], dtype=x.dtype, device=x.device)
+    if T == 0:
+        return out
+    with torch.cuda.device(x.device):
+        check(_lib.load().spgt_ffn_scalar_forward(
+            ptr(xr), ldx, ptr(weight1_kn), ptr(bias1) if bias1 is not None else None, ptr(weight2),
+            ptr(bias2) if bias2 is not None else None, ACTIVATIONS[activation], ptr(out), T, K, HID, stream_of(x)))
+    return out

@@ -11,7 +11,7 @@ import torch
 import torch.nn.functional as F
 from torch import Tensor, nn
 
-from ..extension.bind.linear import fused_linear, linear_supported
+from ..extension.bind.linear import ffn_scalar_supported, fused_ffn_scalar, fused_linear, linear_supported
 
 
 def make_activation(name: str) -> nn.Module:
@@ -75,6 +75,13 @@ class FeedForward(nn.Module):
 
     def forward(self, X: Tensor, residual: Tensor = None) -> Tensor:
         """ffn(X), or residual + ffn(X) when a residual is given."""
+        if (self.layer2.out_features == 1 and residual is None and
+                gpu_inference(X, *self.parameters()) and
+                ffn_scalar_supported(self.layer1.in_features, self.layer1.out_features)):
+            # single output feature: both layers in one kernel, the hidden activations stay in registers
+            Y = fused_ffn_scalar(X, linear_weight_kn(self.layer1), self.layer1.bias, self.layer2.weight.detach(),
+                                 self.layer2.bias, activation_name(self.activation_layer))
+            return always_dropout(Y, self.droprate)
         if fused_linear_usable(X, self.layer1, self.layer2) and (residual is None or self.droprate == 0):
             # inference: bias + activation and bias + residual ride in the two GEMMs' epilogues
             H = fused_linear(X, linear_weight_kn(self.layer1), self.layer1.bias, activation_name(self.activation_layer))

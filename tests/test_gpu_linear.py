@@ -113,3 +113,36 @@ def test_linear_errors(gpu):
         fused_linear(torch.randn(8, 128), torch.randn(128, 128, device=gpu))
     out = fused_linear(torch.empty(0, 128, device=gpu), torch.randn(128, 128, device=gpu))
     assert out.shape == (0, 128)
+
+
+@pytest.mark.parametrize("K,HID", [(64, 256), (64, 128), (128, 256), (128, 128)])
+@pytest.mark.parametrize("T", [1, 45, 5000])
+@pytest.mark.parametrize("act", ["relu", "silu"])
+def test_ffn_scalar(gpu, K, HID, T, act):
+    """Both FeedForward layers with one output feature in one kernel, against float64."""
+    from spgt_amd.extension.bind.linear import ffn_scalar_supported, fused_ffn_scalar
+    assert ffn_scalar_supported(K, HID) and not ffn_scalar_supported(96, 256)
+    g = torch.Generator().manual_seed(K + HID + T)
+    x = torch.randn(T, K, generator=g)
+    w1 = torch.randn(K, HID, generator=g) / K ** 0.5
+    b1 = torch.randn(HID, generator=g)
+    w2 = torch.randn(1, HID, generator=g) / HID ** 0.5
+    b2 = torch.randn(1, generator=g)
+    got = fused_ffn_scalar(x.to(gpu), w1.to(gpu), b1.to(gpu), w2.to(gpu), b2.to(gpu), act).cpu()
+    h = _expected(x, w1, b1, act, None, False)
+    want = h @ w2.double().t() + b2.double()
+    assert got.shape == (T, 1)
+    assert (got.double() - want).abs().max().item() <= 1e-5 * max(1.0, want.abs().max().item())
+
+
+def test_feedforward_module_scalar_head(gpu):
+    """FeedForward(64 -> 256 -> 1) under no_grad takes the one-kernel path and matches its nn.Linear graph."""
+    from spgt_amd.network.layer import FeedForward
+    torch.manual_seed(2)
+    ffn = FeedForward(64, 1, 256, 0.0, "silu").to(gpu)
+    x = torch.randn(2, 37, 37, 64, device=gpu)
+    want = ffn.layer2(ffn.activation_layer(ffn.layer1(x))).detach()
+    with torch.no_grad():
+        got = ffn(x)
+    assert got.shape == want.shape
+    assert (got - want).abs().max().item() <= 1e-5 * max(1.0, want.abs().max().item())
