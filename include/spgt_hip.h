@@ -192,9 +192,23 @@ int spgt_bilinear_align_corners(const float* src, float* dst, int planes, int H_
 int spgt_bilinear_align_corners_nhwc(const float* src, float* dst, int N, int C, int H_in, int W_in,
                                      int H_out, int W_out, spgt_stream_t stream);
 
-/* Activation and residual placement for spgt_linear_forward. */
+/* Tensor layouts for spgt_bilinear_resample. */
+enum { SPGT_LAYOUT_NCHW = 0, SPGT_LAYOUT_NHWC = 1 };
+
+/* Activations (spgt_linear_forward, spgt_ffn_scalar_forward, spgt_bilinear_resample) and
+ * residual placement for spgt_linear_forward. */
 enum { SPGT_ACT_NONE = 0, SPGT_ACT_RELU = 1, SPGT_ACT_SILU = 2 };
 enum { SPGT_RES_NONE = 0, SPGT_RES_BEFORE_ACT = 1, SPGT_RES_AFTER_ACT = 2 };
+
+/* The resampling of DownScaler2D / UpScaler2D (network/model.py:30-38, 59-64) together with the
+ * permutes and activations around it: F.interpolate(mode='bilinear', align_corners=True) from
+ * src [N, C, H_in, W_in] or [N, H_in, W_in, C] to dst [N, C, H_out, W_out] or [N, H_out, W_out, C]
+ * (NCHW->NCHW, NCHW->NHWC and NHWC->NCHW), with pre_activation applied pre_activation_count
+ * (0..2) times to every source sample (the activation of ConvResBlock2D, network/layer.py:7-24,
+ * and the scaler's own) and post_activation applied to the result. */
+int spgt_bilinear_resample(const float* src, float* dst, int N, int C, int H_in, int W_in, int H_out,
+                           int W_out, int src_layout, int dst_layout, int pre_activation,
+                           int pre_activation_count, int post_activation, spgt_stream_t stream);
 
 /* 1 when spgt_linear_forward has a kernel for this shape (in_features 64, 128, 136 or 256;
  * out_features a multiple of 32), else 0. */

@@ -26,7 +26,7 @@ namespace {
 
 __device__ __forceinline__ float activate(float v, int act) {
     if (act == SPGT_ACT_RELU) return fmaxf(v, 0.f);
-    if (act == SPGT_ACT_SILU) return v / (1.f + __expf(-v));
+    if (act == SPGT_ACT_SILU) return v * __builtin_amdgcn_rcpf(1.f + __expf(-v));
     return v;
 }
 
@@ -106,6 +106,13 @@ __global__ __launch_bounds__(256) void linear_tm_k(
                 if (bt * BK + j < KH) xv[bt & 1][j] = xr[2 * (bt * BK + j)];
         };
         lds_batch(0);
+        // the residual is fetched ahead of the MFMAs so that its latency hides behind them
+        const int64_t t = t0 + sub * 32 + tk;
+        float4 rq[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+            rq[q] = (res_mode && t < t_end) ? *reinterpret_cast<const float4*>(res + t * ldr + n0 + 4 * kh + 8 * q)
+                                            : make_float4(0.f, 0.f, 0.f, 0.f);
         v16f acc;
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[r] = 0.f;
@@ -119,15 +126,12 @@ __global__ __launch_bounds__(256) void linear_tm_k(
             __builtin_amdgcn_sched_barrier(0);
         }
 
-        const int64_t t = t0 + sub * 32 + tk;
         if (t < t_end) {
             // output column n lives in plane n / plane_cols at column n % plane_cols
             float* orow = out + (n0 / plane_cols) * plane_stride + t * ldo + n0 % plane_cols + 4 * kh;
-            const float* rrow = res_mode ? res + t * ldr + n0 + 4 * kh : nullptr;
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-                float4 r4 = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (res_mode) r4 = *reinterpret_cast<const float4*>(rrow + 8 * q);
+                const float4 r4 = rq[q];
                 float4 y;
                 y.x = acc[4 * q + 0] + breg[4 * q + 0];
                 y.y = acc[4 * q + 1] + breg[4 * q + 1];

@@ -106,6 +106,23 @@ __global__ __launch_bounds__(256) void spectrum_zero_outside_k(float2* __restric
     }
 }
 
+// Activations that the resampling kernels can apply to the source samples (`pre_n` times) and to
+// the result, standing in for the separate elementwise kernels of ConvResBlock2D and the scalers.
+struct ResampleAct {
+    int pre, pre_n, post;
+};
+
+__device__ __forceinline__ float act_apply(float v, int act) {
+    if (act == SPGT_ACT_RELU) return fmaxf(v, 0.f);
+    if (act == SPGT_ACT_SILU) return v * __builtin_amdgcn_rcpf(1.f + __expf(-v));
+    return v;
+}
+
+__device__ __forceinline__ float act_pre(float v, ResampleAct a) {
+    for (int i = 0; i < a.pre_n; ++i) v = act_apply(v, a.pre);
+    return v;
+}
+
 // Bilinear resampling with align_corners=True of [planes, Hin, Win] -> [planes, Hout, Wout].
 // Same arithmetic as torch's upsample_bilinear2d: scale = (in-1)/(out-1) in fp32
 // (0 when out == 1), source coordinate scale*dst, weights (1-l, l), rows blended last.
@@ -113,7 +130,7 @@ __global__ __launch_bounds__(256) void spectrum_zero_outside_k(float2* __restric
 __global__ __launch_bounds__(256) void bilinear_align_corners_k(const float* __restrict__ src,
                                                                 float* __restrict__ dst, int planes, int Hin,
                                                                 int Win, int Hout, int Wout, float hscale,
-                                                                float wscale) {
+                                                                float wscale, ResampleAct act) {
     const int ox = blockIdx.x * 64 + threadIdx.x;
     const int oy = blockIdx.y * 4 + threadIdx.y;
     if (ox >= Wout || oy >= Hout) return;
@@ -130,9 +147,9 @@ __global__ __launch_bounds__(256) void bilinear_align_corners_k(const float* __r
     for (int64_t pl = blockIdx.z; pl < planes; pl += gridDim.z) {
         const float* r0 = src + pl * Hin * Win + (int64_t)h1 * Win + w1;
         const float* r1 = r0 + (int64_t)hp * Win;
-        const float top = w0l * r0[0] + w1l * r0[wp];
-        const float bot = w0l * r1[0] + w1l * r1[wp];
-        dst[(pl * Hout + oy) * Wout + ox] = h0l * top + h1l * bot;
+        const float top = w0l * act_pre(r0[0], act) + w1l * act_pre(r0[wp], act);
+        const float bot = w0l * act_pre(r1[0], act) + w1l * act_pre(r1[wp], act);
+        dst[(pl * Hout + oy) * Wout + ox] = act_apply(h0l * top + h1l * bot, act.post);
     }
 }
 
@@ -142,7 +159,7 @@ __global__ __launch_bounds__(256) void bilinear_align_corners_k(const float* __r
 __global__ __launch_bounds__(256) void bilinear_align_corners_nhwc_k(const float* __restrict__ src,
                                                                      float* __restrict__ dst, int C, int Hin,
                                                                      int Win, int Hout, int Wout, float hscale,
-                                                                     float wscale) {
+                                                                     float wscale, ResampleAct act) {
     __shared__ float tile[32 * 33];
     const int tx = threadIdx.x & 31;
     const int ty = threadIdx.x >> 5;
@@ -171,9 +188,9 @@ __global__ __launch_bounds__(256) void bilinear_align_corners_nhwc_k(const float
             if (c0 + cl < C) {
                 const float* r0 = base + (int64_t)(c0 + cl) * plane;
                 const float* r1 = r0 + (int64_t)hp * Win;
-                const float top = w0l * r0[0] + w1l * r0[wp];
-                const float bot = w0l * r1[0] + w1l * r1[wp];
-                v = h0l * top + h1l * bot;
+                const float top = w0l * act_pre(r0[0], act) + w1l * act_pre(r0[wp], act);
+                const float bot = w0l * act_pre(r1[0], act) + w1l * act_pre(r1[wp], act);
+                v = act_apply(h0l * top + h1l * bot, act.post);
             }
             tile[cl * 33 + tx] = v;
         }
@@ -183,6 +200,58 @@ __global__ __launch_bounds__(256) void bilinear_align_corners_nhwc_k(const float
             const int xl = 8 * i + ty;
             const int x = blockIdx.x * 32 + xl;
             if (x < Wout && c0 + tx < C) drow[(int64_t)x * C + c0 + tx] = tile[tx * 33 + xl];
+        }
+        __syncthreads();
+    }
+}
+
+// The same resampling from a channels-last source: src [N, Hin, Win, C] -> dst [N, C, Hout, Wout].
+// grid (ceil(Wout/32), Hout, N), block 256 = 32 channels x 8 column lanes.  Reads run along C (the
+// four source pixels of an output column are 128-byte runs), a 32 x 32 (column x channel) tile is
+// turned in LDS, writes run along the output row of one channel.
+__global__ __launch_bounds__(256) void bilinear_align_corners_from_nhwc_k(const float* __restrict__ src,
+                                                                          float* __restrict__ dst, int C, int Hin,
+                                                                          int Win, int Hout, int Wout, float hscale,
+                                                                          float wscale, ResampleAct act) {
+    __shared__ float tile[32 * 33];
+    const int tx = threadIdx.x & 31;
+    const int ty = threadIdx.x >> 5;
+    const int oy = blockIdx.y;
+    const int64_t n = blockIdx.z;
+    const float hr = hscale * (float)oy;
+    const int h1 = (int)hr;
+    const int hp = (h1 < Hin - 1) ? 1 : 0;
+    const float h1l = hr - (float)h1;
+    const float h0l = 1.0f - h1l;
+    const float* rows = src + (n * Hin + h1) * (int64_t)Win * C;
+    const int64_t rstep = (int64_t)hp * Win * C;
+    for (int c0 = 0; c0 < C; c0 += 32) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int xl = 8 * i + ty;
+            const int ox = min(blockIdx.x * 32 + xl, Wout - 1);
+            const float wr = wscale * (float)ox;
+            const int w1 = (int)wr;
+            const int wp = (w1 < Win - 1) ? 1 : 0;
+            const float w1l = wr - (float)w1;
+            const float w0l = 1.0f - w1l;
+            float v = 0.f;
+            if (c0 + tx < C) {
+                const float* p0 = rows + (int64_t)w1 * C + c0 + tx;
+                const float* p1 = p0 + rstep;
+                const float top = w0l * act_pre(p0[0], act) + w1l * act_pre(p0[wp * C], act);
+                const float bot = w0l * act_pre(p1[0], act) + w1l * act_pre(p1[wp * C], act);
+                v = act_apply(h0l * top + h1l * bot, act.post);
+            }
+            tile[xl * 33 + tx] = v;
+        }
+        __syncthreads();
+        const int ox = blockIdx.x * 32 + tx;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int cl = 8 * i + ty;
+            if (ox < Wout && c0 + cl < C)
+                dst[((n * C + c0 + cl) * Hout + oy) * (int64_t)Wout + ox] = tile[tx * 33 + cl];
         }
         __syncthreads();
     }
@@ -248,36 +317,64 @@ extern "C" int spgt_spectral_modes_compact(const float* Z, const float* weight_1
     return check_launch("spectral_modes_compact");
 }
 
-extern "C" int spgt_bilinear_align_corners(const float* src, float* dst, int planes, int H_in, int W_in, int H_out,
-                                           int W_out, hipStream_t stream) {
-    if (!src || !dst) return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear_align_corners: null pointer argument");
-    if (planes <= 0 || H_in <= 0 || W_in <= 0 || H_out <= 0 || W_out <= 0)
-        return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear_align_corners: sizes must be positive");
-    if (ceil_div(H_out, 4) > 65535)
-        return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear_align_corners: H_out/4 exceeds 65535");
+namespace {
+
+bool act_known(int a) { return a == SPGT_ACT_NONE || a == SPGT_ACT_RELU || a == SPGT_ACT_SILU; }
+
+int resample_common(const char* who, const float* src, float* dst, int N, int C, int H_in, int W_in, int H_out,
+                    int W_out, int src_layout, int dst_layout, ResampleAct act, hipStream_t stream) {
+    if (!src || !dst) return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear resampling: null pointer argument");
+    if (N <= 0 || C <= 0 || H_in <= 0 || W_in <= 0 || H_out <= 0 || W_out <= 0)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear resampling: sizes must be positive");
     if (!aligned4(src) || !aligned4(dst))
-        return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear_align_corners: operands must be 4-byte aligned");
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear resampling: operands must be 4-byte aligned");
+    if (!act_known(act.pre) || !act_known(act.post) || act.pre_n < 0 || act.pre_n > 2)
+        return fail(SPGT_ERR_INVALID_ARGUMENT,
+                    "bilinear resampling: unknown activation, or more than two source activations");
     const float hscale = H_out > 1 ? (float)(H_in - 1) / (float)(H_out - 1) : 0.f;
     const float wscale = W_out > 1 ? (float)(W_in - 1) / (float)(W_out - 1) : 0.f;
-    const dim3 grid(ceil_div(W_out, 64), ceil_div(H_out, 4), std::min(planes, 65535));
-    hipLaunchKernelGGL(bilinear_align_corners_k, grid, dim3(64, 4), 0, stream, src, dst, planes, H_in, W_in, H_out,
-                       W_out, hscale, wscale);
-    return check_launch("bilinear_align_corners");
+    if (src_layout == SPGT_LAYOUT_NCHW && dst_layout == SPGT_LAYOUT_NCHW) {
+        const int64_t planes = (int64_t)N * C;
+        if (ceil_div(H_out, 4) > 65535 || planes > INT32_MAX)
+            return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear resampling: H_out/4 exceeds 65535 or too many planes");
+        const dim3 grid(ceil_div(W_out, 64), ceil_div(H_out, 4), (unsigned)std::min<int64_t>(planes, 65535));
+        hipLaunchKernelGGL(bilinear_align_corners_k, grid, dim3(64, 4), 0, stream, src, dst, (int)planes, H_in, W_in,
+                           H_out, W_out, hscale, wscale, act);
+    } else if (src_layout != dst_layout && (src_layout == SPGT_LAYOUT_NCHW || src_layout == SPGT_LAYOUT_NHWC) &&
+               (dst_layout == SPGT_LAYOUT_NCHW || dst_layout == SPGT_LAYOUT_NHWC)) {
+        if (H_out > 65535 || N > 65535)
+            return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear resampling: N or H_out exceeds 65535");
+        const dim3 grid(ceil_div(W_out, 32), H_out, N);
+        if (dst_layout == SPGT_LAYOUT_NHWC)
+            hipLaunchKernelGGL(bilinear_align_corners_nhwc_k, grid, dim3(256), 0, stream, src, dst, C, H_in, W_in,
+                               H_out, W_out, hscale, wscale, act);
+        else
+            hipLaunchKernelGGL(bilinear_align_corners_from_nhwc_k, grid, dim3(256), 0, stream, src, dst, C, H_in,
+                               W_in, H_out, W_out, hscale, wscale, act);
+    } else {
+        return fail(SPGT_ERR_INVALID_ARGUMENT,
+                    "bilinear resampling: layouts must be NCHW->NCHW, NCHW->NHWC or NHWC->NCHW");
+    }
+    return check_launch(who);
+}
+
+}  // namespace
+
+extern "C" int spgt_bilinear_align_corners(const float* src, float* dst, int planes, int H_in, int W_in, int H_out,
+                                           int W_out, hipStream_t stream) {
+    return resample_common("bilinear_align_corners", src, dst, 1, planes, H_in, W_in, H_out, W_out, SPGT_LAYOUT_NCHW,
+                           SPGT_LAYOUT_NCHW, ResampleAct{SPGT_ACT_NONE, 0, SPGT_ACT_NONE}, stream);
 }
 
 extern "C" int spgt_bilinear_align_corners_nhwc(const float* src, float* dst, int N, int C, int H_in, int W_in,
                                                 int H_out, int W_out, hipStream_t stream) {
-    if (!src || !dst) return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear_align_corners_nhwc: null pointer argument");
-    if (N <= 0 || C <= 0 || H_in <= 0 || W_in <= 0 || H_out <= 0 || W_out <= 0)
-        return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear_align_corners_nhwc: sizes must be positive");
-    if (H_out > 65535 || N > 65535)
-        return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear_align_corners_nhwc: N or H_out exceeds 65535");
-    if (!aligned4(src) || !aligned4(dst))
-        return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear_align_corners_nhwc: operands must be 4-byte aligned");
-    const float hscale = H_out > 1 ? (float)(H_in - 1) / (float)(H_out - 1) : 0.f;
-    const float wscale = W_out > 1 ? (float)(W_in - 1) / (float)(W_out - 1) : 0.f;
-    const dim3 grid(ceil_div(W_out, 32), H_out, N);
-    hipLaunchKernelGGL(bilinear_align_corners_nhwc_k, grid, dim3(256), 0, stream, src, dst, C, H_in, W_in, H_out,
-                       W_out, hscale, wscale);
-    return check_launch("bilinear_align_corners_nhwc");
+    return resample_common("bilinear_align_corners_nhwc", src, dst, N, C, H_in, W_in, H_out, W_out, SPGT_LAYOUT_NCHW,
+                           SPGT_LAYOUT_NHWC, ResampleAct{SPGT_ACT_NONE, 0, SPGT_ACT_NONE}, stream);
+}
+
+extern "C" int spgt_bilinear_resample(const float* src, float* dst, int N, int C, int H_in, int W_in, int H_out,
+                                      int W_out, int src_layout, int dst_layout, int pre_activation,
+                                      int pre_activation_count, int post_activation, hipStream_t stream) {
+    return resample_common("bilinear_resample", src, dst, N, C, H_in, W_in, H_out, W_out, src_layout, dst_layout,
+                           ResampleAct{pre_activation, pre_activation_count, post_activation}, stream);
 }

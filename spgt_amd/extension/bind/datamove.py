@@ -156,7 +156,40 @@ def _bilinear_align_corners_nhwc(X: Tensor, size) -> Tensor:
     return out
 
 
+_ACT = {None: 0, "none": 0, "relu": 1, "silu": 2}
+
+
+def _bilinear_resample(X: Tensor, size, src_nhwc: bool = False, dst_nhwc: bool = False, pre_activation=None,
+                       pre_count: int = 1, post_activation=None) -> Tensor:
+    """Bilinear align_corners resampling between layouts with the surrounding activations fused in:
+    X [N, C, H, W] (or [N, H, W, C] with src_nhwc) -> [N, C, H', W'] (or [N, H', W', C] with dst_nhwc);
+    pre_activation is applied pre_count times to the source samples, post_activation to the result."""
+    require_gpu_f32("X", X)
+    if X.dim() != 4:
+        raise ValueError("X must have four dimensions")
+    if src_nhwc and dst_nhwc:
+        raise ValueError("channels-last to channels-last resampling is not provided")
+    if pre_activation not in _ACT or post_activation not in _ACT:
+        raise ValueError("activations must be None, 'none', 'relu' or 'silu'")
+    H_out, W_out = (size, size) if isinstance(size, int) else tuple(size)
+    if src_nhwc:
+        N, H_in, W_in, C = X.shape
+    else:
+        N, C, H_in, W_in = X.shape
+    shape = (N, H_out, W_out, C) if dst_nhwc else (N, C, H_out, W_out)
+    out = torch.empty(shape, dtype=X.dtype, device=X.device)
+    if out.numel() == 0:
+        return out
+    npre = int(pre_count) if _ACT[pre_activation] else 0
+    with torch.cuda.device(X.device):
+        check(_lib.load().spgt_bilinear_resample(ptr(X), ptr(out), N, C, H_in, W_in, H_out, W_out, int(src_nhwc),
+                                                 int(dst_nhwc), _ACT[pre_activation], npre, _ACT[post_activation],
+                                                 stream_of(X)))
+    return out
+
+
 dexts = SimpleNamespace(
+    bilinear_resample=_bilinear_resample,
     bilinear_align_corners_nhwc=_bilinear_align_corners_nhwc,
     batched_transpose=_batched_transpose,
     transpose_gather_dual=_transpose_gather_dual,
@@ -245,3 +278,9 @@ def bilinear_align_corners(X: Tensor, size) -> Tensor:
 def bilinear_align_corners_nhwc(X: Tensor, size) -> Tensor:
     """F.interpolate(X, size, mode='bilinear', align_corners=True).permute(0, 2, 3, 1), contiguous (inference only)."""
     return dexts.bilinear_align_corners_nhwc(X.detach(), size)
+
+
+def bilinear_resample(X: Tensor, size, src_nhwc: bool = False, dst_nhwc: bool = False, pre_activation=None,
+                      pre_count: int = 1, post_activation=None) -> Tensor:
+    """post(interpolate(pre^pre_count(X))) between NCHW / NHWC layouts in one pass (inference only)."""
+    return dexts.bilinear_resample(X.detach(), size, src_nhwc, dst_nhwc, pre_activation, pre_count, post_activation)

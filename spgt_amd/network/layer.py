@@ -59,8 +59,10 @@ class ConvResBlock2D(nn.Module):
         self.conv_layer = nn.Conv2d(in_dim, out_dim, kernel_size=kernel_size, padding=padding)
         self.activation_layer = make_activation(activation)
 
-    def forward(self, X: Tensor) -> Tensor:
-        return self.activation_layer(always_dropout(self.conv_layer(X), self.droprate))
+    def forward(self, X: Tensor, activate: bool = True) -> Tensor:
+        """With activate=False the caller applies the activation (fused into its next kernel)."""
+        X = always_dropout(self.conv_layer(X), self.droprate)
+        return self.activation_layer(X) if activate else X
 
 
 class FeedForward(nn.Module):

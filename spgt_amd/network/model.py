@@ -7,8 +7,8 @@ import torch
 import torch.nn.functional as F
 from torch import Tensor, nn
 
-from ..extension.bind.datamove import bilinear_align_corners, bilinear_align_corners_nhwc
-from .layer import ConvResBlock2D, always_dropout, make_activation
+from ..extension.bind.datamove import bilinear_align_corners, bilinear_align_corners_nhwc, bilinear_resample
+from .layer import ConvResBlock2D, activation_name, always_dropout, gpu_inference, make_activation
 
 
 def resample(X: Tensor, size) -> Tensor:
@@ -49,13 +49,24 @@ class DownScaler2D(nn.Module):
         self.activation_layer = make_activation(activation)
 
     def forward(self, X: Tensor) -> Tensor:
-        X = self.conv0(nhwc_to_nchw(X))
-        X = self.activation_layer(resample(X, self.resolution_size[1]))
+        fused = gpu_inference(X, *self.parameters())
+        act = activation_name(self.activation_layer)
+        if fused:
+            # conv0's activation, the resampling and the scaler's activation in one pass
+            X = self.conv0(nhwc_to_nchw(X), activate=False)
+            X = bilinear_resample(X, self.resolution_size[1], pre_activation=activation_name(self.conv0.activation_layer),
+                                  post_activation=act)
+        else:
+            X = self.conv0(nhwc_to_nchw(X))
+            X = self.activation_layer(resample(X, self.resolution_size[1]))
         X1 = self.conv1(X)
         X2 = self.conv2(X1)
         X3 = self.conv3(X2)
+        X = torch.cat([X1, X2, X3], dim=1)
         # the activation commutes with the permute, so the second resampling can write channels-last directly
-        return self.activation_layer(resample_to_nhwc(torch.cat([X1, X2, X3], dim=1), self.resolution_size[2]))
+        if fused:
+            return bilinear_resample(X, self.resolution_size[2], dst_nhwc=True, post_activation=act)
+        return self.activation_layer(resample_to_nhwc(X, self.resolution_size[2]))
 
 
 class UpScaler2D(nn.Module):
@@ -69,6 +80,18 @@ class UpScaler2D(nn.Module):
         self.activation_layer = make_activation(activation)
 
     def forward(self, X: Tensor) -> Tensor:
+        if gpu_inference(X, *self.parameters()) and self.droprate == 0:
+            # channels-last in, NCHW out for the convolution; then the block's activation and the scaler's
+            # own are applied to the source samples of the second resampling, which writes channels-last
+            X = bilinear_resample(X.contiguous(), self.resolution_size[3], src_nhwc=True)
+            X = self.conv(X, activate=False)
+            if isinstance(self.activation_layer, nn.ReLU) and isinstance(self.conv.activation_layer, nn.ReLU):
+                # relu(relu(x)) = relu(x): one cheap clamp on the source samples of the resampling
+                return bilinear_resample(X, self.resolution_size[4], dst_nhwc=True, pre_activation="relu")
+            # an upsampling reads every source sample several times, so transcendental activations are
+            # applied once, in place, before it
+            X = self.activation_layer(self.conv.activation_layer(X))
+            return bilinear_resample(X, self.resolution_size[4], dst_nhwc=True)
         X = resample(X.permute(0, 3, 1, 2), self.resolution_size[3])
         X = self.activation_layer(always_dropout(self.conv(X), self.droprate))
         return resample_to_nhwc(X, self.resolution_size[4])

@@ -213,3 +213,38 @@ def test_bilinear_nhwc_matches_nchw_kernel(gpu, shape, size):
     got = dm.bilinear_align_corners_nhwc(x, size)
     assert got.is_contiguous() and got.shape == want.shape
     assert torch.equal(got, want)
+
+
+def _act64(x, name, count=1):
+    for _ in range(count if name else 0):
+        x = torch.relu(x) if name == "relu" else x * torch.sigmoid(x)
+    return x
+
+
+@pytest.mark.parametrize("shape,size", [((2, 3, 7, 9), (4, 5)), ((1, 128, 71, 71), (122, 122)), ((2, 40, 9, 33), (9, 70)),
+                                        ((1, 1, 5, 5), (1, 1))])
+@pytest.mark.parametrize("src_nhwc,dst_nhwc", [(False, False), (False, True), (True, False)])
+@pytest.mark.parametrize("pre,count,post", [(None, 0, None), ("silu", 1, "silu"), ("relu", 2, None), (None, 0, "relu"),
+                                            ("silu", 2, None)])
+def test_bilinear_resample_layouts_and_activations(gpu, shape, size, src_nhwc, dst_nhwc, pre, count, post):
+    """post(interpolate(pre^count(x))) between layouts, against the float64 oracle resampling
+    (network/model.py:30-38, 59-64 with the activations of network/layer.py:7-24 around it)."""
+    x = rnd(*shape, seed=41)  # NCHW master copy
+    want = _act64(O.bilinear_align_corners(_act64(x.double(), pre, count), size), post)
+    src = x.permute(0, 2, 3, 1).contiguous() if src_nhwc else x
+    got = dm.bilinear_resample(src.to(gpu), size, src_nhwc=src_nhwc, dst_nhwc=dst_nhwc, pre_activation=pre,
+                               pre_count=max(count, 1), post_activation=post)
+    assert got.is_contiguous()
+    got = got.cpu().double()
+    if dst_nhwc:
+        got = got.permute(0, 3, 1, 2)
+    assert got.shape == want.shape
+    assert (got - want).abs().max().item() <= 1e-5 * max(1.0, want.abs().max().item())
+
+
+def test_bilinear_resample_rejects(gpu):
+    x = rnd(1, 4, 5, 5, seed=1).to(gpu)
+    with pytest.raises(ValueError):
+        dm.bilinear_resample(x, (3, 3), src_nhwc=True, dst_nhwc=True)
+    with pytest.raises(ValueError):
+        dm.bilinear_resample(x, (3, 3), pre_activation="tanh")
