@@ -205,10 +205,19 @@ enum { SPGT_RES_NONE = 0, SPGT_RES_BEFORE_ACT = 1, SPGT_RES_AFTER_ACT = 2 };
  * src [N, C, H_in, W_in] or [N, H_in, W_in, C] to dst [N, C, H_out, W_out] or [N, H_out, W_out, C]
  * (NCHW->NCHW, NCHW->NHWC and NHWC->NCHW), with pre_activation applied pre_activation_count
  * (0..2) times to every source sample (the activation of ConvResBlock2D, network/layer.py:7-24,
- * and the scaler's own) and post_activation applied to the result. */
-int spgt_bilinear_resample(const float* src, float* dst, int N, int C, int H_in, int W_in, int H_out,
-                           int W_out, int src_layout, int dst_layout, int pre_activation,
-                           int pre_activation_count, int post_activation, spgt_stream_t stream);
+ * and the scaler's own) and post_activation applied to the result.  pre_bias [C] (may be null) is
+ * added to every source sample first: the bias of a convolution that was run without it. */
+int spgt_bilinear_resample(const float* src, const float* pre_bias, float* dst, int N, int C, int H_in,
+                           int W_in, int H_out, int W_out, int src_layout, int dst_layout,
+                           int pre_activation, int pre_activation_count, int post_activation,
+                           spgt_stream_t stream);
+
+/* The tail of ConvResBlock2D (network/layer.py:7-24) after a bias-free convolution, and the
+ * scaler's own activation where it follows directly (network/model.py:61-62), in place:
+ * x[n, c, :] = activation^activation_count(x[n, c, :] + bias[c]) on x [N, C, HW]; bias may be null,
+ * activation_count is 0..2. */
+int spgt_bias_activation_nchw(float* x, const float* bias, int N, int C, int64_t HW, int activation,
+                              int activation_count, spgt_stream_t stream);
 
 /* 1 when spgt_linear_forward has a kernel for this shape (in_features 64, 128, 136 or 256;
  * out_features a multiple of 32), else 0. */

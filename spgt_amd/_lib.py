@@ -45,7 +45,8 @@ SIGNATURES = {
     "spgt_spectral_modes_compact": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _i, _p]),
     "spgt_bilinear_align_corners": (_i, [_p, _p, _i, _i, _i, _i, _i, _p]),
     "spgt_bilinear_align_corners_nhwc": (_i, [_p, _p, _i, _i, _i, _i, _i, _i, _p]),
-    "spgt_bilinear_resample": (_i, [_p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p]),
+    "spgt_bilinear_resample": (_i, [_p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p]),
+    "spgt_bias_activation_nchw": (_i, [_p, _p, _i, _i, _i64, _i, _i, _p]),
     "spgt_linear_supported": (_i, [_i, _i]),
     "spgt_linear_forward": (_i, [_p, _i64, _p, _p, _p, _i64, _i, _i, _p, _i64, _i, _i64, _i64, _i, _i, _p]),
     "spgt_ffn_scalar_supported": (_i, [_i, _i]),

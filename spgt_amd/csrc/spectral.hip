@@ -128,6 +128,7 @@ __device__ __forceinline__ float act_pre(float v, ResampleAct a) {
 // (0 when out == 1), source coordinate scale*dst, weights (1-l, l), rows blended last.
 // grid (ceil(Wout/64), ceil(Hout/4), planes), block (64, 4).
 __global__ __launch_bounds__(256) void bilinear_align_corners_k(const float* __restrict__ src,
+                                                                const float* __restrict__ pre_bias, int C,
                                                                 float* __restrict__ dst, int planes, int Hin,
                                                                 int Win, int Hout, int Wout, float hscale,
                                                                 float wscale, ResampleAct act) {
@@ -147,8 +148,9 @@ __global__ __launch_bounds__(256) void bilinear_align_corners_k(const float* __r
     for (int64_t pl = blockIdx.z; pl < planes; pl += gridDim.z) {
         const float* r0 = src + pl * Hin * Win + (int64_t)h1 * Win + w1;
         const float* r1 = r0 + (int64_t)hp * Win;
-        const float top = w0l * act_pre(r0[0], act) + w1l * act_pre(r0[wp], act);
-        const float bot = w0l * act_pre(r1[0], act) + w1l * act_pre(r1[wp], act);
+        const float pb = pre_bias ? pre_bias[pl % C] : 0.f;
+        const float top = w0l * act_pre(r0[0] + pb, act) + w1l * act_pre(r0[wp] + pb, act);
+        const float bot = w0l * act_pre(r1[0] + pb, act) + w1l * act_pre(r1[wp] + pb, act);
         dst[(pl * Hout + oy) * Wout + ox] = act_apply(h0l * top + h1l * bot, act.post);
     }
 }
@@ -157,6 +159,7 @@ __global__ __launch_bounds__(256) void bilinear_align_corners_k(const float* __r
 // grid (ceil(Wout/32), Hout, N), block 256 = 32 output columns x 8 channel lanes.  Reads run along the
 // source rows of one channel, a 32 x 32 (channel x column) tile is turned in LDS, writes run along C.
 __global__ __launch_bounds__(256) void bilinear_align_corners_nhwc_k(const float* __restrict__ src,
+                                                                     const float* __restrict__ pre_bias,
                                                                      float* __restrict__ dst, int C, int Hin,
                                                                      int Win, int Hout, int Wout, float hscale,
                                                                      float wscale, ResampleAct act) {
@@ -188,8 +191,9 @@ __global__ __launch_bounds__(256) void bilinear_align_corners_nhwc_k(const float
             if (c0 + cl < C) {
                 const float* r0 = base + (int64_t)(c0 + cl) * plane;
                 const float* r1 = r0 + (int64_t)hp * Win;
-                const float top = w0l * act_pre(r0[0], act) + w1l * act_pre(r0[wp], act);
-                const float bot = w0l * act_pre(r1[0], act) + w1l * act_pre(r1[wp], act);
+                const float pb = pre_bias ? pre_bias[c0 + cl] : 0.f;
+                const float top = w0l * act_pre(r0[0] + pb, act) + w1l * act_pre(r0[wp] + pb, act);
+                const float bot = w0l * act_pre(r1[0] + pb, act) + w1l * act_pre(r1[wp] + pb, act);
                 v = act_apply(h0l * top + h1l * bot, act.post);
             }
             tile[cl * 33 + tx] = v;
@@ -210,6 +214,7 @@ __global__ __launch_bounds__(256) void bilinear_align_corners_nhwc_k(const float
 // four source pixels of an output column are 128-byte runs), a 32 x 32 (column x channel) tile is
 // turned in LDS, writes run along the output row of one channel.
 __global__ __launch_bounds__(256) void bilinear_align_corners_from_nhwc_k(const float* __restrict__ src,
+                                                                          const float* __restrict__ pre_bias,
                                                                           float* __restrict__ dst, int C, int Hin,
                                                                           int Win, int Hout, int Wout, float hscale,
                                                                           float wscale, ResampleAct act) {
@@ -239,8 +244,9 @@ __global__ __launch_bounds__(256) void bilinear_align_corners_from_nhwc_k(const 
             if (c0 + tx < C) {
                 const float* p0 = rows + (int64_t)w1 * C + c0 + tx;
                 const float* p1 = p0 + rstep;
-                const float top = w0l * act_pre(p0[0], act) + w1l * act_pre(p0[wp * C], act);
-                const float bot = w0l * act_pre(p1[0], act) + w1l * act_pre(p1[wp * C], act);
+                const float pb = pre_bias ? pre_bias[c0 + tx] : 0.f;
+                const float top = w0l * act_pre(p0[0] + pb, act) + w1l * act_pre(p0[wp * C] + pb, act);
+                const float bot = w0l * act_pre(p1[0] + pb, act) + w1l * act_pre(p1[wp * C] + pb, act);
                 v = act_apply(h0l * top + h1l * bot, act.post);
             }
             tile[xl * 33 + tx] = v;
@@ -254,6 +260,20 @@ __global__ __launch_bounds__(256) void bilinear_align_corners_from_nhwc_k(const 
                 dst[((n * C + c0 + cl) * Hout + oy) * (int64_t)Wout + ox] = tile[tx * 33 + cl];
         }
         __syncthreads();
+    }
+}
+
+// x[n, c, :] = act^count(x[n, c, :] + bias[c]) in place on [planes = N*C, HW]: the bias add and the
+// activation(s) that follow a bias-free convolution.  grid (chunks, planes), block 256.
+__global__ __launch_bounds__(256) void bias_activation_nchw_k(float* __restrict__ x, const float* __restrict__ bias,
+                                                              int C, int64_t HW, int act, int count) {
+    const int64_t pl = blockIdx.y;
+    const float b = bias ? bias[pl % C] : 0.f;
+    float* row = x + pl * HW;
+    for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < HW; e += (int64_t)gridDim.x * 256) {
+        float v = row[e] + b;
+        for (int i = 0; i < count; ++i) v = act_apply(v, act);
+        row[e] = v;
     }
 }
 
@@ -321,7 +341,7 @@ namespace {
 
 bool act_known(int a) { return a == SPGT_ACT_NONE || a == SPGT_ACT_RELU || a == SPGT_ACT_SILU; }
 
-int resample_common(const char* who, const float* src, float* dst, int N, int C, int H_in, int W_in, int H_out,
+int resample_common(const char* who, const float* src, const float* pre_bias, float* dst, int N, int C, int H_in, int W_in, int H_out,
                     int W_out, int src_layout, int dst_layout, ResampleAct act, hipStream_t stream) {
     if (!src || !dst) return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear resampling: null pointer argument");
     if (N <= 0 || C <= 0 || H_in <= 0 || W_in <= 0 || H_out <= 0 || W_out <= 0)
@@ -338,19 +358,19 @@ int resample_common(const char* who, const float* src, float* dst, int N, int C,
         if (ceil_div(H_out, 4) > 65535 || planes > INT32_MAX)
             return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear resampling: H_out/4 exceeds 65535 or too many planes");
         const dim3 grid(ceil_div(W_out, 64), ceil_div(H_out, 4), (unsigned)std::min<int64_t>(planes, 65535));
-        hipLaunchKernelGGL(bilinear_align_corners_k, grid, dim3(64, 4), 0, stream, src, dst, (int)planes, H_in, W_in,
-                           H_out, W_out, hscale, wscale, act);
+        hipLaunchKernelGGL(bilinear_align_corners_k, grid, dim3(64, 4), 0, stream, src, pre_bias, C, dst, (int)planes, H_in,
+                           W_in, H_out, W_out, hscale, wscale, act);
     } else if (src_layout != dst_layout && (src_layout == SPGT_LAYOUT_NCHW || src_layout == SPGT_LAYOUT_NHWC) &&
                (dst_layout == SPGT_LAYOUT_NCHW || dst_layout == SPGT_LAYOUT_NHWC)) {
         if (H_out > 65535 || N > 65535)
             return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear resampling: N or H_out exceeds 65535");
         const dim3 grid(ceil_div(W_out, 32), H_out, N);
         if (dst_layout == SPGT_LAYOUT_NHWC)
-            hipLaunchKernelGGL(bilinear_align_corners_nhwc_k, grid, dim3(256), 0, stream, src, dst, C, H_in, W_in,
-                               H_out, W_out, hscale, wscale, act);
-        else
-            hipLaunchKernelGGL(bilinear_align_corners_from_nhwc_k, grid, dim3(256), 0, stream, src, dst, C, H_in,
+            hipLaunchKernelGGL(bilinear_align_corners_nhwc_k, grid, dim3(256), 0, stream, src, pre_bias, dst, C, H_in,
                                W_in, H_out, W_out, hscale, wscale, act);
+        else
+            hipLaunchKernelGGL(bilinear_align_corners_from_nhwc_k, grid, dim3(256), 0, stream, src, pre_bias, dst, C,
+                               H_in, W_in, H_out, W_out, hscale, wscale, act);
     } else {
         return fail(SPGT_ERR_INVALID_ARGUMENT,
                     "bilinear resampling: layouts must be NCHW->NCHW, NCHW->NHWC or NHWC->NCHW");
@@ -362,19 +382,37 @@ int resample_common(const char* who, const float* src, float* dst, int N, int C,
 
 extern "C" int spgt_bilinear_align_corners(const float* src, float* dst, int planes, int H_in, int W_in, int H_out,
                                            int W_out, hipStream_t stream) {
-    return resample_common("bilinear_align_corners", src, dst, 1, planes, H_in, W_in, H_out, W_out, SPGT_LAYOUT_NCHW,
+    return resample_common("bilinear_align_corners", src, nullptr, dst, 1, planes, H_in, W_in, H_out, W_out, SPGT_LAYOUT_NCHW,
                            SPGT_LAYOUT_NCHW, ResampleAct{SPGT_ACT_NONE, 0, SPGT_ACT_NONE}, stream);
 }
 
 extern "C" int spgt_bilinear_align_corners_nhwc(const float* src, float* dst, int N, int C, int H_in, int W_in,
                                                 int H_out, int W_out, hipStream_t stream) {
-    return resample_common("bilinear_align_corners_nhwc", src, dst, N, C, H_in, W_in, H_out, W_out, SPGT_LAYOUT_NCHW,
+    return resample_common("bilinear_align_corners_nhwc", src, nullptr, dst, N, C, H_in, W_in, H_out, W_out, SPGT_LAYOUT_NCHW,
                            SPGT_LAYOUT_NHWC, ResampleAct{SPGT_ACT_NONE, 0, SPGT_ACT_NONE}, stream);
 }
 
-extern "C" int spgt_bilinear_resample(const float* src, float* dst, int N, int C, int H_in, int W_in, int H_out,
-                                      int W_out, int src_layout, int dst_layout, int pre_activation,
-                                      int pre_activation_count, int post_activation, hipStream_t stream) {
-    return resample_common("bilinear_resample", src, dst, N, C, H_in, W_in, H_out, W_out, src_layout, dst_layout,
+extern "C" int spgt_bilinear_resample(const float* src, const float* pre_bias, float* dst, int N, int C, int H_in,
+                                      int W_in, int H_out, int W_out, int src_layout, int dst_layout,
+                                      int pre_activation, int pre_activation_count, int post_activation,
+                                      hipStream_t stream) {
+    if (pre_bias && !aligned4(pre_bias))
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear_resample: pre_bias must be 4-byte aligned");
+    return resample_common("bilinear_resample", src, pre_bias, dst, N, C, H_in, W_in, H_out, W_out, src_layout, dst_layout,
                            ResampleAct{pre_activation, pre_activation_count, post_activation}, stream);
+}
+
+extern "C" int spgt_bias_activation_nchw(float* x, const float* bias, int N, int C, int64_t HW, int activation,
+                                         int activation_count, hipStream_t stream) {
+    if (!x) return fail(SPGT_ERR_INVALID_ARGUMENT, "bias_activation_nchw: null pointer argument");
+    if (N <= 0 || C <= 0 || HW <= 0) return fail(SPGT_ERR_INVALID_ARGUMENT, "bias_activation_nchw: sizes must be positive");
+    if ((int64_t)N * C > 65535) return fail(SPGT_ERR_INVALID_ARGUMENT, "bias_activation_nchw: N*C exceeds 65535");
+    if (!act_known(activation) || activation_count < 0 || activation_count > 2)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "bias_activation_nchw: unknown activation or count outside 0..2");
+    if (!aligned4(x) || (bias && !aligned4(bias)))
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "bias_activation_nchw: operands must be 4-byte aligned");
+    const int chunks = (int)std::min<int64_t>(ceil_div(HW, (int64_t)1024), 64);
+    hipLaunchKernelGGL(bias_activation_nchw_k, dim3(chunks, N * C), dim3(256), 0, stream, x, bias, C, HW, activation,
+                       activation == SPGT_ACT_NONE ? 0 : activation_count);
+    return check_launch("bias_activation_nchw");
 }

@@ -160,10 +160,11 @@ _ACT = {None: 0, "none": 0, "relu": 1, "silu": 2}
 
 
 def _bilinear_resample(X: Tensor, size, src_nhwc: bool = False, dst_nhwc: bool = False, pre_activation=None,
-                       pre_count: int = 1, post_activation=None) -> Tensor:
-    """Bilinear align_corners resampling between layouts with the surrounding activations fused in:
+                       pre_count: int = 1, post_activation=None, pre_bias: Tensor = None) -> Tensor:
+    """Bilinear align_corners resampling between layouts with the surrounding elementwise steps fused in:
     X [N, C, H, W] (or [N, H, W, C] with src_nhwc) -> [N, C, H', W'] (or [N, H', W', C] with dst_nhwc);
-    pre_activation is applied pre_count times to the source samples, post_activation to the result."""
+    pre_bias [C] is added to the source samples, pre_activation is then applied to them pre_count times,
+    post_activation is applied to the result."""
     require_gpu_f32("X", X)
     if X.dim() != 4:
         raise ValueError("X must have four dimensions")
@@ -181,14 +182,40 @@ def _bilinear_resample(X: Tensor, size, src_nhwc: bool = False, dst_nhwc: bool =
     if out.numel() == 0:
         return out
     npre = int(pre_count) if _ACT[pre_activation] else 0
+    if pre_bias is not None:
+        require_gpu_f32("pre_bias", pre_bias)
+        if pre_bias.numel() != C:
+            raise ValueError(f"pre_bias has {pre_bias.numel()} elements, expected {C}")
     with torch.cuda.device(X.device):
-        check(_lib.load().spgt_bilinear_resample(ptr(X), ptr(out), N, C, H_in, W_in, H_out, W_out, int(src_nhwc),
+        check(_lib.load().spgt_bilinear_resample(ptr(X), ptr(pre_bias) if pre_bias is not None else None, ptr(out), N, C, H_in, W_in, H_out, W_out, int(src_nhwc),
                                                  int(dst_nhwc), _ACT[pre_activation], npre, _ACT[post_activation],
                                                  stream_of(X)))
     return out
 
 
+def _bias_activation_nchw_(X: Tensor, bias, activation=None, count: int = 1) -> Tensor:
+    """In place on X [N, C, ...]: X = activation^count(X + bias[c]); returns X."""
+    require_gpu_f32("X", X)
+    if X.dim() < 2:
+        raise ValueError("X needs at least two dimensions")
+    if activation not in _ACT:
+        raise ValueError("activation must be None, 'none', 'relu' or 'silu'")
+    N, C = X.shape[:2]
+    HW = prod(X.shape[2:])
+    if bias is not None:
+        require_gpu_f32("bias", bias)
+        if bias.numel() != C:
+            raise ValueError(f"bias has {bias.numel()} elements, expected {C}")
+    if X.numel() == 0:
+        return X
+    with torch.cuda.device(X.device):
+        check(_lib.load().spgt_bias_activation_nchw(ptr(X), ptr(bias) if bias is not None else None, N, C, HW,
+                                                    _ACT[activation], int(count), stream_of(X)))
+    return X
+
+
 dexts = SimpleNamespace(
+    bias_activation_nchw_=_bias_activation_nchw_,
     bilinear_resample=_bilinear_resample,
     bilinear_align_corners_nhwc=_bilinear_align_corners_nhwc,
     batched_transpose=_batched_transpose,
@@ -281,6 +308,12 @@ def bilinear_align_corners_nhwc(X: Tensor, size) -> Tensor:
 
 
 def bilinear_resample(X: Tensor, size, src_nhwc: bool = False, dst_nhwc: bool = False, pre_activation=None,
-                      pre_count: int = 1, post_activation=None) -> Tensor:
-    """post(interpolate(pre^pre_count(X))) between NCHW / NHWC layouts in one pass (inference only)."""
-    return dexts.bilinear_resample(X.detach(), size, src_nhwc, dst_nhwc, pre_activation, pre_count, post_activation)
+                      pre_count: int = 1, post_activation=None, pre_bias: Tensor = None) -> Tensor:
+    """post(interpolate(pre^pre_count(X + pre_bias))) between NCHW / NHWC layouts in one pass (inference only)."""
+    return dexts.bilinear_resample(X.detach(), size, src_nhwc, dst_nhwc, pre_activation, pre_count, post_activation,
+                                   None if pre_bias is None else pre_bias.detach())
+
+
+def bias_activation_nchw_(X: Tensor, bias, activation=None, count: int = 1) -> Tensor:
+    """In place: X = activation^count(X + bias[c]) on [N, C, ...] (inference only)."""
+    return dexts.bias_activation_nchw_(X, None if bias is None else bias.detach(), activation, count)

@@ -11,6 +11,7 @@ import torch
 import torch.nn.functional as F
 from torch import Tensor, nn
 
+from ..extension.bind.datamove import bias_activation_nchw_
 from ..extension.bind.linear import ffn_scalar_supported, fused_ffn_scalar, fused_linear, linear_supported
 
 
@@ -59,10 +60,25 @@ class ConvResBlock2D(nn.Module):
         self.conv_layer = nn.Conv2d(in_dim, out_dim, kernel_size=kernel_size, padding=padding)
         self.activation_layer = make_activation(activation)
 
-    def forward(self, X: Tensor, activate: bool = True) -> Tensor:
-        """With activate=False the caller applies the activation (fused into its next kernel)."""
-        X = always_dropout(self.conv_layer(X), self.droprate)
-        return self.activation_layer(X) if activate else X
+    def fusable(self, X: Tensor) -> bool:
+        """Inference without dropout: the bias and the activation can ride in the caller's next kernel."""
+        return self.droprate == 0 and gpu_inference(X, *self.parameters())
+
+    def conv_raw(self, X: Tensor) -> Tensor:
+        """The convolution without its bias (to be added by the kernel that consumes the result)."""
+        c = self.conv_layer
+        Y = F.conv2d(X, c.weight, None, c.stride, c.padding, c.dilation, c.groups)
+        return Y if Y.is_contiguous() else Y.contiguous()
+
+    def forward(self, X: Tensor, extra_activations: int = 0) -> Tensor:
+        """conv -> dropout -> activation, the activation applied 1 + extra_activations times."""
+        if self.fusable(X):
+            return bias_activation_nchw_(self.conv_raw(X), self.conv_layer.bias, activation_name(self.activation_layer),
+                                         1 + extra_activations)
+        X = self.activation_layer(always_dropout(self.conv_layer(X), self.droprate))
+        for _ in range(extra_activations):
+            X = self.activation_layer(X)
+        return X
 
 
 class FeedForward(nn.Module):

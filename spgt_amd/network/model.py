@@ -51,14 +51,13 @@ class DownScaler2D(nn.Module):
     def forward(self, X: Tensor) -> Tensor:
         fused = gpu_inference(X, *self.parameters())
         act = activation_name(self.activation_layer)
-        if fused:
-            # conv0's activation, the resampling and the scaler's activation in one pass
-            X = self.conv0(nhwc_to_nchw(X), activate=False)
-            X = bilinear_resample(X, self.resolution_size[1], pre_activation=activation_name(self.conv0.activation_layer),
-                                  post_activation=act)
+        X = nhwc_to_nchw(X)
+        if fused and self.conv0.fusable(X):
+            # conv0's bias and activation, the resampling and the scaler's activation in one pass
+            X = bilinear_resample(self.conv0.conv_raw(X), self.resolution_size[1], pre_bias=self.conv0.conv_layer.bias,
+                                  pre_activation=activation_name(self.conv0.activation_layer), post_activation=act)
         else:
-            X = self.conv0(nhwc_to_nchw(X))
-            X = self.activation_layer(resample(X, self.resolution_size[1]))
+            X = self.activation_layer(resample(self.conv0(X), self.resolution_size[1]))
         X1 = self.conv1(X)
         X2 = self.conv2(X1)
         X3 = self.conv3(X2)
@@ -81,16 +80,14 @@ class UpScaler2D(nn.Module):
 
     def forward(self, X: Tensor) -> Tensor:
         if gpu_inference(X, *self.parameters()) and self.droprate == 0:
-            # channels-last in, NCHW out for the convolution; then the block's activation and the scaler's
-            # own are applied to the source samples of the second resampling, which writes channels-last
+            # channels-last in, NCHW out for the convolution; the block's bias and activation and the
+            # scaler's own activation are one in-place pass (an upsampling reads every source sample
+            # several times, so they are not applied inside it); the second resampling writes channels-last
             X = bilinear_resample(X.contiguous(), self.resolution_size[3], src_nhwc=True)
-            X = self.conv(X, activate=False)
-            if isinstance(self.activation_layer, nn.ReLU) and isinstance(self.conv.activation_layer, nn.ReLU):
-                # relu(relu(x)) = relu(x): one cheap clamp on the source samples of the resampling
-                return bilinear_resample(X, self.resolution_size[4], dst_nhwc=True, pre_activation="relu")
-            # an upsampling reads every source sample several times, so transcendental activations are
-            # applied once, in place, before it
-            X = self.activation_layer(self.conv.activation_layer(X))
+            if type(self.conv.activation_layer) is type(self.activation_layer):
+                X = self.conv(X, extra_activations=1)
+            else:
+                X = self.activation_layer(self.conv(X))
             return bilinear_resample(X, self.resolution_size[4], dst_nhwc=True)
         X = resample(X.permute(0, 3, 1, 2), self.resolution_size[3])
         X = self.activation_layer(always_dropout(self.conv(X), self.droprate))

@@ -248,3 +248,34 @@ def test_bilinear_resample_rejects(gpu):
         dm.bilinear_resample(x, (3, 3), src_nhwc=True, dst_nhwc=True)
     with pytest.raises(ValueError):
         dm.bilinear_resample(x, (3, 3), pre_activation="tanh")
+
+
+@pytest.mark.parametrize("shape", [(2, 5, 7, 9), (4, 42, 122, 122), (1, 3, 1), (2, 128, 33, 31)])
+@pytest.mark.parametrize("act,count", [(None, 1), ("relu", 1), ("silu", 1), ("silu", 2), ("relu", 2)])
+@pytest.mark.parametrize("with_bias", [True, False])
+def test_bias_activation_nchw(gpu, shape, act, count, with_bias):
+    """In-place bias + activation(s) after a bias-free convolution (network/layer.py:7-24), against float64."""
+    x = rnd(*shape, seed=51)
+    b = rnd(shape[1], seed=52) if with_bias else None
+    want = x.double()
+    if with_bias:
+        want = want + b.double().view(1, -1, *([1] * (len(shape) - 2)))
+    want = _act64(want, act, count)
+    xd = x.to(gpu)
+    got = dm.bias_activation_nchw_(xd, b.to(gpu) if with_bias else None, act, count)
+    assert got.data_ptr() == xd.data_ptr()
+    assert (got.cpu().double() - want).abs().max().item() <= 1e-5 * max(1.0, want.abs().max().item())
+
+
+@pytest.mark.parametrize("src_nhwc,dst_nhwc", [(False, False), (False, True), (True, False)])
+def test_bilinear_resample_pre_bias(gpu, src_nhwc, dst_nhwc):
+    """The bias of a bias-free convolution added to the source samples before the activation."""
+    x = rnd(2, 40, 9, 33, seed=61)
+    b = rnd(40, seed=62)
+    want = O.bilinear_align_corners(_act64(x.double() + b.double().view(1, -1, 1, 1), "silu"), (13, 20))
+    src = x.permute(0, 2, 3, 1).contiguous() if src_nhwc else x
+    got = dm.bilinear_resample(src.to(gpu), (13, 20), src_nhwc=src_nhwc, dst_nhwc=dst_nhwc, pre_activation="silu",
+                               pre_bias=b.to(gpu)).cpu().double()
+    if dst_nhwc:
+        got = got.permute(0, 3, 1, 2)
+    assert (got - want).abs().max().item() <= 1e-5 * max(1.0, want.abs().max().item())
