@@ -192,6 +192,26 @@ int spgt_bilinear_align_corners(const float* src, float* dst, int planes, int H_
 int spgt_bilinear_align_corners_nhwc(const float* src, float* dst, int N, int C, int H_in, int W_in,
                                      int H_out, int W_out, spgt_stream_t stream);
 
+/* 1 when the truncated-DFT row kernels serve this shape (r <= 1024, channels a multiple of 32,
+ * modes <= 16), else 0. */
+int spgt_truncated_dft_rows_supported(int r, int channels, int modes);
+
+/* The w-direction of rfft2 restricted to the modes Sp_SpectralConv2D keeps
+ * (network/sp_layer.py:136-141: rfft2, then only columns kw < modes are read):
+ *   Y[row, c, j] = sum_w x[row, w, c] * table[w, j],   j = (kw, re|im) < 2*modes
+ * x [rows, r, channels] (rows = N*r grid rows of the channels-last tensor), table [r, 2*modes]
+ * holds (cos, -sin)(2 pi kw w / r) / sqrt(r), Y [rows, channels, 2*modes]. */
+int spgt_truncated_dft_rows_forward(const float* x, const float* table, float* Y, int64_t rows, int r,
+                                    int channels, int modes, spgt_stream_t stream);
+
+/* The w-direction of irfft2 for a spectrum that is zero beyond column `modes`
+ * (network/sp_layer.py:149-151):
+ *   y[row, w, o] = sum_j table[w, j] * U[row, o, j]
+ * U [rows, channels, 2*modes], table [r, 2*modes] (the forward table with columns scaled by 1 for
+ * kw = 0 and the Nyquist column, else 2), y [rows, r, channels]. */
+int spgt_truncated_dft_rows_inverse(const float* U, const float* table, float* y, int64_t rows, int r,
+                                    int channels, int modes, spgt_stream_t stream);
+
 /* Tensor layouts for spgt_bilinear_resample. */
 enum { SPGT_LAYOUT_NCHW = 0, SPGT_LAYOUT_NHWC = 1 };
 

@@ -33,6 +33,7 @@ struct SpecLayout {
 // (NB batch entries at a time), the mode's weight block [Cin, 64] is streamed
 // once per batch group with 512-byte coalesced rows.
 constexpr int kSpecNB = 16;
+constexpr int kSpecWB = 32;  // weight rows per load batch
 
 __global__ __launch_bounds__(256) void spectral_mode_contract_k(
     const float2* __restrict__ X, const float2* __restrict__ W0, const float2* __restrict__ W1,
@@ -69,18 +70,26 @@ __global__ __launch_bounds__(256) void spectral_mode_contract_k(
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[j] = make_float2(0.f, 0.f);
         if (o < Cout) {
-#pragma unroll 8
-            for (int i = 0; i < Cin; ++i) {
-                const float2 wv = Wm[(int64_t)i * Cout + o];
+            // the weight rows are fetched kSpecWB at a time, all loads of a batch in flight together:
+            // the kernel's time is a few memory round trips, not one per input channel
+            for (int i0 = 0; i0 < Cin; i0 += kSpecWB) {
+                float2 wv[kSpecWB];
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const int n = ng + 4 * j;
-                    if (n < nb) {
-                        const float2 xv = xs[n * Cin + i];
-                        acc[j].x = fmaf(xv.x, wv.x, acc[j].x);
-                        acc[j].x = fmaf(-xv.y, wv.y, acc[j].x);
-                        acc[j].y = fmaf(xv.y, wv.x, acc[j].y);
-                        acc[j].y = fmaf(xv.x, wv.y, acc[j].y);
+                for (int u = 0; u < kSpecWB; ++u)
+                    wv[u] = (i0 + u < Cin) ? Wm[(int64_t)(i0 + u) * Cout + o] : make_float2(0.f, 0.f);
+#pragma unroll
+                for (int u = 0; u < kSpecWB; ++u) {
+                    const int i = min(i0 + u, Cin - 1);  // rows past Cin carry zero weights
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const int n = ng + 4 * j;
+                        if (n < nb) {
+                            const float2 xv = xs[n * Cin + i];
+                            acc[j].x = fmaf(xv.x, wv[u].x, acc[j].x);
+                            acc[j].x = fmaf(-xv.y, wv[u].y, acc[j].x);
+                            acc[j].y = fmaf(xv.y, wv[u].x, acc[j].y);
+                            acc[j].y = fmaf(xv.x, wv[u].y, acc[j].y);
+                        }
                     }
                 }
             }

@@ -156,6 +156,36 @@ def _bilinear_align_corners_nhwc(X: Tensor, size) -> Tensor:
     return out
 
 
+def _truncated_dft_rows_supported(r: int, channels: int, modes: int) -> bool:
+    return bool(_lib.load().spgt_truncated_dft_rows_supported(int(r), int(channels), int(modes)))
+
+
+def _truncated_dft_rows(src: Tensor, table: Tensor, inverse: bool) -> Tensor:
+    """forward: src [..., r, C] x table [r, 2m] -> [..., C, 2m];  inverse: src [..., C, 2m] -> [..., r, C]."""
+    require_gpu_f32("src", src)
+    require_gpu_f32("table", table)
+    r, m2 = table.shape
+    if inverse:
+        C = src.shape[-2]
+        if src.shape[-1] != m2:
+            raise ValueError(f"src has last dimension {src.shape[-1]}, the table has {m2} columns")
+        lead = tuple(src.shape[:-2])
+        out = torch.empty(lead + (r, C), dtype=src.dtype, device=src.device)
+    else:
+        C = src.shape[-1]
+        if src.shape[-2] != r:
+            raise ValueError(f"src has {src.shape[-2]} grid points per row, the table has {r} rows")
+        lead = tuple(src.shape[:-2])
+        out = torch.empty(lead + (C, m2), dtype=src.dtype, device=src.device)
+    rows = prod(lead)
+    if rows == 0:
+        return out
+    fn = _lib.load().spgt_truncated_dft_rows_inverse if inverse else _lib.load().spgt_truncated_dft_rows_forward
+    with torch.cuda.device(src.device):
+        check(fn(ptr(src), ptr(table), ptr(out), rows, r, C, m2 // 2, stream_of(src)))
+    return out
+
+
 _ACT = {None: 0, "none": 0, "relu": 1, "silu": 2}
 
 
@@ -215,6 +245,8 @@ def _bias_activation_nchw_(X: Tensor, bias, activation=None, count: int = 1) -> 
 
 
 dexts = SimpleNamespace(
+    truncated_dft_rows_supported=_truncated_dft_rows_supported,
+    truncated_dft_rows=_truncated_dft_rows,
     bias_activation_nchw_=_bias_activation_nchw_,
     bilinear_resample=_bilinear_resample,
     bilinear_align_corners_nhwc=_bilinear_align_corners_nhwc,
@@ -317,3 +349,18 @@ def bilinear_resample(X: Tensor, size, src_nhwc: bool = False, dst_nhwc: bool = 
 def bias_activation_nchw_(X: Tensor, bias, activation=None, count: int = 1) -> Tensor:
     """In place: X = activation^count(X + bias[c]) on [N, C, ...] (inference only)."""
     return dexts.bias_activation_nchw_(X, None if bias is None else bias.detach(), activation, count)
+
+
+def truncated_dft_rows_supported(r: int, channels: int, modes: int) -> bool:
+    """True when truncated_dft_rows_forward / _inverse have a kernel for this shape."""
+    return dexts.truncated_dft_rows_supported(r, channels, modes)
+
+
+def truncated_dft_rows_forward(X: Tensor, table: Tensor) -> Tensor:
+    """Y[..., c, j] = sum_w X[..., w, c] table[w, j]: X [..., r, C], table [r, 2m] -> [..., C, 2m] (inference only)."""
+    return dexts.truncated_dft_rows(X.detach(), table, False)
+
+
+def truncated_dft_rows_inverse(U: Tensor, table: Tensor) -> Tensor:
+    """y[..., w, o] = sum_j table[w, j] U[..., o, j]: U [..., C, 2m], table [r, 2m] -> [..., r, C] (inference only)."""
+    return dexts.truncated_dft_rows(U.detach(), table, True)

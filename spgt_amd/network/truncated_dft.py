@@ -14,8 +14,9 @@ gives the same result as the FFT route up to fp32 rounding (the real part in the
 complex-to-real transform of irfft2 computes from a half spectrum), works directly on the [N, r, r, C]
 layout of the module - both full-tensor transposes, the full-size spectra, the corner gather/scatter and
 the zero fill disappear - and does not depend on r having small prime factors (r = 211 is prime).
-The four products are library GEMMs; the per-mode channel contraction between them is the HIP kernel
-behind `spectral_modes_compact`.
+The two products along w, which touch the full tensor, are the HIP kernels behind `truncated_dft_rows_*`;
+the two small ones along h are library GEMMs; the per-mode channel contraction between them is the HIP
+kernel behind `spectral_modes_compact`.
 """
 import math
 from typing import Dict, Tuple
@@ -23,7 +24,8 @@ from typing import Dict, Tuple
 import torch
 from torch import Tensor
 
-from ..extension.bind.datamove import spectral_modes_compact
+from ..extension.bind.datamove import (spectral_modes_compact, truncated_dft_rows_forward, truncated_dft_rows_inverse,
+                                       truncated_dft_rows_supported)
 
 _TABLES: Dict[Tuple[int, int, str], Tuple[Tensor, Tensor, Tensor, Tensor]] = {}
 
@@ -63,10 +65,16 @@ def spectral_modes_apply(x: Tensor, weight_1: Tensor, weight_2: Tensor, m: int) 
     N, r, _, cin = x.shape
     cout = weight_1.shape[3]
     fw, gh, ghi, fwi = dft_tables(r, m, x.device)
-    y = torch.matmul(x.reshape(N * r, r, cin).transpose(1, 2), fw)                       # [N r, Cin, 2m]
+    rows_kernel = truncated_dft_rows_supported(r, cin, m) and truncated_dft_rows_supported(r, cout, m)
+    if rows_kernel:
+        y = truncated_dft_rows_forward(x.reshape(N * r, r, cin), fw)                     # [N r, Cin, 2m]
+    else:
+        y = torch.matmul(x.reshape(N * r, r, cin).transpose(1, 2), fw)
     yc = torch.view_as_complex(y.view(N, r, cin, m, 2)).reshape(N, r, cin * m)
     z = torch.matmul(gh, yc).view(N, 2 * m, cin, m)                                      # [N, 2m, Cin, m]
     o = spectral_modes_compact(z, weight_1, weight_2)                                    # [N, 2m, Cout, m]
     u = torch.matmul(ghi, o.view(N, 2 * m, cout * m))                                    # [N, r, Cout m]
     ur = torch.view_as_real(u).view(N * r, cout, 2 * m)
+    if rows_kernel:
+        return truncated_dft_rows_inverse(ur, fwi).view(N, r, r, cout)
     return torch.matmul(fwi, ur.transpose(1, 2)).view(N, r, r, cout)

@@ -279,3 +279,34 @@ def test_bilinear_resample_pre_bias(gpu, src_nhwc, dst_nhwc):
     if dst_nhwc:
         got = got.permute(0, 3, 1, 2)
     assert (got - want).abs().max().item() <= 1e-5 * max(1.0, want.abs().max().item())
+
+
+@pytest.mark.parametrize("rows,r,C,m", [(3, 211, 64, 12), (5, 16, 32, 8), (2, 33, 96, 16), (1, 7, 32, 3), (844, 211, 64, 12)])
+def test_truncated_dft_rows_against_float64(gpu, rows, r, C, m):
+    """Both row kernels against float64 matrix products with the same tables, and the forward one against
+    torch.fft.rfft on the CPU (network/sp_layer.py:136-141 keeps columns kw < m of the ortho-normalised rfft2)."""
+    from spgt_amd.network.truncated_dft import dft_tables
+    fw, _, _, fwi = dft_tables(max(r, 2 * m), m, "cpu") if r >= 2 * m else dft_tables(r, m, "cpu")
+    fw, fwi = fw[:r].contiguous(), fwi[:r].contiguous()
+    x = rnd(rows, r, C, seed=71)
+    got = dm.truncated_dft_rows_forward(x.to(gpu), fw.to(gpu)).cpu().double()
+    want = torch.matmul(x.double().transpose(1, 2), fw.double())
+    assert got.shape == (rows, C, 2 * m)
+    assert (got - want).abs().max().item() <= 1e-5 * max(1.0, want.abs().max().item())
+    if r >= 2 * m:
+        ft = torch.fft.rfft(x.double(), dim=1, norm="ortho")[:, :m]          # [rows, m, C]
+        ref = torch.view_as_real(ft.permute(0, 2, 1).contiguous()).reshape(rows, C, 2 * m)
+        assert (got - ref).abs().max().item() <= 1e-5 * max(1.0, ref.abs().max().item())
+    u = rnd(rows, C, 2 * m, seed=72)
+    got = dm.truncated_dft_rows_inverse(u.to(gpu), fwi.to(gpu)).cpu().double()
+    want = torch.matmul(fwi.double(), u.double().transpose(1, 2))
+    assert got.shape == (rows, r, C)
+    assert (got - want).abs().max().item() <= 1e-5 * max(1.0, want.abs().max().item())
+
+
+def test_truncated_dft_rows_rejects(gpu):
+    from spgt_amd._lib import SpgtError
+    assert not dm.truncated_dft_rows_supported(211, 48, 12)
+    assert not dm.truncated_dft_rows_supported(211, 64, 17)
+    with pytest.raises(SpgtError):
+        dm.truncated_dft_rows_forward(rnd(2, 9, 48, seed=1).to(gpu), rnd(9, 8, seed=2).to(gpu))
