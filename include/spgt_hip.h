@@ -253,14 +253,19 @@ int spgt_linear_supported(int in_features, int out_features);
  * weight_kn is the transpose of nn.Linear.weight, contiguous.  x, residual and out are
  * row-major with row strides ldx, ldr, ldo (in floats, multiples of 4, 16-byte aligned
  * bases); bias may be null; residual may alias out, x may not.
+ * x_extra [tokens, extra_features] (row stride ldx_extra) with weight_extra_kn [extra_features,
+ * out_features] adds up to four more input columns, y += x_extra @ weight_extra_kn: the grid
+ * coordinates that Sp_DecoderRegressor concatenates to its input (network/sp_model.py:59-60).
  * The output columns may be split into planes of out_plane_cols columns (a multiple of 32
  * that divides out_features; 0 = one plane): column n of token t is written to
  * out[(n / out_plane_cols) * out_plane_stride + t * ldo + n % out_plane_cols], which lets one
  * call with the packed [W_Q | W_K | W_V] produce three contiguous projections. */
 int spgt_linear_forward(const float* x, int64_t ldx, const float* weight_kn, const float* bias,
-                        const float* residual, int64_t ldr, int residual_mode, int activation, float* out,
-                        int64_t ldo, int out_plane_cols, int64_t out_plane_stride, int64_t tokens,
-                        int in_features, int out_features, spgt_stream_t stream);
+                        const float* residual, int64_t ldr, int residual_mode, int activation,
+                        const float* x_extra, int64_t ldx_extra, const float* weight_extra_kn,
+                        int extra_features, float* out, int64_t ldo, int out_plane_cols,
+                        int64_t out_plane_stride, int64_t tokens, int in_features, int out_features,
+                        spgt_stream_t stream);
 
 /* 1 when spgt_ffn_scalar_forward has a kernel for this shape (in_features 64 or 128,
  * hidden_features 128 or 256), else 0. */

@@ -51,7 +51,8 @@ SIGNATURES = {
     "spgt_truncated_dft_rows_forward": (_i, [_p, _p, _p, _i64, _i, _i, _i, _p]),
     "spgt_truncated_dft_rows_inverse": (_i, [_p, _p, _p, _i64, _i, _i, _i, _p]),
     "spgt_linear_supported": (_i, [_i, _i]),
-    "spgt_linear_forward": (_i, [_p, _i64, _p, _p, _p, _i64, _i, _i, _p, _i64, _i, _i64, _i64, _i, _i, _p]),
+    "spgt_linear_forward": (_i, [_p, _i64, _p, _p, _p, _i64, _i, _i, _p, _i64, _p, _i, _p, _i64, _i, _i64, _i64, _i, _i,
+                                 _p]),
     "spgt_ffn_scalar_supported": (_i, [_i, _i]),
     "spgt_ffn_scalar_forward": (_i, [_p, _i64, _p, _p, _p, _p, _i, _p, _i64, _i, _i, _p]),
     "spgt_galerkin_attention_fused_profile": (

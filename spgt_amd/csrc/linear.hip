@@ -39,6 +39,7 @@ template <int K, int NCB>
 __global__ __launch_bounds__(256) void linear_tm_k(
     const float* __restrict__ x, int64_t ldx, const float* __restrict__ W, int ldw,
     const float* __restrict__ bias, const float* res, int64_t ldr, int res_mode, int act,
+    const float* __restrict__ x2, int64_t ldx2, const float* __restrict__ W2, int r2,
     float* out, int64_t ldo, int plane_cols, int64_t plane_stride, int64_t T, int tiles_per_wg) {
     constexpr int KH = K / 2;
     constexpr int PITCH = K + 1;
@@ -113,6 +114,11 @@ __global__ __launch_bounds__(256) void linear_tm_k(
         for (int q = 0; q < 4; ++q)
             rq[q] = (res_mode && t < t_end) ? *reinterpret_cast<const float4*>(res + t * ldr + n0 + 4 * kh + 8 * q)
                                             : make_float4(0.f, 0.f, 0.f, 0.f);
+        // the few extra input columns (r2 <= 4) are a rank-r2 update of the tile, done on the vector ALU
+        float x2v[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int p = 0; p < 4; ++p)
+            if (p < r2 && t < t_end) x2v[p] = x2[t * ldx2 + p];
         v16f acc;
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[r] = 0.f;
@@ -137,6 +143,11 @@ __global__ __launch_bounds__(256) void linear_tm_k(
                 y.y = acc[4 * q + 1] + breg[4 * q + 1];
                 y.z = acc[4 * q + 2] + breg[4 * q + 2];
                 y.w = acc[4 * q + 3] + breg[4 * q + 3];
+                for (int p = 0; p < r2; ++p) {
+                    const float4 w4 = *reinterpret_cast<const float4*>(W2 + (int64_t)p * ldw + n0 + 4 * kh + 8 * q);
+                    y.x = fmaf(x2v[p], w4.x, y.x); y.y = fmaf(x2v[p], w4.y, y.y);
+                    y.z = fmaf(x2v[p], w4.z, y.z); y.w = fmaf(x2v[p], w4.w, y.w);
+                }
                 if (res_mode == SPGT_RES_BEFORE_ACT) { y.x += r4.x; y.y += r4.y; y.z += r4.z; y.w += r4.w; }
                 y.x = activate(y.x, act); y.y = activate(y.y, act);
                 y.z = activate(y.z, act); y.w = activate(y.w, act);
@@ -289,8 +300,8 @@ inline int pick_tiles_per_wg(int64_t tiles, int gy, int cus) {
 
 template <int K, int NCB>
 void launch_linear(const float* x, int64_t ldx, const float* W, const float* bias, const float* res, int64_t ldr,
-                   int res_mode, int act, float* out, int64_t ldo, int plane_cols, int64_t plane_stride, int64_t T,
-                   int N, hipStream_t stream) {
+                   int res_mode, int act, const float* x2, int64_t ldx2, const float* W2, int r2, float* out,
+                   int64_t ldo, int plane_cols, int64_t plane_stride, int64_t T, int N, hipStream_t stream) {
     constexpr int TT = 32 * (4 / NCB);
     const size_t lds = (size_t)TT * (K + 1) * sizeof(float);
     const int gy = N / (32 * NCB);
@@ -301,15 +312,16 @@ void launch_linear(const float* x, int64_t ldx, const float* W, const float* bia
     if (lds > 64 * 1024)
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                   (int)lds);
-    hipLaunchKernelGGL(kernel, grid, dim3(256), lds, stream, x, ldx, W, N, bias, res, ldr, res_mode, act, out, ldo,
-                       plane_cols, plane_stride, T, tpw);
+    hipLaunchKernelGGL(kernel, grid, dim3(256), lds, stream, x, ldx, W, N, bias, res, ldr, res_mode, act, x2, ldx2, W2,
+                       r2, out, ldo, plane_cols, plane_stride, T, tpw);
 }
 
 template <int K>
 void launch_linear_k(int ncb, const float* x, int64_t ldx, const float* W, const float* bias, const float* res,
-                     int64_t ldr, int res_mode, int act, float* out, int64_t ldo, int plane_cols, int64_t plane_stride,
-                     int64_t T, int N, hipStream_t stream) {
-#define SPGT_ARGS x, ldx, W, bias, res, ldr, res_mode, act, out, ldo, plane_cols, plane_stride, T, N, stream
+                     int64_t ldr, int res_mode, int act, const float* x2, int64_t ldx2, const float* W2, int r2,
+                     float* out, int64_t ldo, int plane_cols, int64_t plane_stride, int64_t T, int N,
+                     hipStream_t stream) {
+#define SPGT_ARGS x, ldx, W, bias, res, ldr, res_mode, act, x2, ldx2, W2, r2, out, ldo, plane_cols, plane_stride, T, N, stream
     if (ncb == 4) launch_linear<K, 4>(SPGT_ARGS);
     else if (ncb == 2) launch_linear<K, 2>(SPGT_ARGS);
     else launch_linear<K, 1>(SPGT_ARGS);
@@ -337,9 +349,11 @@ extern "C" int spgt_linear_supported(int in_features, int out_features) {
 }
 
 extern "C" int spgt_linear_forward(const float* x, int64_t ldx, const float* weight_kn, const float* bias,
-                                   const float* residual, int64_t ldr, int residual_mode, int activation, float* out,
-                                   int64_t ldo, int out_plane_cols, int64_t out_plane_stride, int64_t tokens,
-                                   int in_features, int out_features, hipStream_t stream) {
+                                   const float* residual, int64_t ldr, int residual_mode, int activation,
+                                   const float* x_extra, int64_t ldx_extra, const float* weight_extra_kn,
+                                   int extra_features, float* out, int64_t ldo, int out_plane_cols,
+                                   int64_t out_plane_stride, int64_t tokens, int in_features, int out_features,
+                                   hipStream_t stream) {
     if (!x || !weight_kn || !out) return fail(SPGT_ERR_INVALID_ARGUMENT, "linear_forward: null pointer argument");
     if (tokens < 0) return fail(SPGT_ERR_INVALID_ARGUMENT, "linear_forward: negative token count");
     if (!spgt_linear_supported(in_features, out_features))
@@ -351,6 +365,12 @@ extern "C" int spgt_linear_forward(const float* x, int64_t ldx, const float* wei
         return fail(SPGT_ERR_INVALID_ARGUMENT, "linear_forward: unknown residual_mode");
     if (residual_mode != SPGT_RES_NONE && !residual)
         return fail(SPGT_ERR_INVALID_ARGUMENT, "linear_forward: residual is null with a residual_mode");
+    if (extra_features < 0 || extra_features > 4)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "linear_forward: extra_features must be 0..4");
+    if (extra_features > 0 && (!x_extra || !weight_extra_kn || ldx_extra < extra_features || !aligned4(x_extra) ||
+                               !aligned16(weight_extra_kn)))
+        return fail(SPGT_ERR_INVALID_ARGUMENT,
+                    "linear_forward: x_extra / weight_extra_kn missing, misaligned or with too small a row stride");
     if (out_plane_cols <= 0 || out_plane_cols > out_features) out_plane_cols = out_features;
     if (out_plane_cols % 32 != 0 || out_features % out_plane_cols != 0)
         return fail(SPGT_ERR_INVALID_ARGUMENT,
@@ -367,8 +387,9 @@ extern "C" int spgt_linear_forward(const float* x, int64_t ldx, const float* wei
     const int ncb = out_features % 128 == 0 ? 4 : (out_features % 64 == 0 ? 2 : 1);
     const float* res = residual_mode ? residual : nullptr;
 #define SPGT_LIN(KV) \
-    launch_linear_k<KV>(ncb, x, ldx, weight_kn, bias, res, ldr, residual_mode, activation, out, ldo, out_plane_cols, \
-                        out_plane_stride, tokens, out_features, stream)
+    launch_linear_k<KV>(ncb, x, ldx, weight_kn, bias, res, ldr, residual_mode, activation, x_extra, ldx_extra,      \
+                        weight_extra_kn, extra_features, out, ldo, out_plane_cols, out_plane_stride, tokens,        \
+                        out_features, stream)
     switch (in_features) {
         case 64: SPGT_LIN(64); break;
         case 128: SPGT_LIN(128); break;

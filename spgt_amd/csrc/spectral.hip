@@ -127,7 +127,11 @@ __device__ __forceinline__ float act_apply(float v, int act) {
     return v;
 }
 
-__device__ __forceinline__ float act_pre(float v, ResampleAct a) {
+// PRE = false compiles the bias and source activations out: the plain resampling stays as cheap as before.
+template <bool PRE>
+__device__ __forceinline__ float act_pre(float v, float bias, ResampleAct a) {
+    if (!PRE) return v;
+    v += bias;
     for (int i = 0; i < a.pre_n; ++i) v = act_apply(v, a.pre);
     return v;
 }
@@ -136,6 +140,7 @@ __device__ __forceinline__ float act_pre(float v, ResampleAct a) {
 // Same arithmetic as torch's upsample_bilinear2d: scale = (in-1)/(out-1) in fp32
 // (0 when out == 1), source coordinate scale*dst, weights (1-l, l), rows blended last.
 // grid (ceil(Wout/64), ceil(Hout/4), planes), block (64, 4).
+template <bool PRE>
 __global__ __launch_bounds__(256) void bilinear_align_corners_k(const float* __restrict__ src,
                                                                 const float* __restrict__ pre_bias, int C,
                                                                 float* __restrict__ dst, int planes, int Hin,
@@ -157,9 +162,9 @@ __global__ __launch_bounds__(256) void bilinear_align_corners_k(const float* __r
     for (int64_t pl = blockIdx.z; pl < planes; pl += gridDim.z) {
         const float* r0 = src + pl * Hin * Win + (int64_t)h1 * Win + w1;
         const float* r1 = r0 + (int64_t)hp * Win;
-        const float pb = pre_bias ? pre_bias[pl % C] : 0.f;
-        const float top = w0l * act_pre(r0[0] + pb, act) + w1l * act_pre(r0[wp] + pb, act);
-        const float bot = w0l * act_pre(r1[0] + pb, act) + w1l * act_pre(r1[wp] + pb, act);
+        const float pb = (PRE && pre_bias) ? pre_bias[pl % C] : 0.f;
+        const float top = w0l * act_pre<PRE>(r0[0], pb, act) + w1l * act_pre<PRE>(r0[wp], pb, act);
+        const float bot = w0l * act_pre<PRE>(r1[0], pb, act) + w1l * act_pre<PRE>(r1[wp], pb, act);
         dst[(pl * Hout + oy) * Wout + ox] = act_apply(h0l * top + h1l * bot, act.post);
     }
 }
@@ -167,6 +172,7 @@ __global__ __launch_bounds__(256) void bilinear_align_corners_k(const float* __r
 // The same resampling with a channels-last result: src [N, C, Hin, Win] -> dst [N, Hout, Wout, C].
 // grid (ceil(Wout/32), Hout, N), block 256 = 32 output columns x 8 channel lanes.  Reads run along the
 // source rows of one channel, a 32 x 32 (channel x column) tile is turned in LDS, writes run along C.
+template <bool PRE>
 __global__ __launch_bounds__(256) void bilinear_align_corners_nhwc_k(const float* __restrict__ src,
                                                                      const float* __restrict__ pre_bias,
                                                                      float* __restrict__ dst, int C, int Hin,
@@ -200,9 +206,9 @@ __global__ __launch_bounds__(256) void bilinear_align_corners_nhwc_k(const float
             if (c0 + cl < C) {
                 const float* r0 = base + (int64_t)(c0 + cl) * plane;
                 const float* r1 = r0 + (int64_t)hp * Win;
-                const float pb = pre_bias ? pre_bias[c0 + cl] : 0.f;
-                const float top = w0l * act_pre(r0[0] + pb, act) + w1l * act_pre(r0[wp] + pb, act);
-                const float bot = w0l * act_pre(r1[0] + pb, act) + w1l * act_pre(r1[wp] + pb, act);
+                const float pb = (PRE && pre_bias) ? pre_bias[c0 + cl] : 0.f;
+                const float top = w0l * act_pre<PRE>(r0[0], pb, act) + w1l * act_pre<PRE>(r0[wp], pb, act);
+                const float bot = w0l * act_pre<PRE>(r1[0], pb, act) + w1l * act_pre<PRE>(r1[wp], pb, act);
                 v = act_apply(h0l * top + h1l * bot, act.post);
             }
             tile[cl * 33 + tx] = v;
@@ -222,6 +228,7 @@ __global__ __launch_bounds__(256) void bilinear_align_corners_nhwc_k(const float
 // grid (ceil(Wout/32), Hout, N), block 256 = 32 channels x 8 column lanes.  Reads run along C (the
 // four source pixels of an output column are 128-byte runs), a 32 x 32 (column x channel) tile is
 // turned in LDS, writes run along the output row of one channel.
+template <bool PRE>
 __global__ __launch_bounds__(256) void bilinear_align_corners_from_nhwc_k(const float* __restrict__ src,
                                                                           const float* __restrict__ pre_bias,
                                                                           float* __restrict__ dst, int C, int Hin,
@@ -253,9 +260,9 @@ __global__ __launch_bounds__(256) void bilinear_align_corners_from_nhwc_k(const 
             if (c0 + tx < C) {
                 const float* p0 = rows + (int64_t)w1 * C + c0 + tx;
                 const float* p1 = p0 + rstep;
-                const float pb = pre_bias ? pre_bias[c0 + tx] : 0.f;
-                const float top = w0l * act_pre(p0[0] + pb, act) + w1l * act_pre(p0[wp * C] + pb, act);
-                const float bot = w0l * act_pre(p1[0] + pb, act) + w1l * act_pre(p1[wp * C] + pb, act);
+                const float pb = (PRE && pre_bias) ? pre_bias[c0 + tx] : 0.f;
+                const float top = w0l * act_pre<PRE>(p0[0], pb, act) + w1l * act_pre<PRE>(p0[wp * C], pb, act);
+                const float bot = w0l * act_pre<PRE>(p1[0], pb, act) + w1l * act_pre<PRE>(p1[wp * C], pb, act);
                 v = act_apply(h0l * top + h1l * bot, act.post);
             }
             tile[xl * 33 + tx] = v;
@@ -362,24 +369,28 @@ int resample_common(const char* who, const float* src, const float* pre_bias, fl
                     "bilinear resampling: unknown activation, or more than two source activations");
     const float hscale = H_out > 1 ? (float)(H_in - 1) / (float)(H_out - 1) : 0.f;
     const float wscale = W_out > 1 ? (float)(W_in - 1) / (float)(W_out - 1) : 0.f;
+    if (act.pre == SPGT_ACT_NONE) act.pre_n = 0;
+    const bool pre = pre_bias != nullptr || act.pre_n > 0;
     if (src_layout == SPGT_LAYOUT_NCHW && dst_layout == SPGT_LAYOUT_NCHW) {
         const int64_t planes = (int64_t)N * C;
         if (ceil_div(H_out, 4) > 65535 || planes > INT32_MAX)
             return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear resampling: H_out/4 exceeds 65535 or too many planes");
         const dim3 grid(ceil_div(W_out, 64), ceil_div(H_out, 4), (unsigned)std::min<int64_t>(planes, 65535));
-        hipLaunchKernelGGL(bilinear_align_corners_k, grid, dim3(64, 4), 0, stream, src, pre_bias, C, dst, (int)planes, H_in,
-                           W_in, H_out, W_out, hscale, wscale, act);
+        hipLaunchKernelGGL(pre ? bilinear_align_corners_k<true> : bilinear_align_corners_k<false>, grid, dim3(64, 4), 0,
+                           stream, src, pre_bias, C, dst, (int)planes, H_in, W_in, H_out, W_out, hscale, wscale, act);
     } else if (src_layout != dst_layout && (src_layout == SPGT_LAYOUT_NCHW || src_layout == SPGT_LAYOUT_NHWC) &&
                (dst_layout == SPGT_LAYOUT_NCHW || dst_layout == SPGT_LAYOUT_NHWC)) {
         if (H_out > 65535 || N > 65535)
             return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear resampling: N or H_out exceeds 65535");
         const dim3 grid(ceil_div(W_out, 32), H_out, N);
         if (dst_layout == SPGT_LAYOUT_NHWC)
-            hipLaunchKernelGGL(bilinear_align_corners_nhwc_k, grid, dim3(256), 0, stream, src, pre_bias, dst, C, H_in,
-                               W_in, H_out, W_out, hscale, wscale, act);
+            hipLaunchKernelGGL(pre ? bilinear_align_corners_nhwc_k<true> : bilinear_align_corners_nhwc_k<false>, grid,
+                               dim3(256), 0, stream, src, pre_bias, dst, C, H_in, W_in, H_out, W_out, hscale, wscale,
+                               act);
         else
-            hipLaunchKernelGGL(bilinear_align_corners_from_nhwc_k, grid, dim3(256), 0, stream, src, pre_bias, dst, C,
-                               H_in, W_in, H_out, W_out, hscale, wscale, act);
+            hipLaunchKernelGGL(pre ? bilinear_align_corners_from_nhwc_k<true> : bilinear_align_corners_from_nhwc_k<false>,
+                               grid, dim3(256), 0, stream, src, pre_bias, dst, C, H_in, W_in, H_out, W_out, hscale,
+                               wscale, act);
     } else {
         return fail(SPGT_ERR_INVALID_ARGUMENT,
                     "bilinear resampling: layouts must be NCHW->NCHW, NCHW->NHWC or NHWC->NCHW");

@@ -21,23 +21,35 @@
 
 namespace spgt {
 
-// grid (ceil(rows * C/32 / 4)), block 256.  tab [r][m2] row-major, m2 <= 32.
+// grid (workgroups), block 256; waves stride over the rows * C/32 (row, channel block) items.
+// tab [r][m2] row-major, m2 <= 32.
 // Y [rows][C][m2].
 __global__ __launch_bounds__(256) void dft_rows_forward_k(const float* __restrict__ x, const float* __restrict__ tab,
                                                           float* __restrict__ Y, int64_t rows, int r, int C, int m2) {
     extern __shared__ float ts[];  // [2*KH][32], zero beyond r rows and m2 columns
     const int KH = (r + 1) / 2;
-    for (int e = threadIdx.x; e < 2 * KH * 32; e += 256) {
-        const int w = e >> 5, j = e & 31;
-        ts[e] = (w < r && j < m2) ? tab[w * m2 + j] : 0.f;
+    {
+        // table fill with eight loads in flight per thread
+        const int total = 2 * KH * 32;
+        for (int e0 = threadIdx.x; e0 < total; e0 += 256 * 8) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int e = e0 + 256 * u;
+                const int w = e >> 5, j = e & 31;
+                v[u] = (e < total && w < r && j < m2) ? tab[w * m2 + j] : 0.f;
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (e0 + 256 * u < total) ts[e0 + 256 * u] = v[u];
+        }
     }
     __syncthreads();
     const int lane = threadIdx.x & 63;
     const int tk = lane & 31;
     const int kh = lane >> 5;
     const int CB = C / 32;
-    const int64_t gw = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (gw >= rows * CB) return;
+    for (int64_t gw = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6); gw < rows * CB; gw += (int64_t)gridDim.x * 4) {
     const int64_t row = gw / CB;
     const int cb = (int)(gw % CB);
     const float* xr = x + row * (int64_t)r * C + cb * 32 + tk;
@@ -98,26 +110,39 @@ __global__ __launch_bounds__(256) void dft_rows_forward_k(const float* __restric
             const int j = 8 * q + 4 * kh + e;
             if (j < m2) yr[j] = acc[4 * q + e];
         }
+    }
 }
 
-// grid (ceil(rows * C/32 / 4)), block 256.  tab [r][m2] row-major, m2 <= 32 and even.
+// grid (workgroups), block 256; waves stride over the (row, channel block) items.
+// tab [r][m2] row-major, m2 <= 32 and even.
 // U [rows][C][m2] -> y [rows][r][C].
 __global__ __launch_bounds__(256) void dft_rows_inverse_k(const float* __restrict__ U, const float* __restrict__ tab,
                                                           float* __restrict__ y, int64_t rows, int r, int C, int m2) {
     extern __shared__ float ts[];  // [32 * ceil(r/32)][m2 + 1], zero beyond r rows
     const int pitch = m2 + 1;
     const int WT = (r + 31) / 32;
-    for (int e = threadIdx.x; e < WT * 32 * m2; e += 256) {
-        const int w = e / m2, j = e - w * m2;
-        ts[w * pitch + j] = (w < r) ? tab[e] : 0.f;
+    {
+        const int total = WT * 32 * m2;
+        for (int e0 = threadIdx.x; e0 < total; e0 += 256 * 8) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int e = e0 + 256 * u;
+                v[u] = (e < r * m2) ? tab[e] : 0.f;
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int e = e0 + 256 * u;
+                if (e < total) ts[(e / m2) * pitch + e % m2] = v[u];
+            }
+        }
     }
     __syncthreads();
     const int lane = threadIdx.x & 63;
     const int tk = lane & 31;
     const int kh = lane >> 5;
     const int CB = C / 32;
-    const int64_t gw = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (gw >= rows * CB) return;
+    for (int64_t gw = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6); gw < rows * CB; gw += (int64_t)gridDim.x * 4) {
     const int64_t row = gw / CB;
     const int cb = (int)(gw % CB);
     // B operand: U[o = cb*32 + tk][j = 2kk + kh]
@@ -141,6 +166,7 @@ __global__ __launch_bounds__(256) void dft_rows_inverse_k(const float* __restric
             const int w = wt * 32 + 8 * (q >> 2) + 4 * kh + (q & 3);
             if (w < r) yr[(int64_t)w * C] = acc[q];
         }
+    }
     }
 }
 
@@ -181,7 +207,8 @@ extern "C" int spgt_truncated_dft_rows_forward(const float* x, const float* tabl
     if (lds > 64 * 1024)
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                   (int)lds);
-    const unsigned grid = (unsigned)ceil_div(rows * (channels / 32), (int64_t)4);
+    // workgroups loop over (row, channel block) items: about two per CU, so the table is staged few times
+    const unsigned grid = (unsigned)std::min<int64_t>(ceil_div(rows * (channels / 32), (int64_t)4), 2 * device_cu_count());
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), lds, stream, x, table, Y, rows, r, channels, m2);
     return check_launch("truncated_dft_rows_forward");
 }
@@ -195,7 +222,7 @@ extern "C" int spgt_truncated_dft_rows_inverse(const float* U, const float* tabl
     if (lds > 64 * 1024)
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                   (int)lds);
-    const unsigned grid = (unsigned)ceil_div(rows * (channels / 32), (int64_t)4);
+    const unsigned grid = (unsigned)std::min<int64_t>(ceil_div(rows * (channels / 32), (int64_t)4), 2 * device_cu_count());
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), lds, stream, U, table, y, rows, r, channels, m2);
     return check_launch("truncated_dft_rows_inverse");
 }

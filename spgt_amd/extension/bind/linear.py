@@ -36,11 +36,14 @@ def _rows(name: str, t: Tensor, width: int):
 
 def fused_linear(x: Tensor, weight_kn: Tensor, bias: Optional[Tensor] = None, activation: str = "none",
                  residual: Optional[Tensor] = None, residual_after_activation: bool = False,
-                 planes: int = 1) -> Tensor:
+                 planes: int = 1, x_extra: Optional[Tensor] = None,
+                 weight_extra_kn: Optional[Tensor] = None) -> Tensor:
     """act(x @ weight_kn + bias [+ residual]) or act(x @ weight_kn + bias) + residual.
 
     x [..., K] (a 2-D x may have a row stride larger than K), weight_kn [K, N] contiguous
     (the transpose of nn.Linear.weight), bias [N] or None, residual [..., N] or None.
+    x_extra [..., E] with weight_extra_kn [E, N] (E <= 4) adds x_extra @ weight_extra_kn before the residual and
+    the activation: a few more input columns without a concatenation.
     Returns a new contiguous [..., N] tensor, or with planes > 1 a [planes, ..., N / planes] tensor whose
     plane p holds output columns p*N/planes .. (p+1)*N/planes - 1.
     """
@@ -66,12 +69,22 @@ def fused_linear(x: Tensor, weight_kn: Tensor, bias: Optional[Tensor] = None, ac
         if Tr != T:
             raise ValueError("residual must have the shape of the output")
         mode = RES_AFTER_ACT if residual_after_activation else RES_BEFORE_ACT
+    xe, we, ne, ldxe = None, None, 0, 0
+    if x_extra is not None:
+        require_gpu_f32("weight_extra_kn", weight_extra_kn)
+        ne = weight_extra_kn.shape[0]
+        if weight_extra_kn.shape[1] != N or x_extra.shape[-1] != ne or x_extra.numel() != T * ne:
+            raise ValueError("x_extra must be [..., E] and weight_extra_kn [E, N]")
+        require_gpu_f32("x_extra", x_extra, contiguous=False)
+        xe, we, ldxe = x_extra.contiguous(), weight_extra_kn, ne
     if T == 0:
         return out
     with torch.cuda.device(x.device):
         check(_lib.load().spgt_linear_forward(
             ptr(xr), ldx, ptr(weight_kn), ptr(bias) if bias is not None else None,
-            ptr(rr) if rr is not None else None, ldr, mode, ACTIVATIONS[activation], ptr(out), pc, pc, T * pc, T, K, N,
+            ptr(rr) if rr is not None else None, ldr, mode, ACTIVATIONS[activation],
+            ptr(xe) if xe is not None else None, ldxe, ptr(we) if we is not None else None, ne, ptr(out), pc, pc,
+            T * pc, T, K, N,
             stream_of(x)))
     return out
 

@@ -56,25 +56,27 @@ class Sp_DecoderRegressor(nn.Module):
         self.ffn_layer = FeedForward(dim_spatial_hidden, out_dim, 2 * dim_position * dim_spatial_hidden, droprate,
                                      activation)
 
-    def _weight_x_kn(self, dim_x: int) -> Tensor:
-        """The hidden-feature columns of spatial_fc_layer.weight as [dim_x, C], rebuilt when the parameter changes."""
+    def _split_weight_kn(self, dim_x: int):
+        """spatial_fc_layer.weight as ([dim_x, C], [dim_position, C]): the hidden-feature and the grid columns,
+        transposed; rebuilt when the parameter changes."""
         w = self.spatial_fc_layer.weight
         key = (w.data_ptr(), w._version, w.device, dim_x)
-        cache = getattr(self, "_spgt_weight_x_kn", None)
+        cache = getattr(self, "_spgt_weight_split", None)
         if cache is None or cache[0] != key:
-            cache = (key, w.detach()[:, :dim_x].t().contiguous())
-            self._spgt_weight_x_kn = cache
-        return cache[1]
+            wd = w.detach()
+            cache = (key, wd[:, :dim_x].t().contiguous(), wd[:, dim_x:].t().contiguous())
+            self._spgt_weight_split = cache
+        return cache[1], cache[2]
 
     def forward(self, X: Tensor, grid: Tensor = None) -> Tensor:
         """X [N, r, r, dim_hidden], grid [N, r, r, dim_position] -> [N, r, r, dim_target]."""
         # Linear(cat([X, grid])) without materialising the concatenation: W = [W_x | W_grid]
         W, dim_x = self.spatial_fc_layer.weight, X.size(-1)
-        if gpu_inference(X, W, self.spatial_fc_layer.bias) and linear_supported(dim_x, W.size(0)):
-            # the grid columns first (a [T, dim_position] x [dim_position, C] product); the GEMM over the
-            # hidden features adds it in its epilogue
-            X = fused_linear(X, self._weight_x_kn(dim_x), self.spatial_fc_layer.bias, "none",
-                             F.linear(grid, W[:, dim_x:]))
+        if (gpu_inference(X, W, self.spatial_fc_layer.bias) and linear_supported(dim_x, W.size(0)) and
+                W.size(1) - dim_x <= 4):
+            # the GEMM runs over the hidden features; the grid columns are a rank-2 update in its epilogue
+            w_x, w_grid = self._split_weight_kn(dim_x)
+            X = fused_linear(X, w_x, self.spatial_fc_layer.bias, "none", x_extra=grid, weight_extra_kn=w_grid)
         else:
             X = F.linear(X, W[:, :dim_x], self.spatial_fc_layer.bias) + F.linear(grid, W[:, dim_x:])
         for layer in self.layers:

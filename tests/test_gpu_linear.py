@@ -86,6 +86,22 @@ def test_linear_output_planes(gpu):
         fused_linear(x.to(gpu), w.to(gpu), b.to(gpu), planes=5)
 
 
+@pytest.mark.parametrize("E", [1, 2, 4])
+def test_linear_extra_columns(gpu, E):
+    """x_extra @ weight_extra_kn added in the epilogue equals a Linear over the concatenated input
+    (network/sp_model.py:59-60 concatenates the grid coordinates)."""
+    from spgt_amd.extension.bind.linear import fused_linear
+    g = torch.Generator().manual_seed(21 + E)
+    x = torch.randn(3, 211, 128, generator=g)
+    xe = torch.randn(3, 211, E, generator=g)
+    w = torch.randn(128 + E, 64, generator=g) / 11.0
+    b = torch.randn(64, generator=g)
+    want = _expected(torch.cat([x, xe], -1), w, b, "silu", None, False)
+    got = fused_linear(x.to(gpu), w[:128].contiguous().to(gpu), b.to(gpu), "silu", x_extra=xe.to(gpu),
+                       weight_extra_kn=w[128:].contiguous().to(gpu)).cpu()
+    assert (got.double() - want).abs().max().item() <= 1e-5 * max(1.0, want.abs().max().item())
+
+
 def test_linear_matches_nn_linear(gpu):
     """Same result as torch's own Linear on the device, to fp32 rounding."""
     from spgt_amd.extension.bind.linear import fused_linear
