@@ -335,6 +335,43 @@ def kernel_rooflines(dev):
     hbm("bilinear_211_to_122", 4 * 4 * 128 * (211 * 211 + 122 * 122), lambda: dm.bilinear_align_corners(img, (122, 122)))
     small = rn(4, 128, 71, 71)
     hbm("bilinear_71_to_122", 4 * 4 * 128 * (71 * 71 + 122 * 122), lambda: dm.bilinear_align_corners(small, (122, 122)))
+    mid = rn(4, 128, 122, 122)
+    hbm("bilinear_122_to_211_nchw_to_nhwc", 4 * 4 * 128 * (211 * 211 + 122 * 122),
+        lambda: dm.bilinear_resample(mid, (211, 211), dst_nhwc=True))
+    cb = rn(128)
+    hbm("bilinear_211_to_122_bias_silu_silu", 4 * 4 * 128 * (211 * 211 + 122 * 122),
+        lambda: dm.bilinear_resample(img, (122, 122), pre_activation="silu", post_activation="silu", pre_bias=cb))
+    hbm("bias_activation_nchw_silu2", 2 * mid.numel() * 4, lambda: dm.bias_activation_nchw_(mid, cb, "silu", 2))
+    del img, small, mid
+    # fused linear layers at the encoder's and the decoder's token counts of the Darcy model
+    from spgt_amd.extension.bind import linear as ln
+    for T, tag in ((B * S, "356k"), (4 * 71 * 71, "20k")):
+        xt_ = rn(T, 128)
+        res = rn(T, 128)
+        mfma(f"linear_128_to_128_T{tag}", 2 * T * 128 * 128, lambda: ln.fused_linear(xt_, W, bias))
+        w3, b3 = rn(128, 384) / 11.3, rn(384)
+        mfma(f"linear_qkv_128_to_384_planes_T{tag}", 2 * T * 128 * 384, lambda: ln.fused_linear(xt_, w3, b3, planes=3))
+        w4, b4 = rn(128, 256) / 11.3, rn(256)
+        mfma(f"linear_128_to_256_silu_T{tag}", 2 * T * 128 * 256, lambda: ln.fused_linear(xt_, w4, b4, "silu"))
+        hdn = rn(T, 256)
+        w5 = rn(256, 128) / 16.0
+        mfma(f"linear_256_to_128_residual_T{tag}", 2 * T * 256 * 128, lambda: ln.fused_linear(hdn, w5, bias, "none", res))
+        del xt_, res, hdn
+    Tf = 4 * 211 * 211
+    xf_, yf_ = rn(Tf, 64), rn(Tf, 64)
+    w6, b6 = rn(64, 64) / 8.0, rn(64)
+    mfma("linear_64_to_64_residual_silu_T178k", 2 * Tf * 64 * 64, lambda: ln.fused_linear(xf_, w6, b6, "silu", yf_))
+    w7, b7, w8, b8 = rn(64, 256) / 8.0, rn(256), rn(1, 256) / 16.0, rn(1)
+    mfma("ffn_scalar_64_256_1_T178k", 2 * Tf * 64 * 256 + 2 * Tf * 256,
+         lambda: ln.fused_ffn_scalar(xf_, w7, b7, w8, b8, "silu"))
+    del yf_
+    # truncated DFT along w at the decoder's grid: rows = 4*211, r = 211, C = 64, 12 modes
+    from spgt_amd.network.truncated_dft import dft_tables
+    fw, _, _, fwi = dft_tables(211, 12, dev)
+    xr_ = xf_.view(4 * 211, 211, 64)
+    hbm("truncated_dft_rows_forward", (xr_.numel() + 4 * 211 * 64 * 24) * 4, lambda: dm.truncated_dft_rows_forward(xr_, fw))
+    ur_ = rn(4 * 211, 64, 24)
+    hbm("truncated_dft_rows_inverse", (xr_.numel() + 4 * 211 * 64 * 24) * 4, lambda: dm.truncated_dft_rows_inverse(ur_, fwi))
     return rows
 
 

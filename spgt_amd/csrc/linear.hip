@@ -32,7 +32,8 @@ __device__ __forceinline__ float activate(float v, int act) {
 
 }  // namespace
 
-// grid (workgroups, column groups), block 256.  NCB column blocks of 32 per
+// grid (token groups * column groups), block 256, the column group varying fastest so that the
+// workgroups that share an x tile run together and the tile comes from HBM once.  NCB column blocks of 32 per
 // workgroup; the 4/NCB waves that share a column block take different 32-token
 // sub-tiles of the workgroup's TT = 32*(4/NCB)-token tile.
 template <int K, int NCB>
@@ -40,7 +41,7 @@ __global__ __launch_bounds__(256) void linear_tm_k(
     const float* __restrict__ x, int64_t ldx, const float* __restrict__ W, int ldw,
     const float* __restrict__ bias, const float* res, int64_t ldr, int res_mode, int act,
     const float* __restrict__ x2, int64_t ldx2, const float* __restrict__ W2, int r2,
-    float* out, int64_t ldo, int plane_cols, int64_t plane_stride, int64_t T, int tiles_per_wg) {
+    float* out, int64_t ldo, int plane_cols, int64_t plane_stride, int64_t T, int tiles_per_wg, int gy) {
     constexpr int KH = K / 2;
     constexpr int PITCH = K + 1;
     constexpr int TT = 32 * (4 / NCB);
@@ -53,7 +54,9 @@ __global__ __launch_bounds__(256) void linear_tm_k(
     const int wave = threadIdx.x >> 6;
     const int tk = lane & 31;
     const int kh = lane >> 5;
-    const int n0 = (blockIdx.y * NCB + wave % NCB) * 32;
+    const int cg = blockIdx.x % gy;
+    const int tg = blockIdx.x / gy;
+    const int n0 = (cg * NCB + wave % NCB) * 32;
     const int sub = wave / NCB;
 
     // A operand: W[2kk + kh][n0 + tk]
@@ -65,7 +68,7 @@ __global__ __launch_bounds__(256) void linear_tm_k(
 #pragma unroll
     for (int r = 0; r < 16; ++r) breg[r] = bias ? bias[n0 + 8 * (r >> 2) + 4 * kh + (r & 3)] : 0.f;
 
-    const int64_t t_begin = (int64_t)blockIdx.x * tiles_per_wg * TT;
+    const int64_t t_begin = (int64_t)tg * tiles_per_wg * TT;
     const int64_t t_end = min(T, t_begin + (int64_t)tiles_per_wg * TT);
     float4 stage[NLD];
     auto load_tile = [&](int64_t t0) {
@@ -275,19 +278,21 @@ __global__ __launch_bounds__(256) void ffn_scalar_k(
 
 namespace {
 
-// Tiles per workgroup.  With every workgroup resident at once, the time is set by the
-// CU with the most work, ceil(workgroups / CUs) * tiles_per_wg tile-times; among the
-// choices with the least such work, two workgroups per CU hide each other's load
-// latency best (one has nothing to overlap with, more re-read W more often).
-inline int pick_tiles_per_wg(int64_t tiles, int gy, int cus) {
+// Tiles per workgroup.  A CU runs `occ` workgroups at a time; co-resident workgroups hide each
+// other's load latency and share the matrix pipe, so a round of k >= 2 of them costs k * tiles_per_wg
+// tile-times, while a workgroup that runs alone costs twice its tiles.  The CU with the most
+// workgroups sets the time; ties go to the choice closest to two workgroups per CU (fewer W reloads).
+inline int pick_tiles_per_wg(int64_t tiles, int gy, int cus, int occ) {
+    occ = std::max(1, occ);
     int best = 1;
     int64_t best_cost = INT64_MAX;
     double best_dist = 0;
     for (int tpw = 1; tpw <= 64; ++tpw) {
         const int64_t wgs = ceil_div(tiles, (int64_t)tpw) * gy;
         const int64_t per_cu = ceil_div(wgs, (int64_t)cus);
-        const int64_t cost = per_cu * tpw;
-        const double dist = per_cu >= 2 ? (double)per_cu / 2 : 2.5;  // 2 -> 1, 3 -> 1.5, 4 -> 2, 1 -> 2.5
+        const int64_t rem = per_cu % occ;
+        const int64_t cost = tpw * ((per_cu / occ) * occ + (rem == 1 ? 2 : rem));
+        const double dist = per_cu >= 2 ? (double)per_cu / 2 : 2.5;
         if (cost < best_cost || (cost == best_cost && dist < best_dist)) {
             best = tpw;
             best_cost = cost;
@@ -298,6 +303,17 @@ inline int pick_tiles_per_wg(int64_t tiles, int gy, int cus) {
     return best;
 }
 
+// Workgroups of `kernel` that fit on one CU at a time (queried once per kernel).
+template <typename Kernel>
+int resident_workgroups(Kernel kernel, size_t lds) {
+    int occ = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, kernel, 256, lds) != hipSuccess || occ < 1) {
+        (void)hipGetLastError();
+        occ = 2;
+    }
+    return occ;
+}
+
 template <int K, int NCB>
 void launch_linear(const float* x, int64_t ldx, const float* W, const float* bias, const float* res, int64_t ldr,
                    int res_mode, int act, const float* x2, int64_t ldx2, const float* W2, int r2, float* out,
@@ -306,14 +322,15 @@ void launch_linear(const float* x, int64_t ldx, const float* W, const float* bia
     const size_t lds = (size_t)TT * (K + 1) * sizeof(float);
     const int gy = N / (32 * NCB);
     const int64_t tiles = ceil_div(T, (int64_t)TT);
-    const int tpw = pick_tiles_per_wg(tiles, gy, device_cu_count());
-    const dim3 grid((unsigned)ceil_div(tiles, (int64_t)tpw), gy);
     auto kernel = linear_tm_k<K, NCB>;
     if (lds > 64 * 1024)
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                   (int)lds);
+    static const int occ = resident_workgroups(kernel, lds);
+    const int tpw = pick_tiles_per_wg(tiles, gy, device_cu_count(), occ);
+    const dim3 grid((unsigned)(ceil_div(tiles, (int64_t)tpw) * gy));
     hipLaunchKernelGGL(kernel, grid, dim3(256), lds, stream, x, ldx, W, N, bias, res, ldr, res_mode, act, x2, ldx2, W2,
-                       r2, out, ldo, plane_cols, plane_stride, T, tpw);
+                       r2, out, ldo, plane_cols, plane_stride, T, tpw, gy);
 }
 
 template <int K>
@@ -332,7 +349,8 @@ template <int K, int CBW>
 void launch_ffn_scalar(const float* x, int64_t ldx, const float* W1, const float* b1, const float* w2, const float* b2,
                        int act, float* out, int64_t T, hipStream_t stream) {
     const int64_t tiles = ceil_div(T, (int64_t)32);
-    const int tpw = pick_tiles_per_wg(tiles, 1, device_cu_count());
+    static const int occ = resident_workgroups(ffn_scalar_k<K, CBW>, 0);
+    const int tpw = pick_tiles_per_wg(tiles, 1, device_cu_count(), occ);
     hipLaunchKernelGGL((ffn_scalar_k<K, CBW>), dim3((unsigned)ceil_div(tiles, (int64_t)tpw)), dim3(256), 0, stream, x,
                        ldx, W1, b1, w2, b2, act, out, T, tpw);
 }
