@@ -24,6 +24,8 @@
 
 namespace spgt {
 
+constexpr int kProjTile = 32;
+
 // grid (nchunk, H/4, B), block 256.  KC = dim_hidden / 128.
 template <int KC, int DP, bool LN>
 __global__ __launch_bounds__(256) void projection_rrc_k(
@@ -33,7 +35,8 @@ __global__ __launch_bounds__(256) void projection_rrc_k(
     constexpr int K = 128 * KC;
     constexpr int D = DP + 32;
     constexpr int PITCH = K + 1;
-    extern __shared__ float xs[];  // [64][PITCH]
+    constexpr int TT = kProjTile;  // tokens per tile
+    extern __shared__ float xs[];  // [TT][PITCH]
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int h = blockIdx.y * 4 + wave;
@@ -61,7 +64,7 @@ __global__ __launch_bounds__(256) void projection_rrc_k(
 
     const float* xb = x + (int64_t)b * S * K;
     float* ob = out + ((int64_t)b * H + h) * D * S;
-    constexpr int NLD = K / 16;  // float4 loads per thread per tile (64*K/4 / 256)
+    constexpr int NLD = TT * K / 4 / 256;  // float4 loads per thread per tile
     float4 stage[NLD];
     auto load_tile = [&](int s0) {
 #pragma unroll
@@ -86,19 +89,35 @@ __global__ __launch_bounds__(256) void projection_rrc_k(
     };
 
     if (s_begin < s_end) load_tile(s_begin);
-    for (int s0 = s_begin; s0 < s_end; s0 += 64) {
+    for (int s0 = s_begin; s0 < s_end; s0 += TT) {
         __syncthreads();  // previous tile fully consumed
         store_tile();
         __syncthreads();
-        if (s0 + 64 < s_end) load_tile(s0 + 64);
+        if (s0 + TT < s_end) load_tile(s0 + TT);
 #pragma unroll
-        for (int tb = 0; tb < 2; ++tb) {
+        for (int tb = 0; tb < TT / 32; ++tb) {
             v16f acc;
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[r] = 0.f;
             const float* xr = xs + (tb * 32 + tk) * PITCH + kh;
+            // LDS reads for the next batch of MFMAs are issued before the current batch, so their
+            // latency hides behind the matrix pipe
+            constexpr int BK = 16;
+            constexpr int NB = K / 2 / BK;
+            float xv[2][BK];
 #pragma unroll
-            for (int kk = 0; kk < K / 2; ++kk) acc = mfma32(wreg[kk], xr[2 * kk], acc);
+            for (int j = 0; j < BK; ++j) xv[0][j] = xr[2 * j];
+#pragma unroll
+            for (int bt = 0; bt < NB; ++bt) {
+                if (bt + 1 < NB) {
+#pragma unroll
+                    for (int j = 0; j < BK; ++j) xv[(bt + 1) & 1][j] = xr[2 * ((bt + 1) * BK + j)];
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int j = 0; j < BK; ++j) acc = mfma32(wreg[bt * BK + j], xv[bt & 1][j], acc);
+                __builtin_amdgcn_sched_barrier(0);
+            }
             const int s = s0 + tb * 32 + tk;
             float y[16];
 #pragma unroll
@@ -140,10 +159,10 @@ void launch_projection(const float* x, const float* W, const float* bias, const 
                        const float* pos, float* out, float* invsigma, int B, int S, int H, float eps,
                        hipStream_t stream) {
     constexpr int K = 128 * KC;
-    const size_t lds = (size_t)64 * (K + 1) * sizeof(float);
-    // about two workgroups per CU; chunks are whole 64-token tiles
-    const int per_b = std::max(1, 512 / std::max(1, B * (H / 4)));
-    const int tpc = std::max(64, ceil_div(ceil_div(S, per_b), 64) * 64);
+    const size_t lds = (size_t)kProjTile * (K + 1) * sizeof(float);
+    // about two workgroups per CU; chunks are whole tiles
+    const int per_b = std::max(1, 2 * device_cu_count() / std::max(1, B * (H / 4)));
+    const int tpc = std::max(kProjTile, ceil_div(ceil_div(S, per_b), kProjTile) * kProjTile);
     const dim3 grid(ceil_div(S, tpc), H / 4, B);
     auto kernel = projection_rrc_k<KC, DP, LN>;
     if (lds > 64 * 1024)
