@@ -200,17 +200,40 @@ int spgt_truncated_dft_rows_supported(int r, int channels, int modes);
  * (network/sp_layer.py:136-141: rfft2, then only columns kw < modes are read):
  *   Y[row, c, j] = sum_w x[row, w, c] * table[w, j],   j = (kw, re|im) < 2*modes
  * x [rows, r, channels] (rows = N*r grid rows of the channels-last tensor), table [r, 2*modes]
- * holds (cos, -sin)(2 pi kw w / r) / sqrt(r), Y [rows, channels, 2*modes]. */
+ * holds (cos, -sin)(2 pi kw w / r) / sqrt(r).  Y is [rows, channels, 2*modes], or with planar != 0
+ * [N, 2*modes, r, channels] (row = n*r + h), the layout spgt_spectral_modes_middle works on. */
 int spgt_truncated_dft_rows_forward(const float* x, const float* table, float* Y, int64_t rows, int r,
-                                    int channels, int modes, spgt_stream_t stream);
+                                    int channels, int modes, int planar, spgt_stream_t stream);
 
 /* The w-direction of irfft2 for a spectrum that is zero beyond column `modes`
  * (network/sp_layer.py:149-151):
  *   y[row, w, o] = sum_j table[w, j] * U[row, o, j]
- * U [rows, channels, 2*modes], table [r, 2*modes] (the forward table with columns scaled by 1 for
- * kw = 0 and the Nyquist column, else 2), y [rows, r, channels]. */
+ * U [rows, channels, 2*modes] (or planar [N, 2*modes, r, channels]), table [r, 2*modes] (the
+ * forward table with columns scaled by 1 for kw = 0 and the Nyquist column, else 2),
+ * y [rows, r, channels]. */
 int spgt_truncated_dft_rows_inverse(const float* U, const float* table, float* y, int64_t rows, int r,
-                                    int channels, int modes, spgt_stream_t stream);
+                                    int channels, int modes, int planar, spgt_stream_t stream);
+
+/* 1 when spgt_spectral_modes_middle serves this shape (Cin, Cout <= 64, 2*modes <= min(32, r),
+ * r <= 4096). */
+int spgt_spectral_modes_middle_supported(int r, int Cin, int Cout, int modes);
+
+/* Bytes of device scratch spgt_spectral_modes_middle needs (the contracted modes O). */
+size_t spgt_spectral_modes_middle_workspace_bytes(int N, int Cout, int modes);
+
+/* Everything between the two w-direction products of Sp_SpectralConv2D's inference path
+ * (network/sp_layer.py:136-151 restricted to the kept modes; contraction as complex_matmul_2D,
+ * network/layer.py:249-261), two launches with O in the caller's workspace:
+ *   Z[n, kh, c, kw] = sum_h table_h[kh, h] Y[n, h, c, kw]              kh: the 2*modes kept rows
+ *   O[n, kh, o, kw] = sum_c Z[n, kh, c, kw] W[kh, kw, c, o]            W = weight_1 (kh < modes) | weight_2
+ *   U[n, h, o, kw]  = sum_kh table_h_inverse[h, kh] O[n, kh, o, kw]
+ * Y [N, 2*modes, r, Cin] and U [N, 2*modes, r, Cout] are the planar layouts of the row kernels
+ * (plane 2*kw real, 2*kw+1 imaginary); table_h [2*modes, r] and table_h_inverse [r, 2*modes] are
+ * complex64; weight_1, weight_2 [modes, modes, Cin, Cout, 2] as network/sp_layer.py:119-121. */
+int spgt_spectral_modes_middle(const float* Y, const float* table_h, const float* table_h_inverse,
+                               const float* weight_1, const float* weight_2, float* U, void* workspace,
+                               size_t workspace_bytes, int N, int r, int Cin, int Cout, int modes,
+                               spgt_stream_t stream);
 
 /* Tensor layouts for spgt_bilinear_resample. */
 enum { SPGT_LAYOUT_NCHW = 0, SPGT_LAYOUT_NHWC = 1 };

@@ -48,8 +48,11 @@ SIGNATURES = {
     "spgt_bilinear_resample": (_i, [_p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p]),
     "spgt_bias_activation_nchw": (_i, [_p, _p, _i, _i, _i64, _i, _i, _p]),
     "spgt_truncated_dft_rows_supported": (_i, [_i, _i, _i]),
-    "spgt_truncated_dft_rows_forward": (_i, [_p, _p, _p, _i64, _i, _i, _i, _p]),
-    "spgt_truncated_dft_rows_inverse": (_i, [_p, _p, _p, _i64, _i, _i, _i, _p]),
+    "spgt_truncated_dft_rows_forward": (_i, [_p, _p, _p, _i64, _i, _i, _i, _i, _p]),
+    "spgt_truncated_dft_rows_inverse": (_i, [_p, _p, _p, _i64, _i, _i, _i, _i, _p]),
+    "spgt_spectral_modes_middle_supported": (_i, [_i, _i, _i, _i]),
+    "spgt_spectral_modes_middle_workspace_bytes": (_sz, [_i, _i, _i]),
+    "spgt_spectral_modes_middle": (_i, [_p, _p, _p, _p, _p, _p, _p, _sz, _i, _i, _i, _i, _i, _p]),
     "spgt_linear_supported": (_i, [_i, _i]),
     "spgt_linear_forward": (_i, [_p, _i64, _p, _p, _p, _i64, _i, _i, _p, _i64, _p, _i, _p, _i64, _i, _i64, _i64, _i, _i,
                                  _p]),

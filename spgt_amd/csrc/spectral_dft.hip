@@ -23,9 +23,10 @@ namespace spgt {
 
 // grid (workgroups), block 256; waves stride over the rows * C/32 (row, channel block) items.
 // tab [r][m2] row-major, m2 <= 32.
-// Y [rows][C][m2].
+// Y [rows][C][m2], or planar [rows/r][m2][r][C].
 __global__ __launch_bounds__(256) void dft_rows_forward_k(const float* __restrict__ x, const float* __restrict__ tab,
-                                                          float* __restrict__ Y, int64_t rows, int r, int C, int m2) {
+                                                          float* __restrict__ Y, int64_t rows, int r, int C, int m2,
+                                                          int planar) {
     extern __shared__ float ts[];  // [2*KH][32], zero beyond r rows and m2 columns
     const int KH = (r + 1) / 2;
     {
@@ -102,22 +103,37 @@ __global__ __launch_bounds__(256) void dft_rows_forward_k(const float* __restric
         __builtin_amdgcn_sched_barrier(0);
     }
     // acc[r] = Y[c = cb*32 + tk][j = 8*(r/4) + 4*kh + r%4]
-    float* yr = Y + (row * C + cb * 32 + tk) * (int64_t)m2;
+    if (planar) {
+        // Y[n][j][h][c] with row = n*r + h: every store is a 128-byte run along c
+        const int64_t n = row / r;
+        const int64_t h = row - n * r;
+        float* yp = Y + (n * m2 * r + h) * (int64_t)C + cb * 32 + tk;
 #pragma unroll
-    for (int q = 0; q < 4; ++q)
+        for (int q = 0; q < 4; ++q)
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const int j = 8 * q + 4 * kh + e;
-            if (j < m2) yr[j] = acc[4 * q + e];
-        }
+            for (int e = 0; e < 4; ++e) {
+                const int j = 8 * q + 4 * kh + e;
+                if (j < m2) yp[(int64_t)j * r * C] = acc[4 * q + e];
+            }
+    } else {
+        float* yr = Y + (row * C + cb * 32 + tk) * (int64_t)m2;
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int j = 8 * q + 4 * kh + e;
+                if (j < m2) yr[j] = acc[4 * q + e];
+            }
+    }
     }
 }
 
 // grid (workgroups), block 256; waves stride over the (row, channel block) items.
 // tab [r][m2] row-major, m2 <= 32 and even.
-// U [rows][C][m2] -> y [rows][r][C].
+// U [rows][C][m2] (or planar [rows/r][m2][r][C]) -> y [rows][r][C].
 __global__ __launch_bounds__(256) void dft_rows_inverse_k(const float* __restrict__ U, const float* __restrict__ tab,
-                                                          float* __restrict__ y, int64_t rows, int r, int C, int m2) {
+                                                          float* __restrict__ y, int64_t rows, int r, int C, int m2,
+                                                          int planar) {
     extern __shared__ float ts[];  // [32 * ceil(r/32)][m2 + 1], zero beyond r rows
     const int pitch = m2 + 1;
     const int WT = (r + 31) / 32;
@@ -146,10 +162,18 @@ __global__ __launch_bounds__(256) void dft_rows_inverse_k(const float* __restric
     const int64_t row = gw / CB;
     const int cb = (int)(gw % CB);
     // B operand: U[o = cb*32 + tk][j = 2kk + kh]
-    const float* ur = U + (row * C + cb * 32 + tk) * (int64_t)m2;
     float ureg[16];
+    if (planar) {
+        const int64_t n = row / r;
+        const int64_t h = row - n * r;
+        const float* up = U + (n * m2 * r + h) * (int64_t)C + cb * 32 + tk;  // U[n][j][h][o]
 #pragma unroll
-    for (int kk = 0; kk < 16; ++kk) ureg[kk] = (2 * kk + kh < m2) ? ur[2 * kk + kh] : 0.f;
+        for (int kk = 0; kk < 16; ++kk) ureg[kk] = (2 * kk + kh < m2) ? up[(int64_t)(2 * kk + kh) * r * C] : 0.f;
+    } else {
+        const float* ur = U + (row * C + cb * 32 + tk) * (int64_t)m2;
+#pragma unroll
+        for (int kk = 0; kk < 16; ++kk) ureg[kk] = (2 * kk + kh < m2) ? ur[2 * kk + kh] : 0.f;
+    }
     float* yr = y + row * (int64_t)r * C + cb * 32 + tk;
     const int KH = m2 / 2;
     for (int wt = 0; wt < WT; ++wt) {
@@ -167,6 +191,165 @@ __global__ __launch_bounds__(256) void dft_rows_inverse_k(const float* __restric
             if (w < r) yr[(int64_t)w * C] = acc[q];
         }
     }
+    }
+}
+
+// Everything between the two w-direction products of the spectral layer
+// (network/sp_layer.py:136-151 restricted to the kept modes), in two launches:
+//   Z[kh, c] = sum_h G[kh, h] Y[h, c]          forward DFT along h, 2m kept rows kh      } spectral_rows_contract_k
+//   O[kh, o] = sum_c Z[kh, c] W[kh, kw, c, o]  complex contraction (network/layer.py:249-261) }
+//   U[h, o]  = sum_kh Gi[h, kh] O[kh, o]       inverse DFT along h                        } spectral_rows_expand_k
+// on planar operands Y [N][2m][r][Cin] and U [N][2m][r][Cout] (plane 2kw = real, 2kw+1 = imaginary).
+// Lanes run along channels, so every global access is a 256-byte run; twiddle factors sit in LDS and
+// are wave-uniform.  All loads of a phase are in flight together (the data is a few MB: the kernels
+// are bound by memory round trips, not bandwidth), and every sum runs in a fixed order.
+constexpr int kMidC = 64;     // channels per operand (lanes)
+constexpr int kMidRows = 3;   // kept rows kh per workgroup of the first kernel
+constexpr int kMidHB = 32;    // grid rows h fetched per batch
+
+// grid (m, N, ceil(2m / kMidRows)), block 256.  O [N][m][2m][Cout] complex.
+__global__ __launch_bounds__(256) void spectral_rows_contract_k(
+    const float* __restrict__ Y, const float2* __restrict__ G, const float2* __restrict__ W1,
+    const float2* __restrict__ W2, float2* __restrict__ O, int r, int Cin, int Cout, int m) {
+    extern __shared__ float2 lds[];
+    // [tab: kMidRows x r][part: 4 x kMidRows x 64]; part doubles as the per-c-quarter partial O
+    float2* tab = lds;
+    float2 (*part)[kMidRows][kMidC] = reinterpret_cast<float2 (*)[kMidRows][kMidC]>(lds + kMidRows * r);
+    __shared__ float2 Zs[kMidRows][kMidC];
+    const int m2 = 2 * m;
+    const int kw = blockIdx.x;
+    const int64_t n = blockIdx.y;
+    const int kh0 = blockIdx.z * kMidRows;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    for (int e = threadIdx.x; e < kMidRows * r; e += 256) {
+        const int q = e / r, h = e - q * r;
+        tab[e] = (kh0 + q < m2) ? G[(int64_t)(kh0 + q) * r + h] : make_float2(0.f, 0.f);
+    }
+    __syncthreads();
+
+    // Z = G Y: wave hq sums its quarter of h for the workgroup's rows; lane = input channel
+    {
+        const int hlen = (r + 3) / 4;
+        const int h0 = wave * hlen;
+        const int h1 = min(r, h0 + hlen);
+        const float* yre = Y + ((n * m2 + 2 * kw) * r) * (int64_t)Cin + lane;
+        const float* yim = yre + (int64_t)r * Cin;
+        const bool cok = lane < Cin;
+        float2 acc[kMidRows];
+#pragma unroll
+        for (int q = 0; q < kMidRows; ++q) acc[q] = make_float2(0.f, 0.f);
+        for (int hb = h0; hb < h1; hb += kMidHB) {
+            float a[kMidHB], b[kMidHB];
+#pragma unroll
+            for (int u = 0; u < kMidHB; ++u) {
+                const int h = min(hb + u, h1 - 1);
+                a[u] = cok ? yre[(int64_t)h * Cin] : 0.f;
+                b[u] = cok ? yim[(int64_t)h * Cin] : 0.f;
+            }
+#pragma unroll
+            for (int u = 0; u < kMidHB; ++u) {
+                if (hb + u < h1) {
+#pragma unroll
+                    for (int q = 0; q < kMidRows; ++q) {
+                        const float2 g = tab[q * r + hb + u];
+                        acc[q].x = fmaf(g.x, a[u], acc[q].x);
+                        acc[q].x = fmaf(-g.y, b[u], acc[q].x);
+                        acc[q].y = fmaf(g.x, b[u], acc[q].y);
+                        acc[q].y = fmaf(g.y, a[u], acc[q].y);
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int q = 0; q < kMidRows; ++q) part[wave][q][lane] = acc[q];
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < kMidRows * kMidC; e += 256) {
+        const int q = e / kMidC, c = e % kMidC;
+        const float2 p0 = part[0][q][c], p1 = part[1][q][c], p2 = part[2][q][c], p3 = part[3][q][c];
+        Zs[q][c] = make_float2((p0.x + p1.x) + (p2.x + p3.x), (p0.y + p1.y) + (p2.y + p3.y));
+    }
+    __syncthreads();
+
+    // O = Z . W: wave w takes input channels [16w, 16w+16) of every row; lane = output channel
+    {
+        constexpr int CQ = kMidC / 4;
+        const bool ook = lane < Cout;
+        float2 wv[kMidRows][CQ];
+#pragma unroll
+        for (int q = 0; q < kMidRows; ++q) {
+            const int kh = min(kh0 + q, m2 - 1);
+            const float2* Wm = (kh < m ? W1 + ((int64_t)kh * m + kw) * Cin * Cout
+                                       : W2 + ((int64_t)(kh - m) * m + kw) * Cin * Cout) + lane;
+#pragma unroll
+            for (int u = 0; u < CQ; ++u) {
+                const int c = wave * CQ + u;
+                wv[q][u] = (ook && c < Cin) ? Wm[(int64_t)c * Cout] : make_float2(0.f, 0.f);
+            }
+        }
+#pragma unroll
+        for (int q = 0; q < kMidRows; ++q) {
+            float2 o = make_float2(0.f, 0.f);
+#pragma unroll
+            for (int u = 0; u < CQ; ++u) {
+                const float2 z = Zs[q][wave * CQ + u];
+                o.x = fmaf(z.x, wv[q][u].x, o.x);
+                o.x = fmaf(-z.y, wv[q][u].y, o.x);
+                o.y = fmaf(z.y, wv[q][u].x, o.y);
+                o.y = fmaf(z.x, wv[q][u].y, o.y);
+            }
+            part[wave][q][lane] = o;
+        }
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < kMidRows * kMidC; e += 256) {
+        const int q = e / kMidC, o = e % kMidC;
+        if (kh0 + q < m2 && o < Cout) {
+            const float2 p0 = part[0][q][o], p1 = part[1][q][o], p2 = part[2][q][o], p3 = part[3][q][o];
+            O[((n * m + kw) * m2 + kh0 + q) * (int64_t)Cout + o] =
+                make_float2((p0.x + p1.x) + (p2.x + p3.x), (p0.y + p1.y) + (p2.y + p3.y));
+        }
+    }
+}
+
+// grid (m, N, chunks of h), block 256.  Wave w of a workgroup takes rows h = h0 + w, h0 + w + 4, ...
+__global__ __launch_bounds__(256) void spectral_rows_expand_k(
+    const float2* __restrict__ O, const float2* __restrict__ Gi, float* __restrict__ U, int r, int Cout, int m,
+    int rows_per_wg) {
+    extern __shared__ float2 lds[];  // Gi rows of the chunk: [rows_per_wg][2m]
+    const int m2 = 2 * m;
+    const int kw = blockIdx.x;
+    const int64_t n = blockIdx.y;
+    const int h0 = blockIdx.z * rows_per_wg;
+    const int h1 = min(r, h0 + rows_per_wg);
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    for (int e = threadIdx.x; e < (h1 - h0) * m2; e += 256) lds[e] = Gi[(int64_t)h0 * m2 + e];
+    // the mode's O[kh][o] for all kept rows stays in registers
+    float2 ov[32];
+    const float2* Om = O + ((n * m + kw) * m2) * (int64_t)Cout + lane;
+#pragma unroll
+    for (int kh = 0; kh < 32; ++kh) ov[kh] = (kh < m2 && lane < Cout) ? Om[(int64_t)kh * Cout] : make_float2(0.f, 0.f);
+    __syncthreads();
+    float* ure = U + ((n * m2 + 2 * kw) * r) * (int64_t)Cout + lane;
+    float* uim = ure + (int64_t)r * Cout;
+    for (int h = h0 + wave; h < h1; h += 4) {
+        const float2* g = lds + (h - h0) * m2;
+        float2 acc = make_float2(0.f, 0.f);
+#pragma unroll
+        for (int kh = 0; kh < 32; ++kh) {
+            if (kh < m2) {
+                acc.x = fmaf(g[kh].x, ov[kh].x, acc.x);
+                acc.x = fmaf(-g[kh].y, ov[kh].y, acc.x);
+                acc.y = fmaf(g[kh].x, ov[kh].y, acc.y);
+                acc.y = fmaf(g[kh].y, ov[kh].x, acc.y);
+            }
+        }
+        if (lane < Cout) {
+            ure[(int64_t)h * Cout] = acc.x;
+            uim[(int64_t)h * Cout] = acc.y;
+        }
     }
 }
 
@@ -199,7 +382,7 @@ extern "C" int spgt_truncated_dft_rows_supported(int r, int channels, int modes)
 }
 
 extern "C" int spgt_truncated_dft_rows_forward(const float* x, const float* table, float* Y, int64_t rows, int r,
-                                               int channels, int modes, hipStream_t stream) {
+                                               int channels, int modes, int planar, hipStream_t stream) {
     const int m2 = 2 * modes;
     if (int rc = dft_rows_check("truncated_dft_rows_forward", x, table, Y, rows, r, channels, m2)) return rc;
     const size_t lds = (size_t)2 * ((r + 1) / 2) * 32 * sizeof(float);
@@ -209,12 +392,14 @@ extern "C" int spgt_truncated_dft_rows_forward(const float* x, const float* tabl
                                   (int)lds);
     // workgroups loop over (row, channel block) items: about two per CU, so the table is staged few times
     const unsigned grid = (unsigned)std::min<int64_t>(ceil_div(rows * (channels / 32), (int64_t)4), 2 * device_cu_count());
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), lds, stream, x, table, Y, rows, r, channels, m2);
+    if (planar && rows % r != 0)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "truncated_dft_rows_forward: planar output needs rows = N * r");
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), lds, stream, x, table, Y, rows, r, channels, m2, planar);
     return check_launch("truncated_dft_rows_forward");
 }
 
 extern "C" int spgt_truncated_dft_rows_inverse(const float* U, const float* table, float* y, int64_t rows, int r,
-                                               int channels, int modes, hipStream_t stream) {
+                                               int channels, int modes, int planar, hipStream_t stream) {
     const int m2 = 2 * modes;
     if (int rc = dft_rows_check("truncated_dft_rows_inverse", U, table, y, rows, r, channels, m2)) return rc;
     const size_t lds = (size_t)((r + 31) / 32) * 32 * (m2 + 1) * sizeof(float);
@@ -223,6 +408,51 @@ extern "C" int spgt_truncated_dft_rows_inverse(const float* U, const float* tabl
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                   (int)lds);
     const unsigned grid = (unsigned)std::min<int64_t>(ceil_div(rows * (channels / 32), (int64_t)4), 2 * device_cu_count());
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), lds, stream, U, table, y, rows, r, channels, m2);
+    if (planar && rows % r != 0)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "truncated_dft_rows_inverse: planar input needs rows = N * r");
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), lds, stream, U, table, y, rows, r, channels, m2, planar);
     return check_launch("truncated_dft_rows_inverse");
+}
+
+extern "C" int spgt_spectral_modes_middle_supported(int r, int Cin, int Cout, int modes) {
+    return (r > 0 && r <= 4096 && Cin > 0 && Cin <= kMidC && Cout > 0 && Cout <= kMidC && modes > 0 &&
+            2 * modes <= 32 && 2 * modes <= r) ? 1 : 0;
+}
+
+extern "C" size_t spgt_spectral_modes_middle_workspace_bytes(int N, int Cout, int modes) {
+    if (N <= 0 || Cout <= 0 || modes <= 0) return 0;
+    return (size_t)N * modes * 2 * modes * Cout * sizeof(float2);
+}
+
+extern "C" int spgt_spectral_modes_middle(const float* Y, const float* table_h, const float* table_h_inverse,
+                                          const float* weight_1, const float* weight_2, float* U, void* workspace,
+                                          size_t workspace_bytes, int N, int r, int Cin, int Cout, int modes,
+                                          hipStream_t stream) {
+    if (!Y || !table_h || !table_h_inverse || !weight_1 || !weight_2 || !U || !workspace)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "spectral_modes_middle: null pointer argument");
+    if (N <= 0 || N > 65535) return fail(SPGT_ERR_INVALID_ARGUMENT, "spectral_modes_middle: N must be 1..65535");
+    if (!spgt_spectral_modes_middle_supported(r, Cin, Cout, modes))
+        return fail(SPGT_ERR_INVALID_ARGUMENT,
+                    "spectral_modes_middle: needs Cin, Cout <= 64, 2*modes <= min(32, r), r <= 4096");
+    if (workspace_bytes < spgt_spectral_modes_middle_workspace_bytes(N, Cout, modes))
+        return fail(SPGT_ERR_WORKSPACE, "spectral_modes_middle: workspace too small");
+    if (!aligned4(Y) || !aligned4(U) || !aligned8(table_h) || !aligned8(table_h_inverse) || !aligned8(weight_1) ||
+        !aligned8(weight_2) || !aligned8(workspace))
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "spectral_modes_middle: complex operands must be 8-byte aligned");
+    const int m2 = 2 * modes;
+    float2* O = reinterpret_cast<float2*>(workspace);
+    const size_t lds1 = ((size_t)kMidRows * r + 4 * kMidRows * kMidC) * sizeof(float2);
+    static const hipError_t opt_in = hipFuncSetAttribute(reinterpret_cast<const void*>(spectral_rows_contract_k),
+                                                         hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
+    (void)opt_in;
+    hipLaunchKernelGGL(spectral_rows_contract_k, dim3(modes, N, ceil_div(m2, kMidRows)), dim3(256), lds1, stream, Y,
+                       reinterpret_cast<const float2*>(table_h), reinterpret_cast<const float2*>(weight_1),
+                       reinterpret_cast<const float2*>(weight_2), O, r, Cin, Cout, modes);
+    // about three workgroups per CU for the expansion
+    const int chunks = std::max(1, std::min(ceil_div(r, 4), ceil_div(3 * device_cu_count(), modes * N)));
+    const int rows_per_wg = ceil_div(r, chunks);
+    const size_t lds2 = (size_t)rows_per_wg * m2 * sizeof(float2);
+    hipLaunchKernelGGL(spectral_rows_expand_k, dim3(modes, N, ceil_div(r, rows_per_wg)), dim3(256), lds2, stream, O,
+                       reinterpret_cast<const float2*>(table_h_inverse), U, r, Cout, modes, rows_per_wg);
+    return check_launch("spectral_modes_middle");
 }

@@ -14,7 +14,7 @@ import torch
 from torch import Tensor
 
 from ... import _lib
-from ..._lib import check, ptr, require_gpu_f32, stream_of
+from ..._lib import check, ptr, require_gpu_f32, stream_of, workspace
 
 
 # --------------------------------------------------------------------------- #
@@ -160,30 +160,73 @@ def _truncated_dft_rows_supported(r: int, channels: int, modes: int) -> bool:
     return bool(_lib.load().spgt_truncated_dft_rows_supported(int(r), int(channels), int(modes)))
 
 
-def _truncated_dft_rows(src: Tensor, table: Tensor, inverse: bool) -> Tensor:
-    """forward: src [..., r, C] x table [r, 2m] -> [..., C, 2m];  inverse: src [..., C, 2m] -> [..., r, C]."""
+def _truncated_dft_rows(src: Tensor, table: Tensor, inverse: bool, planar: bool = False) -> Tensor:
+    """forward: src [..., r, C] x table [r, 2m] -> [..., C, 2m], or planar [N, 2m, r, C] from src [N, r, r, C];
+    inverse: src [..., C, 2m] (or planar [N, 2m, r, C]) -> [..., r, C]."""
     require_gpu_f32("src", src)
     require_gpu_f32("table", table)
     r, m2 = table.shape
     if inverse:
-        C = src.shape[-2]
-        if src.shape[-1] != m2:
-            raise ValueError(f"src has last dimension {src.shape[-1]}, the table has {m2} columns")
-        lead = tuple(src.shape[:-2])
+        if planar:
+            if src.dim() != 4 or src.shape[1] != m2 or src.shape[2] != r:
+                raise ValueError(f"planar src must be [N, {m2}, {r}, C]")
+            N, C = src.shape[0], src.shape[3]
+            lead = (N, r)
+        else:
+            C = src.shape[-2]
+            if src.shape[-1] != m2:
+                raise ValueError(f"src has last dimension {src.shape[-1]}, the table has {m2} columns")
+            lead = tuple(src.shape[:-2])
         out = torch.empty(lead + (r, C), dtype=src.dtype, device=src.device)
     else:
         C = src.shape[-1]
         if src.shape[-2] != r:
             raise ValueError(f"src has {src.shape[-2]} grid points per row, the table has {r} rows")
         lead = tuple(src.shape[:-2])
-        out = torch.empty(lead + (C, m2), dtype=src.dtype, device=src.device)
+        if planar:
+            if src.dim() != 4 or src.shape[1] != r:
+                raise ValueError(f"planar output needs src [N, {r}, {r}, C]")
+            out = torch.empty((src.shape[0], m2, r, C), dtype=src.dtype, device=src.device)
+        else:
+            out = torch.empty(lead + (C, m2), dtype=src.dtype, device=src.device)
     rows = prod(lead)
     if rows == 0:
         return out
     fn = _lib.load().spgt_truncated_dft_rows_inverse if inverse else _lib.load().spgt_truncated_dft_rows_forward
     with torch.cuda.device(src.device):
-        check(fn(ptr(src), ptr(table), ptr(out), rows, r, C, m2 // 2, stream_of(src)))
+        check(fn(ptr(src), ptr(table), ptr(out), rows, r, C, m2 // 2, int(planar), stream_of(src)))
     return out
+
+
+def _spectral_modes_middle_supported(r: int, cin: int, cout: int, modes: int) -> bool:
+    return bool(_lib.load().spgt_spectral_modes_middle_supported(int(r), int(cin), int(cout), int(modes)))
+
+
+def _spectral_modes_middle(Y: Tensor, table_h: Tensor, table_h_inverse: Tensor, weight_1: Tensor,
+                           weight_2: Tensor) -> Tensor:
+    """Y planar [N, 2m, r, Cin] -> U planar [N, 2m, r, Cout]: DFT along h onto the 2m kept rows, complex
+    channel contraction with weight_1 | weight_2 [m, m, Cin, Cout, 2], inverse DFT along h."""
+    require_gpu_f32("Y", Y)
+    require_gpu_f32("table_h", table_h, torch.complex64)
+    require_gpu_f32("table_h_inverse", table_h_inverse, torch.complex64)
+    require_gpu_f32("weight_1", weight_1)
+    require_gpu_f32("weight_2", weight_2)
+    N, m2, r, cin = Y.shape
+    m = m2 // 2
+    cout = weight_1.shape[3]
+    if tuple(weight_1.shape) != (m, m, cin, cout, 2) or weight_2.shape != weight_1.shape:
+        raise ValueError(f"weights must be [{m}, {m}, {cin}, Cout, 2]")
+    if tuple(table_h.shape) != (m2, r) or tuple(table_h_inverse.shape) != (r, m2):
+        raise ValueError(f"tables must be [{m2}, {r}] and [{r}, {m2}]")
+    U = torch.empty((N, m2, r, cout), dtype=Y.dtype, device=Y.device)
+    if U.numel() == 0:
+        return U
+    lib = _lib.load()
+    ws = workspace(lib.spgt_spectral_modes_middle_workspace_bytes(N, cout, m), Y)
+    with torch.cuda.device(Y.device):
+        check(lib.spgt_spectral_modes_middle(ptr(Y), ptr(table_h), ptr(table_h_inverse), ptr(weight_1), ptr(weight_2),
+                                             ptr(U), ptr(ws), ws.numel(), N, r, cin, cout, m, stream_of(Y)))
+    return U
 
 
 _ACT = {None: 0, "none": 0, "relu": 1, "silu": 2}
@@ -247,6 +290,8 @@ def _bias_activation_nchw_(X: Tensor, bias, activation=None, count: int = 1) -> 
 dexts = SimpleNamespace(
     truncated_dft_rows_supported=_truncated_dft_rows_supported,
     truncated_dft_rows=_truncated_dft_rows,
+    spectral_modes_middle_supported=_spectral_modes_middle_supported,
+    spectral_modes_middle=_spectral_modes_middle,
     bias_activation_nchw_=_bias_activation_nchw_,
     bilinear_resample=_bilinear_resample,
     bilinear_align_corners_nhwc=_bilinear_align_corners_nhwc,
@@ -356,11 +401,25 @@ def truncated_dft_rows_supported(r: int, channels: int, modes: int) -> bool:
     return dexts.truncated_dft_rows_supported(r, channels, modes)
 
 
-def truncated_dft_rows_forward(X: Tensor, table: Tensor) -> Tensor:
-    """Y[..., c, j] = sum_w X[..., w, c] table[w, j]: X [..., r, C], table [r, 2m] -> [..., C, 2m] (inference only)."""
-    return dexts.truncated_dft_rows(X.detach(), table, False)
+def truncated_dft_rows_forward(X: Tensor, table: Tensor, planar: bool = False) -> Tensor:
+    """Y[..., c, j] = sum_w X[..., w, c] table[w, j]: X [..., r, C], table [r, 2m] -> [..., C, 2m], or with
+    planar X [N, r, r, C] -> [N, 2m, r, C] (inference only)."""
+    return dexts.truncated_dft_rows(X.detach(), table, False, planar)
 
 
-def truncated_dft_rows_inverse(U: Tensor, table: Tensor) -> Tensor:
-    """y[..., w, o] = sum_j table[w, j] U[..., o, j]: U [..., C, 2m], table [r, 2m] -> [..., r, C] (inference only)."""
-    return dexts.truncated_dft_rows(U.detach(), table, True)
+def truncated_dft_rows_inverse(U: Tensor, table: Tensor, planar: bool = False) -> Tensor:
+    """y[..., w, o] = sum_j table[w, j] U[..., o, j]: U [..., C, 2m] (or planar [N, 2m, r, C]), table [r, 2m]
+    -> [..., r, C] (inference only)."""
+    return dexts.truncated_dft_rows(U.detach(), table, True, planar)
+
+
+def spectral_modes_middle_supported(r: int, cin: int, cout: int, modes: int) -> bool:
+    """True when spectral_modes_middle has a kernel for this shape."""
+    return dexts.spectral_modes_middle_supported(r, cin, cout, modes)
+
+
+def spectral_modes_middle(Y: Tensor, table_h: Tensor, table_h_inverse: Tensor, weight_1: Tensor,
+                          weight_2: Tensor) -> Tensor:
+    """DFT along h onto the kept rows, mode-wise complex channel contraction, inverse DFT along h, on the
+    planar operands of the row kernels (inference only)."""
+    return dexts.spectral_modes_middle(Y.detach(), table_h, table_h_inverse, weight_1.detach(), weight_2.detach())

@@ -24,7 +24,8 @@ from typing import Dict, Tuple
 import torch
 from torch import Tensor
 
-from ..extension.bind.datamove import (spectral_modes_compact, truncated_dft_rows_forward, truncated_dft_rows_inverse,
+from ..extension.bind.datamove import (spectral_modes_compact, spectral_modes_middle, spectral_modes_middle_supported,
+                                       truncated_dft_rows_forward, truncated_dft_rows_inverse,
                                        truncated_dft_rows_supported)
 
 _TABLES: Dict[Tuple[int, int, str], Tuple[Tensor, Tensor, Tensor, Tensor]] = {}
@@ -66,6 +67,11 @@ def spectral_modes_apply(x: Tensor, weight_1: Tensor, weight_2: Tensor, m: int) 
     cout = weight_1.shape[3]
     fw, gh, ghi, fwi = dft_tables(r, m, x.device)
     rows_kernel = truncated_dft_rows_supported(r, cin, m) and truncated_dft_rows_supported(r, cout, m)
+    if rows_kernel and spectral_modes_middle_supported(r, cin, cout, m):
+        # three launches: DFT along w, everything on the retained modes, inverse DFT along w
+        yp = truncated_dft_rows_forward(x, fw, planar=True)                               # [N, 2m, r, Cin]
+        up = spectral_modes_middle(yp, gh, ghi, weight_1, weight_2)                       # [N, 2m, r, Cout]
+        return truncated_dft_rows_inverse(up, fwi, planar=True)                           # [N, r, r, Cout]
     if rows_kernel:
         y = truncated_dft_rows_forward(x.reshape(N * r, r, cin), fw)                     # [N r, Cin, 2m]
     else:

@@ -310,3 +310,37 @@ def test_truncated_dft_rows_rejects(gpu):
     assert not dm.truncated_dft_rows_supported(211, 64, 17)
     with pytest.raises(SpgtError):
         dm.truncated_dft_rows_forward(rnd(2, 9, 48, seed=1).to(gpu), rnd(9, 8, seed=2).to(gpu))
+
+
+@pytest.mark.parametrize("N,r,cin,cout,m", [(2, 211, 64, 64, 12), (1, 21, 32, 32, 4), (3, 16, 64, 32, 8), (2, 33, 24, 40, 16)])
+def test_spectral_modes_middle_against_float64(gpu, N, r, cin, cout, m):
+    """DFT along h onto the kept rows, complex contraction, inverse DFT along h (network/sp_layer.py:136-151
+    restricted to the kept modes) against the same three products in float64."""
+    from spgt_amd.network.truncated_dft import dft_tables
+    _, gh, ghi, _ = dft_tables(r, m, "cpu")
+    y = rnd(N, 2 * m, r, cin, seed=81)
+    w1, w2 = rnd(m, m, cin, cout, 2, seed=82) / cin ** 0.5, rnd(m, m, cin, cout, 2, seed=83) / cin ** 0.5
+    assert dm.spectral_modes_middle_supported(r, cin, cout, m)
+    got = dm.spectral_modes_middle(y.to(gpu), gh.to(gpu), ghi.to(gpu), w1.to(gpu), w2.to(gpu)).cpu().double()
+    yc = torch.complex(y[:, 0::2].double(), y[:, 1::2].double())               # [N, kw, h, c]
+    z = torch.einsum("kh,nwhc->nkcw", gh.to(torch.complex128), yc)             # [N, kh, c, kw]
+    wc = torch.cat([torch.view_as_complex(w1.double()), torch.view_as_complex(w2.double())], 0)  # [2m kh, kw, c, o]
+    o = torch.einsum("nkcw,kwco->nkow", z, wc)
+    u = torch.einsum("hk,nkow->nwho", ghi.to(torch.complex128), o)             # [N, kw, h, o]
+    want = torch.stack([u.real, u.imag], 2).reshape(N, 2 * m, r, cout)
+    assert got.shape == want.shape
+    assert (got - want).abs().max().item() <= 1e-5 * max(1.0, want.abs().max().item())
+
+
+def test_truncated_dft_rows_planar_layout(gpu):
+    """planar=True is the interleaved result with the mode axis moved ahead of the grid row."""
+    from spgt_amd.network.truncated_dft import dft_tables
+    fw, _, _, fwi = dft_tables(33, 8, "cpu")
+    x = rnd(2, 33, 33, 64, seed=91).to(gpu)
+    a = dm.truncated_dft_rows_forward(x.view(66, 33, 64), fw.to(gpu)).view(2, 33, 64, 16)
+    b = dm.truncated_dft_rows_forward(x, fw.to(gpu), planar=True)
+    assert torch.equal(b, a.permute(0, 3, 1, 2).contiguous())
+    u = rnd(2, 16, 33, 64, seed=92).to(gpu)
+    c = dm.truncated_dft_rows_inverse(u, fwi.to(gpu), planar=True)
+    d = dm.truncated_dft_rows_inverse(u.permute(0, 2, 3, 1).contiguous().view(66, 64, 16), fwi.to(gpu)).view(2, 33, 33, 64)
+    assert torch.equal(c, d)
