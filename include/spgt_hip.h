@@ -199,8 +199,9 @@ int spgt_truncated_dft_rows_supported(int r, int channels, int modes);
 /* The w-direction of rfft2 restricted to the modes Sp_SpectralConv2D keeps
  * (network/sp_layer.py:136-141: rfft2, then only columns kw < modes are read):
  *   Y[row, c, j] = sum_w x[row, w, c] * table[w, j],   j = (kw, re|im) < 2*modes
- * x [rows, r, channels] (rows = N*r grid rows of the channels-last tensor), table [r, 2*modes]
- * holds (cos, -sin)(2 pi kw w / r) / sqrt(r).  Y is [rows, channels, 2*modes], or with planar != 0
+ * x [rows, r, channels] (rows = N*r grid rows of the channels-last tensor); table[w, j] =
+ * (cos, -sin)(2 pi kw w / r) / sqrt(r), handed over zero-padded to [2*ceil(r/2), 32] (the layout
+ * the kernel keeps in LDS, 16-byte aligned).  Y is [rows, channels, 2*modes], or with planar != 0
  * [N, 2*modes, r, channels] (row = n*r + h), the layout spgt_spectral_modes_middle works on. */
 int spgt_truncated_dft_rows_forward(const float* x, const float* table, float* Y, int64_t rows, int r,
                                     int channels, int modes, int planar, spgt_stream_t stream);
@@ -208,9 +209,9 @@ int spgt_truncated_dft_rows_forward(const float* x, const float* table, float* Y
 /* The w-direction of irfft2 for a spectrum that is zero beyond column `modes`
  * (network/sp_layer.py:149-151):
  *   y[row, w, o] = sum_j table[w, j] * U[row, o, j]
- * U [rows, channels, 2*modes] (or planar [N, 2*modes, r, channels]), table [r, 2*modes] (the
- * forward table with columns scaled by 1 for kw = 0 and the Nyquist column, else 2),
- * y [rows, r, channels]. */
+ * U [rows, channels, 2*modes] (or planar [N, 2*modes, r, channels]); table = the forward table
+ * with columns scaled by 1 for kw = 0 and the Nyquist column, else 2, handed over zero-padded to
+ * [32*ceil(r/32), 2*modes + 1] (16-byte aligned); y [rows, r, channels]. */
 int spgt_truncated_dft_rows_inverse(const float* U, const float* table, float* y, int64_t rows, int r,
                                     int channels, int modes, int planar, spgt_stream_t stream);
 

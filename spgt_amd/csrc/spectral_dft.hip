@@ -22,27 +22,29 @@
 namespace spgt {
 
 // grid (workgroups), block 256; waves stride over the rows * C/32 (row, channel block) items.
-// tab [r][m2] row-major, m2 <= 32.
-// Y [rows][C][m2], or planar [rows/r][m2][r][C].
+// tab [2*ceil(r/2)][32]: row w holds the m2 table entries of grid point w, zero elsewhere.
+// Y [rows][C][m2], or planar [rows/r][m2][r][C].  CT = C when known at compile time (row offsets
+// become immediates), 0 = any C.
+template <int CT>
 __global__ __launch_bounds__(256) void dft_rows_forward_k(const float* __restrict__ x, const float* __restrict__ tab,
-                                                          float* __restrict__ Y, int64_t rows, int r, int C, int m2,
+                                                          float* __restrict__ Y, int64_t rows, int r, int C_, int m2,
                                                           int planar) {
-    extern __shared__ float ts[];  // [2*KH][32], zero beyond r rows and m2 columns
+    extern __shared__ float ts[];  // a copy of `tab`
+    const int C = CT ? CT : C_;
     const int KH = (r + 1) / 2;
     {
-        // table fill with eight loads in flight per thread
-        const int total = 2 * KH * 32;
-        for (int e0 = threadIdx.x; e0 < total; e0 += 256 * 8) {
-            float v[8];
-#pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                const int e = e0 + 256 * u;
-                const int w = e >> 5, j = e & 31;
-                v[u] = (e < total && w < r && j < m2) ? tab[w * m2 + j] : 0.f;
-            }
+        // straight 16-byte copy, eight loads in flight per thread: one memory round trip for r <= 256
+        const int total4 = 2 * KH * 8;
+        const float4* src = reinterpret_cast<const float4*>(tab);
+        float4* dst = reinterpret_cast<float4*>(ts);
+        for (int e0 = threadIdx.x; e0 < total4; e0 += 256 * 8) {
+            float4 v[8];
 #pragma unroll
             for (int u = 0; u < 8; ++u)
-                if (e0 + 256 * u < total) ts[e0 + 256 * u] = v[u];
+                v[u] = (e0 + 256 * u < total4) ? src[e0 + 256 * u] : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (e0 + 256 * u < total4) dst[e0 + 256 * u] = v[u];
         }
     }
     __syncthreads();
@@ -50,107 +52,111 @@ __global__ __launch_bounds__(256) void dft_rows_forward_k(const float* __restric
     const int tk = lane & 31;
     const int kh = lane >> 5;
     const int CB = C / 32;
-    for (int64_t gw = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6); gw < rows * CB; gw += (int64_t)gridDim.x * 4) {
-    const int64_t row = gw / CB;
-    const int cb = (int)(gw % CB);
-    const float* xr = x + row * (int64_t)r * C + cb * 32 + tk;
-
-    constexpr int BK = 32;
-    float xv[2][BK];
-    auto load_batch = [&](int b) {
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const float* tl = ts + kh * 32 + tk;  // step kk reads tl[64 * kk]
+    constexpr int BK = 16;
+    const int nfull = (KH - 1) / BK;  // batches whose steps all lie before the final one
+    const int nb = nfull + 1;
+    for (int64_t gw = (int64_t)blockIdx.x * 4 + wave; gw < rows * CB; gw += (int64_t)gridDim.x * 4) {
+        const int64_t row = gw / CB;
+        const int cb = (int)(gw % CB);
+        // wave-uniform row base + 32-bit lane offset: step kk reads grid points 2kk (lanes 0-31) and 2kk+1
+        const float* base = x + row * (int64_t)r * C;
+        const uint32_t voff = (uint32_t)(kh * C + cb * 32 + tk);
+        // the last step of an odd r would read point r: those lanes re-read point r-1 against a zero table row
+        const uint32_t voff_tail = (uint32_t)(min(2 * (KH - 1) + kh, r - 1) * C + cb * 32 + tk);
+        float xa[BK], ta[BK], xb[BK], tb[BK];
+        v16f acc;
 #pragma unroll
-        for (int u = 0; u < BK; ++u) {
-            const int w = min(2 * (b * BK + u) + kh, r - 1);  // rows past r meet zero table entries
-            xv[b & 1][u] = xr[(int64_t)w * C];
+        for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+        // Full batches read 2*BK grid points at compile-time offsets; the last batch holds the
+        // remaining steps and the (possibly clamped) final one.
+#define SPGT_DFT_FETCH_FULL(XV, TV, B)                                                   \
+        {                                                                                \
+            const float* xb_ = base + (int64_t)(B) * (2 * BK) * C;                       \
+            const float* tb_ = tl + (B) * (64 * BK);                                     \
+            _Pragma("unroll") for (int u = 0; u < BK; ++u) {                             \
+                XV[u] = xb_[voff + (uint32_t)(2 * u * C)];                               \
+                TV[u] = tb_[64 * u];                                                     \
+            }                                                                            \
         }
-    };
-    v16f acc;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) acc[i] = 0.f;
-    const int nb = (KH + BK - 1) / BK;
-    load_batch(0);
-    for (int b = 0; b < nb; b += 2) {
-        // two batches per trip so that the buffer index is a compile-time constant
-        if (b + 1 < nb) {
-#pragma unroll
-            for (int u = 0; u < BK; ++u) {
-                const int w = min(2 * ((b + 1) * BK + u) + kh, r - 1);
-                xv[1][u] = xr[(int64_t)w * C];
-            }
+#define SPGT_DFT_FETCH_TAIL(XV, TV)                                                      \
+        _Pragma("unroll") for (int u = 0; u < BK; ++u) {                                 \
+            const int kk = nfull * BK + u;                                               \
+            XV[u] = (kk < KH - 1) ? base[voff + (uint32_t)(2 * kk * C)] : base[voff_tail]; \
+            TV[u] = tl[64 * min(kk, KH - 1)];                                            \
         }
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int u = 0; u < BK; ++u) {
-            const int kk = b * BK + u;
-            if (kk < KH) acc = mfma32(ts[(2 * kk + kh) * 32 + tk], xv[0][u], acc);
+#define SPGT_DFT_FETCH(XV, TV, B)                                                        \
+        if ((B) < nfull) SPGT_DFT_FETCH_FULL(XV, TV, B) else { SPGT_DFT_FETCH_TAIL(XV, TV) }
+#define SPGT_DFT_MUL(XV, TV, B)                                                          \
+        if ((B) < nfull) {                                                               \
+            _Pragma("unroll") for (int u = 0; u < BK; ++u) acc = mfma32(TV[u], XV[u], acc); \
+        } else {                                                                         \
+            _Pragma("unroll") for (int u = 0; u < BK; ++u)                               \
+                if (nfull * BK + u < KH) acc = mfma32(TV[u], XV[u], acc);                \
         }
-        __builtin_amdgcn_sched_barrier(0);
-        if (b + 2 < nb) {
-#pragma unroll
-            for (int u = 0; u < BK; ++u) {
-                const int w = min(2 * ((b + 2) * BK + u) + kh, r - 1);
-                xv[0][u] = xr[(int64_t)w * C];
-            }
+        SPGT_DFT_FETCH(xa, ta, 0)
+        for (int b = 0; b < nb; b += 2) {
+            if (b + 1 < nb) { SPGT_DFT_FETCH(xb, tb, b + 1) }
+            __builtin_amdgcn_sched_barrier(0);
+            SPGT_DFT_MUL(xa, ta, b)
+            __builtin_amdgcn_sched_barrier(0);
+            if (b + 2 < nb) { SPGT_DFT_FETCH(xa, ta, b + 2) }
+            __builtin_amdgcn_sched_barrier(0);
+            if (b + 1 < nb) { SPGT_DFT_MUL(xb, tb, b + 1) }
+            __builtin_amdgcn_sched_barrier(0);
         }
-        __builtin_amdgcn_sched_barrier(0);
-        if (b + 1 < nb) {
+#undef SPGT_DFT_FETCH_FULL
+#undef SPGT_DFT_FETCH_TAIL
+#undef SPGT_DFT_FETCH
+#undef SPGT_DFT_MUL
+        // acc[r] = Y[c = cb*32 + tk][j = 8*(r/4) + 4*kh + r%4]
+        if (planar) {
+            // Y[n][j][h][c] with row = n*r + h: every store is a 128-byte run along c
+            const int64_t n = row / r;
+            const int64_t h = row - n * r;
+            float* yp = Y + (n * m2 * r + h) * (int64_t)C + cb * 32 + tk;
 #pragma unroll
-            for (int u = 0; u < BK; ++u) {
-                const int kk = (b + 1) * BK + u;
-                if (kk < KH) acc = mfma32(ts[(2 * kk + kh) * 32 + tk], xv[1][u], acc);
-            }
+            for (int q = 0; q < 4; ++q)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int j = 8 * q + 4 * kh + e;
+                    if (j < m2) yp[(int64_t)j * r * C] = acc[4 * q + e];
+                }
+        } else {
+            float* yr = Y + (row * C + cb * 32 + tk) * (int64_t)m2;
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int j = 8 * q + 4 * kh + e;
+                    if (j < m2) yr[j] = acc[4 * q + e];
+                }
         }
-        __builtin_amdgcn_sched_barrier(0);
-    }
-    // acc[r] = Y[c = cb*32 + tk][j = 8*(r/4) + 4*kh + r%4]
-    if (planar) {
-        // Y[n][j][h][c] with row = n*r + h: every store is a 128-byte run along c
-        const int64_t n = row / r;
-        const int64_t h = row - n * r;
-        float* yp = Y + (n * m2 * r + h) * (int64_t)C + cb * 32 + tk;
-#pragma unroll
-        for (int q = 0; q < 4; ++q)
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const int j = 8 * q + 4 * kh + e;
-                if (j < m2) yp[(int64_t)j * r * C] = acc[4 * q + e];
-            }
-    } else {
-        float* yr = Y + (row * C + cb * 32 + tk) * (int64_t)m2;
-#pragma unroll
-        for (int q = 0; q < 4; ++q)
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const int j = 8 * q + 4 * kh + e;
-                if (j < m2) yr[j] = acc[4 * q + e];
-            }
-    }
     }
 }
 
 // grid (workgroups), block 256; waves stride over the (row, channel block) items.
-// tab [r][m2] row-major, m2 <= 32 and even.
+// tab [32*ceil(r/32)][m2 + 1]: row w holds the m2 table entries of grid point w, zero elsewhere.
 // U [rows][C][m2] (or planar [rows/r][m2][r][C]) -> y [rows][r][C].
 __global__ __launch_bounds__(256) void dft_rows_inverse_k(const float* __restrict__ U, const float* __restrict__ tab,
                                                           float* __restrict__ y, int64_t rows, int r, int C, int m2,
                                                           int planar) {
-    extern __shared__ float ts[];  // [32 * ceil(r/32)][m2 + 1], zero beyond r rows
+    extern __shared__ float ts[];  // [32 * ceil(r/32)][m2 + 1], zero beyond r rows: a copy of `tab`
     const int pitch = m2 + 1;
     const int WT = (r + 31) / 32;
     {
-        const int total = WT * 32 * m2;
-        for (int e0 = threadIdx.x; e0 < total; e0 += 256 * 8) {
-            float v[8];
+        const int total4 = WT * 32 * pitch / 4;  // 32 * pitch is a multiple of 4
+        const float4* src = reinterpret_cast<const float4*>(tab);
+        float4* dst = reinterpret_cast<float4*>(ts);
+        for (int e0 = threadIdx.x; e0 < total4; e0 += 256 * 8) {
+            float4 v[8];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                const int e = e0 + 256 * u;
-                v[u] = (e < r * m2) ? tab[e] : 0.f;
-            }
+            for (int u = 0; u < 8; ++u)
+                v[u] = (e0 + 256 * u < total4) ? src[e0 + 256 * u] : make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                const int e = e0 + 256 * u;
-                if (e < total) ts[(e / m2) * pitch + e % m2] = v[u];
-            }
+            for (int u = 0; u < 8; ++u)
+                if (e0 + 256 * u < total4) dst[e0 + 256 * u] = v[u];
         }
     }
     __syncthreads();
@@ -369,8 +375,9 @@ int dft_rows_check(const char* who, const void* a, const void* tab, const void* 
     if (r > 1024) return fail(SPGT_ERR_INVALID_ARGUMENT, "truncated_dft_rows: r exceeds 1024");
     if (ceil_div(rows * (C / 32), (int64_t)4) > INT32_MAX)
         return fail(SPGT_ERR_INVALID_ARGUMENT, "truncated_dft_rows: too many rows");
-    if (!aligned4(a) || !aligned4(tab) || !aligned4(b))
-        return fail(SPGT_ERR_INVALID_ARGUMENT, "truncated_dft_rows: operands must be 4-byte aligned");
+    if (!aligned4(a) || !aligned16(tab) || !aligned4(b))
+        return fail(SPGT_ERR_INVALID_ARGUMENT,
+                    "truncated_dft_rows: operands must be 4-byte aligned, the table 16-byte aligned");
     (void)who;
     return SPGT_OK;
 }
@@ -386,7 +393,7 @@ extern "C" int spgt_truncated_dft_rows_forward(const float* x, const float* tabl
     const int m2 = 2 * modes;
     if (int rc = dft_rows_check("truncated_dft_rows_forward", x, table, Y, rows, r, channels, m2)) return rc;
     const size_t lds = (size_t)2 * ((r + 1) / 2) * 32 * sizeof(float);
-    auto kernel = dft_rows_forward_k;
+    auto kernel = channels == 64 ? dft_rows_forward_k<64> : (channels == 32 ? dft_rows_forward_k<32> : dft_rows_forward_k<0>);
     if (lds > 64 * 1024)
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                   (int)lds);

@@ -160,12 +160,43 @@ def _truncated_dft_rows_supported(r: int, channels: int, modes: int) -> bool:
     return bool(_lib.load().spgt_truncated_dft_rows_supported(int(r), int(channels), int(modes)))
 
 
+def pad_dft_table(table: Tensor, inverse: bool) -> Tensor:
+    """The [r, 2m] twiddle table in the zero-padded layout the row kernels keep in LDS:
+    [2*ceil(r/2), 32] for the forward kernel, [32*ceil(r/32), 2m + 1] for the inverse one."""
+    r, m2 = table.shape
+    if inverse:
+        out = table.new_zeros(((r + 31) // 32 * 32, m2 + 1))
+    else:
+        out = table.new_zeros(((r + 1) // 2 * 2, 32))
+    out[:r, :m2] = table
+    return out
+
+
+_PADDED = {}
+
+
+def _padded(table: Tensor, inverse: bool) -> Tensor:
+    key = (table.data_ptr(), table._version, tuple(table.shape), str(table.device), inverse)
+    hit = _PADDED.get(key)
+    if hit is None or hit[0]() is not table:
+        import weakref
+        if len(_PADDED) > 64:
+            _PADDED.clear()
+        hit = (weakref.ref(table), pad_dft_table(table, inverse))
+        _PADDED[key] = hit
+    return hit[1]
+
+
 def _truncated_dft_rows(src: Tensor, table: Tensor, inverse: bool, planar: bool = False) -> Tensor:
     """forward: src [..., r, C] x table [r, 2m] -> [..., C, 2m], or planar [N, 2m, r, C] from src [N, r, r, C];
-    inverse: src [..., C, 2m] (or planar [N, 2m, r, C]) -> [..., r, C]."""
+    inverse: src [..., C, 2m] (or planar [N, 2m, r, C]) -> [..., r, C].  The table is padded to the kernels'
+    layout once per table tensor."""
     require_gpu_f32("src", src)
     require_gpu_f32("table", table)
     r, m2 = table.shape
+    if m2 > 32 or m2 % 2:
+        raise ValueError("the table must have an even number of at most 32 columns")
+    padded = _padded(table, inverse)
     if inverse:
         if planar:
             if src.dim() != 4 or src.shape[1] != m2 or src.shape[2] != r:
@@ -194,7 +225,7 @@ def _truncated_dft_rows(src: Tensor, table: Tensor, inverse: bool, planar: bool 
         return out
     fn = _lib.load().spgt_truncated_dft_rows_inverse if inverse else _lib.load().spgt_truncated_dft_rows_forward
     with torch.cuda.device(src.device):
-        check(fn(ptr(src), ptr(table), ptr(out), rows, r, C, m2 // 2, int(planar), stream_of(src)))
+        check(fn(ptr(src), ptr(padded), ptr(out), rows, r, C, m2 // 2, int(planar), stream_of(src)))
     return out
 
 
