@@ -305,6 +305,25 @@ int spgt_ffn_scalar_forward(const float* x, int64_t ldx, const float* weight1_kn
                             const float* weight2, const float* bias2, int activation, float* out,
                             int64_t tokens, int in_features, int hidden_features, spgt_stream_t stream);
 
+/* 1 when spgt_encoder_tail_forward has a kernel for this shape (attn_features 128 or 136,
+ * dim_hidden 128, ffn_hidden 256), else 0. */
+int spgt_encoder_tail_supported(int attn_features, int dim_hidden, int ffn_hidden);
+
+/* Everything an encoder layer does after the attention core (Sp_EncoderLayer.forward,
+ * network/sp_layer.py:97-103, with the attention's fc_layer, network/sp_layer.py:75, and
+ * FeedForward, network/layer.py:155-174), in one launch:
+ *   y1  = x + attn_out @ fc_weight_kn + fc_bias
+ *   out = y1 + act(y1 @ ffn1_weight_kn + ffn1_bias) @ ffn2_weight_kn + ffn2_bias
+ * attn_out [tokens, attn_features] (row stride ld_attn) is the attention core's output, x and out
+ * [tokens, dim_hidden] are the residual stream before and after; the *_kn weights are the
+ * transposes of the nn.Linear weights ([in, out], contiguous).  Intermediates stay in LDS. */
+int spgt_encoder_tail_forward(const float* attn_out, int64_t ld_attn, const float* x,
+                              const float* fc_weight_kn, const float* fc_bias,
+                              const float* ffn1_weight_kn, const float* ffn1_bias,
+                              const float* ffn2_weight_kn, const float* ffn2_bias, int activation,
+                              float* out, int64_t tokens, int attn_features, int dim_hidden,
+                              int ffn_hidden, spgt_stream_t stream);
+
 /* Instrumented variant of spgt_galerkin_attention_fused_forward for benchmarks
  * (no reference counterpart): runs the call `iterations` times, synchronising
  * after each, with HIP events recorded on `stream` around each of its three

@@ -276,6 +276,142 @@ __global__ __launch_bounds__(256) void ffn_scalar_k(
     }
 }
 
+// The tail of an encoder layer after the attention core, one launch per layer
+// (Sp_EncoderLayer.forward, network/sp_layer.py:97-103, with the attention's fc_layer, :75, and
+// FeedForward, network/layer.py:155-174):
+//   y1  = x + a @ Wfc + bfc                       a = attention output [T, K1], x = residual stream [T, 128]
+//   out = y1 + act(y1 @ W1 + b1) @ W2 + b2        hidden width 256
+// A workgroup takes 32 tokens through all three products: y1 and the hidden activations live in
+// LDS (and y1 also in the registers that add it back at the end), never in HBM.  Per product a wave
+// owns 32 output columns and holds their weights in registers as the MFMA A operand, as in
+// linear_tm_k; the weights are re-read from L2 per tile, which is what three separate launches do at
+// one tile per workgroup as well.  grid (ceil(T/32)), block 256.
+template <int K1>
+__global__ __launch_bounds__(256) void encoder_tail_k(
+    const float* __restrict__ a, int64_t lda, const float* __restrict__ x, const float* __restrict__ Wfc,
+    const float* __restrict__ bfc, const float* __restrict__ W1, const float* __restrict__ b1,
+    const float* __restrict__ W2, const float* __restrict__ b2, int act, float* __restrict__ out, int64_t T) {
+    constexpr int D = 128, F = 256, TT = 32, BK = 16;
+    constexpr int PA = K1 + 1, PY = D + 1, PH = F + 1;
+    extern __shared__ float lds[];
+    float* bufA = lds;               // [TT][PA]
+    float* bufY = bufA + TT * PA;    // [TT][PY]
+    float* bufH = bufY + TT * PY;    // [TT][PH]
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int tk = lane & 31;
+    const int kh = lane >> 5;
+    const int64_t t0 = (int64_t)blockIdx.x * TT;
+    const int64_t t = t0 + tk;
+    const bool tok = t < T;
+
+    // stage the attention-output tile (coalesced 16-byte reads, scalar LDS writes at an odd pitch)
+    {
+        constexpr int NVEC = TT * K1 / 4;
+        constexpr int NLD = (NVEC + 255) / 256;
+        float4 stage[NLD];
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) {
+            const int e = threadIdx.x + 256 * i;
+            const int row = e / (K1 / 4), c4 = e % (K1 / 4);
+            stage[i] = (e < NVEC && t0 + row < T) ? *reinterpret_cast<const float4*>(a + (t0 + row) * lda + 4 * c4)
+                                                  : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) {
+            const int e = threadIdx.x + 256 * i;
+            if (e < NVEC) {
+                const int row = e / (K1 / 4), c4 = e % (K1 / 4);
+                float* d = bufA + row * PA + 4 * c4;
+                d[0] = stage[i].x; d[1] = stage[i].y; d[2] = stage[i].z; d[3] = stage[i].w;
+            }
+        }
+    }
+
+    // one product: acc[r] = sum_k src[tk][k] * W[k][n0 + 8*(r/4) + 4*kh + r%4], W [K][N] row-major
+#define SPGT_TAIL_GEMM(ACC, KK, W, N, N0, SRC, PITCH)                                            \
+    {                                                                                            \
+        constexpr int KH_ = (KK) / 2;                                                            \
+        constexpr int NB_ = (KH_ + BK - 1) / BK;                                                 \
+        float wreg_[KH_];                                                                        \
+        _Pragma("unroll") for (int kk = 0; kk < KH_; ++kk)                                       \
+            wreg_[kk] = (W)[(int64_t)(2 * kk + kh) * (N) + (N0) + tk];                           \
+        const float* xr_ = (SRC) + tk * (PITCH) + kh;                                            \
+        float xv_[2][BK];                                                                        \
+        _Pragma("unroll") for (int j = 0; j < BK; ++j) xv_[0][j] = xr_[2 * j];                   \
+        _Pragma("unroll") for (int r_ = 0; r_ < 16; ++r_) ACC[r_] = 0.f;                         \
+        _Pragma("unroll") for (int bt = 0; bt < NB_; ++bt) {                                     \
+            if (bt + 1 < NB_) {                                                                  \
+                _Pragma("unroll") for (int j = 0; j < BK; ++j)                                   \
+                    if ((bt + 1) * BK + j < KH_) xv_[(bt + 1) & 1][j] = xr_[2 * ((bt + 1) * BK + j)]; \
+            }                                                                                    \
+            __builtin_amdgcn_sched_barrier(0);                                                   \
+            _Pragma("unroll") for (int j = 0; j < BK; ++j)                                       \
+                if (bt * BK + j < KH_) ACC = mfma32(wreg_[bt * BK + j], xv_[bt & 1][j], ACC);    \
+            __builtin_amdgcn_sched_barrier(0);                                                   \
+        }                                                                                        \
+    }
+
+    // ---- y1 = x + a @ Wfc + bfc: wave w owns columns 32w .. 32w+31
+    const int n0 = wave * 32;
+    float y1[16];
+    {
+        float4 xq[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+            xq[q] = tok ? *reinterpret_cast<const float4*>(x + t * D + n0 + 4 * kh + 8 * q) : make_float4(0.f, 0.f, 0.f, 0.f);
+        __syncthreads();  // bufA complete
+        v16f acc;
+        SPGT_TAIL_GEMM(acc, K1, Wfc, D, n0, bufA, PA)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const float4 bq = *reinterpret_cast<const float4*>(bfc + n0 + 4 * kh + 8 * q);
+            y1[4 * q + 0] = acc[4 * q + 0] + bq.x + xq[q].x;
+            y1[4 * q + 1] = acc[4 * q + 1] + bq.y + xq[q].y;
+            y1[4 * q + 2] = acc[4 * q + 2] + bq.z + xq[q].z;
+            y1[4 * q + 3] = acc[4 * q + 3] + bq.w + xq[q].w;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) bufY[tk * PY + n0 + 8 * q + 4 * kh + e] = y1[4 * q + e];
+        }
+    }
+    __syncthreads();  // bufY complete
+
+    // ---- h = act(y1 @ W1 + b1): wave w owns column blocks w and w + 4 of the 8
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+        const int h0 = (wave + 4 * c) * 32;
+        v16f acc;
+        SPGT_TAIL_GEMM(acc, D, W1, F, h0, bufY, PY)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const float4 bq = *reinterpret_cast<const float4*>(b1 + h0 + 4 * kh + 8 * q);
+            const float bb[4] = {bq.x, bq.y, bq.z, bq.w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) bufH[tk * PH + h0 + 8 * q + 4 * kh + e] = activate(acc[4 * q + e] + bb[e], act);
+        }
+    }
+    __syncthreads();  // bufH complete
+
+    // ---- out = y1 + h @ W2 + b2
+    {
+        v16f acc;
+        SPGT_TAIL_GEMM(acc, F, W2, D, n0, bufH, PH)
+        if (tok) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const float4 bq = *reinterpret_cast<const float4*>(b2 + n0 + 4 * kh + 8 * q);
+                float4 o;
+                o.x = acc[4 * q + 0] + bq.x + y1[4 * q + 0];
+                o.y = acc[4 * q + 1] + bq.y + y1[4 * q + 1];
+                o.z = acc[4 * q + 2] + bq.z + y1[4 * q + 2];
+                o.w = acc[4 * q + 3] + bq.w + y1[4 * q + 3];
+                *reinterpret_cast<float4*>(out + t * D + n0 + 4 * kh + 8 * q) = o;
+            }
+        }
+    }
+#undef SPGT_TAIL_GEMM
+}
+
 namespace {
 
 // Tiles per workgroup.  A CU runs `occ` workgroups at a time; co-resident workgroups hide each
@@ -444,4 +580,50 @@ extern "C" int spgt_ffn_scalar_forward(const float* x, int64_t ldx, const float*
     else                   { if (hidden_features == 128) SPGT_FFN(128, 1); else SPGT_FFN(128, 2); }
 #undef SPGT_FFN
     return check_launch("ffn_scalar_forward");
+}
+
+extern "C" int spgt_encoder_tail_supported(int attn_features, int dim_hidden, int ffn_hidden) {
+    return ((attn_features == 128 || attn_features == 136) && dim_hidden == 128 && ffn_hidden == 256) ? 1 : 0;
+}
+
+extern "C" int spgt_encoder_tail_forward(const float* attn_out, int64_t ld_attn, const float* x,
+                                         const float* fc_weight_kn, const float* fc_bias,
+                                         const float* ffn1_weight_kn, const float* ffn1_bias,
+                                         const float* ffn2_weight_kn, const float* ffn2_bias, int activation,
+                                         float* out, int64_t tokens, int attn_features, int dim_hidden,
+                                         int ffn_hidden, hipStream_t stream) {
+    if (!attn_out || !x || !fc_weight_kn || !fc_bias || !ffn1_weight_kn || !ffn1_bias || !ffn2_weight_kn ||
+        !ffn2_bias || !out)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "encoder_tail_forward: null pointer argument");
+    if (tokens < 0) return fail(SPGT_ERR_INVALID_ARGUMENT, "encoder_tail_forward: negative token count");
+    if (!spgt_encoder_tail_supported(attn_features, dim_hidden, ffn_hidden))
+        return fail(SPGT_ERR_INVALID_ARGUMENT,
+                    "encoder_tail_forward: needs attn_features 128 or 136, dim_hidden 128, ffn_hidden 256");
+    if (activation != SPGT_ACT_NONE && activation != SPGT_ACT_RELU && activation != SPGT_ACT_SILU)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "encoder_tail_forward: unknown activation");
+    if (ld_attn < attn_features || (ld_attn & 3) || !aligned16(attn_out) || !aligned16(x) || !aligned16(out) ||
+        !aligned16(fc_bias) || !aligned16(ffn1_bias) || !aligned16(ffn2_bias) || !aligned4(fc_weight_kn) ||
+        !aligned4(ffn1_weight_kn) || !aligned4(ffn2_weight_kn))
+        return fail(SPGT_ERR_INVALID_ARGUMENT,
+                    "encoder_tail_forward: activations and biases must be 16-byte aligned, ld_attn a multiple of 4");
+    if (out == x || out == attn_out)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "encoder_tail_forward: out must not alias an input");
+    if (tokens == 0) return SPGT_OK;
+    if (ceil_div(tokens, (int64_t)32) > INT32_MAX)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "encoder_tail_forward: too many tokens");
+    const unsigned grid = (unsigned)ceil_div(tokens, (int64_t)32);
+    const size_t lds = (size_t)32 * ((attn_features + 1) + 129 + 257) * sizeof(float);
+    static const hipError_t opt136 = hipFuncSetAttribute(reinterpret_cast<const void*>(encoder_tail_k<136>),
+                                                         hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+    static const hipError_t opt128 = hipFuncSetAttribute(reinterpret_cast<const void*>(encoder_tail_k<128>),
+                                                         hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+    (void)opt136;
+    (void)opt128;
+    if (attn_features == 136)
+        hipLaunchKernelGGL(encoder_tail_k<136>, dim3(grid), dim3(256), lds, stream, attn_out, ld_attn, x, fc_weight_kn,
+                           fc_bias, ffn1_weight_kn, ffn1_bias, ffn2_weight_kn, ffn2_bias, activation, out, tokens);
+    else
+        hipLaunchKernelGGL(encoder_tail_k<128>, dim3(grid), dim3(256), lds, stream, attn_out, ld_attn, x, fc_weight_kn,
+                           fc_bias, ffn1_weight_kn, ffn1_bias, ffn2_weight_kn, ffn2_bias, activation, out, tokens);
+    return check_launch("encoder_tail_forward");
 }

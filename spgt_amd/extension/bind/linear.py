@@ -121,3 +121,38 @@ def fused_ffn_scalar(x: Tensor, weight1_kn: Tensor, bias1: Optional[Tensor], wei
             ptr(xr), ldx, ptr(weight1_kn), ptr(bias1) if bias1 is not None else None, ptr(weight2),
             ptr(bias2) if bias2 is not None else None, ACTIVATIONS[activation], ptr(out), T, K, HID, stream_of(x)))
     return out
+
+
+def encoder_tail_supported(attn_features: int, dim_hidden: int, ffn_hidden: int) -> bool:
+    """True when fused_encoder_tail has a kernel for this shape."""
+    return bool(_lib.load().spgt_encoder_tail_supported(int(attn_features), int(dim_hidden), int(ffn_hidden)))
+
+
+def fused_encoder_tail(attn_out: Tensor, x: Tensor, fc_weight_kn: Tensor, fc_bias: Tensor, ffn1_weight_kn: Tensor,
+                       ffn1_bias: Tensor, ffn2_weight_kn: Tensor, ffn2_bias: Tensor, activation: str) -> Tensor:
+    """y1 = x + attn_out @ fc_weight_kn + fc_bias;  returns y1 + act(y1 @ ffn1_weight_kn + ffn1_bias) @ ffn2_weight_kn
+    + ffn2_bias: the attention's output projection, both residual adds and the feed-forward net of an encoder layer
+    in one kernel.  attn_out [..., K1], x [..., D]; weights [in, out] contiguous."""
+    if activation not in ACTIVATIONS:
+        raise ValueError(f"activation must be one of {sorted(ACTIVATIONS)}")
+    for name, w in (("fc_weight_kn", fc_weight_kn), ("fc_bias", fc_bias), ("ffn1_weight_kn", ffn1_weight_kn),
+                    ("ffn1_bias", ffn1_bias), ("ffn2_weight_kn", ffn2_weight_kn), ("ffn2_bias", ffn2_bias)):
+        require_gpu_f32(name, w)
+    K1, D = fc_weight_kn.shape
+    F = ffn1_weight_kn.shape[1]
+    if tuple(ffn1_weight_kn.shape) != (D, F) or tuple(ffn2_weight_kn.shape) != (F, D):
+        raise ValueError("ffn weights must be [D, F] and [F, D]")
+    if fc_bias.numel() != D or ffn1_bias.numel() != F or ffn2_bias.numel() != D:
+        raise ValueError("bias sizes do not match the weights")
+    ar, T, lda = _rows("attn_out", attn_out, K1)
+    require_gpu_f32("x", x)
+    if x.shape[-1] != D or x.numel() != T * D:
+        raise ValueError("x must be [..., D] with as many rows as attn_out")
+    out = torch.empty_like(x)
+    if T == 0:
+        return out
+    with torch.cuda.device(x.device):
+        check(_lib.load().spgt_encoder_tail_forward(
+            ptr(ar), lda, ptr(x), ptr(fc_weight_kn), ptr(fc_bias), ptr(ffn1_weight_kn), ptr(ffn1_bias),
+            ptr(ffn2_weight_kn), ptr(ffn2_bias), ACTIVATIONS[activation], ptr(out), T, K1, D, F, stream_of(x)))
+    return out

@@ -30,9 +30,9 @@ from ..extension.bind.galerkin_attention import (galerkin_attention_fused, multi
                                                  multihead_projection_layernorm_with_position_rrc_cuda,
                                                  multihead_projection_with_position_rrc_cuda)
 from . import truncated_dft
-from ..extension.bind.linear import fused_linear
-from .layer import (FeedForward, activation_name, always_dropout, fused_linear_usable, linear_weight_kn,
-                    make_activation)
+from ..extension.bind.linear import encoder_tail_supported, fused_encoder_tail, fused_linear
+from .layer import (FeedForward, activation_name, always_dropout, fused_linear_usable, gpu_inference,
+                    linear_weight_kn, make_activation)
 
 
 class Sp_GalerkinAttention(nn.Module):
@@ -87,6 +87,10 @@ class Sp_GalerkinAttention(nn.Module):
     def forward(self, Q: Tensor, K: Tensor, V: Tensor, position: Tensor, residual: Tensor = None) -> Tensor:
         """Q, K, V [N, seqlen, dim_hidden], position [N, seqlen, dim_position] -> [N, seqlen, dim_hidden];
         with `residual` the result is residual + attention(Q, K, V)."""
+        return self.project(self.attend(Q, K, V, position), residual)
+
+    def attend(self, Q: Tensor, K: Tensor, V: Tensor, position: Tensor) -> Tensor:
+        """The attention core before fc_layer: [N, seqlen, num_head * (dim_position + dim_head)]."""
         N, seqlen, C = Q.size()
         H, dp = self.num_head, self.dim_position
         if self._needs_graph(Q, K, V):
@@ -112,6 +116,10 @@ class Sp_GalerkinAttention(nn.Module):
             pos = position.contiguous() if dp else None
             X = galerkin_attention_fused(q, k, v, pos, self.ln_weight_K.detach(), self.ln_bias_K.detach(),
                                          self.ln_weight_V.detach(), self.ln_bias_V.detach(), self.norm_eps, H, dp)
+        return X
+
+    def project(self, X: Tensor, residual: Tensor = None) -> Tensor:
+        """fc_layer (+ dropout) on the attention core's output, plus the residual when given."""
         if fused_linear_usable(X, self.fc_layer) and (residual is None or self.fc_droprate == 0):
             Y = fused_linear(X, linear_weight_kn(self.fc_layer), self.fc_layer.bias, "none", residual)
             return always_dropout(Y, self.fc_droprate)
@@ -130,6 +138,15 @@ class Sp_EncoderLayer(nn.Module):
         self.ffn_layer = FeedForward(dim_hidden, dim_hidden, ffn_dim_hidden, ffn_droprate, ffn_activation)
 
     def forward(self, X: Tensor, position: Tensor) -> Tensor:
+        att, ffn = self.attention_layer, self.ffn_layer
+        if (att.fc_droprate == 0 and ffn.droprate == 0 and gpu_inference(X, *self.parameters()) and
+                encoder_tail_supported(att.fc_layer.in_features, att.fc_layer.out_features, ffn.layer1.out_features)
+                and ffn.layer2.out_features == att.fc_layer.out_features):
+            # output projection, both residual adds and the feed-forward net in one launch
+            A = att.attend(X, X, X, position)
+            return fused_encoder_tail(A, X.contiguous(), linear_weight_kn(att.fc_layer), att.fc_layer.bias,
+                                      linear_weight_kn(ffn.layer1), ffn.layer1.bias, linear_weight_kn(ffn.layer2),
+                                      ffn.layer2.bias, activation_name(ffn.activation_layer))
         X = self.attention_layer(X, X, X, position, residual=X)
         return self.ffn_layer(X, residual=X)
 

@@ -162,3 +162,24 @@ def test_feedforward_module_scalar_head(gpu):
         got = ffn(x)
     assert got.shape == want.shape
     assert (got - want).abs().max().item() <= 1e-5 * max(1.0, want.abs().max().item())
+
+
+@pytest.mark.parametrize("K1", [128, 136])
+@pytest.mark.parametrize("T", [1, 33, 5041])
+@pytest.mark.parametrize("act", ["relu", "silu"])
+def test_encoder_tail(gpu, K1, T, act):
+    """fc_layer + residual + FeedForward + residual (network/sp_layer.py:75, 97-103; network/layer.py:155-174)
+    in one kernel, against the same chain in float64."""
+    from spgt_amd.extension.bind.linear import encoder_tail_supported, fused_encoder_tail
+    assert encoder_tail_supported(K1, 128, 256) and not encoder_tail_supported(K1, 128, 512)
+    g = torch.Generator().manual_seed(K1 + T)
+    a = torch.randn(T, K1, generator=g)
+    x = torch.randn(T, 128, generator=g)
+    wfc, bfc = torch.randn(K1, 128, generator=g) / K1 ** 0.5, torch.randn(128, generator=g)
+    w1, b1 = torch.randn(128, 256, generator=g) / 128 ** 0.5, torch.randn(256, generator=g)
+    w2, b2 = torch.randn(256, 128, generator=g) / 16.0, torch.randn(128, generator=g)
+    got = fused_encoder_tail(*[v.to(gpu) for v in (a, x, wfc, bfc, w1, b1, w2, b2)], act).cpu().double()
+    y1 = x.double() + a.double() @ wfc.double() + bfc.double()
+    want = y1 + _expected(y1, w1, b1, act, None, False) @ w2.double() + b2.double()
+    assert got.shape == want.shape
+    assert (got - want).abs().max().item() <= 2e-5 * max(1.0, want.abs().max().item())
