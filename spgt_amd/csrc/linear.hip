@@ -62,7 +62,7 @@ __global__ __launch_bounds__(256) void linear_tm_k(
     // A operand: W[2kk + kh][n0 + tk]
     float wreg[KH];
 #pragma unroll
-    for (int kk = 0; kk < KH; ++kk) wreg[kk] = W[(int64_t)(2 * kk + kh) * ldw + n0 + tk];
+    for (int kk = 0; kk < KH; ++kk) wreg[kk] = (W + (int64_t)(2 * kk) * ldw)[(uint32_t)(kh * ldw + n0 + tk)];
     // accumulator element r holds column n0 + 8*(r/4) + 4*kh + r%4
     float breg[16];
 #pragma unroll
@@ -191,7 +191,7 @@ __global__ __launch_bounds__(256) void ffn_scalar_k(
     for (int c = 0; c < CBW; ++c) {
         const int n0 = 32 * (wave + 4 * c);
 #pragma unroll
-        for (int kk = 0; kk < KH; ++kk) wreg[c][kk] = W1[(int64_t)(2 * kk + kh) * HID + n0 + tk];
+        for (int kk = 0; kk < KH; ++kk) wreg[c][kk] = (W1 + (int64_t)(2 * kk) * HID)[(uint32_t)(kh * HID + n0 + tk)];
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
             const int n = n0 + 8 * (r >> 2) + 4 * kh + (r & 3);
@@ -287,7 +287,7 @@ __global__ __launch_bounds__(256) void ffn_scalar_k(
 // linear_tm_k; the weights are re-read from L2 per tile, which is what three separate launches do at
 // one tile per workgroup as well.  grid (ceil(T/32)), block 256.
 template <int K1>
-__global__ __launch_bounds__(256) void encoder_tail_k(
+__global__ __launch_bounds__(256, 2) void encoder_tail_k(
     const float* __restrict__ a, int64_t lda, const float* __restrict__ x, const float* __restrict__ Wfc,
     const float* __restrict__ bfc, const float* __restrict__ W1, const float* __restrict__ b1,
     const float* __restrict__ W2, const float* __restrict__ b2, int act, float* __restrict__ out, int64_t T) {
@@ -328,18 +328,21 @@ __global__ __launch_bounds__(256) void encoder_tail_k(
         }
     }
 
-    // one product: acc[r] = sum_k src[tk][k] * W[k][n0 + 8*(r/4) + 4*kh + r%4], W [K][N] row-major
-#define SPGT_TAIL_GEMM(ACC, KK, W, N, N0, SRC, PITCH)                                            \
+    // Weights of one product for this wave: WR[kk] = W[K0 + 2kk + kh][N0 + tk], W [.][N] row-major
+    // (wave-uniform row base + one 32-bit lane offset, so the loads need no per-load address registers).
+#define SPGT_TAIL_LOADW(WR, KK, W, N, N0, K0)                                                    \
+    __builtin_amdgcn_sched_barrier(0);                                                           \
+    _Pragma("unroll") for (int kk = 0; kk < (KK) / 2; ++kk)                                      \
+        WR[kk] = ((W) + (int64_t)((K0) + 2 * kk) * (N))[(uint32_t)(kh * (N) + (N0) + tk)];       \
+    __builtin_amdgcn_sched_barrier(0);
+    // ACC[r] += sum_k SRC[tk][k] * (weights in WR), k < KK; operands are read from LDS a batch ahead.
+#define SPGT_TAIL_MMA(ACC, WR, KK, SRC, PITCH)                                                   \
     {                                                                                            \
         constexpr int KH_ = (KK) / 2;                                                            \
         constexpr int NB_ = (KH_ + BK - 1) / BK;                                                 \
-        float wreg_[KH_];                                                                        \
-        _Pragma("unroll") for (int kk = 0; kk < KH_; ++kk)                                       \
-            wreg_[kk] = (W)[(int64_t)(2 * kk + kh) * (N) + (N0) + tk];                           \
         const float* xr_ = (SRC) + tk * (PITCH) + kh;                                            \
         float xv_[2][BK];                                                                        \
         _Pragma("unroll") for (int j = 0; j < BK; ++j) xv_[0][j] = xr_[2 * j];                   \
-        _Pragma("unroll") for (int r_ = 0; r_ < 16; ++r_) ACC[r_] = 0.f;                         \
         _Pragma("unroll") for (int bt = 0; bt < NB_; ++bt) {                                     \
             if (bt + 1 < NB_) {                                                                  \
                 _Pragma("unroll") for (int j = 0; j < BK; ++j)                                   \
@@ -347,22 +350,29 @@ __global__ __launch_bounds__(256) void encoder_tail_k(
             }                                                                                    \
             __builtin_amdgcn_sched_barrier(0);                                                   \
             _Pragma("unroll") for (int j = 0; j < BK; ++j)                                       \
-                if (bt * BK + j < KH_) ACC = mfma32(wreg_[bt * BK + j], xv_[bt & 1][j], ACC);    \
+                if (bt * BK + j < KH_) ACC = mfma32(WR[bt * BK + j], xv_[bt & 1][j], ACC);       \
             __builtin_amdgcn_sched_barrier(0);                                                   \
         }                                                                                        \
     }
+#define SPGT_TAIL_ZERO(ACC) _Pragma("unroll") for (int r_ = 0; r_ < 16; ++r_) ACC[r_] = 0.f;
 
-    // ---- y1 = x + a @ Wfc + bfc: wave w owns columns 32w .. 32w+31
+    // The weights of each product are requested before the MFMAs of the product ahead of it, so
+    // that their trip from L2 is hidden: wA/wB/wC/wD/wE are live two at a time.
     const int n0 = wave * 32;
+    float wA[K1 / 2], wB[D / 2], wC[D / 2], wD[D / 2], wE[D / 2];
+    SPGT_TAIL_LOADW(wA, K1, Wfc, D, n0, 0)
     float y1[16];
+    // ---- y1 = x + a @ Wfc + bfc: wave w owns columns 32w .. 32w+31
     {
         float4 xq[4];
 #pragma unroll
         for (int q = 0; q < 4; ++q)
             xq[q] = tok ? *reinterpret_cast<const float4*>(x + t * D + n0 + 4 * kh + 8 * q) : make_float4(0.f, 0.f, 0.f, 0.f);
         __syncthreads();  // bufA complete
+        SPGT_TAIL_LOADW(wB, D, W1, F, n0, 0)  // first hidden column block of this wave
         v16f acc;
-        SPGT_TAIL_GEMM(acc, K1, Wfc, D, n0, bufA, PA)
+        SPGT_TAIL_ZERO(acc)
+        SPGT_TAIL_MMA(acc, wA, K1, bufA, PA)
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
             const float4 bq = *reinterpret_cast<const float4*>(bfc + n0 + 4 * kh + 8 * q);
@@ -376,12 +386,8 @@ __global__ __launch_bounds__(256) void encoder_tail_k(
     }
     __syncthreads();  // bufY complete
 
-    // ---- h = act(y1 @ W1 + b1): wave w owns column blocks w and w + 4 of the 8
-#pragma unroll
-    for (int c = 0; c < 2; ++c) {
-        const int h0 = (wave + 4 * c) * 32;
-        v16f acc;
-        SPGT_TAIL_GEMM(acc, D, W1, F, h0, bufY, PY)
+    // ---- h = act(y1 @ W1 + b1): wave w owns hidden column blocks w and w + 4 of the 8
+    auto store_hidden = [&](const v16f& acc, int h0) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
             const float4 bq = *reinterpret_cast<const float4*>(b1 + h0 + 4 * kh + 8 * q);
@@ -389,13 +395,30 @@ __global__ __launch_bounds__(256) void encoder_tail_k(
 #pragma unroll
             for (int e = 0; e < 4; ++e) bufH[tk * PH + h0 + 8 * q + 4 * kh + e] = activate(acc[4 * q + e] + bb[e], act);
         }
+    };
+    {
+        SPGT_TAIL_LOADW(wC, D, W1, F, n0 + 128, 0)  // second hidden column block
+        v16f acc;
+        SPGT_TAIL_ZERO(acc)
+        SPGT_TAIL_MMA(acc, wB, D, bufY, PY)
+        store_hidden(acc, n0);
+    }
+    {
+        SPGT_TAIL_LOADW(wD, D, W2, D, n0, 0)  // rows 0..127 of W2 for the last product
+        v16f acc;
+        SPGT_TAIL_ZERO(acc)
+        SPGT_TAIL_MMA(acc, wC, D, bufY, PY)
+        store_hidden(acc, n0 + 128);
     }
     __syncthreads();  // bufH complete
 
     // ---- out = y1 + h @ W2 + b2
     {
+        SPGT_TAIL_LOADW(wE, D, W2, D, n0, 128)  // rows 128..255
         v16f acc;
-        SPGT_TAIL_GEMM(acc, F, W2, D, n0, bufH, PH)
+        SPGT_TAIL_ZERO(acc)
+        SPGT_TAIL_MMA(acc, wD, D, bufH, PH)
+        SPGT_TAIL_MMA(acc, wE, D, bufH + 128, PH)
         if (tok) {
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
@@ -409,7 +432,9 @@ __global__ __launch_bounds__(256) void encoder_tail_k(
             }
         }
     }
-#undef SPGT_TAIL_GEMM
+#undef SPGT_TAIL_LOADW
+#undef SPGT_TAIL_MMA
+#undef SPGT_TAIL_ZERO
 }
 
 namespace {
