@@ -256,6 +256,18 @@ int spgt_bilinear_resample(const float* src, const float* pre_bias, float* dst, 
                            int pre_activation, int pre_activation_count, int post_activation,
                            spgt_stream_t stream);
 
+/* 1 when spgt_conv3x3_resample serves this number of input channels (1..4), else 0. */
+int spgt_conv3x3_resample_supported(int Cin);
+
+/* DownScaler2D's first stage (network/model.py:30-33: conv0 = ConvResBlock2D(in_dim, out_dim, 3, 1),
+ * bilinear interpolation to resolution_size[1], activation) for a few input channels, one pass:
+ *   out[n, c] = post_activation(interpolate(pre_activation(conv3x3(x, weight, padding 1)[n, c] + bias[c])))
+ * x [N, H_in, W_in, Cin] channels-last (the model's input layout), weight [Cout, Cin, 3, 3], bias
+ * [Cout] or null, out [N, Cout, H_out, W_out]; align_corners=True as in the reference. */
+int spgt_conv3x3_resample(const float* x, const float* weight, const float* bias, float* out, int N, int Cin,
+                          int Cout, int H_in, int W_in, int H_out, int W_out, int pre_activation,
+                          int post_activation, spgt_stream_t stream);
+
 /* The tail of ConvResBlock2D (network/layer.py:7-24) after a bias-free convolution, and the
  * scaler's own activation where it follows directly (network/model.py:61-62), in place:
  * x[n, c, :] = activation^activation_count(x[n, c, :] + bias[c]) on x [N, C, HW]; bias may be null,

@@ -53,6 +53,8 @@ SIGNATURES = {
     "spgt_spectral_modes_middle_supported": (_i, [_i, _i, _i, _i]),
     "spgt_spectral_modes_middle_workspace_bytes": (_sz, [_i, _i, _i]),
     "spgt_spectral_modes_middle": (_i, [_p, _p, _p, _p, _p, _p, _p, _sz, _i, _i, _i, _i, _i, _p]),
+    "spgt_conv3x3_resample_supported": (_i, [_i]),
+    "spgt_conv3x3_resample": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p]),
     "spgt_linear_supported": (_i, [_i, _i]),
     "spgt_linear_forward": (_i, [_p, _i64, _p, _p, _p, _i64, _i, _i, _p, _i64, _p, _i, _p, _i64, _i, _i64, _i64, _i, _i,
                                  _p]),

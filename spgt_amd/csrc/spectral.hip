@@ -279,6 +279,74 @@ __global__ __launch_bounds__(256) void bilinear_align_corners_from_nhwc_k(const 
     }
 }
 
+// DownScaler2D's first stage in one pass for a few input channels (network/model.py:30-33:
+// conv0 = ConvResBlock2D(in_dim, out_dim, 3x3, padding 1), interpolate to resolution_size[1],
+// activation): out[n, c, oy, ox] = post(bilinear(pre(conv3x3(x)[n, c] + bias[c]))).  The four
+// convolution outputs an output pixel blends need a 4x4 input patch per input channel, which the
+// thread keeps in registers while it walks the output channels (weights are wave-uniform), so the
+// full-resolution convolution output (91 MB at the Darcy shape) never exists.
+// x [N, H, W, CIN] channels-last, weight [Cout, CIN, 3, 3], out [N, Cout, Hout, Wout].
+// grid (ceil(Wout/64), Hout, N), block (64, 4): threadIdx.y walks the output channels 4 apart.
+template <int CIN>
+__global__ __launch_bounds__(256) void conv3x3_resample_k(const float* __restrict__ x,
+                                                          const float* __restrict__ weight,
+                                                          const float* __restrict__ bias, float* __restrict__ out,
+                                                          int Cout, int H, int W, int Hout, int Wout, float hscale,
+                                                          float wscale, ResampleAct act) {
+    const int ox = blockIdx.x * 64 + threadIdx.x;
+    const int oy = blockIdx.y;
+    const int64_t n = blockIdx.z;
+    const int oxc = min(ox, Wout - 1);
+    const float hr = hscale * (float)oy;
+    const int h1 = (int)hr;
+    const int hp = (h1 < H - 1) ? 1 : 0;
+    const float h1l = hr - (float)h1;
+    const float h0l = 1.0f - h1l;
+    const float wr = wscale * (float)oxc;
+    const int w1 = (int)wr;
+    const int wp = (w1 < W - 1) ? 1 : 0;
+    const float w1l = wr - (float)w1;
+    const float w0l = 1.0f - w1l;
+    // patch[ci][dy][dx] = x[n, h1 - 1 + dy, w1 - 1 + dx, ci], zero outside the image
+    float patch[CIN][4][4];
+#pragma unroll
+    for (int dy = 0; dy < 4; ++dy)
+#pragma unroll
+        for (int dx = 0; dx < 4; ++dx) {
+            const int yy = h1 - 1 + dy, xx = w1 - 1 + dx;
+            const bool in = yy >= 0 && yy < H && xx >= 0 && xx < W;
+            const float* px = x + ((n * H + min(max(yy, 0), H - 1)) * (int64_t)W + min(max(xx, 0), W - 1)) * CIN;
+#pragma unroll
+            for (int ci = 0; ci < CIN; ++ci) patch[ci][dy][dx] = in ? px[ci] : 0.f;
+        }
+    const int wave_c = __builtin_amdgcn_readfirstlane(threadIdx.y);
+    for (int c = wave_c; c < Cout; c += 4) {
+        const float* wc = weight + (int64_t)c * CIN * 9;
+        const float b = bias ? bias[c] : 0.f;
+        float v00 = b, v01 = b, v10 = b, v11 = b;  // conv at (h1, w1), (h1, w1+wp), (h1+hp, w1), (h1+hp, w1+wp)
+#pragma unroll
+        for (int ci = 0; ci < CIN; ++ci)
+#pragma unroll
+            for (int ky = 0; ky < 3; ++ky)
+#pragma unroll
+                for (int kx = 0; kx < 3; ++kx) {
+                    const float wv = wc[ci * 9 + ky * 3 + kx];
+                    v00 = fmaf(wv, patch[ci][ky][kx], v00);
+                    v01 = fmaf(wv, patch[ci][ky][kx + 1], v01);
+                    v10 = fmaf(wv, patch[ci][ky + 1][kx], v10);
+                    v11 = fmaf(wv, patch[ci][ky + 1][kx + 1], v11);
+                }
+        // at the last row / column (hp or wp = 0) the second sample is the first one again
+        const float s00 = act_pre<true>(v00, 0.f, act);
+        const float s01 = act_pre<true>(wp ? v01 : v00, 0.f, act);
+        const float s10 = act_pre<true>(hp ? v10 : v00, 0.f, act);
+        const float s11 = act_pre<true>(hp ? (wp ? v11 : v10) : (wp ? v01 : v00), 0.f, act);
+        const float top = w0l * s00 + w1l * s01;
+        const float bot = w0l * s10 + w1l * s11;
+        if (ox < Wout) out[((n * Cout + c) * Hout + oy) * (int64_t)Wout + ox] = act_apply(h0l * top + h1l * bot, act.post);
+    }
+}
+
 // x[n, c, :] = act^count(x[n, c, :] + bias[c]) in place on [planes = N*C, HW]: the bias add and the
 // activation(s) that follow a bias-free convolution.  grid (chunks, planes), block 256.
 __global__ __launch_bounds__(256) void bias_activation_nchw_k(float* __restrict__ x, const float* __restrict__ bias,
@@ -435,4 +503,36 @@ extern "C" int spgt_bias_activation_nchw(float* x, const float* bias, int N, int
     hipLaunchKernelGGL(bias_activation_nchw_k, dim3(chunks, N * C), dim3(256), 0, stream, x, bias, C, HW, activation,
                        activation == SPGT_ACT_NONE ? 0 : activation_count);
     return check_launch("bias_activation_nchw");
+}
+
+extern "C" int spgt_conv3x3_resample_supported(int Cin) { return (Cin >= 1 && Cin <= 4) ? 1 : 0; }
+
+extern "C" int spgt_conv3x3_resample(const float* x, const float* weight, const float* bias, float* out, int N,
+                                     int Cin, int Cout, int H_in, int W_in, int H_out, int W_out, int pre_activation,
+                                     int post_activation, hipStream_t stream) {
+    if (!x || !weight || !out) return fail(SPGT_ERR_INVALID_ARGUMENT, "conv3x3_resample: null pointer argument");
+    if (N <= 0 || Cout <= 0 || H_in <= 0 || W_in <= 0 || H_out <= 0 || W_out <= 0)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "conv3x3_resample: sizes must be positive");
+    if (!spgt_conv3x3_resample_supported(Cin))
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "conv3x3_resample: 1 to 4 input channels");
+    if (H_out > 65535 || N > 65535) return fail(SPGT_ERR_INVALID_ARGUMENT, "conv3x3_resample: N or H_out exceeds 65535");
+    if (!act_known(pre_activation) || !act_known(post_activation))
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "conv3x3_resample: unknown activation");
+    if (!aligned4(x) || !aligned4(weight) || !aligned4(out) || (bias && !aligned4(bias)))
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "conv3x3_resample: operands must be 4-byte aligned");
+    const float hscale = H_out > 1 ? (float)(H_in - 1) / (float)(H_out - 1) : 0.f;
+    const float wscale = W_out > 1 ? (float)(W_in - 1) / (float)(W_out - 1) : 0.f;
+    const ResampleAct act{pre_activation, pre_activation == SPGT_ACT_NONE ? 0 : 1, post_activation};
+    const dim3 grid(ceil_div(W_out, 64), H_out, N), block(64, 4);
+#define SPGT_CONV(CI)                                                                                                \
+    hipLaunchKernelGGL(conv3x3_resample_k<CI>, grid, block, 0, stream, x, weight, bias, out, Cout, H_in, W_in, H_out, \
+                       W_out, hscale, wscale, act)
+    switch (Cin) {
+        case 1: SPGT_CONV(1); break;
+        case 2: SPGT_CONV(2); break;
+        case 3: SPGT_CONV(3); break;
+        default: SPGT_CONV(4); break;
+    }
+#undef SPGT_CONV
+    return check_launch("conv3x3_resample");
 }

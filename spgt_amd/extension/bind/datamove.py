@@ -318,7 +318,34 @@ def _bias_activation_nchw_(X: Tensor, bias, activation=None, count: int = 1) -> 
     return X
 
 
+def _conv3x3_resample(X: Tensor, weight: Tensor, bias, size, pre_activation=None, post_activation=None) -> Tensor:
+    """post(interpolate(pre(conv3x3(X, weight, padding=1) + bias))) for X [N, H, W, Cin] channels-last with
+    Cin <= 4: [N, Cout, H', W'] without the full-resolution convolution output ever being stored."""
+    require_gpu_f32("X", X)
+    require_gpu_f32("weight", weight)
+    if X.dim() != 4 or weight.dim() != 4 or tuple(weight.shape[2:]) != (3, 3) or weight.shape[1] != X.shape[3]:
+        raise ValueError("X must be [N, H, W, Cin] and weight [Cout, Cin, 3, 3]")
+    if pre_activation not in _ACT or post_activation not in _ACT:
+        raise ValueError("activations must be None, 'none', 'relu' or 'silu'")
+    N, H, W, Cin = X.shape
+    Cout = weight.shape[0]
+    if bias is not None:
+        require_gpu_f32("bias", bias)
+        if bias.numel() != Cout:
+            raise ValueError(f"bias has {bias.numel()} elements, expected {Cout}")
+    H_out, W_out = (size, size) if isinstance(size, int) else tuple(size)
+    out = torch.empty((N, Cout, H_out, W_out), dtype=X.dtype, device=X.device)
+    if out.numel() == 0:
+        return out
+    with torch.cuda.device(X.device):
+        check(_lib.load().spgt_conv3x3_resample(ptr(X), ptr(weight), ptr(bias) if bias is not None else None, ptr(out),
+                                                N, Cin, Cout, H, W, H_out, W_out, _ACT[pre_activation],
+                                                _ACT[post_activation], stream_of(X)))
+    return out
+
+
 dexts = SimpleNamespace(
+    conv3x3_resample=_conv3x3_resample,
     truncated_dft_rows_supported=_truncated_dft_rows_supported,
     truncated_dft_rows=_truncated_dft_rows,
     spectral_modes_middle_supported=_spectral_modes_middle_supported,
@@ -454,3 +481,15 @@ def spectral_modes_middle(Y: Tensor, table_h: Tensor, table_h_inverse: Tensor, w
     """DFT along h onto the kept rows, mode-wise complex channel contraction, inverse DFT along h, on the
     planar operands of the row kernels (inference only)."""
     return dexts.spectral_modes_middle(Y.detach(), table_h, table_h_inverse, weight_1.detach(), weight_2.detach())
+
+
+def conv3x3_resample_supported(cin: int) -> bool:
+    """True when conv3x3_resample has a kernel for this number of input channels."""
+    return bool(_lib.load().spgt_conv3x3_resample_supported(int(cin)))
+
+
+def conv3x3_resample(X: Tensor, weight: Tensor, bias, size, pre_activation=None, post_activation=None) -> Tensor:
+    """3x3 convolution (padding 1) of a channels-last input with few channels, bias, activation, bilinear
+    align_corners resampling and a second activation in one pass: [N, H, W, Cin] -> [N, Cout, H', W'] (inference only)."""
+    return dexts.conv3x3_resample(X.detach(), weight.detach(), None if bias is None else bias.detach(), size,
+                                  pre_activation, post_activation)

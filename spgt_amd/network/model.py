@@ -7,7 +7,8 @@ import torch
 import torch.nn.functional as F
 from torch import Tensor, nn
 
-from ..extension.bind.datamove import bilinear_align_corners, bilinear_align_corners_nhwc, bilinear_resample
+from ..extension.bind.datamove import (bilinear_align_corners, bilinear_align_corners_nhwc, bilinear_resample,
+                                       conv3x3_resample, conv3x3_resample_supported)
 from .layer import ConvResBlock2D, activation_name, always_dropout, gpu_inference, make_activation
 
 
@@ -51,13 +52,20 @@ class DownScaler2D(nn.Module):
     def forward(self, X: Tensor) -> Tensor:
         fused = gpu_inference(X, *self.parameters())
         act = activation_name(self.activation_layer)
-        X = nhwc_to_nchw(X)
-        if fused and self.conv0.fusable(X):
+        c0 = self.conv0.conv_layer
+        if (fused and self.conv0.fusable(X) and conv3x3_resample_supported(X.size(-1)) and c0.kernel_size == (3, 3) and
+                c0.padding == (1, 1) and c0.stride == (1, 1) and c0.dilation == (1, 1) and c0.groups == 1):
+            # few input channels: convolution, bias, activation, resampling and the scaler's activation in one
+            # pass straight from the channels-last input; the full-resolution convolution output is never stored
+            X = conv3x3_resample(X.contiguous(), c0.weight, c0.bias, self.resolution_size[1],
+                                 pre_activation=activation_name(self.conv0.activation_layer), post_activation=act)
+        elif fused and self.conv0.fusable(X):
+            X = nhwc_to_nchw(X)
             # conv0's bias and activation, the resampling and the scaler's activation in one pass
             X = bilinear_resample(self.conv0.conv_raw(X), self.resolution_size[1], pre_bias=self.conv0.conv_layer.bias,
                                   pre_activation=activation_name(self.conv0.activation_layer), post_activation=act)
         else:
-            X = self.activation_layer(resample(self.conv0(X), self.resolution_size[1]))
+            X = self.activation_layer(resample(self.conv0(nhwc_to_nchw(X)), self.resolution_size[1]))
         X1 = self.conv1(X)
         X2 = self.conv2(X1)
         X3 = self.conv3(X2)

@@ -344,3 +344,22 @@ def test_truncated_dft_rows_planar_layout(gpu):
     c = dm.truncated_dft_rows_inverse(u, fwi.to(gpu), planar=True)
     d = dm.truncated_dft_rows_inverse(u.permute(0, 2, 3, 1).contiguous().view(66, 64, 16), fwi.to(gpu)).view(2, 33, 33, 64)
     assert torch.equal(c, d)
+
+
+@pytest.mark.parametrize("N,H,W,cin,cout,size", [(2, 21, 21, 1, 128, (15, 15)), (1, 9, 13, 3, 20, (17, 5)), (2, 33, 33, 4, 7, (33, 33)),
+                                                 (1, 211, 211, 1, 128, (122, 122)), (1, 5, 5, 2, 3, (1, 1))])
+@pytest.mark.parametrize("pre,post", [("silu", "silu"), ("relu", None), (None, None)])
+def test_conv3x3_resample(gpu, N, H, W, cin, cout, size, pre, post):
+    """conv3x3 (padding 1) + bias + activation + bilinear resampling + activation in one pass
+    (network/model.py:30-33 with network/layer.py:7-24) against torch's float64 conv2d and the oracle resampling."""
+    x = rnd(N, H, W, cin, seed=101)
+    w = rnd(cout, cin, 3, 3, seed=102) / 3.0
+    b = rnd(cout, seed=103)
+    conv = F.conv2d(x.permute(0, 3, 1, 2).double(), w.double(), b.double(), padding=1)
+    want = _act64(O.bilinear_align_corners(_act64(conv, pre), size), post)
+    assert dm.conv3x3_resample_supported(cin) and not dm.conv3x3_resample_supported(5)
+    got = dm.conv3x3_resample(x.to(gpu), w.to(gpu), b.to(gpu), size, pre, post).cpu().double()
+    assert got.shape == want.shape
+    # fp32 source coordinates (as torch's own kernel computes them) times the slope of a random convolution
+    # output reach 1e-5 of the output scale at 211 -> 122; the bound is 3e-5, far inside the path's 1e-4
+    assert (got - want).abs().max().item() <= 3e-5 * max(1.0, want.abs().max().item())
