@@ -135,8 +135,11 @@ def darcy_bench(dev, with_cpu, steps=30):
         torch.cuda.synchronize()
         ms = (time.perf_counter() - t0) / steps * 1e3
         graph_equal = bool(torch.equal(gout, out))
+    graph_ms = ms
+    ms = min(graph_ms, eager_ms)
     res = {"ms_per_forward": round(ms, 3), "samples_per_s": round(B / ms * 1e3, 1), "batch": B,
-           "mode": "HIP graph replay of the forward (input copy included)", "eager_ms_per_forward": round(eager_ms, 3),
+           "mode": "faster of eager launches and HIP graph replay (input copy included)",
+           "eager_ms_per_forward": round(eager_ms, 3), "graph_ms_per_forward": round(graph_ms, 3),
            "graph_output_equals_eager": graph_equal,
            "config": "r=211 -> 122 -> 71, 4 encoder layers (d_model 128, 4 heads, dp 2, FFN 256), "
                      "2 FNO blocks (width 64, 12 modes), random init, drop rates 0"}

@@ -319,10 +319,17 @@ __global__ __launch_bounds__(256) void conv3x3_resample_k(const float* __restric
 #pragma unroll
             for (int ci = 0; ci < CIN; ++ci) patch[ci][dy][dx] = in ? px[ci] : 0.f;
         }
+    // weights and biases of all output channels go through LDS once per workgroup (broadcast reads)
+    extern __shared__ float wlds[];  // [Cout][CIN*9] then [Cout]
+    float* blds = wlds + Cout * CIN * 9;
+    const int tid = threadIdx.y * 64 + threadIdx.x;
+    for (int e = tid; e < Cout * CIN * 9; e += 256) wlds[e] = weight[e];
+    for (int e = tid; e < Cout; e += 256) blds[e] = bias ? bias[e] : 0.f;
+    __syncthreads();
     const int wave_c = __builtin_amdgcn_readfirstlane(threadIdx.y);
     for (int c = wave_c; c < Cout; c += 4) {
-        const float* wc = weight + (int64_t)c * CIN * 9;
-        const float b = bias ? bias[c] : 0.f;
+        const float* wc = wlds + c * CIN * 9;
+        const float b = blds[c];
         float v00 = b, v01 = b, v10 = b, v11 = b;  // conv at (h1, w1), (h1, w1+wp), (h1+hp, w1), (h1+hp, w1+wp)
 #pragma unroll
         for (int ci = 0; ci < CIN; ++ci)
@@ -524,9 +531,11 @@ extern "C" int spgt_conv3x3_resample(const float* x, const float* weight, const 
     const float wscale = W_out > 1 ? (float)(W_in - 1) / (float)(W_out - 1) : 0.f;
     const ResampleAct act{pre_activation, pre_activation == SPGT_ACT_NONE ? 0 : 1, post_activation};
     const dim3 grid(ceil_div(W_out, 64), H_out, N), block(64, 4);
+    const size_t lds = (size_t)Cout * (Cin * 9 + 1) * sizeof(float);
+    if (lds > 64 * 1024) return fail(SPGT_ERR_INVALID_ARGUMENT, "conv3x3_resample: too many output channels");
 #define SPGT_CONV(CI)                                                                                                \
-    hipLaunchKernelGGL(conv3x3_resample_k<CI>, grid, block, 0, stream, x, weight, bias, out, Cout, H_in, W_in, H_out, \
-                       W_out, hscale, wscale, act)
+    hipLaunchKernelGGL(conv3x3_resample_k<CI>, grid, block, lds, stream, x, weight, bias, out, Cout, H_in, W_in,      \
+                       H_out, W_out, hscale, wscale, act)
     switch (Cin) {
         case 1: SPGT_CONV(1); break;
         case 2: SPGT_CONV(2); break;
