@@ -282,21 +282,21 @@ __global__ __launch_bounds__(256) void ffn_scalar_k(
 //   y1  = x + a @ Wfc + bfc                       a = attention output [T, K1], x = residual stream [T, 128]
 //   out = y1 + act(y1 @ W1 + b1) @ W2 + b2        hidden width 256
 // A workgroup takes 32 tokens through all three products: y1 and the hidden activations live in
-// LDS (and y1 also in the registers that add it back at the end), never in HBM.  Per product a wave
+// LDS, never in HBM.  Per product a wave
 // owns 32 output columns and holds their weights in registers as the MFMA A operand, as in
 // linear_tm_k; the weights are re-read from L2 per tile, which is what three separate launches do at
 // one tile per workgroup as well.  grid (ceil(T/32)), block 256.
 template <int K1>
-__global__ __launch_bounds__(256, 2) void encoder_tail_k(
+__global__ __launch_bounds__(256) void encoder_tail_k(
     const float* __restrict__ a, int64_t lda, const float* __restrict__ x, const float* __restrict__ Wfc,
     const float* __restrict__ bfc, const float* __restrict__ W1, const float* __restrict__ b1,
     const float* __restrict__ W2, const float* __restrict__ b2, int act, float* __restrict__ out, int64_t T) {
     constexpr int D = 128, F = 256, TT = 32, BK = 16;
     constexpr int PA = K1 + 1, PY = D + 1, PH = F + 1;
     extern __shared__ float lds[];
-    float* bufA = lds;               // [TT][PA]
-    float* bufY = bufA + TT * PA;    // [TT][PY]
+    float* bufY = lds;               // [TT][PY]
     float* bufH = bufY + TT * PY;    // [TT][PH]
+    float* bufA = bufH;              // [TT][PA], dead before bufH is written (PA <= PH)
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int tk = lane & 31;
@@ -356,78 +356,74 @@ __global__ __launch_bounds__(256, 2) void encoder_tail_k(
     }
 #define SPGT_TAIL_ZERO(ACC) _Pragma("unroll") for (int r_ = 0; r_ < 16; ++r_) ACC[r_] = 0.f;
 
-    // The weights of each product are requested before the MFMAs of the product ahead of it, so
-    // that their trip from L2 is hidden: wA/wB/wC/wD/wE are live two at a time.
+    // Register budget: one product's weights (<= 68), a batch pair of operands (32) and the accumulator, so
+    // that three workgroups fit on a CU and the 20k-token case of the Darcy model runs in one round.
     const int n0 = wave * 32;
-    float wA[K1 / 2], wB[D / 2], wC[D / 2], wD[D / 2], wE[D / 2];
-    SPGT_TAIL_LOADW(wA, K1, Wfc, D, n0, 0)
-    float y1[16];
     // ---- y1 = x + a @ Wfc + bfc: wave w owns columns 32w .. 32w+31
     {
+        float wA[K1 / 2];
+        SPGT_TAIL_LOADW(wA, K1, Wfc, D, n0, 0)
         float4 xq[4];
 #pragma unroll
         for (int q = 0; q < 4; ++q)
             xq[q] = tok ? *reinterpret_cast<const float4*>(x + t * D + n0 + 4 * kh + 8 * q) : make_float4(0.f, 0.f, 0.f, 0.f);
         __syncthreads();  // bufA complete
-        SPGT_TAIL_LOADW(wB, D, W1, F, n0, 0)  // first hidden column block of this wave
         v16f acc;
         SPGT_TAIL_ZERO(acc)
         SPGT_TAIL_MMA(acc, wA, K1, bufA, PA)
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
             const float4 bq = *reinterpret_cast<const float4*>(bfc + n0 + 4 * kh + 8 * q);
-            y1[4 * q + 0] = acc[4 * q + 0] + bq.x + xq[q].x;
-            y1[4 * q + 1] = acc[4 * q + 1] + bq.y + xq[q].y;
-            y1[4 * q + 2] = acc[4 * q + 2] + bq.z + xq[q].z;
-            y1[4 * q + 3] = acc[4 * q + 3] + bq.w + xq[q].w;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) bufY[tk * PY + n0 + 8 * q + 4 * kh + e] = y1[4 * q + e];
+            float* d = bufY + tk * PY + n0 + 8 * q + 4 * kh;
+            d[0] = acc[4 * q + 0] + bq.x + xq[q].x;
+            d[1] = acc[4 * q + 1] + bq.y + xq[q].y;
+            d[2] = acc[4 * q + 2] + bq.z + xq[q].z;
+            d[3] = acc[4 * q + 3] + bq.w + xq[q].w;
         }
     }
-    __syncthreads();  // bufY complete
+    __syncthreads();  // bufY complete, bufA free: bufH takes its place
 
     // ---- h = act(y1 @ W1 + b1): wave w owns hidden column blocks w and w + 4 of the 8
-    auto store_hidden = [&](const v16f& acc, int h0) {
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const float4 bq = *reinterpret_cast<const float4*>(b1 + h0 + 4 * kh + 8 * q);
-            const float bb[4] = {bq.x, bq.y, bq.z, bq.w};
-#pragma unroll
-            for (int e = 0; e < 4; ++e) bufH[tk * PH + h0 + 8 * q + 4 * kh + e] = activate(acc[4 * q + e] + bb[e], act);
-        }
-    };
-    {
-        SPGT_TAIL_LOADW(wC, D, W1, F, n0 + 128, 0)  // second hidden column block
+    for (int c = 0; c < 2; ++c) {
+        const int h0 = n0 + 128 * c;
+        float wB[D / 2];
+        SPGT_TAIL_LOADW(wB, D, W1, F, h0, 0)
         v16f acc;
         SPGT_TAIL_ZERO(acc)
         SPGT_TAIL_MMA(acc, wB, D, bufY, PY)
-        store_hidden(acc, n0);
-    }
-    {
-        SPGT_TAIL_LOADW(wD, D, W2, D, n0, 0)  // rows 0..127 of W2 for the last product
-        v16f acc;
-        SPGT_TAIL_ZERO(acc)
-        SPGT_TAIL_MMA(acc, wC, D, bufY, PY)
-        store_hidden(acc, n0 + 128);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const float4 bq = *reinterpret_cast<const float4*>(b1 + h0 + 4 * kh + 8 * q);
+            float* d = bufH + tk * PH + h0 + 8 * q + 4 * kh;
+            d[0] = activate(acc[4 * q + 0] + bq.x, act);
+            d[1] = activate(acc[4 * q + 1] + bq.y, act);
+            d[2] = activate(acc[4 * q + 2] + bq.z, act);
+            d[3] = activate(acc[4 * q + 3] + bq.w, act);
+        }
     }
     __syncthreads();  // bufH complete
 
-    // ---- out = y1 + h @ W2 + b2
+    // ---- out = y1 + h @ W2 + b2, the 256 hidden features in two halves
     {
-        SPGT_TAIL_LOADW(wE, D, W2, D, n0, 128)  // rows 128..255
         v16f acc;
         SPGT_TAIL_ZERO(acc)
-        SPGT_TAIL_MMA(acc, wD, D, bufH, PH)
-        SPGT_TAIL_MMA(acc, wE, D, bufH + 128, PH)
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            float wC[D / 2];
+            SPGT_TAIL_LOADW(wC, D, W2, D, n0, 128 * half)
+            SPGT_TAIL_MMA(acc, wC, D, bufH + 128 * half, PH)
+        }
         if (tok) {
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 const float4 bq = *reinterpret_cast<const float4*>(b2 + n0 + 4 * kh + 8 * q);
+                const float* y1 = bufY + tk * PY + n0 + 8 * q + 4 * kh;
                 float4 o;
-                o.x = acc[4 * q + 0] + bq.x + y1[4 * q + 0];
-                o.y = acc[4 * q + 1] + bq.y + y1[4 * q + 1];
-                o.z = acc[4 * q + 2] + bq.z + y1[4 * q + 2];
-                o.w = acc[4 * q + 3] + bq.w + y1[4 * q + 3];
+                o.x = acc[4 * q + 0] + bq.x + y1[0];
+                o.y = acc[4 * q + 1] + bq.y + y1[1];
+                o.z = acc[4 * q + 2] + bq.z + y1[2];
+                o.w = acc[4 * q + 3] + bq.w + y1[3];
                 *reinterpret_cast<float4*>(out + t * D + n0 + 4 * kh + 8 * q) = o;
             }
         }
@@ -637,7 +633,7 @@ extern "C" int spgt_encoder_tail_forward(const float* attn_out, int64_t ld_attn,
     if (ceil_div(tokens, (int64_t)32) > INT32_MAX)
         return fail(SPGT_ERR_INVALID_ARGUMENT, "encoder_tail_forward: too many tokens");
     const unsigned grid = (unsigned)ceil_div(tokens, (int64_t)32);
-    const size_t lds = (size_t)32 * ((attn_features + 1) + 129 + 257) * sizeof(float);
+    const size_t lds = (size_t)32 * (129 + 257) * sizeof(float);
     static const hipError_t opt136 = hipFuncSetAttribute(reinterpret_cast<const void*>(encoder_tail_k<136>),
                                                          hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
     static const hipError_t opt128 = hipFuncSetAttribute(reinterpret_cast<const void*>(encoder_tail_k<128>),
