@@ -32,16 +32,17 @@ __device__ __forceinline__ float activate(float v, int act) {
 
 }  // namespace
 
-// grid (token groups * column groups), block 256, the column group varying fastest so that the
-// workgroups that share an x tile run together and the tile comes from HBM once.  NCB column blocks of 32 per
+// grid (token groups * column groups, rounded up to a multiple of 8), block 256, the column group
+// varying fastest so that the workgroups that share an x tile run together, on one XCD.  NCB column blocks of 32 per
 // workgroup; the 4/NCB waves that share a column block take different 32-token
 // sub-tiles of the workgroup's TT = 32*(4/NCB)-token tile.
-template <int K, int NCB>
+template <int K, int NCB, bool RES>
 __global__ __launch_bounds__(256) void linear_tm_k(
     const float* __restrict__ x, int64_t ldx, const float* __restrict__ W, int ldw,
     const float* __restrict__ bias, const float* res, int64_t ldr, int res_mode, int act,
     const float* __restrict__ x2, int64_t ldx2, const float* __restrict__ W2, int r2,
-    float* out, int64_t ldo, int plane_cols, int64_t plane_stride, int64_t T, int tiles_per_wg, int gy) {
+    float* out, int64_t ldo, int plane_cols, int64_t plane_stride, int64_t T, int tiles_per_wg, int gy,
+    int total_wgs) {
     constexpr int KH = K / 2;
     constexpr int PITCH = K + 1;
     constexpr int TT = 32 * (4 / NCB);
@@ -54,8 +55,13 @@ __global__ __launch_bounds__(256) void linear_tm_k(
     const int wave = threadIdx.x >> 6;
     const int tk = lane & 31;
     const int kh = lane >> 5;
-    const int cg = blockIdx.x % gy;
-    const int tg = blockIdx.x / gy;
+    // Workgroups go round-robin to the 8 XCDs, each with its own L2: consecutive logical ids are mapped
+    // onto one XCD so that the column groups of a token tile share the x rows in that L2.
+    const int per_xcd = gridDim.x >> 3;
+    const int logical = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (logical >= total_wgs) return;
+    const int cg = logical % gy;
+    const int tg = logical / gy;
     const int n0 = (cg * NCB + wave % NCB) * 32;
     const int sub = wave / NCB;
 
@@ -63,10 +69,11 @@ __global__ __launch_bounds__(256) void linear_tm_k(
     float wreg[KH];
 #pragma unroll
     for (int kk = 0; kk < KH; ++kk) wreg[kk] = (W + (int64_t)(2 * kk) * ldw)[(uint32_t)(kh * ldw + n0 + tk)];
-    // accumulator element r holds column n0 + 8*(r/4) + 4*kh + r%4
-    float breg[16];
-#pragma unroll
-    for (int r = 0; r < 16; ++r) breg[r] = bias ? bias[n0 + 8 * (r >> 2) + 4 * kh + (r & 3)] : 0.f;
+    // accumulator element r holds column n0 + 8*(r/4) + 4*kh + r%4; the workgroup's 32*NCB bias values
+    // wait in LDS for the epilogue (16 registers less per lane: a third wave per SIMD fits)
+    __shared__ __align__(16) float bias_s[32 * NCB];
+    if (threadIdx.x < 32 * NCB) bias_s[threadIdx.x] = bias ? bias[cg * NCB * 32 + threadIdx.x] : 0.f;
+    const float* bias_l = bias_s + (wave % NCB) * 32 + 4 * kh;
 
     const int64_t t_begin = (int64_t)tg * tiles_per_wg * TT;
     const int64_t t_end = min(T, t_begin + (int64_t)tiles_per_wg * TT);
@@ -112,11 +119,13 @@ __global__ __launch_bounds__(256) void linear_tm_k(
         lds_batch(0);
         // the residual is fetched ahead of the MFMAs so that its latency hides behind them
         const int64_t t = t0 + sub * 32 + tk;
-        float4 rq[4];
+        float4 rq[RES ? 4 : 1];
+        if (RES) {
 #pragma unroll
-        for (int q = 0; q < 4; ++q)
-            rq[q] = (res_mode && t < t_end) ? *reinterpret_cast<const float4*>(res + t * ldr + n0 + 4 * kh + 8 * q)
-                                            : make_float4(0.f, 0.f, 0.f, 0.f);
+            for (int q = 0; q < 4; ++q)
+                rq[q] = (t < t_end) ? *reinterpret_cast<const float4*>(res + t * ldr + n0 + 4 * kh + 8 * q)
+                                    : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
         // the few extra input columns (r2 <= 4) are a rank-r2 update of the tile, done on the vector ALU
         float x2v[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -140,21 +149,22 @@ __global__ __launch_bounds__(256) void linear_tm_k(
             float* orow = out + (n0 / plane_cols) * plane_stride + t * ldo + n0 % plane_cols + 4 * kh;
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-                const float4 r4 = rq[q];
+                const float4 r4 = RES ? rq[RES ? q : 0] : make_float4(0.f, 0.f, 0.f, 0.f);
+                const float4 bq = *reinterpret_cast<const float4*>(bias_l + 8 * q);
                 float4 y;
-                y.x = acc[4 * q + 0] + breg[4 * q + 0];
-                y.y = acc[4 * q + 1] + breg[4 * q + 1];
-                y.z = acc[4 * q + 2] + breg[4 * q + 2];
-                y.w = acc[4 * q + 3] + breg[4 * q + 3];
+                y.x = acc[4 * q + 0] + bq.x;
+                y.y = acc[4 * q + 1] + bq.y;
+                y.z = acc[4 * q + 2] + bq.z;
+                y.w = acc[4 * q + 3] + bq.w;
                 for (int p = 0; p < r2; ++p) {
                     const float4 w4 = *reinterpret_cast<const float4*>(W2 + (int64_t)p * ldw + n0 + 4 * kh + 8 * q);
                     y.x = fmaf(x2v[p], w4.x, y.x); y.y = fmaf(x2v[p], w4.y, y.y);
                     y.z = fmaf(x2v[p], w4.z, y.z); y.w = fmaf(x2v[p], w4.w, y.w);
                 }
-                if (res_mode == SPGT_RES_BEFORE_ACT) { y.x += r4.x; y.y += r4.y; y.z += r4.z; y.w += r4.w; }
+                if (RES && res_mode == SPGT_RES_BEFORE_ACT) { y.x += r4.x; y.y += r4.y; y.z += r4.z; y.w += r4.w; }
                 y.x = activate(y.x, act); y.y = activate(y.y, act);
                 y.z = activate(y.z, act); y.w = activate(y.w, act);
-                if (res_mode == SPGT_RES_AFTER_ACT) { y.x += r4.x; y.y += r4.y; y.z += r4.z; y.w += r4.w; }
+                if (RES && res_mode == SPGT_RES_AFTER_ACT) { y.x += r4.x; y.y += r4.y; y.z += r4.z; y.w += r4.w; }
                 *reinterpret_cast<float4*>(orow + 8 * q) = y;
             }
         }
@@ -435,20 +445,19 @@ __global__ __launch_bounds__(256) void encoder_tail_k(
 
 namespace {
 
-// Tiles per workgroup.  A CU runs `occ` workgroups at a time; co-resident workgroups hide each
-// other's load latency and share the matrix pipe, so a round of k >= 2 of them costs k * tiles_per_wg
-// tile-times, while a workgroup that runs alone costs twice its tiles.  The CU with the most
-// workgroups sets the time; ties go to the choice closest to two workgroups per CU (fewer W reloads).
-inline int pick_tiles_per_wg(int64_t tiles, int gy, int cus, int occ) {
-    occ = std::max(1, occ);
+// Tiles per workgroup.  Measured on MI355X at 356k tokens: grids of 2 or 4 workgroups per CU run the
+// 128 -> 384 product in 355-370 us, a grid of 3 per CU in 450-520 us, whether two or three workgroups
+// fit on a CU at once.  The plan therefore counts workgroups per CU in pairs (an odd one costs as much
+// as two), takes the cheapest tiles_per_wg, and among equals the one closest to two per CU (fewer
+// re-reads of W than with more, something to overlap with unlike one).
+inline int pick_tiles_per_wg(int64_t tiles, int gy, int cus) {
     int best = 1;
     int64_t best_cost = INT64_MAX;
     double best_dist = 0;
     for (int tpw = 1; tpw <= 64; ++tpw) {
         const int64_t wgs = ceil_div(tiles, (int64_t)tpw) * gy;
         const int64_t per_cu = ceil_div(wgs, (int64_t)cus);
-        const int64_t rem = per_cu % occ;
-        const int64_t cost = tpw * ((per_cu / occ) * occ + (rem == 1 ? 2 : rem));
+        const int64_t cost = tpw * 2 * ceil_div(per_cu, (int64_t)2);
         const double dist = per_cu >= 2 ? (double)per_cu / 2 : 2.5;
         if (cost < best_cost || (cost == best_cost && dist < best_dist)) {
             best = tpw;
@@ -460,18 +469,7 @@ inline int pick_tiles_per_wg(int64_t tiles, int gy, int cus, int occ) {
     return best;
 }
 
-// Workgroups of `kernel` that fit on one CU at a time (queried once per kernel).
-template <typename Kernel>
-int resident_workgroups(Kernel kernel, size_t lds) {
-    int occ = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, kernel, 256, lds) != hipSuccess || occ < 1) {
-        (void)hipGetLastError();
-        occ = 2;
-    }
-    return occ;
-}
-
-template <int K, int NCB>
+template <int K, int NCB, bool RES>
 void launch_linear(const float* x, int64_t ldx, const float* W, const float* bias, const float* res, int64_t ldr,
                    int res_mode, int act, const float* x2, int64_t ldx2, const float* W2, int r2, float* out,
                    int64_t ldo, int plane_cols, int64_t plane_stride, int64_t T, int N, hipStream_t stream) {
@@ -479,15 +477,19 @@ void launch_linear(const float* x, int64_t ldx, const float* W, const float* bia
     const size_t lds = (size_t)TT * (K + 1) * sizeof(float);
     const int gy = N / (32 * NCB);
     const int64_t tiles = ceil_div(T, (int64_t)TT);
-    auto kernel = linear_tm_k<K, NCB>;
-    if (lds > 64 * 1024)
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                  (int)lds);
-    static const int occ = resident_workgroups(kernel, lds);
-    const int tpw = pick_tiles_per_wg(tiles, gy, device_cu_count(), occ);
-    const dim3 grid((unsigned)(ceil_div(tiles, (int64_t)tpw) * gy));
-    hipLaunchKernelGGL(kernel, grid, dim3(256), lds, stream, x, ldx, W, N, bias, res, ldr, res_mode, act, x2, ldx2, W2,
-                       r2, out, ldo, plane_cols, plane_stride, T, tpw, gy);
+    auto kernel = linear_tm_k<K, NCB, RES>;
+    static const hipError_t lds_opt_in = hipFuncSetAttribute(
+        reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+    (void)lds_opt_in;
+    const int tpw = pick_tiles_per_wg(tiles, gy, device_cu_count());
+    const int total_wgs = (int)(ceil_div(tiles, (int64_t)tpw) * gy);
+    // More than two workgroups per CU run in rounds of two (see pick_tiles_per_wg): asking for more
+    // than a third of the CU's 160 KB of LDS keeps a third workgroup from joining a round.
+    size_t lds_request = lds;
+    if (total_wgs > 2 * device_cu_count()) lds_request = std::max<size_t>(lds, 72 * 1024);
+    const dim3 grid((unsigned)(ceil_div(total_wgs, 8) * 8));  // whole rounds over the 8 XCDs
+    hipLaunchKernelGGL(kernel, grid, dim3(256), lds_request, stream, x, ldx, W, N, bias, res, ldr, res_mode, act, x2, ldx2, W2,
+                       r2, out, ldo, plane_cols, plane_stride, T, tpw, gy, total_wgs);
 }
 
 template <int K>
@@ -496,9 +498,15 @@ void launch_linear_k(int ncb, const float* x, int64_t ldx, const float* W, const
                      float* out, int64_t ldo, int plane_cols, int64_t plane_stride, int64_t T, int N,
                      hipStream_t stream) {
 #define SPGT_ARGS x, ldx, W, bias, res, ldr, res_mode, act, x2, ldx2, W2, r2, out, ldo, plane_cols, plane_stride, T, N, stream
-    if (ncb == 4) launch_linear<K, 4>(SPGT_ARGS);
-    else if (ncb == 2) launch_linear<K, 2>(SPGT_ARGS);
-    else launch_linear<K, 1>(SPGT_ARGS);
+    if (res_mode != SPGT_RES_NONE) {
+        if (ncb == 4) launch_linear<K, 4, true>(SPGT_ARGS);
+        else if (ncb == 2) launch_linear<K, 2, true>(SPGT_ARGS);
+        else launch_linear<K, 1, true>(SPGT_ARGS);
+    } else {
+        if (ncb == 4) launch_linear<K, 4, false>(SPGT_ARGS);
+        else if (ncb == 2) launch_linear<K, 2, false>(SPGT_ARGS);
+        else launch_linear<K, 1, false>(SPGT_ARGS);
+    }
 #undef SPGT_ARGS
 }
 
@@ -506,8 +514,7 @@ template <int K, int CBW>
 void launch_ffn_scalar(const float* x, int64_t ldx, const float* W1, const float* b1, const float* w2, const float* b2,
                        int act, float* out, int64_t T, hipStream_t stream) {
     const int64_t tiles = ceil_div(T, (int64_t)32);
-    static const int occ = resident_workgroups(ffn_scalar_k<K, CBW>, 0);
-    const int tpw = pick_tiles_per_wg(tiles, 1, device_cu_count(), occ);
+    const int tpw = pick_tiles_per_wg(tiles, 1, device_cu_count());
     hipLaunchKernelGGL((ffn_scalar_k<K, CBW>), dim3((unsigned)ceil_div(tiles, (int64_t)tpw)), dim3(256), 0, stream, x,
                        ldx, W1, b1, w2, b2, act, out, T, tpw);
 }
