@@ -54,11 +54,10 @@ __global__ __launch_bounds__(256) void apply_to_fm(const float* __restrict__ W, 
     const float* Xb = X + bh * D * (int64_t)S;
     float* ob = out + bh * D * (int64_t)S;
 
-    for (int sb = s0 + 32 * wave; sb < s1; sb += 128) {
-        const int s = sb + tk;
-        const bool valid = s < s1;
-        const int sl = valid ? s : s1 - 1;
-        float x[NK];
+    // Two register buffers in ping-pong: the loads of the next 32-token block are issued (clamped to
+    // the chunk, so unconditionally) before the MFMAs and stores of the current one.
+    auto load_block = [&](float (&x)[NK], int sb) {
+        const int sl = min(sb + tk, s1 - 1);
         if (X_TM) {
             const float* row = Xb + (int64_t)sl * D + NK * kh;
 #pragma unroll
@@ -67,6 +66,10 @@ __global__ __launch_bounds__(256) void apply_to_fm(const float* __restrict__ W, 
 #pragma unroll
             for (int kk = 0; kk < NK; ++kk) x[kk] = Xb[(int64_t)(2 * kk + kh) * S + sl];
         }
+    };
+    auto compute_block = [&](const float (&x)[NK], int sb) {
+        const int s = sb + tk;
+        const bool valid = s < s1;
         v16f acc;
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[r] = 0.f;
@@ -90,6 +93,19 @@ __global__ __launch_bounds__(256) void apply_to_fm(const float* __restrict__ W, 
             }
             if (D == 34) ob[(int64_t)(32 + kh) * S + s] = kh == 0 ? e0 : e1;
         }
+    };
+    float xa[NK], xb[NK];
+    int sb = s0 + 32 * wave;
+    if (sb < s1) load_block(xa, sb);
+    for (; sb < s1; sb += 256) {
+        load_block(xb, sb + 128);
+        __builtin_amdgcn_sched_barrier(0);
+        compute_block(xa, sb);
+        __builtin_amdgcn_sched_barrier(0);
+        load_block(xa, sb + 256);
+        __builtin_amdgcn_sched_barrier(0);
+        if (sb + 128 < s1) compute_block(xb, sb + 128);
+        __builtin_amdgcn_sched_barrier(0);
     }
 }
 
