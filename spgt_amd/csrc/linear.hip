@@ -30,6 +30,72 @@ __device__ __forceinline__ float activate(float v, int act) {
     return v;
 }
 
+// The same on N values with the choice made once, outside the loop: per-element calls with a run-time
+// `act` compile to a branch tree per element, which is most of an epilogue's time.
+template <int N>
+__device__ __forceinline__ void activate_all(float (&v)[N], int act) {
+    if (act == SPGT_ACT_RELU) {
+#pragma unroll
+        for (int i = 0; i < N; ++i) v[i] = fmaxf(v[i], 0.f);
+    } else if (act == SPGT_ACT_SILU) {
+#pragma unroll
+        for (int i = 0; i < N; ++i) v[i] = v[i] * __builtin_amdgcn_rcpf(1.f + __expf(-v[i]));
+    }
+}
+
+// Epilogue shared by the linear kernels: y = acc + bias (+ extra columns) (+ residual before or after
+// the activation), written as four 16-byte pieces of the lane's token row.  Uniform choices (activation,
+// residual placement, extra columns) are made once per call, not per element.
+template <bool RES>
+__device__ __forceinline__ void linear_epilogue(const v16f& acc, const float4 (&bq)[4], const float4* rq, int res_mode,
+                                                int act, const float (&x2v)[4], const float* W2row, int ldw, int r2,
+                                                float* orow) {
+    float y[16];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        y[4 * q + 0] = acc[4 * q + 0] + bq[q].x;
+        y[4 * q + 1] = acc[4 * q + 1] + bq[q].y;
+        y[4 * q + 2] = acc[4 * q + 2] + bq[q].z;
+        y[4 * q + 3] = acc[4 * q + 3] + bq[q].w;
+    }
+    if (r2 > 0) {
+        for (int p = 0; p < r2; ++p) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const float4 w4 = *reinterpret_cast<const float4*>(W2row + (int64_t)p * ldw + 8 * q);
+                y[4 * q + 0] = fmaf(x2v[p], w4.x, y[4 * q + 0]);
+                y[4 * q + 1] = fmaf(x2v[p], w4.y, y[4 * q + 1]);
+                y[4 * q + 2] = fmaf(x2v[p], w4.z, y[4 * q + 2]);
+                y[4 * q + 3] = fmaf(x2v[p], w4.w, y[4 * q + 3]);
+            }
+        }
+    }
+    const float before = (RES && res_mode == SPGT_RES_BEFORE_ACT) ? 1.f : 0.f;
+    if (RES) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            y[4 * q + 0] = fmaf(rq[q].x, before, y[4 * q + 0]);
+            y[4 * q + 1] = fmaf(rq[q].y, before, y[4 * q + 1]);
+            y[4 * q + 2] = fmaf(rq[q].z, before, y[4 * q + 2]);
+            y[4 * q + 3] = fmaf(rq[q].w, before, y[4 * q + 3]);
+        }
+    }
+    activate_all(y, act);
+    if (RES) {
+        const float after = 1.f - before;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            y[4 * q + 0] = fmaf(rq[q].x, after, y[4 * q + 0]);
+            y[4 * q + 1] = fmaf(rq[q].y, after, y[4 * q + 1]);
+            y[4 * q + 2] = fmaf(rq[q].z, after, y[4 * q + 2]);
+            y[4 * q + 3] = fmaf(rq[q].w, after, y[4 * q + 3]);
+        }
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+        *reinterpret_cast<float4*>(orow + 8 * q) = make_float4(y[4 * q], y[4 * q + 1], y[4 * q + 2], y[4 * q + 3]);
+}
+
 }  // namespace
 
 // grid (token groups * column groups, rounded up to a multiple of 8), block 256, the column group
@@ -74,6 +140,8 @@ __global__ __launch_bounds__(256) void linear_tm_k(
     __shared__ __align__(16) float bias_s[32 * NCB];
     if (threadIdx.x < 32 * NCB) bias_s[threadIdx.x] = bias ? bias[cg * NCB * 32 + threadIdx.x] : 0.f;
     const float* bias_l = bias_s + (wave % NCB) * 32 + 4 * kh;
+    // output column n lives in plane n / plane_cols at column n % plane_cols
+    const int64_t out_col = (n0 / plane_cols) * plane_stride + n0 % plane_cols + 4 * kh;
 
     const int64_t t_begin = (int64_t)tg * tiles_per_wg * TT;
     const int64_t t_end = min(T, t_begin + (int64_t)tiles_per_wg * TT);
@@ -145,29 +213,137 @@ __global__ __launch_bounds__(256) void linear_tm_k(
         }
 
         if (t < t_end) {
-            // output column n lives in plane n / plane_cols at column n % plane_cols
-            float* orow = out + (n0 / plane_cols) * plane_stride + t * ldo + n0 % plane_cols + 4 * kh;
+            float4 bq[4];
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const float4 r4 = RES ? rq[RES ? q : 0] : make_float4(0.f, 0.f, 0.f, 0.f);
-                const float4 bq = *reinterpret_cast<const float4*>(bias_l + 8 * q);
-                float4 y;
-                y.x = acc[4 * q + 0] + bq.x;
-                y.y = acc[4 * q + 1] + bq.y;
-                y.z = acc[4 * q + 2] + bq.z;
-                y.w = acc[4 * q + 3] + bq.w;
-                for (int p = 0; p < r2; ++p) {
-                    const float4 w4 = *reinterpret_cast<const float4*>(W2 + (int64_t)p * ldw + n0 + 4 * kh + 8 * q);
-                    y.x = fmaf(x2v[p], w4.x, y.x); y.y = fmaf(x2v[p], w4.y, y.y);
-                    y.z = fmaf(x2v[p], w4.z, y.z); y.w = fmaf(x2v[p], w4.w, y.w);
-                }
-                if (RES && res_mode == SPGT_RES_BEFORE_ACT) { y.x += r4.x; y.y += r4.y; y.z += r4.z; y.w += r4.w; }
-                y.x = activate(y.x, act); y.y = activate(y.y, act);
-                y.z = activate(y.z, act); y.w = activate(y.w, act);
-                if (RES && res_mode == SPGT_RES_AFTER_ACT) { y.x += r4.x; y.y += r4.y; y.z += r4.z; y.w += r4.w; }
-                *reinterpret_cast<float4*>(orow + 8 * q) = y;
-            }
+            for (int q = 0; q < 4; ++q) bq[q] = *reinterpret_cast<const float4*>(bias_l + 8 * q);
+            linear_epilogue<RES>(acc, bq, rq, res_mode, act, x2v, W2 + n0 + 4 * kh, ldw, r2, out + out_col + t * ldo);
         }
+    }
+}
+
+// The same product with the waves of a workgroup split by role.  On this part two waves that both issue
+// long chains of fp32 MFMAs with many distinct operand registers share a SIMD badly (a register-only loop
+// drops from 136 to 77 TFLOP/s), while an MFMA wave next to a wave that only loads and writes LDS keeps its
+// rate.  So: 512 threads = 4 compute waves (one per SIMD: weights in registers, operands from LDS, MFMAs,
+// epilogue) + 4 loader waves (global -> registers -> LDS, one tile ahead, two LDS buffers), one workgroup
+// per CU, one barrier per tile.  Used for 256 input features and out_features % 128 == 0 on long inputs.
+// grid (slots * column groups), block 512; workgroup (slot, cg) takes tiles slot, slot + slots, ...
+template <int K, bool RES>
+__global__ __launch_bounds__(512) void linear_ws_k(
+    const float* __restrict__ x, int64_t ldx, const float* __restrict__ W, int ldw,
+    const float* __restrict__ bias, const float* res, int64_t ldr, int res_mode, int act,
+    const float* __restrict__ x2, int64_t ldx2, const float* __restrict__ W2, int r2,
+    float* out, int64_t ldo, int plane_cols, int64_t plane_stride, int64_t T, int gy) {
+    constexpr int KH = K / 2;
+    constexpr int PITCH = K + 1;
+    constexpr int SUBT = (K <= 136) ? 2 : 1;  // 32-token sub-tiles per stage: a stage outlasts a memory round trip
+    constexpr int TT = 32 * SUBT;
+    constexpr int BK = 16;
+    constexpr int NB = (KH + BK - 1) / BK;
+    constexpr int NVEC = TT * K / 4;
+    constexpr int NLD = (NVEC + 255) / 256;
+    extern __shared__ float xs[];  // [2][TT][PITCH]
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int cg = blockIdx.x % gy;
+    const int slot = blockIdx.x / gy;
+    const int slots = gridDim.x / gy;
+    const int64_t ntiles = (T + TT - 1) / TT;
+    const int64_t mine = slot < ntiles ? (ntiles - slot + slots - 1) / slots : 0;  // tiles of this workgroup
+
+    if (wave >= 4) {
+        // ---- loader waves: tile i+1 goes into buffer (i+1)&1 while the compute waves work on buffer i&1
+        const int lt = threadIdx.x - 256;
+        float4 stage[NLD];
+        auto load_tile = [&](int64_t tile) {
+            const int64_t t0 = tile * TT;
+#pragma unroll
+            for (int i = 0; i < NLD; ++i) {
+                const int e = lt + 256 * i;
+                const int row = e / (K / 4);
+                const int c4 = e % (K / 4);
+                const int64_t t = t0 + row;
+                stage[i] = (e < NVEC && t < T) ? *reinterpret_cast<const float4*>(x + t * ldx + 4 * c4)
+                                               : make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+        };
+        auto store_tile = [&](float* buf) {
+#pragma unroll
+            for (int i = 0; i < NLD; ++i) {
+                const int e = lt + 256 * i;
+                if (e < NVEC) {
+                    const int row = e / (K / 4);
+                    const int c4 = e % (K / 4);
+                    float* d = buf + row * PITCH + 4 * c4;
+                    d[0] = stage[i].x; d[1] = stage[i].y; d[2] = stage[i].z; d[3] = stage[i].w;
+                }
+            }
+        };
+        if (mine > 0) {
+            load_tile(slot);
+            store_tile(xs);
+        }
+        if (mine > 1) load_tile(slot + slots);
+        __syncthreads();  // buffer 0 ready
+        for (int64_t i = 0; i < mine; ++i) {
+            if (i + 1 < mine) store_tile(xs + ((i + 1) & 1) * TT * PITCH);
+            if (i + 2 < mine) load_tile(slot + (i + 2) * slots);
+            __syncthreads();  // tile i consumed, tile i+1 in place
+        }
+        return;
+    }
+
+    // ---- compute waves: wave w owns columns cg*128 + 32w .. +31
+    const int tk = lane & 31;
+    const int kh = lane >> 5;
+    const int n0 = (cg * 4 + wave) * 32;
+    float wreg[KH];
+#pragma unroll
+    for (int kk = 0; kk < KH; ++kk) wreg[kk] = (W + (int64_t)(2 * kk) * ldw)[(uint32_t)(kh * ldw + n0 + tk)];
+    float4 bq[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+        bq[q] = bias ? *reinterpret_cast<const float4*>(bias + n0 + 4 * kh + 8 * q) : make_float4(0.f, 0.f, 0.f, 0.f);
+    const int64_t out_col = (n0 / plane_cols) * plane_stride + n0 % plane_cols + 4 * kh;
+    __syncthreads();  // buffer 0 ready
+    for (int64_t i = 0; i < mine; ++i) {
+#pragma unroll
+        for (int st = 0; st < SUBT; ++st) {
+        const float* xr = xs + (i & 1) * TT * PITCH + (st * 32 + tk) * PITCH + kh;
+        const int64_t t = (slot + i * slots) * TT + st * 32 + tk;
+        float xv[2][BK];
+#pragma unroll
+        for (int j = 0; j < BK; ++j) xv[0][j] = xr[2 * j];
+        float4 rq[RES ? 4 : 1];
+        if (RES) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                rq[q] = (t < T) ? *reinterpret_cast<const float4*>(res + t * ldr + n0 + 4 * kh + 8 * q)
+                                : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+        float x2v[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int p = 0; p < 4; ++p)
+            if (p < r2 && t < T) x2v[p] = x2[t * ldx2 + p];
+        v16f acc;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+#pragma unroll
+        for (int bt = 0; bt < NB; ++bt) {
+            if (bt + 1 < NB) {
+#pragma unroll
+                for (int j = 0; j < BK; ++j)
+                    if ((bt + 1) * BK + j < KH) xv[(bt + 1) & 1][j] = xr[2 * ((bt + 1) * BK + j)];
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int j = 0; j < BK; ++j)
+                if (bt * BK + j < KH) acc = mfma32(wreg[bt * BK + j], xv[bt & 1][j], acc);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (t < T) linear_epilogue<RES>(acc, bq, rq, res_mode, act, x2v, W2 + n0 + 4 * kh, ldw, r2, out + out_col + t * ldo);
+        }
+        __syncthreads();  // tile i consumed, tile i+1 in place
     }
 }
 
@@ -273,9 +449,14 @@ __global__ __launch_bounds__(256) void ffn_scalar_k(
         // this lane's share of token t0 + tk: 16*CBW hidden columns
         float part = 0.f;
 #pragma unroll
-        for (int c = 0; c < CBW; ++c)
+        for (int c = 0; c < CBW; ++c) {
+                float hv[16];
 #pragma unroll
-            for (int r = 0; r < 16; ++r) part = fmaf(activate(acc[c][r] + breg[c][r], act), vreg[c][r], part);
+                for (int r = 0; r < 16; ++r) hv[r] = acc[c][r] + breg[c][r];
+                activate_all(hv, act);
+#pragma unroll
+                for (int r = 0; r < 16; ++r) part = fmaf(hv[r], vreg[c][r], part);
+            }
         part += __shfl_xor(part, 32, 64);
         if (kh == 0) red[wave][tk] = part;
         __syncthreads();
@@ -402,14 +583,20 @@ __global__ __launch_bounds__(256) void encoder_tail_k(
         v16f acc;
         SPGT_TAIL_ZERO(acc)
         SPGT_TAIL_MMA(acc, wB, D, bufY, PY)
+        float hv[16];
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
             const float4 bq = *reinterpret_cast<const float4*>(b1 + h0 + 4 * kh + 8 * q);
+            hv[4 * q + 0] = acc[4 * q + 0] + bq.x;
+            hv[4 * q + 1] = acc[4 * q + 1] + bq.y;
+            hv[4 * q + 2] = acc[4 * q + 2] + bq.z;
+            hv[4 * q + 3] = acc[4 * q + 3] + bq.w;
+        }
+        activate_all(hv, act);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
             float* d = bufH + tk * PH + h0 + 8 * q + 4 * kh;
-            d[0] = activate(acc[4 * q + 0] + bq.x, act);
-            d[1] = activate(acc[4 * q + 1] + bq.y, act);
-            d[2] = activate(acc[4 * q + 2] + bq.z, act);
-            d[3] = activate(acc[4 * q + 3] + bq.w, act);
+            d[0] = hv[4 * q + 0]; d[1] = hv[4 * q + 1]; d[2] = hv[4 * q + 2]; d[3] = hv[4 * q + 3];
         }
     }
     __syncthreads();  // bufH complete
@@ -492,12 +679,35 @@ void launch_linear(const float* x, int64_t ldx, const float* W, const float* bia
                        r2, out, ldo, plane_cols, plane_stride, T, tpw, gy, total_wgs);
 }
 
+template <int K, bool RES>
+void launch_linear_ws(const float* x, int64_t ldx, const float* W, const float* bias, const float* res, int64_t ldr,
+                      int res_mode, int act, const float* x2, int64_t ldx2, const float* W2, int r2, float* out,
+                      int64_t ldo, int plane_cols, int64_t plane_stride, int64_t T, int N, hipStream_t stream) {
+    const int gy = N / 128;
+    const int slots = std::max(1, device_cu_count() / gy);  // one workgroup per CU
+    // two 32-token buffers, and at least half of the CU's LDS so that no second workgroup joins
+    const size_t lds = std::max<size_t>((size_t)2 * 32 * (K <= 136 ? 2 : 1) * (K + 1) * sizeof(float), 84 * 1024);
+    auto kernel = linear_ws_k<K, RES>;
+    static const hipError_t lds_opt_in = hipFuncSetAttribute(
+        reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+    (void)lds_opt_in;
+    hipLaunchKernelGGL(kernel, dim3(slots * gy), dim3(512), lds, stream, x, ldx, W, N, bias, res, ldr, res_mode, act, x2,
+                       ldx2, W2, r2, out, ldo, plane_cols, plane_stride, T, gy);
+}
+
 template <int K>
 void launch_linear_k(int ncb, const float* x, int64_t ldx, const float* W, const float* bias, const float* res,
                      int64_t ldr, int res_mode, int act, const float* x2, int64_t ldx2, const float* W2, int r2,
                      float* out, int64_t ldo, int plane_cols, int64_t plane_stride, int64_t T, int N,
                      hipStream_t stream) {
 #define SPGT_ARGS x, ldx, W, bias, res, ldr, res_mode, act, x2, ldx2, W2, r2, out, ldo, plane_cols, plane_stride, T, N, stream
+    // long inputs with whole 128-column groups and 256 input features: role-split workgroups, one per CU
+    // (with fewer input features the plain kernel is as fast or faster)
+    if constexpr (K >= 256) if (ncb == 4 && T >= (int64_t)64 * device_cu_count() && N / 128 <= device_cu_count()) {
+        if (res_mode != SPGT_RES_NONE) launch_linear_ws<K, true>(SPGT_ARGS);
+        else launch_linear_ws<K, false>(SPGT_ARGS);
+        return;
+    }
     if (res_mode != SPGT_RES_NONE) {
         if (ncb == 4) launch_linear<K, 4, true>(SPGT_ARGS);
         else if (ncb == 2) launch_linear<K, 2, true>(SPGT_ARGS);
