@@ -17,6 +17,8 @@
 // and tokens along lanes, so a lane stores four 16-byte pieces of its token's
 // row.  LDS reads for the next batch of MFMAs are issued before the current
 // batch so that their latency hides behind the matrix pipe.
+#include <type_traits>
+
 #include "spgt_device.h"
 #include "spgt_host.h"
 
@@ -223,26 +225,52 @@ __global__ __launch_bounds__(256) void linear_tm_k(
 
 // The same product with the waves of a workgroup split by role.  On this part two waves that both issue
 // long chains of fp32 MFMAs with many distinct operand registers share a SIMD badly (a register-only loop
-// drops from 136 to 77 TFLOP/s), while an MFMA wave next to a wave that only loads and writes LDS keeps its
-// rate.  So: 512 threads = 4 compute waves (one per SIMD: weights in registers, operands from LDS, MFMAs,
-// epilogue) + 4 loader waves (global -> registers -> LDS, one tile ahead, two LDS buffers), one workgroup
-// per CU, one barrier per tile.  Used for 256 input features and out_features % 128 == 0 on long inputs.
+// drops from 136 to 77 TFLOP/s), so there is one MFMA wave per SIMD, and with a single MFMA wave per SIMD
+// nothing else fills the matrix pipe while that wave does anything but MFMAs.  So:
+//  - the wave's own epilogue is software-pipelined: the residual / activation arithmetic of tile i-1 is
+//    spread, a quarter of a 32-token half at a time, between the MFMAs of tile i (two sets of accumulators;
+//    the bias is the first MFMA's addend), and its result goes to an LDS output tile rather than to memory;
+//  - with 64-token tiles the two 32-token halves are two independent MFMA chains issued alternately, so
+//    that no MFMA waits for the one before it;
+//  - lane (token, kh) takes k = kh*K/2 + j for MFMA j, so that four consecutive MFMAs' operands are one
+//    16-byte LDS read, and rows are K+4 words apart, which makes those reads and the movers' 16-byte
+//    writes both free of bank conflicts.
+// Alone, the compute waves then take 8400 cycles for the 128 MFMAs of a 64-token tile at 128 input features
+// (8192 is the matrix pipe's own time).  What bounds the kernel is the data movement beside them: next to a
+// busy MFMA wave, another wave's LDS write or global store of 16 bytes per lane takes about 500 cycles,
+// whatever its priority or its target (a global load -> LDS without registers is no quicker once stores
+// run beside it), so the 32 + 32 such instructions of a tile are spread over all four SIMDs: 2 load waves
+// (global -> registers -> LDS, one tile ahead) and 2 store waves (LDS -> global as whole 512-byte rows, two
+// tiles behind) each need about one tile time for their share.
+// 512 threads = 4 compute + 2 load + 2 store waves, two LDS buffers each way, one workgroup per CU, one
+// barrier per tile.  Used for out_features % 128 == 0 on long inputs without extra input columns.
 // grid (slots * column groups), block 512; workgroup (slot, cg) takes tiles slot, slot + slots, ...
-template <int K, bool RES>
+template <int K>
+struct LinearWs {
+    static constexpr int SUBT = (K <= 136) ? 2 : 1;  // 32-token halves per tile = MFMA chains
+    static constexpr int TT = 32 * SUBT;
+    static constexpr int PITCH = K + 4;   // input tile rows
+    static constexpr int OPITCH = 132;    // output tile rows
+    static constexpr size_t lds_bytes = (size_t)2 * TT * (PITCH + OPITCH) * sizeof(float);
+};
+
+template <int K, bool RES, int ACT>
 __global__ __launch_bounds__(512) void linear_ws_k(
     const float* __restrict__ x, int64_t ldx, const float* __restrict__ W, int ldw,
-    const float* __restrict__ bias, const float* res, int64_t ldr, int res_mode, int act,
-    const float* __restrict__ x2, int64_t ldx2, const float* __restrict__ W2, int r2,
+    const float* __restrict__ bias, const float* res, int64_t ldr, int res_mode,
     float* out, int64_t ldo, int plane_cols, int64_t plane_stride, int64_t T, int gy) {
     constexpr int KH = K / 2;
-    constexpr int PITCH = K + 1;
-    constexpr int SUBT = (K <= 136) ? 2 : 1;  // 32-token sub-tiles per stage: a stage outlasts a memory round trip
-    constexpr int TT = 32 * SUBT;
-    constexpr int BK = 16;
+    constexpr int PITCH = LinearWs<K>::PITCH;
+    constexpr int OPITCH = LinearWs<K>::OPITCH;
+    constexpr int SUBT = LinearWs<K>::SUBT;
+    constexpr int TT = LinearWs<K>::TT;
+    constexpr int BK = 8;
     constexpr int NB = (KH + BK - 1) / BK;
     constexpr int NVEC = TT * K / 4;
-    constexpr int NLD = (NVEC + 255) / 256;
-    extern __shared__ float xs[];  // [2][TT][PITCH]
+    constexpr int NLD = (NVEC + 127) / 128;
+    static_assert(KH % 4 == 0, "16-byte operand reads");
+    extern __shared__ float xs[];                 // [2][TT][PITCH]
+    float* const os = xs + 2 * TT * PITCH;        // [2][TT][OPITCH]
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int cg = blockIdx.x % gy;
@@ -250,16 +278,62 @@ __global__ __launch_bounds__(512) void linear_ws_k(
     const int slots = gridDim.x / gy;
     const int64_t ntiles = (T + TT - 1) / TT;
     const int64_t mine = slot < ntiles ? (ntiles - slot + slots - 1) / slots : 0;  // tiles of this workgroup
+    // Step s (s = 0 .. mine): the compute waves run the MFMAs of tile s (s < mine) and, under them, the epilogue
+    // of tile s-1 into output buffer s&1; the store waves write out buffer (s-1)&1 = tile s-2; the load waves
+    // put tile s+1's input in place and start the loads of tile s+2.
 
+    if (wave >= 6) {
+        // ---- store waves (2): LDS output tile -> global, whole 512-byte rows.  Their stores may wait for
+        // room in the memory pipeline; nothing else depends on these waves within a step.
+        __builtin_amdgcn_s_setprio(3);  // their few vector ALU instructions otherwise queue behind the MFMA wave's
+        const int lt = threadIdx.x - 384;
+        // this thread's output pieces: column 4*(lt%32) of the group, rows lt/32 + 4*r
+        const int oc = cg * 128 + 4 * (lt & 31);
+        float* const ocol = out + (oc / plane_cols) * plane_stride + oc % plane_cols;
+        auto flush_tile = [&](int64_t ti) {
+            if (ti < 0 || ti >= mine) return;
+#pragma unroll
+            for (int h = 0; h < TT / 16; ++h) {
+                const float* buf = os + (((ti + 1) & 1) * TT + h * 16 + (lt >> 5)) * OPITCH + 4 * (lt & 31);
+                const int64_t t0 = (slot + ti * slots) * TT + h * 16;
+                float4 v0 = *reinterpret_cast<const float4*>(buf);
+                float4 v1 = *reinterpret_cast<const float4*>(buf + 4 * OPITCH);
+                float4 v2 = *reinterpret_cast<const float4*>(buf + 8 * OPITCH);
+                float4 v3 = *reinterpret_cast<const float4*>(buf + 12 * OPITCH);
+                float* const o = ocol + (t0 + (lt >> 5)) * ldo;
+                if (t0 + 16 <= T) {
+                    // whole block in range: straight-line code, so the reads go out together
+                    *reinterpret_cast<float4*>(o) = v0;
+                    *reinterpret_cast<float4*>(o + 4 * ldo) = v1;
+                    *reinterpret_cast<float4*>(o + 8 * ldo) = v2;
+                    *reinterpret_cast<float4*>(o + 12 * ldo) = v3;
+                } else {
+                    const int64_t left = T - t0 - (lt >> 5);  // rows of this thread's column that exist
+                    if (left > 0) *reinterpret_cast<float4*>(o) = v0;
+                    if (left > 4) *reinterpret_cast<float4*>(o + 4 * ldo) = v1;
+                    if (left > 8) *reinterpret_cast<float4*>(o + 8 * ldo) = v2;
+                    if (left > 12) *reinterpret_cast<float4*>(o + 12 * ldo) = v3;
+                }
+            }
+        };
+        __syncthreads();  // input buffer 0 ready
+        for (int64_t s = 0; s <= mine; ++s) {
+            flush_tile(s - 2);
+            __syncthreads();  // step s done
+        }
+        flush_tile(mine - 1);
+        return;
+    }
     if (wave >= 4) {
-        // ---- loader waves: tile i+1 goes into buffer (i+1)&1 while the compute waves work on buffer i&1
+        // ---- load waves (2): global -> registers -> LDS input tile, one tile ahead
+        __builtin_amdgcn_s_setprio(3);
         const int lt = threadIdx.x - 256;
         float4 stage[NLD];
         auto load_tile = [&](int64_t tile) {
             const int64_t t0 = tile * TT;
 #pragma unroll
             for (int i = 0; i < NLD; ++i) {
-                const int e = lt + 256 * i;
+                const int e = lt + 128 * i;
                 const int row = e / (K / 4);
                 const int c4 = e % (K / 4);
                 const int64_t t = t0 + row;
@@ -270,13 +344,8 @@ __global__ __launch_bounds__(512) void linear_ws_k(
         auto store_tile = [&](float* buf) {
 #pragma unroll
             for (int i = 0; i < NLD; ++i) {
-                const int e = lt + 256 * i;
-                if (e < NVEC) {
-                    const int row = e / (K / 4);
-                    const int c4 = e % (K / 4);
-                    float* d = buf + row * PITCH + 4 * c4;
-                    d[0] = stage[i].x; d[1] = stage[i].y; d[2] = stage[i].z; d[3] = stage[i].w;
-                }
+                const int e = lt + 128 * i;
+                if (e < NVEC) *reinterpret_cast<float4*>(buf + (e / (K / 4)) * PITCH + 4 * (e % (K / 4))) = stage[i];
             }
         };
         if (mine > 0) {
@@ -284,11 +353,11 @@ __global__ __launch_bounds__(512) void linear_ws_k(
             store_tile(xs);
         }
         if (mine > 1) load_tile(slot + slots);
-        __syncthreads();  // buffer 0 ready
-        for (int64_t i = 0; i < mine; ++i) {
-            if (i + 1 < mine) store_tile(xs + ((i + 1) & 1) * TT * PITCH);
-            if (i + 2 < mine) load_tile(slot + (i + 2) * slots);
-            __syncthreads();  // tile i consumed, tile i+1 in place
+        __syncthreads();  // input buffer 0 ready
+        for (int64_t s = 0; s <= mine; ++s) {
+            if (s + 1 < mine) store_tile(xs + ((s + 1) & 1) * TT * PITCH);
+            if (s + 2 < mine) load_tile(slot + (s + 2) * slots);
+            __syncthreads();  // step s done
         }
         return;
     }
@@ -297,54 +366,133 @@ __global__ __launch_bounds__(512) void linear_ws_k(
     const int tk = lane & 31;
     const int kh = lane >> 5;
     const int n0 = (cg * 4 + wave) * 32;
-    float wreg[KH];
+    float wreg[KH];  // W[kh*KH + j][n0 + tk]
 #pragma unroll
-    for (int kk = 0; kk < KH; ++kk) wreg[kk] = (W + (int64_t)(2 * kk) * ldw)[(uint32_t)(kh * ldw + n0 + tk)];
-    float4 bq[4];
+    for (int j = 0; j < KH; ++j) wreg[j] = (W + (int64_t)j * ldw)[(uint32_t)(kh * KH * ldw + n0 + tk)];
+    // the bias in accumulator layout: every chain's first MFMA adds to it
+    v16f biasv;
 #pragma unroll
-    for (int q = 0; q < 4; ++q)
-        bq[q] = bias ? *reinterpret_cast<const float4*>(bias + n0 + 4 * kh + 8 * q) : make_float4(0.f, 0.f, 0.f, 0.f);
-    const int64_t out_col = (n0 / plane_cols) * plane_stride + n0 % plane_cols + 4 * kh;
-    __syncthreads();  // buffer 0 ready
-    for (int64_t i = 0; i < mine; ++i) {
+    for (int q = 0; q < 4; ++q) {
+        const float4 b4 = bias ? *reinterpret_cast<const float4*>(bias + n0 + 4 * kh + 8 * q) : make_float4(0.f, 0.f, 0.f, 0.f);
+        biasv[4 * q + 0] = b4.x; biasv[4 * q + 1] = b4.y; biasv[4 * q + 2] = b4.z; biasv[4 * q + 3] = b4.w;
+    }
+    const float before = (RES && res_mode == SPGT_RES_BEFORE_ACT) ? 1.f : 0.f;
+    const float after = 1.f - before;
+    v16f acc[2][SUBT];  // [tile parity][chain]
 #pragma unroll
-        for (int st = 0; st < SUBT; ++st) {
-        const float* xr = xs + (i & 1) * TT * PITCH + (st * 32 + tk) * PITCH + kh;
-        const int64_t t = (slot + i * slots) * TT + st * 32 + tk;
-        float xv[2][BK];
+    for (int c = 0; c < SUBT; ++c)
 #pragma unroll
-        for (int j = 0; j < BK; ++j) xv[0][j] = xr[2 * j];
-        float4 rq[RES ? 4 : 1];
+        for (int r = 0; r < 16; ++r) acc[0][c][r] = acc[1][c][r] = 0.f;
+    __builtin_amdgcn_s_waitcnt(0);  // weights are in: no wait for them is left inside the loop
+
+    // A quarter of an epilogue: residual + activation of values 4q .. 4q+3 of chain c of accumulator set P,
+    // as one 16-byte LDS write into this lane's token row.  Straight-line code that the scheduler can spread
+    // between MFMAs; a step has 4*SUBT of these.
+    auto quarter = [&](auto Pc, int c, int q, const float4& rq, float* orow) {
+        constexpr int P = decltype(Pc)::value;
+        float y[4] = {acc[P][c][4 * q + 0], acc[P][c][4 * q + 1], acc[P][c][4 * q + 2], acc[P][c][4 * q + 3]};
         if (RES) {
-#pragma unroll
-            for (int q = 0; q < 4; ++q)
-                rq[q] = (t < T) ? *reinterpret_cast<const float4*>(res + t * ldr + n0 + 4 * kh + 8 * q)
-                                : make_float4(0.f, 0.f, 0.f, 0.f);
+            y[0] = fmaf(rq.x, before, y[0]); y[1] = fmaf(rq.y, before, y[1]);
+            y[2] = fmaf(rq.z, before, y[2]); y[3] = fmaf(rq.w, before, y[3]);
         }
-        float x2v[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int p = 0; p < 4; ++p)
-            if (p < r2 && t < T) x2v[p] = x2[t * ldx2 + p];
-        v16f acc;
+        for (int r = 0; r < 4; ++r) {
+            if (ACT == SPGT_ACT_RELU) y[r] = fmaxf(y[r], 0.f);
+            if (ACT == SPGT_ACT_SILU) y[r] = y[r] * __builtin_amdgcn_rcpf(1.f + __expf(-y[r]));
+        }
+        if (RES) {
+            y[0] = fmaf(rq.x, after, y[0]); y[1] = fmaf(rq.y, after, y[1]);
+            y[2] = fmaf(rq.z, after, y[2]); y[3] = fmaf(rq.w, after, y[3]);
+        }
+        *reinterpret_cast<float4*>(orow + 8 * q) = make_float4(y[0], y[1], y[2], y[3]);
+    };
+    // this lane's row of chain c in the output buffer of step s
+    auto out_row = [&](int64_t s, int c) { return os + ((s & 1) * TT + c * 32 + tk) * OPITCH + wave * 32 + 4 * kh; };
+    // residual rows of tile s-1 (rows outside the input read a valid row: their results are never written out)
+    auto load_residual = [&](int64_t s, float4 (&rq)[SUBT][RES ? 4 : 1]) {
+        if (!RES) return;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+        for (int c = 0; c < SUBT; ++c) {
+            const int64_t t = min(max((slot + (s - 1) * slots) * TT + c * 32 + tk, (int64_t)0), T - 1);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) rq[c][q] = *reinterpret_cast<const float4*>(res + t * ldr + n0 + 4 * kh + 8 * q);
+        }
+    };
+    constexpr int NQ = 4 * SUBT;                  // epilogue quarters per step
+    constexpr int QPB = (NQ + NB - 1) / NB;       // quarters per batch, from batch 0 on
+
+    // step s < mine: MFMAs of tile s into accumulator set P, epilogue of set P^1 (tile s-1) under the first batches
+    auto step = [&](auto Pc, int64_t s) {
+        constexpr int P = decltype(Pc)::value;
+        const float* xr = xs + ((s & 1) * TT + tk) * PITCH + kh * KH;
+        float4 xv[2][SUBT][BK / 4];
+#pragma unroll
+        for (int c = 0; c < SUBT; ++c)
+#pragma unroll
+            for (int g = 0; g < BK / 4; ++g) xv[0][c][g] = *reinterpret_cast<const float4*>(xr + c * 32 * PITCH + 4 * g);
+        float4 rq[SUBT][RES ? 4 : 1];
+        load_residual(s, rq);
 #pragma unroll
         for (int bt = 0; bt < NB; ++bt) {
             if (bt + 1 < NB) {
 #pragma unroll
-                for (int j = 0; j < BK; ++j)
-                    if ((bt + 1) * BK + j < KH) xv[(bt + 1) & 1][j] = xr[2 * ((bt + 1) * BK + j)];
+                for (int c = 0; c < SUBT; ++c)
+#pragma unroll
+                    for (int g = 0; g < BK / 4; ++g)
+                        if ((bt + 1) * BK + 4 * g < KH)
+                            xv[(bt + 1) & 1][c][g] =
+                                *reinterpret_cast<const float4*>(xr + c * 32 * PITCH + (bt + 1) * BK + 4 * g);
             }
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int j = 0; j < BK; ++j)
-                if (bt * BK + j < KH) acc = mfma32(wreg[bt * BK + j], xv[bt & 1][j], acc);
+            for (int u = bt * QPB; u < (bt + 1) * QPB && u < NQ; ++u)
+                quarter(std::integral_constant<int, P ^ 1>{}, u / 4, u % 4, rq[u / 4][RES ? u % 4 : 0], out_row(s, u / 4));
+#pragma unroll
+            for (int j = 0; j < BK; ++j) {
+                if (bt * BK + j < KH) {
+                    const int g = j / 4, e = j % 4;
+#pragma unroll
+                    for (int c = 0; c < SUBT; ++c) {
+                        const float4 v4 = xv[bt & 1][c][g];
+                        const float b = e == 0 ? v4.x : e == 1 ? v4.y : e == 2 ? v4.z : v4.w;
+                        acc[P][c] = mfma32(wreg[bt * BK + j], b, (bt == 0 && j == 0) ? biasv : acc[P][c]);
+                    }
+                }
+            }
+            if (bt * QPB < NQ) {
+                // one MFMA, then a slice of the epilogue in its shadow
+#pragma unroll
+                for (int j = 0; j < BK * SUBT; ++j) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x002, (QPB * 44 + BK * SUBT - 1) / (BK * SUBT), 0);
+                }
+            }
             __builtin_amdgcn_sched_barrier(0);
         }
-        if (t < T) linear_epilogue<RES>(acc, bq, rq, res_mode, act, x2v, W2 + n0 + 4 * kh, ldw, r2, out + out_col + t * ldo);
+    };
+    // step mine: only the epilogue of the last tile
+    auto last_step = [&](auto Pc) {
+        constexpr int P = decltype(Pc)::value;
+        float4 rq[SUBT][RES ? 4 : 1];
+        load_residual(mine, rq);
+#pragma unroll
+        for (int u = 0; u < NQ; ++u)
+            quarter(std::integral_constant<int, P>{}, u / 4, u % 4, rq[u / 4][RES ? u % 4 : 0], out_row(mine, u / 4));
+    };
+
+    __syncthreads();  // input buffer 0 ready
+    for (int64_t s = 0; s < mine; s += 2) {
+        step(std::integral_constant<int, 0>{}, s);
+        __syncthreads();  // step s done
+        if (s + 1 < mine) {
+            step(std::integral_constant<int, 1>{}, s + 1);
+            __syncthreads();
         }
-        __syncthreads();  // tile i consumed, tile i+1 in place
     }
+    // accumulator set (mine-1)&1 holds the last tile
+    if (mine & 1) last_step(std::integral_constant<int, 0>{});
+    else if (mine > 0) last_step(std::integral_constant<int, 1>{});
+    __syncthreads();  // step mine done
 }
 
 // Two-layer feed-forward net with a single output feature:
@@ -679,20 +827,31 @@ void launch_linear(const float* x, int64_t ldx, const float* W, const float* bia
                        r2, out, ldo, plane_cols, plane_stride, T, tpw, gy, total_wgs);
 }
 
-template <int K, bool RES>
+template <int K, bool RES, int ACT>
 void launch_linear_ws(const float* x, int64_t ldx, const float* W, const float* bias, const float* res, int64_t ldr,
-                      int res_mode, int act, const float* x2, int64_t ldx2, const float* W2, int r2, float* out,
-                      int64_t ldo, int plane_cols, int64_t plane_stride, int64_t T, int N, hipStream_t stream) {
+                      int res_mode, float* out, int64_t ldo, int plane_cols, int64_t plane_stride, int64_t T, int N,
+                      hipStream_t stream) {
     const int gy = N / 128;
     const int slots = std::max(1, device_cu_count() / gy);  // one workgroup per CU
-    // two 32-token buffers, and at least half of the CU's LDS so that no second workgroup joins
-    const size_t lds = std::max<size_t>((size_t)2 * 32 * (K <= 136 ? 2 : 1) * (K + 1) * sizeof(float), 84 * 1024);
-    auto kernel = linear_ws_k<K, RES>;
+    // at least half of the CU's LDS so that no second workgroup joins
+    const size_t lds = std::max<size_t>(LinearWs<K>::lds_bytes, 84 * 1024);
+    auto kernel = linear_ws_k<K, RES, ACT>;
     static const hipError_t lds_opt_in = hipFuncSetAttribute(
-        reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+        reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     (void)lds_opt_in;
-    hipLaunchKernelGGL(kernel, dim3(slots * gy), dim3(512), lds, stream, x, ldx, W, N, bias, res, ldr, res_mode, act, x2,
-                       ldx2, W2, r2, out, ldo, plane_cols, plane_stride, T, gy);
+    hipLaunchKernelGGL(kernel, dim3(slots * gy), dim3(512), lds, stream, x, ldx, W, N, bias, res, ldr, res_mode, out,
+                       ldo, plane_cols, plane_stride, T, gy);
+}
+
+template <int K, bool RES>
+void launch_linear_ws_act(const float* x, int64_t ldx, const float* W, const float* bias, const float* res, int64_t ldr,
+                          int res_mode, int act, float* out, int64_t ldo, int plane_cols, int64_t plane_stride,
+                          int64_t T, int N, hipStream_t stream) {
+#define SPGT_WS_ARGS x, ldx, W, bias, res, ldr, res_mode, out, ldo, plane_cols, plane_stride, T, N, stream
+    if (act == SPGT_ACT_RELU) launch_linear_ws<K, RES, SPGT_ACT_RELU>(SPGT_WS_ARGS);
+    else if (act == SPGT_ACT_SILU) launch_linear_ws<K, RES, SPGT_ACT_SILU>(SPGT_WS_ARGS);
+    else launch_linear_ws<K, RES, SPGT_ACT_NONE>(SPGT_WS_ARGS);
+#undef SPGT_WS_ARGS
 }
 
 template <int K>
@@ -701,11 +860,15 @@ void launch_linear_k(int ncb, const float* x, int64_t ldx, const float* W, const
                      float* out, int64_t ldo, int plane_cols, int64_t plane_stride, int64_t T, int N,
                      hipStream_t stream) {
 #define SPGT_ARGS x, ldx, W, bias, res, ldr, res_mode, act, x2, ldx2, W2, r2, out, ldo, plane_cols, plane_stride, T, N, stream
-    // long inputs with whole 128-column groups and 256 input features: role-split workgroups, one per CU
-    // (with fewer input features the plain kernel is as fast or faster)
-    if constexpr (K >= 256) if (ncb == 4 && T >= (int64_t)64 * device_cu_count() && N / 128 <= device_cu_count()) {
-        if (res_mode != SPGT_RES_NONE) launch_linear_ws<K, true>(SPGT_ARGS);
-        else launch_linear_ws<K, false>(SPGT_ARGS);
+    // Long inputs with whole 128-column groups and no extra columns: role-split workgroups, one per CU.
+    // With 256 input features they win from one 64-token tile per CU on; with fewer, from four on (below
+    // that the plain kernel's finer split balances the CUs better).
+    const int64_t ws_tokens = (int64_t)(K >= 256 ? 64 : 256) * device_cu_count();
+    if (ncb == 4 && r2 == 0 && T >= ws_tokens && N / 128 <= device_cu_count()) {
+        if (res_mode != SPGT_RES_NONE)
+            launch_linear_ws_act<K, true>(x, ldx, W, bias, res, ldr, res_mode, act, out, ldo, plane_cols, plane_stride, T, N, stream);
+        else
+            launch_linear_ws_act<K, false>(x, ldx, W, bias, res, ldr, res_mode, act, out, ldo, plane_cols, plane_stride, T, N, stream);
         return;
     }
     if (res_mode != SPGT_RES_NONE) {

@@ -86,6 +86,31 @@ def test_linear_output_planes(gpu):
         fused_linear(x.to(gpu), w.to(gpu), b.to(gpu), planes=5)
 
 
+@pytest.mark.parametrize("K,N,planes", [(64, 128, 1), (128, 128, 1), (128, 384, 3), (136, 128, 1), (256, 128, 1),
+                                        (256, 256, 1)])
+@pytest.mark.parametrize("act,res_mode", [("none", None), ("silu", None), ("relu", "before"), ("none", "after")])
+def test_linear_long_inputs(gpu, K, N, planes, act, res_mode):
+    """70001 tokens (a ragged last tile): the size class that runs on role-split workgroups, one per CU.
+    Expected values from a float64 product on the GPU (the CPU product of this size takes too long)."""
+    from spgt_amd.extension.bind.linear import fused_linear
+    T = 70001
+    g = torch.Generator().manual_seed(K + N)
+    wide = torch.randn(T, K + 4, generator=g).to(gpu)
+    x = wide[:, 4:] if K % 8 == 0 else wide[:, :K].contiguous()  # a strided view where K allows the alignment
+    w = (torch.randn(K, N, generator=g) / K ** 0.5).to(gpu)
+    b = torch.randn(N, generator=g).to(gpu)
+    res = torch.randn(T, N, generator=g).to(gpu) if res_mode and planes == 1 else None
+    got = fused_linear(x, w, b, act, res, res_mode == "after", planes=planes)
+    want = _expected(x, w, b, act, res, res_mode == "after")
+    if planes > 1:
+        assert got.shape == (planes, T, N // planes)
+        got = got.permute(1, 0, 2).reshape(T, N)
+    err = (got.double() - want).abs().max().item()
+    assert err <= 1e-5 * max(1.0, want.abs().max().item())
+    # nothing written past the last row's neighbours: the rows around the ragged end are exact too
+    assert torch.isfinite(got[-70:]).all()
+
+
 @pytest.mark.parametrize("E", [1, 2, 4])
 def test_linear_extra_columns(gpu, E):
     """x_extra @ weight_extra_kn added in the epilogue equals a Linear over the concatenated input
