@@ -615,167 +615,243 @@ __global__ __launch_bounds__(256) void ffn_scalar_k(
     }
 }
 
+// MFMA with the weight operand and the accumulator in accumulation registers.  A kernel that keeps more than
+// 256 registers of weights has most of them there, and the compiler's own form copies each one into a vector
+// register first (v_accvgpr_read), which next to a running MFMA costs about 20 cycles per MFMA (85 against 64
+// cycles per instruction measured).  The compiler does not see an MFMA in these statements, so the wait states
+// it would insert are written out: two before (operand just written by a vector instruction), and
+// mfma_acc_done() before the accumulator is read (an MFMA of 16 passes needs 18 after it).
+__device__ __forceinline__ void mfma32_acc_first(v16f& acc, float w, float x) {
+    asm volatile("s_nop 1\n\tv_mfma_f32_32x32x2_f32 %0, %1, %2, 0" : "=a"(acc) : "a"(w), "v"(x));
+}
+__device__ __forceinline__ void mfma32_acc(v16f& acc, float w, float x) {
+    asm volatile("s_nop 1\n\tv_mfma_f32_32x32x2_f32 %0, %1, %2, %0" : "+a"(acc) : "a"(w), "v"(x));
+}
+__device__ __forceinline__ void mfma_acc_done(v16f& acc) { asm volatile("s_nop 15\n\ts_nop 7" : "+a"(acc)); }
+
 // The tail of an encoder layer after the attention core, one launch per layer
 // (Sp_EncoderLayer.forward, network/sp_layer.py:97-103, with the attention's fc_layer, :75, and
 // FeedForward, network/layer.py:155-174):
 //   y1  = x + a @ Wfc + bfc                       a = attention output [T, K1], x = residual stream [T, 128]
 //   out = y1 + act(y1 @ W1 + b1) @ W2 + b2        hidden width 256
-// A workgroup takes 32 tokens through all three products: y1 and the hidden activations live in
-// LDS, never in HBM.  Per product a wave
-// owns 32 output columns and holds their weights in registers as the MFMA A operand, as in
-// linear_tm_k; the weights are re-read from L2 per tile, which is what three separate launches do at
-// one tile per workgroup as well.  grid (ceil(T/32)), block 256.
+// y1 and the hidden activations live in LDS, never in HBM, and every weight is resident: one workgroup of
+// four waves per CU, one wave per SIMD, and each wave keeps its 32-column slices of all three weight matrices
+// in registers for the whole kernel (68 + 128 + 128 of the 512 a lone wave may use), so the 82k weights are
+// read once per CU instead of once per 32 tokens, and a single MFMA wave per SIMD runs at the matrix pipe's
+// rate instead of sharing it badly with others.
+// Workgroups loop over 32-token tiles (tile = blockIdx.x + i*gridDim.x); the next tile's attention rows and
+// residual rows are requested a tile ahead.  Operand layout as in linear_ws_k: lane (token, kh) takes
+// k = kh*KK/2 + j for MFMA j, rows KK+4 words apart, 16-byte conflict-free LDS reads; each product runs as two
+// independent MFMA chains (the two hidden column blocks of the first feed-forward product, alternate groups
+// of four k-steps otherwise).  In-kernel cycle counts per tile (MFMA pipe time 4352 + 8192 + 8192): 4650 +
+// 900 epilogue, 10 700 (2500 of it the SiLU epilogue), 9000, 2000 for loads, LDS staging and barriers.
+// grid (min(tiles, CUs)), block 256.
 template <int K1>
-__global__ __launch_bounds__(256) void encoder_tail_k(
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void encoder_tail_k(
     const float* __restrict__ a, int64_t lda, const float* __restrict__ x, const float* __restrict__ Wfc,
     const float* __restrict__ bfc, const float* __restrict__ W1, const float* __restrict__ b1,
     const float* __restrict__ W2, const float* __restrict__ b2, int act, float* __restrict__ out, int64_t T) {
-    constexpr int D = 128, F = 256, TT = 32, BK = 16;
-    constexpr int PA = K1 + 1, PY = D + 1, PH = F + 1;
+    constexpr int D = 128, F = 256, TT = 32;
+    constexpr int PA = K1 + 4, PY = D + 4, PH = F + 4;
+    constexpr int NVEC = TT * K1 / 4;          // 16-byte pieces of an attention tile
+    constexpr int NLD = (NVEC + 255) / 256;
     extern __shared__ float lds[];
-    float* bufY = lds;               // [TT][PY]
-    float* bufH = bufY + TT * PY;    // [TT][PH]
-    float* bufA = bufH;              // [TT][PA], dead before bufH is written (PA <= PH)
+    float* const bufA = lds;                   // [TT][PA]
+    float* const bufY = bufA + TT * PA;        // [TT][PY]
+    float* const bufH = bufY + TT * PY;        // [TT][PH]
+    float* const bias_s = bufH + TT * PH;      // bfc[128] | b1[256] | b2[128]
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int tk = lane & 31;
     const int kh = lane >> 5;
-    const int64_t t0 = (int64_t)blockIdx.x * TT;
-    const int64_t t = t0 + tk;
-    const bool tok = t < T;
-
-    // stage the attention-output tile (coalesced 16-byte reads, scalar LDS writes at an odd pitch)
-    {
-        constexpr int NVEC = TT * K1 / 4;
-        constexpr int NLD = (NVEC + 255) / 256;
-        float4 stage[NLD];
-#pragma unroll
-        for (int i = 0; i < NLD; ++i) {
-            const int e = threadIdx.x + 256 * i;
-            const int row = e / (K1 / 4), c4 = e % (K1 / 4);
-            stage[i] = (e < NVEC && t0 + row < T) ? *reinterpret_cast<const float4*>(a + (t0 + row) * lda + 4 * c4)
-                                                  : make_float4(0.f, 0.f, 0.f, 0.f);
-        }
-#pragma unroll
-        for (int i = 0; i < NLD; ++i) {
-            const int e = threadIdx.x + 256 * i;
-            if (e < NVEC) {
-                const int row = e / (K1 / 4), c4 = e % (K1 / 4);
-                float* d = bufA + row * PA + 4 * c4;
-                d[0] = stage[i].x; d[1] = stage[i].y; d[2] = stage[i].z; d[3] = stage[i].w;
-            }
-        }
-    }
-
-    // Weights of one product for this wave: WR[kk] = W[K0 + 2kk + kh][N0 + tk], W [.][N] row-major
-    // (wave-uniform row base + one 32-bit lane offset, so the loads need no per-load address registers).
-#define SPGT_TAIL_LOADW(WR, KK, W, N, N0, K0)                                                    \
-    __builtin_amdgcn_sched_barrier(0);                                                           \
-    _Pragma("unroll") for (int kk = 0; kk < (KK) / 2; ++kk)                                      \
-        WR[kk] = ((W) + (int64_t)((K0) + 2 * kk) * (N))[(uint32_t)(kh * (N) + (N0) + tk)];       \
-    __builtin_amdgcn_sched_barrier(0);
-    // ACC[r] += sum_k SRC[tk][k] * (weights in WR), k < KK; operands are read from LDS a batch ahead.
-#define SPGT_TAIL_MMA(ACC, WR, KK, SRC, PITCH)                                                   \
-    {                                                                                            \
-        constexpr int KH_ = (KK) / 2;                                                            \
-        constexpr int NB_ = (KH_ + BK - 1) / BK;                                                 \
-        const float* xr_ = (SRC) + tk * (PITCH) + kh;                                            \
-        float xv_[2][BK];                                                                        \
-        _Pragma("unroll") for (int j = 0; j < BK; ++j) xv_[0][j] = xr_[2 * j];                   \
-        _Pragma("unroll") for (int bt = 0; bt < NB_; ++bt) {                                     \
-            if (bt + 1 < NB_) {                                                                  \
-                _Pragma("unroll") for (int j = 0; j < BK; ++j)                                   \
-                    if ((bt + 1) * BK + j < KH_) xv_[(bt + 1) & 1][j] = xr_[2 * ((bt + 1) * BK + j)]; \
-            }                                                                                    \
-            __builtin_amdgcn_sched_barrier(0);                                                   \
-            _Pragma("unroll") for (int j = 0; j < BK; ++j)                                       \
-                if (bt * BK + j < KH_) ACC = mfma32(WR[bt * BK + j], xv_[bt & 1][j], ACC);       \
-            __builtin_amdgcn_sched_barrier(0);                                                   \
-        }                                                                                        \
-    }
-#define SPGT_TAIL_ZERO(ACC) _Pragma("unroll") for (int r_ = 0; r_ < 16; ++r_) ACC[r_] = 0.f;
-
-    // Register budget: one product's weights (<= 68), a batch pair of operands (32) and the accumulator, so
-    // that three workgroups fit on a CU and the 20k-token case of the Darcy model runs in one round.
     const int n0 = wave * 32;
-    // ---- y1 = x + a @ Wfc + bfc: wave w owns columns 32w .. 32w+31
-    {
-        float wA[K1 / 2];
-        SPGT_TAIL_LOADW(wA, K1, Wfc, D, n0, 0)
-        float4 xq[4];
-#pragma unroll
-        for (int q = 0; q < 4; ++q)
-            xq[q] = tok ? *reinterpret_cast<const float4*>(x + t * D + n0 + 4 * kh + 8 * q) : make_float4(0.f, 0.f, 0.f, 0.f);
-        __syncthreads();  // bufA complete
-        v16f acc;
-        SPGT_TAIL_ZERO(acc)
-        SPGT_TAIL_MMA(acc, wA, K1, bufA, PA)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const float4 bq = *reinterpret_cast<const float4*>(bfc + n0 + 4 * kh + 8 * q);
-            float* d = bufY + tk * PY + n0 + 8 * q + 4 * kh;
-            d[0] = acc[4 * q + 0] + bq.x + xq[q].x;
-            d[1] = acc[4 * q + 1] + bq.y + xq[q].y;
-            d[2] = acc[4 * q + 2] + bq.z + xq[q].z;
-            d[3] = acc[4 * q + 3] + bq.w + xq[q].w;
-        }
-    }
-    __syncthreads();  // bufY complete, bufA free: bufH takes its place
+    const int64_t ntiles = (T + TT - 1) / TT;
 
-    // ---- h = act(y1 @ W1 + b1): wave w owns hidden column blocks w and w + 4 of the 8
+    // ---- resident weights: W?[kh*KK/2 + j][column block + tk]
+    float wA[K1 / 2], wB[2][D / 2], wC[F / 2];
 #pragma unroll
-    for (int c = 0; c < 2; ++c) {
-        const int h0 = n0 + 128 * c;
-        float wB[D / 2];
-        SPGT_TAIL_LOADW(wB, D, W1, F, h0, 0)
-        v16f acc;
-        SPGT_TAIL_ZERO(acc)
-        SPGT_TAIL_MMA(acc, wB, D, bufY, PY)
-        float hv[16];
+    for (int j = 0; j < K1 / 2; ++j) wA[j] = (Wfc + (int64_t)j * D)[(uint32_t)(kh * (K1 / 2) * D + n0 + tk)];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const float4 bq = *reinterpret_cast<const float4*>(b1 + h0 + 4 * kh + 8 * q);
-            hv[4 * q + 0] = acc[4 * q + 0] + bq.x;
-            hv[4 * q + 1] = acc[4 * q + 1] + bq.y;
-            hv[4 * q + 2] = acc[4 * q + 2] + bq.z;
-            hv[4 * q + 3] = acc[4 * q + 3] + bq.w;
-        }
-        activate_all(hv, act);
+    for (int c = 0; c < 2; ++c)
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            float* d = bufH + tk * PH + h0 + 8 * q + 4 * kh;
-            d[0] = hv[4 * q + 0]; d[1] = hv[4 * q + 1]; d[2] = hv[4 * q + 2]; d[3] = hv[4 * q + 3];
-        }
-    }
-    __syncthreads();  // bufH complete
+        for (int j = 0; j < D / 2; ++j) wB[c][j] = (W1 + (int64_t)j * F)[(uint32_t)(kh * (D / 2) * F + n0 + 128 * c + tk)];
+#pragma unroll
+    for (int j = 0; j < F / 2; ++j) wC[j] = (W2 + (int64_t)j * D)[(uint32_t)(kh * (F / 2) * D + n0 + tk)];
+    for (int i = threadIdx.x; i < 512; i += 256)
+        bias_s[i] = i < 128 ? bfc[i] : i < 384 ? b1[i - 128] : b2[i - 384];
 
-    // ---- out = y1 + h @ W2 + b2, the 256 hidden features in two halves
-    {
-        v16f acc;
-        SPGT_TAIL_ZERO(acc)
+    // attention rows of a tile: coalesced 16-byte loads into registers, 16-byte LDS writes a tile later
+    float4 stage[NLD];
+    auto load_a = [&](int64_t tile) {
+        const int64_t t0 = tile * TT;
 #pragma unroll
-        for (int half = 0; half < 2; ++half) {
-            float wC[D / 2];
-            SPGT_TAIL_LOADW(wC, D, W2, D, n0, 128 * half)
-            SPGT_TAIL_MMA(acc, wC, D, bufH + 128 * half, PH)
+        for (int i = 0; i < NLD; ++i) {
+            const int e = threadIdx.x + 256 * i;
+            const int64_t row = t0 + e / (K1 / 4);
+            stage[i] = (e < NVEC && row < T) ? *reinterpret_cast<const float4*>(a + row * lda + 4 * (e % (K1 / 4)))
+                                             : make_float4(0.f, 0.f, 0.f, 0.f);
         }
-        if (tok) {
+    };
+    auto store_a = [&]() {
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) {
+            const int e = threadIdx.x + 256 * i;
+            if (e < NVEC) *reinterpret_cast<float4*>(bufA + (e / (K1 / 4)) * PA + 4 * (e % (K1 / 4))) = stage[i];
+        }
+    };
+    // acc0/acc1 += src[tk][k] * w over k-step groups [0, NG) of four; group g goes to chain chain_of(g).
+    // Operands are read from LDS 16 k-steps ahead of their MFMAs.
+    constexpr int GB = 4;  // groups per operand batch
+    auto read_batch = [&](float4 (&xv)[GB], const float* xr, int g0, int NG) {
+#pragma unroll
+        for (int g = 0; g < GB; ++g)
+            if (g0 + g < NG) xv[g] = *reinterpret_cast<const float4*>(xr + 4 * (g0 + g));
+    };
+    auto comp = [](const float4& v, int e) { return e == 0 ? v.x : e == 1 ? v.y : e == 2 ? v.z : v.w; };
+
+    // residual rows of a tile, requested a tile ahead too (rows past the end read the last row: never written out)
+    float4 xq[4];
+    auto load_x = [&](int64_t tile) {
+        const int64_t row = min(tile * TT + tk, T - 1);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) xq[q] = *reinterpret_cast<const float4*>(x + row * D + n0 + 4 * kh + 8 * q);
+    };
+    const int64_t first = blockIdx.x;
+    if (first < ntiles) {
+        load_a(first);
+        store_a();
+        load_x(first);
+    }
+    __builtin_amdgcn_s_waitcnt(0);  // weights are in: no wait for them is left inside the loop
+    __syncthreads();
+    for (int64_t tile = first; tile < ntiles; tile += gridDim.x) {
+        const int64_t t = tile * TT + tk;
+        const bool tok = t < T;
+        const bool more = tile + gridDim.x < ntiles;
+        if (more) load_a(tile + gridDim.x);
+
+        // ---- y1 = x + a @ Wfc + bfc: wave w owns columns 32w .. 32w+31
+        {
+            constexpr int NG = K1 / 8;
+            const float* xr = bufA + tk * PA + kh * (K1 / 2);
+            v16f acc[2];
+            float4 xv[2][GB];
+            read_batch(xv[0], xr, 0, NG);
+#pragma unroll
+            for (int g0 = 0; g0 < NG; g0 += GB) {
+                if (g0 + GB < NG) read_batch(xv[((g0 / GB) + 1) & 1], xr, g0 + GB, NG);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+#pragma unroll
+                    for (int g = 0; g < GB; ++g)
+                        if (g0 + g < NG) {
+                            if (g0 == 0 && e == 0 && g < 2) mfma32_acc_first(acc[g & 1], wA[4 * g + e], comp(xv[0][g], e));
+                            else mfma32_acc(acc[g & 1], wA[4 * (g0 + g) + e], comp(xv[(g0 / GB) & 1][g], e));
+                        }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            mfma_acc_done(acc[0]);
+            mfma_acc_done(acc[1]);
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-                const float4 bq = *reinterpret_cast<const float4*>(b2 + n0 + 4 * kh + 8 * q);
-                const float* y1 = bufY + tk * PY + n0 + 8 * q + 4 * kh;
-                float4 o;
-                o.x = acc[4 * q + 0] + bq.x + y1[0];
-                o.y = acc[4 * q + 1] + bq.y + y1[1];
-                o.z = acc[4 * q + 2] + bq.z + y1[2];
-                o.w = acc[4 * q + 3] + bq.w + y1[3];
-                *reinterpret_cast<float4*>(out + t * D + n0 + 4 * kh + 8 * q) = o;
+                const float4 bq = *reinterpret_cast<const float4*>(bias_s + n0 + 4 * kh + 8 * q);
+                float4 y;
+                y.x = (acc[0][4 * q + 0] + acc[1][4 * q + 0]) + bq.x + xq[q].x;
+                y.y = (acc[0][4 * q + 1] + acc[1][4 * q + 1]) + bq.y + xq[q].y;
+                y.z = (acc[0][4 * q + 2] + acc[1][4 * q + 2]) + bq.z + xq[q].z;
+                y.w = (acc[0][4 * q + 3] + acc[1][4 * q + 3]) + bq.w + xq[q].w;
+                *reinterpret_cast<float4*>(bufY + tk * PY + n0 + 8 * q + 4 * kh) = y;
             }
         }
+        if (more) load_x(tile + gridDim.x);
+        __syncthreads();  // bufY complete
+
+        // ---- h = act(y1 @ W1 + b1): wave w owns hidden column blocks w and w + 4, one MFMA chain each
+        {
+            constexpr int NG = D / 8;
+            const float* xr = bufY + tk * PY + kh * (D / 2);
+            v16f acc[2];
+            float4 xv[2][GB];
+            read_batch(xv[0], xr, 0, NG);
+#pragma unroll
+            for (int g0 = 0; g0 < NG; g0 += GB) {
+                if (g0 + GB < NG) read_batch(xv[((g0 / GB) + 1) & 1], xr, g0 + GB, NG);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int g = 0; g < GB; ++g)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const float b = comp(xv[(g0 / GB) & 1][g], e);
+                        if (g0 == 0 && g == 0 && e == 0) {
+                            mfma32_acc_first(acc[0], wB[0][0], b);
+                            mfma32_acc_first(acc[1], wB[1][0], b);
+                        } else {
+                            mfma32_acc(acc[0], wB[0][4 * (g0 + g) + e], b);
+                            mfma32_acc(acc[1], wB[1][4 * (g0 + g) + e], b);
+                        }
+                    }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            mfma_acc_done(acc[0]);
+            mfma_acc_done(acc[1]);
+#pragma unroll
+            for (int c = 0; c < 2; ++c) {
+                float hv[16];
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const float4 bq = *reinterpret_cast<const float4*>(bias_s + 128 + n0 + 128 * c + 4 * kh + 8 * q);
+                    hv[4 * q + 0] = acc[c][4 * q + 0] + bq.x;
+                    hv[4 * q + 1] = acc[c][4 * q + 1] + bq.y;
+                    hv[4 * q + 2] = acc[c][4 * q + 2] + bq.z;
+                    hv[4 * q + 3] = acc[c][4 * q + 3] + bq.w;
+                }
+                activate_all(hv, act);
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                    *reinterpret_cast<float4*>(bufH + tk * PH + n0 + 128 * c + 8 * q + 4 * kh) =
+                        make_float4(hv[4 * q + 0], hv[4 * q + 1], hv[4 * q + 2], hv[4 * q + 3]);
+            }
+        }
+        __syncthreads();  // bufH complete
+
+        // ---- out = y1 + h @ W2 + b2
+        {
+            constexpr int NG = F / 8;
+            const float* xr = bufH + tk * PH + kh * (F / 2);
+            v16f acc[2];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[0][r] = acc[1][r] = 0.f;
+            float4 xv[2][GB];
+            read_batch(xv[0], xr, 0, NG);
+#pragma unroll
+            for (int g0 = 0; g0 < NG; g0 += GB) {
+                if (g0 + GB < NG) read_batch(xv[((g0 / GB) + 1) & 1], xr, g0 + GB, NG);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+#pragma unroll
+                    for (int g = 0; g < GB; ++g)
+                        acc[g & 1] = mfma32(wC[4 * (g0 + g) + e], comp(xv[(g0 / GB) & 1][g], e), acc[g & 1]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (tok) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const float4 bq = *reinterpret_cast<const float4*>(bias_s + 384 + n0 + 4 * kh + 8 * q);
+                    const float4 y1 = *reinterpret_cast<const float4*>(bufY + tk * PY + n0 + 8 * q + 4 * kh);
+                    float4 o;
+                    o.x = (acc[0][4 * q + 0] + acc[1][4 * q + 0]) + bq.x + y1.x;
+                    o.y = (acc[0][4 * q + 1] + acc[1][4 * q + 1]) + bq.y + y1.y;
+                    o.z = (acc[0][4 * q + 2] + acc[1][4 * q + 2]) + bq.z + y1.z;
+                    o.w = (acc[0][4 * q + 3] + acc[1][4 * q + 3]) + bq.w + y1.w;
+                    *reinterpret_cast<float4*>(out + t * D + n0 + 4 * kh + 8 * q) = o;
+                }
+            }
+        }
+        if (more) store_a();  // bufA was last read two barriers ago
+        __syncthreads();      // next tile's bufA in place; bufH free
     }
-#undef SPGT_TAIL_LOADW
-#undef SPGT_TAIL_MMA
-#undef SPGT_TAIL_ZERO
 }
 
 namespace {
@@ -1012,8 +1088,10 @@ extern "C" int spgt_encoder_tail_forward(const float* attn_out, int64_t ld_attn,
     if (tokens == 0) return SPGT_OK;
     if (ceil_div(tokens, (int64_t)32) > INT32_MAX)
         return fail(SPGT_ERR_INVALID_ARGUMENT, "encoder_tail_forward: too many tokens");
-    const unsigned grid = (unsigned)ceil_div(tokens, (int64_t)32);
-    const size_t lds = (size_t)32 * (129 + 257) * sizeof(float);
+    const unsigned grid = (unsigned)std::min<int64_t>(ceil_div(tokens, (int64_t)32), device_cu_count());
+    // attention tile + y1 + hidden tile + biases; at least half of the CU's LDS (one workgroup per CU anyway:
+    // a wave uses most of its SIMD's registers)
+    const size_t lds = std::max<size_t>(((size_t)32 * ((size_t)attn_features + 4 + 132 + 260) + 512) * sizeof(float), 84 * 1024);
     static const hipError_t opt136 = hipFuncSetAttribute(reinterpret_cast<const void*>(encoder_tail_k<136>),
                                                          hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
     static const hipError_t opt128 = hipFuncSetAttribute(reinterpret_cast<const void*>(encoder_tail_k<128>),

@@ -128,13 +128,6 @@ def encoder_tail_supported(attn_features: int, dim_hidden: int, ffn_hidden: int)
     return bool(_lib.load().spgt_encoder_tail_supported(int(attn_features), int(dim_hidden), int(ffn_hidden)))
 
 
-def encoder_tail_pays(tokens: int, device) -> bool:
-    """The one-launch tail re-reads its 82k weights for every 32 tokens; it wins while launches and short
-    grids dominate.  From four 64-token tiles per CU on, three fused_linear launches (weights resident in
-    registers, intermediates through memory) are faster: 254 against 306 us at 159k tokens."""
-    return int(tokens) < 256 * torch.cuda.get_device_properties(device).multi_processor_count
-
-
 def fused_encoder_tail(attn_out: Tensor, x: Tensor, fc_weight_kn: Tensor, fc_bias: Tensor, ffn1_weight_kn: Tensor,
                        ffn1_bias: Tensor, ffn2_weight_kn: Tensor, ffn2_bias: Tensor, activation: str) -> Tensor:
     """y1 = x + attn_out @ fc_weight_kn + fc_bias;  returns y1 + act(y1 @ ffn1_weight_kn + ffn1_bias) @ ffn2_weight_kn

@@ -30,7 +30,7 @@ from ..extension.bind.galerkin_attention import (galerkin_attention_fused, multi
                                                  multihead_projection_layernorm_with_position_rrc_cuda,
                                                  multihead_projection_with_position_rrc_cuda)
 from . import truncated_dft
-from ..extension.bind.linear import encoder_tail_pays, encoder_tail_supported, fused_encoder_tail, fused_linear
+from ..extension.bind.linear import encoder_tail_supported, fused_encoder_tail, fused_linear
 from .layer import (FeedForward, activation_name, always_dropout, fused_linear_usable, gpu_inference,
                     linear_weight_kn, make_activation)
 
@@ -141,8 +141,7 @@ class Sp_EncoderLayer(nn.Module):
         att, ffn = self.attention_layer, self.ffn_layer
         if (att.fc_droprate == 0 and ffn.droprate == 0 and gpu_inference(X, *self.parameters()) and
                 encoder_tail_supported(att.fc_layer.in_features, att.fc_layer.out_features, ffn.layer1.out_features)
-                and ffn.layer2.out_features == att.fc_layer.out_features
-                and encoder_tail_pays(X.numel() // X.size(-1), X.device)):
+                and ffn.layer2.out_features == att.fc_layer.out_features):
             # output projection, both residual adds and the feed-forward net in one launch
             A = att.attend(X, X, X, position)
             return fused_encoder_tail(A, X.contiguous(), linear_weight_kn(att.fc_layer), att.fc_layer.bias,
