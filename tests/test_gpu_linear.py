@@ -208,3 +208,25 @@ def test_encoder_tail(gpu, K1, T, act):
     want = y1 + _expected(y1, w1, b1, act, None, False) @ w2.double() + b2.double()
     assert got.shape == want.shape
     assert (got - want).abs().max().item() <= 2e-5 * max(1.0, want.abs().max().item())
+
+@pytest.mark.parametrize("K1", [128, 136])
+@pytest.mark.parametrize("T", [8192 + 5, 70001])
+def test_encoder_tail_many_tiles(gpu, K1, T):
+    """More 32-token tiles than compute units, so that workgroups loop (a tile in LDS, the next one's rows in
+    flight) and some take one tile more than others; a ragged last tile.  Expected values in float64 on the GPU.
+    The attention rows are a strided view (row stride K1 + 8)."""
+    from spgt_amd.extension.bind.linear import fused_encoder_tail
+    g = torch.Generator().manual_seed(K1 * 7 + T)
+    wide = torch.randn(T, K1 + 8, generator=g).to(gpu)
+    a = wide[:, 8:]
+    x = torch.randn(T, 128, generator=g).to(gpu)
+    wfc, bfc = (torch.randn(K1, 128, generator=g) / K1 ** 0.5).to(gpu), torch.randn(128, generator=g).to(gpu)
+    w1, b1 = (torch.randn(128, 256, generator=g) / 128 ** 0.5).to(gpu), torch.randn(256, generator=g).to(gpu)
+    w2, b2 = (torch.randn(256, 128, generator=g) / 16.0).to(gpu), torch.randn(128, generator=g).to(gpu)
+    got = fused_encoder_tail(a, x, wfc, bfc, w1, b1, w2, b2, "silu").double()
+    y1 = x.double() + a.double() @ wfc.double() + bfc.double()
+    want = y1 + _expected(y1, w1, b1, "silu", None, False) @ w2.double() + b2.double()
+    assert (got - want).abs().max().item() <= 2e-5 * max(1.0, want.abs().max().item())
+    # a second call on the same inputs gives the same bits (fixed summation order, no atomics)
+    again = fused_encoder_tail(a, x, wfc, bfc, w1, b1, w2, b2, "silu").double()
+    assert torch.equal(got, again)
