@@ -985,6 +985,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
             }
             __builtin_amdgcn_sched_barrier(0);
         }
+        // the compiler does not know that set P was written by MFMAs: keep any read of it the needed distance away
+#pragma unroll
+        for (int c = 0; c < NCB; ++c) mfma_acc_done(acc[P][c]);
         if (more) store_x((int)((i + 1) & 1));
         __syncthreads();  // next tile in place; this tile's buffer free for the tile after
     };
@@ -1007,16 +1010,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         } else {
             // the last tile went into set 0
 #pragma unroll
-            for (int c = 0; c < NCB; ++c) mfma_acc_done(acc[0][c]);
-#pragma unroll
             for (int u = 0; u < 4 * NCB; ++u) quarter(std::integral_constant<int, 0>{}, u / 4, u % 4, tprev0 + tk);
             return;
         }
     }
     if (tprev0 >= 0) {
         // the last tile went into set 1
-#pragma unroll
-        for (int c = 0; c < NCB; ++c) mfma_acc_done(acc[1][c]);
 #pragma unroll
         for (int u = 0; u < 4 * NCB; ++u) quarter(std::integral_constant<int, 1>{}, u / 4, u % 4, tprev0 + tk);
     }
