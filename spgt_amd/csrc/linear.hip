@@ -680,24 +680,32 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     for (int i = threadIdx.x; i < 512; i += 256)
         bias_s[i] = i < 128 ? bfc[i] : i < 384 ? b1[i - 128] : b2[i - 384];
 
-    // attention rows of a tile: coalesced 16-byte loads into registers, 16-byte LDS writes a tile later
-    float4 stage[NLD];
+    // attention rows of a tile: coalesced 16-byte loads into registers, 16-byte LDS writes a tile later.
+    // Piece e = threadIdx + 256 i of a tile is row e / (K1/4), columns 4 (e % (K1/4)) ..; its offset from the
+    // tile's first row is the same for every tile but for the row clamp (rows past the end read the last row:
+    // their results are never written out).
+    // (named registers: an array reached through these lambdas ends up in scratch memory)
+    static_assert(NLD == 4 || NLD == 5, "attention tile pieces per thread");
+    float4 sg0, sg1, sg2, sg3, sg4;
+    auto piece_row = [&](int i) { return min((int)threadIdx.x + 256 * i, NVEC - 1) / (K1 / 4); };
+    auto piece_col = [&](int i) { return 4 * (min((int)threadIdx.x + 256 * i, NVEC - 1) % (K1 / 4)); };
+    const uint32_t ulda = (uint32_t)lda;
     auto load_a = [&](int64_t tile) {
         const int64_t t0 = tile * TT;
-#pragma unroll
-        for (int i = 0; i < NLD; ++i) {
-            const int e = threadIdx.x + 256 * i;
-            const int64_t row = t0 + e / (K1 / 4);
-            stage[i] = (e < NVEC && row < T) ? *reinterpret_cast<const float4*>(a + row * lda + 4 * (e % (K1 / 4)))
-                                             : make_float4(0.f, 0.f, 0.f, 0.f);
-        }
+        const float* const base = a + t0 * lda;
+        const int lastrow = (int)min((int64_t)TT - 1, T - 1 - t0);  // wave-uniform
+        auto ld = [&](int i) {
+            return *reinterpret_cast<const float4*>(base + (uint32_t)min(piece_row(i), lastrow) * ulda + (uint32_t)piece_col(i));
+        };
+        sg0 = ld(0); sg1 = ld(1); sg2 = ld(2); sg3 = ld(3);
+        if (NLD > 4) sg4 = ld(4);
     };
     auto store_a = [&]() {
-#pragma unroll
-        for (int i = 0; i < NLD; ++i) {
-            const int e = threadIdx.x + 256 * i;
-            if (e < NVEC) *reinterpret_cast<float4*>(bufA + (e / (K1 / 4)) * PA + 4 * (e % (K1 / 4))) = stage[i];
-        }
+        auto st = [&](int i, const float4& v) {
+            if ((int)threadIdx.x + 256 * i < NVEC) *reinterpret_cast<float4*>(bufA + piece_row(i) * PA + piece_col(i)) = v;
+        };
+        st(0, sg0); st(1, sg1); st(2, sg2); st(3, sg3);
+        if (NLD > 4) st(4, sg4);
     };
     // acc0/acc1 += src[tk][k] * w over k-step groups [0, NG) of four; group g goes to chain chain_of(g).
     // Operands are read from LDS 16 k-steps ahead of their MFMAs.
@@ -835,6 +843,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                         acc[g & 1] = mfma32(wC[4 * (g0 + g) + e], comp(xv[(g0 / GB) & 1][g], e), acc[g & 1]);
                 __builtin_amdgcn_sched_barrier(0);
             }
+            // the next tile's attention rows go to LDS before this tile's stores are issued: the wait for
+            // their loads would otherwise also wait for those stores (bufA was last read two barriers ago)
+            if (more) store_a();
             if (tok) {
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
@@ -849,8 +860,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                 }
             }
         }
-        if (more) store_a();  // bufA was last read two barriers ago
-        __syncthreads();      // next tile's bufA in place; bufH free
+        __syncthreads();  // next tile's bufA in place; bufH free
     }
 }
 
