@@ -375,7 +375,12 @@ def kernel_rooflines(dev):
         hdn = rn(T, 256)
         w5 = rn(256, 128) / 16.0
         mfma(f"linear_256_to_128_residual_T{tag}", 2 * T * 256 * 128, lambda: ln.fused_linear(hdn, w5, bias, "none", res))
-        del xt_, res, hdn
+        # an encoder layer after the attention core in one launch (output projection 136 -> 128, residuals, FFN 256)
+        att = rn(T, 136)
+        wfc = rn(136, 128) / 11.7
+        mfma(f"encoder_tail_136_128_256_T{tag}", 2 * T * (136 * 128 + 2 * 128 * 256),
+             lambda: ln.fused_encoder_tail(att, res, wfc, bias, w4, b4, w5, bias, "silu"))
+        del xt_, res, hdn, att
     Tf = 4 * 211 * 211
     xf_, yf_ = rn(Tf, 64), rn(Tf, 64)
     w6, b6 = rn(64, 64) / 8.0, rn(64)
