@@ -275,6 +275,14 @@ int spgt_conv3x3_resample(const float* x, const float* weight, const float* bias
 int spgt_bias_activation_nchw(float* x, const float* bias, int N, int C, int64_t HW, int activation,
                               int activation_count, spgt_stream_t stream);
 
+/* The end of the model's forward (Sp_GalerkinTransformer2D.forward, network/sp_model.py:109-111) in one pass:
+ * out = x * scale + shift (the target normalizer's inverse_transform with scale = std + eps, shift = mean;
+ * multiply and add rounded separately, like the two tensor operations), and with zero_boundary the outermost
+ * rows and columns of the [H, W] grid set to zero (the Dirichlet branch pads the interior with zeros).
+ * x, out [N, H, W, C]; scale and shift point to one value each, or with per_point to H*W*C values. */
+int spgt_denormalize_boundary(const float* x, const float* scale, const float* shift, int per_point, float* out,
+                              int N, int H, int W, int C, int zero_boundary, spgt_stream_t stream);
+
 /* 1 when spgt_linear_forward has a kernel for this shape (in_features 64, 128, 136 or 256;
  * out_features a multiple of 32), else 0. */
 int spgt_linear_supported(int in_features, int out_features);

@@ -17,6 +17,13 @@
 // and tokens along lanes, so a lane stores four 16-byte pieces of its token's
 // row.  LDS reads for the next batch of MFMAs are issued before the current
 // batch so that their latency hides behind the matrix pipe.
+//
+// Kernels in this file, all on that scheme:
+//   linear_tm_k        any supported shape; several workgroups per CU share the matrix pipes
+//   linear_ws_k        long inputs, whole 128-column groups: one MFMA wave per SIMD fed by load and store waves
+//   linear_resident_k  the packed 128 -> 384 projection on long inputs: one wave per SIMD, all weights resident
+//   ffn_scalar_k       two-layer net with one output feature (regression head)
+//   encoder_tail_k     output projection + residuals + feed-forward net of an encoder layer, all weights resident
 #include <type_traits>
 
 #include "spgt_device.h"
@@ -26,13 +33,7 @@ namespace spgt {
 
 namespace {
 
-__device__ __forceinline__ float activate(float v, int act) {
-    if (act == SPGT_ACT_RELU) return fmaxf(v, 0.f);
-    if (act == SPGT_ACT_SILU) return v * __builtin_amdgcn_rcpf(1.f + __expf(-v));
-    return v;
-}
-
-// The same on N values with the choice made once, outside the loop: per-element calls with a run-time
+// Activation of N values with the choice made once, outside the loop: per-element calls with a run-time
 // `act` compile to a branch tree per element, which is most of an epilogue's time.
 template <int N>
 __device__ __forceinline__ void activate_all(float (&v)[N], int act) {

@@ -497,6 +497,55 @@ extern "C" int spgt_bilinear_resample(const float* src, const float* pre_bias, f
                            ResampleAct{pre_activation, pre_activation_count, post_activation}, stream);
 }
 
+namespace spgt {
+namespace {
+
+// The last two steps of the model's forward (Sp_GalerkinTransformer2D.forward, network/sp_model.py:109-111):
+// out = x * scale + shift (the target normalizer's inverse, rounded after the multiply and after the add like
+// the two tensor operations it stands for), then zero on the boundary of the [H, W] grid (Dirichlet condition:
+// the reference pads the interior with zeros).  x, out [N, H, W, C]; scale and shift hold one value, or one per
+// (h, w, c) when per_point is set.  grid (ceil(H*W*C / 256), N), block 256.
+__global__ __launch_bounds__(256) void denormalize_boundary_k(const float* __restrict__ x, const float* __restrict__ scale,
+                                                              const float* __restrict__ shift, int per_point,
+                                                              float* __restrict__ out, int H, int W, int C,
+                                                              int zero_boundary) {
+    const int64_t plane = (int64_t)H * W * C;
+    const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (e >= plane) return;
+    const int64_t i = (int64_t)blockIdx.y * plane + e;
+    const int w = (int)((e / C) % W);
+    const int h = (int)(e / ((int64_t)C * W));
+    float v = 0.f;
+    if (!zero_boundary || (h > 0 && h < H - 1 && w > 0 && w < W - 1)) {
+#pragma clang fp contract(off)  // two roundings, as two tensor operations give; the default would fuse them
+        const float sc = scale[per_point ? e : 0], sh = shift[per_point ? e : 0];
+        const float prod = x[i] * sc;
+        v = prod + sh;
+    }
+    out[i] = v;
+}
+
+}  // namespace
+}  // namespace spgt
+
+extern "C" int spgt_denormalize_boundary(const float* x, const float* scale, const float* shift, int per_point,
+                                         float* out, int N, int H, int W, int C, int zero_boundary,
+                                         hipStream_t stream) {
+    if (!x || !scale || !shift || !out)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "denormalize_boundary: null pointer argument");
+    if (N <= 0 || H <= 0 || W <= 0 || C <= 0)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "denormalize_boundary: sizes must be positive");
+    if (N > 65535) return fail(SPGT_ERR_INVALID_ARGUMENT, "denormalize_boundary: N exceeds 65535");
+    if (!aligned4(x) || !aligned4(scale) || !aligned4(shift) || !aligned4(out))
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "denormalize_boundary: operands must be 4-byte aligned");
+    const int64_t plane = (int64_t)H * W * C;
+    if (ceil_div(plane, (int64_t)256) > INT32_MAX)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "denormalize_boundary: grid too large");
+    hipLaunchKernelGGL(denormalize_boundary_k, dim3((unsigned)ceil_div(plane, (int64_t)256), N), dim3(256), 0, stream, x,
+                       scale, shift, per_point ? 1 : 0, out, H, W, C, zero_boundary ? 1 : 0);
+    return check_launch("denormalize_boundary");
+}
+
 extern "C" int spgt_bias_activation_nchw(float* x, const float* bias, int N, int C, int64_t HW, int activation,
                                          int activation_count, hipStream_t stream) {
     if (!x) return fail(SPGT_ERR_INVALID_ARGUMENT, "bias_activation_nchw: null pointer argument");

@@ -318,6 +318,28 @@ def _bias_activation_nchw_(X: Tensor, bias, activation=None, count: int = 1) -> 
     return X
 
 
+def _denormalize_boundary(X: Tensor, scale: Tensor, shift: Tensor, zero_boundary: bool) -> Tensor:
+    """X * scale + shift on X [N, H, W, C], zero on the grid's boundary if asked; scale and shift hold one
+    value or H*W*C values."""
+    require_gpu_f32("X", X)
+    require_gpu_f32("scale", scale)
+    require_gpu_f32("shift", shift)
+    if X.dim() != 4:
+        raise ValueError("X must be [N, H, W, C]")
+    N, H, W, C = X.shape
+    if scale.numel() != shift.numel() or scale.numel() not in (1, H * W * C):
+        raise ValueError("scale and shift must hold one value or H*W*C values")
+    if zero_boundary and min(H, W) < 2:
+        raise ValueError("a grid with fewer than two rows or columns has no interior to pad")
+    out = torch.empty_like(X)
+    if X.numel() == 0:
+        return out
+    with torch.cuda.device(X.device):
+        check(_lib.load().spgt_denormalize_boundary(ptr(X), ptr(scale), ptr(shift), int(scale.numel() > 1), ptr(out),
+                                                    N, H, W, C, int(bool(zero_boundary)), stream_of(X)))
+    return out
+
+
 def _conv3x3_resample(X: Tensor, weight: Tensor, bias, size, pre_activation=None, post_activation=None) -> Tensor:
     """post(interpolate(pre(conv3x3(X, weight, padding=1) + bias))) for X [N, H, W, Cin] channels-last with
     Cin <= 4: [N, Cout, H', W'] without the full-resolution convolution output ever being stored."""
@@ -346,6 +368,7 @@ def _conv3x3_resample(X: Tensor, weight: Tensor, bias, size, pre_activation=None
 
 dexts = SimpleNamespace(
     conv3x3_resample=_conv3x3_resample,
+    denormalize_boundary=_denormalize_boundary,
     truncated_dft_rows_supported=_truncated_dft_rows_supported,
     truncated_dft_rows=_truncated_dft_rows,
     spectral_modes_middle_supported=_spectral_modes_middle_supported,
@@ -452,6 +475,12 @@ def bilinear_resample(X: Tensor, size, src_nhwc: bool = False, dst_nhwc: bool = 
 def bias_activation_nchw_(X: Tensor, bias, activation=None, count: int = 1) -> Tensor:
     """In place: X = activation^count(X + bias[c]) on [N, C, ...] (inference only)."""
     return dexts.bias_activation_nchw_(X, None if bias is None else bias.detach(), activation, count)
+
+
+def denormalize_boundary(X: Tensor, scale: Tensor, shift: Tensor, zero_boundary: bool) -> Tensor:
+    """The end of the model's forward in one pass: X * scale + shift on [N, H, W, C] (multiply and add rounded
+    separately), then zero on the outermost rows and columns of the grid if asked (inference only)."""
+    return dexts.denormalize_boundary(X.detach(), scale, shift, zero_boundary)
 
 
 def truncated_dft_rows_supported(r: int, channels: int, modes: int) -> bool:

@@ -8,6 +8,7 @@ import torch
 import torch.nn.functional as F
 from torch import Tensor, nn
 
+from ..extension.bind.datamove import denormalize_boundary
 from ..extension.bind.linear import fused_linear, linear_supported
 from .layer import FeedForward, always_dropout, gpu_inference
 from .model import DownScaler2D, UpScaler2D
@@ -109,7 +110,47 @@ class Sp_GalerkinTransformer2D(nn.Module):
         X = self.encoder_mixer(X, position)
         X = always_dropout(self.up_scaler(X), self.droprate)
         X = self.decoder_regressor(X, grid)
+        dirichlet = self.boundary_condition == "dirichlet"
+        # (a grid with fewer than two rows or columns has no interior: the padded result would change shape)
+        affine = self._normalizer_affine(X) if gpu_inference(X) and min(X.shape[1:3]) >= 2 else None
+        if affine is not None:
+            # de-normalisation and the zero boundary in one pass
+            return denormalize_boundary(X, affine[0], affine[1], dirichlet)
         X = self.normalizer.inverse_transform(X)
-        if self.boundary_condition == "dirichlet":
+        if dirichlet:
             X = F.pad(X[:, 1:-1, 1:-1], (0, 0, 1, 1, 1, 1), "constant", 0.0)
         return X
+
+    def _normalizer_affine(self, X: Tensor):
+        """(std + eps, mean) of the target normalizer as device tensors of one value or of one value per grid
+        point and channel, or None when the normalizer is of another kind.  Cached per device."""
+        nz = self.normalizer
+        if not all(hasattr(nz, k) for k in ("mean", "std", "eps")):
+            return None
+        key = (id(nz.mean), id(nz.std), getattr(nz.mean, "_version", None), getattr(nz.std, "_version", None), nz.eps,
+               X.device, tuple(X.shape[1:]))
+        cache = getattr(self, "_spgt_affine", None)
+        if cache is not None and cache[0] == key:
+            return cache[1]
+        mean, std = nz.mean, nz.std
+        if isinstance(mean, Tensor) != isinstance(std, Tensor):
+            return None
+        if isinstance(mean, Tensor):
+            if mean.dtype != torch.float32 or std.dtype != torch.float32:
+                return None
+            scale = (std + nz.eps).to(X.device)
+            shift = mean.to(X.device)
+            if scale.numel() != 1 or shift.numel() != 1:
+                try:
+                    scale = scale.expand(X.shape[1:]).contiguous()
+                    shift = shift.expand(X.shape[1:]).contiguous()
+                except RuntimeError:
+                    return None
+            else:
+                scale, shift = scale.reshape(1).contiguous(), shift.reshape(1).contiguous()
+        else:
+            # python numbers: torch multiplies a float32 tensor by float32(std + eps)
+            scale = torch.tensor([float(std) + float(nz.eps)], dtype=torch.float32, device=X.device)
+            shift = torch.tensor([float(mean)], dtype=torch.float32, device=X.device)
+        self._spgt_affine = (key, (scale, shift))
+        return scale, shift

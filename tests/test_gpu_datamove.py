@@ -363,3 +363,35 @@ def test_conv3x3_resample(gpu, N, H, W, cin, cout, size, pre, post):
     # fp32 source coordinates (as torch's own kernel computes them) times the slope of a random convolution
     # output reach 1e-5 of the output scale at 211 -> 122; the bound is 3e-5, far inside the path's 1e-4
     assert (got - want).abs().max().item() <= 3e-5 * max(1.0, want.abs().max().item())
+
+
+@pytest.mark.parametrize("shape", [(2, 9, 7, 1), (1, 2, 5, 3), (3, 2, 2, 2), (4, 211, 211, 1)])
+@pytest.mark.parametrize("per_point", [False, True])
+@pytest.mark.parametrize("zero_boundary", [False, True])
+def test_denormalize_boundary_matches_tensor_ops(gpu, shape, per_point, zero_boundary):
+    """The end of the model's forward (network/sp_model.py:109-111): X * (std + eps) + mean, then the interior
+    padded with zeros.  Bit-exact against the tensor operations it replaces."""
+    import torch.nn.functional as F
+    from spgt_amd.extension.bind.datamove import denormalize_boundary
+    g = torch.Generator().manual_seed(sum(shape))
+    X = torch.randn(*shape, generator=g).to(gpu)
+    if per_point:
+        scale = (torch.rand(*shape[1:], generator=g) + 0.5).to(gpu)
+        shift = torch.randn(*shape[1:], generator=g).to(gpu)
+    else:
+        scale = torch.tensor([1.7 + 1e-5], device=gpu)
+        shift = torch.tensor([-0.3], device=gpu)
+    got = denormalize_boundary(X, scale, shift, zero_boundary)
+    want = X * scale + shift
+    if zero_boundary:
+        want = F.pad(want[:, 1:-1, 1:-1], (0, 0, 1, 1, 1, 1), "constant", 0.0)
+    assert got.shape == want.shape and torch.equal(got, want)
+
+
+def test_denormalize_boundary_rejects_bad_shapes(gpu):
+    from spgt_amd.extension.bind.datamove import denormalize_boundary
+    X = torch.zeros(2, 4, 4, 1, device=gpu)
+    with pytest.raises(ValueError):
+        denormalize_boundary(X, torch.ones(3, device=gpu), torch.ones(3, device=gpu), True)
+    with pytest.raises(ValueError):
+        denormalize_boundary(X[0], torch.ones(1, device=gpu), torch.ones(1, device=gpu), True)
