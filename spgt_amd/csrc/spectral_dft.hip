@@ -359,6 +359,110 @@ __global__ __launch_bounds__(256) void spectral_rows_expand_k(
     }
 }
 
+// The end of Sp_SpectralConv2D.forward (network/sp_layer.py:132, 149-155) in one pass over the grid:
+//   out[row, w, o] = act( sum_c x[row, w, c] W[c, o] + bias[o] + sum_j table[w, j] U[row, o, j] )
+// i.e. the residual Linear, the inverse DFT along w of the retained modes, their sum and the activation;
+// the inverse transform's result never goes to memory.  64 channels in and out, planar U [N][2m][r][64].
+// Both terms are MFMA products with output channels along the accumulator's registers and grid points along
+// its lanes (so a lane stores four 16-byte pieces of its grid point's row): A = W resp. U in registers,
+// B = x tile (from a wave-private LDS tile, 16-byte reads, lane (w, kh) takes channels kh*32 + kk) resp.
+// table entries (handed over in operand order, tabA[tile][kk][lane] = table[32 tile + lane%32][2kk +
+// lane/32], zero outside).  A wave owns one half of the channels and every second 32-point tile of a grid
+// row; no barriers.  grid (rows), block 256.
+__global__ __launch_bounds__(256) void spectral_inverse_linear_k(
+    const float* __restrict__ U, const float* __restrict__ tabA, const float* __restrict__ x,
+    const float* __restrict__ Wkn, const float* __restrict__ bias, int act, float* __restrict__ out, int r, int m2) {
+    constexpr int C = 64, PX = C + 4;
+    __shared__ __attribute__((aligned(16))) float xs[4][32 * PX];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int tk = lane & 31;
+    const int kh = lane >> 5;
+    const int cb = wave & 1;
+    const int64_t row = blockIdx.x;
+    const int64_t n = row / r;
+    const int64_t h = row - n * r;
+    const int WT = (r + 31) / 32;
+    const int KS = m2 / 2;
+
+    float wreg[32];  // W[c = kh*32 + kk][o = cb*32 + tk]
+#pragma unroll
+    for (int kk = 0; kk < 32; ++kk) wreg[kk] = Wkn[(kh * 32 + kk) * C + cb * 32 + tk];
+    float ureg[16];  // U[j = 2kk + kh][o]
+    {
+        const float* up = U + (n * m2 * r + h) * (int64_t)C + cb * 32 + tk;  // U[n][j][h][o]
+#pragma unroll
+        for (int kk = 0; kk < 16; ++kk) ureg[kk] = (2 * kk + kh < m2) ? up[(int64_t)(2 * kk + kh) * r * C] : 0.f;
+    }
+    // bias in accumulator layout: element 4q + e belongs to channel cb*32 + 8q + 4kh + e
+    v16f bo;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const float4 b4 = bias ? *reinterpret_cast<const float4*>(bias + cb * 32 + 8 * q + 4 * kh) : make_float4(0.f, 0.f, 0.f, 0.f);
+        bo[4 * q + 0] = b4.x; bo[4 * q + 1] = b4.y; bo[4 * q + 2] = b4.z; bo[4 * q + 3] = b4.w;
+    }
+    float* const xw = xs[wave];
+    const float* const xrow = x + row * (int64_t)r * C;
+    float* const orow = out + row * (int64_t)r * C + cb * 32 + 4 * kh;
+
+    // this wave's tiles: wave>>1, wave>>1 + 2, ...; tile rows past the end of the grid row read its last point
+    // (named registers and macros: a register array that lives across the loop ends up in scratch memory)
+    float4 s0, s1, s2, s3, s4, s5, s6, s7;
+#define SPGT_X_PIECE(WT_, I_) \
+    (*reinterpret_cast<const float4*>(xrow + (int64_t)min((WT_) * 32 + ((lane + 64 * (I_)) >> 4), r - 1) * C + 4 * (lane & 15)))
+#define SPGT_LOAD_X_TILE(WT_)                                                                            \
+    s0 = SPGT_X_PIECE(WT_, 0); s1 = SPGT_X_PIECE(WT_, 1); s2 = SPGT_X_PIECE(WT_, 2); s3 = SPGT_X_PIECE(WT_, 3); \
+    s4 = SPGT_X_PIECE(WT_, 4); s5 = SPGT_X_PIECE(WT_, 5); s6 = SPGT_X_PIECE(WT_, 6); s7 = SPGT_X_PIECE(WT_, 7);
+#define SPGT_STORE_X_PIECE(I_, V_) \
+    *reinterpret_cast<float4*>(xw + ((lane + 64 * (I_)) >> 4) * PX + 4 * (lane & 15)) = V_;
+    int wt = wave >> 1;
+    if (wt < WT) { SPGT_LOAD_X_TILE(wt) }
+    for (; wt < WT; wt += 2) {
+        SPGT_STORE_X_PIECE(0, s0) SPGT_STORE_X_PIECE(1, s1) SPGT_STORE_X_PIECE(2, s2) SPGT_STORE_X_PIECE(3, s3)
+        SPGT_STORE_X_PIECE(4, s4) SPGT_STORE_X_PIECE(5, s5) SPGT_STORE_X_PIECE(6, s6) SPGT_STORE_X_PIECE(7, s7)
+        if (wt + 2 < WT) { SPGT_LOAD_X_TILE(wt + 2) }
+        float ta[16];
+#pragma unroll
+        for (int kk = 0; kk < 16; ++kk) ta[kk] = (kk < KS) ? tabA[((int64_t)wt * 16 + kk) * 64 + lane] : 0.f;
+        v16f acc = bo;
+        const float* xr = xw + tk * PX + kh * 32;
+        float4 xv[8];
+#pragma unroll
+        for (int g = 0; g < 8; ++g) xv[g] = *reinterpret_cast<const float4*>(xr + 4 * g);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int g = 0; g < 8; ++g) {
+            acc = mfma32(wreg[4 * g + 0], xv[g].x, acc);
+            acc = mfma32(wreg[4 * g + 1], xv[g].y, acc);
+            acc = mfma32(wreg[4 * g + 2], xv[g].z, acc);
+            acc = mfma32(wreg[4 * g + 3], xv[g].w, acc);
+        }
+#pragma unroll
+        for (int kk = 0; kk < 16; ++kk)
+            if (kk < KS) acc = mfma32(ureg[kk], ta[kk], acc);
+        float y[16];
+#pragma unroll
+        for (int q = 0; q < 16; ++q) y[q] = acc[q];
+        if (act == SPGT_ACT_RELU) {
+#pragma unroll
+            for (int q = 0; q < 16; ++q) y[q] = fmaxf(y[q], 0.f);
+        } else if (act == SPGT_ACT_SILU) {
+#pragma unroll
+            for (int q = 0; q < 16; ++q) y[q] = y[q] * __builtin_amdgcn_rcpf(1.f + __expf(-y[q]));
+        }
+        // y[4q + e] = out[w = wt*32 + tk][o = cb*32 + 8q + 4kh + e]
+        const int w = wt * 32 + tk;
+        if (w < r) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                *reinterpret_cast<float4*>(orow + (int64_t)w * C + 8 * q) = make_float4(y[4 * q], y[4 * q + 1], y[4 * q + 2], y[4 * q + 3]);
+        }
+    }
+#undef SPGT_LOAD_X_TILE
+#undef SPGT_X_PIECE
+#undef SPGT_STORE_X_PIECE
+}
+
 }  // namespace spgt
 
 using namespace spgt;
@@ -462,4 +566,30 @@ extern "C" int spgt_spectral_modes_middle(const float* Y, const float* table_h, 
     hipLaunchKernelGGL(spectral_rows_expand_k, dim3(modes, N, ceil_div(r, rows_per_wg)), dim3(256), lds2, stream, O,
                        reinterpret_cast<const float2*>(table_h_inverse), U, r, Cout, modes, rows_per_wg);
     return check_launch("spectral_modes_middle");
+}
+
+extern "C" int spgt_spectral_inverse_linear_supported(int r, int in_features, int out_features, int modes) {
+    return (r > 0 && r <= 1024 && in_features == 64 && out_features == 64 && modes > 0 && 2 * modes <= 32 &&
+            2 * modes <= r) ? 1 : 0;
+}
+
+extern "C" int spgt_spectral_inverse_linear(const float* U, const float* table_operand, const float* x,
+                                            const float* weight_kn, const float* bias, int activation, float* out,
+                                            int64_t rows, int r, int channels, int modes, hipStream_t stream) {
+    if (!U || !table_operand || !x || !weight_kn || !out)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "spectral_inverse_linear: null pointer argument");
+    if (!spgt_spectral_inverse_linear_supported(r, channels, channels, modes))
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "spectral_inverse_linear: needs 64 channels, 2*modes <= min(32, r), r <= 1024");
+    if (rows <= 0 || rows % r != 0 || rows > INT32_MAX)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "spectral_inverse_linear: rows must be a positive multiple of r");
+    if (activation != SPGT_ACT_NONE && activation != SPGT_ACT_RELU && activation != SPGT_ACT_SILU)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "spectral_inverse_linear: unknown activation");
+    if (!aligned4(U) || !aligned4(table_operand) || !aligned16(x) || !aligned4(weight_kn) || !aligned16(out) ||
+        (bias && !aligned16(bias)))
+        return fail(SPGT_ERR_INVALID_ARGUMENT,
+                    "spectral_inverse_linear: x, out and bias must be 16-byte aligned, the rest 4-byte aligned");
+    if (out == x) return fail(SPGT_ERR_INVALID_ARGUMENT, "spectral_inverse_linear: out must not alias x");
+    hipLaunchKernelGGL(spectral_inverse_linear_k, dim3((unsigned)rows), dim3(256), 0, stream, U, table_operand, x,
+                       weight_kn, bias, activation, out, r, 2 * modes);
+    return check_launch("spectral_inverse_linear");
 }

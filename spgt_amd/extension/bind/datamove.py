@@ -340,6 +340,42 @@ def _denormalize_boundary(X: Tensor, scale: Tensor, shift: Tensor, zero_boundary
     return out
 
 
+def _spectral_inverse_linear_supported(r: int, cin: int, cout: int, modes: int) -> bool:
+    return bool(_lib.load().spgt_spectral_inverse_linear_supported(int(r), int(cin), int(cout), int(modes)))
+
+
+def _spectral_inverse_linear(U: Tensor, table_operand: Tensor, X: Tensor, weight_kn: Tensor, bias, activation) -> Tensor:
+    """act(X @ weight_kn + bias + inverse row DFT of U): U planar [N, 2m, r, C], X [N, r, r, C] -> [N, r, r, C]."""
+    for name, t in (("U", U), ("table_operand", table_operand), ("X", X), ("weight_kn", weight_kn)):
+        require_gpu_f32(name, t)
+    if activation not in _ACT:
+        raise ValueError("activation must be None, 'none', 'relu' or 'silu'")
+    if X.dim() != 4 or X.shape[1] != X.shape[2]:
+        raise ValueError("X must be [N, r, r, C]")
+    N, r, _, C = X.shape
+    if U.dim() != 4 or U.shape[0] != N or U.shape[2] != r or U.shape[3] != C or U.shape[1] % 2:
+        raise ValueError("U must be planar [N, 2*modes, r, C]")
+    modes = U.shape[1] // 2
+    if tuple(weight_kn.shape) != (C, C):
+        raise ValueError("weight_kn must be [C, C]")
+    if tuple(table_operand.shape) != ((r + 31) // 32, 16, 64):
+        raise ValueError("table_operand must be [ceil(r/32), 16, 64]")
+    if bias is not None:
+        require_gpu_f32("bias", bias)
+        if bias.numel() != C:
+            raise ValueError(f"bias has {bias.numel()} elements, expected {C}")
+    if not _spectral_inverse_linear_supported(r, C, C, modes):
+        raise ValueError("spectral_inverse_linear: needs 64 channels, 2*modes <= min(32, r), r <= 1024")
+    out = torch.empty_like(X)
+    if X.numel() == 0:
+        return out
+    with torch.cuda.device(X.device):
+        check(_lib.load().spgt_spectral_inverse_linear(ptr(U), ptr(table_operand), ptr(X), ptr(weight_kn),
+                                                       ptr(bias) if bias is not None else None, _ACT[activation],
+                                                       ptr(out), N * r, r, C, modes, stream_of(X)))
+    return out
+
+
 def _conv3x3_resample(X: Tensor, weight: Tensor, bias, size, pre_activation=None, post_activation=None) -> Tensor:
     """post(interpolate(pre(conv3x3(X, weight, padding=1) + bias))) for X [N, H, W, Cin] channels-last with
     Cin <= 4: [N, Cout, H', W'] without the full-resolution convolution output ever being stored."""
@@ -368,6 +404,8 @@ def _conv3x3_resample(X: Tensor, weight: Tensor, bias, size, pre_activation=None
 
 dexts = SimpleNamespace(
     conv3x3_resample=_conv3x3_resample,
+    spectral_inverse_linear_supported=_spectral_inverse_linear_supported,
+    spectral_inverse_linear=_spectral_inverse_linear,
     denormalize_boundary=_denormalize_boundary,
     truncated_dft_rows_supported=_truncated_dft_rows_supported,
     truncated_dft_rows=_truncated_dft_rows,
@@ -475,6 +513,30 @@ def bilinear_resample(X: Tensor, size, src_nhwc: bool = False, dst_nhwc: bool = 
 def bias_activation_nchw_(X: Tensor, bias, activation=None, count: int = 1) -> Tensor:
     """In place: X = activation^count(X + bias[c]) on [N, C, ...] (inference only)."""
     return dexts.bias_activation_nchw_(X, None if bias is None else bias.detach(), activation, count)
+
+
+def spectral_inverse_linear_supported(r: int, cin: int, cout: int, modes: int) -> bool:
+    """True when spectral_inverse_linear has a kernel for this shape."""
+    return dexts.spectral_inverse_linear_supported(r, cin, cout, modes)
+
+
+def inverse_table_operand(table: Tensor) -> Tensor:
+    """The inverse row-DFT table [r, 2m] in the order the fused kernel's lanes read it: [ceil(r/32), 16, 64] with
+    entry (t, kk, l) = table[32 t + l % 32, 2 kk + l // 32], zero outside the table."""
+    r, m2 = table.shape
+    wt = (r + 31) // 32
+    full = torch.zeros(wt * 32, 32, dtype=table.dtype, device=table.device)
+    full[:r, :m2] = table
+    # [t, w', kk, kh] -> [t, kk, kh, w'] -> lanes l = kh*32 + w'
+    return full.view(wt, 32, 16, 2).permute(0, 2, 3, 1).reshape(wt, 16, 64).contiguous()
+
+
+def spectral_inverse_linear(U: Tensor, table_operand: Tensor, X: Tensor, weight_kn: Tensor, bias, activation) -> Tensor:
+    """The end of Sp_SpectralConv2D.forward in one pass: act(X @ weight_kn + bias + y) with y the inverse DFT
+    along w of the planar spectrum U [N, 2m, r, C] (what truncated_dft_rows_inverse(U, table, planar=True)
+    returns); X [N, r, r, C], 64 channels (inference only)."""
+    return dexts.spectral_inverse_linear(U.detach(), table_operand, X.detach(), weight_kn,
+                                         None if bias is None else bias.detach(), activation)
 
 
 def denormalize_boundary(X: Tensor, scale: Tensor, shift: Tensor, zero_boundary: bool) -> Tensor:

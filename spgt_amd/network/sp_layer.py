@@ -176,6 +176,11 @@ class Sp_SpectralConv2D(nn.Module):
             # only the retained modes are ever computed: no FFT, no transposes, no full-size spectrum;
             # the residual Linear, the add and the activation are one kernel
             X0 = X.contiguous()
+            if self.droprate == 0 and truncated_dft.fused_tail_supported(r, cin, cout, m):
+                # ... and the inverse transform along w happens inside that kernel too
+                return truncated_dft.spectral_modes_apply_linear(
+                    X0, self.fourier_weight[0], self.fourier_weight[1], m, linear_weight_kn(self.residual_layer),
+                    self.residual_layer.bias, activation_name(self.activation_layer))
             Y = truncated_dft.spectral_modes_apply(always_dropout(X0, self.droprate), self.fourier_weight[0],
                                                    self.fourier_weight[1], m)
             return fused_linear(X0, linear_weight_kn(self.residual_layer), self.residual_layer.bias,

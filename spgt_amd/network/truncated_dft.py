@@ -24,9 +24,10 @@ from typing import Dict, Tuple
 import torch
 from torch import Tensor
 
-from ..extension.bind.datamove import (spectral_modes_compact, spectral_modes_middle, spectral_modes_middle_supported,
-                                       truncated_dft_rows_forward, truncated_dft_rows_inverse,
-                                       truncated_dft_rows_supported)
+from ..extension.bind.datamove import (inverse_table_operand, spectral_inverse_linear,
+                                       spectral_inverse_linear_supported, spectral_modes_compact, spectral_modes_middle,
+                                       spectral_modes_middle_supported, truncated_dft_rows_forward,
+                                       truncated_dft_rows_inverse, truncated_dft_rows_supported)
 
 _TABLES: Dict[Tuple[int, int, str], Tuple[Tensor, Tensor, Tensor, Tensor]] = {}
 
@@ -59,6 +60,30 @@ def dft_tables(r: int, m: int, device) -> Tuple[Tensor, Tensor, Tensor, Tensor]:
 def supported(r: int, m: int) -> bool:
     """The two retained row windows must not overlap."""
     return 2 * m <= r
+
+
+_OPERAND_TABLES: Dict[Tuple[int, int, str], Tensor] = {}
+
+
+def fused_tail_supported(r: int, cin: int, cout: int, m: int) -> bool:
+    """True when spectral_modes_apply_linear runs in three launches (row DFT, retained modes, inverse row DFT fused
+    with the residual Linear and the activation)."""
+    return (truncated_dft_rows_supported(r, cin, m) and spectral_modes_middle_supported(r, cin, cout, m) and
+            spectral_inverse_linear_supported(r, cin, cout, m))
+
+
+def spectral_modes_apply_linear(x: Tensor, weight_1: Tensor, weight_2: Tensor, m: int, linear_weight_kn: Tensor,
+                                linear_bias, activation) -> Tensor:
+    """act(x @ linear_weight_kn + linear_bias + irfft2(W . truncate(rfft2(x)))) for x [N, r, r, C]: the whole
+    spectral layer after dropout; requires fused_tail_supported."""
+    N, r, _, cin = x.shape
+    fw, gh, ghi, fwi = dft_tables(r, m, x.device)
+    key = (r, m, str(x.device))
+    if key not in _OPERAND_TABLES:
+        _OPERAND_TABLES[key] = inverse_table_operand(fwi)
+    yp = truncated_dft_rows_forward(x, fw, planar=True)             # [N, 2m, r, Cin]
+    up = spectral_modes_middle(yp, gh, ghi, weight_1, weight_2)     # [N, 2m, r, Cout]
+    return spectral_inverse_linear(up, _OPERAND_TABLES[key], x, linear_weight_kn, linear_bias, activation)
 
 
 def spectral_modes_apply(x: Tensor, weight_1: Tensor, weight_2: Tensor, m: int) -> Tensor:

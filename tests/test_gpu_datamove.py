@@ -395,3 +395,36 @@ def test_denormalize_boundary_rejects_bad_shapes(gpu):
         denormalize_boundary(X, torch.ones(3, device=gpu), torch.ones(3, device=gpu), True)
     with pytest.raises(ValueError):
         denormalize_boundary(X[0], torch.ones(1, device=gpu), torch.ones(1, device=gpu), True)
+
+
+
+@pytest.mark.parametrize("N,r,m", [(1, 33, 4), (2, 64, 12), (4, 211, 12), (2, 141, 16), (1, 32, 16)])
+@pytest.mark.parametrize("act", [None, "relu", "silu"])
+def test_spectral_inverse_linear_matches_separate_kernels(gpu, N, r, m, act):
+    """The fused end of the spectral layer against its parts: truncated_dft_rows_inverse + fused_linear with the
+    transform's result as residual (which are tested against the FFT route and a float64 product themselves).
+    Tolerance 2e-6 of the output scale: the fused kernel adds the spectral term in the accumulator, the parts
+    round it to fp32 in memory first."""
+    from spgt_amd.extension.bind.linear import fused_linear
+    from spgt_amd.network.truncated_dft import dft_tables
+    C = 64
+    assert dm.spectral_inverse_linear_supported(r, C, C, m) and not dm.spectral_inverse_linear_supported(r, 32, 32, m)
+    g = torch.Generator().manual_seed(N * 1000 + r + m)
+    x = torch.randn(N, r, r, C, generator=g).to(gpu)
+    U = torch.randn(N, 2 * m, r, C, generator=g).to(gpu)
+    w = (torch.randn(C, C, generator=g) / 8.0).to(gpu)
+    b = torch.randn(C, generator=g).to(gpu)
+    _, _, _, fwi = dft_tables(r, m, gpu)
+    got = dm.spectral_inverse_linear(U, dm.inverse_table_operand(fwi), x, w, b, act)
+    y = dm.truncated_dft_rows_inverse(U, fwi, planar=True)
+    want = fused_linear(x, w, b, act or "none", y)
+    assert got.shape == want.shape
+    assert (got - want).abs().max().item() <= 2e-6 * max(1.0, want.abs().max().item())
+    # and against float64 arithmetic
+    y64 = torch.einsum("wj,njho->nhwo", fwi.double(), U.double())
+    z = x.double() @ w.double() + b.double() + y64
+    z = torch.relu(z) if act == "relu" else (z * torch.sigmoid(z) if act == "silu" else z)
+    assert (got.double() - z).abs().max().item() <= 1e-5 * max(1.0, z.abs().max().item())
+    no_bias = dm.spectral_inverse_linear(U, dm.inverse_table_operand(fwi), x, w, None, act)
+    want_nb = fused_linear(x, w, None, act or "none", y)
+    assert (no_bias - want_nb).abs().max().item() <= 2e-6 * max(1.0, want_nb.abs().max().item())
