@@ -122,16 +122,18 @@ def darcy_bench(dev, with_cpu, steps=30):
             out = model(ad, pd, gd)
         torch.cuda.synchronize()
         eager_ms = (time.perf_counter() - t0) / steps * 1e3
-        # the same forward replayed from a HIP graph (inputs are copied into the captured buffers on every
-        # call; a second input tensor keeps that copy inside the timed region)
+        # the same forward replayed from a HIP graph: the coefficient field is copied into the captured buffer on
+        # every call (a second tensor keeps that copy inside the timed region); the position and grid inputs are
+        # constants of the model's resolution and live in the captured buffers
         graphed = GraphedInference(model, ad, pd, gd)
         a2 = ad.clone()
+        pos_s, grid_s = graphed.static_inputs[1], graphed.static_inputs[2]
         for _ in range(3):
-            gout = graphed(a2, pd, gd)
+            gout = graphed(a2, pos_s, grid_s)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for _ in range(steps):
-            gout = graphed(a2, pd, gd)
+            gout = graphed(a2, pos_s, grid_s)
         torch.cuda.synchronize()
         ms = (time.perf_counter() - t0) / steps * 1e3
         graph_equal = bool(torch.equal(gout, out))
