@@ -230,3 +230,18 @@ def test_encoder_tail_many_tiles(gpu, K1, T):
     # a second call on the same inputs gives the same bits (fixed summation order, no atomics)
     again = fused_encoder_tail(a, x, wfc, bfc, w1, b1, w2, b2, "silu").double()
     assert torch.equal(got, again)
+
+@pytest.mark.parametrize("act", ["none", "relu", "silu"])
+def test_linear_long_inputs_wide_output_without_planes_or_bias(gpu, act):
+    """128 -> 384 on 70001 tokens into one [T, 384] tensor, no bias: the resident-weight kernel's other output
+    form (the packed projection above writes three planes)."""
+    from spgt_amd.extension.bind.linear import fused_linear
+    T = 70001
+    g = torch.Generator().manual_seed(384)
+    x = torch.randn(T, 128, generator=g).to(gpu)
+    w = (torch.randn(128, 384, generator=g) / 128 ** 0.5).to(gpu)
+    got = fused_linear(x, w, None, act)
+    want = _expected(x, w, None, act, None, False)
+    assert got.shape == (T, 384)
+    assert (got.double() - want).abs().max().item() <= 1e-5 * max(1.0, want.abs().max().item())
+    assert torch.equal(got, fused_linear(x, w, None, act))
