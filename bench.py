@@ -359,6 +359,12 @@ def kernel_rooflines(dev):
     mid = rn(4, 128, 122, 122)
     hbm("bilinear_122_to_211_nchw_to_nhwc", 4 * 4 * 128 * (211 * 211 + 122 * 122),
         lambda: dm.bilinear_resample(mid, (211, 211), dst_nhwc=True))
+    hbm("bilinear_122_to_71_nchw_to_nhwc", 4 * 4 * 128 * (71 * 71 + 122 * 122),
+        lambda: dm.bilinear_resample(mid, (71, 71), dst_nhwc=True))
+    small_nhwc = rn(4, 71, 71, 128)
+    hbm("bilinear_71_to_122_nhwc_to_nchw", 4 * 4 * 128 * (71 * 71 + 122 * 122),
+        lambda: dm.bilinear_resample(small_nhwc, (122, 122), src_nhwc=True))
+    del small_nhwc
     cb = rn(128)
     hbm("bilinear_211_to_122_bias_silu_silu", 4 * 4 * 128 * (211 * 211 + 122 * 122),
         lambda: dm.bilinear_resample(img, (122, 122), pre_activation="silu", post_activation="silu", pre_bias=cb))

@@ -136,10 +136,60 @@ __device__ __forceinline__ float act_pre(float v, float bias, ResampleAct a) {
     return v;
 }
 
+// act applied `count` times to every element of v, with the choice of activation made once for all of them: the
+// element-wise form puts a branch tree between the loads of successive samples, which then go out a few at a time.
+template <int N>
+__device__ __forceinline__ void act_many(float (&v)[N], int act, int count) {
+    if (act == SPGT_ACT_SILU) {
+        for (int r = 0; r < count; ++r) {
+#pragma unroll
+            for (int j = 0; j < N; ++j) v[j] = v[j] * __builtin_amdgcn_rcpf(1.f + __expf(-v[j]));
+        }
+    } else if (act == SPGT_ACT_RELU && count > 0) {
+#pragma unroll
+        for (int j = 0; j < N; ++j) v[j] = fmaxf(v[j], 0.f);
+    }
+}
+
+// NV output values from their 4 * NV source samples: t[4j .. 4j+3] = (top left, top right, bottom left, bottom
+// right) of value j, bias[j] its channel's bias.  Same arithmetic as torch's upsample_bilinear2d: columns are
+// blended first, rows last.
+template <bool PRE, int NV>
+__device__ __forceinline__ void blend_many(float (&t)[4 * NV], const float (&bias)[NV], float w0l, float w1l,
+                                           float h0l, float h1l, ResampleAct act, float (&v)[NV]) {
+    if (PRE) {
+#pragma unroll
+        for (int j = 0; j < 4 * NV; ++j) t[j] += bias[j >> 2];
+        act_many<4 * NV>(t, act.pre, act.pre_n);
+    }
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+        const float top = w0l * t[4 * j] + w1l * t[4 * j + 1];
+        const float bot = w0l * t[4 * j + 2] + w1l * t[4 * j + 3];
+        v[j] = h0l * top + h1l * bot;
+    }
+    act_many<NV>(v, act.post, 1);
+}
+
+// Source row, its lower neighbour and the two row weights of output row oy (align_corners=True:
+// scale = (in-1)/(out-1) in fp32, 0 when out == 1; source coordinate scale*dst, weights (1-l, l)).
+struct ResampleTap {
+    int i1, ip;  // first source index and the step (0 or 1) to the second
+    float l0, l1;
+};
+__device__ __forceinline__ ResampleTap resample_tap(float scale, int o, int in_size) {
+    const float r = scale * (float)o;
+    ResampleTap t;
+    t.i1 = (int)r;
+    t.ip = (t.i1 < in_size - 1) ? 1 : 0;
+    t.l1 = r - (float)t.i1;
+    t.l0 = 1.0f - t.l1;
+    return t;
+}
+
 // Bilinear resampling with align_corners=True of [planes, Hin, Win] -> [planes, Hout, Wout].
-// Same arithmetic as torch's upsample_bilinear2d: scale = (in-1)/(out-1) in fp32
-// (0 when out == 1), source coordinate scale*dst, weights (1-l, l), rows blended last.
-// grid (ceil(Wout/64), ceil(Hout/4), planes), block (64, 4).
+// grid (ceil(Wout/64), ceil(Hout/4), ceil(planes/4) or fewer), block (64, 4); a thread makes one output position
+// of 4 consecutive planes at a time, 16 source samples in flight.
 template <bool PRE>
 __global__ __launch_bounds__(256) void bilinear_align_corners_k(const float* __restrict__ src,
                                                                 const float* __restrict__ pre_bias, int C,
@@ -149,23 +199,22 @@ __global__ __launch_bounds__(256) void bilinear_align_corners_k(const float* __r
     const int ox = blockIdx.x * 64 + threadIdx.x;
     const int oy = blockIdx.y * 4 + threadIdx.y;
     if (ox >= Wout || oy >= Hout) return;
-    const float hr = hscale * (float)oy;
-    const int h1 = (int)hr;
-    const int hp = (h1 < Hin - 1) ? 1 : 0;
-    const float h1l = hr - (float)h1;
-    const float h0l = 1.0f - h1l;
-    const float wr = wscale * (float)ox;
-    const int w1 = (int)wr;
-    const int wp = (w1 < Win - 1) ? 1 : 0;
-    const float w1l = wr - (float)w1;
-    const float w0l = 1.0f - w1l;
-    for (int64_t pl = blockIdx.z; pl < planes; pl += gridDim.z) {
-        const float* r0 = src + pl * Hin * Win + (int64_t)h1 * Win + w1;
-        const float* r1 = r0 + (int64_t)hp * Win;
-        const float pb = (PRE && pre_bias) ? pre_bias[pl % C] : 0.f;
-        const float top = w0l * act_pre<PRE>(r0[0], pb, act) + w1l * act_pre<PRE>(r0[wp], pb, act);
-        const float bot = w0l * act_pre<PRE>(r1[0], pb, act) + w1l * act_pre<PRE>(r1[wp], pb, act);
-        dst[(pl * Hout + oy) * Wout + ox] = act_apply(h0l * top + h1l * bot, act.post);
+    const ResampleTap th = resample_tap(hscale, oy, Hin), tw = resample_tap(wscale, ox, Win);
+    const float* base = src + (int64_t)th.i1 * Win + tw.i1;
+    for (int64_t p0 = (int64_t)blockIdx.z * 4; p0 < planes; p0 += (int64_t)gridDim.z * 4) {
+        float t[16], pb[4], v[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int64_t pl = min(p0 + j, (int64_t)planes - 1);  // planes past the end repeat the last, unwritten
+            const float* r0 = base + pl * Hin * Win;
+            const float* r1 = r0 + (int64_t)th.ip * Win;
+            t[4 * j] = r0[0], t[4 * j + 1] = r0[tw.ip], t[4 * j + 2] = r1[0], t[4 * j + 3] = r1[tw.ip];
+            pb[j] = (PRE && pre_bias) ? pre_bias[pl % C] : 0.f;
+        }
+        blend_many<PRE, 4>(t, pb, tw.l0, tw.l1, th.l0, th.l1, act, v);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if (p0 + j < planes) dst[((p0 + j) * Hout + oy) * Wout + ox] = v[j];
     }
 }
 
@@ -181,38 +230,26 @@ __global__ __launch_bounds__(256) void bilinear_align_corners_nhwc_k(const float
     __shared__ float tile[32 * 33];
     const int tx = threadIdx.x & 31;
     const int ty = threadIdx.x >> 5;
-    const int ox = blockIdx.x * 32 + tx;
     const int oy = blockIdx.y;
     const int64_t n = blockIdx.z;
-    const float hr = hscale * (float)oy;
-    const int h1 = (int)hr;
-    const int hp = (h1 < Hin - 1) ? 1 : 0;
-    const float h1l = hr - (float)h1;
-    const float h0l = 1.0f - h1l;
-    const int oxc = min(ox, Wout - 1);
-    const float wr = wscale * (float)oxc;
-    const int w1 = (int)wr;
-    const int wp = (w1 < Win - 1) ? 1 : 0;
-    const float w1l = wr - (float)w1;
-    const float w0l = 1.0f - w1l;
+    const ResampleTap th = resample_tap(hscale, oy, Hin);
+    const ResampleTap tw = resample_tap(wscale, min((int)blockIdx.x * 32 + tx, Wout - 1), Win);
     const int64_t plane = (int64_t)Hin * Win;
-    const float* base = src + n * C * plane + (int64_t)h1 * Win + w1;
+    const float* base = src + n * C * plane + (int64_t)th.i1 * Win + tw.i1;
     float* drow = dst + ((n * Hout + oy) * (int64_t)Wout) * C;
     for (int c0 = 0; c0 < C; c0 += 32) {
+        float t[16], pb[4], v[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const int cl = 8 * i + ty;
-            float v = 0.f;
-            if (c0 + cl < C) {
-                const float* r0 = base + (int64_t)(c0 + cl) * plane;
-                const float* r1 = r0 + (int64_t)hp * Win;
-                const float pb = (PRE && pre_bias) ? pre_bias[c0 + cl] : 0.f;
-                const float top = w0l * act_pre<PRE>(r0[0], pb, act) + w1l * act_pre<PRE>(r0[wp], pb, act);
-                const float bot = w0l * act_pre<PRE>(r1[0], pb, act) + w1l * act_pre<PRE>(r1[wp], pb, act);
-                v = act_apply(h0l * top + h1l * bot, act.post);
-            }
-            tile[cl * 33 + tx] = v;
+            const int c = min(c0 + 8 * i + ty, C - 1);  // channels past the end repeat the last one and are not written
+            const float* r0 = base + (int64_t)c * plane;
+            const float* r1 = r0 + (int64_t)th.ip * Win;
+            t[4 * i] = r0[0], t[4 * i + 1] = r0[tw.ip], t[4 * i + 2] = r1[0], t[4 * i + 3] = r1[tw.ip];
+            pb[i] = (PRE && pre_bias) ? pre_bias[c] : 0.f;
         }
+        blend_many<PRE, 4>(t, pb, tw.l0, tw.l1, th.l0, th.l1, act, v);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) tile[(8 * i + ty) * 33 + tx] = v[i];
         __syncthreads();
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -239,33 +276,23 @@ __global__ __launch_bounds__(256) void bilinear_align_corners_from_nhwc_k(const 
     const int ty = threadIdx.x >> 5;
     const int oy = blockIdx.y;
     const int64_t n = blockIdx.z;
-    const float hr = hscale * (float)oy;
-    const int h1 = (int)hr;
-    const int hp = (h1 < Hin - 1) ? 1 : 0;
-    const float h1l = hr - (float)h1;
-    const float h0l = 1.0f - h1l;
-    const float* rows = src + (n * Hin + h1) * (int64_t)Win * C;
-    const int64_t rstep = (int64_t)hp * Win * C;
+    const ResampleTap th = resample_tap(hscale, oy, Hin);
+    const float* rows = src + (n * Hin + th.i1) * (int64_t)Win * C;
+    const int64_t rstep = (int64_t)th.ip * Win * C;
     for (int c0 = 0; c0 < C; c0 += 32) {
+        const int c = min(c0 + tx, C - 1);  // channels past the end repeat the last one and are not written
+        const float pb1 = (PRE && pre_bias) ? pre_bias[c] : 0.f;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int xl = 8 * i + ty;
-            const int ox = min(blockIdx.x * 32 + xl, Wout - 1);
-            const float wr = wscale * (float)ox;
-            const int w1 = (int)wr;
-            const int wp = (w1 < Win - 1) ? 1 : 0;
-            const float w1l = wr - (float)w1;
-            const float w0l = 1.0f - w1l;
-            float v = 0.f;
-            if (c0 + tx < C) {
-                const float* p0 = rows + (int64_t)w1 * C + c0 + tx;
-                const float* p1 = p0 + rstep;
-                const float pb = (PRE && pre_bias) ? pre_bias[c0 + tx] : 0.f;
-                const float top = w0l * act_pre<PRE>(p0[0], pb, act) + w1l * act_pre<PRE>(p0[wp * C], pb, act);
-                const float bot = w0l * act_pre<PRE>(p1[0], pb, act) + w1l * act_pre<PRE>(p1[wp * C], pb, act);
-                v = act_apply(h0l * top + h1l * bot, act.post);
-            }
-            tile[xl * 33 + tx] = v;
+            const ResampleTap tw = resample_tap(wscale, min((int)blockIdx.x * 32 + xl, Wout - 1), Win);
+            const float* p0 = rows + (int64_t)tw.i1 * C + c;
+            const float* p1 = p0 + rstep;
+            float t[4] = {p0[0], p0[tw.ip * C], p1[0], p1[tw.ip * C]};
+            const float pb[1] = {pb1};
+            float v[1];
+            blend_many<PRE, 1>(t, pb, tw.l0, tw.l1, th.l0, th.l1, act, v);
+            tile[xl * 33 + tx] = v[0];
         }
         __syncthreads();
         const int ox = blockIdx.x * 32 + tx;
@@ -274,6 +301,125 @@ __global__ __launch_bounds__(256) void bilinear_align_corners_from_nhwc_k(const 
             const int cl = 8 * i + ty;
             if (ox < Wout && c0 + cl < C)
                 dst[((n * C + c0 + cl) * Hout + oy) * (int64_t)Wout + ox] = tile[tx * 33 + cl];
+        }
+        __syncthreads();
+    }
+}
+
+// Logical tile of a one-dimensional launch whose size is a multiple of 8.  Workgroups go round-robin to the 8
+// XCDs, each with its own L2; consecutive logical tiles are mapped onto one XCD, so that tiles which share
+// source rows, or halves of an output cache line, meet in one L2.
+__device__ __forceinline__ int xcd_contiguous_tile() {
+    const int per_xcd = gridDim.x >> 3;
+    return (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+}
+
+// NCHW -> channels-last for C a multiple of 4 with a 16-byte aligned result: one workgroup makes 32 output
+// columns x 128 channels of one output row.  A thread blends 4 consecutive channels of one column and puts them
+// into LDS as one 16-byte piece; the workgroup then writes the tile as whole pixels, 1 KB contiguous per wave.
+// grid: tiles = N * Hout * ceil(Wout/32), rounded up to a multiple of 8; block 256.
+template <bool PRE>
+__global__ __launch_bounds__(256) void bilinear_to_nhwc_wide_k(const float* __restrict__ src,
+                                                               const float* __restrict__ pre_bias,
+                                                               float* __restrict__ dst, int C, int Hin, int Win,
+                                                               int Hout, int Wout, float hscale, float wscale,
+                                                               ResampleAct act, int xtiles, int tiles) {
+    __shared__ float4 tile[32 * 33];  // [column][channel quad], 33 quads apart: 8 lanes' pieces fall in 8 bank groups
+    const int logical = xcd_contiguous_tile();
+    if (logical >= tiles) return;
+    const int x0 = (logical % xtiles) * 32;
+    const int oy = (logical / xtiles) % Hout;
+    const int64_t n = logical / (xtiles * Hout);
+    const int tx = threadIdx.x & 31;
+    const int ty = threadIdx.x >> 5;
+    const ResampleTap th = resample_tap(hscale, oy, Hin);
+    const ResampleTap tw = resample_tap(wscale, min(x0 + tx, Wout - 1), Win);
+    const int64_t plane = (int64_t)Hin * Win;
+    const float* base = src + n * C * plane + (int64_t)th.i1 * Win + tw.i1;
+    float* drow = dst + ((n * Hout + oy) * (int64_t)Wout) * C;
+    for (int c0 = 0; c0 < C; c0 += 128) {
+#pragma unroll 2
+        for (int i = 0; i < 4; ++i) {
+            const int q = 8 * i + ty;
+            const int c = min(c0 + 4 * q, C - 4);  // quads past the end repeat the last one and are not written
+            float t[16], pb[4], v[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const float* r0 = base + (int64_t)(c + k) * plane;
+                const float* r1 = r0 + (int64_t)th.ip * Win;
+                t[4 * k] = r0[0], t[4 * k + 1] = r0[tw.ip], t[4 * k + 2] = r1[0], t[4 * k + 3] = r1[tw.ip];
+                pb[k] = (PRE && pre_bias) ? pre_bias[c + k] : 0.f;
+            }
+            blend_many<PRE, 4>(t, pb, tw.l0, tw.l1, th.l0, th.l1, act, v);
+            tile[tx * 33 + q] = make_float4(v[0], v[1], v[2], v[3]);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int xl = 8 * j + ty;
+            const int x = x0 + xl;
+            const int c = c0 + 4 * tx;
+            if (x < Wout && c < C) *reinterpret_cast<float4*>(drow + (int64_t)x * C + c) = tile[xl * 33 + tx];
+        }
+        __syncthreads();
+    }
+}
+
+// Channels-last -> NCHW for C a multiple of 4 with a 16-byte aligned source: one workgroup makes 32 output columns
+// x 128 channels of one output row.  A thread reads the four source pixels of a column 16 bytes (4 channels) at a
+// time, 512-byte runs per 32 lanes, and blends them; the tile is turned in LDS and written along the output rows.
+// Row c of the LDS tile holds column x at position x ^ (c / 32 % 4): the 32 lanes that write one column for 128
+// channels then hit 32 banks, and a row read is a permutation of one row.
+// grid: tiles = N * Hout * ceil(Wout/32), rounded up to a multiple of 8; block 256.
+template <bool PRE>
+__global__ __launch_bounds__(256) void bilinear_from_nhwc_wide_k(const float* __restrict__ src,
+                                                                 const float* __restrict__ pre_bias,
+                                                                 float* __restrict__ dst, int C, int Hin, int Win,
+                                                                 int Hout, int Wout, float hscale, float wscale,
+                                                                 ResampleAct act, int xtiles, int tiles) {
+    __shared__ float tile[128 * 33];
+    const int logical = xcd_contiguous_tile();
+    if (logical >= tiles) return;
+    const int x0 = (logical % xtiles) * 32;
+    const int oy = (logical / xtiles) % Hout;
+    const int64_t n = logical / (xtiles * Hout);
+    const int tx = threadIdx.x & 31;
+    const int ty = threadIdx.x >> 5;
+    const ResampleTap th = resample_tap(hscale, oy, Hin);
+    const float* rows = src + (n * Hin + th.i1) * (int64_t)Win * C;
+    const int64_t rstep = (int64_t)th.ip * Win * C;
+    for (int c0 = 0; c0 < C; c0 += 128) {
+        const int c = min(c0 + 4 * tx, C - 4);  // quads past the end repeat the last one and are not written
+        float pb[4] = {0.f, 0.f, 0.f, 0.f};
+        if (PRE && pre_bias) {
+            const float4 b4 = *reinterpret_cast<const float4*>(pre_bias + c);
+            pb[0] = b4.x, pb[1] = b4.y, pb[2] = b4.z, pb[3] = b4.w;
+        }
+#pragma unroll 2
+        for (int i = 0; i < 4; ++i) {
+            const int xl = 8 * i + ty;
+            const ResampleTap tw = resample_tap(wscale, min(x0 + xl, Wout - 1), Win);
+            const float* p0 = rows + (int64_t)tw.i1 * C + c;
+            const float* p1 = p0 + rstep;
+            const float4 a00 = *reinterpret_cast<const float4*>(p0);
+            const float4 a01 = *reinterpret_cast<const float4*>(p0 + tw.ip * C);
+            const float4 a10 = *reinterpret_cast<const float4*>(p1);
+            const float4 a11 = *reinterpret_cast<const float4*>(p1 + tw.ip * C);
+            float t[16] = {a00.x, a01.x, a10.x, a11.x, a00.y, a01.y, a10.y, a11.y,
+                           a00.z, a01.z, a10.z, a11.z, a00.w, a01.w, a10.w, a11.w};
+            float v[4];
+            blend_many<PRE, 4>(t, pb, tw.l0, tw.l1, th.l0, th.l1, act, v);
+            const int pos = xl ^ (tx >> 3);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) tile[(4 * tx + k) * 33 + pos] = v[k];
+        }
+        __syncthreads();
+        const int ox = x0 + tx;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int cl = 8 * i + ty;
+            if (ox < Wout && c0 + cl < C)
+                dst[((n * C + c0 + cl) * Hout + oy) * (int64_t)Wout + ox] = tile[cl * 33 + (tx ^ (cl >> 5))];
         }
         __syncthreads();
     }
@@ -450,7 +596,8 @@ int resample_common(const char* who, const float* src, const float* pre_bias, fl
         const int64_t planes = (int64_t)N * C;
         if (ceil_div(H_out, 4) > 65535 || planes > INT32_MAX)
             return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear resampling: H_out/4 exceeds 65535 or too many planes");
-        const dim3 grid(ceil_div(W_out, 64), ceil_div(H_out, 4), (unsigned)std::min<int64_t>(planes, 65535));
+        const dim3 grid(ceil_div(W_out, 64), ceil_div(H_out, 4),
+                        (unsigned)std::min<int64_t>(ceil_div(planes, (int64_t)4), 65535));
         hipLaunchKernelGGL(pre ? bilinear_align_corners_k<true> : bilinear_align_corners_k<false>, grid, dim3(64, 4), 0,
                            stream, src, pre_bias, C, dst, (int)planes, H_in, W_in, H_out, W_out, hscale, wscale, act);
     } else if (src_layout != dst_layout && (src_layout == SPGT_LAYOUT_NCHW || src_layout == SPGT_LAYOUT_NHWC) &&
@@ -458,7 +605,21 @@ int resample_common(const char* who, const float* src, const float* pre_bias, fl
         if (H_out > 65535 || N > 65535)
             return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear resampling: N or H_out exceeds 65535");
         const dim3 grid(ceil_div(W_out, 32), H_out, N);
-        if (dst_layout == SPGT_LAYOUT_NHWC)
+        // whole pixels of 4-channel pieces: the wide kernels, with a one-dimensional XCD-aware launch
+        const int xtiles = ceil_div(W_out, 32);
+        const int64_t tiles = (int64_t)N * H_out * xtiles;
+        const bool wide = C % 4 == 0 && tiles <= (1 << 30) && (!pre_bias || aligned16(pre_bias)) &&
+                          aligned16(dst_layout == SPGT_LAYOUT_NHWC ? (const void*)dst : (const void*)src);
+        const dim3 wide_grid((unsigned)(ceil_div(tiles, (int64_t)8) * 8));
+        if (wide && dst_layout == SPGT_LAYOUT_NHWC)
+            hipLaunchKernelGGL(pre ? bilinear_to_nhwc_wide_k<true> : bilinear_to_nhwc_wide_k<false>, wide_grid,
+                               dim3(256), 0, stream, src, pre_bias, dst, C, H_in, W_in, H_out, W_out, hscale, wscale,
+                               act, xtiles, (int)tiles);
+        else if (wide)
+            hipLaunchKernelGGL(pre ? bilinear_from_nhwc_wide_k<true> : bilinear_from_nhwc_wide_k<false>, wide_grid,
+                               dim3(256), 0, stream, src, pre_bias, dst, C, H_in, W_in, H_out, W_out, hscale, wscale,
+                               act, xtiles, (int)tiles);
+        else if (dst_layout == SPGT_LAYOUT_NHWC)
             hipLaunchKernelGGL(pre ? bilinear_align_corners_nhwc_k<true> : bilinear_align_corners_nhwc_k<false>, grid,
                                dim3(256), 0, stream, src, pre_bias, dst, C, H_in, W_in, H_out, W_out, hscale, wscale,
                                act);

@@ -120,5 +120,6 @@ __device__ __forceinline__ void st_stream(float4* p, float4 v) {
 }
 
 __host__ __device__ __forceinline__ int ceil_div(int a, int b) { return (a + b - 1) / b; }
+__host__ __device__ __forceinline__ int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 }  // namespace spgt

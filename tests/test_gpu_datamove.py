@@ -205,7 +205,8 @@ def test_truncated_dft_spectral_layer_vs_oracle(gpu, N, r, Cin, Cout, m):
 
 
 @pytest.mark.parametrize("shape,size", [((2, 3, 7, 9), (7, 9)), ((2, 3, 7, 9), (4, 5)), ((1, 128, 122, 122), (211, 211)),
-                                        ((2, 130, 16, 33), (40, 65)), ((1, 1, 5, 5), (1, 1)), ((3, 40, 9, 9), (9, 70))])
+                                        ((2, 130, 16, 33), (40, 65)), ((1, 1, 5, 5), (1, 1)), ((3, 40, 9, 9), (9, 70)),
+                                        ((2, 132, 16, 33), (40, 65)), ((4, 128, 122, 122), (71, 71))])
 def test_bilinear_nhwc_matches_nchw_kernel(gpu, shape, size):
     """The channels-last variant is the planar kernel followed by a permute, value for value."""
     x = rnd(*shape, seed=30).to(gpu)
@@ -222,7 +223,7 @@ def _act64(x, name, count=1):
 
 
 @pytest.mark.parametrize("shape,size", [((2, 3, 7, 9), (4, 5)), ((1, 128, 71, 71), (122, 122)), ((2, 40, 9, 33), (9, 70)),
-                                        ((1, 1, 5, 5), (1, 1))])
+                                        ((1, 1, 5, 5), (1, 1)), ((2, 260, 6, 7), (11, 37))])
 @pytest.mark.parametrize("src_nhwc,dst_nhwc", [(False, False), (False, True), (True, False)])
 @pytest.mark.parametrize("pre,count,post", [(None, 0, None), ("silu", 1, "silu"), ("relu", 2, None), (None, 0, "relu"),
                                             ("silu", 2, None)])
