@@ -121,21 +121,6 @@ struct ResampleAct {
     int pre, pre_n, post;
 };
 
-__device__ __forceinline__ float act_apply(float v, int act) {
-    if (act == SPGT_ACT_RELU) return fmaxf(v, 0.f);
-    if (act == SPGT_ACT_SILU) return v * __builtin_amdgcn_rcpf(1.f + __expf(-v));
-    return v;
-}
-
-// PRE = false compiles the bias and source activations out: the plain resampling stays as cheap as before.
-template <bool PRE>
-__device__ __forceinline__ float act_pre(float v, float bias, ResampleAct a) {
-    if (!PRE) return v;
-    v += bias;
-    for (int i = 0; i < a.pre_n; ++i) v = act_apply(v, a.pre);
-    return v;
-}
-
 // act applied `count` times to every element of v, with the choice of activation made once for all of them: the
 // element-wise form puts a branch tree between the loads of successive samples, which then go out a few at a time.
 template <int N>
@@ -490,13 +475,11 @@ __global__ __launch_bounds__(256) void conv3x3_resample_k(const float* __restric
                     v11 = fmaf(wv, patch[ci][ky + 1][kx + 1], v11);
                 }
         // at the last row / column (hp or wp = 0) the second sample is the first one again
-        const float s00 = act_pre<true>(v00, 0.f, act);
-        const float s01 = act_pre<true>(wp ? v01 : v00, 0.f, act);
-        const float s10 = act_pre<true>(hp ? v10 : v00, 0.f, act);
-        const float s11 = act_pre<true>(hp ? (wp ? v11 : v10) : (wp ? v01 : v00), 0.f, act);
-        const float top = w0l * s00 + w1l * s01;
-        const float bot = w0l * s10 + w1l * s11;
-        if (ox < Wout) out[((n * Cout + c) * Hout + oy) * (int64_t)Wout + ox] = act_apply(h0l * top + h1l * bot, act.post);
+        float t[4] = {v00, wp ? v01 : v00, hp ? v10 : v00, hp ? (wp ? v11 : v10) : (wp ? v01 : v00)};
+        const float no_bias[1] = {0.f};  // the bias is in the convolution sums already
+        float v[1];
+        blend_many<true, 1>(t, no_bias, w0l, w1l, h0l, h1l, act, v);
+        if (ox < Wout) out[((n * Cout + c) * Hout + oy) * (int64_t)Wout + ox] = v[0];
     }
 }
 
@@ -507,10 +490,15 @@ __global__ __launch_bounds__(256) void bias_activation_nchw_k(float* __restrict_
     const int64_t pl = blockIdx.y;
     const float b = bias ? bias[pl % C] : 0.f;
     float* row = x + pl * HW;
-    for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < HW; e += (int64_t)gridDim.x * 256) {
-        float v = row[e] + b;
-        for (int i = 0; i < count; ++i) v = act_apply(v, act);
-        row[e] = v;
+    const int64_t stride = (int64_t)gridDim.x * 256;
+    for (int64_t e0 = (int64_t)blockIdx.x * 256 + threadIdx.x; e0 < HW; e0 += 4 * stride) {
+        float v[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[j] = row[min(e0 + j * stride, HW - 1)] + b;  // past the end: read, not written
+        act_many<4>(v, act, count);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if (e0 + j * stride < HW) row[e0 + j * stride] = v[j];
     }
 }
 
