@@ -365,7 +365,13 @@ def kernel_rooflines(dev):
     hbm("bilinear_71_to_122_nhwc_to_nchw", 4 * 4 * 128 * (71 * 71 + 122 * 122),
         lambda: dm.bilinear_resample(small_nhwc, (122, 122), src_nhwc=True))
     del small_nhwc
+    low64, grid2, wg = rn(4, 122, 122, 64), rn(4, 211, 211, 2), rn(2, 64)
+    hbm("bilinear_122_to_211_nhwc_plus_grid_columns", 4 * 4 * (64 * (211 * 211 + 122 * 122) + 2 * 211 * 211),
+        lambda: dm.bilinear_nhwc_affine(low64, (211, 211), grid2, wg))
+    del low64, grid2, wg
     cb = rn(128)
+    hbm("bias_silu2_nchw_to_nhwc_122", 2 * mid.numel() * 4,
+        lambda: dm.bilinear_resample(mid, (122, 122), dst_nhwc=True, pre_bias=cb, pre_activation="silu", pre_count=2))
     hbm("bilinear_211_to_122_bias_silu_silu", 4 * 4 * 128 * (211 * 211 + 122 * 122),
         lambda: dm.bilinear_resample(img, (122, 122), pre_activation="silu", post_activation="silu", pre_bias=cb))
     hbm("bias_activation_nchw_silu2", 2 * mid.numel() * 4, lambda: dm.bias_activation_nchw_(mid, cb, "silu", 2))

@@ -272,6 +272,17 @@ int spgt_bilinear_resample(const float* src, const float* pre_bias, float* dst, 
                            int pre_activation, int pre_activation_count, int post_activation,
                            spgt_stream_t stream);
 
+/* UpScaler2D's last F.interpolate (network/model.py:63-64) on a channels-last source together with the grid
+ * columns' share of the decoder's input layer Linear(cat([X, grid])) (network/sp_model.py:60, 118):
+ *   dst[n, y, x, c] = bilinear(src)[n, y, x, c] + sum_e extra[n, y, x, e] * w_extra[e, c]
+ * with align_corners=True.  The Linear over the hidden features commutes with the resampling, so a caller can
+ * run it on the low-resolution tensor and hand its result in as src.  src [N, H_in, W_in, C],
+ * dst [N, H_out, W_out, C], extra [N, H_out, W_out, n_extra] and w_extra [n_extra, C] (n_extra 0..4; both may
+ * be null when it is 0).  C must be a multiple of 4; src, dst and w_extra 16-byte aligned. */
+int spgt_bilinear_nhwc_affine(const float* src, float* dst, int N, int C, int H_in, int W_in, int H_out,
+                              int W_out, const float* extra, const float* w_extra, int n_extra,
+                              spgt_stream_t stream);
+
 /* 1 when spgt_conv3x3_resample serves this number of input channels (1..4), else 0. */
 int spgt_conv3x3_resample_supported(int Cin);
 

@@ -303,7 +303,9 @@ __device__ __forceinline__ int xcd_contiguous_tile() {
 // columns x 128 channels of one output row.  A thread blends 4 consecutive channels of one column and puts them
 // into LDS as one 16-byte piece; the workgroup then writes the tile as whole pixels, 1 KB contiguous per wave.
 // grid: tiles = N * Hout * ceil(Wout/32), rounded up to a multiple of 8; block 256.
-template <bool PRE>
+// SAME: input and output sizes are equal, every output is its own source sample (weights 1 and 0), and the kernel
+// is bias + activation + permute with one load per value.
+template <bool PRE, bool SAME>
 __global__ __launch_bounds__(256) void bilinear_to_nhwc_wide_k(const float* __restrict__ src,
                                                                const float* __restrict__ pre_bias,
                                                                float* __restrict__ dst, int C, int Hin, int Win,
@@ -327,15 +329,24 @@ __global__ __launch_bounds__(256) void bilinear_to_nhwc_wide_k(const float* __re
         for (int i = 0; i < 4; ++i) {
             const int q = 8 * i + ty;
             const int c = min(c0 + 4 * q, C - 4);  // quads past the end repeat the last one and are not written
-            float t[16], pb[4], v[4];
+            float pb[4], v[4];
 #pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                const float* r0 = base + (int64_t)(c + k) * plane;
-                const float* r1 = r0 + (int64_t)th.ip * Win;
-                t[4 * k] = r0[0], t[4 * k + 1] = r0[tw.ip], t[4 * k + 2] = r1[0], t[4 * k + 3] = r1[tw.ip];
-                pb[k] = (PRE && pre_bias) ? pre_bias[c + k] : 0.f;
+            for (int k = 0; k < 4; ++k) pb[k] = (PRE && pre_bias) ? pre_bias[c + k] : 0.f;
+            if (SAME) {
+#pragma unroll
+                for (int k = 0; k < 4; ++k) v[k] = base[(int64_t)(c + k) * plane] + pb[k];
+                if (PRE) act_many<4>(v, act.pre, act.pre_n);
+                act_many<4>(v, act.post, 1);
+            } else {
+                float t[16];
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const float* r0 = base + (int64_t)(c + k) * plane;
+                    const float* r1 = r0 + (int64_t)th.ip * Win;
+                    t[4 * k] = r0[0], t[4 * k + 1] = r0[tw.ip], t[4 * k + 2] = r1[0], t[4 * k + 3] = r1[tw.ip];
+                }
+                blend_many<PRE, 4>(t, pb, tw.l0, tw.l1, th.l0, th.l1, act, v);
             }
-            blend_many<PRE, 4>(t, pb, tw.l0, tw.l1, th.l0, th.l1, act, v);
             tile[tx * 33 + q] = make_float4(v[0], v[1], v[2], v[3]);
         }
         __syncthreads();
@@ -407,6 +418,72 @@ __global__ __launch_bounds__(256) void bilinear_from_nhwc_wide_k(const float* __
                 dst[((n * C + c0 + cl) * Hout + oy) * (int64_t)Wout + ox] = tile[cl * 33 + (tx ^ (cl >> 5))];
         }
         __syncthreads();
+    }
+}
+
+// Channels-last on both sides for C a multiple of 4, with the few extra input columns of a following Linear
+// folded in: dst[n, y, x, c] = bilinear(src)[n, y, x, c] + sum_e extra[n, y, x, e] * w_extra[e, c].  A Linear over
+// the channels commutes with the resampling (the blend weights of an output sum to 1), so the decoder's input
+// layer Linear(cat([X, grid])) (network/sp_model.py:60) can run on the low-resolution X before UpScaler2D's last
+// interpolate (network/model.py:63) instead of after it; what remains for the full resolution is the grid
+// columns' rank-E update, applied here.  A thread makes 4 channels of 4 neighbouring pixels of an output row: the
+// source pixels are 16-byte loads, contiguous across the lanes of a pixel and all 16 in flight together, and the
+// results are 16-byte stores.
+// grid: ceil(N*Hout*ceil(Wout/4)*C/4 / 256) rounded up to a multiple of 8, block 256.
+__global__ __launch_bounds__(256) void bilinear_nhwc_affine_k(const float* __restrict__ src, float* __restrict__ dst,
+                                                              int C4, int Hin, int Win, int Hout, int Wout,
+                                                              float hscale, float wscale,
+                                                              const float* __restrict__ extra,
+                                                              const float* __restrict__ w_extra, int E,
+                                                              unsigned items) {
+    const unsigned f = (unsigned)xcd_contiguous_tile() * 256u + threadIdx.x;  // items < 2^31: 32-bit divisions
+    if (f >= items) return;
+    const unsigned xgroups = (unsigned)(Wout + 3) >> 2;
+    const int q = (int)(f % (unsigned)C4);
+    const unsigned group = f / (unsigned)C4;
+    const int ox0 = (int)(group % xgroups) * 4;
+    const unsigned line = group / xgroups;
+    const int oy = (int)(line % (unsigned)Hout);
+    const int64_t n = line / (unsigned)Hout;
+    const ResampleTap th = resample_tap(hscale, oy, Hin);
+    const int64_t C = 4 * (int64_t)C4;
+    const float* row0 = src + (n * Hin + th.i1) * (int64_t)Win * C + 4 * q;
+    const float* row1 = row0 + (int64_t)th.ip * Win * C;
+    ResampleTap tw[4];
+    float4 a00[4], a01[4], a10[4], a11[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        tw[j] = resample_tap(wscale, min(ox0 + j, Wout - 1), Win);  // pixels past the row's end: computed, not stored
+        const int64_t o0 = (int64_t)tw[j].i1 * C, o1 = o0 + tw[j].ip * C;
+        a00[j] = *reinterpret_cast<const float4*>(row0 + o0);
+        a01[j] = *reinterpret_cast<const float4*>(row0 + o1);
+        a10[j] = *reinterpret_cast<const float4*>(row1 + o0);
+        a11[j] = *reinterpret_cast<const float4*>(row1 + o1);
+    }
+    const int64_t pix0 = ((n * Hout + oy) * (int64_t)Wout) + ox0;
+    float4 wx[4];
+    float gx[4][4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        wx[e] = e < E ? *reinterpret_cast<const float4*>(w_extra + e * C + 4 * q) : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) gx[j][e] = (e < E && ox0 + j < Wout) ? extra[(pix0 + j) * E + e] : 0.f;
+    }
+    const float no_bias[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        float t[16] = {a00[j].x, a01[j].x, a10[j].x, a11[j].x, a00[j].y, a01[j].y, a10[j].y, a11[j].y,
+                       a00[j].z, a01[j].z, a10[j].z, a11[j].z, a00[j].w, a01[j].w, a10[j].w, a11[j].w};
+        float v[4];
+        blend_many<false, 4>(t, no_bias, tw[j].l0, tw[j].l1, th.l0, th.l1, ResampleAct{SPGT_ACT_NONE, 0, SPGT_ACT_NONE},
+                             v);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            v[0] = fmaf(gx[j][e], wx[e].x, v[0]), v[1] = fmaf(gx[j][e], wx[e].y, v[1]);
+            v[2] = fmaf(gx[j][e], wx[e].z, v[2]), v[3] = fmaf(gx[j][e], wx[e].w, v[3]);
+        }
+        if (ox0 + j < Wout)
+            *reinterpret_cast<float4*>(dst + (pix0 + j) * C + 4 * q) = make_float4(v[0], v[1], v[2], v[3]);
     }
 }
 
@@ -599,10 +676,12 @@ int resample_common(const char* who, const float* src, const float* pre_bias, fl
         const bool wide = C % 4 == 0 && tiles <= (1 << 30) && (!pre_bias || aligned16(pre_bias)) &&
                           aligned16(dst_layout == SPGT_LAYOUT_NHWC ? (const void*)dst : (const void*)src);
         const dim3 wide_grid((unsigned)(ceil_div(tiles, (int64_t)8) * 8));
+        const bool same = H_in == H_out && W_in == W_out;
         if (wide && dst_layout == SPGT_LAYOUT_NHWC)
-            hipLaunchKernelGGL(pre ? bilinear_to_nhwc_wide_k<true> : bilinear_to_nhwc_wide_k<false>, wide_grid,
-                               dim3(256), 0, stream, src, pre_bias, dst, C, H_in, W_in, H_out, W_out, hscale, wscale,
-                               act, xtiles, (int)tiles);
+            hipLaunchKernelGGL(same ? (pre ? bilinear_to_nhwc_wide_k<true, true> : bilinear_to_nhwc_wide_k<false, true>)
+                                    : (pre ? bilinear_to_nhwc_wide_k<true, false> : bilinear_to_nhwc_wide_k<false, false>),
+                               wide_grid, dim3(256), 0, stream, src, pre_bias, dst, C, H_in, W_in, H_out, W_out, hscale,
+                               wscale, act, xtiles, (int)tiles);
         else if (wide)
             hipLaunchKernelGGL(pre ? bilinear_from_nhwc_wide_k<true> : bilinear_from_nhwc_wide_k<false>, wide_grid,
                                dim3(256), 0, stream, src, pre_bias, dst, C, H_in, W_in, H_out, W_out, hscale, wscale,
@@ -634,6 +713,29 @@ extern "C" int spgt_bilinear_align_corners_nhwc(const float* src, float* dst, in
                                                 int H_out, int W_out, hipStream_t stream) {
     return resample_common("bilinear_align_corners_nhwc", src, nullptr, dst, N, C, H_in, W_in, H_out, W_out, SPGT_LAYOUT_NCHW,
                            SPGT_LAYOUT_NHWC, ResampleAct{SPGT_ACT_NONE, 0, SPGT_ACT_NONE}, stream);
+}
+
+extern "C" int spgt_bilinear_nhwc_affine(const float* src, float* dst, int N, int C, int H_in, int W_in, int H_out,
+                                         int W_out, const float* extra, const float* w_extra, int n_extra,
+                                         hipStream_t stream) {
+    if (!src || !dst) return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear_nhwc_affine: null pointer argument");
+    if (N <= 0 || C <= 0 || H_in <= 0 || W_in <= 0 || H_out <= 0 || W_out <= 0)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear_nhwc_affine: sizes must be positive");
+    if (C % 4 != 0) return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear_nhwc_affine: C must be a multiple of 4");
+    if (n_extra < 0 || n_extra > 4 || (n_extra > 0 && (!extra || !w_extra)))
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear_nhwc_affine: 0..4 extra columns, with both of their operands");
+    if (!aligned16(src) || !aligned16(dst) || (n_extra > 0 && (!aligned4(extra) || !aligned16(w_extra))))
+        return fail(SPGT_ERR_INVALID_ARGUMENT,
+                    "bilinear_nhwc_affine: src, dst and w_extra must be 16-byte aligned, extra 4-byte aligned");
+    const int64_t items = (int64_t)N * H_out * ceil_div(W_out, 4) * (C / 4);  // 4 pixels x 4 channels each
+    if (items > (int64_t)INT32_MAX - 2048)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear_nhwc_affine: more than 2^35 output elements");
+    const int64_t blocks = ceil_div(ceil_div(items, (int64_t)256), (int64_t)8) * 8;
+    const float hscale = H_out > 1 ? (float)(H_in - 1) / (float)(H_out - 1) : 0.f;
+    const float wscale = W_out > 1 ? (float)(W_in - 1) / (float)(W_out - 1) : 0.f;
+    hipLaunchKernelGGL(spgt::bilinear_nhwc_affine_k, dim3((unsigned)blocks), dim3(256), 0, stream, src, dst, C / 4,
+                       H_in, W_in, H_out, W_out, hscale, wscale, extra, w_extra, n_extra, (unsigned)items);
+    return check_launch("bilinear_nhwc_affine");
 }
 
 extern "C" int spgt_bilinear_resample(const float* src, const float* pre_bias, float* dst, int N, int C, int H_in,

@@ -297,6 +297,34 @@ def _bilinear_resample(X: Tensor, size, src_nhwc: bool = False, dst_nhwc: bool =
     return out
 
 
+def _bilinear_nhwc_affine(X: Tensor, size, extra: Tensor = None, weight_extra_kn: Tensor = None) -> Tensor:
+    """Channels-last bilinear align_corners resampling X [N, H, W, C] -> [N, H', W', C] (C a multiple of 4), plus
+    extra @ weight_extra_kn for extra [N, H', W', E] and weight_extra_kn [E, C], E <= 4: the few columns that a
+    Linear applied before the resampling could not see."""
+    require_gpu_f32("X", X)
+    if X.dim() != 4:
+        raise ValueError("X must have four dimensions")
+    N, H_in, W_in, C = X.shape
+    if C % 4:
+        raise ValueError("the channel count must be a multiple of 4")
+    H_out, W_out = (size, size) if isinstance(size, int) else tuple(size)
+    E = 0
+    if extra is not None:
+        require_gpu_f32("extra", extra)
+        require_gpu_f32("weight_extra_kn", weight_extra_kn)
+        E = weight_extra_kn.shape[0]
+        if E > 4 or tuple(weight_extra_kn.shape) != (E, C) or tuple(extra.shape) != (N, H_out, W_out, E):
+            raise ValueError("extra must be [N, H', W', E] and weight_extra_kn [E, C] with E <= 4")
+    out = torch.empty((N, H_out, W_out, C), dtype=X.dtype, device=X.device)
+    if out.numel() == 0:
+        return out
+    with torch.cuda.device(X.device):
+        check(_lib.load().spgt_bilinear_nhwc_affine(ptr(X), ptr(out), N, C, H_in, W_in, H_out, W_out,
+                                                    ptr(extra) if E else None, ptr(weight_extra_kn) if E else None, E,
+                                                    stream_of(X)))
+    return out
+
+
 def _bias_activation_nchw_(X: Tensor, bias, activation=None, count: int = 1) -> Tensor:
     """In place on X [N, C, ...]: X = activation^count(X + bias[c]); returns X."""
     require_gpu_f32("X", X)
@@ -413,6 +441,7 @@ dexts = SimpleNamespace(
     spectral_modes_middle=_spectral_modes_middle,
     bias_activation_nchw_=_bias_activation_nchw_,
     bilinear_resample=_bilinear_resample,
+    bilinear_nhwc_affine=_bilinear_nhwc_affine,
     bilinear_align_corners_nhwc=_bilinear_align_corners_nhwc,
     batched_transpose=_batched_transpose,
     transpose_gather_dual=_transpose_gather_dual,
@@ -508,6 +537,12 @@ def bilinear_resample(X: Tensor, size, src_nhwc: bool = False, dst_nhwc: bool = 
     """post(interpolate(pre^pre_count(X + pre_bias))) between NCHW / NHWC layouts in one pass (inference only)."""
     return dexts.bilinear_resample(X.detach(), size, src_nhwc, dst_nhwc, pre_activation, pre_count, post_activation,
                                    None if pre_bias is None else pre_bias.detach())
+
+
+def bilinear_nhwc_affine(X: Tensor, size, extra: Tensor = None, weight_extra_kn: Tensor = None) -> Tensor:
+    """interpolate(X) + extra @ weight_extra_kn, channels-last on both sides (inference only)."""
+    return dexts.bilinear_nhwc_affine(X.detach(), size, None if extra is None else extra.detach(),
+                                      None if weight_extra_kn is None else weight_extra_kn.detach())
 
 
 def bias_activation_nchw_(X: Tensor, bias, activation=None, count: int = 1) -> Tensor:

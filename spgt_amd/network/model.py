@@ -86,7 +86,22 @@ class UpScaler2D(nn.Module):
         self.conv = ConvResBlock2D(in_dim, out_dim, 3, 1, droprate, activation)
         self.activation_layer = make_activation(activation)
 
-    def forward(self, X: Tensor) -> Tensor:
+    def can_defer_last_resample(self, X: Tensor) -> bool:
+        """True when forward(X, defer_last_resample=True) is available: fused inference with one kind of activation."""
+        return (gpu_inference(X, *self.parameters()) and self.droprate == 0 and self.conv.fusable(X) and
+                type(self.conv.activation_layer) is type(self.activation_layer))
+
+    def forward(self, X: Tensor, defer_last_resample: bool = False) -> Tensor:
+        """With defer_last_resample (see can_defer_last_resample) the result is the channels-last tensor at
+        resolution_size[3], [N, r_mid, r_mid, out_dim], and the caller owes the interpolation to resolution_size[4]:
+        a Linear over the channels commutes with it and is cheaper at the lower resolution."""
+        if defer_last_resample:
+            X = bilinear_resample(X.contiguous(), self.resolution_size[3], src_nhwc=True)
+            # the block's bias, its activation and the scaler's own on the way to channels-last: a resampling to
+            # the same size has weights (1, 0) and copies the samples exactly
+            Y = self.conv.conv_raw(X)
+            return bilinear_resample(Y, tuple(Y.shape[-2:]), dst_nhwc=True, pre_bias=self.conv.conv_layer.bias,
+                                     pre_activation=activation_name(self.activation_layer), pre_count=2)
         if gpu_inference(X, *self.parameters()) and self.droprate == 0:
             # channels-last in, NCHW out for the convolution; the block's bias and activation and the
             # scaler's own activation are one in-place pass (an upsampling reads every source sample

@@ -8,7 +8,7 @@ import torch
 import torch.nn.functional as F
 from torch import Tensor, nn
 
-from ..extension.bind.datamove import denormalize_boundary
+from ..extension.bind.datamove import bilinear_nhwc_affine, denormalize_boundary
 from ..extension.bind.linear import fused_linear, linear_supported
 from .layer import FeedForward, always_dropout, gpu_inference
 from .model import DownScaler2D, UpScaler2D
@@ -69,11 +69,27 @@ class Sp_DecoderRegressor(nn.Module):
             self._spgt_weight_split = cache
         return cache[1], cache[2]
 
-    def forward(self, X: Tensor, grid: Tensor = None) -> Tensor:
-        """X [N, r, r, dim_hidden], grid [N, r, r, dim_position] -> [N, r, r, dim_target]."""
+    def accepts_low_resolution(self, X: Tensor, grid: Tensor) -> bool:
+        """True when forward(X, grid, resample_to=size) is available for a channels-last X."""
+        W, dim_x = self.spatial_fc_layer.weight, X.size(-1)
+        return (grid is not None and grid.is_cuda and grid.dtype == torch.float32 and
+                gpu_inference(X, grid, W, self.spatial_fc_layer.bias) and linear_supported(dim_x, W.size(0)) and
+                W.size(0) % 4 == 0 and 0 < W.size(1) - dim_x <= 4 and grid.size(-1) == W.size(1) - dim_x)
+
+    def forward(self, X: Tensor, grid: Tensor = None, resample_to=None) -> Tensor:
+        """X [N, r, r, dim_hidden], grid [N, r, r, dim_position] -> [N, r, r, dim_target].
+        With resample_to = (r, r) (see accepts_low_resolution), X is [N, r_low, r_low, dim_hidden] and stands for
+        its bilinear (align_corners) interpolation to r x r: the input layer runs on the low-resolution X, which
+        gives the same result up to rounding because the layer is linear and interpolation weights sum to 1, and
+        the interpolation then moves dim_spatial_hidden channels instead of dim_hidden."""
         # Linear(cat([X, grid])) without materialising the concatenation: W = [W_x | W_grid]
         W, dim_x = self.spatial_fc_layer.weight, X.size(-1)
-        if (gpu_inference(X, W, self.spatial_fc_layer.bias) and linear_supported(dim_x, W.size(0)) and
+        if resample_to is not None:
+            w_x, w_grid = self._split_weight_kn(dim_x)
+            X = fused_linear(X, w_x, self.spatial_fc_layer.bias, "none")
+            # the grid columns are a rank-2 update at the full resolution, applied by the resampling kernel
+            X = bilinear_nhwc_affine(X, resample_to, grid.contiguous(), w_grid)
+        elif (gpu_inference(X, W, self.spatial_fc_layer.bias) and linear_supported(dim_x, W.size(0)) and
                 W.size(1) - dim_x <= 4):
             # the GEMM runs over the hidden features; the grid columns are a rank-2 update in its epilogue
             w_x, w_grid = self._split_weight_kn(dim_x)
@@ -108,8 +124,14 @@ class Sp_GalerkinTransformer2D(nn.Module):
         -> [N, r, r, dim_target] (de-normalised; zero on the boundary for the Dirichlet condition)."""
         X = always_dropout(self.down_scaler(X), self.droprate)
         X = self.encoder_mixer(X, position)
-        X = always_dropout(self.up_scaler(X), self.droprate)
-        X = self.decoder_regressor(X, grid)
+        if (self.droprate == 0 and self.up_scaler.can_defer_last_resample(X) and
+                self.decoder_regressor.accepts_low_resolution(X, grid)):
+            # the decoder's input layer moves in front of the up-scaler's last interpolation
+            X = self.decoder_regressor(self.up_scaler(X, defer_last_resample=True), grid,
+                                       resample_to=self.up_scaler.resolution_size[4])
+        else:
+            X = always_dropout(self.up_scaler(X), self.droprate)
+            X = self.decoder_regressor(X, grid)
         dirichlet = self.boundary_condition == "dirichlet"
         # (a grid with fewer than two rows or columns has no interior: the padded result would change shape)
         affine = self._normalizer_affine(X) if gpu_inference(X) and min(X.shape[1:3]) >= 2 else None

@@ -223,7 +223,7 @@ def _act64(x, name, count=1):
 
 
 @pytest.mark.parametrize("shape,size", [((2, 3, 7, 9), (4, 5)), ((1, 128, 71, 71), (122, 122)), ((2, 40, 9, 33), (9, 70)),
-                                        ((1, 1, 5, 5), (1, 1)), ((2, 260, 6, 7), (11, 37))])
+                                        ((1, 1, 5, 5), (1, 1)), ((2, 260, 6, 7), (11, 37)), ((2, 12, 9, 7), (9, 7))])
 @pytest.mark.parametrize("src_nhwc,dst_nhwc", [(False, False), (False, True), (True, False)])
 @pytest.mark.parametrize("pre,count,post", [(None, 0, None), ("silu", 1, "silu"), ("relu", 2, None), (None, 0, "relu"),
                                             ("silu", 2, None)])
@@ -241,6 +241,40 @@ def test_bilinear_resample_layouts_and_activations(gpu, shape, size, src_nhwc, d
         got = got.permute(0, 3, 1, 2)
     assert got.shape == want.shape
     assert (got - want).abs().max().item() <= 1e-5 * max(1.0, want.abs().max().item())
+
+
+@pytest.mark.parametrize("shape,size,E", [((2, 7, 9, 8), (13, 17), 2), ((1, 122, 122, 64), (211, 211), 2),
+                                          ((3, 5, 5, 4), (5, 5), 0), ((2, 9, 4, 12), (3, 11), 4),
+                                          ((1, 1, 1, 4), (3, 2), 1), ((2, 6, 6, 132), (1, 1), 3)])
+def test_bilinear_nhwc_affine(gpu, shape, size, E):
+    """Channels-last resampling plus extra @ W (network/model.py:63-64 followed by the grid columns of
+    network/sp_model.py:60), against the float64 oracle resampling and a float64 matmul."""
+    x = rnd(*shape, seed=71)
+    N, _, _, C = shape
+    want = O.bilinear_align_corners(x.double().permute(0, 3, 1, 2), size).permute(0, 2, 3, 1)
+    extra = w = None
+    if E:
+        extra, w = rnd(N, size[0], size[1], E, seed=72), rnd(E, C, seed=73)
+        want = want + extra.double() @ w.double()
+    got = dm.bilinear_nhwc_affine(x.to(gpu), size, None if extra is None else extra.to(gpu),
+                                  None if w is None else w.to(gpu))
+    assert got.is_contiguous() and got.shape == want.shape
+    assert (got.cpu().double() - want).abs().max().item() <= 1e-5 * max(1.0, want.abs().max().item())
+
+
+def test_bilinear_nhwc_affine_rejects(gpu):
+    with pytest.raises(ValueError):
+        dm.bilinear_nhwc_affine(rnd(1, 4, 4, 6, seed=1).to(gpu), (5, 5))  # 6 channels: not a multiple of 4
+    with pytest.raises(ValueError):
+        dm.bilinear_nhwc_affine(rnd(1, 4, 4, 8, seed=1).to(gpu), (5, 5), rnd(1, 5, 5, 5, seed=2).to(gpu),
+                                rnd(5, 8, seed=3).to(gpu))  # more than 4 extra columns
+
+
+def test_resampling_to_the_same_size_copies(gpu):
+    """Weights (1, 0): the layout-changing kernels double as bias + activation + permute."""
+    x = rnd(2, 12, 9, 7, seed=81).to(gpu)
+    assert torch.equal(dm.bilinear_resample(x, (9, 7), dst_nhwc=True), x.permute(0, 2, 3, 1).contiguous())
+    assert torch.equal(dm.bilinear_resample(x, (9, 7)), x)
 
 
 def test_bilinear_resample_rejects(gpu):

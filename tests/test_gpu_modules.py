@@ -133,6 +133,27 @@ def test_full_model_vs_oracle_mid_size(gpu):
     assert rel_l2(got.cpu().double(), want) < TOL
 
 
+def test_deferred_upsampling_matches_module_order(gpu):
+    """The decoder's input layer in front of the up-scaler's last interpolation (a Linear over the channels commutes
+    with it) against the reference's order of the same modules (network/model.py:59-64, network/sp_model.py:60):
+    grid values that are not a linear ramp, so that only the rank-2 grid update can place them."""
+    p, i, _, meta = load_golden("galerkin_transformer_2d")
+    m = load_into(SM.Sp_GalerkinTransformer2D(model_cfg(meta)), p, gpu)
+    rs = meta["resolution_size"].tolist()
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(2, rs[2][0], rs[2][1], 128, generator=g).to(gpu)
+    grid = torch.rand(2, rs[4][0], rs[4][1], 2, generator=g).to(gpu)
+    up, dec = m.up_scaler, m.decoder_regressor
+    with torch.no_grad():
+        assert up.can_defer_last_resample(x)
+        low = up(x, defer_last_resample=True)
+        assert tuple(low.shape) == (2, rs[3][0], rs[3][1], 128) and dec.accepts_low_resolution(low, grid)
+        want = dec(up(x), grid)
+        got = dec(low, grid, resample_to=rs[4])
+    assert got.shape == want.shape
+    assert rel_l2(got.cpu(), want.cpu()) < 1e-5 and max_rel(got.cpu(), want.cpu()) < 1e-4
+
+
 def test_graphed_inference_replays_match_eager(gpu):
     """A HIP-graph capture of the whole forward: every replay, with eager work and synchronisation between
     replays and with fresh inputs, reproduces the eager forward.  The convolution library picks algorithms
