@@ -283,6 +283,18 @@ int spgt_bilinear_nhwc_affine(const float* src, float* dst, int N, int C, int H_
                               int W_out, const float* extra, const float* w_extra, int n_extra,
                               spgt_stream_t stream);
 
+/* DownScaler2D's cat([X1, X2, X3], dim=1) -> F.interpolate -> permute -> activation (network/model.py:35-38)
+ * without the concatenated tensor: srcs[s] is an NCHW tensor [N, channels[s], H_in, W_in] (n_src 1..4), dst
+ * [N, H_out, W_out, sum channels] channels-last.  Where pre_flags[s] is non-zero, source s is a convolution
+ * output that still lacks its bias pre_biases[s] (may be null) and its activation: pre_activation is applied
+ * pre_activation_count (0..2) times to its samples first (ConvResBlock2D, network/layer.py:7-24).
+ * post_activation is applied to every result.  pre_biases and pre_flags may be null (no source needs them).
+ * The channel counts must add up to a multiple of 4; dst 16-byte aligned. */
+int spgt_bilinear_resample_concat(const float* const* srcs, const float* const* pre_biases, const int* channels,
+                                  const int* pre_flags, int n_src, float* dst, int N, int H_in, int W_in,
+                                  int H_out, int W_out, int pre_activation, int pre_activation_count,
+                                  int post_activation, spgt_stream_t stream);
+
 /* 1 when spgt_conv3x3_resample serves this number of input channels (1..4), else 0. */
 int spgt_conv3x3_resample_supported(int Cin);
 

@@ -361,6 +361,79 @@ __global__ __launch_bounds__(256) void bilinear_to_nhwc_wide_k(const float* __re
     }
 }
 
+// Up to four NCHW tensors that stand for their concatenation along C (DownScaler2D's cat([X1, X2, X3]) before its
+// second interpolate, network/model.py:35-36).  Source s holds channels first[s] .. first[s+1]-1 of the result;
+// bit s of pre_mask says that its samples still lack their bias and activation(s).
+struct ResampleSources {
+    const float *src0, *src1, *src2, *src3;
+    const float *bias0, *bias1, *bias2, *bias3;  // null: no bias
+    int first1, first2, first3;                  // the total channel count for absent sources
+    int pre_mask;
+};
+
+// bilinear_to_nhwc_wide_k over such a concatenation, which is never materialised: every channel finds its tensor.
+// The source activations are computed for all samples and kept where the mask asks for them.
+// grid: tiles = N * Hout * ceil(Wout/32), rounded up to a multiple of 8; block 256.
+__global__ __launch_bounds__(256) void bilinear_concat_to_nhwc_k(ResampleSources S, float* __restrict__ dst, int C,
+                                                                 int Hin, int Win, int Hout, int Wout, float hscale,
+                                                                 float wscale, ResampleAct act, int xtiles, int tiles) {
+    __shared__ float4 tile[32 * 33];
+    const int logical = xcd_contiguous_tile();
+    if (logical >= tiles) return;
+    const int x0 = (logical % xtiles) * 32;
+    const int oy = (logical / xtiles) % Hout;
+    const int64_t n = logical / (xtiles * Hout);
+    const int tx = threadIdx.x & 31;
+    const int ty = threadIdx.x >> 5;
+    const ResampleTap th = resample_tap(hscale, oy, Hin);
+    const ResampleTap tw = resample_tap(wscale, min(x0 + tx, Wout - 1), Win);
+    const int64_t plane = (int64_t)Hin * Win;
+    const int64_t off = (int64_t)th.i1 * Win + tw.i1;
+    float* drow = dst + ((n * Hout + oy) * (int64_t)Wout) * C;
+    for (int c0 = 0; c0 < C; c0 += 128) {
+#pragma unroll 2
+        for (int i = 0; i < 4; ++i) {
+            const int q = 8 * i + ty;
+            const int c = min(c0 + 4 * q, C - 4);  // quads past the end repeat the last one and are not written
+            float t[16], u[16], v[4];
+            bool pre[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const int ch = c + k;
+                const int s = (ch >= S.first1) + (ch >= S.first2) + (ch >= S.first3);
+                const float* p = s == 0 ? S.src0 : s == 1 ? S.src1 : s == 2 ? S.src2 : S.src3;
+                const float* b = s == 0 ? S.bias0 : s == 1 ? S.bias1 : s == 2 ? S.bias2 : S.bias3;
+                const int lo = s == 0 ? 0 : s == 1 ? S.first1 : s == 2 ? S.first2 : S.first3;
+                const int hi = s == 0 ? S.first1 : s == 1 ? S.first2 : s == 2 ? S.first3 : C;
+                pre[k] = (S.pre_mask >> s) & 1;
+                const float* r0 = p + (n * (hi - lo) + (ch - lo)) * plane + off;
+                const float* r1 = r0 + (int64_t)th.ip * Win;
+                t[4 * k] = r0[0], t[4 * k + 1] = r0[tw.ip], t[4 * k + 2] = r1[0], t[4 * k + 3] = r1[tw.ip];
+                const float pb = (pre[k] && b) ? b[ch - lo] : 0.f;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) u[4 * k + j] = t[4 * k + j] + pb;
+            }
+            if (S.pre_mask) {
+                act_many<16>(u, act.pre, act.pre_n);
+#pragma unroll
+                for (int j = 0; j < 16; ++j) t[j] = pre[j >> 2] ? u[j] : t[j];
+            }
+            const float no_bias[4] = {0.f, 0.f, 0.f, 0.f};
+            blend_many<false, 4>(t, no_bias, tw.l0, tw.l1, th.l0, th.l1, act, v);
+            tile[tx * 33 + q] = make_float4(v[0], v[1], v[2], v[3]);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int xl = 8 * j + ty;
+            const int x = x0 + xl;
+            const int c = c0 + 4 * tx;
+            if (x < Wout && c < C) *reinterpret_cast<float4*>(drow + (int64_t)x * C + c) = tile[xl * 33 + tx];
+        }
+        __syncthreads();
+    }
+}
+
 // Channels-last -> NCHW for C a multiple of 4 with a 16-byte aligned source: one workgroup makes 32 output columns
 // x 128 channels of one output row.  A thread reads the four source pixels of a column 16 bytes (4 channels) at a
 // time, 512-byte runs per 32 lanes, and blends them; the tile is turned in LDS and written along the output rows.
@@ -713,6 +786,53 @@ extern "C" int spgt_bilinear_align_corners_nhwc(const float* src, float* dst, in
                                                 int H_out, int W_out, hipStream_t stream) {
     return resample_common("bilinear_align_corners_nhwc", src, nullptr, dst, N, C, H_in, W_in, H_out, W_out, SPGT_LAYOUT_NCHW,
                            SPGT_LAYOUT_NHWC, ResampleAct{SPGT_ACT_NONE, 0, SPGT_ACT_NONE}, stream);
+}
+
+extern "C" int spgt_bilinear_resample_concat(const float* const* srcs, const float* const* pre_biases,
+                                             const int* channels, const int* pre_flags, int n_src, float* dst, int N,
+                                             int H_in, int W_in, int H_out, int W_out, int pre_activation,
+                                             int pre_activation_count, int post_activation, hipStream_t stream) {
+    if (!srcs || !channels || !dst) return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear_resample_concat: null pointer argument");
+    if (n_src < 1 || n_src > 4) return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear_resample_concat: 1 to 4 sources");
+    if (N <= 0 || H_in <= 0 || W_in <= 0 || H_out <= 0 || W_out <= 0)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear_resample_concat: sizes must be positive");
+    ResampleAct act{pre_activation, pre_activation_count, post_activation};
+    if (!act_known(act.pre) || !act_known(act.post) || act.pre_n < 0 || act.pre_n > 2)
+        return fail(SPGT_ERR_INVALID_ARGUMENT,
+                    "bilinear_resample_concat: unknown activation, or more than two source activations");
+    if (act.pre == SPGT_ACT_NONE) act.pre_n = 0;
+    const float* src[4] = {nullptr, nullptr, nullptr, nullptr};
+    const float* bias[4] = {nullptr, nullptr, nullptr, nullptr};
+    int first[5] = {0, 0, 0, 0, 0}, mask = 0;
+    int64_t C = 0;
+    for (int s = 0; s < n_src; ++s) {
+        if (!srcs[s] || channels[s] <= 0 || !aligned4(srcs[s]))
+            return fail(SPGT_ERR_INVALID_ARGUMENT,
+                        "bilinear_resample_concat: every source needs a 4-byte aligned pointer and a positive channel count");
+        src[s] = srcs[s];
+        first[s] = (int)C;
+        C += channels[s];
+        if (pre_flags && pre_flags[s]) {
+            mask |= 1 << s;
+            bias[s] = pre_biases ? pre_biases[s] : nullptr;
+            if (bias[s] && !aligned4(bias[s]))
+                return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear_resample_concat: biases must be 4-byte aligned");
+        }
+    }
+    if (C % 4 != 0 || C > (1 << 24) || !aligned16(dst))
+        return fail(SPGT_ERR_INVALID_ARGUMENT,
+                    "bilinear_resample_concat: the channels must add up to a multiple of 4 and dst be 16-byte aligned");
+    for (int s = n_src; s < 5; ++s) first[s] = (int)C;
+    const int xtiles = ceil_div(W_out, 32);
+    const int64_t tiles = (int64_t)N * H_out * xtiles;
+    if (tiles > (1 << 30)) return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear_resample_concat: too many output tiles");
+    const float hscale = H_out > 1 ? (float)(H_in - 1) / (float)(H_out - 1) : 0.f;
+    const float wscale = W_out > 1 ? (float)(W_in - 1) / (float)(W_out - 1) : 0.f;
+    const ResampleSources S{src[0], src[1], src[2], src[3], bias[0], bias[1], bias[2], bias[3],
+                            first[1], first[2], first[3], mask};
+    hipLaunchKernelGGL(spgt::bilinear_concat_to_nhwc_k, dim3((unsigned)(ceil_div(tiles, (int64_t)8) * 8)), dim3(256), 0,
+                       stream, S, dst, (int)C, H_in, W_in, H_out, W_out, hscale, wscale, act, xtiles, (int)tiles);
+    return check_launch("bilinear_resample_concat");
 }
 
 extern "C" int spgt_bilinear_nhwc_affine(const float* src, float* dst, int N, int C, int H_in, int W_in, int H_out,

@@ -6,6 +6,7 @@ extension/bind/datamove.cu:66-70 (the `dexts` module surface), plus two
 operators the reference leaves to library calls: the fused spectral-mode
 contraction and bilinear resampling.  Tensors must be contiguous and on a GPU.
 """
+import ctypes
 from math import prod
 from types import SimpleNamespace
 from typing import Any, List, Tuple
@@ -297,6 +298,48 @@ def _bilinear_resample(X: Tensor, size, src_nhwc: bool = False, dst_nhwc: bool =
     return out
 
 
+def _bilinear_resample_concat(sources, size, pre_biases=None, pre_flags=None, pre_activation=None,
+                              pre_count: int = 1, post_activation=None) -> Tensor:
+    """post(interpolate(cat(sources, dim=1))) into channels-last without the concatenated tensor: sources are 1 to 4
+    NCHW tensors [N, C_s, H, W] whose channel counts add up to a multiple of 4.  Where pre_flags[s] is set, source s
+    first gets pre_biases[s] (or nothing, if None) added and pre_activation applied pre_count times."""
+    n = len(sources)
+    if not 1 <= n <= 4:
+        raise ValueError("1 to 4 sources")
+    if pre_activation not in _ACT or post_activation not in _ACT:
+        raise ValueError("activations must be None, 'none', 'relu' or 'silu'")
+    pre_biases = list(pre_biases) if pre_biases is not None else [None] * n
+    pre_flags = [int(bool(f)) for f in pre_flags] if pre_flags is not None else [0] * n
+    if len(pre_biases) != n or len(pre_flags) != n:
+        raise ValueError("pre_biases and pre_flags need one entry per source")
+    for s, X in enumerate(sources):
+        require_gpu_f32(f"sources[{s}]", X)
+        if X.dim() != 4 or X.shape[0] != sources[0].shape[0] or X.shape[2:] != sources[0].shape[2:]:
+            raise ValueError("sources must be [N, C_s, H, W] with the same N, H and W")
+        if pre_biases[s] is not None:
+            require_gpu_f32(f"pre_biases[{s}]", pre_biases[s])
+            if pre_biases[s].numel() != X.shape[1]:
+                raise ValueError(f"pre_biases[{s}] has {pre_biases[s].numel()} elements, expected {X.shape[1]}")
+    N, _, H_in, W_in = sources[0].shape
+    C = sum(X.shape[1] for X in sources)
+    if C % 4:
+        raise ValueError("the channel counts must add up to a multiple of 4")
+    H_out, W_out = (size, size) if isinstance(size, int) else tuple(size)
+    out = torch.empty((N, H_out, W_out, C), dtype=sources[0].dtype, device=sources[0].device)
+    if out.numel() == 0:
+        return out
+    srcs = (ctypes.c_void_p * n)(*[X.data_ptr() for X in sources])
+    biases = (ctypes.c_void_p * n)(*[b.data_ptr() if b is not None else None for b in pre_biases])
+    chans = (ctypes.c_int * n)(*[int(X.shape[1]) for X in sources])
+    flags = (ctypes.c_int * n)(*pre_flags)
+    npre = int(pre_count) if _ACT[pre_activation] else 0
+    with torch.cuda.device(out.device):
+        check(_lib.load().spgt_bilinear_resample_concat(srcs, biases, chans, flags, n, ptr(out), N, H_in, W_in, H_out,
+                                                        W_out, _ACT[pre_activation], npre, _ACT[post_activation],
+                                                        stream_of(out)))
+    return out
+
+
 def _bilinear_nhwc_affine(X: Tensor, size, extra: Tensor = None, weight_extra_kn: Tensor = None) -> Tensor:
     """Channels-last bilinear align_corners resampling X [N, H, W, C] -> [N, H', W', C] (C a multiple of 4), plus
     extra @ weight_extra_kn for extra [N, H', W', E] and weight_extra_kn [E, C], E <= 4: the few columns that a
@@ -442,6 +485,7 @@ dexts = SimpleNamespace(
     bias_activation_nchw_=_bias_activation_nchw_,
     bilinear_resample=_bilinear_resample,
     bilinear_nhwc_affine=_bilinear_nhwc_affine,
+    bilinear_resample_concat=_bilinear_resample_concat,
     bilinear_align_corners_nhwc=_bilinear_align_corners_nhwc,
     batched_transpose=_batched_transpose,
     transpose_gather_dual=_transpose_gather_dual,
@@ -537,6 +581,15 @@ def bilinear_resample(X: Tensor, size, src_nhwc: bool = False, dst_nhwc: bool = 
     """post(interpolate(pre^pre_count(X + pre_bias))) between NCHW / NHWC layouts in one pass (inference only)."""
     return dexts.bilinear_resample(X.detach(), size, src_nhwc, dst_nhwc, pre_activation, pre_count, post_activation,
                                    None if pre_bias is None else pre_bias.detach())
+
+
+def bilinear_resample_concat(sources, size, pre_biases=None, pre_flags=None, pre_activation=None, pre_count: int = 1,
+                             post_activation=None) -> Tensor:
+    """post(interpolate(cat(sources, dim=1))) into channels-last, the concatenation never stored (inference only)."""
+    return dexts.bilinear_resample_concat([X.detach() for X in sources], size,
+                                          None if pre_biases is None else [None if b is None else b.detach()
+                                                                           for b in pre_biases],
+                                          pre_flags, pre_activation, pre_count, post_activation)
 
 
 def bilinear_nhwc_affine(X: Tensor, size, extra: Tensor = None, weight_extra_kn: Tensor = None) -> Tensor:

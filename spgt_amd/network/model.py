@@ -8,7 +8,7 @@ import torch.nn.functional as F
 from torch import Tensor, nn
 
 from ..extension.bind.datamove import (bilinear_align_corners, bilinear_align_corners_nhwc, bilinear_resample,
-                                       conv3x3_resample, conv3x3_resample_supported)
+                                       bilinear_resample_concat, conv3x3_resample, conv3x3_resample_supported)
 from .layer import ConvResBlock2D, activation_name, always_dropout, gpu_inference, make_activation
 
 
@@ -68,6 +68,14 @@ class DownScaler2D(nn.Module):
             X = self.activation_layer(resample(self.conv0(nhwc_to_nchw(X)), self.resolution_size[1]))
         X1 = self.conv1(X)
         X2 = self.conv2(X1)
+        if fused and self.conv3.fusable(X2) and (X1.size(1) + X2.size(1) + self.conv3.conv_layer.out_channels) % 4 == 0:
+            # the second resampling reads the three blocks where they are (no concatenated tensor), gives the last
+            # one its bias and activation on the way, and writes channels-last: the scaler's activation commutes
+            # with the permute
+            return bilinear_resample_concat(
+                [X1, X2, self.conv3.conv_raw(X2)], self.resolution_size[2],
+                pre_biases=[None, None, self.conv3.conv_layer.bias], pre_flags=[0, 0, 1],
+                pre_activation=activation_name(self.conv3.activation_layer), post_activation=act)
         X3 = self.conv3(X2)
         X = torch.cat([X1, X2, X3], dim=1)
         # the activation commutes with the permute, so the second resampling can write channels-last directly

@@ -262,6 +262,43 @@ def test_bilinear_nhwc_affine(gpu, shape, size, E):
     assert (got.cpu().double() - want).abs().max().item() <= 1e-5 * max(1.0, want.abs().max().item())
 
 
+@pytest.mark.parametrize("chans,hw,size", [((42, 42, 44), (13, 9), (7, 11)), ((4,), (5, 5), (9, 3)), ((3, 5), (6, 7), (6, 7)),
+                                           ((100, 1, 1, 30), (4, 6), (9, 13)), ((42, 42, 44), (122, 122), (71, 71))])
+@pytest.mark.parametrize("pre,count,post,flags", [(None, 0, None, None), ("silu", 1, "silu", (0, 0, 1, 1)),
+                                                   ("relu", 2, "relu", (1, 0, 1, 0)), (None, 1, "silu", (1, 1, 1, 1))])
+def test_bilinear_resample_concat(gpu, chans, hw, size, pre, count, post, flags):
+    """cat -> interpolate -> permute -> activation (network/model.py:35-38) from the separate blocks, flagged ones
+    still lacking bias and activation (network/layer.py:7-24), against the float64 oracle on the concatenation."""
+    n = len(chans)
+    xs = [rnd(2, c, hw[0], hw[1], seed=90 + s) for s, c in enumerate(chans)]
+    bs = [rnd(c, seed=95 + s) if s % 2 == 0 else None for s, c in enumerate(chans)]
+    fl = list(flags[:n]) if flags is not None else None
+    parts = []
+    for s in range(n):
+        x = xs[s].double()
+        if fl is not None and fl[s]:
+            if bs[s] is not None:
+                x = x + bs[s].double().view(1, -1, 1, 1)
+            x = _act64(x, pre, count)
+        parts.append(x)
+    want = _act64(O.bilinear_align_corners(torch.cat(parts, dim=1), size), post).permute(0, 2, 3, 1)
+    got = dm.bilinear_resample_concat([x.to(gpu) for x in xs], size,
+                                      pre_biases=[None if b is None else b.to(gpu) for b in bs] if fl else None,
+                                      pre_flags=fl, pre_activation=pre, pre_count=max(count, 1), post_activation=post)
+    assert got.is_contiguous() and got.shape == want.shape
+    assert (got.cpu().double() - want).abs().max().item() <= 1e-5 * max(1.0, want.abs().max().item())
+
+
+def test_bilinear_resample_concat_rejects(gpu):
+    x = rnd(1, 3, 4, 4, seed=1).to(gpu)
+    with pytest.raises(ValueError):
+        dm.bilinear_resample_concat([x, x], (5, 5))  # 6 channels
+    with pytest.raises(ValueError):
+        dm.bilinear_resample_concat([x] * 5, (5, 5))
+    with pytest.raises(ValueError):
+        dm.bilinear_resample_concat([x, rnd(1, 1, 4, 5, seed=2).to(gpu)], (5, 5))
+
+
 def test_bilinear_nhwc_affine_rejects(gpu):
     with pytest.raises(ValueError):
         dm.bilinear_nhwc_affine(rnd(1, 4, 4, 6, seed=1).to(gpu), (5, 5))  # 6 channels: not a multiple of 4
