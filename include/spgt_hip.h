@@ -295,6 +295,18 @@ int spgt_bilinear_resample_concat(const float* const* srcs, const float* const* 
                                   int H_out, int W_out, int pre_activation, int pre_activation_count,
                                   int post_activation, spgt_stream_t stream);
 
+/* UpScaler2D's F.interpolate -> conv3x3(padding 1) -> bias -> activation(s) (network/model.py:59-62,
+ * network/layer.py:7-24) with the channel mixing done before the interpolation: both are linear, so
+ *   conv(interp(X))[y, x, :] = sum over taps t = 3 ky + kx of interp(X . W_t)[y + ky - 1, x + kx - 1, :],
+ * taps outside the interpolated image contributing nothing (zero padding).  The caller computes
+ * Z [N, H_in, W_in, 9, C] = X . [W_0 | ... | W_8] with one GEMM on the low-resolution tokens
+ * (W_t[ci, co] = weight[co, ci, ky, kx]); this call gathers and blends (align_corners=True), adds bias [C]
+ * (may be null) and applies `activation` activation_count (0..2) times.  dst [N, H_out, W_out, C]
+ * channels-last.  C must be a multiple of 4; Z, bias and dst 16-byte aligned. */
+int spgt_upsample_conv3x3_gather(const float* Z, const float* bias, float* dst, int N, int C, int H_in, int W_in,
+                                 int H_out, int W_out, int activation, int activation_count,
+                                 spgt_stream_t stream);
+
 /* 1 when spgt_conv3x3_resample serves this number of input channels (1..4), else 0. */
 int spgt_conv3x3_resample_supported(int Cin);
 

@@ -560,6 +560,79 @@ __global__ __launch_bounds__(256) void bilinear_nhwc_affine_k(const float* __res
     }
 }
 
+// UpScaler2D's interpolate -> conv3x3(padding 1) -> bias -> activation(s) (network/model.py:59-62) with the channel
+// mixing done before the interpolation.  Both steps are linear, so
+//   conv(interp(X))[y, x, co] = sum over the 9 taps (ky, kx) of interp(Z_t)[y + ky - 1, x + kx - 1, co],
+//   Z_t = X . W_t  (the 1x1 product with the tap's [Cin, Cout] weight slice), t = 3 ky + kx,
+// where a tap that falls outside the interpolated image contributes nothing (the convolution's zero padding).
+// The products Z [N, Hin, Win, 9, C] come from one GEMM on the low-resolution tokens, (Hout/Hin)^2 times fewer
+// than the convolution would see; this kernel gathers: per output pixel and tap the four source pixels of
+// Z_t, blended as in the resampling kernels, summed over the taps in a fixed order, then bias and the
+// activation `act` applied `count` times.  Channels-last result [N, Hout, Wout, C], C a multiple of 4.
+// A thread makes 4 channels of one pixel; the lanes of a pixel read 16-byte pieces of one 4*C-byte run, and the
+// 8 (or more) neighbouring pixels of a workgroup share most of their source pixels through the L1.
+// grid: ceil(N*Hout*Wout*C/4 / 256) rounded up to a multiple of 8, block 256.
+__global__ __launch_bounds__(256) void upsample_conv3x3_gather_k(const float* __restrict__ Z,
+                                                                 const float* __restrict__ bias,
+                                                                 float* __restrict__ dst, int C4, int Hin, int Win,
+                                                                 int Hout, int Wout, float hscale, float wscale, int act,
+                                                                 int count, unsigned items) {
+    const unsigned f = (unsigned)xcd_contiguous_tile() * 256u + threadIdx.x;  // items < 2^31: 32-bit divisions
+    if (f >= items) return;
+    const int q = (int)(f % (unsigned)C4);
+    const unsigned pixel = f / (unsigned)C4;
+    const int ox = (int)(pixel % (unsigned)Wout);
+    const unsigned line = pixel / (unsigned)Wout;
+    const int oy = (int)(line % (unsigned)Hout);
+    const int64_t n = line / (unsigned)Hout;
+    const int64_t C = 4 * (int64_t)C4;
+    const int64_t pitch = 9 * C;  // floats per source pixel
+    const float* Zn = Z + n * Hin * (int64_t)Win * pitch + 4 * q;
+    ResampleTap tw[3];
+    bool xin[3];
+#pragma unroll
+    for (int kx = 0; kx < 3; ++kx) {
+        const int qx = ox + kx - 1;
+        xin[kx] = qx >= 0 && qx < Wout;
+        tw[kx] = resample_tap(wscale, min(max(qx, 0), Wout - 1), Win);
+    }
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ky = 0; ky < 3; ++ky) {
+        const int qy = oy + ky - 1;
+        if (qy < 0 || qy >= Hout) continue;  // the same for all lanes of a pixel and for most of a workgroup
+        const ResampleTap th = resample_tap(hscale, qy, Hin);
+        const float* row0 = Zn + (int64_t)th.i1 * Win * pitch + (3 * ky) * C;
+        const float* row1 = row0 + (int64_t)th.ip * Win * pitch;
+        float4 a00[3], a01[3], a10[3], a11[3];
+#pragma unroll
+        for (int kx = 0; kx < 3; ++kx) {
+            const int64_t o0 = (int64_t)tw[kx].i1 * pitch + kx * C, o1 = o0 + tw[kx].ip * pitch;
+            a00[kx] = *reinterpret_cast<const float4*>(row0 + o0);
+            a01[kx] = *reinterpret_cast<const float4*>(row0 + o1);
+            a10[kx] = *reinterpret_cast<const float4*>(row1 + o0);
+            a11[kx] = *reinterpret_cast<const float4*>(row1 + o1);
+        }
+#pragma unroll
+        for (int kx = 0; kx < 3; ++kx) {
+            float t[16] = {a00[kx].x, a01[kx].x, a10[kx].x, a11[kx].x, a00[kx].y, a01[kx].y, a10[kx].y, a11[kx].y,
+                           a00[kx].z, a01[kx].z, a10[kx].z, a11[kx].z, a00[kx].w, a01[kx].w, a10[kx].w, a11[kx].w};
+            const float no_bias[4] = {0.f, 0.f, 0.f, 0.f};
+            float v[4];
+            blend_many<false, 4>(t, no_bias, tw[kx].l0, tw[kx].l1, th.l0, th.l1,
+                                 ResampleAct{SPGT_ACT_NONE, 0, SPGT_ACT_NONE}, v);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) acc[k] += xin[kx] ? v[k] : 0.f;
+        }
+    }
+    if (bias) {
+        const float4 b = *reinterpret_cast<const float4*>(bias + 4 * q);
+        acc[0] += b.x, acc[1] += b.y, acc[2] += b.z, acc[3] += b.w;
+    }
+    act_many<4>(acc, act, count);
+    *reinterpret_cast<float4*>(dst + (int64_t)pixel * C + 4 * q) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+}
+
 // DownScaler2D's first stage in one pass for a few input channels (network/model.py:30-33:
 // conv0 = ConvResBlock2D(in_dim, out_dim, 3x3, padding 1), interpolate to resolution_size[1],
 // activation): out[n, c, oy, ox] = post(bilinear(pre(conv3x3(x)[n, c] + bias[c]))).  The four
@@ -833,6 +906,29 @@ extern "C" int spgt_bilinear_resample_concat(const float* const* srcs, const flo
     hipLaunchKernelGGL(spgt::bilinear_concat_to_nhwc_k, dim3((unsigned)(ceil_div(tiles, (int64_t)8) * 8)), dim3(256), 0,
                        stream, S, dst, (int)C, H_in, W_in, H_out, W_out, hscale, wscale, act, xtiles, (int)tiles);
     return check_launch("bilinear_resample_concat");
+}
+
+extern "C" int spgt_upsample_conv3x3_gather(const float* Z, const float* bias, float* dst, int N, int C, int H_in,
+                                            int W_in, int H_out, int W_out, int activation, int activation_count,
+                                            hipStream_t stream) {
+    if (!Z || !dst) return fail(SPGT_ERR_INVALID_ARGUMENT, "upsample_conv3x3_gather: null pointer argument");
+    if (N <= 0 || C <= 0 || H_in <= 0 || W_in <= 0 || H_out <= 0 || W_out <= 0)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "upsample_conv3x3_gather: sizes must be positive");
+    if (C % 4 != 0) return fail(SPGT_ERR_INVALID_ARGUMENT, "upsample_conv3x3_gather: C must be a multiple of 4");
+    if (!act_known(activation) || activation_count < 0 || activation_count > 2)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "upsample_conv3x3_gather: unknown activation or count outside 0..2");
+    if (!aligned16(Z) || !aligned16(dst) || (bias && !aligned16(bias)))
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "upsample_conv3x3_gather: operands must be 16-byte aligned");
+    const int64_t items = (int64_t)N * H_out * W_out * (C / 4);
+    if (items > (int64_t)INT32_MAX - 2048)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "upsample_conv3x3_gather: more than 2^33 output elements");
+    const int64_t blocks = ceil_div(ceil_div(items, (int64_t)256), (int64_t)8) * 8;
+    const float hscale = H_out > 1 ? (float)(H_in - 1) / (float)(H_out - 1) : 0.f;
+    const float wscale = W_out > 1 ? (float)(W_in - 1) / (float)(W_out - 1) : 0.f;
+    hipLaunchKernelGGL(spgt::upsample_conv3x3_gather_k, dim3((unsigned)blocks), dim3(256), 0, stream, Z, bias, dst,
+                       C / 4, H_in, W_in, H_out, W_out, hscale, wscale, activation,
+                       activation == SPGT_ACT_NONE ? 0 : activation_count, (unsigned)items);
+    return check_launch("upsample_conv3x3_gather");
 }
 
 extern "C" int spgt_bilinear_nhwc_affine(const float* src, float* dst, int N, int C, int H_in, int W_in, int H_out,

@@ -340,6 +340,32 @@ def _bilinear_resample_concat(sources, size, pre_biases=None, pre_flags=None, pr
     return out
 
 
+def _upsample_conv3x3_gather(Z: Tensor, bias, size, activation=None, count: int = 1) -> Tensor:
+    """Z [N, H, W, 9, C] (the nine per-tap 1x1 products of a 3x3 convolution's input at low resolution) ->
+    act^count(conv3x3(interpolate(X)) + bias) as [N, H', W', C] channels-last; C a multiple of 4."""
+    require_gpu_f32("Z", Z)
+    if Z.dim() != 5 or Z.shape[3] != 9:
+        raise ValueError("Z must be [N, H, W, 9, C]")
+    if activation not in _ACT:
+        raise ValueError("activation must be None, 'none', 'relu' or 'silu'")
+    N, H_in, W_in, _, C = Z.shape
+    if C % 4:
+        raise ValueError("the channel count must be a multiple of 4")
+    if bias is not None:
+        require_gpu_f32("bias", bias)
+        if bias.numel() != C:
+            raise ValueError(f"bias has {bias.numel()} elements, expected {C}")
+    H_out, W_out = (size, size) if isinstance(size, int) else tuple(size)
+    out = torch.empty((N, H_out, W_out, C), dtype=Z.dtype, device=Z.device)
+    if out.numel() == 0:
+        return out
+    with torch.cuda.device(Z.device):
+        check(_lib.load().spgt_upsample_conv3x3_gather(ptr(Z), ptr(bias) if bias is not None else None, ptr(out), N, C,
+                                                       H_in, W_in, H_out, W_out, _ACT[activation], int(count),
+                                                       stream_of(Z)))
+    return out
+
+
 def _bilinear_nhwc_affine(X: Tensor, size, extra: Tensor = None, weight_extra_kn: Tensor = None) -> Tensor:
     """Channels-last bilinear align_corners resampling X [N, H, W, C] -> [N, H', W', C] (C a multiple of 4), plus
     extra @ weight_extra_kn for extra [N, H', W', E] and weight_extra_kn [E, C], E <= 4: the few columns that a
@@ -485,6 +511,7 @@ dexts = SimpleNamespace(
     bias_activation_nchw_=_bias_activation_nchw_,
     bilinear_resample=_bilinear_resample,
     bilinear_nhwc_affine=_bilinear_nhwc_affine,
+    upsample_conv3x3_gather=_upsample_conv3x3_gather,
     bilinear_resample_concat=_bilinear_resample_concat,
     bilinear_align_corners_nhwc=_bilinear_align_corners_nhwc,
     batched_transpose=_batched_transpose,
@@ -590,6 +617,11 @@ def bilinear_resample_concat(sources, size, pre_biases=None, pre_flags=None, pre
                                           None if pre_biases is None else [None if b is None else b.detach()
                                                                            for b in pre_biases],
                                           pre_flags, pre_activation, pre_count, post_activation)
+
+
+def upsample_conv3x3_gather(Z: Tensor, bias, size, activation=None, count: int = 1) -> Tensor:
+    """act^count(conv3x3(interpolate(X)) + bias) from the per-tap products Z of X at low resolution (inference only)."""
+    return dexts.upsample_conv3x3_gather(Z.detach(), None if bias is None else bias.detach(), size, activation, count)
 
 
 def bilinear_nhwc_affine(X: Tensor, size, extra: Tensor = None, weight_extra_kn: Tensor = None) -> Tensor:

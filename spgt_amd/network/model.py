@@ -7,8 +7,10 @@ import torch
 import torch.nn.functional as F
 from torch import Tensor, nn
 
-from ..extension.bind.datamove import (bilinear_align_corners, bilinear_align_corners_nhwc, bilinear_resample,
-                                       bilinear_resample_concat, conv3x3_resample, conv3x3_resample_supported)
+from ..extension.bind.datamove import (bilinear_align_corners, bilinear_align_corners_nhwc, bilinear_nhwc_affine,
+                                       bilinear_resample, bilinear_resample_concat, conv3x3_resample,
+                                       conv3x3_resample_supported, upsample_conv3x3_gather)
+from ..extension.bind.linear import fused_linear, linear_supported
 from .layer import ConvResBlock2D, activation_name, always_dropout, gpu_inference, make_activation
 
 
@@ -99,10 +101,45 @@ class UpScaler2D(nn.Module):
         return (gpu_inference(X, *self.parameters()) and self.droprate == 0 and self.conv.fusable(X) and
                 type(self.conv.activation_layer) is type(self.activation_layer))
 
+    def _tap_weight_kn(self) -> Tensor:
+        """The convolution's weight as [Cin, 9 * Cout], column (3 ky + kx) * Cout + co: the nine per-tap 1x1
+        products as one GEMM operand; rebuilt when the parameter changes."""
+        w = self.conv.conv_layer.weight
+        key = (w.data_ptr(), w._version, w.device)
+        cache = getattr(self, "_spgt_tap_weight", None)
+        if cache is None or cache[0] != key:
+            cache = (key, w.detach().permute(1, 2, 3, 0).reshape(w.size(1), 9 * w.size(0)).contiguous())
+            self._spgt_tap_weight = cache
+        return cache[1]
+
+    def _mixes_before_resampling(self, X: Tensor) -> bool:
+        """True when interpolate -> conv3x3 -> activations is computed as GEMM at the low resolution + gather:
+        fused inference, a plain 3x3 convolution, one kind of activation, and enough up-sampling to pay."""
+        c = self.conv.conv_layer
+        size = self.resolution_size[3]
+        size = (size, size) if isinstance(size, int) else size
+        return (self.can_defer_last_resample(X) and c.kernel_size == (3, 3) and c.padding == (1, 1) and
+                c.stride == (1, 1) and c.dilation == (1, 1) and c.groups == 1 and c.padding_mode == "zeros" and
+                c.out_channels % 4 == 0 and linear_supported(c.in_channels, 9 * c.out_channels) and
+                size[0] * size[1] >= 2 * X.size(1) * X.size(2))
+
+    def _mid_resolution_nhwc(self, X: Tensor) -> Tensor:
+        """interpolate -> conv -> activation -> activation as [N, r_mid, r_mid, out_dim] channels-last."""
+        N, H, W, C = X.shape
+        c = self.conv.conv_layer
+        # conv(interp(X)) = sum over the taps of shifted interp(X . W_tap): the channel mixing runs on the
+        # low-resolution tokens, (r_mid / r_attn)^2 times fewer than the convolution would see
+        Z = fused_linear(X.reshape(N * H * W, C), self._tap_weight_kn())
+        return upsample_conv3x3_gather(Z.view(N, H, W, 9, c.out_channels), c.bias, self.resolution_size[3],
+                                       activation_name(self.activation_layer), 2)
+
     def forward(self, X: Tensor, defer_last_resample: bool = False) -> Tensor:
         """With defer_last_resample (see can_defer_last_resample) the result is the channels-last tensor at
         resolution_size[3], [N, r_mid, r_mid, out_dim], and the caller owes the interpolation to resolution_size[4]:
         a Linear over the channels commutes with it and is cheaper at the lower resolution."""
+        if (defer_last_resample or self.can_defer_last_resample(X)) and self._mixes_before_resampling(X):
+            X = self._mid_resolution_nhwc(X.contiguous())
+            return X if defer_last_resample else bilinear_nhwc_affine(X, self.resolution_size[4])
         if defer_last_resample:
             X = bilinear_resample(X.contiguous(), self.resolution_size[3], src_nhwc=True)
             # the block's bias, its activation and the scaler's own on the way to channels-last: a resampling to

@@ -299,6 +299,37 @@ def test_bilinear_resample_concat_rejects(gpu):
         dm.bilinear_resample_concat([x, rnd(1, 1, 4, 5, seed=2).to(gpu)], (5, 5))
 
 
+@pytest.mark.parametrize("N,hw,size,cin,cout", [(2, (5, 7), (9, 12), 6, 8), (1, (71, 71), (122, 122), 16, 128),
+                                                 (2, (4, 4), (4, 4), 3, 4), (1, (3, 5), (1, 2), 5, 12),
+                                                 (2, (1, 1), (3, 3), 2, 4)])
+@pytest.mark.parametrize("act,count", [(None, 1), ("relu", 1), ("silu", 2)])
+def test_upsample_conv3x3_gather(gpu, N, hw, size, cin, cout, act, count):
+    """interpolate -> conv3x3(padding 1) -> bias -> activations (network/model.py:59-62) from the per-tap products
+    of the low-resolution input, against torch's float64 convolution of the float64 oracle resampling."""
+    x = rnd(N, cin, hw[0], hw[1], seed=101).double()
+    w = rnd(cout, cin, 3, 3, seed=102).double()
+    b = rnd(cout, seed=103).double()
+    want = torch.nn.functional.conv2d(O.bilinear_align_corners(x, size), w, b, padding=1)
+    want = _act64(want, act, count).permute(0, 2, 3, 1)
+    # Z[n, h, w, 3 ky + kx, co] = sum_ci x[n, ci, h, w] * w[co, ci, ky, kx]
+    Z = torch.einsum("nchw,ocyx->nhwyxo", x, w).reshape(N, hw[0], hw[1], 9, cout).float().contiguous()
+    got = dm.upsample_conv3x3_gather(Z.to(gpu), b.float().to(gpu), size, act, count)
+    assert got.is_contiguous() and got.shape == want.shape
+    assert (got.cpu().double() - want).abs().max().item() <= 2e-5 * max(1.0, want.abs().max().item())
+    no_bias = dm.upsample_conv3x3_gather(Z.to(gpu), None, size, None, 1).cpu().double()
+    want0 = torch.nn.functional.conv2d(O.bilinear_align_corners(x, size), w, None, padding=1).permute(0, 2, 3, 1)
+    assert (no_bias - want0).abs().max().item() <= 2e-5 * max(1.0, want0.abs().max().item())
+
+
+def test_upsample_conv3x3_gather_rejects(gpu):
+    with pytest.raises(ValueError):
+        dm.upsample_conv3x3_gather(rnd(1, 4, 4, 8, 4, seed=1).to(gpu), None, (5, 5))  # 8 taps
+    with pytest.raises(ValueError):
+        dm.upsample_conv3x3_gather(rnd(1, 4, 4, 9, 6, seed=1).to(gpu), None, (5, 5))  # 6 channels
+    with pytest.raises(ValueError):
+        dm.upsample_conv3x3_gather(rnd(1, 4, 4, 9, 4, seed=1).to(gpu), rnd(5, seed=2).to(gpu), (5, 5))
+
+
 def test_bilinear_nhwc_affine_rejects(gpu):
     with pytest.raises(ValueError):
         dm.bilinear_nhwc_affine(rnd(1, 4, 4, 6, seed=1).to(gpu), (5, 5))  # 6 channels: not a multiple of 4
