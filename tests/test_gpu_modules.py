@@ -101,10 +101,12 @@ def test_state_dict_layout_matches_reference(gpu):
     assert tuple(fw.shape) == (mode, mode, width, width, 2)
 
 
-def test_full_model_vs_oracle_mid_size(gpu):
-    """r = 43 -> r_attn = 22 with the resolution rule of the reference, random init, against the oracle in fp64."""
+@pytest.mark.parametrize("r,ra", [(43, 22), (40, 12)])
+def test_full_model_vs_oracle_mid_size(gpu, r, ra):
+    """r = 43 -> r_attn = 22 with the resolution rule of the reference, and r = 40 -> 24 -> 12, where the up-scaler's
+    convolution mixes channels before its interpolation; random init, against the oracle in fp64."""
     torch.manual_seed(3)
-    rs = O.resolution_sizes(43, 22)
+    rs = O.resolution_sizes(r, ra) if (r, ra) == (43, 22) else [[40, 40], [24, 24], [12, 12], [24, 24], [40, 40]]
     cfg = dict(
         drop_module=0.0, boundary_condition="dirichlet", target_normalizer=SM.UnitNormalizer(), resolution_size=rs,
         dim_node=1, dim_hidden=128, drop_downscaler=0.0, acti_downscaler="relu", num_encoder_layer=3, num_head=4,
@@ -115,10 +117,10 @@ def test_full_model_vs_oracle_mid_size(gpu):
     m = SM.Sp_GalerkinTransformer2D(cfg)
     sd = {k: v.clone() for k, v in m.state_dict().items()}
     g = torch.Generator().manual_seed(4)
-    x = torch.randn(2, 43, 43, 1, generator=g)
+    x = torch.randn(2, r, r, 1, generator=g)
     lin = lambda n: torch.linspace(0, 1, n)
     mesh = lambda n: torch.stack(torch.meshgrid(lin(n), lin(n), indexing="ij"), dim=-1)[None].repeat(2, 1, 1, 1)
-    pos, grid = mesh(22), mesh(43)
+    pos, grid = mesh(ra), mesh(r)
     # oracle parameters: it computes x @ W^T with [Cin, Cout, m, m, 2] Fourier weights
     po = {}
     for k, v in sd.items():
@@ -152,6 +154,29 @@ def test_deferred_upsampling_matches_module_order(gpu):
         got = dec(low, grid, resample_to=rs[4])
     assert got.shape == want.shape
     assert rel_l2(got.cpu(), want.cpu()) < 1e-5 and max_rel(got.cpu(), want.cpu()) < 1e-4
+
+
+@pytest.mark.parametrize("act", ["silu", "relu"])
+def test_up_scaler_mixing_before_resampling(gpu, act):
+    """interpolate -> conv3x3 -> activations (network/model.py:59-62) computed as a GEMM on the low-resolution
+    tokens plus a 9-tap gather, against the float64 oracle in the reference's order of operations; sizes with
+    enough up-sampling for the fused path to choose this form (the golden vectors' sizes do not)."""
+    torch.manual_seed(21)
+    rs = [[20, 20], [14, 14], [8, 8], [14, 14], [20, 20]]
+    m = M.UpScaler2D(rs, 128, 128, 0.0, act).eval()
+    x = torch.randn(2, 8, 8, 128)
+    want = O.up_scaler({k: v.double() for k, v in m.state_dict().items()}, x.double(), rs, act)
+    with torch.no_grad():
+        mg = m.to(gpu)
+        xg = x.to(gpu)
+        assert mg._mixes_before_resampling(xg)
+        got = mg(xg)
+        low = mg(xg, defer_last_resample=True)
+    assert got.shape == want.shape and tuple(low.shape) == (2, 14, 14, 128)
+    assert max_rel(got.cpu().double(), want) < 1e-5
+    # the deferred form is the same tensor before the last interpolation
+    from spgt_amd.extension.bind.datamove import bilinear_nhwc_affine
+    assert torch.equal(bilinear_nhwc_affine(low, (20, 20)), got)
 
 
 def test_graphed_inference_replays_match_eager(gpu):
