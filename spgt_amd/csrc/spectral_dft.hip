@@ -1,3 +1,12 @@
+#define SPGT_LOAD_X_ONE(BASE_, W0_, I_)                        \
+    if ((I_) == 0) s0 = SPGT_X_PIECE(BASE_, W0_, 0);           \
+    else if ((I_) == 1) s1 = SPGT_X_PIECE(BASE_, W0_, 1);      \
+    else if ((I_) == 2) s2 = SPGT_X_PIECE(BASE_, W0_, 2);      \
+    else if ((I_) == 3) s3 = SPGT_X_PIECE(BASE_, W0_, 3);      \
+    else if ((I_) == 4) s4 = SPGT_X_PIECE(BASE_, W0_, 4);      \
+    else if ((I_) == 5) s5 = SPGT_X_PIECE(BASE_, W0_, 5);      \
+    else if ((I_) == 6) s6 = SPGT_X_PIECE(BASE_, W0_, 6);      \
+    else s7 = SPGT_X_PIECE(BASE_, W0_, 7);
 // Truncated DFT along the last grid axis of the FNO spectral layer, as MFMA products
 // against a small table of twiddle factors.
 //
@@ -364,99 +373,136 @@ __global__ __launch_bounds__(256) void spectral_rows_expand_k(
 // i.e. the residual Linear, the inverse DFT along w of the retained modes, their sum and the activation;
 // the inverse transform's result never goes to memory.  64 channels in and out, planar U [N][2m][r][64].
 // Both terms are MFMA products with output channels along the accumulator's registers and grid points along
-// its lanes (so a lane stores four 16-byte pieces of its grid point's row): A = W resp. U in registers,
+// its lanes (so a lane stores 16-byte pieces of its grid point's row): A = W resp. U in registers,
 // B = x tile (from a wave-private LDS tile, 16-byte reads, lane (w, kh) takes channels kh*32 + kk) resp.
 // table entries (handed over in operand order, tabA[tile][kk][lane] = table[32 tile + lane%32][2kk +
-// lane/32], zero outside).  A wave owns one half of the channels and every second 32-point tile of a grid
-// row; no barriers.  grid (rows), block 256.
-__global__ __launch_bounds__(256) void spectral_inverse_linear_k(
+// lane/32], zero outside).  No barriers.
+// One wave per SIMD (waves that share a SIMD's matrix pipe run their MFMAs at about half the rate of a lone
+// wave; with four waves per SIMD and a wave per half of the channels this pass took 44 us at [4, 211, 211, 64],
+// with two fatter waves 43-51 us, with one 34 us): a wave makes all 64 channels of a 32-point tile, two
+// independent accumulator chains off the same x and table operands, and walks the (grid row, tile) pairs of the
+// whole input 4 * gridDim.x apart.  Per pair: the parked x rows go to the wave's LDS tile; this pair's U and table entries and the next
+// pair's x rows are requested (wave-uniform base + 32-bit lane offsets, computed once for U); then the 64 MFMAs
+// of the Linear, the MFMAs of the inverse transform, activation and stores.  Stores are unconditional: points
+// past the end of a grid row are computed from the row's last point and that point's table entries, and write
+// its own values to its address.
+// KSU: MFMA steps of the inverse transform, modes rounded up to a multiple of 4 (the table entries of the steps
+// past the modes are zero); a template parameter so that neither the loads nor the MFMAs sit behind branches.
+// grid (min(ceil(pairs / 4), CUs)), block 256.
+template <int ACT, int KSU>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void spectral_inverse_linear_k(
     const float* __restrict__ U, const float* __restrict__ tabA, const float* __restrict__ x,
-    const float* __restrict__ Wkn, const float* __restrict__ bias, int act, float* __restrict__ out, int r, int m2) {
+    const float* __restrict__ Wkn, const float* __restrict__ bias, float* __restrict__ out, int r, int m2,
+    unsigned pairs) {
     constexpr int C = 64, PX = C + 4;
+    static_assert(KSU % 4 == 0 && KSU >= 4 && KSU <= 16, "4, 8, 12 or 16 steps");
     __shared__ __attribute__((aligned(16))) float xs[4][32 * PX];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int tk = lane & 31;
     const int kh = lane >> 5;
-    const int cb = wave & 1;
-    const int64_t row = blockIdx.x;
-    const int64_t n = row / r;
-    const int64_t h = row - n * r;
-    const int WT = (r + 31) / 32;
-    const int KS = m2 / 2;
+    const unsigned WT = (unsigned)(r + 31) / 32;
+    const unsigned stride = gridDim.x * 4;
 
-    float wreg[32];  // W[c = kh*32 + kk][o = cb*32 + tk]
+    float wreg0[32], wreg1[32];  // W[c = kh*32 + kk][o = cb*32 + tk], cb = 0, 1
 #pragma unroll
-    for (int kk = 0; kk < 32; ++kk) wreg[kk] = Wkn[(kh * 32 + kk) * C + cb * 32 + tk];
-    float ureg[16];  // U[j = 2kk + kh][o]
-    {
-        const float* up = U + (n * m2 * r + h) * (int64_t)C + cb * 32 + tk;  // U[n][j][h][o]
-#pragma unroll
-        for (int kk = 0; kk < 16; ++kk) ureg[kk] = (2 * kk + kh < m2) ? up[(int64_t)(2 * kk + kh) * r * C] : 0.f;
+    for (int kk = 0; kk < 32; ++kk) {
+        wreg0[kk] = Wkn[(kh * 32 + kk) * C + tk];
+        wreg1[kk] = Wkn[(kh * 32 + kk) * C + 32 + tk];
     }
-    // bias in accumulator layout: element 4q + e belongs to channel cb*32 + 8q + 4kh + e
-    v16f bo;
+    // bias in accumulator layout (element 4q + e of half cb belongs to channel cb*32 + 8q + 4kh + e): the C operand
+    // of a pair's first MFMAs
+    v16f bo0, bo1;
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-        const float4 b4 = bias ? *reinterpret_cast<const float4*>(bias + cb * 32 + 8 * q + 4 * kh) : make_float4(0.f, 0.f, 0.f, 0.f);
-        bo[4 * q + 0] = b4.x; bo[4 * q + 1] = b4.y; bo[4 * q + 2] = b4.z; bo[4 * q + 3] = b4.w;
+        const float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
+        const float4 b0 = bias ? *reinterpret_cast<const float4*>(bias + 8 * q + 4 * kh) : z;
+        const float4 b1 = bias ? *reinterpret_cast<const float4*>(bias + 32 + 8 * q + 4 * kh) : z;
+        bo0[4 * q + 0] = b0.x; bo0[4 * q + 1] = b0.y; bo0[4 * q + 2] = b0.z; bo0[4 * q + 3] = b0.w;
+        bo1[4 * q + 0] = b1.x; bo1[4 * q + 1] = b1.y; bo1[4 * q + 2] = b1.z; bo1[4 * q + 3] = b1.w;
     }
+    // lane offsets of U[n][j = 2kk + kh][h][o = tk] from U[n][0][h][0]; steps past the modes read the last mode
+    // (finite values that meet zero table entries)
+    uint32_t uoff[KSU];
+#pragma unroll
+    for (int kk = 0; kk < KSU; ++kk) uoff[kk] = (uint32_t)min(2 * kk + kh, m2 - 1) * (uint32_t)(r * C) + (uint32_t)tk;
     float* const xw = xs[wave];
-    const float* const xrow = x + row * (int64_t)r * C;
-    float* const orow = out + row * (int64_t)r * C + cb * 32 + 4 * kh;
 
-    // this wave's tiles: wave>>1, wave>>1 + 2, ...; tile rows past the end of the grid row read its last point
     // (named registers and macros: a register array that lives across the loop ends up in scratch memory)
+    // piece I of a tile is row (lane + 64 I) / 16, channels 4 (lane % 16) ..; rows past the end of the grid row
+    // read its last point
     float4 s0, s1, s2, s3, s4, s5, s6, s7;
-#define SPGT_X_PIECE(WT_, I_) \
-    (*reinterpret_cast<const float4*>(xrow + (int64_t)min((WT_) * 32 + ((lane + 64 * (I_)) >> 4), r - 1) * C + 4 * (lane & 15)))
-#define SPGT_LOAD_X_TILE(WT_)                                                                            \
-    s0 = SPGT_X_PIECE(WT_, 0); s1 = SPGT_X_PIECE(WT_, 1); s2 = SPGT_X_PIECE(WT_, 2); s3 = SPGT_X_PIECE(WT_, 3); \
-    s4 = SPGT_X_PIECE(WT_, 4); s5 = SPGT_X_PIECE(WT_, 5); s6 = SPGT_X_PIECE(WT_, 6); s7 = SPGT_X_PIECE(WT_, 7);
+#define SPGT_X_PIECE(BASE_, W0_, I_) \
+    (*reinterpret_cast<const float4*>((BASE_) + (uint32_t)(min((W0_) + ((lane + 64 * (I_)) >> 4), r - 1) * C + 4 * (lane & 15))))
+#define SPGT_LOAD_X_TILE(T_)                                                                        \
+    {                                                                                               \
+        const unsigned row_ = (T_) / WT;                                                            \
+        const int w0_ = (int)((T_) - row_ * WT) * 32;                                               \
+        const float* xb_ = x + (int64_t)row_ * r * C;                                               \
+        s0 = SPGT_X_PIECE(xb_, w0_, 0); s1 = SPGT_X_PIECE(xb_, w0_, 1); s2 = SPGT_X_PIECE(xb_, w0_, 2); \
+        s3 = SPGT_X_PIECE(xb_, w0_, 3); s4 = SPGT_X_PIECE(xb_, w0_, 4); s5 = SPGT_X_PIECE(xb_, w0_, 5); \
+        s6 = SPGT_X_PIECE(xb_, w0_, 6); s7 = SPGT_X_PIECE(xb_, w0_, 7);                             \
+    }
 #define SPGT_STORE_X_PIECE(I_, V_) \
     *reinterpret_cast<float4*>(xw + ((lane + 64 * (I_)) >> 4) * PX + 4 * (lane & 15)) = V_;
-    int wt = wave >> 1;
-    if (wt < WT) { SPGT_LOAD_X_TILE(wt) }
-    for (; wt < WT; wt += 2) {
+    unsigned t = blockIdx.x * 4 + wave;
+    if (t < pairs) SPGT_LOAD_X_TILE(t)
+    for (; t < pairs; t += stride) {
+        const unsigned row = t / WT;
+        const int wt = (int)(t - row * WT);
+        const unsigned n = row / (unsigned)r;
+        const unsigned h = row - n * (unsigned)r;
         SPGT_STORE_X_PIECE(0, s0) SPGT_STORE_X_PIECE(1, s1) SPGT_STORE_X_PIECE(2, s2) SPGT_STORE_X_PIECE(3, s3)
         SPGT_STORE_X_PIECE(4, s4) SPGT_STORE_X_PIECE(5, s5) SPGT_STORE_X_PIECE(6, s6) SPGT_STORE_X_PIECE(7, s7)
-        if (wt + 2 < WT) { SPGT_LOAD_X_TILE(wt + 2) }
-        float ta[16];
+        const float* ub = U + ((int64_t)n * m2 * r + h) * C;  // U[n][0][h][0]
+        float ureg0[KSU], ureg1[KSU];
 #pragma unroll
-        for (int kk = 0; kk < 16; ++kk) ta[kk] = (kk < KS) ? tabA[((int64_t)wt * 16 + kk) * 64 + lane] : 0.f;
-        v16f acc = bo;
+        for (int kk = 0; kk < KSU; ++kk) {
+            ureg0[kk] = ub[uoff[kk]];
+            ureg1[kk] = ub[uoff[kk] + 32u];
+        }
+        // the operand table holds 16 steps per tile; points past the row's end take the last point's entries
+        const float* tb = tabA + (int64_t)wt * (16 * 64);
+        const uint32_t tl = (uint32_t)(kh * 32 + min(tk, r - 1 - wt * 32));
+        float ta[KSU];
+#pragma unroll
+        for (int kk = 0; kk < KSU; ++kk) ta[kk] = tb[tl + (uint32_t)(kk * 64)];
+        SPGT_LOAD_X_TILE(min(t + stride, pairs - 1))  // after the last pair: loaded again, not used
         const float* xr = xw + tk * PX + kh * 32;
         float4 xv[8];
 #pragma unroll
         for (int g = 0; g < 8; ++g) xv[g] = *reinterpret_cast<const float4*>(xr + 4 * g);
         __builtin_amdgcn_sched_barrier(0);
+        v16f acc0 = bo0, acc1 = bo1;
 #pragma unroll
         for (int g = 0; g < 8; ++g) {
-            acc = mfma32(wreg[4 * g + 0], xv[g].x, acc);
-            acc = mfma32(wreg[4 * g + 1], xv[g].y, acc);
-            acc = mfma32(wreg[4 * g + 2], xv[g].z, acc);
-            acc = mfma32(wreg[4 * g + 3], xv[g].w, acc);
+            acc0 = mfma32(wreg0[4 * g + 0], xv[g].x, acc0);
+            acc1 = mfma32(wreg1[4 * g + 0], xv[g].x, acc1);
+            acc0 = mfma32(wreg0[4 * g + 1], xv[g].y, acc0);
+            acc1 = mfma32(wreg1[4 * g + 1], xv[g].y, acc1);
+            acc0 = mfma32(wreg0[4 * g + 2], xv[g].z, acc0);
+            acc1 = mfma32(wreg1[4 * g + 2], xv[g].z, acc1);
+            acc0 = mfma32(wreg0[4 * g + 3], xv[g].w, acc0);
+            acc1 = mfma32(wreg1[4 * g + 3], xv[g].w, acc1);
         }
 #pragma unroll
-        for (int kk = 0; kk < 16; ++kk)
-            if (kk < KS) acc = mfma32(ureg[kk], ta[kk], acc);
-        float y[16];
-#pragma unroll
-        for (int q = 0; q < 16; ++q) y[q] = acc[q];
-        if (act == SPGT_ACT_RELU) {
-#pragma unroll
-            for (int q = 0; q < 16; ++q) y[q] = fmaxf(y[q], 0.f);
-        } else if (act == SPGT_ACT_SILU) {
-#pragma unroll
-            for (int q = 0; q < 16; ++q) y[q] = y[q] * __builtin_amdgcn_rcpf(1.f + __expf(-y[q]));
+        for (int kk = 0; kk < KSU; ++kk) {
+            acc0 = mfma32(ureg0[kk], ta[kk], acc0);
+            acc1 = mfma32(ureg1[kk], ta[kk], acc1);
         }
-        // y[4q + e] = out[w = wt*32 + tk][o = cb*32 + 8q + 4kh + e]
-        const int w = wt * 32 + tk;
-        if (w < r) {
+        // acc{cb}[4q + e] = out[w][o = cb*32 + 8q + 4kh + e] before the activation
+        float y[32];
 #pragma unroll
-            for (int q = 0; q < 4; ++q)
-                *reinterpret_cast<float4*>(orow + (int64_t)w * C + 8 * q) = make_float4(y[4 * q], y[4 * q + 1], y[4 * q + 2], y[4 * q + 3]);
+        for (int q = 0; q < 16; ++q) y[q] = acc0[q], y[16 + q] = acc1[q];
+#pragma unroll
+        for (int q = 0; q < 32; ++q) {
+            if (ACT == SPGT_ACT_RELU) y[q] = fmaxf(y[q], 0.f);
+            if (ACT == SPGT_ACT_SILU) y[q] = y[q] * __builtin_amdgcn_rcpf(1.f + __expf(-y[q]));
         }
+        float* const op = out + ((int64_t)row * r + min(wt * 32 + tk, r - 1)) * C + 4 * kh;
+#pragma unroll
+        for (int q = 0; q < 8; ++q)
+            *reinterpret_cast<float4*>(op + 8 * q) = make_float4(y[4 * q], y[4 * q + 1], y[4 * q + 2], y[4 * q + 3]);
     }
 #undef SPGT_LOAD_X_TILE
 #undef SPGT_X_PIECE
@@ -589,7 +635,22 @@ extern "C" int spgt_spectral_inverse_linear(const float* U, const float* table_o
         return fail(SPGT_ERR_INVALID_ARGUMENT,
                     "spectral_inverse_linear: x, out and bias must be 16-byte aligned, the rest 4-byte aligned");
     if (out == x) return fail(SPGT_ERR_INVALID_ARGUMENT, "spectral_inverse_linear: out must not alias x");
-    hipLaunchKernelGGL(spectral_inverse_linear_k, dim3((unsigned)rows), dim3(256), 0, stream, U, table_operand, x,
-                       weight_kn, bias, activation, out, r, 2 * modes);
+    const int64_t pairs = (int64_t)rows * ((r + 31) / 32);
+    if (pairs > (int64_t)INT32_MAX - 4096)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "spectral_inverse_linear: more than 2^31 tiles of 32 grid points");
+    const dim3 grid((unsigned)std::min<int64_t>(ceil_div(pairs, (int64_t)4), (int64_t)device_cu_count()));
+#define SPGT_SIL_LAUNCH(ACT, KSU)                                                                                 \
+    hipLaunchKernelGGL((spectral_inverse_linear_k<ACT, KSU>), grid, dim3(256), 0, stream, U, table_operand, x, \
+                       weight_kn, bias, out, r, 2 * modes, (unsigned)pairs)
+#define SPGT_SIL_STEPS(ACT)                         \
+    if (modes <= 4) SPGT_SIL_LAUNCH(ACT, 4);        \
+    else if (modes <= 8) SPGT_SIL_LAUNCH(ACT, 8);   \
+    else if (modes <= 12) SPGT_SIL_LAUNCH(ACT, 12); \
+    else SPGT_SIL_LAUNCH(ACT, 16)
+    if (activation == SPGT_ACT_RELU) { SPGT_SIL_STEPS(SPGT_ACT_RELU); }
+    else if (activation == SPGT_ACT_SILU) { SPGT_SIL_STEPS(SPGT_ACT_SILU); }
+    else { SPGT_SIL_STEPS(SPGT_ACT_NONE); }
+#undef SPGT_SIL_STEPS
+#undef SPGT_SIL_LAUNCH
     return check_launch("spectral_inverse_linear");
 }
