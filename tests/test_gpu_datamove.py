@@ -501,7 +501,8 @@ def test_denormalize_boundary_rejects_bad_shapes(gpu):
 
 
 
-@pytest.mark.parametrize("N,r,m", [(1, 33, 4), (2, 64, 12), (4, 211, 12), (2, 141, 16), (1, 32, 16)])
+@pytest.mark.parametrize("N,r,m", [(1, 33, 4), (2, 64, 12), (4, 211, 12), (2, 141, 16), (1, 32, 16), (1, 40, 6),
+                                   (2, 7, 3), (3, 5, 1), (1, 97, 9)])
 @pytest.mark.parametrize("act", [None, "relu", "silu"])
 def test_spectral_inverse_linear_matches_separate_kernels(gpu, N, r, m, act):
     """The fused end of the spectral layer against its parts: truncated_dft_rows_inverse + fused_linear with the
