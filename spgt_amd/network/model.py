@@ -137,7 +137,7 @@ class UpScaler2D(nn.Module):
         """With defer_last_resample (see can_defer_last_resample) the result is the channels-last tensor at
         resolution_size[3], [N, r_mid, r_mid, out_dim], and the caller owes the interpolation to resolution_size[4]:
         a Linear over the channels commutes with it and is cheaper at the lower resolution."""
-        if (defer_last_resample or self.can_defer_last_resample(X)) and self._mixes_before_resampling(X):
+        if self._mixes_before_resampling(X):
             X = self._mid_resolution_nhwc(X.contiguous())
             return X if defer_last_resample else bilinear_nhwc_affine(X, self.resolution_size[4])
         if defer_last_resample:
