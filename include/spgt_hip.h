@@ -395,6 +395,32 @@ int spgt_encoder_tail_forward(const float* attn_out, int64_t ld_attn, const floa
                               float* out, int64_t tokens, int attn_features, int dim_hidden,
                               int ffn_hidden, spgt_stream_t stream);
 
+/* The attention core with its last product folded into the layer's output projection
+ * (Sp_GalerkinAttention.forward, network/sp_layer.py:64-75: out = fc_layer(Q~ (K~^T V~ / S))).  The product is
+ * associative, (Q~ M_h) Wfc_h = Q~ (M_h Wfc_h), so the pass over Q and the [tokens, H*(dp+32)] attention
+ * output disappear; three calls replace spgt_galerkin_attention_fused_forward + spgt_encoder_tail_forward:
+ *   spgt_galerkin_attention_ktv_forward   K/V pass and tile reduction only: ktv [B, H, dp+32, dp+32] = M
+ *                                         (arguments as in spgt_galerkin_attention_fused_forward, same workspace)
+ *   spgt_fold_ktv_into_fc                 folded [B, H*32, out_features]: row h*32 + i = (M_h Wfc_h)[dp + i], and
+ *                                         folded_pos [B, dp, out_features]: row p = sum_h (M_h Wfc_h)[p]
+ *                                         (fc_weight_kn [H*(dp+32), out_features], the transposed fc_layer weight)
+ *   spgt_encoder_tail_folded_forward      y1 = x + q @ folded[b] + position @ folded_pos[b] + fc_bias, then the
+ *                                         feed-forward net as in spgt_encoder_tail_forward; q [B*S, 128] (row
+ *                                         stride ld_q) is the projected Q, position [B*S, 2] (dp == 2) or null */
+int spgt_galerkin_attention_ktv_forward(const float* K, const float* V, int64_t ld_in, const float* position,
+                                        const float* ln_weight_K, const float* ln_bias_K,
+                                        const float* ln_weight_V, const float* ln_bias_V, float norm_eps,
+                                        float* ktv, void* workspace, size_t workspace_bytes, int B, int S, int H,
+                                        int dp, spgt_stream_t stream);
+int spgt_fold_ktv_into_fc(const float* ktv, const float* fc_weight_kn, float* folded, float* folded_pos, int B,
+                          int H, int dp, int out_features, spgt_stream_t stream);
+int spgt_encoder_tail_folded_forward(const float* q, int64_t ld_q, const float* position, const float* x,
+                                     const float* folded_fc, const float* folded_pos, const float* fc_bias,
+                                     const float* ffn1_weight_kn, const float* ffn1_bias,
+                                     const float* ffn2_weight_kn, const float* ffn2_bias, int activation,
+                                     float* out, int B, int64_t S, int dp, int dim_hidden, int ffn_hidden,
+                                     spgt_stream_t stream);
+
 /* Instrumented variant of spgt_galerkin_attention_fused_forward for benchmarks
  * (no reference counterpart): runs the call `iterations` times, synchronising
  * after each, with HIP events recorded on `stream` around each of its three

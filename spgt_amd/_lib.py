@@ -68,6 +68,11 @@ SIGNATURES = {
     "spgt_ffn_scalar_forward": (_i, [_p, _i64, _p, _p, _p, _p, _i, _p, _i64, _i, _i, _p]),
     "spgt_encoder_tail_supported": (_i, [_i, _i, _i]),
     "spgt_encoder_tail_forward": (_i, [_p, _i64, _p, _p, _p, _p, _p, _p, _p, _i, _p, _i64, _i, _i, _i, _p]),
+    "spgt_galerkin_attention_ktv_forward": (
+        _i, [_p, _p, _i64, _p, _p, _p, _p, _p, _f, _p, _p, _sz, _i, _i, _i, _i, _p]),
+    "spgt_fold_ktv_into_fc": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _p]),
+    "spgt_encoder_tail_folded_forward": (
+        _i, [_p, _i64, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _p, _i, _i64, _i, _i, _i, _p]),
     "spgt_galerkin_attention_fused_profile": (
         _i, [_p, _p, _p, _i64, _p, _p, _p, _p, _p, _f, _p, _p, _p, _sz, _i, _i, _i, _i, _p, _i,
              ctypes.POINTER(ctypes.c_float)]),

@@ -588,7 +588,8 @@ int fused_forward_impl(
     const float* ln_weight_K, const float* ln_bias_K, const float* ln_weight_V,
     const float* ln_bias_V, float norm_eps, float* out, float* ktv, void* workspace,
     size_t workspace_bytes, int B, int S, int H, int dp, hipStream_t stream, hipEvent_t* ev) {
-    if (!Q || !K || !V || !out || !ktv || !ln_weight_K || !ln_bias_K || !ln_weight_V || !ln_bias_V)
+    const bool apply = Q != nullptr || out != nullptr;  // neither: K/V pass and reduction only
+    if ((apply && (!Q || !out)) || !K || !V || !ktv || !ln_weight_K || !ln_bias_K || !ln_weight_V || !ln_bias_V)
         return fail(SPGT_ERR_INVALID_ARGUMENT, "galerkin_attention_fused: null pointer argument");
     if (B <= 0 || S <= 0 || H <= 0)
         return fail(SPGT_ERR_INVALID_ARGUMENT, "galerkin_attention_fused: B, S, H must be positive");
@@ -601,7 +602,7 @@ int fused_forward_impl(
     if (ld_in < (int64_t)H * 32 || (ld_in % 4) != 0)
         return fail(SPGT_ERR_INVALID_ARGUMENT,
                     "galerkin_attention_fused: row stride must be >= H*32 and a multiple of 4 floats");
-    if (!aligned16(Q) || !aligned16(K) || !aligned16(V) || !aligned16(out) || !aligned16(ktv) ||
+    if ((apply && (!aligned16(Q) || !aligned16(out))) || !aligned16(K) || !aligned16(V) || !aligned16(ktv) ||
         (position && !aligned8(position)))
         return fail(SPGT_ERR_INVALID_ARGUMENT, "galerkin_attention_fused: operands must be 16-byte aligned");
     if (B > 65535 || H / 4 > 65535)
@@ -618,7 +619,7 @@ int fused_forward_impl(
     const dim3 grid2(p.nchunk2, H / 4, B);
     const dim3 gridr(ceil_div(D * D, 256), B * H);
     const dim3 blockr(1024);
-    const float* pos = position ? position : Q;  // never dereferenced when dp == 0
+    const float* pos = position ? position : K;  // never dereferenced when dp == 0
     if (ev) (void)hipEventRecord(ev[0], stream);
     if (dp == 0) {
         hipLaunchKernelGGL((ktv_ln_partial_tm<0, kU1>), grid1, block, 0, stream, K, V, pos, ln_weight_K,
@@ -630,6 +631,7 @@ int fused_forward_impl(
     if (ev) (void)hipEventRecord(ev[1], stream);
     hipLaunchKernelGGL(tile_reduce, gridr, blockr, 0, stream, partial, ktv, D * D, p.nchunk1, 1.0f / (float)S);
     if (ev) (void)hipEventRecord(ev[2], stream);
+    if (!apply) return check_launch("galerkin_attention_ktv");
     if (dp == 0) {
         hipLaunchKernelGGL((qm_apply_tm<0, kU2>), grid2, block, 0, stream, Q, pos, ktv, out, S, H, ld_in, p.tpc2);
     } else {
@@ -648,6 +650,108 @@ extern "C" int spgt_galerkin_attention_fused_forward(
     size_t workspace_bytes, int B, int S, int H, int dp, hipStream_t stream) {
     return fused_forward_impl(Q, K, V, ld_in, position, ln_weight_K, ln_bias_K, ln_weight_V, ln_bias_V, norm_eps,
                               out, ktv, workspace, workspace_bytes, B, S, H, dp, stream, nullptr);
+}
+
+extern "C" int spgt_galerkin_attention_ktv_forward(
+    const float* K, const float* V, int64_t ld_in, const float* position, const float* ln_weight_K,
+    const float* ln_bias_K, const float* ln_weight_V, const float* ln_bias_V, float norm_eps, float* ktv,
+    void* workspace, size_t workspace_bytes, int B, int S, int H, int dp, hipStream_t stream) {
+    return fused_forward_impl(nullptr, K, V, ld_in, position, ln_weight_K, ln_bias_K, ln_weight_V, ln_bias_V,
+                              norm_eps, nullptr, ktv, workspace, workspace_bytes, B, S, H, dp, stream, nullptr);
+}
+
+namespace spgt {
+namespace {
+
+// folded[b][h*32 + i][n] = sum_j ktv[b][h][dp + i][j] * fc[h*D + j][n]          (feature rows, i < 32)
+// wpos[b][p][n]          = sum_h sum_j ktv[b][h][p][j] * fc[h*D + j][n]         (position rows, p < dp)
+// i.e. M_h Wfc_h for every head, with the rows split the way the folded encoder tail reads them: the head's 32
+// feature rows meet the projected Q, the position rows of all heads meet the same token position and are summed.
+// grid (4 H + 1, B), block 256.  Workgroup x < 4 H makes 8 feature rows of head x / 4: thread = (output column n,
+// n + 128, ...; half of the rows), with the D values fc[h*D + j][n] of its column in registers (requested before
+// anything else) and the head's M in LDS.  Workgroup 4 H makes the position rows, all heads' columns requested
+// together.  D is a compile-time value so that these loads go out together, behind no branch.
+template <int DP>
+__global__ __launch_bounds__(256) void fold_ktv_into_fc_k(const float* __restrict__ ktv, const float* __restrict__ fc,
+                                                          float* __restrict__ folded, float* __restrict__ wpos,
+                                                          int H, int N) {
+    constexpr int D = DP + 32;
+    extern __shared__ float ms[];  // feature workgroups: the head's M [D][D]; position workgroup: [H][DP][D]
+    const int64_t b = blockIdx.y;
+    const int half = threadIdx.x >> 7;
+    const int n0 = threadIdx.x & 127;
+    if ((int)blockIdx.x < 4 * H) {
+        const int h = blockIdx.x >> 2;
+        const int i0 = 8 * (blockIdx.x & 3) + 4 * half;  // this thread's 4 feature rows
+        float w[D];
+        const int nc = min(n0, N - 1);
+#pragma unroll
+        for (int j = 0; j < D; ++j) w[j] = fc[(int64_t)(h * D + j) * N + nc];
+        for (int e = threadIdx.x; e < D * D; e += 256) ms[e] = ktv[(b * H + h) * D * D + e];
+        __syncthreads();
+        for (int n = n0; n < N; n += 128) {
+            if (n != n0) {
+#pragma unroll
+                for (int j = 0; j < D; ++j) w[j] = fc[(int64_t)(h * D + j) * N + n];
+            }
+#pragma unroll
+            for (int i = i0; i < i0 + 4; ++i) {
+                const float* m = ms + (DP + i) * D;
+                float acc = 0.f;
+#pragma unroll
+                for (int j = 0; j < D; ++j) acc = fmaf(m[j], w[j], acc);
+                folded[(b * H * 32 + h * 32 + i) * (int64_t)N + n] = acc;
+            }
+        }
+    } else if constexpr (DP > 0) {
+        for (int e = threadIdx.x; e < H * DP * D; e += 256) {
+            const int hh = e / (DP * D), rest = e - hh * (DP * D);
+            ms[e] = ktv[(b * H + hh) * D * D + rest];  // rows 0 .. DP-1 of head hh
+        }
+        __syncthreads();
+        if (half < DP) {
+            for (int n = n0; n < N; n += 128) {
+                float acc = 0.f;
+                for (int hh = 0; hh < H; hh += 4) {  // four heads' columns in flight
+                    float w[4][D];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u)
+#pragma unroll
+                        for (int j = 0; j < D; ++j) w[u][j] = fc[(int64_t)(min(hh + u, H - 1) * D + j) * N + n];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        if (hh + u < H) {
+                            const float* m = ms + ((hh + u) * DP + half) * D;
+#pragma unroll
+                            for (int j = 0; j < D; ++j) acc = fmaf(m[j], w[u][j], acc);
+                        }
+                    }
+                }
+                wpos[(b * DP + half) * (int64_t)N + n] = acc;
+            }
+        }
+    }
+}
+
+}  // namespace
+}  // namespace spgt
+
+extern "C" int spgt_fold_ktv_into_fc(const float* ktv, const float* fc_weight_kn, float* folded, float* folded_pos,
+                                     int B, int H, int dp, int out_features, hipStream_t stream) {
+    if (!ktv || !fc_weight_kn || !folded || (dp > 0 && !folded_pos))
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "fold_ktv_into_fc: null pointer argument");
+    if (B <= 0 || H <= 0 || out_features <= 0 || (dp != 0 && dp != 2) || B > 65535 || H > 16000)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "fold_ktv_into_fc: B, H, out_features must be positive, dp 0 or 2");
+    const int D = dp + 32;
+    const size_t lds = (size_t)std::max(D * D, H * dp * D) * sizeof(float);
+    if (lds > 64 * 1024) return fail(SPGT_ERR_INVALID_ARGUMENT, "fold_ktv_into_fc: too many heads for one workgroup");
+    if (dp == 2)
+        hipLaunchKernelGGL(spgt::fold_ktv_into_fc_k<2>, dim3(4 * H + 1, B), dim3(256), lds, stream, ktv, fc_weight_kn,
+                           folded, folded_pos, H, out_features);
+    else
+        hipLaunchKernelGGL(spgt::fold_ktv_into_fc_k<0>, dim3(4 * H, B), dim3(256), lds, stream, ktv, fc_weight_kn,
+                           folded, folded_pos, H, out_features);
+    return check_launch("fold_ktv_into_fc");
 }
 
 extern "C" int spgt_galerkin_attention_fused_profile(

@@ -647,11 +647,19 @@ __device__ __forceinline__ void mfma_acc_done(v16f& acc) { asm volatile("s_nop 1
 // of four k-steps otherwise).  In-kernel cycle counts per tile (MFMA pipe time 4352 + 8192 + 8192): 4650 +
 // 900 epilogue, 10 700 (2500 of it the SiLU epilogue), 9000, 2000 for loads, LDS staging and barriers.
 // grid (min(tiles, CUs)), block 256.
-template <int K1>
+// FOLD: the attention's Q.(K^T V / S) product is folded into the output projection.  (Q~ M_h) Wfc_h = Q~ (M_h Wfc_h),
+// so `a` is the projected Q [T, 128] itself, Wfc a per-batch matrix [B][128][128] (M folded in, the head's
+// feature rows), and the rows of M Wfc that belong to the position columns, summed over the heads, Wpos
+// [B][2][128], meet the token's position pos [T][2] as a rank-2 update of y1 (no Wpos: no position columns).
+// Tiles then never straddle two of the B sequences of S tokens, a workgroup takes consecutive tiles (so that
+// the sequence, and with it the resident fc weights, changes at most a few times), and T = B * S.
+template <int K1, bool FOLD>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void encoder_tail_k(
     const float* __restrict__ a, int64_t lda, const float* __restrict__ x, const float* __restrict__ Wfc,
     const float* __restrict__ bfc, const float* __restrict__ W1, const float* __restrict__ b1,
-    const float* __restrict__ W2, const float* __restrict__ b2, int act, float* __restrict__ out, int64_t T) {
+    const float* __restrict__ W2, const float* __restrict__ b2, int act, float* __restrict__ out, int64_t T,
+    const float* __restrict__ Wpos, const float* __restrict__ pos, int64_t S) {
+    static_assert(!FOLD || K1 == 128, "the folded form reads the projected Q");
     constexpr int D = 128, F = 256, TT = 32;
     constexpr int PA = K1 + 4, PY = D + 4, PH = F + 4;
     constexpr int NVEC = TT * K1 / 4;          // 16-byte pieces of an attention tile
@@ -661,17 +669,35 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     float* const bufY = bufA + TT * PA;        // [TT][PY]
     float* const bufH = bufY + TT * PY;        // [TT][PH]
     float* const bias_s = bufH + TT * PH;      // bfc[128] | b1[256] | b2[128]
+    float* const posw_s = bias_s + 512;        // FOLD: Wpos of the current sequence [2][128]
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int tk = lane & 31;
     const int kh = lane >> 5;
     const int n0 = wave * 32;
-    const int64_t ntiles = (T + TT - 1) / TT;
+    // tile -> first token, end of its sequence; the workgroup's tiles are first, first + step, ... below limit
+    const int64_t tpb = FOLD ? (S + TT - 1) / TT : 0;  // tiles per sequence
+    const int64_t ntiles = FOLD ? (T / S) * tpb : (T + TT - 1) / TT;
+    const int64_t per_wg = (ntiles + gridDim.x - 1) / gridDim.x;
+    const int64_t first = FOLD ? blockIdx.x * per_wg : blockIdx.x;
+    const int64_t limit = FOLD ? min(ntiles, first + per_wg) : ntiles;
+    const int64_t step = FOLD ? 1 : gridDim.x;
+    // (tile counts fit 32 bits: the divisions are cheap ones)
+    auto tile_seq = [&](int64_t tile) { return FOLD ? (int64_t)((uint32_t)tile / (uint32_t)max(tpb, (int64_t)1)) : (int64_t)0; };
+    auto tile_t0 = [&](int64_t tile) {
+        if (!FOLD) return tile * TT;
+        const int64_t b = tile_seq(tile);
+        return b * S + (tile - b * tpb) * TT;
+    };
+    auto tile_end = [&](int64_t tile) { return FOLD ? (tile_seq(tile) + 1) * S : T; };
 
     // ---- resident weights: W?[kh*KK/2 + j][column block + tk]
     float wA[K1 / 2], wB[2][D / 2], wC[F / 2];
+    auto load_fc = [&](const float* W) {
 #pragma unroll
-    for (int j = 0; j < K1 / 2; ++j) wA[j] = (Wfc + (int64_t)j * D)[(uint32_t)(kh * (K1 / 2) * D + n0 + tk)];
+        for (int j = 0; j < K1 / 2; ++j) wA[j] = (W + (int64_t)j * D)[(uint32_t)(kh * (K1 / 2) * D + n0 + tk)];
+    };
+    if (!FOLD) load_fc(Wfc);
 #pragma unroll
     for (int c = 0; c < 2; ++c)
 #pragma unroll
@@ -692,9 +718,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     auto piece_col = [&](int i) { return 4 * (min((int)threadIdx.x + 256 * i, NVEC - 1) % (K1 / 4)); };
     const uint32_t ulda = (uint32_t)lda;
     auto load_a = [&](int64_t tile) {
-        const int64_t t0 = tile * TT;
+        const int64_t t0 = tile_t0(tile);
         const float* const base = a + t0 * lda;
-        const int lastrow = (int)min((int64_t)TT - 1, T - 1 - t0);  // wave-uniform
+        const int lastrow = (int)min((int64_t)TT - 1, tile_end(tile) - 1 - t0);  // wave-uniform
         auto ld = [&](int i) {
             return *reinterpret_cast<const float4*>(base + (uint32_t)min(piece_row(i), lastrow) * ulda + (uint32_t)piece_col(i));
         };
@@ -720,24 +746,35 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 
     // residual rows of a tile, requested a tile ahead too (rows past the end read the last row: never written out)
     float4 xq[4];
+    float2 pq = make_float2(0.f, 0.f);  // FOLD: the token's position
     auto load_x = [&](int64_t tile) {
-        const int64_t row = min(tile * TT + tk, T - 1);
+        const int64_t row = min(tile_t0(tile) + tk, tile_end(tile) - 1);
 #pragma unroll
         for (int q = 0; q < 4; ++q) xq[q] = *reinterpret_cast<const float4*>(x + row * D + n0 + 4 * kh + 8 * q);
+        if (FOLD && Wpos) pq = *reinterpret_cast<const float2*>(pos + row * 2);
     };
-    const int64_t first = blockIdx.x;
-    if (first < ntiles) {
+    int64_t cur_b = -1;  // FOLD: the sequence whose fc weights are resident
+    if (first < limit) {
         load_a(first);
         store_a();
         load_x(first);
     }
     __builtin_amdgcn_s_waitcnt(0);  // weights are in: no wait for them is left inside the loop
     __syncthreads();
-    for (int64_t tile = first; tile < ntiles; tile += gridDim.x) {
-        const int64_t t = tile * TT + tk;
-        const bool tok = t < T;
-        const bool more = tile + gridDim.x < ntiles;
-        if (more) load_a(tile + gridDim.x);
+    for (int64_t tile = first; tile < limit; tile += step) {
+        const int64_t t = tile_t0(tile) + tk;
+        const bool tok = t < tile_end(tile);
+        const bool more = tile + step < limit;
+        if (FOLD && tile_seq(tile) != cur_b) {
+            // another sequence: its fc weights into the registers, its position rows into LDS (last read before
+            // the barrier that ended the previous tile)
+            cur_b = tile_seq(tile);
+            load_fc(Wfc + cur_b * (int64_t)(K1 * D));
+            if (Wpos) posw_s[threadIdx.x] = Wpos[cur_b * 2 * D + threadIdx.x];
+            __builtin_amdgcn_s_waitcnt(0);
+            __syncthreads();
+        }
+        if (more) load_a(tile + step);
 
         // ---- y1 = x + a @ Wfc + bfc: wave w owns columns 32w .. 32w+31
         {
@@ -770,10 +807,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                 y.y = (acc[0][4 * q + 1] + acc[1][4 * q + 1]) + bq.y + xq[q].y;
                 y.z = (acc[0][4 * q + 2] + acc[1][4 * q + 2]) + bq.z + xq[q].z;
                 y.w = (acc[0][4 * q + 3] + acc[1][4 * q + 3]) + bq.w + xq[q].w;
+                if (FOLD && Wpos) {
+                    const float4 w0 = *reinterpret_cast<const float4*>(posw_s + n0 + 4 * kh + 8 * q);
+                    const float4 w1 = *reinterpret_cast<const float4*>(posw_s + D + n0 + 4 * kh + 8 * q);
+                    y.x += pq.x * w0.x + pq.y * w1.x; y.y += pq.x * w0.y + pq.y * w1.y;
+                    y.z += pq.x * w0.z + pq.y * w1.z; y.w += pq.x * w0.w + pq.y * w1.w;
+                }
                 *reinterpret_cast<float4*>(bufY + tk * PY + n0 + 8 * q + 4 * kh) = y;
             }
         }
-        if (more) load_x(tile + gridDim.x);
+        if (more) load_x(tile + step);
         __syncthreads();  // bufY complete
 
         // ---- h = act(y1 @ W1 + b1): wave w owns hidden column blocks w and w + 4, one MFMA chain each
@@ -1265,6 +1308,44 @@ extern "C" int spgt_ffn_scalar_forward(const float* x, int64_t ldx, const float*
     return check_launch("ffn_scalar_forward");
 }
 
+extern "C" int spgt_encoder_tail_folded_forward(const float* q, int64_t ld_q, const float* position, const float* x,
+                                                const float* folded_fc, const float* folded_pos,
+                                                const float* fc_bias, const float* ffn1_weight_kn,
+                                                const float* ffn1_bias, const float* ffn2_weight_kn,
+                                                const float* ffn2_bias, int activation, float* out, int B,
+                                                int64_t S, int dp, int dim_hidden, int ffn_hidden,
+                                                hipStream_t stream) {
+    if (!q || !x || !folded_fc || !fc_bias || !ffn1_weight_kn || !ffn1_bias || !ffn2_weight_kn || !ffn2_bias || !out)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "encoder_tail_folded_forward: null pointer argument");
+    if ((dp != 0 && dp != 2) || (dp == 2 && (!position || !folded_pos)))
+        return fail(SPGT_ERR_INVALID_ARGUMENT,
+                    "encoder_tail_folded_forward: dp must be 0 or 2, with positions and their folded rows for 2");
+    if (B <= 0 || S <= 0) return fail(SPGT_ERR_INVALID_ARGUMENT, "encoder_tail_folded_forward: B and S must be positive");
+    if (dim_hidden != 128 || ffn_hidden != 256)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "encoder_tail_folded_forward: needs dim_hidden 128, ffn_hidden 256");
+    if (activation != SPGT_ACT_NONE && activation != SPGT_ACT_RELU && activation != SPGT_ACT_SILU)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "encoder_tail_folded_forward: unknown activation");
+    if (ld_q < 128 || (ld_q & 3) || !aligned16(q) || !aligned16(x) || !aligned16(out) || !aligned16(fc_bias) ||
+        !aligned16(ffn1_bias) || !aligned16(ffn2_bias) || !aligned4(folded_fc) || !aligned4(ffn1_weight_kn) ||
+        !aligned4(ffn2_weight_kn) || (dp == 2 && (!aligned8(position) || !aligned4(folded_pos))))
+        return fail(SPGT_ERR_INVALID_ARGUMENT,
+                    "encoder_tail_folded_forward: activations and biases must be 16-byte aligned, ld_q a multiple of 4");
+    if (out == x || out == q) return fail(SPGT_ERR_INVALID_ARGUMENT, "encoder_tail_folded_forward: out must not alias an input");
+    const int64_t tiles = (int64_t)B * ceil_div(S, (int64_t)32);
+    if (tiles > INT32_MAX) return fail(SPGT_ERR_INVALID_ARGUMENT, "encoder_tail_folded_forward: too many tokens");
+    // as many workgroups as CUs at most, each with the same number of consecutive tiles
+    const int64_t per_wg = ceil_div(tiles, (int64_t)device_cu_count());
+    const unsigned grid = (unsigned)ceil_div(tiles, per_wg);
+    const size_t lds = std::max<size_t>(((size_t)32 * (128 + 4 + 132 + 260) + 512 + 256) * sizeof(float), 84 * 1024);
+    static const hipError_t opt = hipFuncSetAttribute(reinterpret_cast<const void*>(encoder_tail_k<128, true>),
+                                                      hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+    (void)opt;
+    hipLaunchKernelGGL((encoder_tail_k<128, true>), dim3(grid), dim3(256), lds, stream, q, ld_q, x, folded_fc, fc_bias,
+                       ffn1_weight_kn, ffn1_bias, ffn2_weight_kn, ffn2_bias, activation, out, (int64_t)B * S,
+                       dp == 2 ? folded_pos : nullptr, position, S);
+    return check_launch("encoder_tail_folded_forward");
+}
+
 extern "C" int spgt_encoder_tail_supported(int attn_features, int dim_hidden, int ffn_hidden) {
     return ((attn_features == 128 || attn_features == 136) && dim_hidden == 128 && ffn_hidden == 256) ? 1 : 0;
 }
@@ -1297,18 +1378,20 @@ extern "C" int spgt_encoder_tail_forward(const float* attn_out, int64_t ld_attn,
     const unsigned grid = (unsigned)std::min<int64_t>(ceil_div(tokens, (int64_t)32), device_cu_count());
     // attention tile + y1 + hidden tile + biases; at least half of the CU's LDS (one workgroup per CU anyway:
     // a wave uses most of its SIMD's registers)
-    const size_t lds = std::max<size_t>(((size_t)32 * ((size_t)attn_features + 4 + 132 + 260) + 512) * sizeof(float), 84 * 1024);
-    static const hipError_t opt136 = hipFuncSetAttribute(reinterpret_cast<const void*>(encoder_tail_k<136>),
+    const size_t lds = std::max<size_t>(((size_t)32 * ((size_t)attn_features + 4 + 132 + 260) + 512 + 256) * sizeof(float), 84 * 1024);
+    static const hipError_t opt136 = hipFuncSetAttribute(reinterpret_cast<const void*>(encoder_tail_k<136, false>),
                                                          hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
-    static const hipError_t opt128 = hipFuncSetAttribute(reinterpret_cast<const void*>(encoder_tail_k<128>),
+    static const hipError_t opt128 = hipFuncSetAttribute(reinterpret_cast<const void*>(encoder_tail_k<128, false>),
                                                          hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
     (void)opt136;
     (void)opt128;
     if (attn_features == 136)
-        hipLaunchKernelGGL(encoder_tail_k<136>, dim3(grid), dim3(256), lds, stream, attn_out, ld_attn, x, fc_weight_kn,
-                           fc_bias, ffn1_weight_kn, ffn1_bias, ffn2_weight_kn, ffn2_bias, activation, out, tokens);
+        hipLaunchKernelGGL((encoder_tail_k<136, false>), dim3(grid), dim3(256), lds, stream, attn_out, ld_attn, x,
+                           fc_weight_kn, fc_bias, ffn1_weight_kn, ffn1_bias, ffn2_weight_kn, ffn2_bias, activation, out,
+                           tokens, nullptr, nullptr, (int64_t)0);
     else
-        hipLaunchKernelGGL(encoder_tail_k<128>, dim3(grid), dim3(256), lds, stream, attn_out, ld_attn, x, fc_weight_kn,
-                           fc_bias, ffn1_weight_kn, ffn1_bias, ffn2_weight_kn, ffn2_bias, activation, out, tokens);
+        hipLaunchKernelGGL((encoder_tail_k<128, false>), dim3(grid), dim3(256), lds, stream, attn_out, ld_attn, x,
+                           fc_weight_kn, fc_bias, ffn1_weight_kn, ffn1_bias, ffn2_weight_kn, ffn2_bias, activation, out,
+                           tokens, nullptr, nullptr, (int64_t)0);
     return check_launch("encoder_tail_forward");
 }

@@ -247,6 +247,66 @@ def _attention_fused_forward(QKV_or_Q, K, V, position, ln_weight_K, ln_bias_K, l
     return (out, ktv) if return_ktv else out
 
 
+def _attention_ktv_forward(K, V, position, ln_weight_K, ln_bias_K, ln_weight_V, ln_bias_V, norm_eps: float,
+                           num_head: int, dim_position: int):
+    """K'^T V' / S [B, H, d, d] of the fused attention core (K/V pass and tile reduction, no pass over Q):
+    K, V [B, S, H*32] (contiguous, or equal-stride column slices of one projection output), position [B, S, dp]."""
+    H = num_head
+    for name, t in (("K", K), ("V", V)):
+        if not t.is_cuda:
+            raise _lib.SpgtError(f"{name} must live on a GPU; there is no CPU implementation")
+        if t.dtype != torch.float32:
+            raise TypeError(f"{name} must be float32")
+        if t.dim() != 3 or t.shape[-1] != H * 32 or t.stride(-1) != 1:
+            raise ValueError(f"{name} must be [B, S, {H * 32}] with unit stride on the last axis")
+    B, S, _ = K.shape
+    ld = K.stride(1)
+    for name, t in (("K", K), ("V", V)):
+        if tuple(t.shape) != (B, S, H * 32) or t.stride(1) != ld or (B > 1 and t.stride(0) != S * ld):
+            raise ValueError(f"{name}: K and V must share shape and strides [S*ld, ld, 1]")
+    for name, t in (("ln_weight_K", ln_weight_K), ("ln_bias_K", ln_bias_K), ("ln_weight_V", ln_weight_V),
+                    ("ln_bias_V", ln_bias_V)):
+        require_gpu_f32(name, t)
+        if t.numel() != H * 32:
+            raise ValueError(f"{name} must have {H * 32} elements")
+    if dim_position not in (0, 2):
+        raise ValueError("dim_position must be 0 or 2")
+    if dim_position == 2:
+        require_gpu_f32("position", position)
+        if tuple(position.shape) != (B, S, 2):
+            raise ValueError(f"position must be [{B}, {S}, 2]")
+    D = dim_position + 32
+    lib = _lib.load()
+    ktv = torch.empty((B, H, D, D), dtype=torch.float32, device=K.device)
+    ws = workspace(lib.spgt_galerkin_attention_fused_workspace_bytes(B, S, H, dim_position), K)
+    with torch.cuda.device(K.device):
+        check(lib.spgt_galerkin_attention_ktv_forward(
+            ptr(K), ptr(V), ld, ptr(position) if dim_position == 2 else None, ptr(ln_weight_K), ptr(ln_bias_K),
+            ptr(ln_weight_V), ptr(ln_bias_V), float(norm_eps), ptr(ktv), ptr(ws), ws.numel(), B, S, H, dim_position,
+            stream_of(K)))
+    return ktv
+
+
+def _fold_ktv_into_fc(ktv, fc_weight_kn, dim_position: int):
+    """(folded [B, H*32, N], folded_pos [B, dp, N] or None): M_h Wfc_h per head with the rows arranged for
+    fused_encoder_tail_folded; ktv [B, H, d, d], fc_weight_kn [H*d, N] (the transposed fc_layer weight)."""
+    require_gpu_f32("ktv", ktv)
+    require_gpu_f32("fc_weight_kn", fc_weight_kn)
+    B, H, D, D2 = ktv.shape
+    if D != D2 or D != dim_position + 32 or dim_position not in (0, 2):
+        raise ValueError("ktv must be [B, H, dp + 32, dp + 32] with dp 0 or 2")
+    if fc_weight_kn.dim() != 2 or fc_weight_kn.shape[0] != H * D:
+        raise ValueError(f"fc_weight_kn must be [{H * D}, N]")
+    N = fc_weight_kn.shape[1]
+    folded = torch.empty((B, H * 32, N), dtype=torch.float32, device=ktv.device)
+    folded_pos = torch.empty((B, dim_position, N), dtype=torch.float32, device=ktv.device) if dim_position else None
+    with torch.cuda.device(ktv.device):
+        check(_lib.load().spgt_fold_ktv_into_fc(ptr(ktv), ptr(fc_weight_kn), ptr(folded),
+                                                ptr(folded_pos) if folded_pos is not None else None, B, H,
+                                                dim_position, N, stream_of(ktv)))
+    return folded, folded_pos
+
+
 def _attention_fused_profile(Q, K, V, position, ln_weight_K, ln_bias_K, ln_weight_V, ln_bias_V, norm_eps: float,
                              num_head: int, dim_position: int, iterations: int):
     """Mean milliseconds of the three launches of the fused attention core
@@ -275,6 +335,8 @@ gexts = SimpleNamespace(
     multihead_galerkin_attention_cccr_backward=_attention_cccr_backward,
     heads_feature_to_token_major=_heads_feature_to_token_major,
     galerkin_attention_fused_profile=_attention_fused_profile,
+    galerkin_attention_ktv_forward=_attention_ktv_forward,
+    fold_ktv_into_fc=_fold_ktv_into_fc,
     multihead_galerkin_attention_cccr_forward=_attention_cccr_forward,
     batched_skinny_gemm=_batched_skinny_gemm,
     galerkin_attention_fused_forward=_attention_fused_forward,
@@ -366,6 +428,20 @@ def multihead_galerkin_attention_cccr_cuda(Q: Tensor, K: Tensor, V: Tensor) -> T
 
 def batched_skinny_gemm(A: Tensor, B: Tensor, alpha: float = 1.0) -> Tensor:
     return gexts.batched_skinny_gemm(A, B, alpha)
+
+
+def galerkin_attention_ktv(K: Tensor, V: Tensor, position, ln_weight_K: Tensor, ln_bias_K: Tensor,
+                           ln_weight_V: Tensor, ln_bias_V: Tensor, norm_eps: float, num_head: int,
+                           dim_position: int) -> Tensor:
+    """LayerNorm(K), LayerNorm(V) and K'^T V'/S [B, H, d, d] on token-major projections (inference only)."""
+    return gexts.galerkin_attention_ktv_forward(K, V, position, ln_weight_K, ln_bias_K, ln_weight_V, ln_bias_V,
+                                                norm_eps, num_head, dim_position)
+
+
+def fold_ktv_into_fc(ktv: Tensor, fc_weight_kn: Tensor, dim_position: int):
+    """The attention's last product folded into its output projection: (folded [B, H*32, N], folded_pos [B, dp, N]
+    or None) such that Q~ (K'^T V'/S) @ fc_weight_kn = q @ folded[b] + position @ folded_pos[b] (inference only)."""
+    return gexts.fold_ktv_into_fc(ktv, fc_weight_kn, dim_position)
 
 
 def galerkin_attention_fused(Q: Tensor, K: Tensor, V: Tensor, position, ln_weight_K: Tensor, ln_bias_K: Tensor,

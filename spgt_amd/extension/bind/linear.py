@@ -156,3 +156,45 @@ def fused_encoder_tail(attn_out: Tensor, x: Tensor, fc_weight_kn: Tensor, fc_bia
             ptr(ar), lda, ptr(x), ptr(fc_weight_kn), ptr(fc_bias), ptr(ffn1_weight_kn), ptr(ffn1_bias),
             ptr(ffn2_weight_kn), ptr(ffn2_bias), ACTIVATIONS[activation], ptr(out), T, K1, D, F, stream_of(x)))
     return out
+
+
+def fused_encoder_tail_folded(q: Tensor, position, x: Tensor, folded_fc: Tensor, folded_pos, fc_bias: Tensor,
+                              ffn1_weight_kn: Tensor, ffn1_bias: Tensor, ffn2_weight_kn: Tensor, ffn2_bias: Tensor,
+                              activation: str) -> Tensor:
+    """fused_encoder_tail with the attention's last product folded into the output projection (see
+    galerkin_attention.fold_ktv_into_fc): y1 = x + q @ folded_fc[b] + position @ folded_pos[b] + fc_bias, then the
+    feed-forward net.  q [B, S, 128] (the projected Q; a column slice of the packed projection is fine),
+    position [B, S, 2] or None, x [B, S, 128], folded_fc [B, 128, 128], folded_pos [B, 2, 128] or None."""
+    if activation not in ACTIVATIONS:
+        raise ValueError(f"activation must be one of {sorted(ACTIVATIONS)}")
+    for name, w in (("folded_fc", folded_fc), ("fc_bias", fc_bias), ("ffn1_weight_kn", ffn1_weight_kn),
+                    ("ffn1_bias", ffn1_bias), ("ffn2_weight_kn", ffn2_weight_kn), ("ffn2_bias", ffn2_bias), ("x", x)):
+        require_gpu_f32(name, w)
+    require_gpu_f32("q", q, contiguous=False)
+    if q.dim() != 3 or x.dim() != 3 or q.shape != x.shape or q.shape[-1] != 128:
+        raise ValueError("q and x must be [B, S, 128]")
+    B, S, D = x.shape
+    ld = q.stride(1)
+    if q.stride(2) != 1 or ld < D or ld % 4 or (B > 1 and q.stride(0) != S * ld) or q.data_ptr() % 16:
+        raise ValueError("q must have unit stride on the last axis, one row stride (a multiple of 4) and 16-byte alignment")
+    F = ffn1_weight_kn.shape[1]
+    if tuple(folded_fc.shape) != (B, D, D) or tuple(ffn1_weight_kn.shape) != (D, F) or tuple(ffn2_weight_kn.shape) != (F, D):
+        raise ValueError("folded_fc must be [B, 128, 128], the ffn weights [128, F] and [F, 128]")
+    if fc_bias.numel() != D or ffn1_bias.numel() != F or ffn2_bias.numel() != D:
+        raise ValueError("bias sizes do not match the weights")
+    dp = 0
+    if folded_pos is not None:
+        require_gpu_f32("folded_pos", folded_pos)
+        require_gpu_f32("position", position)
+        dp = 2
+        if tuple(folded_pos.shape) != (B, 2, D) or tuple(position.shape) != (B, S, 2):
+            raise ValueError("folded_pos must be [B, 2, 128] and position [B, S, 2]")
+    out = torch.empty_like(x)
+    if out.numel() == 0:
+        return out
+    with torch.cuda.device(x.device):
+        check(_lib.load().spgt_encoder_tail_folded_forward(
+            ptr(q), ld, ptr(position) if dp else None, ptr(x), ptr(folded_fc), ptr(folded_pos) if dp else None,
+            ptr(fc_bias), ptr(ffn1_weight_kn), ptr(ffn1_bias), ptr(ffn2_weight_kn), ptr(ffn2_bias),
+            ACTIVATIONS[activation], ptr(out), B, S, dp, D, F, stream_of(x)))
+    return out

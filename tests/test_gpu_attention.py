@@ -61,6 +61,45 @@ def test_fused_attention_vs_oracle(gpu, dp, B, S, H):
     assert max_rel(out.cpu().double(), want) < TOL
 
 
+@pytest.mark.parametrize("dp", [0, 2])
+@pytest.mark.parametrize("B,S,H", [(1, 1, 4), (2, 50, 4), (3, 4099, 4), (2, 1000, 8)])
+def test_attention_folded_into_projection(gpu, dp, B, S, H):
+    """K/V pass alone, and the fold of K~^T V~ / S into the output projection: the attention output times fc_layer's
+    weight (network/sp_layer.py:64-75) must equal Q times the folded weight plus the position rows' share, by
+    associativity; against the oracle in float64."""
+    C = H * 32
+    D = dp + 32
+    q, k, v = rnd(B, S, C, seed=1), rnd(B, S, C, seed=2) * 1.7 + 0.3, rnd(B, S, C, seed=3) * 0.6 - 0.2
+    pos = torch.rand(B, S, 2, generator=torch.Generator().manual_seed(4))
+    gK, bK, gV, bV = (1 + 0.3 * rnd(H, 32, seed=5)), 0.2 * rnd(H, 32, seed=6), (1 + 0.3 * rnd(H, 32, seed=7)), \
+        0.2 * rnd(H, 32, seed=8)
+    eps = 1e-6
+    want_out, want_ktv = fused_reference(q, k, v, pos, gK, bK, gV, bV, eps, H, dp)
+    d = lambda t: t.to(gpu)
+    ktv = ga.galerkin_attention_ktv(d(k), d(v), d(pos) if dp else None, d(gK), d(bK), d(gV), d(bV), eps, H, dp)
+    _, ktv_full = ga.galerkin_attention_fused(d(q), d(k), d(v), d(pos) if dp else None, d(gK), d(bK), d(gV), d(bV),
+                                              eps, H, dp, return_ktv=True)
+    assert torch.equal(ktv, ktv_full)  # the same two launches
+    assert max_rel(ktv.cpu().double(), want_ktv) < TOL
+    N = 128
+    wfc = rnd(H * D, N, seed=9) / 8
+    folded, folded_pos = ga.fold_ktv_into_fc(ktv, d(wfc), dp)
+    assert folded.shape == (B, H * 32, N) and (folded_pos is None) == (dp == 0)
+    got = torch.einsum("bsc,bcn->bsn", q.double(), folded.cpu().double())
+    if dp:
+        assert folded_pos.shape == (B, dp, N)
+        got = got + torch.einsum("bsp,bpn->bsn", pos.double(), folded_pos.cpu().double())
+    want = want_out @ wfc.double()
+    assert max_rel(got, want) < TOL
+    # the folded weight itself: M_h Wfc_h, feature rows per head and position rows summed over the heads
+    m = ktv.cpu().double()
+    w = wfc.double().view(H, D, N)
+    full = torch.einsum("bhij,hjn->bhin", m, w)
+    assert max_rel(folded.cpu().double(), full[:, :, dp:].reshape(B, H * 32, N)) < 1e-5
+    if dp:
+        assert max_rel(folded_pos.cpu().double(), full[:, :, :dp].sum(1)) < 1e-5
+
+
 def test_fused_attention_strided_qkv(gpu):
     """Q, K, V as column slices of one [B, S, 384] projection output."""
     B, S, H = 2, 333, 4

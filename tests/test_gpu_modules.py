@@ -179,6 +179,27 @@ def test_up_scaler_mixing_before_resampling(gpu, act):
     assert torch.equal(bilinear_nhwc_affine(low, (20, 20)), got)
 
 
+@pytest.mark.parametrize("dp,B,S", [(2, 3, 77), (0, 2, 200), (2, 1, 32), (2, 5, 1000)])
+def test_encoder_layer_folded_attention(gpu, dp, B, S):
+    """The attention's Q.(K^T V / S) product folded into fc_layer's weight (associativity of network/sp_layer.py:64-75)
+    against the unfolded fused layer; sequences whose length is not a multiple of the 32-token tile, and more
+    workgroups than tiles as well as fewer."""
+    torch.manual_seed(7)
+    layer = L.Sp_EncoderLayer(128, 4, dp, 1e-6, 0.0, 0.0, 0.5, 0.01, False, 256, 0.0, "silu").to(gpu).eval()
+    x = torch.randn(B, S, 128, device=gpu)
+    pos = torch.rand(B, S, max(dp, 1), device=gpu)[:, :, :dp]
+    with torch.no_grad():
+        layer.fold_attention = False
+        want = layer(x, pos)
+        layer.fold_attention = True
+        got = layer(x, pos)
+        again = layer(x, pos)
+        layer.fold_attention = None  # by size: these are short
+        assert torch.equal(layer(x, pos), want)
+    assert got.shape == want.shape and torch.equal(got, again)
+    assert rel_l2(got.cpu(), want.cpu()) < 1e-5 and max_rel(got.cpu(), want.cpu()) < 1e-4
+
+
 def test_graphed_inference_replays_match_eager(gpu):
     """A HIP-graph capture of the whole forward: every replay, with eager work and synchronisation between
     replays and with fresh inputs, reproduces the eager forward.  The convolution library picks algorithms
