@@ -179,7 +179,8 @@ def test_up_scaler_mixing_before_resampling(gpu, act):
     assert torch.equal(bilinear_nhwc_affine(low, (20, 20)), got)
 
 
-@pytest.mark.parametrize("dp,B,S", [(2, 3, 77), (0, 2, 200), (2, 1, 32), (2, 5, 1000)])
+@pytest.mark.parametrize("dp,B,S", [(2, 3, 77), (0, 2, 200), (2, 1, 32), (2, 5, 1000), (0, 8, 19881), (2, 4, 5041),
+                                     (2, 300, 33)])
 def test_encoder_layer_folded_attention(gpu, dp, B, S):
     """The attention's Q.(K^T V / S) product folded into fc_layer's weight (associativity of network/sp_layer.py:64-75)
     against the unfolded fused layer; sequences whose length is not a multiple of the 32-token tile, and more
@@ -194,8 +195,8 @@ def test_encoder_layer_folded_attention(gpu, dp, B, S):
         layer.fold_attention = True
         got = layer(x, pos)
         again = layer(x, pos)
-        layer.fold_attention = None  # by size: these are short
-        assert torch.equal(layer(x, pos), want)
+        layer.fold_attention = None  # by size
+        assert torch.equal(layer(x, pos), got if B * S >= layer.fold_attention_min_tokens else want)
     assert got.shape == want.shape and torch.equal(got, again)
     assert rel_l2(got.cpu(), want.cpu()) < 1e-5 and max_rel(got.cpu(), want.cpu()) < 1e-4
 
