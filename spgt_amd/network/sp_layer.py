@@ -148,10 +148,11 @@ class Sp_EncoderLayer(nn.Module):
     """x + attention(x); then x + ffn(x).  No normalisation on the residual stream."""
 
     # inference path: fold the attention's last product into fc_layer's weight (see folded_projection).  The fold
-    # costs a fixed 5 us per layer plus 2 us in the tail, the pass over Q it replaces 7.6 us at 20k tokens and 31 us
-    # at 159k: None folds from fold_attention_min_tokens tokens on, True / False force the choice.
+    # costs a fixed 5 us per layer plus 2 us in the tail, the pass over Q it replaces 7.6 us at 20k tokens (a whole
+    # Darcy forward measures 0.883-0.888 ms folded against 0.890-0.895 ms) and 31 us at 159k: None folds from
+    # fold_attention_min_tokens tokens on, True / False force the choice.
     fold_attention = None
-    fold_attention_min_tokens = 65536
+    fold_attention_min_tokens = 16384
 
     def __init__(self, dim_hidden, num_head, dim_position, norm_eps, attn_droprate, fc_droprate, xavier, diagonal,
                  symmetric, ffn_dim_hidden, ffn_droprate, ffn_activation) -> None:
