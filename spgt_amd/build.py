@@ -38,16 +38,48 @@ def find_hipcc() -> str:
     raise RuntimeError("hipcc not found (set HIPCC or install ROCm under /opt/rocm)")
 
 
-def build(verbose: bool = False) -> str:
-    """Compile the library from scratch and return its path."""
-    srcs = [os.path.join(CSRC_DIR, s) for s in SOURCES]
+def _newest_header_mtime() -> float:
+    hdrs = [os.path.join(CSRC_DIR, f) for f in os.listdir(CSRC_DIR) if f.endswith(".h")]
+    hdrs.append(os.path.join(PKG_DIR, "..", "include", "spgt_hip.h"))
+    return max(os.path.getmtime(h) for h in hdrs)
+
+
+def build(verbose: bool = False, incremental: bool = False, jobs: int = 8) -> str:
+    """Compile the library and return its path.  Every source is compiled to an object of its own
+    (up to `jobs` at a time) and the objects are linked.  By default everything is recompiled;
+    with `incremental` an object newer than its source and every header is kept."""
+    from concurrent.futures import ThreadPoolExecutor
+
+    hipcc = find_hipcc()
+    obj_dir = os.path.join(PKG_DIR, "build")
+    os.makedirs(obj_dir, exist_ok=True)
+    hdr_mtime = _newest_header_mtime()
+    flags = [f for f in HIPCC_FLAGS if f != "-shared"]
+
+    def clean(text):
+        # hipcc's host pass does not know the device-only feature name and says so.
+        return "\n".join(l for l in text.splitlines() if "not a recognized feature" not in l)
+
+    def compile_one(name):
+        src = os.path.join(CSRC_DIR, name)
+        obj = os.path.join(obj_dir, name + ".o")
+        if incremental and os.path.exists(obj) and os.path.getmtime(obj) > max(os.path.getmtime(src), hdr_mtime):
+            return obj, ""
+        cmd = [hipcc, *flags, "-x", "hip", "-c", src, "-o", obj]
+        proc = subprocess.run(cmd, cwd=CSRC_DIR, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+        if proc.returncode != 0:
+            raise RuntimeError("hipcc failed:\n" + " ".join(cmd) + "\n" + clean(proc.stdout))
+        return obj, clean(proc.stdout)
+
+    with ThreadPoolExecutor(max_workers=max(1, jobs)) as pool:
+        results = list(pool.map(compile_one, SOURCES))
+    objs = [o for o, _ in results]
+    log = "\n".join(t for _, t in results if t.strip())
     tmp = LIB_PATH + ".tmp"
-    cmd = [find_hipcc(), *HIPCC_FLAGS, "-x", "hip", *srcs, "-o", tmp]
+    cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", tmp]
     proc = subprocess.run(cmd, cwd=CSRC_DIR, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    # hipcc's host pass does not know the device-only feature name and says so.
-    log = "\n".join(l for l in proc.stdout.splitlines() if "not a recognized feature" not in l)
     if proc.returncode != 0:
-        raise RuntimeError("hipcc failed:\n" + " ".join(cmd) + "\n" + log)
+        raise RuntimeError("link failed:\n" + " ".join(cmd) + "\n" + clean(proc.stdout))
     if verbose and log.strip():
         print(log)
     os.replace(tmp, LIB_PATH)
@@ -55,5 +87,5 @@ def build(verbose: bool = False) -> str:
 
 
 if __name__ == "__main__":
-    print(build(verbose=True))
+    print(build(verbose=True, incremental="--incremental" in sys.argv))
     sys.exit(0)
