@@ -115,6 +115,24 @@ int spgt_galerkin_attention_fused_forward(const float* Q, const float* K, const 
                                           size_t workspace_bytes, int B, int S, int H, int dp,
                                           spgt_stream_t stream);
 
+/* spgt_galerkin_attention_fused_forward for callers that cannot allocate device memory or hand in
+ * a workspace (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).
+ * It has no counterpart in the reference.  The partial tiles of the K/V pass go to a device array
+ * of spgt_galerkin_attention_fused_static_max_bytes() bytes (16 MiB) that is part of the library's
+ * code object: every GPU the library runs on holds one copy until the process ends.  The call
+ * allocates and frees nothing; a shape whose spgt_galerkin_attention_fused_workspace_bytes exceeds
+ * the array is rejected with SPGT_ERR_WORKSPACE (B=8, S=44521, H=4 needs 12.6 MB).  All calls on
+ * one GPU share that GPU's array: calls that overlap in time on one GPU (two streams, two threads)
+ * race and must be serialised by the caller.  Arguments and results otherwise as
+ * spgt_galerkin_attention_fused_forward (Q and out are required). */
+size_t spgt_galerkin_attention_fused_static_max_bytes(void);
+int spgt_galerkin_attention_fused_forward_static(const float* Q, const float* K, const float* V,
+                                                 int64_t ld_in, const float* position,
+                                                 const float* ln_weight_K, const float* ln_bias_K,
+                                                 const float* ln_weight_V, const float* ln_bias_V,
+                                                 float norm_eps, float* out, float* ktv, int B, int S,
+                                                 int H, int dp, spgt_stream_t stream);
+
 /* ---- backward of the attention operators ------------------------------------ */
 
 /* Replaces multihead_galerkin_attention_cccr_backward (extension/bind/galerkin_attention.cu:126-173).

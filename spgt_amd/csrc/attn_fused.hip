@@ -22,6 +22,14 @@
 #include "spgt_host.h"
 #include "spgt_kernels.h"
 
+#include <atomic>
+
+// Size of the device array behind spgt_galerkin_attention_fused_forward_static (16 MiB: the headline shape
+// B=8, S=44521, H=4 needs 12.6 MB of partial tiles).
+#ifndef SPGT_STATIC_SCRATCH_BYTES
+#define SPGT_STATIC_SCRATCH_BYTES (16u << 20)
+#endif
+
 // Cache policy of the three touch-once streams (K/V reads, Q reads, out
 // writes).  Measured on MI355X at B=8, S=44521 over all eight combinations:
 // non-temporal K/V loads and out stores with plain Q loads is the fastest
@@ -650,6 +658,72 @@ extern "C" int spgt_galerkin_attention_fused_forward(
     size_t workspace_bytes, int B, int S, int H, int dp, hipStream_t stream) {
     return fused_forward_impl(Q, K, V, ld_in, position, ln_weight_K, ln_bias_K, ln_weight_V, ln_bias_V, norm_eps,
                               out, ktv, workspace, workspace_bytes, B, S, H, dp, stream, nullptr);
+}
+
+// ---------------------------------------------------------------------------
+// allocation-free variant: the partial tiles live in a device array of the library
+// ---------------------------------------------------------------------------
+
+namespace spgt {
+namespace {
+
+constexpr size_t kStaticScratchBytes = SPGT_STATIC_SCRATCH_BYTES;
+
+// One copy per GPU the library's code object is loaded on, held until the process ends.
+static __device__ __align__(256) float scratch[kStaticScratchBytes / sizeof(float)];
+
+constexpr int kMaxDevices = 64;
+std::atomic<float*> g_scratch_ptr[kMaxDevices];
+
+// Device address of `scratch` on the current device (looked up once per device), or null with the
+// error recorded.  The array's name is only a host-side handle for this lookup; every launch and
+// copy uses the pointer returned here.
+float* static_scratch_ptr() {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        (void)fail(SPGT_ERR_LAUNCH, "galerkin_attention_fused_static: no current device");
+        return nullptr;
+    }
+    float* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (ptr) return ptr;
+    void* sym = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&sym, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !sym) {
+        (void)fail(SPGT_ERR_LAUNCH, "galerkin_attention_fused_static: hipGetSymbolAddress(scratch) failed");
+        return nullptr;
+    }
+    ptr = static_cast<float*>(sym);
+    g_scratch_ptr[dev].store(ptr, std::memory_order_release);
+    return ptr;
+}
+
+}  // namespace
+}  // namespace spgt
+
+extern "C" size_t spgt_galerkin_attention_fused_static_max_bytes(void) { return kStaticScratchBytes; }
+
+extern "C" int spgt_galerkin_attention_fused_forward_static(
+    const float* Q, const float* K, const float* V, int64_t ld_in, const float* position,
+    const float* ln_weight_K, const float* ln_bias_K, const float* ln_weight_V,
+    const float* ln_bias_V, float norm_eps, float* out, float* ktv, int B, int S, int H, int dp,
+    hipStream_t stream) {
+    if (!Q || !out)  // the K/V-only form of the shared implementation is not offered here
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "galerkin_attention_fused_static: null pointer argument");
+    const size_t need = spgt_galerkin_attention_fused_workspace_bytes(B, S, H, dp);
+    if (need == 0)
+        return fail(SPGT_ERR_INVALID_ARGUMENT,
+                    "galerkin_attention_fused_static: B, S, H must be positive and dim_position 0 or 2");
+    if (need > kStaticScratchBytes)
+        return fail(SPGT_ERR_WORKSPACE,
+                    "galerkin_attention_fused_static: shape needs more partial-tile scratch than the library's "
+                    "static array holds (spgt_galerkin_attention_fused_static_max_bytes); use "
+                    "spgt_galerkin_attention_fused_forward with a caller workspace");
+    float* ws = static_scratch_ptr();
+    if (!ws) return SPGT_ERR_LAUNCH;
+    // Every partial tile the reduction reads is written by the K/V pass of the same call, so nothing
+    // in the array has to start at zero.
+    return fused_forward_impl(Q, K, V, ld_in, position, ln_weight_K, ln_bias_K, ln_weight_V, ln_bias_V, norm_eps,
+                              out, ktv, ws, kStaticScratchBytes, B, S, H, dp, stream, nullptr);
 }
 
 extern "C" int spgt_galerkin_attention_ktv_forward(
