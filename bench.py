@@ -62,6 +62,12 @@ def cpu_baseline(B, S, H, seed, budget_s=20.0):
     }
 
 
+def max_rel_elementwise(got, want, floor=1e-3):
+    """max |got - want| / |want| over the entries with |want| > floor * max|want|."""
+    keep = want.abs() > floor * want.abs().max()
+    return float(((got - want).abs()[keep] / want.abs()[keep]).max().item())
+
+
 def darcy_inputs(B, r, r_attn, seed):
     """Synthetic Darcy batch: a = 12 where a Gaussian random field with covariance (-Laplace + 9 I)^-2
     is >= 0 and 3 elsewhere (the reference's dataset/darcy_generate recipe: alpha 2, tau 3, cosine
@@ -138,10 +144,11 @@ def darcy_bench(dev, with_cpu, steps=30):
         ms = (time.perf_counter() - t0) / steps * 1e3
         graph_equal = bool(torch.equal(gout, out))
     graph_ms = ms
-    ms = min(graph_ms, eager_ms)
-    res = {"ms_per_forward": round(ms, 3), "samples_per_s": round(B / ms * 1e3, 1), "batch": B,
-           "mode": "faster of eager launches and HIP graph replay (input copy included)",
+    res = {"ms_per_forward": round(eager_ms, 3), "samples_per_s": round(B / eager_ms * 1e3, 1), "batch": B,
+           "mode": "eager launches (model(x, position, grid) as a user calls it); the HIP graph replay of the same "
+                   "forward, input copy included, is reported separately",
            "eager_ms_per_forward": round(eager_ms, 3), "graph_ms_per_forward": round(graph_ms, 3),
+           "graph_samples_per_s": round(B / graph_ms * 1e3, 1),
            "graph_output_equals_eager": graph_equal,
            "config": "r=211 -> 122 -> 71, 4 encoder layers (d_model 128, 4 heads, dp 2, FFN 256), "
                      "2 FNO blocks (width 64, 12 modes), random init, drop rates 0"}
@@ -160,6 +167,7 @@ def darcy_bench(dev, with_cpu, steps=30):
         res["cpu_oracle_samples_per_s"] = round(B / cpu_ms * 1e3, 2)
         res["cpu_cores"] = torch.get_num_threads()
         res["rel_l2_vs_cpu_oracle"] = float(((out.cpu() - want).norm() / want.norm()).item())
+        res["max_rel_elementwise_vs_cpu_oracle"] = max_rel_elementwise(out.cpu(), want)
     return res
 
 
@@ -230,7 +238,8 @@ def encoder_stack_bench(dev, with_cpu):
             cpu_ms = _cpu_ms(cpu_fwd)
             want = cpu_fwd()
         res.update(cpu_oracle_ms_per_forward=round(cpu_ms, 1), cpu_cores=torch.get_num_threads(),
-                   rel_l2_vs_cpu_oracle=float(((out.cpu() - want).norm() / want.norm()).item()))
+                   rel_l2_vs_cpu_oracle=float(((out.cpu() - want).norm() / want.norm()).item()),
+                   max_rel_elementwise_vs_cpu_oracle=max_rel_elementwise(out.cpu(), want))
     return res
 
 
@@ -276,7 +285,8 @@ def fno_stack_bench(dev, with_cpu):
             cpu_ms = _cpu_ms(cpu_fwd)
             want = cpu_fwd()
         res.update(cpu_oracle_ms_per_forward=round(cpu_ms, 1), cpu_cores=torch.get_num_threads(),
-                   rel_l2_vs_cpu_oracle=float(((out.cpu() - want).norm() / want.norm()).item()))
+                   rel_l2_vs_cpu_oracle=float(((out.cpu() - want).norm() / want.norm()).item()),
+                   max_rel_elementwise_vs_cpu_oracle=max_rel_elementwise(out.cpu(), want))
     return res
 
 
@@ -435,6 +445,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--input-sets", type=int, default=3,
+                    help="independent (Q, K, V) sets the timed steps rotate through")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -454,32 +466,55 @@ def main():
 
     B, S, H, dp = 8, 44521, 4, 0
     g = torch.Generator(device=dev).manual_seed(0)
-    q, k, v = (torch.randn(B, S, H * 32, device=dev, generator=g) for _ in range(3))
+    # Independent (Q, K, V) sets visited in turn: one set is 547 MB, so when a set comes round again
+    # 1.6 GB of other inputs and outputs have passed through the 256 MB last-level cache.
+    n_sets = max(1, args.input_sets)
+    sets = [tuple(torch.randn(B, S, H * 32, device=dev, generator=g) for _ in range(3)) for _ in range(n_sets)]
     one, zero = torch.ones(H, 32, device=dev), torch.zeros(H, 32, device=dev)
-    step = lambda: ga.galerkin_attention_fused(q, k, v, None, one, zero, one, zero, 1e-6, H, dp)
+    step = lambda i: ga.galerkin_attention_fused(*sets[i % n_sets], None, one, zero, one, zero, 1e-6, H, dp)
     nbytes = 4 * B * H * 32 * S * 4
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    ms_per_step = elapsed / args.steps * 1e3
-    value = nbytes / (elapsed / args.steps) / 1e9
+    def wall_ms(fn):
+        for i in range(args.warmup):
+            fn(i)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(args.steps):
+            fn(i)
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / args.steps * 1e3
 
-    # dominant kernel: the K/V pass, HIP events around its launch on the launch stream
-    stage_ms = ga.gexts.galerkin_attention_fused_profile(q, k, v, None, one, zero, one, zero, 1e-6, H, dp, 30)
+    ms_per_step = wall_ms(step)  # the timed region: exactly `steps` calls, inputs rotated
+    value = nbytes / (ms_per_step * 1e-3) / 1e9
+    same_ms = wall_ms(lambda i: step(0))  # every step on one input set (Q fits the last-level cache)
+
+    # per-call and per-launch durations of the same rotated sequence: HIP events on the launch stream
+    # around every launch, calls back to back, one synchronisation at the end
+    n_prof = max(30, min(args.steps, 400))
+    ga.gexts.galerkin_attention_fused_profile(sets, None, one, zero, one, zero, 1e-6, H, dp, 10)
+    stages = ga.gexts.galerkin_attention_fused_profile(sets, None, one, zero, one, zero, 1e-6, H, dp, n_prof)
+
+    def dist(vals):
+        vs = sorted(vals)
+        pick = lambda f: vs[min(len(vs) - 1, int(f * len(vs)))]
+        return {"median": round(pick(0.5) * 1e3, 2), "p10": round(pick(0.1) * 1e3, 2), "p90": round(pick(0.9) * 1e3, 2)}
+
+    kv = dist([st[0] for st in stages])
     kv_bytes = 2 * B * H * 32 * S * 4  # K and V read once; partial tiles are not counted
-    achieved = kv_bytes / (stage_ms[0] * 1e-3) / 1e9
+    achieved = kv_bytes / (kv["median"] * 1e-6) / 1e9
+    q_bytes = 2 * B * H * 32 * S * 4
+    qd = dist([st[2] for st in stages])
     roofline = {
         "bound": "hbm", "kernel": "ktv_ln_partial_tm<0,4>", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
         "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": recorded_kv_pass_traffic(),
-        "kernel_us": round(stage_ms[0] * 1e3, 2), "algorithmic_bytes": kv_bytes,
-        "stages_us": {"kv_pass": round(stage_ms[0] * 1e3, 2), "tile_reduce": round(stage_ms[1] * 1e3, 2),
-                      "q_pass": round(stage_ms[2] * 1e3, 2)},
+        "traffic_source": "recorded: rocprofv3 FETCH_SIZE + WRITE_SIZE summary under profiles/ for this kernel and "
+                          "shape (counters need runs of their own), not a reading of this run",
+        "kernel_us": kv["median"], "kernel_us_p10_p90": [kv["p10"], kv["p90"]], "algorithmic_bytes": kv_bytes,
+        "timing": f"HIP events around each launch, {n_prof} calls back to back over {n_sets} rotated input sets, "
+                  "median",
+        "stages_us": {"kv_pass": kv, "tile_reduce": dist([st[1] for st in stages]), "q_pass": qd,
+                      "call": dist([sum(st) for st in stages])},
+        "q_pass_GBps": round(q_bytes / (qd["median"] * 1e-6) / 1e9, 1),
     }
 
     extra = {}
@@ -504,6 +539,18 @@ def main():
             torch.cuda.synchronize()
             return e0.elapsed_time(e1) / n
 
+        # what this part copies at: torch's elementwise copy of the Q pass's bytes (182 MB read, 182 MB written),
+        # sources and destinations rotated like the benchmark's inputs
+        dsts = [torch.empty_like(sets[0][0]) for _ in range(2)]
+        cnt = [0]
+
+        def plain_copy():
+            cnt[0] += 1
+            dsts[cnt[0] % 2].copy_(sets[cnt[0] % n_sets][cnt[0] % 3])
+
+        ms = timed(plain_copy)
+        extra["plain_copy_182MB_rotated"] = {"ms": round(ms, 4), "GB/s": round(q_bytes / ms / 1e6, 1)}
+        del dsts
         Qf, Kf, Vf = (torch.randn(B, H, 32, S, device=dev, generator=g) for _ in range(3))
         ms = timed(lambda: ga.multihead_galerkin_attention_cccr_cuda(Qf, Kf, Vf))
         extra["attention_cccr_d32"] = {"ms": round(ms, 4), "GB/s": round(nbytes / ms / 1e6, 1)}
@@ -528,7 +575,10 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "fused Galerkin attention core (LayerNorm K,V + K^T V/S + Q(K^T V/S)), "
                                "B=8 S=44521 d_model=128 heads=4 dp=0, token-major projections resident in HBM",
-                   "algorithmic_bytes_per_step": nbytes, "hbm_frac_of_8TBps": round(value / HBM_PEAK_GBPS, 4)},
+                   "algorithmic_bytes_per_step": nbytes, "hbm_frac_of_8TBps": round(value / HBM_PEAK_GBPS, 4),
+                   "input_sets_rotated": n_sets,
+                   "ms_per_step_one_input_set": round(same_ms, 4),
+                   "GBps_one_input_set": round(nbytes / same_ms / 1e6, 1)},
         "roofline": roofline,
         "cpu_baseline": None if args.no_cpu_baseline else cpu_baseline(B, S, H, 0),
         "extra": extra,

@@ -23,6 +23,7 @@
 #include "spgt_kernels.h"
 
 #include <atomic>
+#include <vector>
 
 // Size of the device array behind spgt_galerkin_attention_fused_forward_static (16 MiB: the headline shape
 // B=8, S=44521, H=4 needs 12.6 MB of partial tiles).
@@ -31,19 +32,20 @@
 #endif
 
 // Cache policy of the three touch-once streams (K/V reads, Q reads, out
-// writes).  Measured on MI355X at B=8, S=44521 over all eight combinations:
-// non-temporal K/V loads and out stores with plain Q loads is the fastest
-// (146 us per call against 174 us with plain accesses everywhere); the
-// non-temporal out stores keep 182 MB of dirty lines from draining under the
-// next call's K/V pass.
+// writes).  Measured on MI355X at B=8, S=44521 over all eight combinations,
+// with consecutive calls on different inputs (so that no call finds its Q in
+// the 256 MB last-level cache): non-temporal K/V and Q loads with plain out
+// stores is the fastest (147 us per call; non-temporal stores as well 154 us;
+// plain Q loads with non-temporal stores 151 us; everything plain 171 us,
+// because the K/V pass then runs at 102 us instead of 67 us).
 #ifndef SPGT_NT_P1LD
 #define SPGT_NT_P1LD true
 #endif
 #ifndef SPGT_NT_P2LD
-#define SPGT_NT_P2LD false
+#define SPGT_NT_P2LD true
 #endif
 #ifndef SPGT_NT_P2ST
-#define SPGT_NT_P2ST true
+#define SPGT_NT_P2ST false
 #endif
 
 namespace spgt {
@@ -590,12 +592,14 @@ extern "C" size_t spgt_galerkin_attention_fused_workspace_bytes(int B, int S, in
 namespace {
 
 // Validates, then enqueues the three launches.  With `ev` (4 events) an event
-// is recorded before the first launch and after each launch.
+// is recorded before the first launch (unless record_first is false: the caller
+// has recorded it already) and after each launch.
 int fused_forward_impl(
     const float* Q, const float* K, const float* V, int64_t ld_in, const float* position,
     const float* ln_weight_K, const float* ln_bias_K, const float* ln_weight_V,
     const float* ln_bias_V, float norm_eps, float* out, float* ktv, void* workspace,
-    size_t workspace_bytes, int B, int S, int H, int dp, hipStream_t stream, hipEvent_t* ev) {
+    size_t workspace_bytes, int B, int S, int H, int dp, hipStream_t stream, hipEvent_t* ev,
+    bool record_first = true) {
     const bool apply = Q != nullptr || out != nullptr;  // neither: K/V pass and reduction only
     if ((apply && (!Q || !out)) || !K || !V || !ktv || !ln_weight_K || !ln_bias_K || !ln_weight_V || !ln_bias_V)
         return fail(SPGT_ERR_INVALID_ARGUMENT, "galerkin_attention_fused: null pointer argument");
@@ -628,7 +632,7 @@ int fused_forward_impl(
     const dim3 gridr(ceil_div(D * D, 256), B * H);
     const dim3 blockr(1024);
     const float* pos = position ? position : K;  // never dereferenced when dp == 0
-    if (ev) (void)hipEventRecord(ev[0], stream);
+    if (ev && record_first) (void)hipEventRecord(ev[0], stream);
     if (dp == 0) {
         hipLaunchKernelGGL((ktv_ln_partial_tm<0, kU1>), grid1, block, 0, stream, K, V, pos, ln_weight_K,
                            ln_bias_K, ln_weight_V, ln_bias_V, norm_eps, partial, S, H, ld_in, p.tpc1);
@@ -829,37 +833,39 @@ extern "C" int spgt_fold_ktv_into_fc(const float* ktv, const float* fc_weight_kn
 }
 
 extern "C" int spgt_galerkin_attention_fused_profile(
-    const float* Q, const float* K, const float* V, int64_t ld_in, const float* position,
-    const float* ln_weight_K, const float* ln_bias_K, const float* ln_weight_V,
-    const float* ln_bias_V, float norm_eps, float* out, float* ktv, void* workspace,
-    size_t workspace_bytes, int B, int S, int H, int dp, hipStream_t stream, int iterations,
-    float* stage_ms) {
-    if (iterations <= 0 || !stage_ms)
-        return fail(SPGT_ERR_INVALID_ARGUMENT, "galerkin_attention_fused_profile: iterations and stage_ms required");
-    hipEvent_t ev[4];
-    for (int i = 0; i < 4; ++i)
+    const float* const* Q_sets, const float* const* K_sets, const float* const* V_sets, int n_sets, int64_t ld_in,
+    const float* position, const float* ln_weight_K, const float* ln_bias_K, const float* ln_weight_V,
+    const float* ln_bias_V, float norm_eps, float* out, float* ktv, void* workspace, size_t workspace_bytes, int B,
+    int S, int H, int dp, hipStream_t stream, int iterations, float* stage_ms) {
+    if (iterations <= 0 || iterations > 4096 || !stage_ms || n_sets <= 0 || !Q_sets || !K_sets || !V_sets)
+        return fail(SPGT_ERR_INVALID_ARGUMENT,
+                    "galerkin_attention_fused_profile: 1..4096 iterations, stage_ms and at least one input set required");
+    // event 3 i + k: before launch k of iteration i; the last event closes the last launch
+    const int nev = 3 * iterations + 1;
+    std::vector<hipEvent_t> ev(nev);
+    for (int i = 0; i < nev; ++i)
         if (hipEventCreate(&ev[i]) != hipSuccess) {
             for (int j = 0; j < i; ++j) (void)hipEventDestroy(ev[j]);
             return fail(SPGT_ERR_LAUNCH, "galerkin_attention_fused_profile: hipEventCreate failed");
         }
-    double acc[3] = {0.0, 0.0, 0.0};
     int rc = SPGT_OK;
     for (int it = 0; it < iterations && rc == SPGT_OK; ++it) {
-        rc = fused_forward_impl(Q, K, V, ld_in, position, ln_weight_K, ln_bias_K, ln_weight_V, ln_bias_V,
-                                norm_eps, out, ktv, workspace, workspace_bytes, B, S, H, dp, stream, ev);
-        if (rc != SPGT_OK) break;
-        if (hipEventSynchronize(ev[3]) != hipSuccess) {
-            rc = fail(SPGT_ERR_LAUNCH, "galerkin_attention_fused_profile: hipEventSynchronize failed");
-            break;
-        }
-        for (int k = 0; k < 3; ++k) {
-            float ms = 0.f;
-            (void)hipEventElapsedTime(&ms, ev[k], ev[k + 1]);
-            acc[k] += ms;
-        }
+        const int s = it % n_sets;
+        hipEvent_t four[4] = {ev[3 * it], ev[3 * it + 1], ev[3 * it + 2], ev[3 * it + 3]};
+        // the closing event of one iteration is the opening event of the next: it is recorded once, by the
+        // iteration it closes, and iteration 0 records its own opening event
+        rc = fused_forward_impl(Q_sets[s], K_sets[s], V_sets[s], ld_in, position, ln_weight_K, ln_bias_K, ln_weight_V,
+                                ln_bias_V, norm_eps, out, ktv, workspace, workspace_bytes, B, S, H, dp, stream, four,
+                                it == 0);
     }
-    for (int i = 0; i < 4; ++i) (void)hipEventDestroy(ev[i]);
+    if (rc == SPGT_OK && hipEventSynchronize(ev[nev - 1]) != hipSuccess)
+        rc = fail(SPGT_ERR_LAUNCH, "galerkin_attention_fused_profile: hipEventSynchronize failed");
     if (rc == SPGT_OK)
-        for (int k = 0; k < 3; ++k) stage_ms[k] = (float)(acc[k] / iterations);
+        for (int i = 0; i < 3 * iterations; ++i) {
+            float ms = 0.f;
+            (void)hipEventElapsedTime(&ms, ev[i], ev[i + 1]);
+            stage_ms[i] = ms;
+        }
+    for (int i = 0; i < nev; ++i) (void)hipEventDestroy(ev[i]);
     return rc;
 }

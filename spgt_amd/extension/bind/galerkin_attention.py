@@ -307,24 +307,33 @@ def _fold_ktv_into_fc(ktv, fc_weight_kn, dim_position: int):
     return folded, folded_pos
 
 
-def _attention_fused_profile(Q, K, V, position, ln_weight_K, ln_bias_K, ln_weight_V, ln_bias_V, norm_eps: float,
+def _attention_fused_profile(input_sets, position, ln_weight_K, ln_bias_K, ln_weight_V, ln_bias_V, norm_eps: float,
                              num_head: int, dim_position: int, iterations: int):
-    """Mean milliseconds of the three launches of the fused attention core
-    (K/V pass, tile reduction, Q pass), measured with HIP events on the current stream."""
+    """Per-iteration milliseconds [iterations][3] of the three launches of the fused attention core (K/V pass,
+    tile reduction, Q pass) over `iterations` back-to-back calls, iteration i on input_sets[i % len(input_sets)]
+    (a list of (Q, K, V) triples of one shape), measured with HIP events on the current stream."""
     import ctypes
-    B, S, _ = Q.shape
+    Q0 = input_sets[0][0]
+    B, S, _ = Q0.shape
     H, D = num_head, dim_position + 32
+    for trip in input_sets:
+        for t in trip:
+            require_gpu_f32("profile input", t)
+            if t.shape != Q0.shape:
+                raise ValueError("all profile inputs must share one shape")
     lib = _lib.load()
-    out = torch.empty((B, S, H * D), dtype=torch.float32, device=Q.device)
-    ktv = torch.empty((B, H, D, D), dtype=torch.float32, device=Q.device)
-    ws = workspace(lib.spgt_galerkin_attention_fused_workspace_bytes(B, S, H, dim_position), Q)
-    stage = (ctypes.c_float * 3)()
-    with torch.cuda.device(Q.device):
+    out = torch.empty((B, S, H * D), dtype=torch.float32, device=Q0.device)
+    ktv = torch.empty((B, H, D, D), dtype=torch.float32, device=Q0.device)
+    ws = workspace(lib.spgt_galerkin_attention_fused_workspace_bytes(B, S, H, dim_position), Q0)
+    n = len(input_sets)
+    arrs = [(ctypes.c_void_p * n)(*[trip[j].data_ptr() for trip in input_sets]) for j in range(3)]
+    stage = (ctypes.c_float * (3 * int(iterations)))()
+    with torch.cuda.device(Q0.device):
         check(lib.spgt_galerkin_attention_fused_profile(
-            ptr(Q), ptr(K), ptr(V), Q.stride(1), ptr(position) if dim_position == 2 else None, ptr(ln_weight_K),
-            ptr(ln_bias_K), ptr(ln_weight_V), ptr(ln_bias_V), float(norm_eps), ptr(out), ptr(ktv), ptr(ws),
-            ws.numel(), B, S, H, dim_position, stream_of(Q), int(iterations), stage))
-    return [float(x) for x in stage]
+            arrs[0], arrs[1], arrs[2], n, Q0.stride(1), ptr(position) if dim_position == 2 else None,
+            ptr(ln_weight_K), ptr(ln_bias_K), ptr(ln_weight_V), ptr(ln_bias_V), float(norm_eps), ptr(out), ptr(ktv),
+            ptr(ws), ws.numel(), B, S, H, dim_position, stream_of(Q0), int(iterations), stage))
+    return [[float(stage[3 * i + k]) for k in range(3)] for i in range(int(iterations))]
 
 
 gexts = SimpleNamespace(

@@ -38,6 +38,12 @@ def max_rel(a, b):
     return ((a - b).abs().max() / b.abs().max().clamp_min(1e-30)).item()
 
 
+def max_rel_elementwise(a, b, floor=1e-3):
+    """max |a-b| / |b| over the entries with |b| > floor * max|b|."""
+    keep = b.abs() > floor * b.abs().max()
+    return ((a - b).abs()[keep] / b.abs()[keep]).max().item()
+
+
 def rel_l2(a, b):
     return ((a - b).norm() / b.norm().clamp_min(1e-30)).item()
 
