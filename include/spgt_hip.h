@@ -439,6 +439,23 @@ int spgt_encoder_tail_folded_forward(const float* q, int64_t ld_q, const float* 
                                      float* out, int B, int64_t S, int dp, int dim_hidden, int ffn_hidden,
                                      spgt_stream_t stream);
 
+/* One strided copy: dst[i0*dst_stride[0] + i1*dst_stride[1] + i2*dst_stride[2]] =
+ * src[i0*src_stride[0] + i1*src_stride[1] + i2*src_stride[2]] for i_k < size[k]; 32-bit words, strides in words. */
+typedef struct {
+    const float* src;
+    float* dst;
+    int32_t size[3];
+    int32_t src_stride[3];
+    int32_t dst_stride[3];
+} spgt_copy_desc;
+
+/* Runs `count` strided copies (descs: host array) in ceil(count / 64) launches.  No counterpart in the
+ * reference, whose kernels read nn.Parameter layouts directly: the kernels here take some operands in
+ * derived layouts (nn.Linear weights transposed to [in, out], [W_Q | W_K | W_V] packed, a 3x3 convolution's
+ * weight as nine [Cin, Cout] taps), and the modules refresh all of them from the parameters with this call
+ * at the start of a forward, so that a parameter changed in place by any means is never served stale. */
+int spgt_strided_copy_batch(const spgt_copy_desc* descs, int count, spgt_stream_t stream);
+
 /* Instrumented variant of spgt_galerkin_attention_fused_forward for benchmarks (no reference
  * counterpart): enqueues the call `iterations` times back to back (no synchronisation between
  * them, as a caller's loop would), iteration i reading the input set i % n_sets (Q_sets, K_sets,

@@ -76,10 +76,19 @@ SIGNATURES = {
     "spgt_fold_ktv_into_fc": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _p]),
     "spgt_encoder_tail_folded_forward": (
         _i, [_p, _i64, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _p, _i, _i64, _i, _i, _i, _p]),
+    "spgt_strided_copy_batch": (_i, [_p, _i, _p]),
     "spgt_galerkin_attention_fused_profile": (
         _i, [_p, _p, _p, _i, _i64, _p, _p, _p, _p, _p, _f, _p, _p, _p, _sz, _i, _i, _i, _i, _p, _i,
              ctypes.POINTER(ctypes.c_float)]),
 }
+
+
+
+class CopyDesc(ctypes.Structure):
+    """spgt_copy_desc of include/spgt_hip.h."""
+    _fields_ = [("src", ctypes.c_void_p), ("dst", ctypes.c_void_p), ("size", ctypes.c_int32 * 3),
+                ("src_stride", ctypes.c_int32 * 3), ("dst_stride", ctypes.c_int32 * 3)]
+
 
 _lock = threading.Lock()
 _lib = None

@@ -113,6 +113,29 @@ __global__ __launch_bounds__(256) void transpose_scatter_dual_k(const uint64_t* 
     }
 }
 
+// One launch that refreshes many small derived tensors: block (x, y) copies elements of descriptor y.
+// Elements are walked in dst order (axis 2 fastest), so writes coalesce; reads follow the source strides
+// (a transposed weight is read column-wise out of the caches: these are kilobytes).
+struct CopyBatch {
+    spgt_copy_desc d[64];
+};
+
+__global__ __launch_bounds__(256) void strided_copy_batch_k(const CopyBatch batch) {
+    const spgt_copy_desc& d = batch.d[blockIdx.y];
+    const int n1 = d.size[1], n2 = d.size[2];
+    const int total = d.size[0] * n1 * n2;
+    const uint32_t* __restrict__ src = reinterpret_cast<const uint32_t*>(d.src);
+    uint32_t* __restrict__ dst = reinterpret_cast<uint32_t*>(d.dst);
+    for (int e = blockIdx.x * 256 + threadIdx.x; e < total; e += gridDim.x * 256) {
+        const int i2 = e % n2;
+        const int r = e / n2;
+        const int i1 = r % n1;
+        const int i0 = r / n1;
+        dst[(int64_t)i0 * d.dst_stride[0] + (int64_t)i1 * d.dst_stride[1] + (int64_t)i2 * d.dst_stride[2]] =
+            src[(int64_t)i0 * d.src_stride[0] + (int64_t)i1 * d.src_stride[1] + (int64_t)i2 * d.src_stride[2]];
+    }
+}
+
 namespace {
 
 int check_windows(const char* who, int dim, int H_all, int W_all, int H_low, int W_low, int hb1, int wb1, int hb2,
@@ -182,4 +205,35 @@ extern "C" int spgt_transpose_scatter_dual(const float* src1, const float* src2,
                        reinterpret_cast<const uint64_t*>(src1), reinterpret_cast<const uint64_t*>(src2),
                        reinterpret_cast<uint64_t*>(out), dim, H_all, W_all, H_low, W_low, win);
     return check_launch("transpose_scatter_dual");
+}
+
+extern "C" int spgt_strided_copy_batch(const spgt_copy_desc* descs, int count, hipStream_t stream) {
+    if (count < 0 || (count > 0 && !descs))
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "strided_copy_batch: descriptor array missing");
+    for (int i = 0; i < count; ++i) {
+        const spgt_copy_desc& d = descs[i];
+        if (!d.src || !d.dst || !aligned4(d.src) || !aligned4(d.dst))
+            return fail(SPGT_ERR_INVALID_ARGUMENT, "strided_copy_batch: null or misaligned pointer in a descriptor");
+        int64_t total = 1;
+        for (int a = 0; a < 3; ++a) {
+            if (d.size[a] <= 0 || d.src_stride[a] < 0 || d.dst_stride[a] < 0)
+                return fail(SPGT_ERR_INVALID_ARGUMENT, "strided_copy_batch: sizes must be positive, strides non-negative");
+            total *= d.size[a];
+        }
+        if (total > (int64_t)1 << 30)
+            return fail(SPGT_ERR_INVALID_ARGUMENT, "strided_copy_batch: a descriptor exceeds 2^30 elements");
+    }
+    for (int first = 0; first < count; first += 64) {
+        const int n = std::min(64, count - first);
+        CopyBatch batch;
+        int64_t largest = 0;
+        for (int i = 0; i < n; ++i) {
+            batch.d[i] = descs[first + i];
+            largest = std::max<int64_t>(largest, (int64_t)batch.d[i].size[0] * batch.d[i].size[1] * batch.d[i].size[2]);
+        }
+        for (int i = n; i < 64; ++i) batch.d[i] = batch.d[0];
+        const int bx = (int)std::min<int64_t>(64, ceil_div(largest, (int64_t)1024));
+        hipLaunchKernelGGL(strided_copy_batch_k, dim3(bx, n), dim3(256), 0, stream, batch);
+    }
+    return check_launch("strided_copy_batch");
 }

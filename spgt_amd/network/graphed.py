@@ -16,8 +16,11 @@ class GraphedInference:
     """`g = GraphedInference(model, *example_inputs)`; `g(*inputs)` copies the inputs into the captured
     buffers, replays the graph and returns the captured output tensor(s), which the next call overwrites.
 
-    Inputs must keep the example's shapes and dtypes.  The module's parameters are read in place at every
-    replay, so in-place weight updates are seen; replacing a parameter tensor needs a new capture."""
+    Inputs must keep the example's shapes and dtypes.  Every replay reads the module's parameters where they
+    were at capture: kernels that take a parameter as stored read it in place, and the launch that rewrites the
+    derived layouts (transposed and packed weights, see derived.py) is part of the graph.  In-place updates
+    (optimizer steps, `copy_`, writes through `.data`, `load_state_dict`) are therefore seen by the next replay;
+    a parameter that moves to new storage (`.to()`, `load_state_dict(assign=True)`) needs a new capture."""
 
     def __init__(self, module: nn.Module, *example_inputs: Tensor, warmup: int = 3) -> None:
         if not example_inputs or not all(isinstance(x, Tensor) and x.is_cuda for x in example_inputs):

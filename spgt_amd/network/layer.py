@@ -13,6 +13,7 @@ from torch import Tensor, nn
 
 from ..extension.bind.datamove import bias_activation_nchw_
 from ..extension.bind.linear import ffn_scalar_supported, fused_ffn_scalar, fused_linear, linear_supported
+from .derived import derived, refreshes_derived, transposed_2d
 
 
 def make_activation(name: str) -> nn.Module:
@@ -24,14 +25,9 @@ def activation_name(module: nn.Module) -> str:
 
 
 def linear_weight_kn(lin: nn.Linear) -> Tensor:
-    """lin.weight transposed to [in_features, out_features], contiguous; rebuilt when the parameter changes."""
-    w = lin.weight
-    key = (w.data_ptr(), w._version, w.device)
-    cache = getattr(lin, "_spgt_weight_kn", None)
-    if cache is None or cache[0] != key:
-        cache = (key, w.detach().t().contiguous())
-        lin._spgt_weight_kn = cache
-    return cache[1]
+    """lin.weight transposed to [in_features, out_features], contiguous: a derived tensor, rewritten from the
+    parameter at the start of every inference forward (see derived.py)."""
+    return derived(lin, "weight_kn", lambda: transposed_2d(lin.weight))
 
 
 def gpu_inference(X: Tensor, *params: Tensor) -> bool:
@@ -91,6 +87,7 @@ class FeedForward(nn.Module):
         self.layer2 = nn.Linear(dim_hidden, out_dim)
         self.activation_layer = make_activation(activation)
 
+    @refreshes_derived
     def forward(self, X: Tensor, residual: Tensor = None) -> Tensor:
         """ffn(X), or residual + ffn(X) when a residual is given."""
         if (self.layer2.out_features == 1 and residual is None and

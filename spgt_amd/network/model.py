@@ -11,6 +11,7 @@ from ..extension.bind.datamove import (bilinear_align_corners, bilinear_align_co
                                        bilinear_resample, bilinear_resample_concat, conv3x3_resample,
                                        conv3x3_resample_supported, upsample_conv3x3_gather)
 from ..extension.bind.linear import fused_linear, linear_supported
+from .derived import derived, refreshes_derived
 from .layer import ConvResBlock2D, activation_name, always_dropout, gpu_inference, make_activation
 
 
@@ -103,14 +104,14 @@ class UpScaler2D(nn.Module):
 
     def _tap_weight_kn(self) -> Tensor:
         """The convolution's weight as [Cin, 9 * Cout], column (3 ky + kx) * Cout + co: the nine per-tap 1x1
-        products as one GEMM operand; rebuilt when the parameter changes."""
+        products as one GEMM operand; a derived tensor, rewritten from the parameter at the start of every
+        inference forward."""
         w = self.conv.conv_layer.weight
-        key = (w.data_ptr(), w._version, w.device)
-        cache = getattr(self, "_spgt_tap_weight", None)
-        if cache is None or cache[0] != key:
-            cache = (key, w.detach().permute(1, 2, 3, 0).reshape(w.size(1), 9 * w.size(0)).contiguous())
-            self._spgt_tap_weight = cache
-        return cache[1]
+        if w.stride(2) != 3 * w.stride(3):  # the nine taps are walked as one axis
+            return w.detach().permute(1, 2, 3, 0).reshape(w.size(1), 9 * w.size(0)).contiguous()
+        cout, cin = w.size(0), w.size(1)
+        return derived(self, "tap_weight_kn", lambda: (
+            (cin, 9 * cout), [(w, 0, (cin, 9, cout), (w.stride(1), w.stride(3), w.stride(0)), 0, (9 * cout, cout, 1))]))
 
     def _mixes_before_resampling(self, X: Tensor) -> bool:
         """True when interpolate -> conv3x3 -> activations is computed as GEMM at the low resolution + gather:
@@ -133,6 +134,7 @@ class UpScaler2D(nn.Module):
         return upsample_conv3x3_gather(Z.view(N, H, W, 9, c.out_channels), c.bias, self.resolution_size[3],
                                        activation_name(self.activation_layer), 2)
 
+    @refreshes_derived
     def forward(self, X: Tensor, defer_last_resample: bool = False) -> Tensor:
         """With defer_last_resample (see can_defer_last_resample) the result is the channels-last tensor at
         resolution_size[3], [N, r_mid, r_mid, out_dim], and the caller owes the interpolation to resolution_size[4]:

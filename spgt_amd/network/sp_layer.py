@@ -33,6 +33,7 @@ from ..extension.bind.galerkin_attention import (fold_ktv_into_fc, galerkin_atte
 from . import truncated_dft
 from ..extension.bind.linear import (encoder_tail_supported, fused_encoder_tail, fused_encoder_tail_folded,
                                      fused_linear)
+from .derived import derived, refreshes_derived
 from .layer import (FeedForward, activation_name, always_dropout, fused_linear_usable, gpu_inference,
                     linear_weight_kn, make_activation)
 
@@ -58,7 +59,6 @@ class Sp_GalerkinAttention(nn.Module):
                 setattr(self, f"ln_{kind}_{n}", nn.Parameter(torch.empty(num_head, self.dim_head)))
         self.fc_layer = nn.Linear(dim_hidden + dim_position * num_head, dim_hidden)
         self._reset_parameters(xavier, diagonal, symmetric)
-        self._qkv_cache = None
 
     def _reset_parameters(self, xavier, diagonal, symmetric) -> None:
         with torch.no_grad():
@@ -74,18 +74,26 @@ class Sp_GalerkinAttention(nn.Module):
                 g.fill_(1.0)
 
     def _packed_qkv(self):
-        """[W_Q | W_K | W_V] (dim_hidden x 3 dim_hidden) and the packed bias, rebuilt when a parameter changes."""
-        ps = (self.weight_Q, self.weight_K, self.weight_V, self.bias_Q, self.bias_K, self.bias_V)
-        key = tuple((p.data_ptr(), p._version) for p in ps)
-        if self._qkv_cache is None or self._qkv_cache[0] != key:
-            with torch.no_grad():
-                self._qkv_cache = (key, torch.cat(ps[:3], dim=1).contiguous(), torch.cat(ps[3:]).contiguous())
-        return self._qkv_cache[1], self._qkv_cache[2]
+        """[W_Q | W_K | W_V] (dim_hidden x 3 dim_hidden) and the packed bias: derived tensors, rewritten from the
+        six parameters at the start of every inference forward."""
+        C = self.dim_hidden
+
+        def weight_spec():
+            ws = (self.weight_Q, self.weight_K, self.weight_V)
+            return (C, 3 * C), [(w, 0, (1, C, C), (0, w.stride(0), w.stride(1)), j * C, (0, 3 * C, 1))
+                                for j, w in enumerate(ws)]
+
+        def bias_spec():
+            bs = (self.bias_Q, self.bias_K, self.bias_V)
+            return (3 * C,), [(b, 0, (1, 1, C), (0, 0, b.stride(0)), j * C, (0, 0, 1)) for j, b in enumerate(bs)]
+
+        return derived(self, "qkv_weight", weight_spec), derived(self, "qkv_bias", bias_spec)
 
     def _needs_graph(self, *tensors) -> bool:
         return torch.is_grad_enabled() and (any(t.requires_grad for t in tensors) or
                                             any(p.requires_grad for p in self.parameters()))
 
+    @refreshes_derived
     def forward(self, Q: Tensor, K: Tensor, V: Tensor, position: Tensor, residual: Tensor = None) -> Tensor:
         """Q, K, V [N, seqlen, dim_hidden], position [N, seqlen, dim_position] -> [N, seqlen, dim_hidden];
         with `residual` the result is residual + attention(Q, K, V)."""
@@ -161,6 +169,7 @@ class Sp_EncoderLayer(nn.Module):
                                                     fc_droprate, xavier, diagonal, symmetric)
         self.ffn_layer = FeedForward(dim_hidden, dim_hidden, ffn_dim_hidden, ffn_droprate, ffn_activation)
 
+    @refreshes_derived
     def forward(self, X: Tensor, position: Tensor) -> Tensor:
         att, ffn = self.attention_layer, self.ffn_layer
         if (att.fc_droprate == 0 and ffn.droprate == 0 and gpu_inference(X, *self.parameters()) and
@@ -199,6 +208,7 @@ class Sp_SpectralConv2D(nn.Module):
         for w in self.fourier_weight:
             nn.init.xavier_normal_(w, gain=1.0 / (in_dim * out_dim) * math.sqrt(in_dim + out_dim))
 
+    @refreshes_derived
     def forward(self, X: Tensor) -> Tensor:
         """[N, r, r, in_dim] -> [N, r, r, out_dim]."""
         N, r, _, cin = X.size()

@@ -10,6 +10,7 @@ from torch import Tensor, nn
 
 from ..extension.bind.datamove import bilinear_nhwc_affine, denormalize_boundary
 from ..extension.bind.linear import fused_linear, linear_supported
+from .derived import derived, refreshes_derived, transposed_2d
 from .layer import FeedForward, always_dropout, gpu_inference
 from .model import DownScaler2D, UpScaler2D
 from .sp_layer import Sp_EncoderLayer, Sp_SpectralConv2D
@@ -36,6 +37,7 @@ class Sp_EncoderMixer(nn.Module):
             Sp_EncoderLayer(dim_hidden, num_head, dim_position, norm_eps, attn_droprate, fc_droprate, xavier, diagonal,
                             symmetric, ffn_dim_hidden, ffn_droprate, ffn_activation) for _ in range(num_layer)])
 
+    @refreshes_derived
     def forward(self, X: Tensor, position: Tensor) -> Tensor:
         """X [N, ra, ra, dim_hidden], position [N, ra, ra, dim_position] -> [N, ra, ra, dim_hidden]."""
         N, ra, _, C = X.size()
@@ -59,15 +61,10 @@ class Sp_DecoderRegressor(nn.Module):
 
     def _split_weight_kn(self, dim_x: int):
         """spatial_fc_layer.weight as ([dim_x, C], [dim_position, C]): the hidden-feature and the grid columns,
-        transposed; rebuilt when the parameter changes."""
+        transposed; derived tensors, rewritten from the parameter at the start of every inference forward."""
         w = self.spatial_fc_layer.weight
-        key = (w.data_ptr(), w._version, w.device, dim_x)
-        cache = getattr(self, "_spgt_weight_split", None)
-        if cache is None or cache[0] != key:
-            wd = w.detach()
-            cache = (key, wd[:, :dim_x].t().contiguous(), wd[:, dim_x:].t().contiguous())
-            self._spgt_weight_split = cache
-        return cache[1], cache[2]
+        return (derived(self, f"fc_hidden_kn_{dim_x}", lambda: transposed_2d(w, slice(0, dim_x))),
+                derived(self, f"fc_grid_kn_{dim_x}", lambda: transposed_2d(w, slice(dim_x, w.size(1)))))
 
     def accepts_low_resolution(self, X: Tensor, grid: Tensor) -> bool:
         """True when forward(X, grid, resample_to=size) is available for a channels-last X."""
@@ -76,6 +73,7 @@ class Sp_DecoderRegressor(nn.Module):
                 gpu_inference(X, grid, W, self.spatial_fc_layer.bias) and linear_supported(dim_x, W.size(0)) and
                 W.size(0) % 4 == 0 and 0 < W.size(1) - dim_x <= 4 and grid.size(-1) == W.size(1) - dim_x)
 
+    @refreshes_derived
     def forward(self, X: Tensor, grid: Tensor = None, resample_to=None) -> Tensor:
         """X [N, r, r, dim_hidden], grid [N, r, r, dim_position] -> [N, r, r, dim_target].
         With resample_to = (r, r) (see accepts_low_resolution), X is [N, r_low, r_low, dim_hidden] and stands for
@@ -119,6 +117,7 @@ class Sp_GalerkinTransformer2D(nn.Module):
             cfg["num_decoder_layer"], cfg["dim_hidden"], cfg["dim_target"], cfg["dim_position"],
             cfg["dim_spatial_hidden"], cfg["num_frequence_mode"], cfg["drop_decoder_layer"], cfg["acti_decoder_layer"])
 
+    @refreshes_derived
     def forward(self, X: Tensor, position: Tensor, grid: Tensor) -> Tensor:
         """X [N, r, r, dim_node], position [N, ra, ra, dim_position], grid [N, r, r, dim_position]
         -> [N, r, r, dim_target] (de-normalised; zero on the boundary for the Dirichlet condition)."""

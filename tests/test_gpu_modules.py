@@ -223,3 +223,99 @@ def test_graphed_inference_replays_match_eager(gpu):
         _ = (torch.randn(257, 513, device=gpu) @ torch.randn(513, 129, device=gpu)).sum().item()  # eager work between replays
     with pytest.raises(ValueError):
         g(x[:1], pos, grid)
+
+
+def test_parameters_changed_through_data_are_seen(gpu):
+    """Writes through `.data` leave a parameter's version counter alone; the derived layouts the fused kernels read
+    (transposed Linear weights, packed [W_Q | W_K | W_V], convolution taps, the split decoder input weight) must
+    follow them all the same: forward, scale parameters in place, forward, compare with the oracle on the new values."""
+    p, i, _, meta = load_golden("galerkin_transformer_2d")
+    m = load_into(SM.Sp_GalerkinTransformer2D(model_cfg(meta)), p, gpu)
+    x, pos, grid = i["x"].to(gpu), i["position"].to(gpu), i["grid"].to(gpu)
+    cfg = dict(meta)
+    cfg["resolution_size"] = meta["resolution_size"].tolist()
+
+    def oracle_now():
+        sd = {k: v.detach().cpu() for k, v in m.state_dict().items()}
+        po = {k: (v.t() if k.rsplit(".", 1)[-1] in ("weight_Q", "weight_K", "weight_V") else v) for k, v in sd.items()}
+        return O.galerkin_transformer_2d(po, cfg, i["x"], i["position"], i["grid"], weight_layout="sp")
+
+    with torch.no_grad():
+        first = m(x, pos, grid)
+    assert rel_l2(first.cpu(), oracle_now()) < TOL
+    changed = 0
+    for name, prm in m.named_parameters():
+        leaf = name.rsplit(".", 1)[-1]
+        if leaf in ("weight_Q", "weight_V", "bias_K") or "fc_layer.weight" in name or "layer1.weight" in name or \
+                "layer2.weight" in name or "up_scaler.conv.conv_layer.weight" in name or \
+                "residual_layer.weight" in name:
+            before = prm._version
+            prm.data.mul_(1.5)
+            prm.data.add_(0.01)
+            assert prm._version == before  # nothing on the host records the write
+            changed += 1
+    assert changed >= 10
+    with torch.no_grad():
+        second = m(x, pos, grid)
+    want = oracle_now()
+    assert rel_l2(first.cpu(), want) > 1e-2  # the update matters
+    assert rel_l2(second.cpu(), want) < TOL
+
+
+def test_standalone_layers_follow_data_updates(gpu):
+    """The same for layers used on their own, where no enclosing forward refreshes the derived layouts."""
+    torch.manual_seed(5)
+    layer = L.Sp_EncoderLayer(128, 4, 2, 1e-6, 0.0, 0.0, 0.5, 0.01, False, 256, 0.0, "silu").to(gpu).eval()
+    x, pos = torch.randn(2, 300, 128, device=gpu), torch.rand(2, 300, 2, device=gpu)
+
+    def oracle_now():
+        sd = {k: v.detach().cpu().double() for k, v in layer.state_dict().items()}
+        po = {k: (v.t() if k.rsplit(".", 1)[-1] in ("weight_Q", "weight_K", "weight_V") else v) for k, v in sd.items()}
+        return O.encoder_layer(po, x.cpu().double(), pos.cpu().double(), 4, 1e-6, "silu")
+
+    for fold in (False, True):
+        layer.fold_attention = fold
+        with torch.no_grad():
+            assert max_rel(layer(x, pos).cpu().double(), oracle_now()) < TOL
+            layer.attention_layer.weight_K.data.mul_(-0.7)
+            layer.attention_layer.fc_layer.weight.data.mul_(1.3)
+            layer.ffn_layer.layer2.weight.data.add_(0.02)
+            assert max_rel(layer(x, pos).cpu().double(), oracle_now()) < TOL
+            # pieces called outside any forward refresh their own operands
+            att = layer.attention_layer
+            att.weight_Q.data.mul_(2.0)
+            core = att.attend(x, x, x, pos)
+            got = att.project(core, residual=x)
+            sd = {k: v.detach().cpu().double() for k, v in att.state_dict().items()}
+            po = {k: (v.t() if k in ("weight_Q", "weight_K", "weight_V") else v) for k, v in sd.items()}
+            want = x.cpu().double() + O.attention_module(po, x.cpu().double(), x.cpu().double(), x.cpu().double(),
+                                                         pos.cpu().double(), 4, 1e-6)
+            assert max_rel(got.cpu().double(), want) < TOL
+
+
+def test_graphed_inference_follows_in_place_weight_updates(gpu):
+    """A captured forward re-reads the parameters: after in-place updates (through the autograd-visible `copy_`
+    and through `.data`), replays match eager forwards of the updated model."""
+    from spgt_amd.network.graphed import GraphedInference
+    p, i, _, meta = load_golden("galerkin_transformer_2d")
+    m = load_into(SM.Sp_GalerkinTransformer2D(model_cfg(meta)), p, gpu)
+    x, pos, grid = i["x"].to(gpu), i["position"].to(gpu), i["grid"].to(gpu)
+    g = GraphedInference(m, x, pos, grid)
+    with torch.no_grad():
+        before = m(x, pos, grid).clone()
+    torch.cuda.synchronize()
+    assert rel_l2(g(x, pos, grid).cpu(), before.cpu()) < TOL
+    for step in range(2):
+        with torch.no_grad():
+            for name, prm in m.named_parameters():
+                if prm.dim() >= 2 and ("encoder_mixer" in name or "decoder_regressor" in name or "up_scaler" in name):
+                    if step == 0:
+                        prm.data.mul_(1.2)
+                    else:
+                        prm.copy_(prm * 0.9 + 0.003)
+            want = m(x, pos, grid).clone()
+        torch.cuda.synchronize()
+        got = g(x, pos, grid).clone()
+        torch.cuda.synchronize()
+        assert rel_l2(want.cpu(), before.cpu()) > 1e-2
+        assert rel_l2(got.cpu(), want.cpu()) < TOL, f"replay after update {step} used stale weights"
