@@ -297,17 +297,39 @@ def kernel_rooflines(dev):
     from spgt_amd.extension.bind import datamove as dm
     from spgt_amd.extension.bind import galerkin_attention as ga
 
-    def timed(fn, n=30, warm=3):
+    def timed(fn, n=20, warm=3, replays=5):
+        """Seconds per call: `n` calls captured into a HIP graph and replayed, so that short kernels are timed
+        on the GPU's clock and not on the host's launch rate (eager launches if the capture fails)."""
         for _ in range(warm):
             fn()
         torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(n):
-            fn()
-        e1.record()
-        torch.cuda.synchronize()
-        return e0.elapsed_time(e1) / n * 1e-3  # seconds
+        try:
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                fn()
+            torch.cuda.current_stream().wait_stream(side)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                for _ in range(n):
+                    fn()
+            graph.replay()
+            torch.cuda.synchronize()
+            e0.record()
+            for _ in range(replays):
+                graph.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) / (n * replays) * 1e-3
+        except RuntimeError:
+            torch.cuda.synchronize()
+            e0.record()
+            for _ in range(n):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) / n * 1e-3  # seconds
 
     rows = {}
 

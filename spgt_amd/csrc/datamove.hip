@@ -10,33 +10,62 @@
 #include "spgt_device.h"
 #include "spgt_host.h"
 
+// complex elements a zero-fill block writes, roughly (tuned on MI355X)
+#ifndef SPGT_ZERO_CHUNK
+#define SPGT_ZERO_CHUNK 2048
+#endif
+
 namespace spgt {
 
+typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+typedef u4 u4_a4 __attribute__((aligned(4)));  // rows of odd length start at any 4-byte offset
+
 // [batch, M, N] -> [batch, N, M], 32-bit words.  grid (tiles_n, tiles_m, batch), block 256.
-// A 64x64 tile goes through LDS (pitch 65: conflict-free both ways); global
-// reads and writes are 256-byte runs per wave.
+// A 64x64 tile goes through LDS (pitch 65: conflict-free both ways).  Both global sides move 16 bytes per
+// lane: a wave reads four 256-byte row pieces per instruction and writes four; tile edges fall back to words.
 __global__ __launch_bounds__(256) void batched_transpose_64(const uint32_t* __restrict__ src,
                                                             uint32_t* __restrict__ dst, int M, int N) {
     __shared__ uint32_t tile[64 * 65];
-    const int tx = threadIdx.x & 63;
-    const int ty = threadIdx.x >> 6;
+    const int q = threadIdx.x & 15;  // group of four columns
+    const int r = threadIdx.x >> 4;  // row within a pass of 16 rows
     const int n0 = blockIdx.x * 64;
     const int m0 = blockIdx.y * 64;
     const int64_t base = (int64_t)blockIdx.z * M * N;
     const uint32_t* s = src + base;
     uint32_t* d = dst + base;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-        const int m = m0 + 4 * i + ty;
-        const int n = n0 + tx;
-        if (m < M && n < N) tile[(4 * i + ty) * 65 + tx] = s[(int64_t)m * N + n];
+    for (int i = 0; i < 4; ++i) {
+        const int mr = r + 16 * i;
+        const int m = m0 + mr;
+        const int n = n0 + 4 * q;
+        if (m < M) {
+            uint32_t* t = tile + mr * 65 + 4 * q;
+            const uint32_t* g = s + (int64_t)m * N + n;
+            if (n + 3 < N) {
+                const u4 v = *reinterpret_cast<const u4_a4*>(g);
+                t[0] = v.x; t[1] = v.y; t[2] = v.z; t[3] = v.w;
+            } else {
+                for (int j = 0; j < 4 && n + j < N; ++j) t[j] = g[j];
+            }
+        }
     }
     __syncthreads();
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-        const int n = n0 + 4 * i + ty;
-        const int m = m0 + tx;
-        if (m < M && n < N) d[(int64_t)n * M + m] = tile[tx * 65 + 4 * i + ty];
+    for (int i = 0; i < 4; ++i) {
+        const int nr = r + 16 * i;
+        const int n = n0 + nr;
+        const int m = m0 + 4 * q;
+        if (n < N) {
+            const uint32_t* t = tile + (4 * q) * 65 + nr;
+            uint32_t* g = d + (int64_t)n * M + m;
+            if (m + 3 < M) {
+                u4 v;
+                v.x = t[0]; v.y = t[65]; v.z = t[130]; v.w = t[195];
+                *reinterpret_cast<u4_a4*>(g) = v;
+            } else {
+                for (int j = 0; j < 4 && m + j < M; ++j) g[j] = t[65 * j];
+            }
+        }
     }
 }
 
@@ -76,40 +105,66 @@ __global__ __launch_bounds__(256) void transpose_gather_dual_k(const uint64_t* _
 // out [dim, H_all, W_all] (64-bit words): zero everywhere except the two windows,
 // which receive src_k [H_low, W_low, dim] transposed.  Where the windows overlap the
 // second one wins (the reference scatters window 1, then window 2).
-// grid (ceil(dim/64), H_all), block 256: a block writes row h of 64 planes.
+// Blocks [0, nA): (group of 64 planes, window row slot): the block that owns an output row h inside a window
+// writes that row of its planes: window elements through an LDS transposition, zeros elsewhere.  Blocks
+// [nA, ...): zero fill of the rows outside both windows, contiguous spans of a plane with 16-byte stores.
 __global__ __launch_bounds__(256) void transpose_scatter_dual_k(const uint64_t* __restrict__ src1,
                                                                 const uint64_t* __restrict__ src2,
                                                                 uint64_t* __restrict__ out, int dim, int H_all,
-                                                                int W_all, int H_low, int W_low, Windows win) {
+                                                                int W_all, int H_low, int W_low, Windows win,
+                                                                SpecSpans spans, int nA, int chunks_per_plane) {
     extern __shared__ uint64_t stile[];  // [2][W_low][65]
-    const int d0 = blockIdx.x * 64;
-    const int h = blockIdx.y;
+    const int64_t plane = (int64_t)H_all * W_all;
+    if ((int)blockIdx.x >= nA) {
+        const int bz = blockIdx.x - nA;
+        const int64_t p = bz / chunks_per_plane;
+        zero_span_chunk(reinterpret_cast<float2*>(out), spans, p, bz - (int)p * chunks_per_plane, chunks_per_plane,
+                        plane, W_all);
+        return;
+    }
+    const int groups = ceil_div(dim, 64);
+    const int d0 = ((int)blockIdx.x % groups) * 64;
+    const int slot = (int)blockIdx.x / groups;
+    const int k0 = slot / H_low;
+    const int h = win.h_base[k0] + (slot - k0 * H_low);
     bool in_win[2];
+    in_win[0] = h >= win.h_base[0] && h < win.h_base[0] + H_low;
+    in_win[1] = h >= win.h_base[1] && h < win.h_base[1] + H_low;
+    if (k0 == 1 && in_win[0]) return;  // the first window's block owns a row that lies in both
 #pragma unroll
     for (int k = 0; k < 2; ++k) {
-        in_win[k] = h >= win.h_base[k] && h < win.h_base[k] + H_low;
         if (in_win[k]) {
             const uint64_t* s = (k == 0 ? src1 : src2) + (int64_t)(h - win.h_base[k]) * W_low * dim;
             uint64_t* t = stile + k * W_low * 65;
-            for (int e = threadIdx.x; e < 64 * W_low; e += 256) {
-                const int dd = e & 63;
-                const int w = e >> 6;
-                if (d0 + dd < dim) t[w * 65 + dd] = s[(int64_t)w * dim + d0 + dd];
+            // four loads per thread in flight at a time (a plain loop would wait for each before the next)
+            const int dd = threadIdx.x & 63;
+            const int ddc = min(d0 + dd, dim - 1);
+            for (int w0 = threadIdx.x >> 6; w0 < W_low; w0 += 16) {
+                uint64_t v[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) v[u] = s[(int64_t)min(w0 + 4 * u, W_low - 1) * dim + ddc];
+#pragma unroll
+                for (int u = 0; u < 4; ++u)
+                    if (w0 + 4 * u < W_low) t[(w0 + 4 * u) * 65 + dd] = v[u];
             }
         }
     }
     __syncthreads();
-    const int64_t plane = (int64_t)H_all * W_all;
-    for (int e = threadIdx.x; e < 64 * W_all; e += 256) {
-        const int w = e % W_all;
-        const int dd = e / W_all;
-        if (d0 + dd >= dim) continue;
-        uint64_t v = 0;
-        if (in_win[1] && w >= win.w_base[1] && w < win.w_base[1] + W_low)
-            v = stile[(W_low + w - win.w_base[1]) * 65 + dd];
-        else if (in_win[0] && w >= win.w_base[0] && w < win.w_base[0] + W_low)
-            v = stile[(w - win.w_base[0]) * 65 + dd];
-        out[(int64_t)(d0 + dd) * plane + (int64_t)h * W_all + w] = v;
+    // wave v writes row h of planes d0 + 16 v .. d0 + 16 v + 15, lanes along w
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    for (int qq = 0; qq < 16; ++qq) {
+        const int dd = wave * 16 + qq;
+        if (d0 + dd >= dim) break;
+        uint64_t* orow = out + (int64_t)(d0 + dd) * plane + (int64_t)h * W_all;
+        for (int w = lane; w < W_all; w += 64) {
+            uint64_t v = 0;
+            if (in_win[1] && w >= win.w_base[1] && w < win.w_base[1] + W_low)
+                v = stile[(W_low + w - win.w_base[1]) * 65 + dd];
+            else if (in_win[0] && w >= win.w_base[0] && w < win.w_base[0] + W_low)
+                v = stile[(w - win.w_base[0]) * 65 + dd];
+            orow[w] = v;
+        }
     }
 }
 
@@ -200,10 +255,18 @@ extern "C" int spgt_transpose_scatter_dual(const float* src1, const float* src2,
     if (!aligned8(src1) || !aligned8(src2) || !aligned8(out))
         return fail(SPGT_ERR_INVALID_ARGUMENT, "transpose_scatter_dual: complex operands must be 8-byte aligned");
     Windows win{{H_base_1, H_base_2}, {W_base_1, W_base_2}};
-    const dim3 grid(ceil_div(dim, 64), H_all);
-    hipLaunchKernelGGL(transpose_scatter_dual_k, grid, dim3(256), (size_t)W_low * 65 * 8 * 2, stream,
+    const SpecSpans spans = rows_outside_windows(H_all, H_low, H_base_1, H_base_2);
+    int64_t zero_rows = 0;
+    for (int i = 0; i < spans.n; ++i) zero_rows += spans.hi[i] - spans.lo[i];
+    const int chunks = zero_rows == 0 ? 0 : (int)std::max<int64_t>(1, std::min<int64_t>(8, zero_rows * W_all / SPGT_ZERO_CHUNK));
+    const int64_t nA = (int64_t)ceil_div(dim, 64) * 2 * H_low;
+    const int64_t nB = (int64_t)dim * chunks;
+    if (nA + nB >= ((int64_t)1 << 31))
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "transpose_scatter_dual: too many planes for one launch");
+    hipLaunchKernelGGL(transpose_scatter_dual_k, dim3((unsigned)(nA + nB)), dim3(256), (size_t)W_low * 65 * 8 * 2, stream,
                        reinterpret_cast<const uint64_t*>(src1), reinterpret_cast<const uint64_t*>(src2),
-                       reinterpret_cast<uint64_t*>(out), dim, H_all, W_all, H_low, W_low, win);
+                       reinterpret_cast<uint64_t*>(out), dim, H_all, W_all, H_low, W_low, win, spans, (int)nA,
+                       std::max(1, chunks));
     return check_launch("transpose_scatter_dual");
 }
 

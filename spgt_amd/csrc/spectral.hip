@@ -11,6 +11,17 @@
 #include "spgt_device.h"
 #include "spgt_host.h"
 
+// complex elements a zero-fill block writes, roughly (tuned on MI355X)
+#ifndef SPGT_ROWS_NB
+#define SPGT_ROWS_NB 4
+#endif
+#ifndef SPGT_ROWS_WU
+#define SPGT_ROWS_WU 8
+#endif
+#ifndef SPGT_ZERO_CHUNK
+#define SPGT_ZERO_CHUNK 2048
+#endif
+
 namespace spgt {
 
 struct SpecWindows {
@@ -112,6 +123,153 @@ __global__ __launch_bounds__(256) void spectrum_zero_outside_k(float2* __restric
         const bool in0 = h >= win.h_base[0] && h < win.h_base[0] + m_h && w >= win.w_base[0] && w < win.w_base[0] + m_w;
         const bool in1 = h >= win.h_base[1] && h < win.h_base[1] + m_h && w >= win.w_base[1] && w < win.w_base[1] + m_w;
         if (!in0 && !in1) out[e] = make_float2(0.f, 0.f);
+    }
+}
+
+// The full-spectrum form in ONE launch: contraction, scatter into the output spectrum and zero fill.
+// Blocks [0, nA) each own JW window columns of one output row h that lies in a window, for NB batch entries and
+// 64 output planes.  Thread (o, q) multiplies the input channels i = q, q+4, ...: its weights for a step of 32
+// channels are loaded once (JW * 8 loads in flight, 512-byte coalesced rows) and meet the rows of all NB batch
+// entries, which wait in LDS; the four partial sums per output are added in LDS in a fixed order.  Blocks
+// [nA, ...) zero everything else: the rows that lie in no window as contiguous spans of a plane with 16-byte
+// stores, and the window rows' columns outside the windows.  Where the windows overlap the second one wins
+// (the reference scatters it last).
+constexpr int kRowsNB = SPGT_ROWS_NB;
+constexpr int kRowsWU = SPGT_ROWS_WU;  // input channels per thread and step (all blocks of the launch share its register budget)
+
+template <int JW>
+__global__ __launch_bounds__(256) void spectral_contract_rows_k(
+    const float2* __restrict__ X, const float2* __restrict__ W0, const float2* __restrict__ W1,
+    float2* __restrict__ out, int N, int Cin, int Cout, int H_all, int W_all, int m_h, int m_w, SpecWindows win,
+    SpecSpans spans, int nA, int chunks_per_plane) {
+    extern __shared__ float2 xrow[];  // [kRowsNB][Cin][JW] inputs, then [4 entries][4][JW][64] partial sums
+    const int64_t plane = (int64_t)H_all * W_all;
+    if ((int)blockIdx.x >= nA) {
+        // chunks_per_plane blocks per plane for the rows outside the windows, one more for the window rows' rest
+        const int bz = blockIdx.x - nA;
+        const int64_t p = bz / (chunks_per_plane + 1);
+        const int c = bz - (int)p * (chunks_per_plane + 1);
+        if (c < chunks_per_plane)
+            zero_span_chunk(out, spans, p, c, chunks_per_plane, plane, W_all);
+        else
+            zero_window_row_remainders(out, p, plane, W_all, m_h, m_w, win.h_base[0], win.w_base[0], win.h_base[1],
+                                       win.w_base[1]);
+        return;
+    }
+    const int og_count = ceil_div(Cout, 64);
+    const int wq_count = ceil_div(m_w, JW);
+    int a = blockIdx.x;
+    const int wq = a % wq_count;
+    a /= wq_count;
+    const int og = a % og_count;
+    a /= og_count;
+    const int slot = a % (2 * m_h);
+    const int n0 = (a / (2 * m_h)) * kRowsNB;
+    const int nb = min(kRowsNB, N - n0);
+    const int k0 = slot / m_h;
+    const int h = win.h_base[k0] + (slot - k0 * m_h);
+    const bool in0 = h >= win.h_base[0] && h < win.h_base[0] + m_h;
+    const bool in1 = h >= win.h_base[1] && h < win.h_base[1] + m_h;
+    if (k0 == 1 && in0) return;  // the first window's block owns a row that lies in both
+    const bool ink[2] = {in0, in1};
+    const int ww0 = wq * JW;
+    const int ol = threadIdx.x & 63;
+    const int o = og * 64 + ol;
+    const int q = threadIdx.x >> 6;
+    const int oc = min(o, Cout - 1);
+    float2* red = xrow + kRowsNB * Cin * JW;  // [4][4][JW][64]
+    for (int k = 0; k < 2; ++k) {
+        if (!ink[k]) continue;
+        const int hh = h - win.h_base[k];
+        const float2* Wk = (k == 0 ? W0 : W1) + ((int64_t)hh * m_w) * Cin * Cout + oc;
+        float2 wv[JW][kRowsWU];
+        auto load_weights = [&](int i0) {  // channels i0, i0+4, ..., clamped (their products are skipped)
+#pragma unroll
+            for (int j = 0; j < JW; ++j) {
+                const int ww = min(ww0 + j, m_w - 1);
+#pragma unroll
+                for (int u = 0; u < kRowsWU; ++u)
+                    wv[j][u] = Wk[((int64_t)ww * Cin + min(i0 + 4 * u, Cin - 1)) * Cout];
+            }
+        };
+        load_weights(q);  // in flight while the rows travel to LDS
+        __syncthreads();
+        {
+            // eight loads per thread in flight at a time (a plain loop would wait for each before the next)
+            const int total = nb * Cin * JW;
+            const float2* xbase = X + (int64_t)n0 * Cin * plane + (int64_t)h * W_all + win.w_base[k];
+            for (int base = 0; base < total; base += 256 * 8) {
+                float2 tmp[8];
+#pragma unroll
+                for (int t = 0; t < 8; ++t) {
+                    const int e = min(base + (int)threadIdx.x + 256 * t, total - 1);
+                    const int ni = e / JW;  // (entry, channel): planes of X are in this order
+                    tmp[t] = xbase[ni * plane + min(ww0 + (e - ni * JW), m_w - 1)];
+                }
+#pragma unroll
+                for (int t = 0; t < 8; ++t) {
+                    const int e = base + (int)threadIdx.x + 256 * t;
+                    if (e < total) xrow[e] = tmp[t];
+                }
+            }
+        }
+        __syncthreads();
+        float2 acc[kRowsNB][JW];
+#pragma unroll
+        for (int nn = 0; nn < kRowsNB; ++nn)
+#pragma unroll
+            for (int j = 0; j < JW; ++j) acc[nn][j] = make_float2(0.f, 0.f);
+        for (int i0 = q; i0 < Cin; i0 += 4 * kRowsWU) {  // this thread's channels i0, i0+4, ..., kRowsWU per step
+            if (i0 != q) load_weights(i0);
+#pragma unroll
+            for (int u = 0; u < kRowsWU; ++u) {
+                if (i0 + 4 * u < Cin) {
+#pragma unroll
+                    for (int nn = 0; nn < kRowsNB; ++nn) {
+                        if (nn < nb) {
+#pragma unroll
+                            for (int j = 0; j < JW; ++j) {
+                                const float2 xv = xrow[(nn * Cin + i0 + 4 * u) * JW + j];
+                                acc[nn][j].x = fmaf(xv.x, wv[j][u].x, acc[nn][j].x);
+                                acc[nn][j].x = fmaf(-xv.y, wv[j][u].y, acc[nn][j].x);
+                                acc[nn][j].y = fmaf(xv.y, wv[j][u].x, acc[nn][j].y);
+                                acc[nn][j].y = fmaf(xv.x, wv[j][u].y, acc[nn][j].y);
+                            }
+                        }
+                    }
+                }
+            }
+        }
+        // four batch entries at a time: partial sums to LDS, thread (o, q) finishes entry q
+#pragma unroll
+        for (int g = 0; g < kRowsNB; g += 4) {
+            if (g >= nb) break;
+            __syncthreads();
+#pragma unroll
+            for (int e4 = 0; e4 < 4; ++e4)
+#pragma unroll
+                for (int j = 0; j < JW; ++j) red[((e4 * 4 + q) * JW + j) * 64 + ol] = acc[g + e4][j];
+            __syncthreads();
+            const int nn = g + q;
+            if (nn < nb && o < Cout) {
+                float2* orow = out + ((int64_t)(n0 + nn) * Cout + o) * plane + (int64_t)h * W_all;
+#pragma unroll
+                for (int j = 0; j < JW; ++j) {
+                    const int ww = ww0 + j;
+                    const int w = win.w_base[k] + ww;
+                    const bool hidden = k == 0 && in1 && w >= win.w_base[1] && w < win.w_base[1] + m_w;
+                    if (ww >= m_w || hidden) continue;
+                    float2 sum = red[((q * 4 + 0) * JW + j) * 64 + ol];
+#pragma unroll
+                    for (int qq = 1; qq < 4; ++qq) {
+                        const float2 t = red[((q * 4 + qq) * JW + j) * 64 + ol];
+                        sum.x += t.x;
+                        sum.y += t.y;
+                    }
+                    orow[w] = sum;
+                }
+            }
+        }
     }
 }
 
@@ -748,12 +906,38 @@ extern "C" int spgt_spectral_mode_contract(const float* X_ft, const float* weigh
     if (!aligned8(X_ft) || !aligned8(weight_1) || !aligned8(weight_2) || !aligned8(Out_ft))
         return fail(SPGT_ERR_INVALID_ARGUMENT, "spectral_mode_contract: complex operands must be 8-byte aligned");
     SpecWindows win{{H_base_1, H_base_2}, {W_base_1, W_base_2}};
+    const int64_t plane = (int64_t)H_all * W_all;
+    const int jw = W_low % 3 == 0 ? 3 : (W_low < 4 ? W_low : 4);  // window columns per contraction block
+    const size_t row_lds = ((size_t)kRowsNB * Cin * jw + (size_t)4 * 4 * jw * 64) * sizeof(float2);
+    const int64_t nA64 = (int64_t)ceil_div(N, kRowsNB) * 2 * H_low * ceil_div(Cout, 64) * ceil_div(W_low, jw);
+    if (row_lds <= 64 * 1024 && nA64 + (int64_t)N * Cout * 8 < ((int64_t)1 << 31)) {
+        // one launch: window rows by contraction blocks, all other rows by zero-fill blocks
+        const SpecSpans spans = rows_outside_windows(H_all, H_low, H_base_1, H_base_2);
+        int64_t zero_rows = 0;
+        for (int sidx = 0; sidx < spans.n; ++sidx) zero_rows += spans.hi[sidx] - spans.lo[sidx];
+        // 16 KB of zeros per block or thereabouts
+        const int chunks = zero_rows == 0 ? 0 : (int)std::max<int64_t>(1, std::min<int64_t>(8, zero_rows * W_all / SPGT_ZERO_CHUNK));
+        const int nA = (int)nA64;
+        const int64_t nB = (int64_t)N * Cout * (std::max(1, chunks) + 1);
+        const dim3 grid((unsigned)(nA + nB));
+#define SPGT_ROWS_LAUNCH(JW)                                                                                         \
+    hipLaunchKernelGGL((spectral_contract_rows_k<JW>), grid, dim3(256), row_lds, stream,                              \
+                       reinterpret_cast<const float2*>(X_ft), reinterpret_cast<const float2*>(weight_1),             \
+                       reinterpret_cast<const float2*>(weight_2), reinterpret_cast<float2*>(Out_ft), N, Cin, Cout,   \
+                       H_all, W_all, H_low, W_low, win, spans, nA, std::max(1, chunks))
+        if (jw == 1) SPGT_ROWS_LAUNCH(1);
+        else if (jw == 2) SPGT_ROWS_LAUNCH(2);
+        else if (jw == 3) SPGT_ROWS_LAUNCH(3);
+        else SPGT_ROWS_LAUNCH(4);
+#undef SPGT_ROWS_LAUNCH
+        return check_launch("spectral_mode_contract");
+    }
+    // very wide inputs: zero fill, then one workgroup per mode
     const int64_t total = (int64_t)N * Cout * H_all * W_all;
     const int fill_blocks = (int)std::min<int64_t>((total + 255) / 256, 256 * 32);
     hipLaunchKernelGGL(spectrum_zero_outside_k, dim3(fill_blocks), dim3(256), 0, stream,
                        reinterpret_cast<float2*>(Out_ft), total, H_all, W_all, H_low, W_low, win);
     const dim3 grid(H_low * W_low, 2, ceil_div(Cout, 64));
-    const int64_t plane = (int64_t)H_all * W_all;
     const SpecLayout lay{Cin * plane, plane, W_all, 1, Cout * plane, plane, W_all, 1, 0};
     hipLaunchKernelGGL(spectral_mode_contract_k, grid, dim3(256), (size_t)kSpecNB * Cin * sizeof(float2), stream,
                        reinterpret_cast<const float2*>(X_ft), reinterpret_cast<const float2*>(weight_1),

@@ -119,6 +119,90 @@ __device__ __forceinline__ void st_stream(float4* p, float4 v) {
         *p = v;
 }
 
+// Rows [lo, hi) of an [H_all, W_all] plane that lie outside two row windows (at most three spans).
+struct SpecSpans {
+    int lo[3], hi[3];
+    int n;
+};
+
+inline SpecSpans rows_outside_windows(int H_all, int H_low, int H_base_1, int H_base_2) {
+    SpecSpans spans{};
+    const int lo1 = H_base_1 < H_base_2 ? H_base_1 : H_base_2;
+    const int lo2 = H_base_1 < H_base_2 ? H_base_2 : H_base_1;
+    const int edges[4] = {lo1, lo1 + H_low, lo2, lo2 + H_low};
+    int cursor = 0;
+    for (int e = 0; e < 4; e += 2) {
+        if (edges[e] > cursor) {
+            spans.lo[spans.n] = cursor;
+            spans.hi[spans.n] = edges[e];
+            ++spans.n;
+        }
+        cursor = cursor > edges[e + 1] ? cursor : edges[e + 1];
+    }
+    if (cursor < H_all) {
+        spans.lo[spans.n] = cursor;
+        spans.hi[spans.n] = H_all;
+        ++spans.n;
+    }
+    return spans;
+}
+
+// Stores zeros to out[lo, hi) (complex elements) with all 256 threads of a workgroup: 16-byte stores between an
+// 8-byte head and tail.
+__device__ __forceinline__ void zero_complex_range(float2* __restrict__ out, int64_t lo, int64_t hi) {
+    if (lo >= hi) return;
+    if ((reinterpret_cast<uintptr_t>(out + lo) & 15u) != 0) {
+        if (threadIdx.x == 0) out[lo] = make_float2(0.f, 0.f);
+        ++lo;
+    }
+    const int64_t pairs = (hi - lo) >> 1;
+    float4* o4 = reinterpret_cast<float4*>(out + lo);
+    for (int64_t t = threadIdx.x; t < pairs; t += 256) o4[t] = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (((hi - lo) & 1) && threadIdx.x == 0) out[hi - 1] = make_float2(0.f, 0.f);
+}
+
+// Zero fill of chunk c (of `chunks`) of the rows in `spans` of plane p: out [planes, H_all, W_all] complex.
+__device__ __forceinline__ void zero_span_chunk(float2* __restrict__ out, const SpecSpans& spans, int64_t p, int c,
+                                                int chunks, int64_t plane, int W_all) {
+    int64_t total = 0;
+    for (int s = 0; s < spans.n; ++s) total += (int64_t)(spans.hi[s] - spans.lo[s]) * W_all;
+    const int64_t per = ((total + chunks - 1) / chunks + 1) & ~(int64_t)1;
+    const int64_t a = c * per, b = total < a + per ? total : a + per;
+    int64_t off = 0;
+    for (int s = 0; s < spans.n; ++s) {  // the chunk's share of each span
+        const int64_t len = (int64_t)(spans.hi[s] - spans.lo[s]) * W_all;
+        const int64_t lo = a > off ? a : off, hi = b < off + len ? b : off + len;
+        if (lo < hi) {
+            const int64_t base = p * plane + (int64_t)spans.lo[s] * W_all - off;
+            zero_complex_range(out, base + lo, base + hi);
+        }
+        off += len;
+    }
+}
+
+// Zeroes, in plane p of out [planes, H_all, W_all] (complex), the elements of the window rows that lie in
+// neither window: [h_base_k, h_base_k + m_h) x [w_base_k, w_base_k + m_w), k = 0, 1.  Wave v of the
+// workgroup takes the row slots v, v + 4, ...; lanes run along w.
+__device__ __forceinline__ void zero_window_row_remainders(float2* __restrict__ out, int64_t p, int64_t plane,
+                                                           int W_all, int m_h, int m_w, int hb0, int wb0, int hb1,
+                                                           int wb1) {
+    const int lane = threadIdx.x & 63;
+    float2* pl = out + p * plane;
+    for (int slot = threadIdx.x >> 6; slot < 2 * m_h; slot += 4) {
+        const int k0 = slot >= m_h;
+        const int h = (k0 ? hb1 : hb0) + slot - k0 * m_h;
+        const bool in0 = h >= hb0 && h < hb0 + m_h;
+        const bool in1 = h >= hb1 && h < hb1 + m_h;
+        if (k0 && in0) continue;  // counted with the first window's rows
+        float2* orow = pl + (int64_t)h * W_all;
+        for (int w = lane; w < W_all; w += 64) {
+            const bool c0 = in0 && w >= wb0 && w < wb0 + m_w;
+            const bool c1 = in1 && w >= wb1 && w < wb1 + m_w;
+            if (!c0 && !c1) orow[w] = make_float2(0.f, 0.f);
+        }
+    }
+}
+
 __host__ __device__ __forceinline__ int ceil_div(int a, int b) { return (a + b - 1) / b; }
 __host__ __device__ __forceinline__ int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 

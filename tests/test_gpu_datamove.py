@@ -118,6 +118,34 @@ def test_spectral_mode_contract_vs_oracle(gpu, N, Cin, Cout, r, m):
     assert max_rel(torch.view_as_real(seq.cpu()).double(), torch.view_as_real(want)) < 1e-5
 
 
+@pytest.mark.parametrize("N,Cin,Cout,H,W,mh,mw,hb1,wb1,hb2,wb2", [
+    (2, 5, 3, 9, 6, 3, 3, 1, 2, 4, 1),       # windows anywhere, disjoint rows
+    (3, 4, 70, 10, 7, 4, 3, 2, 1, 4, 3),     # rows overlap, columns overlap partly: the second window wins
+    (1, 3, 2, 6, 5, 3, 2, 0, 0, 0, 0),       # identical windows
+    (2, 8, 8, 12, 40, 2, 33, 9, 5, 1, 0),    # wide windows (more than 32 columns), second window first in memory
+    (1, 2, 2, 5, 4, 5, 4, 0, 0, 0, 0),       # windows cover everything: nothing to zero
+])
+def test_spectral_mode_contract_general_windows(gpu, N, Cin, Cout, H, W, mh, mw, hb1, wb1, hb2, wb2):
+    """Windows at arbitrary bases, overlapping and not, against the reference's gather -> matmul -> scatter
+    sequence (extension/bind/datamove.cu:25-64) in complex128; every element outside the windows must be zero
+    even though the output buffer starts out as NaN."""
+    xf = torch.view_as_complex(rnd(N, Cin, H, W, 2, seed=31))
+    w1, w2 = rnd(mh, mw, Cin, Cout, 2, seed=32), rnd(mh, mw, Cin, Cout, 2, seed=33)
+    g1, g2 = O.op_transpose_gather_dual(xf.to(torch.complex128), [N, Cin], H, W, mh, mw, hb1, wb1, hb2, wb2)
+    c = lambda w: torch.view_as_complex(w.double().contiguous())
+    want = O.op_transpose_scatter_dual(g1 @ c(w1), g2 @ c(w2), [N, Cout], H, W, mh, mw, hb1, wb1, hb2, wb2)
+    poison = torch.full((1 << 20,), float("nan"), device=gpu)  # the allocator hands these bytes to the output
+    del poison
+    got = dm.spectral_mode_contract(xf.to(gpu), w1.to(gpu), w2.to(gpu), mh, mw, hb1, wb1, hb2, wb2)
+    assert got.shape == (N, Cout, H, W)
+    mask = torch.zeros(H, W, dtype=torch.bool)
+    mask[hb1:hb1 + mh, wb1:wb1 + mw] = True
+    mask[hb2:hb2 + mh, wb2:wb2 + mw] = True
+    gr = torch.view_as_real(got.cpu())
+    assert (gr[:, :, ~mask] == 0).all()
+    assert max_rel(gr.double(), torch.view_as_real(want)) < 1e-5
+
+
 def test_spectral_mode_contract_golden(gpu):
     """Reference SpectralConv2D fixture: rfft2 / irfft2 by torch on the GPU, the middle by the fused kernel."""
     p, i, want, meta = load_golden("spectral_conv2d")
