@@ -493,8 +493,26 @@ def main():
     n_sets = max(1, args.input_sets)
     sets = [tuple(torch.randn(B, S, H * 32, device=dev, generator=g) for _ in range(3)) for _ in range(n_sets)]
     one, zero = torch.ones(H, 32, device=dev), torch.zeros(H, 32, device=dev)
-    step = lambda i: ga.galerkin_attention_fused(*sets[i % n_sets], None, one, zero, one, zero, 1e-6, H, dp)
     nbytes = 4 * B * H * 32 * S * 4
+
+    # A step goes through the C ABI directly, as a compiled caller would: outputs (one per input set, so that no
+    # step overwrites lines the previous one left in the cache), K^T V / S and the workspace are allocated once.
+    import ctypes
+    from spgt_amd import _lib
+    lib = _lib.load()
+    outs = [torch.empty(B, S, H * 32, device=dev) for _ in range(n_sets)]
+    ktv = torch.empty(B, H, 32, 32, device=dev)
+    ws_bytes = lib.spgt_galerkin_attention_fused_workspace_bytes(B, S, H, dp)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    vp = lambda t: ctypes.c_void_p(t.data_ptr())
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    call_args = [(vp(q), vp(k), vp(v), H * 32, None, vp(one), vp(zero), vp(one), vp(zero), 1e-6, vp(o), vp(ktv), vp(ws),
+                  ws_bytes, B, S, H, dp, stream) for (q, k, v), o in zip(sets, outs)]
+    fused = lib.spgt_galerkin_attention_fused_forward
+
+    def step(i):
+        if fused(*call_args[i % n_sets]) != 0:
+            raise RuntimeError(_lib.last_error())
 
     def wall_ms(fn):
         for i in range(args.warmup):
@@ -506,9 +524,17 @@ def main():
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) / args.steps * 1e3
 
-    ms_per_step = wall_ms(step)  # the timed region: exactly `steps` calls, inputs rotated
+    ms_per_step = wall_ms(step)  # the timed region: exactly `steps` calls, inputs and outputs rotated
     value = nbytes / (ms_per_step * 1e-3) / 1e9
-    same_ms = wall_ms(lambda i: step(0))  # every step on one input set (Q fits the last-level cache)
+    same_ms = wall_ms(lambda i: step(0))  # every step on one set (Q and out fit the last-level cache)
+    binding_ms = wall_ms(lambda i: ga.galerkin_attention_fused(*sets[i % n_sets], None, one, zero, one, zero, 1e-6,
+                                                               H, dp))  # the Python operator, allocating its output
+    # host time per step without the GPU in the way: how far the launch rate is from bounding the loop
+    t0 = time.perf_counter()
+    for i in range(20):
+        step(i)
+    host_us = (time.perf_counter() - t0) / 20 * 1e6
+    torch.cuda.synchronize()
 
     # per-call and per-launch durations of the same rotated sequence: HIP events on the launch stream
     # around every launch, calls back to back, one synchronisation at the end
@@ -600,7 +626,9 @@ def main():
                    "algorithmic_bytes_per_step": nbytes, "hbm_frac_of_8TBps": round(value / HBM_PEAK_GBPS, 4),
                    "input_sets_rotated": n_sets,
                    "ms_per_step_one_input_set": round(same_ms, 4),
-                   "GBps_one_input_set": round(nbytes / same_ms / 1e6, 1)},
+                   "GBps_one_input_set": round(nbytes / same_ms / 1e6, 1),
+                   "ms_per_step_python_operator": round(binding_ms, 4),
+                   "host_us_per_step_issue": round(host_us, 1)},
         "roofline": roofline,
         "cpu_baseline": None if args.no_cpu_baseline else cpu_baseline(B, S, H, 0),
         "extra": extra,

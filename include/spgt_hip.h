@@ -458,21 +458,22 @@ int spgt_strided_copy_batch(const spgt_copy_desc* descs, int count, spgt_stream_
 
 /* Instrumented variant of spgt_galerkin_attention_fused_forward for benchmarks (no reference
  * counterpart): enqueues the call `iterations` times back to back (no synchronisation between
- * them, as a caller's loop would), iteration i reading the input set i % n_sets (Q_sets, K_sets,
- * V_sets: host arrays of n_sets device pointers, so that consecutive iterations need not find
- * their inputs in the last-level cache), with HIP events recorded on `stream` around each of the
+ * them, as a caller's loop would), iteration i reading the input set i % n_sets and writing the
+ * output of the same index (Q_sets, K_sets, V_sets, out_sets: host arrays of n_sets device
+ * pointers, so that consecutive iterations need not find their operands in the last-level
+ * cache), with HIP events recorded on `stream` around each of the
  * three launches.  After one synchronisation at the end it writes, to host memory,
  *   stage_ms[3 i + 0]  K/V pass of iteration i (LayerNorm + partial K'^T V' tiles)
  *   stage_ms[3 i + 1]  fixed-order reduction of the partial tiles
  *   stage_ms[3 i + 2]  Q pass (out = Q' M)
  * in milliseconds, each from the event before the launch to the event after it. */
 int spgt_galerkin_attention_fused_profile(const float* const* Q_sets, const float* const* K_sets,
-                                          const float* const* V_sets, int n_sets, int64_t ld_in,
-                                          const float* position, const float* ln_weight_K,
+                                          const float* const* V_sets, float* const* out_sets, int n_sets,
+                                          int64_t ld_in, const float* position, const float* ln_weight_K,
                                           const float* ln_bias_K, const float* ln_weight_V,
-                                          const float* ln_bias_V, float norm_eps, float* out, float* ktv,
-                                          void* workspace, size_t workspace_bytes, int B, int S, int H,
-                                          int dp, spgt_stream_t stream, int iterations, float* stage_ms);
+                                          const float* ln_bias_V, float norm_eps, float* ktv, void* workspace,
+                                          size_t workspace_bytes, int B, int S, int H, int dp,
+                                          spgt_stream_t stream, int iterations, float* stage_ms);
 
 #ifdef __cplusplus
 }

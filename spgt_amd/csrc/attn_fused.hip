@@ -33,19 +33,19 @@
 
 // Cache policy of the three touch-once streams (K/V reads, Q reads, out
 // writes).  Measured on MI355X at B=8, S=44521 over all eight combinations,
-// with consecutive calls on different inputs (so that no call finds its Q in
-// the 256 MB last-level cache): non-temporal K/V and Q loads with plain out
-// stores is the fastest (147 us per call; non-temporal stores as well 154 us;
-// plain Q loads with non-temporal stores 151 us; everything plain 171 us,
-// because the K/V pass then runs at 102 us instead of 67 us).
+// with consecutive calls on different inputs and outputs (so that no call
+// finds its Q, or the lines it writes, in the 256 MB last-level cache):
+// non-temporal K/V loads and out stores with plain Q loads is the fastest
+// (154 us per call; plain stores 155-159 us; plain K/V loads 157-176 us,
+// because the K/V pass then runs at 71-101 us instead of 69 us).
 #ifndef SPGT_NT_P1LD
 #define SPGT_NT_P1LD true
 #endif
 #ifndef SPGT_NT_P2LD
-#define SPGT_NT_P2LD true
+#define SPGT_NT_P2LD false
 #endif
 #ifndef SPGT_NT_P2ST
-#define SPGT_NT_P2ST false
+#define SPGT_NT_P2ST true
 #endif
 
 namespace spgt {
@@ -833,11 +833,11 @@ extern "C" int spgt_fold_ktv_into_fc(const float* ktv, const float* fc_weight_kn
 }
 
 extern "C" int spgt_galerkin_attention_fused_profile(
-    const float* const* Q_sets, const float* const* K_sets, const float* const* V_sets, int n_sets, int64_t ld_in,
-    const float* position, const float* ln_weight_K, const float* ln_bias_K, const float* ln_weight_V,
-    const float* ln_bias_V, float norm_eps, float* out, float* ktv, void* workspace, size_t workspace_bytes, int B,
-    int S, int H, int dp, hipStream_t stream, int iterations, float* stage_ms) {
-    if (iterations <= 0 || iterations > 4096 || !stage_ms || n_sets <= 0 || !Q_sets || !K_sets || !V_sets)
+    const float* const* Q_sets, const float* const* K_sets, const float* const* V_sets, float* const* out_sets,
+    int n_sets, int64_t ld_in, const float* position, const float* ln_weight_K, const float* ln_bias_K,
+    const float* ln_weight_V, const float* ln_bias_V, float norm_eps, float* ktv, void* workspace,
+    size_t workspace_bytes, int B, int S, int H, int dp, hipStream_t stream, int iterations, float* stage_ms) {
+    if (iterations <= 0 || iterations > 4096 || !stage_ms || n_sets <= 0 || !Q_sets || !K_sets || !V_sets || !out_sets)
         return fail(SPGT_ERR_INVALID_ARGUMENT,
                     "galerkin_attention_fused_profile: 1..4096 iterations, stage_ms and at least one input set required");
     // event 3 i + k: before launch k of iteration i; the last event closes the last launch
@@ -855,8 +855,8 @@ extern "C" int spgt_galerkin_attention_fused_profile(
         // the closing event of one iteration is the opening event of the next: it is recorded once, by the
         // iteration it closes, and iteration 0 records its own opening event
         rc = fused_forward_impl(Q_sets[s], K_sets[s], V_sets[s], ld_in, position, ln_weight_K, ln_bias_K, ln_weight_V,
-                                ln_bias_V, norm_eps, out, ktv, workspace, workspace_bytes, B, S, H, dp, stream, four,
-                                it == 0);
+                                ln_bias_V, norm_eps, out_sets[s], ktv, workspace, workspace_bytes, B, S, H, dp, stream,
+                                four, it == 0);
     }
     if (rc == SPGT_OK && hipEventSynchronize(ev[nev - 1]) != hipSuccess)
         rc = fail(SPGT_ERR_LAUNCH, "galerkin_attention_fused_profile: hipEventSynchronize failed");

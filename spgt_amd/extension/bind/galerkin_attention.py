@@ -311,7 +311,8 @@ def _attention_fused_profile(input_sets, position, ln_weight_K, ln_bias_K, ln_we
                              num_head: int, dim_position: int, iterations: int):
     """Per-iteration milliseconds [iterations][3] of the three launches of the fused attention core (K/V pass,
     tile reduction, Q pass) over `iterations` back-to-back calls, iteration i on input_sets[i % len(input_sets)]
-    (a list of (Q, K, V) triples of one shape), measured with HIP events on the current stream."""
+    (a list of (Q, K, V) triples of one shape) and writing an output buffer of its own per set, measured with HIP
+    events on the current stream."""
     import ctypes
     Q0 = input_sets[0][0]
     B, S, _ = Q0.shape
@@ -322,16 +323,17 @@ def _attention_fused_profile(input_sets, position, ln_weight_K, ln_bias_K, ln_we
             if t.shape != Q0.shape:
                 raise ValueError("all profile inputs must share one shape")
     lib = _lib.load()
-    out = torch.empty((B, S, H * D), dtype=torch.float32, device=Q0.device)
+    n = len(input_sets)
+    outs = [torch.empty((B, S, H * D), dtype=torch.float32, device=Q0.device) for _ in range(n)]
     ktv = torch.empty((B, H, D, D), dtype=torch.float32, device=Q0.device)
     ws = workspace(lib.spgt_galerkin_attention_fused_workspace_bytes(B, S, H, dim_position), Q0)
-    n = len(input_sets)
     arrs = [(ctypes.c_void_p * n)(*[trip[j].data_ptr() for trip in input_sets]) for j in range(3)]
+    out_arr = (ctypes.c_void_p * n)(*[o.data_ptr() for o in outs])
     stage = (ctypes.c_float * (3 * int(iterations)))()
     with torch.cuda.device(Q0.device):
         check(lib.spgt_galerkin_attention_fused_profile(
-            arrs[0], arrs[1], arrs[2], n, Q0.stride(1), ptr(position) if dim_position == 2 else None,
-            ptr(ln_weight_K), ptr(ln_bias_K), ptr(ln_weight_V), ptr(ln_bias_V), float(norm_eps), ptr(out), ptr(ktv),
+            arrs[0], arrs[1], arrs[2], out_arr, n, Q0.stride(1), ptr(position) if dim_position == 2 else None,
+            ptr(ln_weight_K), ptr(ln_bias_K), ptr(ln_weight_V), ptr(ln_bias_V), float(norm_eps), ptr(ktv),
             ptr(ws), ws.numel(), B, S, H, dim_position, stream_of(Q0), int(iterations), stage))
     return [[float(stage[3 * i + k]) for k in range(3)] for i in range(int(iterations))]
 
