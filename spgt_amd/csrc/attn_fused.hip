@@ -44,6 +44,9 @@
 #ifndef SPGT_NT_P2LD
 #define SPGT_NT_P2LD false
 #endif
+#ifndef SPGT_NT_TILE
+#define SPGT_NT_TILE true
+#endif
 #ifndef SPGT_NT_P2ST
 #define SPGT_NT_P2ST true
 #endif
@@ -73,17 +76,23 @@ __device__ __forceinline__ float2 ln_pair(float2 x, float g0, float g1, float b0
 
 }  // namespace
 
-// grid (nchunk, H/4, B), block 256: wave w handles head 4*blockIdx.y + w.
+// grid (nchunk, H/4, B), block 256 * NSUB: wave w handles head 4*blockIdx.y + w % 4 on the sub-range w / 4 of the
+// workgroup's chunk (tokens_per_chunk / NSUB tokens each).  With NSUB > 1 the waves' tiles meet in LDS and the
+// workgroup writes their sum, sub-ranges in increasing order: a third or a quarter of the partial tiles reach
+// memory (at B=8, S=44521 the 12.6 MB of one-tile-per-wave cost the pass 5 us of its 67, most of it the
+// write-back at the end of the kernel).
 // Lane l of a wave: token slot t = l/16, feature pair p = l%16 (features 2p, 2p+1).
-template <int DP, int U>
-__global__ __launch_bounds__(256) void ktv_ln_partial_tm(
+template <int DP, int U, int NSUB>
+__global__ __launch_bounds__(256 * NSUB) void ktv_ln_partial_tm(
     const float* __restrict__ K, const float* __restrict__ V, const float* __restrict__ pos,
     const float* __restrict__ lnwK, const float* __restrict__ lnbK,
     const float* __restrict__ lnwV, const float* __restrict__ lnbV, float eps,
     float* __restrict__ partial, int S, int H, int64_t ld, int tokens_per_chunk) {
     constexpr int D = DP + 32;
+    extern __shared__ __attribute__((aligned(16))) float sub_tiles[];  // NSUB > 1: [NSUB][4 heads][D * D]
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    const int wave = (threadIdx.x >> 6) & 3;
+    const int sub = threadIdx.x >> 8;
     const int h = blockIdx.y * 4 + wave;
     const int b = blockIdx.z;
     const int chunk = blockIdx.x;
@@ -91,8 +100,9 @@ __global__ __launch_bounds__(256) void ktv_ln_partial_tm(
     const int t = lane >> 4;
     const int p = lane & 15;
 
-    const int s0 = chunk * tokens_per_chunk;
-    const int s1 = min(S, s0 + tokens_per_chunk);
+    const int sub_len = tokens_per_chunk / NSUB;
+    const int s0 = min(S, chunk * tokens_per_chunk + sub * sub_len);
+    const int s1 = min(S, s0 + sub_len);
 
     const int f = h * 32 + 2 * p;
     const float gK0 = lnwK[f], gK1 = lnwK[f + 1], bK0 = lnbK[f], bK1 = lnbK[f + 1];
@@ -246,7 +256,8 @@ __global__ __launch_bounds__(256) void ktv_ln_partial_tm(
     }
 
     // acc[ta][tb][r] = M[2*(4t+r)+ta][2p+tb]
-    float* tile = partial + (((int64_t)b * H + h) * nchunk + chunk) * (D * D);
+    float* tile = NSUB > 1 ? sub_tiles + (sub * 4 + wave) * (D * D)
+                           : partial + (((int64_t)b * H + h) * nchunk + chunk) * (D * D);
 #pragma unroll
     for (int ta = 0; ta < 2; ++ta)
 #pragma unroll
@@ -255,7 +266,8 @@ __global__ __launch_bounds__(256) void ktv_ln_partial_tm(
             float2 o;
             o.x = acc[ta][0][r];
             o.y = acc[ta][1][r];
-            *reinterpret_cast<float2*>(tile + i * D + DP + 2 * p) = o;
+            if (NSUB == 1) st_stream<SPGT_NT_TILE>(reinterpret_cast<float2*>(tile + i * D + DP + 2 * p), o);
+            else *reinterpret_cast<float2*>(tile + i * D + DP + 2 * p) = o;
         }
     if (DP == 2) {
 #pragma unroll
@@ -288,6 +300,23 @@ __global__ __launch_bounds__(256) void ktv_ln_partial_tm(
                 tile[D] = pp[1];
                 tile[D + 1] = pp[2];
             }
+        }
+    }
+    if constexpr (NSUB > 1) {
+        __syncthreads();
+        // the four heads' tiles are contiguous in LDS per sub-range and in memory per chunk only within a head
+        constexpr int E4 = D * D / 4;  // float4 per tile
+        for (int e = threadIdx.x; e < 4 * E4; e += 256 * NSUB) {
+            const int hh = e / E4;
+            const int r4 = e - hh * E4;
+            float4 sum = *reinterpret_cast<const float4*>(sub_tiles + hh * (D * D) + 4 * r4);
+#pragma unroll
+            for (int q = 1; q < NSUB; ++q) {
+                const float4 v = *reinterpret_cast<const float4*>(sub_tiles + (q * 4 + hh) * (D * D) + 4 * r4);
+                sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
+            }
+            float* dst = partial + (((int64_t)b * H + blockIdx.y * 4 + hh) * nchunk + chunk) * (D * D) + 4 * r4;
+            st_stream<SPGT_NT_TILE>(reinterpret_cast<float4*>(dst), sum);
         }
     }
 }
@@ -538,6 +567,7 @@ __global__ __launch_bounds__(256) void qm_apply_tm(
 namespace {
 
 struct FusedPlan {
+    int nsub;           // K^T V pass: waves per head in a workgroup
     int tpc1, nchunk1;  // K^T V pass
     int tpc2, nchunk2;  // Q M pass
 };
@@ -554,25 +584,49 @@ int g_target_wg1 = 0, g_target_wg2 = 0;
 constexpr int g_target_wg1 = 0, g_target_wg2 = 0;
 #endif
 
+// Long sequences give every wave of a 1024-thread workgroup (4 heads x 4 sub-ranges) enough tokens: one
+// workgroup per CU then, whose four tiles per head are summed in LDS before they go to memory.
+#ifndef SPGT_KSUB
+#define SPGT_KSUB 4
+#endif
+#ifndef SPGT_SUB_WG_PER_CU
+#define SPGT_SUB_WG_PER_CU 1
+#endif
+constexpr int kSub = SPGT_KSUB;
+constexpr int kSubMinTokens = 256;  // per wave
+
 FusedPlan make_plan(int B, int S, int H) {
     // Chunks are whole unrolled groups so that only the last chunk of a batch has a ragged tail.
     // The K/V pass never uses more chunks than tile_reduce can sum.
     const int bg = std::max(1, B * (H / 4));
-    const int dflt = 3 * device_cu_count();
-    // Short sequences: a chunk of the three-per-CU plan would hold fewer than 128 tokens, and the partial tiles it
-    // writes for the reduction (D*D floats per head) weigh as much as the K and V rows it reads.  One workgroup
-    // per CU then (B=4, S=5041: K/V pass 14.5 -> 10 us, reduction 4.4 -> 3.7 us; fewer still is slower again).
-    const int short_t1 = S / std::max(1, dflt / bg) < 128 ? device_cu_count() : dflt;
-    const int t1 = g_target_wg1 > 0 ? g_target_wg1 : short_t1;
-    const int t2 = g_target_wg2 > 0 ? g_target_wg2 : dflt;
-    const int per_bh1 = std::min(kReduceChains * kReduceMaxPerChain, std::max(1, t1 / bg));
-    const int per_bh2 = std::max(1, t2 / bg);
+    const int cus = device_cu_count();
+    const int dflt = 3 * cus;
     FusedPlan p;
     const int g1 = 4 * kU1, g2 = 16 * kU2;
-    p.tpc1 = std::max(g1, ceil_div(ceil_div(S, per_bh1), g1) * g1);
-    p.nchunk1 = ceil_div(S, p.tpc1);
+    const int t2 = g_target_wg2 > 0 ? g_target_wg2 : dflt;
+    const int per_bh2 = std::max(1, t2 / bg);
     p.tpc2 = std::max(g2, ceil_div(ceil_div(S, per_bh2), g2) * g2);
     p.nchunk2 = ceil_div(S, p.tpc2);
+    // K/V pass: one 1024-thread workgroup per CU when the sequence is long enough ...
+    const int per_bh_sub = std::max(1, SPGT_SUB_WG_PER_CU * cus / bg);
+    const int gs = g1 * kSub;
+    const int tpc_sub = std::max(gs, ceil_div(ceil_div(S, per_bh_sub), gs) * gs);
+    if (g_target_wg1 == 0 && tpc_sub / kSub >= kSubMinTokens && ceil_div(S, tpc_sub) <= kReduceChains * kReduceMaxPerChain) {
+        p.nsub = kSub;
+        p.tpc1 = tpc_sub;
+        p.nchunk1 = ceil_div(S, tpc_sub);
+        return p;
+    }
+    // ... else 256-thread workgroups, three per CU; for short sequences, where a chunk of that plan would hold
+    // fewer than 128 tokens and the partial tiles it writes (D*D floats per head) weigh as much as the K and V
+    // rows it reads, one per CU (B=4, S=5041: K/V pass 14.5 -> 10 us, reduction 4.4 -> 3.7 us; fewer still is
+    // slower again).
+    const int short_t1 = S / std::max(1, dflt / bg) < 128 ? cus : dflt;
+    const int t1 = g_target_wg1 > 0 ? g_target_wg1 : short_t1;
+    const int per_bh1 = std::min(kReduceChains * kReduceMaxPerChain, std::max(1, t1 / bg));
+    p.nsub = 1;
+    p.tpc1 = std::max(g1, ceil_div(ceil_div(S, per_bh1), g1) * g1);
+    p.nchunk1 = ceil_div(S, p.tpc1);
     return p;
 }
 
@@ -633,11 +687,29 @@ int fused_forward_impl(
     const dim3 blockr(1024);
     const float* pos = position ? position : K;  // never dereferenced when dp == 0
     if (ev && record_first) (void)hipEventRecord(ev[0], stream);
-    if (dp == 0) {
-        hipLaunchKernelGGL((ktv_ln_partial_tm<0, kU1>), grid1, block, 0, stream, K, V, pos, ln_weight_K,
+    if (p.nsub > 1) {
+        const dim3 block_sub(256 * kSub);
+        const size_t lds = (size_t)kSub * 4 * D * D * sizeof(float);
+        if (dp == 0) {
+            static const hipError_t attr0 = hipFuncSetAttribute(
+                reinterpret_cast<const void*>(&ktv_ln_partial_tm<0, kU1, kSub>),
+                hipFuncAttributeMaxDynamicSharedMemorySize, (int)(kSub * 4 * 32 * 32 * sizeof(float)));
+            (void)attr0;
+            hipLaunchKernelGGL((ktv_ln_partial_tm<0, kU1, kSub>), grid1, block_sub, lds, stream, K, V, pos, ln_weight_K,
+                               ln_bias_K, ln_weight_V, ln_bias_V, norm_eps, partial, S, H, ld_in, p.tpc1);
+        } else {
+            static const hipError_t attr2 = hipFuncSetAttribute(
+                reinterpret_cast<const void*>(&ktv_ln_partial_tm<2, kU1, kSub>),
+                hipFuncAttributeMaxDynamicSharedMemorySize, (int)(kSub * 4 * 34 * 34 * sizeof(float)));
+            (void)attr2;
+            hipLaunchKernelGGL((ktv_ln_partial_tm<2, kU1, kSub>), grid1, block_sub, lds, stream, K, V, pos, ln_weight_K,
+                               ln_bias_K, ln_weight_V, ln_bias_V, norm_eps, partial, S, H, ld_in, p.tpc1);
+        }
+    } else if (dp == 0) {
+        hipLaunchKernelGGL((ktv_ln_partial_tm<0, kU1, 1>), grid1, block, 0, stream, K, V, pos, ln_weight_K,
                            ln_bias_K, ln_weight_V, ln_bias_V, norm_eps, partial, S, H, ld_in, p.tpc1);
     } else {
-        hipLaunchKernelGGL((ktv_ln_partial_tm<2, kU1>), grid1, block, 0, stream, K, V, pos, ln_weight_K,
+        hipLaunchKernelGGL((ktv_ln_partial_tm<2, kU1, 1>), grid1, block, 0, stream, K, V, pos, ln_weight_K,
                            ln_bias_K, ln_weight_V, ln_bias_V, norm_eps, partial, S, H, ld_in, p.tpc1);
     }
     if (ev) (void)hipEventRecord(ev[1], stream);
