@@ -54,7 +54,8 @@ const char* spgt_last_error(void);
  *   input [batch, seqlen, dim_hidden], weight [dim_hidden, dim_hidden] used as stored
  *   (x @ W), bias [dim_hidden], position [batch, seqlen, dim_position] or NULL,
  *   out [batch, num_head, dim_position + dim_head, seqlen].
- * dim_head must be 32, dim_hidden 128 or 256, dim_position 0 or 2. */
+  * dim_head must be 32, dim_hidden 128, 256, 384 or 512 (the reference accepts multiples of 128,
+ * network/sp_layer.py:17), dim_position 0 or 2. */
 int spgt_multihead_projection_with_position_rrc_forward(
     const float* input, const float* weight, const float* bias, const float* position, float* out,
     int seqlen, int dim_hidden, int num_head, int dim_head, int dim_position, int batch,
@@ -93,6 +94,15 @@ int spgt_batched_skinny_gemm(const float* A, const float* B, float* C, float alp
                              int K, int64_t a_stride, int64_t b_stride, int64_t c_stride, int order,
                              int batch_count, void* workspace, size_t workspace_bytes,
                              spgt_stream_t stream);
+
+/* Replaces sgemm_32x32_4x4::sgemm_cuda (extension/native/sgemm_32x32.cu:683-710), the batched GEMM for a
+ * short contraction axis and long M or N that the reference uses for Q (K^T V) and in the attention backward
+ * (extension/bind/galerkin_attention.cu:118-122, 142-171):
+ *   C[b] = alpha * A[b] * B[b],  A: M x K, B: K x N, C: M x N, any of the eight operand orders,
+ * one launch, every 32 x 32 tile of C computed by one workgroup over the whole of K, no workspace. */
+int spgt_batched_small_k_gemm(const float* A, const float* B, float* C, float alpha, int M, int N, int K,
+                              int64_t a_stride, int64_t b_stride, int64_t c_stride, int order,
+                              int batch_count, spgt_stream_t stream);
 
 /* One-call fused attention core on token-major operands.  No single reference
  * function corresponds to it: it computes what Sp_GalerkinAttention.forward

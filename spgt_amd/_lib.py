@@ -30,6 +30,7 @@ SIGNATURES = {
     "spgt_galerkin_attention_cccr_forward": (_i, [_p, _p, _p, _p, _p, _sz, _i, _i, _i, _i, _p]),
     "spgt_batched_skinny_gemm_workspace_bytes": (_sz, [_i, _i, _i, _i]),
     "spgt_batched_skinny_gemm": (_i, [_p, _p, _p, _f, _i, _i, _i, _i64, _i64, _i64, _i, _i, _p, _sz, _p]),
+    "spgt_batched_small_k_gemm": (_i, [_p, _p, _p, _f, _i, _i, _i, _i64, _i64, _i64, _i, _i, _p]),
     "spgt_galerkin_attention_fused_workspace_bytes": (_sz, [_i, _i, _i, _i]),
     "spgt_galerkin_attention_fused_forward": (
         _i, [_p, _p, _p, _i64, _p, _p, _p, _p, _p, _f, _p, _p, _p, _sz, _i, _i, _i, _i, _p]),

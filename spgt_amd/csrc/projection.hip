@@ -180,8 +180,8 @@ int projection_common(const char* who, const float* input, const float* weight, 
     if (batch <= 0 || seqlen <= 0) return fail(SPGT_ERR_INVALID_ARGUMENT, "multihead_projection: batch and seqlen must be positive");
     if (dim_head != 32 || num_head * dim_head != dim_hidden)
         return fail(SPGT_ERR_INVALID_ARGUMENT, "multihead_projection: dim_head must be 32 and num_head*32 == dim_hidden");
-    if (dim_hidden != 128 && dim_hidden != 256)
-        return fail(SPGT_ERR_INVALID_ARGUMENT, "multihead_projection: dim_hidden must be 128 or 256");
+    if (dim_hidden != 128 && dim_hidden != 256 && dim_hidden != 384 && dim_hidden != 512)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "multihead_projection: dim_hidden must be 128, 256, 384 or 512");
     if (dim_position != 0 && dim_position != 2)
         return fail(SPGT_ERR_INVALID_ARGUMENT, "multihead_projection: dim_position must be 0 or 2");
     if (dim_position == 2 && !position)
@@ -197,9 +197,15 @@ int projection_common(const char* who, const float* input, const float* weight, 
     if (kc == 1) {
         if (ln) { if (dim_position) SPGT_PROJ(1, 2, true); else SPGT_PROJ(1, 0, true); }
         else    { if (dim_position) SPGT_PROJ(1, 2, false); else SPGT_PROJ(1, 0, false); }
-    } else {
+    } else if (kc == 2) {
         if (ln) { if (dim_position) SPGT_PROJ(2, 2, true); else SPGT_PROJ(2, 0, true); }
         else    { if (dim_position) SPGT_PROJ(2, 2, false); else SPGT_PROJ(2, 0, false); }
+    } else if (kc == 3) {
+        if (ln) { if (dim_position) SPGT_PROJ(3, 2, true); else SPGT_PROJ(3, 0, true); }
+        else    { if (dim_position) SPGT_PROJ(3, 2, false); else SPGT_PROJ(3, 0, false); }
+    } else {
+        if (ln) { if (dim_position) SPGT_PROJ(4, 2, true); else SPGT_PROJ(4, 0, true); }
+        else    { if (dim_position) SPGT_PROJ(4, 2, false); else SPGT_PROJ(4, 0, false); }
     }
 #undef SPGT_PROJ
     return check_launch(who);

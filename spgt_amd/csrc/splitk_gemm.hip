@@ -68,10 +68,13 @@ __device__ __forceinline__ float read_tile(const float* __restrict__ Xs, int lan
 
 // grid (tiles_m * tiles_n, nsplit, batch), block 256.
 // partial[((batch * ntile + tile) * nsplit + split) * 1024 + i * 32 + j]
-template <bool AKC, bool BKC>
+// DIRECT (one K range per tile, the small-K case): the tile goes straight to C (`partial` is C then), scaled by
+// alpha, row-major or column-major, and no workspace is involved.
+template <bool AKC, bool BKC, bool DIRECT = false>
 __global__ __launch_bounds__(256) void splitk_partial(
     const float* __restrict__ A, const float* __restrict__ B, float* __restrict__ partial, int M, int N,
-    int K, int64_t a_stride, int64_t b_stride, int split_len) {
+    int K, int64_t a_stride, int64_t b_stride, int split_len, int64_t c_stride = 0, float alpha = 1.f,
+    int c_col = 0) {
     __shared__ float smem[2][2][kTileFloats];  // [buffer][A|B]
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
@@ -126,6 +129,24 @@ __global__ __launch_bounds__(256) void splitk_partial(
         red[wave * 1024 + i * 32 + (lane & 31)] = acc[r];
     }
     __syncthreads();
+    if constexpr (DIRECT) {
+        float* Cb = partial + (int64_t)batch * c_stride;
+        // thread = four consecutive elements along C's contiguous axis
+        const int major = threadIdx.x >> 3;       // row i (row-major C) or column j (column-major C)
+        const int minor = (threadIdx.x & 7) * 4;  // first of the four columns j or rows i
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+            const int i = c_col ? minor + x : major;
+            const int j = c_col ? major : minor + x;
+            const int e1 = i * 32 + j;
+            const float v = (((red[e1] + red[1024 + e1]) + red[2048 + e1]) + red[3072 + e1]) * alpha;
+            if (m0 + i < M && n0 + j < N) {
+                if (c_col) Cb[(int64_t)(n0 + j) * M + m0 + i] = v;
+                else Cb[(int64_t)(m0 + i) * N + n0 + j] = v;
+            }
+        }
+        return;
+    }
     float* dst = partial + (((int64_t)batch * gridDim.x + tile) * nsplit + split) * 1024;
     const int e = threadIdx.x * 4;
     const float4 w0 = *reinterpret_cast<const float4*>(red + e);
@@ -271,4 +292,32 @@ extern "C" int spgt_batched_skinny_gemm(const float* A, const float* B, float* C
     launch_splitk(A, B, C, alpha, M, N, K, a_stride, b_stride, c_stride, order, batch_count,
                   static_cast<float*>(workspace), stream);
     return check_launch("batched_skinny_gemm");
+}
+
+extern "C" int spgt_batched_small_k_gemm(const float* A, const float* B, float* C, float alpha, int M, int N, int K,
+                                         int64_t a_stride, int64_t b_stride, int64_t c_stride, int order,
+                                         int batch_count, hipStream_t stream) {
+    if (!A || !B || !C) return fail(SPGT_ERR_INVALID_ARGUMENT, "batched_small_k_gemm: null pointer argument");
+    if (M <= 0 || N <= 0 || K <= 0 || batch_count <= 0)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "batched_small_k_gemm: M, N, K, batch_count must be positive");
+    if (order < 0 || order > 7) return fail(SPGT_ERR_INVALID_ARGUMENT, "batched_small_k_gemm: unknown operand order");
+    if (batch_count > 65535) return fail(SPGT_ERR_INVALID_ARGUMENT, "batched_small_k_gemm: batch_count exceeds 65535");
+    if (!aligned4(A) || !aligned4(B) || !aligned4(C))
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "batched_small_k_gemm: operands must be 4-byte aligned");
+    const int64_t ntile = (int64_t)ceil_div(M, 32) * ceil_div(N, 32);
+    if (ntile >= ((int64_t)1 << 31)) return fail(SPGT_ERR_INVALID_ARGUMENT, "batched_small_k_gemm: too many tiles");
+    const bool a_kc = (order & 4) == 0;
+    const bool b_kc = (order & 2) != 0;
+    const int c_col = order & 1;
+    const dim3 grid((unsigned)ntile, 1, batch_count);
+    const int split_len = ceil_div(K, kKT) * kKT;  // one K range
+#define SPGT_LAUNCH_DIRECT(AK, BK)                                                                              \
+    hipLaunchKernelGGL((splitk_partial<AK, BK, true>), grid, dim3(256), 0, stream, A, B, C, M, N, K, a_stride, \
+                       b_stride, split_len, c_stride, alpha, c_col)
+    if (a_kc && b_kc) SPGT_LAUNCH_DIRECT(true, true);
+    else if (a_kc && !b_kc) SPGT_LAUNCH_DIRECT(true, false);
+    else if (!a_kc && b_kc) SPGT_LAUNCH_DIRECT(false, true);
+    else SPGT_LAUNCH_DIRECT(false, false);
+#undef SPGT_LAUNCH_DIRECT
+    return check_launch("batched_small_k_gemm");
 }

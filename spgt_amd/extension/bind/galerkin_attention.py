@@ -148,14 +148,46 @@ def _projection_backward(grad_out: Tensor, input: Tensor, weight: Tensor, seqlen
     return _linear_backward(g, input, weight)
 
 
+def _projection_layernorm_backward_from_output(grad_ln: Tensor, input: Tensor, weight: Tensor, hat_ln: Tensor,
+                                               invsigma: Tensor, lnw: Tensor, lnb: Tensor, seqlen: int,
+                                               dim_hidden: int, num_head: int, dim_head: int, dim_position: int,
+                                               batch: int):
+    """-> (dX, dW, db, dgamma, dbeta) with the reference's own arguments
+    (extension/bind/galerkin_attention.cu:70-102; extension/native/multihead_dim32.cu:148-271): the normalised
+    values are recovered from the saved LayerNorm output as x_hat = (hat_ln - beta) / gamma and the reciprocal
+    standard deviations are taken from invsigma [batch, num_head, seqlen].  Where a gamma is zero x_hat cannot be
+    recovered: the reference divides by zero there, this function uses x_hat = 0 (exact for dgamma's other entries,
+    dbeta, and the part of dX, dW, db that does not pass through that feature's x_hat).  The autograd function of
+    this package uses the recomputing form below instead and has no such case."""
+    for name, t in (("hat_ln", hat_ln), ("invsigma", invsigma), ("lnw", lnw), ("lnb", lnb)):
+        require_gpu_f32(name, t)
+    if tuple(invsigma.shape) != (batch, num_head, seqlen):
+        raise ValueError(f"invsigma has shape {tuple(invsigma.shape)}, expected {(batch, num_head, seqlen)}")
+    g = _heads_feature_to_token_major(grad_ln, batch, num_head, dim_position, dim_head, seqlen)
+    y = _heads_feature_to_token_major(hat_ln, batch, num_head, dim_position, dim_head, seqlen)
+    g = g.view(batch, seqlen, num_head, dim_head)
+    y = y.view(batch, seqlen, num_head, dim_head)
+    gamma, beta = lnw.view(1, 1, num_head, dim_head), lnb.view(1, 1, num_head, dim_head)
+    x_hat = torch.where(gamma != 0, (y - beta) / torch.where(gamma != 0, gamma, torch.ones_like(gamma)),
+                        torch.zeros_like(y))
+    dxh = g * gamma
+    inv = invsigma.permute(0, 2, 1).unsqueeze(-1)  # [batch, seqlen, num_head, 1]
+    grad_pre = inv * (dxh - dxh.mean(-1, keepdim=True) - x_hat * (dxh * x_hat).mean(-1, keepdim=True))
+    grad_lnw = (g * x_hat).sum(dim=(0, 1))
+    grad_lnb = g.sum(dim=(0, 1))
+    grad_input, grad_weight, grad_bias = _linear_backward(grad_pre.reshape(batch, seqlen, dim_hidden), input, weight)
+    return grad_input, grad_weight, grad_bias, grad_lnw, grad_lnb
+
+
 def _projection_layernorm_backward(grad_ln: Tensor, input: Tensor, weight: Tensor, bias: Tensor, lnw: Tensor,
                                    norm_eps: float, seqlen: int, dim_hidden: int, num_head: int, dim_head: int,
                                    dim_position: int, batch: int):
-    """-> (dX, dW, db, dgamma, dbeta) (reference: extension/bind/galerkin_attention.cu:70-102).
+    """-> (dX, dW, db, dgamma, dbeta): what the autograd function of this package calls.
 
-    Unlike the reference, which recovers x_hat from the saved LayerNorm output as (y - beta) / gamma and
-    therefore fails when a gamma is zero, the pre-LayerNorm projection is recomputed from input, weight
-    and bias; that is why `bias` and `norm_eps` are arguments here and hat_ln / invsigma are not."""
+    Unlike the reference (see _projection_layernorm_backward_from_output), which recovers x_hat from the saved
+    LayerNorm output as (y - beta) / gamma and therefore fails when a gamma is zero, the pre-LayerNorm projection
+    is recomputed from input, weight and bias; that is why `bias` and `norm_eps` are arguments here and hat_ln /
+    invsigma are not."""
     require_gpu_f32("lnw", lnw)
     g = _heads_feature_to_token_major(grad_ln, batch, num_head, dim_position, dim_head, seqlen)
     pre = torch.addmm(bias, input.reshape(-1, dim_hidden), weight)
@@ -342,7 +374,8 @@ gexts = SimpleNamespace(
     multihead_projection_with_position_rrc_forward=_projection_forward,
     multihead_projection_with_position_rrc_backward=_projection_backward,
     multihead_projection_layernorm_with_position_rrc_forward=_projection_layernorm_forward,
-    multihead_projection_layernorm_with_position_rrc_backward=_projection_layernorm_backward,
+    multihead_projection_layernorm_with_position_rrc_backward=_projection_layernorm_backward_from_output,
+    multihead_projection_layernorm_with_position_rrc_backward_recompute=_projection_layernorm_backward,
     multihead_galerkin_attention_cccr_backward=_attention_cccr_backward,
     heads_feature_to_token_major=_heads_feature_to_token_major,
     galerkin_attention_fused_profile=_attention_fused_profile,
@@ -397,7 +430,7 @@ class Multihead_Porjection_Layernorm_with_Position_Function(torch.autograd.Funct
         input, weight, bias, lnw = ctx.saved_tensors
         num_head, dim_head, dim_position = ctx.shape_kwargs
         batch, seqlen, d_model = input.size()
-        grads = gexts.multihead_projection_layernorm_with_position_rrc_backward(
+        grads = gexts.multihead_projection_layernorm_with_position_rrc_backward_recompute(
             grad_ln, input, weight, bias, lnw, ctx.norm_eps, seqlen, d_model, num_head, dim_head, dim_position, batch)
         return (*grads, None, None, None, None, None)
 

@@ -32,7 +32,7 @@ from ..extension.bind.galerkin_attention import (fold_ktv_into_fc, galerkin_atte
                                                  multihead_projection_with_position_rrc_cuda)
 from . import truncated_dft
 from ..extension.bind.linear import (encoder_tail_supported, fused_encoder_tail, fused_encoder_tail_folded,
-                                     fused_linear)
+                                     fused_linear, linear_supported)
 from .derived import derived, refreshes_derived
 from .layer import (FeedForward, activation_name, always_dropout, fused_linear_usable, gpu_inference,
                     linear_weight_kn, make_activation)
@@ -43,6 +43,13 @@ class Sp_GalerkinAttention(nn.Module):
                  symmetric) -> None:
         super().__init__()
         assert dim_hidden % 128 == 0 and dim_hidden // num_head == 32
+        if dim_position not in (0, 2):
+            # the reference's position kernel is written for two coordinates and skips the case of none
+            # (extension/native/multihead_dim32.cu:6-22, 593-598); any other value corrupts memory there
+            raise ValueError(f"dim_position must be 0 or 2 (got {dim_position})")
+        if dim_hidden > 512:
+            raise ValueError(f"dim_hidden must be 128, 256, 384 or 512 (got {dim_hidden}): the projection operators "
+                             "keep a head's weight columns in registers")
         self.dim_hidden = dim_hidden
         self.num_head = num_head
         self.dim_head = dim_hidden // num_head
@@ -114,13 +121,16 @@ class Sp_GalerkinAttention(nn.Module):
             X = multihead_galerkin_attention_cccr_cuda(q, k, v)
             X = X.transpose(1, 2).contiguous().view(N, seqlen, H * (dp + self.dim_head))
         else:
-            if Q is K and K is V:
+            if Q is K and K is V and linear_supported(C, 3 * C):
                 # one launch over [W_Q | W_K | W_V] with the bias in its epilogue; the three projections land
                 # in contiguous planes (the attention passes run 15 % faster on unit-stride rows)
                 w, b = self._packed_qkv()
                 q, k, v = fused_linear(Q.reshape(N * seqlen, C), w, b, planes=3).view(3, N, seqlen, C).unbind(0)
             else:
-                proj = lambda x, w, b: fused_linear(x.reshape(N * seqlen, C), w.detach(), b.detach()).view(N, seqlen, C)
+                if linear_supported(C, C):
+                    proj = lambda x, w, b: fused_linear(x.reshape(N * seqlen, C), w.detach(), b.detach()).view(N, seqlen, C)
+                else:  # wider models than the fused linear kernel serves: the library GEMM, then the fused core
+                    proj = lambda x, w, b: torch.addmm(b.detach(), x.reshape(N * seqlen, C), w.detach()).view(N, seqlen, C)
                 q, k, v = (proj(Q, self.weight_Q, self.bias_Q), proj(K, self.weight_K, self.bias_K),
                            proj(V, self.weight_V, self.bias_V))
             pos = position.contiguous() if dp else None

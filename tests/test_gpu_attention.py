@@ -190,6 +190,36 @@ def test_skinny_gemm_orders_and_shapes(gpu, order):
         assert max_rel(got.cpu().double(), want) < 1e-5, (order, b, M, N, K)
 
 
+def small_k_gemm_any_order(A, B, alpha, order):
+    """As skinny_gemm_any_order through spgt_batched_small_k_gemm (one launch, no workspace)."""
+    lib = _lib.load()
+    b, M, K = A.shape
+    N = B.shape[-1]
+    a_mem = A.contiguous() if order[0] == "R" else A.transpose(1, 2).contiguous()
+    b_mem = B.contiguous() if order[1] == "R" else B.transpose(1, 2).contiguous()
+    c_mem = torch.full((b, M * N), float("nan"), device=A.device)
+    _lib.check(lib.spgt_batched_small_k_gemm(
+        _lib.ptr(a_mem), _lib.ptr(b_mem), _lib.ptr(c_mem), alpha, M, N, K, M * K, K * N, M * N,
+        ga.GEMM_ORDER[order], b, _lib.stream_of(A)))
+    return c_mem.view(b, M, N) if order[2] == "R" else c_mem.view(b, N, M).transpose(1, 2)
+
+
+@pytest.mark.parametrize("order", ORDERS)
+def test_small_k_gemm_orders_and_shapes(gpu, order):
+    """The reference's small-K batched GEMM (extension/native/sgemm_32x32.cu:683-710) in all eight operand orders:
+    long M with K = d (the Q M product), long N (the backward's products), ragged tiles, K beyond one step."""
+    shapes = [(1, 1, 1, 1), (2, 5041, 34, 34), (3, 32, 777, 32), (2, 100, 65, 48), (1, 33, 31, 7), (2, 64, 64, 130),
+              (4, 1000, 32, 32)]
+    for n, (b, M, N, K) in enumerate(shapes):
+        A, B = rnd(b, M, K, seed=140 + n), rnd(b, K, N, seed=160 + n)
+        want = O.op_batched_skinny_gemm(A.double(), B.double(), 0.25)
+        got = small_k_gemm_any_order(A.to(gpu), B.to(gpu), 0.25, order)
+        assert not torch.isnan(got).any(), (order, b, M, N, K)
+        assert max_rel(got.cpu().double(), want) < 1e-5, (order, b, M, N, K)
+        again = small_k_gemm_any_order(A.to(gpu), B.to(gpu), 0.25, order)
+        assert torch.equal(got, again)
+
+
 def test_skinny_gemm_every_k(gpu):
     """K around every tile/step boundary (the reference's split heuristic can start a split beyond K)."""
     for K in list(range(1, 140)) + [255, 256, 257, 4095, 4096, 4097, 4999]:

@@ -62,6 +62,30 @@ def test_projection_layernorm_backward(gpu, dp, B, S):
         assert max_rel(got.grad.cpu().double(), want.grad) < TOL, name
 
 
+@pytest.mark.parametrize("dp", [0, 2])
+def test_projection_layernorm_backward_with_the_reference_arguments(gpu, dp):
+    """The pybind-level backward as the reference declares it (extension/bind/galerkin_attention.cu:70-102):
+    (grad_ln, input, weight, hat_ln, invsigma, lnw, lnb, ints...) -> (dX, dW, db, dgamma, dbeta), with hat_ln and
+    invsigma as the forward operator returned them; against autograd through the oracle in float64."""
+    B, S, Dm, H = 2, 333, 128, 4
+    X, W, b = rnd(B, S, Dm, seed=30), rnd(Dm, Dm, seed=31) / Dm ** 0.5, rnd(Dm, seed=32)
+    g, be = 1 + 0.3 * rnd(H, 32, seed=33), 0.2 * rnd(H, 32, seed=34)
+    pos = torch.rand(B, S, dp, generator=torch.Generator().manual_seed(35))
+    G = rnd(B, H, dp + 32, S, seed=36)
+    leaves = [t.double().requires_grad_(True) for t in (X, W, b, g, be)]
+    y, _ = O.op_projection_layernorm_rrc(*leaves, pos.double(), 1e-6, H, 32)
+    y.backward(G.double())
+    d = lambda t: t.to(gpu)
+    hat_ln, invsigma = ga.gexts.multihead_projection_layernorm_with_position_rrc_forward(
+        d(X), d(W), d(b), d(g), d(be), 1e-6, d(pos), S, Dm, H, 32, dp, B)
+    grads = ga.gexts.multihead_projection_layernorm_with_position_rrc_backward(
+        d(G), d(X), d(W), hat_ln, invsigma, d(g), d(be), S, Dm, H, 32, dp, B)
+    assert len(grads) == 5
+    for got, want, name in zip(grads, leaves, ("dX", "dW", "db", "dgamma", "dbeta")):
+        assert got.shape == want.shape, name
+        assert max_rel(got.cpu().double(), want.grad) < TOL, name
+
+
 def test_heads_feature_to_token_major(gpu):
     B, H, dp, S = 2, 4, 2, 333
     src = rnd(B, H, dp + 32, S, seed=17)

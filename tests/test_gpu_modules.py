@@ -319,3 +319,37 @@ def test_graphed_inference_follows_in_place_weight_updates(gpu):
         torch.cuda.synchronize()
         assert rel_l2(want.cpu(), before.cpu()) > 1e-2
         assert rel_l2(got.cpu(), want.cpu()) < TOL, f"replay after update {step} used stale weights"
+
+
+@pytest.mark.parametrize("dim_hidden,dp", [(256, 2), (384, 0), (512, 2)])
+def test_attention_module_wider_models(gpu, dim_hidden, dp):
+    """dim_hidden beyond 128 (the reference accepts any multiple of 128 with heads of 32, network/sp_layer.py:17):
+    the inference path (library GEMM where the fused linear kernel has no variant, then the fused core), the
+    packed self-attention form and the operator sequence under autograd, against the oracle in float64."""
+    torch.manual_seed(9)
+    H = dim_hidden // 32
+    m = L.Sp_GalerkinAttention(dim_hidden, H, dp, 1e-6, 0.0, 0.0, 0.7, 0.01, False)
+    with torch.no_grad():
+        for prm in m.parameters():
+            prm.add_(0.05 * torch.randn_like(prm))
+    sd = {k: v.detach().double() for k, v in m.state_dict().items()}
+    po = {k: (v.t() if k in ("weight_Q", "weight_K", "weight_V") else v) for k, v in sd.items()}
+    B, S = 2, 301
+    x = torch.randn(B, S, dim_hidden)
+    pos = torch.rand(B, S, max(dp, 1))[:, :, :dp]
+    want = O.attention_module(po, x.double(), x.double(), x.double(), pos.double(), H, 1e-6)
+    m = m.to(gpu).eval()
+    xg, pg = x.to(gpu), pos.to(gpu)
+    with torch.no_grad():
+        packed = m(xg, xg, xg, pg)
+        separate = m(xg, xg.clone(), xg.clone(), pg)
+    operators = m(xg, xg, xg, pg)  # autograd on: projection operators + attention operator
+    for got, name in ((packed, "packed"), (separate, "separate"), (operators.detach(), "operators")):
+        assert max_rel(got.cpu().double(), want) < TOL, name
+
+
+def test_unsupported_shapes_are_rejected_at_construction():
+    with pytest.raises(ValueError):
+        L.Sp_GalerkinAttention(128, 4, 1, 1e-6, 0.0, 0.0, 1.0, 0.0, False)
+    with pytest.raises(ValueError):
+        L.Sp_GalerkinAttention(640, 20, 0, 1e-6, 0.0, 0.0, 1.0, 0.0, False)

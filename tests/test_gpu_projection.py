@@ -17,7 +17,8 @@ def rnd(*shape, seed=0):
 
 
 @pytest.mark.parametrize("dp", [0, 2])
-@pytest.mark.parametrize("B,S,Dm", [(1, 1, 128), (2, 50, 128), (1, 777, 128), (3, 4099, 128), (2, 130, 256)])
+@pytest.mark.parametrize("B,S,Dm", [(1, 1, 128), (2, 50, 128), (1, 777, 128), (3, 4099, 128), (2, 130, 256),
+                                    (2, 97, 384), (1, 333, 512)])
 def test_projection_vs_oracle(gpu, dp, B, S, Dm):
     H = Dm // 32
     x, W, b = rnd(B, S, Dm, seed=1), rnd(Dm, Dm, seed=2) / Dm ** 0.5, rnd(Dm, seed=3)
@@ -32,7 +33,8 @@ def test_projection_vs_oracle(gpu, dp, B, S, Dm):
 
 
 @pytest.mark.parametrize("dp", [0, 2])
-@pytest.mark.parametrize("B,S,Dm", [(1, 1, 128), (2, 50, 128), (1, 777, 128), (3, 4099, 128), (2, 130, 256)])
+@pytest.mark.parametrize("B,S,Dm", [(1, 1, 128), (2, 50, 128), (1, 777, 128), (3, 4099, 128), (2, 130, 256),
+                                    (2, 97, 384), (1, 333, 512)])
 def test_projection_layernorm_vs_oracle(gpu, dp, B, S, Dm):
     H = Dm // 32
     x, W, b = rnd(B, S, Dm, seed=5), rnd(Dm, Dm, seed=6) / Dm ** 0.5, rnd(Dm, seed=7)
