@@ -105,7 +105,7 @@ def darcy_config():
         num_frequence_mode=12, drop_decoder_layer=0.0, acti_decoder_layer="silu")
 
 
-def darcy_bench(dev, with_cpu, steps=30):
+def darcy_bench(dev, with_cpu, steps=30, graph=True):
     """End-to-end Darcy inference, B=4, random init: samples/s on the GPU and, beside it, the CPU oracle."""
     import torch
     from spgt_amd.network import sp_model as SM
@@ -128,6 +128,9 @@ def darcy_bench(dev, with_cpu, steps=30):
             out = model(ad, pd, gd)
         torch.cuda.synchronize()
         eager_ms = (time.perf_counter() - t0) / steps * 1e3
+        if not graph:
+            return {"ms_per_forward": round(eager_ms, 3), "samples_per_s": round(B / eager_ms * 1e3, 1), "batch": B,
+                    "mode": "eager launches"}
         # the same forward replayed from a HIP graph: the coefficient field is copied into the captured buffer on
         # every call (a second tensor keeps that copy inside the timed region); the position and grid inputs are
         # constants of the model's resolution and live in the captured buffers
@@ -470,6 +473,9 @@ def main():
     ap.add_argument("--input-sets", type=int, default=3,
                     help="independent (Q, K, V) sets the timed steps rotate through")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--only", choices=["kernels", "darcy"], default=None,
+                    help="profiling aid: run only the per-kernel table (every operator of the path at its benchmark "
+                         "shape) or only a few end-to-end Darcy forwards, and print that part as JSON")
     ap.add_argument("--no-extra", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy (a kernel of known traffic, for scaling "
@@ -485,6 +491,14 @@ def main():
         sys.exit("bench.py needs a GPU (the HIP path has no CPU fallback)")
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+
+    if args.only == "kernels":
+        print(json.dumps({"kernel_rooflines": kernel_rooflines(dev)}))
+        return
+    if args.only == "darcy":
+        print(json.dumps({"darcy_inference": darcy_bench(dev, with_cpu=False, steps=max(1, min(args.steps, 20)),
+                                                         graph=False)}))
+        return
 
     B, S, H, dp = 8, 44521, 4, 0
     g = torch.Generator(device=dev).manual_seed(0)
