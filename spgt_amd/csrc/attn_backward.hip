@@ -8,7 +8,7 @@
 // With M = K V^T / S and N = Q G / S (both D x D; G = grad_out, token-major [S, D]):
 //   dQ[i][s] = sum_j M[i][j] G[s][j]      dK[i][s] = sum_j N[i][j] V[j][s]      dV[j][s] = sum_i N[i][j] K[i][s]
 // The two D x D matrices come from the split-K kernels of the forward pass; the
-// three products above are `apply_to_fm`: out[n][s] = sum_k W[n][k] X(k, s) with a
+// three products above are `apply_to_fm_v4`: out[n][s] = sum_k W[n][k] X(k, s) with a
 // feature-major [D, S] result (stores run along the contiguous sequence axis).
 //
 // LayerNorm backward differs from the reference in one point on purpose: it
@@ -22,14 +22,17 @@ namespace spgt {
 
 // out[bh][n][s] = sum_k W[bh][n*wn + k*wk] * X(k, s)
 //   X_TM == false: X is feature-major [D, S];  X_TM == true: X is token-major [S, D].
-// grid (nchunk, BH), block 256: each wave owns runs of 32 tokens.
-// Lane l: token l%32, contraction half kh = l/32.  MFMA step kk contracts the two
-// contraction indices kidx(kk, 0) and kidx(kk, 1).
+// Lane l of a wave: contraction half kh = l/32; MFMA step kk contracts the two contraction indices kidx(kk, 0) and
+// kidx(kk, 1).  Four consecutive tokens per lane: 16-byte accesses along the sequence axis on the
+// feature-major side(s), 512-byte runs per row and wave instruction.  A wave takes blocks of 128 tokens; lane
+// (tk, kh) holds tokens 4 tk .. 4 tk + 3, four accumulators (one per token of the lane) share the weight operand.
+// The chunk's last, partial block goes 32 tokens per wave with word accesses.
+// grid (nchunk, BH), block 256.
 template <int D, bool X_TM>
-__global__ __launch_bounds__(256) void apply_to_fm(const float* __restrict__ W, int wn, int wk,
-                                                   const float* __restrict__ X, float* __restrict__ out, int S,
-                                                   int tokens_per_chunk) {
-    constexpr int NK = D / 2;  // 16 or 17 MFMA steps
+__global__ __launch_bounds__(256) void apply_to_fm_v4(const float* __restrict__ W, int wn, int wk,
+                                                      const float* __restrict__ X, float* __restrict__ out, int S,
+                                                      int tokens_per_chunk) {
+    constexpr int NK = D / 2;
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int tk = lane & 31;
@@ -37,12 +40,12 @@ __global__ __launch_bounds__(256) void apply_to_fm(const float* __restrict__ W, 
     const int64_t bh = blockIdx.y;
     const int s0 = blockIdx.x * tokens_per_chunk;
     const int s1 = min(S, s0 + tokens_per_chunk);
-    // contraction index of MFMA step kk for this lane's half
+    const int nblk = (s1 - s0) / 128;  // whole blocks of this chunk
     auto kidx = [&](int kk) { return X_TM ? (NK * kh + kk) : (2 * kk + kh); };
 
     const float* w = W + bh * (D * D);
-    float wreg[NK];       // A operand: rows n = 0..31
-    float wext[NK][2];    // rows 32, 33 (D == 34)
+    float wreg[NK];
+    float wext[NK][2];
 #pragma unroll
     for (int kk = 0; kk < NK; ++kk) {
         wreg[kk] = w[tk * wn + kidx(kk) * wk];
@@ -54,10 +57,77 @@ __global__ __launch_bounds__(256) void apply_to_fm(const float* __restrict__ W, 
     const float* Xb = X + bh * D * (int64_t)S;
     float* ob = out + bh * D * (int64_t)S;
 
-    // Two register buffers in ping-pong: the loads of the next 32-token block are issued (clamped to
-    // the chunk, so unconditionally) before the MFMAs and stores of the current one.
-    auto load_block = [&](float (&x)[NK], int sb) {
-        const int sl = min(sb + tk, s1 - 1);
+    // x[kk][e]: contraction index kidx(kk), token 4 tk + e of the block
+    auto load_block = [&](float (&x)[NK][4], int blk) {
+        const int sb = s0 + 128 * min(blk, nblk - 1) + 4 * tk;
+        if (X_TM) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float* row = Xb + (int64_t)(sb + e) * D + NK * kh;
+#pragma unroll
+                for (int kk = 0; kk < NK; ++kk) x[kk][e] = row[kk];
+            }
+        } else {
+#pragma unroll
+            for (int kk = 0; kk < NK; ++kk) {
+                const v4f v = *reinterpret_cast<const v4f_a4*>(Xb + (int64_t)(2 * kk + kh) * S + sb);
+                x[kk][0] = v.x; x[kk][1] = v.y; x[kk][2] = v.z; x[kk][3] = v.w;
+            }
+        }
+    };
+    auto compute_block = [&](const float (&x)[NK][4], int blk) {
+        const int sb = s0 + 128 * blk + 4 * tk;
+        v16f acc[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[e][r] = 0.f;
+#pragma unroll
+        for (int kk = 0; kk < NK; ++kk)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[e] = mfma32(wreg[kk], x[kk][e], acc[e]);
+        float e0[4] = {0.f, 0.f, 0.f, 0.f}, e1[4] = {0.f, 0.f, 0.f, 0.f};
+        if (D == 34) {
+#pragma unroll
+            for (int kk = 0; kk < NK; ++kk)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    e0[e] = fmaf(wext[kk][0], x[kk][e], e0[e]);
+                    e1[e] = fmaf(wext[kk][1], x[kk][e], e1[e]);
+                }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                e0[e] += __shfl_xor(e0[e], 32, 64);
+                e1[e] += __shfl_xor(e1[e], 32, 64);
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int n = 8 * (r >> 2) + 4 * kh + (r & 3);
+            *reinterpret_cast<v4f_a4*>(ob + (int64_t)n * S + sb) = v4f{acc[0][r], acc[1][r], acc[2][r], acc[3][r]};
+        }
+        if (D == 34)
+            *reinterpret_cast<v4f_a4*>(ob + (int64_t)(32 + kh) * S + sb) =
+                kh == 0 ? v4f{e0[0], e0[1], e0[2], e0[3]} : v4f{e1[0], e1[1], e1[2], e1[3]};
+    };
+    float xa[NK][4], xb[NK][4];
+    int blk = wave;
+    if (blk < nblk) load_block(xa, blk);
+    for (; blk < nblk; blk += 8) {
+        load_block(xb, blk + 4);
+        __builtin_amdgcn_sched_barrier(0);
+        compute_block(xa, blk);
+        __builtin_amdgcn_sched_barrier(0);
+        load_block(xa, blk + 8);
+        __builtin_amdgcn_sched_barrier(0);
+        if (blk + 4 < nblk) compute_block(xb, blk + 4);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    // the chunk's last, partial block (only the last chunk of a sequence has one): 32 tokens per wave, word accesses
+    const int st = s0 + 128 * nblk + 32 * wave + tk;
+    if (s0 + 128 * nblk + 32 * wave < s1) {
+        const int sl = min(st, s1 - 1);
+        float x[NK];
         if (X_TM) {
             const float* row = Xb + (int64_t)sl * D + NK * kh;
 #pragma unroll
@@ -66,46 +136,29 @@ __global__ __launch_bounds__(256) void apply_to_fm(const float* __restrict__ W, 
 #pragma unroll
             for (int kk = 0; kk < NK; ++kk) x[kk] = Xb[(int64_t)(2 * kk + kh) * S + sl];
         }
-    };
-    auto compute_block = [&](const float (&x)[NK], int sb) {
-        const int s = sb + tk;
-        const bool valid = s < s1;
         v16f acc;
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[r] = 0.f;
 #pragma unroll
         for (int kk = 0; kk < NK; ++kk) acc = mfma32(wreg[kk], x[kk], acc);
-        float e0 = 0.f, e1 = 0.f;
+        float t0 = 0.f, t1 = 0.f;
         if (D == 34) {
 #pragma unroll
             for (int kk = 0; kk < NK; ++kk) {
-                e0 = fmaf(wext[kk][0], x[kk], e0);
-                e1 = fmaf(wext[kk][1], x[kk], e1);
+                t0 = fmaf(wext[kk][0], x[kk], t0);
+                t1 = fmaf(wext[kk][1], x[kk], t1);
             }
-            e0 += __shfl_xor(e0, 32, 64);
-            e1 += __shfl_xor(e1, 32, 64);
+            t0 += __shfl_xor(t0, 32, 64);
+            t1 += __shfl_xor(t1, 32, 64);
         }
-        if (valid) {
+        if (st < s1) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int n = 8 * (r >> 2) + 4 * kh + (r & 3);
-                ob[(int64_t)n * S + s] = acc[r];
+                ob[(int64_t)n * S + st] = acc[r];
             }
-            if (D == 34) ob[(int64_t)(32 + kh) * S + s] = kh == 0 ? e0 : e1;
+            if (D == 34) ob[(int64_t)(32 + kh) * S + st] = kh == 0 ? t0 : t1;
         }
-    };
-    float xa[NK], xb[NK];
-    int sb = s0 + 32 * wave;
-    if (sb < s1) load_block(xa, sb);
-    for (; sb < s1; sb += 256) {
-        load_block(xb, sb + 128);
-        __builtin_amdgcn_sched_barrier(0);
-        compute_block(xa, sb);
-        __builtin_amdgcn_sched_barrier(0);
-        load_block(xa, sb + 256);
-        __builtin_amdgcn_sched_barrier(0);
-        if (sb + 128 < s1) compute_block(xb, sb + 128);
-        __builtin_amdgcn_sched_barrier(0);
     }
 }
 
@@ -236,6 +289,8 @@ BwdPlan make_bwd_plan(int bh, int D, int S) {
 namespace spgt {
 int launch_ktv_fm(const float* K, const float* V, float* m, float* partial, int bh, int D, int S, int tpc, int nchunk,
                   hipStream_t stream);
+int launch_qg_fm(const float* Q, const float* G, float* n, float* partial, int bh, int D, int S, int tpc, int nchunk,
+                 hipStream_t stream);
 size_t ktv_fm_partial_bytes(int bh, int D, int nchunk);
 }  // namespace spgt
 
@@ -245,8 +300,7 @@ extern "C" size_t spgt_galerkin_attention_cccr_backward_workspace_bytes(int batc
     const int bh = batch * num_head;
     const BwdPlan p = make_bwd_plan(bh, d_posk, seqlen);
     const size_t part_m = ktv_fm_partial_bytes(bh, d_posk, p.nchunk1);
-    const size_t part_n = spgt_batched_skinny_gemm_workspace_bytes(d_posk, d_posk, seqlen, bh);
-    return p.bytes + round256(std::max(part_m, part_n));
+    return p.bytes + round256(part_m);  // the two reductions use the partial-tile space one after the other
 }
 
 extern "C" int spgt_galerkin_attention_cccr_backward(const float* grad_out, const float* Q, const float* K,
@@ -273,28 +327,25 @@ extern "C" int spgt_galerkin_attention_cccr_backward(const float* grad_out, cons
     float* m = reinterpret_cast<float*>(ws + p.off_m);      // M[i][j] = sum_t K[i,t] V[j,t] / S, row-major
     float* n = reinterpret_cast<float*>(ws + p.off_n);      // N[i][j] = sum_t Q[i,t] G[t,j] / S, row-major
     float* partial = reinterpret_cast<float*>(ws + p.off_partial);
-    const float inv = 1.0f / (float)S;
-    const int64_t xs = (int64_t)D * S;
     const dim3 grid2(p.nchunk2, bh);
 
     int rc = launch_ktv_fm(K, V, m, partial, bh, D, S, p.tpc1, p.nchunk1, stream);
     if (rc != SPGT_OK) return rc;
     // dQ = M G^T
     if (D == 32)
-        hipLaunchKernelGGL((apply_to_fm<32, true>), grid2, dim3(256), 0, stream, m, D, 1, grad_out, grad_Q, S, p.tpc2);
+        hipLaunchKernelGGL((apply_to_fm_v4<32, true>), grid2, dim3(256), 0, stream, m, D, 1, grad_out, grad_Q, S, p.tpc2);
     else
-        hipLaunchKernelGGL((apply_to_fm<34, true>), grid2, dim3(256), 0, stream, m, D, 1, grad_out, grad_Q, S, p.tpc2);
+        hipLaunchKernelGGL((apply_to_fm_v4<34, true>), grid2, dim3(256), 0, stream, m, D, 1, grad_out, grad_Q, S, p.tpc2);
     // N = Q G / S   (A = Q [D, S] row-major, B = G [S, D] row-major, C row-major)
-    rc = spgt_batched_skinny_gemm(Q, grad_out, n, inv, D, D, S, xs, xs, (int64_t)D * D, SPGT_ORDER_RRR, bh, partial,
-                                  workspace_bytes - p.off_partial, stream);
+    rc = launch_qg_fm(Q, grad_out, n, partial, bh, D, S, p.tpc1, p.nchunk1, stream);
     if (rc != SPGT_OK) return rc;
     // dK = N V ;  dV = N^T K
     if (D == 32) {
-        hipLaunchKernelGGL((apply_to_fm<32, false>), grid2, dim3(256), 0, stream, n, D, 1, V, grad_K, S, p.tpc2);
-        hipLaunchKernelGGL((apply_to_fm<32, false>), grid2, dim3(256), 0, stream, n, 1, D, K, grad_V, S, p.tpc2);
+        hipLaunchKernelGGL((apply_to_fm_v4<32, false>), grid2, dim3(256), 0, stream, n, D, 1, V, grad_K, S, p.tpc2);
+        hipLaunchKernelGGL((apply_to_fm_v4<32, false>), grid2, dim3(256), 0, stream, n, 1, D, K, grad_V, S, p.tpc2);
     } else {
-        hipLaunchKernelGGL((apply_to_fm<34, false>), grid2, dim3(256), 0, stream, n, D, 1, V, grad_K, S, p.tpc2);
-        hipLaunchKernelGGL((apply_to_fm<34, false>), grid2, dim3(256), 0, stream, n, 1, D, K, grad_V, S, p.tpc2);
+        hipLaunchKernelGGL((apply_to_fm_v4<34, false>), grid2, dim3(256), 0, stream, n, D, 1, V, grad_K, S, p.tpc2);
+        hipLaunchKernelGGL((apply_to_fm_v4<34, false>), grid2, dim3(256), 0, stream, n, 1, D, K, grad_V, S, p.tpc2);
     }
     return check_launch("galerkin_attention_cccr_backward");
 }

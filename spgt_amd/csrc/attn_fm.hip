@@ -154,6 +154,143 @@ __global__ __launch_bounds__(256) void ktv_partial_fm(const float* __restrict__ 
         dst[e] = ((red01[e] + red01[D * D + e]) + red23[e]) + red23[D * D + e];
 }
 
+// The backward's second reduction, N[i][j] = sum_t Q[i][t] G[t][j] with Q feature-major [D, S] and G = grad_out
+// token-major [S, D]: the structure of ktv_partial_fm, with the Q rows staged through LDS as K is there and the
+// G operand read straight from memory (a token's feature row is 128 contiguous bytes: two rows per load
+// instruction), one 128-token stage ahead.  grid (nchunk, BH), block 256.
+template <int D>
+__global__ __launch_bounds__(256) void qg_partial_fm(const float* __restrict__ Q, const float* __restrict__ G,
+                                                     float* __restrict__ partial, int S, int tokens_per_chunk) {
+    constexpr int DP = D - 32;
+    constexpr int RPW = (D + 3) / 4;  // rows per wave in the loader
+    // the Q stage [D][kFmPitch]; at the end the four waves' D x D tiles
+    __shared__ float sq[D * kFmPitch > 4 * D * D ? D * kFmPitch : 4 * D * D];
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int64_t bh = blockIdx.y;
+    const int chunk = blockIdx.x;
+    const int s0 = chunk * tokens_per_chunk;
+    const int s1 = min(S, s0 + tokens_per_chunk);
+    const float* Qb = Q + bh * D * (int64_t)S;
+    const float* Gb = G + bh * D * (int64_t)S;
+
+    v16f acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+    float ck[2] = {0.f, 0.f};   // sum_t Q[DP + lane%32][t] * G[t][a]   -> N[DP+i][a]
+    float rv[2] = {0.f, 0.f};   // sum_t Q[a][t] * G[t][DP + lane%32]   -> N[a][DP+j]
+    float pp[4] = {0.f, 0.f, 0.f, 0.f};  // sum_t Q[a][t] * G[t][a']
+
+    float2 rq[RPW];
+    float gb[16];       // G[t][DP + lane%32] for this lane's 16 tokens of the stage
+    float2 gp[16];      // G[t][0], G[t][1] (D == 34)
+    auto load_step = [&](int sb) {
+        const int s = sb + 2 * lane;
+#pragma unroll
+        for (int i = 0; i < RPW; ++i) {
+            const int row = wave + 4 * i;
+            float2 a = make_float2(0.f, 0.f);
+            if (row < D) {
+                const float* qp = Qb + (int64_t)row * S + s;
+                if (s + 1 < s1) {
+                    const v2f qa = __builtin_nontemporal_load(reinterpret_cast<const v2f_a4*>(qp));
+                    a = make_float2(qa.x, qa.y);
+                } else if (s < s1) {
+                    a.x = qp[0];
+                }
+            }
+            rq[i] = a;
+        }
+#pragma unroll
+        for (int kk = 0; kk < 16; ++kk) {
+            const int t = sb + 32 * wave + 2 * kk + (lane >> 5);
+            const float* gr = Gb + (int64_t)min(t, s1 - 1) * D;
+            const float v = gr[DP + (lane & 31)];
+            gb[kk] = t < s1 ? v : 0.f;
+            if (DP == 2) {
+                const float2 pz = *reinterpret_cast<const float2*>(gr);
+                gp[kk] = t < s1 ? pz : make_float2(0.f, 0.f);
+            }
+        }
+    };
+    auto store_step = [&]() {
+#pragma unroll
+        for (int i = 0; i < RPW; ++i) {
+            const int row = wave + 4 * i;
+            if (row < D) {
+                float* dq = sq + row * kFmPitch + 2 * lane;
+                dq[0] = rq[i].x; dq[1] = rq[i].y;
+            }
+        }
+    };
+
+    if (s0 < s1) load_step(s0);
+    for (int sb = s0; sb < s1; sb += kFmKT) {
+        __syncthreads();  // previous stage fully consumed
+        store_step();
+        float gcur[16];
+        float2 pcur[16];
+#pragma unroll
+        for (int kk = 0; kk < 16; ++kk) {
+            gcur[kk] = gb[kk];
+            if (DP == 2) pcur[kk] = gp[kk];
+        }
+        __syncthreads();
+        if (sb + kFmKT < s1) load_step(sb + kFmKT);
+        const float* aq = sq + (DP + (lane & 31)) * kFmPitch;
+#pragma unroll
+        for (int kk = 0; kk < 16; ++kk) {
+            const int k = 32 * wave + 2 * kk + (lane >> 5);
+            const float a = aq[k];
+            const float b = gcur[kk];
+            acc = mfma32(a, b, acc);
+            if (DP == 2) {
+                const float q0 = sq[k], q1 = sq[kFmPitch + k];
+                const float g0 = pcur[kk].x, g1 = pcur[kk].y;
+                ck[0] = fmaf(a, g0, ck[0]);
+                ck[1] = fmaf(a, g1, ck[1]);
+                rv[0] = fmaf(q0, b, rv[0]);
+                rv[1] = fmaf(q1, b, rv[1]);
+                pp[0] = fmaf(q0, g0, pp[0]);
+                pp[1] = fmaf(q0, g1, pp[1]);
+                pp[2] = fmaf(q1, g0, pp[2]);
+                pp[3] = fmaf(q1, g1, pp[3]);
+            }
+        }
+    }
+    __syncthreads();
+    // Cross-wave sum in wave order through LDS.
+    float* tiles = sq;
+    float* mine = tiles + wave * (D * D);
+    if (DP == 2) {
+#pragma unroll
+        for (int a = 0; a < 2; ++a) {
+            ck[a] += __shfl_xor(ck[a], 32, 64);
+            rv[a] += __shfl_xor(rv[a], 32, 64);
+        }
+#pragma unroll
+        for (int a = 0; a < 4; ++a) pp[a] += __shfl_xor(pp[a], 32, 64);
+    }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const int i = 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        mine[(DP + i) * D + DP + (lane & 31)] = acc[r];
+    }
+    if (DP == 2 && lane < 32) {
+        mine[(DP + lane) * D + 0] = ck[0];
+        mine[(DP + lane) * D + 1] = ck[1];
+        mine[0 * D + DP + lane] = rv[0];
+        mine[1 * D + DP + lane] = rv[1];
+        if (lane == 0) {
+            mine[0] = pp[0]; mine[1] = pp[1]; mine[D] = pp[2]; mine[D + 1] = pp[3];
+        }
+    }
+    __syncthreads();
+    float* dst = partial + (bh * gridDim.x + chunk) * (int64_t)(D * D);
+    for (int e = threadIdx.x; e < D * D; e += 256)
+        dst[e] = ((tiles[e] + tiles[D * D + e]) + tiles[2 * D * D + e]) + tiles[3 * D * D + e];
+}
+
 // grid (nchunk, BH), block 256; every wave owns a contiguous quarter of the chunk.
 // Lane l: token slot tk = l%16 (tokens 4*tk .. 4*tk+3 of a 64-token unit), feature
 // group g = l/16.  M is row-major [D][D] (already scaled by 1/S).
@@ -360,6 +497,18 @@ int launch_ktv_fm(const float* K, const float* V, float* m, float* partial, int 
     else
         hipLaunchKernelGGL((ktv_partial_fm<34>), grid1, dim3(256), 0, stream, K, V, partial, S, tpc);
     hipLaunchKernelGGL(tile_reduce, gridr, dim3(1024), 0, stream, partial, m, D * D, nchunk, 1.0f / (float)S);
+    return SPGT_OK;
+}
+
+// n [bh, D, D] = Q G / S by qg_partial_fm and the fixed-order reduction (the backward's second D x D matrix).
+int launch_qg_fm(const float* Q, const float* G, float* n, float* partial, int bh, int D, int S, int tpc, int nchunk,
+                 hipStream_t stream) {
+    const dim3 grid1(nchunk, bh), gridr(ceil_div(D * D, 256), bh);
+    if (D == 32)
+        hipLaunchKernelGGL((qg_partial_fm<32>), grid1, dim3(256), 0, stream, Q, G, partial, S, tpc);
+    else
+        hipLaunchKernelGGL((qg_partial_fm<34>), grid1, dim3(256), 0, stream, Q, G, partial, S, tpc);
+    hipLaunchKernelGGL(tile_reduce, gridr, dim3(1024), 0, stream, partial, n, D * D, nchunk, 1.0f / (float)S);
     return SPGT_OK;
 }
 

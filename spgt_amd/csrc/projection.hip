@@ -24,7 +24,10 @@
 
 namespace spgt {
 
-constexpr int kProjTile = 32;
+#ifndef SPGT_PROJ_TILE
+#define SPGT_PROJ_TILE 32
+#endif
+constexpr int kProjTile = SPGT_PROJ_TILE;  // tokens per tile (64 = two interleaved sub-tiles: 159 us against 150 us at B=8, S=44521)
 
 // grid (nchunk, H/4, B), block 256.  KC = dim_hidden / 128.
 template <int KC, int DP, bool LN>
@@ -35,7 +38,7 @@ __global__ __launch_bounds__(256) void projection_rrc_k(
     constexpr int K = 128 * KC;
     constexpr int D = DP + 32;
     constexpr int PITCH = K + 1;
-    constexpr int TT = kProjTile;  // tokens per tile
+    constexpr int TT = KC <= 2 ? kProjTile : 32;  // tokens per tile (wide inputs: the staging registers decide)
     extern __shared__ float xs[];  // [TT][PITCH]
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
@@ -94,30 +97,46 @@ __global__ __launch_bounds__(256) void projection_rrc_k(
         store_tile();
         __syncthreads();
         if (s0 + TT < s_end) load_tile(s0 + TT);
+        // TB = TT / 32 sub-tiles of 32 tokens share the weight operand: TB independent accumulator chains, whose
+        // MFMAs alternate, so that none waits for its predecessor's result
+        constexpr int TB = TT / 32;
+        v16f accs[TB];
 #pragma unroll
-        for (int tb = 0; tb < TT / 32; ++tb) {
-            v16f acc;
+        for (int tb = 0; tb < TB; ++tb)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) acc[r] = 0.f;
-            const float* xr = xs + (tb * 32 + tk) * PITCH + kh;
+            for (int r = 0; r < 16; ++r) accs[tb][r] = 0.f;
+        {
+            const float* xr = xs + tk * PITCH + kh;
             // LDS reads for the next batch of MFMAs are issued before the current batch, so their
             // latency hides behind the matrix pipe
-            constexpr int BK = 16;
+            constexpr int BK = 16 / TB;
             constexpr int NB = K / 2 / BK;
-            float xv[2][BK];
+            float xv[2][TB][BK];
 #pragma unroll
-            for (int j = 0; j < BK; ++j) xv[0][j] = xr[2 * j];
+            for (int tb = 0; tb < TB; ++tb)
+#pragma unroll
+                for (int j = 0; j < BK; ++j) xv[0][tb][j] = xr[tb * 32 * PITCH + 2 * j];
 #pragma unroll
             for (int bt = 0; bt < NB; ++bt) {
                 if (bt + 1 < NB) {
 #pragma unroll
-                    for (int j = 0; j < BK; ++j) xv[(bt + 1) & 1][j] = xr[2 * ((bt + 1) * BK + j)];
+                    for (int tb = 0; tb < TB; ++tb)
+#pragma unroll
+                        for (int j = 0; j < BK; ++j)
+                            xv[(bt + 1) & 1][tb][j] = xr[tb * 32 * PITCH + 2 * ((bt + 1) * BK + j)];
                 }
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int j = 0; j < BK; ++j) acc = mfma32(wreg[bt * BK + j], xv[bt & 1][j], acc);
+                for (int j = 0; j < BK; ++j)
+#pragma unroll
+                    for (int tb = 0; tb < TB; ++tb)
+                        accs[tb] = mfma32(wreg[bt * BK + j], xv[bt & 1][tb][j], accs[tb]);
                 __builtin_amdgcn_sched_barrier(0);
             }
+        }
+#pragma unroll
+        for (int tb = 0; tb < TB; ++tb) {
+            const v16f acc = accs[tb];
             const int s = s0 + tb * 32 + tk;
             float y[16];
 #pragma unroll
@@ -159,10 +178,11 @@ void launch_projection(const float* x, const float* W, const float* bias, const 
                        const float* pos, float* out, float* invsigma, int B, int S, int H, float eps,
                        hipStream_t stream) {
     constexpr int K = 128 * KC;
-    const size_t lds = (size_t)kProjTile * (K + 1) * sizeof(float);
+    constexpr int TT = KC <= 2 ? kProjTile : 32;
+    const size_t lds = (size_t)TT * (K + 1) * sizeof(float);
     // about two workgroups per CU; chunks are whole tiles
     const int per_b = std::max(1, 2 * device_cu_count() / std::max(1, B * (H / 4)));
-    const int tpc = std::max(kProjTile, ceil_div(ceil_div(S, per_b), kProjTile) * kProjTile);
+    const int tpc = std::max(TT, ceil_div(ceil_div(S, per_b), TT) * TT);
     const dim3 grid(ceil_div(S, tpc), H / 4, B);
     auto kernel = projection_rrc_k<KC, DP, LN>;
     if (lds > 64 * 1024)
