@@ -220,16 +220,16 @@ int spgt_bilinear_align_corners(const float* src, float* dst, int planes, int H_
 int spgt_bilinear_align_corners_nhwc(const float* src, float* dst, int N, int C, int H_in, int W_in,
                                      int H_out, int W_out, spgt_stream_t stream);
 
-/* 1 when the truncated-DFT row kernels serve this shape (r <= 1024, channels a multiple of 32,
- * modes <= 16), else 0. */
+/* 1 when the truncated-DFT row kernels serve this shape (channels a multiple of 32; modes <= 16 with
+ * r <= 1024, or modes <= 32 with r <= 512), else 0. */
 int spgt_truncated_dft_rows_supported(int r, int channels, int modes);
 
 /* The w-direction of rfft2 restricted to the modes Sp_SpectralConv2D keeps
  * (network/sp_layer.py:136-141: rfft2, then only columns kw < modes are read):
  *   Y[row, c, j] = sum_w x[row, w, c] * table[w, j],   j = (kw, re|im) < 2*modes
  * x [rows, r, channels] (rows = N*r grid rows of the channels-last tensor); table[w, j] =
- * (cos, -sin)(2 pi kw w / r) / sqrt(r), handed over zero-padded to [2*ceil(r/2), 32] (the layout
- * the kernel keeps in LDS, 16-byte aligned).  Y is [rows, channels, 2*modes], or with planar != 0
+ * (cos, -sin)(2 pi kw w / r) / sqrt(r), handed over zero-padded to [2*ceil(r/2), 32], or
+ * [2*ceil(r/2), 64] when 2*modes > 32 (the layout the kernel keeps in LDS, 16-byte aligned).  Y is [rows, channels, 2*modes], or with planar != 0
  * [N, 2*modes, r, channels] (row = n*r + h), the layout spgt_spectral_modes_middle works on. */
 int spgt_truncated_dft_rows_forward(const float* x, const float* table, float* Y, int64_t rows, int r,
                                     int channels, int modes, int planar, spgt_stream_t stream);
@@ -243,8 +243,8 @@ int spgt_truncated_dft_rows_forward(const float* x, const float* table, float* Y
 int spgt_truncated_dft_rows_inverse(const float* U, const float* table, float* y, int64_t rows, int r,
                                     int channels, int modes, int planar, spgt_stream_t stream);
 
-/* 1 when spgt_spectral_inverse_linear serves this shape (64 channels in and out, 2*modes <= min(32, r),
- * r <= 1024). */
+/* 1 when spgt_spectral_inverse_linear serves this shape (32 or 64 channels in and out,
+ * 2*modes <= min(64, r), r <= 1024). */
 int spgt_spectral_inverse_linear_supported(int r, int in_features, int out_features, int modes);
 
 /* The end of Sp_SpectralConv2D.forward (network/sp_layer.py:132, 149-155) in one pass:
@@ -253,13 +253,14 @@ int spgt_spectral_inverse_linear_supported(int r, int in_features, int out_featu
  * their sum and the activation, without the inverse transform's result going to memory.
  * U planar [N, 2*modes, r, channels] as spgt_spectral_modes_middle writes it; x, out [rows = N*r, r, channels];
  * weight_kn [channels, channels] (the transpose of nn.Linear.weight); bias [channels] or null;
- * table_operand [ceil(r/32), 16, 64]: entry (t, kk, l) = table[32 t + l % 32, 2 kk + l / 32] of the inverse
- * table above, zero where the row is >= r or the column >= 2*modes. */
+ * table_operand [ceil(r/32), steps, 64], steps = 16 for modes <= 16, else 32: entry (t, kk, l) =
+ * table[32 t + l % 32, 2 kk + l / 32] of the inverse table above, zero where the row is >= r or the column
+ * >= 2*modes. */
 int spgt_spectral_inverse_linear(const float* U, const float* table_operand, const float* x, const float* weight_kn,
                                  const float* bias, int activation, float* out, int64_t rows, int r, int channels,
                                  int modes, spgt_stream_t stream);
 
-/* 1 when spgt_spectral_modes_middle serves this shape (Cin, Cout <= 64, 2*modes <= min(32, r),
+/* 1 when spgt_spectral_modes_middle serves this shape (Cin, Cout <= 64, 2*modes <= min(64, r),
  * r <= 4096). */
 int spgt_spectral_modes_middle_supported(int r, int Cin, int Cout, int modes);
 

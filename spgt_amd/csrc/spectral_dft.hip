@@ -1,12 +1,3 @@
-#define SPGT_LOAD_X_ONE(BASE_, W0_, I_)                        \
-    if ((I_) == 0) s0 = SPGT_X_PIECE(BASE_, W0_, 0);           \
-    else if ((I_) == 1) s1 = SPGT_X_PIECE(BASE_, W0_, 1);      \
-    else if ((I_) == 2) s2 = SPGT_X_PIECE(BASE_, W0_, 2);      \
-    else if ((I_) == 3) s3 = SPGT_X_PIECE(BASE_, W0_, 3);      \
-    else if ((I_) == 4) s4 = SPGT_X_PIECE(BASE_, W0_, 4);      \
-    else if ((I_) == 5) s5 = SPGT_X_PIECE(BASE_, W0_, 5);      \
-    else if ((I_) == 6) s6 = SPGT_X_PIECE(BASE_, W0_, 6);      \
-    else s7 = SPGT_X_PIECE(BASE_, W0_, 7);
 // Truncated DFT along the last grid axis of the FNO spectral layer, as MFMA products
 // against a small table of twiddle factors.
 //
@@ -31,10 +22,11 @@
 namespace spgt {
 
 // grid (workgroups), block 256; waves stride over the rows * C/32 (row, channel block) items.
-// tab [2*ceil(r/2)][32]: row w holds the m2 table entries of grid point w, zero elsewhere.
+// tab [2*ceil(r/2)][32 MB]: row w holds the m2 table entries of grid point w, zero elsewhere.
 // Y [rows][C][m2], or planar [rows/r][m2][r][C].  CT = C when known at compile time (row offsets
-// become immediates), 0 = any C.
-template <int CT>
+// become immediates), 0 = any C.  MB = blocks of 32 table columns (m2 <= 32 MB): one accumulator per block,
+// all fed by the same x operand.
+template <int CT, int MB>
 __global__ __launch_bounds__(256) void dft_rows_forward_k(const float* __restrict__ x, const float* __restrict__ tab,
                                                           float* __restrict__ Y, int64_t rows, int r, int C_, int m2,
                                                           int planar) {
@@ -43,7 +35,7 @@ __global__ __launch_bounds__(256) void dft_rows_forward_k(const float* __restric
     const int KH = (r + 1) / 2;
     {
         // straight 16-byte copy, eight loads in flight per thread: one memory round trip for r <= 256
-        const int total4 = 2 * KH * 8;
+        const int total4 = 2 * KH * 8 * MB;
         const float4* src = reinterpret_cast<const float4*>(tab);
         float4* dst = reinterpret_cast<float4*>(ts);
         for (int e0 = threadIdx.x; e0 < total4; e0 += 256 * 8) {
@@ -62,7 +54,8 @@ __global__ __launch_bounds__(256) void dft_rows_forward_k(const float* __restric
     const int kh = lane >> 5;
     const int CB = C / 32;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const float* tl = ts + kh * 32 + tk;  // step kk reads tl[64 * kk]
+    constexpr int TP = 64 * MB;                // table words per MFMA step (two grid points)
+    const float* tl = ts + kh * 32 * MB + tk;  // step kk, column block mb reads tl[TP * kk + 32 * mb]
     constexpr int BK = 16;
     const int nfull = (KH - 1) / BK;  // batches whose steps all lie before the final one
     const int nb = nfull + 1;
@@ -74,35 +67,43 @@ __global__ __launch_bounds__(256) void dft_rows_forward_k(const float* __restric
         const uint32_t voff = (uint32_t)(kh * C + cb * 32 + tk);
         // the last step of an odd r would read point r: those lanes re-read point r-1 against a zero table row
         const uint32_t voff_tail = (uint32_t)(min(2 * (KH - 1) + kh, r - 1) * C + cb * 32 + tk);
-        float xa[BK], ta[BK], xb[BK], tb[BK];
-        v16f acc;
+        float xa[BK], ta[MB][BK], xb[BK], tb[MB][BK];
+        v16f acc[MB];
 #pragma unroll
-        for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+        for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[mb][i] = 0.f;
         // Full batches read 2*BK grid points at compile-time offsets; the last batch holds the
         // remaining steps and the (possibly clamped) final one.
 #define SPGT_DFT_FETCH_FULL(XV, TV, B)                                                   \
         {                                                                                \
             const float* xb_ = base + (int64_t)(B) * (2 * BK) * C;                       \
-            const float* tb_ = tl + (B) * (64 * BK);                                     \
+            const float* tb_ = tl + (B) * (TP * BK);                                     \
             _Pragma("unroll") for (int u = 0; u < BK; ++u) {                             \
                 XV[u] = xb_[voff + (uint32_t)(2 * u * C)];                               \
-                TV[u] = tb_[64 * u];                                                     \
+                _Pragma("unroll") for (int mb = 0; mb < MB; ++mb) TV[mb][u] = tb_[TP * u + 32 * mb]; \
             }                                                                            \
         }
 #define SPGT_DFT_FETCH_TAIL(XV, TV)                                                      \
         _Pragma("unroll") for (int u = 0; u < BK; ++u) {                                 \
             const int kk = nfull * BK + u;                                               \
             XV[u] = (kk < KH - 1) ? base[voff + (uint32_t)(2 * kk * C)] : base[voff_tail]; \
-            TV[u] = tl[64 * min(kk, KH - 1)];                                            \
+            _Pragma("unroll") for (int mb = 0; mb < MB; ++mb)                            \
+                TV[mb][u] = tl[TP * min(kk, KH - 1) + 32 * mb];                          \
         }
 #define SPGT_DFT_FETCH(XV, TV, B)                                                        \
         if ((B) < nfull) SPGT_DFT_FETCH_FULL(XV, TV, B) else { SPGT_DFT_FETCH_TAIL(XV, TV) }
 #define SPGT_DFT_MUL(XV, TV, B)                                                          \
         if ((B) < nfull) {                                                               \
-            _Pragma("unroll") for (int u = 0; u < BK; ++u) acc = mfma32(TV[u], XV[u], acc); \
+            _Pragma("unroll") for (int u = 0; u < BK; ++u)                               \
+                _Pragma("unroll") for (int mb = 0; mb < MB; ++mb)                        \
+                    acc[mb] = mfma32(TV[mb][u], XV[u], acc[mb]);                         \
         } else {                                                                         \
             _Pragma("unroll") for (int u = 0; u < BK; ++u)                               \
-                if (nfull * BK + u < KH) acc = mfma32(TV[u], XV[u], acc);                \
+                if (nfull * BK + u < KH) {                                               \
+                    _Pragma("unroll") for (int mb = 0; mb < MB; ++mb)                    \
+                        acc[mb] = mfma32(TV[mb][u], XV[u], acc[mb]);                     \
+                }                                                                        \
         }
         SPGT_DFT_FETCH(xa, ta, 0)
         for (int b = 0; b < nb; b += 2) {
@@ -119,35 +120,40 @@ __global__ __launch_bounds__(256) void dft_rows_forward_k(const float* __restric
 #undef SPGT_DFT_FETCH_TAIL
 #undef SPGT_DFT_FETCH
 #undef SPGT_DFT_MUL
-        // acc[r] = Y[c = cb*32 + tk][j = 8*(r/4) + 4*kh + r%4]
+        // acc[mb][r] = Y[c = cb*32 + tk][j = 32*mb + 8*(r/4) + 4*kh + r%4]
         if (planar) {
             // Y[n][j][h][c] with row = n*r + h: every store is a 128-byte run along c
             const int64_t n = row / r;
             const int64_t h = row - n * r;
             float* yp = Y + (n * m2 * r + h) * (int64_t)C + cb * 32 + tk;
 #pragma unroll
-            for (int q = 0; q < 4; ++q)
+            for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int j = 8 * q + 4 * kh + e;
-                    if (j < m2) yp[(int64_t)j * r * C] = acc[4 * q + e];
-                }
+                for (int q = 0; q < 4; ++q)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int j = 32 * mb + 8 * q + 4 * kh + e;
+                        if (j < m2) yp[(int64_t)j * r * C] = acc[mb][4 * q + e];
+                    }
         } else {
             float* yr = Y + (row * C + cb * 32 + tk) * (int64_t)m2;
 #pragma unroll
-            for (int q = 0; q < 4; ++q)
+            for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int j = 8 * q + 4 * kh + e;
-                    if (j < m2) yr[j] = acc[4 * q + e];
-                }
+                for (int q = 0; q < 4; ++q)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int j = 32 * mb + 8 * q + 4 * kh + e;
+                        if (j < m2) yr[j] = acc[mb][4 * q + e];
+                    }
         }
     }
 }
 
 // grid (workgroups), block 256; waves stride over the (row, channel block) items.
 // tab [32*ceil(r/32)][m2 + 1]: row w holds the m2 table entries of grid point w, zero elsewhere.
-// U [rows][C][m2] (or planar [rows/r][m2][r][C]) -> y [rows][r][C].
+// U [rows][C][m2] (or planar [rows/r][m2][r][C]) -> y [rows][r][C].  KMAX >= m2 / 2: MFMA steps held in registers.
+template <int KMAX>
 __global__ __launch_bounds__(256) void dft_rows_inverse_k(const float* __restrict__ U, const float* __restrict__ tab,
                                                           float* __restrict__ y, int64_t rows, int r, int C, int m2,
                                                           int planar) {
@@ -177,17 +183,17 @@ __global__ __launch_bounds__(256) void dft_rows_inverse_k(const float* __restric
     const int64_t row = gw / CB;
     const int cb = (int)(gw % CB);
     // B operand: U[o = cb*32 + tk][j = 2kk + kh]
-    float ureg[16];
+    float ureg[KMAX];
     if (planar) {
         const int64_t n = row / r;
         const int64_t h = row - n * r;
         const float* up = U + (n * m2 * r + h) * (int64_t)C + cb * 32 + tk;  // U[n][j][h][o]
 #pragma unroll
-        for (int kk = 0; kk < 16; ++kk) ureg[kk] = (2 * kk + kh < m2) ? up[(int64_t)(2 * kk + kh) * r * C] : 0.f;
+        for (int kk = 0; kk < KMAX; ++kk) ureg[kk] = (2 * kk + kh < m2) ? up[(int64_t)(2 * kk + kh) * r * C] : 0.f;
     } else {
         const float* ur = U + (row * C + cb * 32 + tk) * (int64_t)m2;
 #pragma unroll
-        for (int kk = 0; kk < 16; ++kk) ureg[kk] = (2 * kk + kh < m2) ? ur[2 * kk + kh] : 0.f;
+        for (int kk = 0; kk < KMAX; ++kk) ureg[kk] = (2 * kk + kh < m2) ? ur[2 * kk + kh] : 0.f;
     }
     float* yr = y + row * (int64_t)r * C + cb * 32 + tk;
     const int KH = m2 / 2;
@@ -197,7 +203,7 @@ __global__ __launch_bounds__(256) void dft_rows_inverse_k(const float* __restric
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[i] = 0.f;
 #pragma unroll
-        for (int kk = 0; kk < 16; ++kk)
+        for (int kk = 0; kk < KMAX; ++kk)
             if (kk < KH) acc = mfma32(ta[2 * kk], ureg[kk], acc);
         // acc[q] = y[w = wt*32 + 8*(q/4) + 4*kh + q%4][o = cb*32 + tk]
 #pragma unroll
@@ -329,6 +335,8 @@ __global__ __launch_bounds__(256) void spectral_rows_contract_k(
 }
 
 // grid (m, N, chunks of h), block 256.  Wave w of a workgroup takes rows h = h0 + w, h0 + w + 4, ...
+// KHMAX >= 2m: kept rows held in registers.
+template <int KHMAX>
 __global__ __launch_bounds__(256) void spectral_rows_expand_k(
     const float2* __restrict__ O, const float2* __restrict__ Gi, float* __restrict__ U, int r, int Cout, int m,
     int rows_per_wg) {
@@ -342,10 +350,10 @@ __global__ __launch_bounds__(256) void spectral_rows_expand_k(
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     for (int e = threadIdx.x; e < (h1 - h0) * m2; e += 256) lds[e] = Gi[(int64_t)h0 * m2 + e];
     // the mode's O[kh][o] for all kept rows stays in registers
-    float2 ov[32];
+    float2 ov[KHMAX];
     const float2* Om = O + ((n * m + kw) * m2) * (int64_t)Cout + lane;
 #pragma unroll
-    for (int kh = 0; kh < 32; ++kh) ov[kh] = (kh < m2 && lane < Cout) ? Om[(int64_t)kh * Cout] : make_float2(0.f, 0.f);
+    for (int kh = 0; kh < KHMAX; ++kh) ov[kh] = (kh < m2 && lane < Cout) ? Om[(int64_t)kh * Cout] : make_float2(0.f, 0.f);
     __syncthreads();
     float* ure = U + ((n * m2 + 2 * kw) * r) * (int64_t)Cout + lane;
     float* uim = ure + (int64_t)r * Cout;
@@ -353,7 +361,7 @@ __global__ __launch_bounds__(256) void spectral_rows_expand_k(
         const float2* g = lds + (h - h0) * m2;
         float2 acc = make_float2(0.f, 0.f);
 #pragma unroll
-        for (int kh = 0; kh < 32; ++kh) {
+        for (int kh = 0; kh < KHMAX; ++kh) {
             if (kh < m2) {
                 acc.x = fmaf(g[kh].x, ov[kh].x, acc.x);
                 acc.x = fmaf(-g[kh].y, ov[kh].y, acc.x);
@@ -371,31 +379,38 @@ __global__ __launch_bounds__(256) void spectral_rows_expand_k(
 // The end of Sp_SpectralConv2D.forward (network/sp_layer.py:132, 149-155) in one pass over the grid:
 //   out[row, w, o] = act( sum_c x[row, w, c] W[c, o] + bias[o] + sum_j table[w, j] U[row, o, j] )
 // i.e. the residual Linear, the inverse DFT along w of the retained modes, their sum and the activation;
-// the inverse transform's result never goes to memory.  64 channels in and out, planar U [N][2m][r][64].
+// the inverse transform's result never goes to memory.  C = 32 or 64 channels in and out, planar U [N][2m][r][C].
 // Both terms are MFMA products with output channels along the accumulator's registers and grid points along
 // its lanes (so a lane stores 16-byte pieces of its grid point's row): A = W resp. U in registers,
-// B = x tile (from a wave-private LDS tile, 16-byte reads, lane (w, kh) takes channels kh*32 + kk) resp.
+// B = x tile (from a wave-private LDS tile, 16-byte reads, lane (w, kh) takes channels kh*C/2 + kk) resp.
 // table entries (handed over in operand order, tabA[tile][kk][lane] = table[32 tile + lane%32][2kk +
 // lane/32], zero outside).  No barriers.
 // One wave per SIMD (waves that share a SIMD's matrix pipe run their MFMAs at about half the rate of a lone
 // wave; with four waves per SIMD and a wave per half of the channels this pass took 44 us at [4, 211, 211, 64],
-// with two fatter waves 43-51 us, with one 34 us): a wave makes all 64 channels of a 32-point tile, two
-// independent accumulator chains off the same x and table operands, and walks the (grid row, tile) pairs of the
+// with two fatter waves 43-51 us, with one 34 us): a wave makes all channels of a 32-point tile (for C = 64 two
+// independent accumulator chains off the same x and table operands), and walks the (grid row, tile) pairs of the
 // whole input 4 * gridDim.x apart.  Per pair: the parked x rows go to the wave's LDS tile; this pair's U and table entries and the next
 // pair's x rows are requested (wave-uniform base + 32-bit lane offsets, computed once for U); then the 64 MFMAs
 // of the Linear, the MFMAs of the inverse transform, activation and stores.  Stores are unconditional: points
 // past the end of a grid row are computed from the row's last point and that point's table entries, and write
 // its own values to its address.
-// KSU: MFMA steps of the inverse transform, modes rounded up to a multiple of 4 (the table entries of the steps
-// past the modes are zero); a template parameter so that neither the loads nor the MFMAs sit behind branches.
+// KSU: MFMA steps of the inverse transform, modes rounded up (the table entries of the steps past the modes are
+// zero); a template parameter so that neither the loads nor the MFMAs sit behind branches.  TS: steps per tile in
+// the operand table.  C: channels in and out, 32 or 64; a lane's contraction channels are kh * C/2 + kk.
 // grid (min(ceil(pairs / 4), CUs)), block 256.
-template <int ACT, int KSU>
+template <int ACT, int KSU, int C>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void spectral_inverse_linear_k(
     const float* __restrict__ U, const float* __restrict__ tabA, const float* __restrict__ x,
     const float* __restrict__ Wkn, const float* __restrict__ bias, float* __restrict__ out, int r, int m2,
     unsigned pairs) {
-    constexpr int C = 64, PX = C + 4;
-    static_assert(KSU % 4 == 0 && KSU >= 4 && KSU <= 16, "4, 8, 12 or 16 steps");
+    constexpr int PX = C + 4;
+    constexpr int NCB = C / 32;    // blocks of 32 output channels, one accumulator chain each
+    constexpr int KL = C / 2;      // contraction channels of the Linear per lane (MFMA steps)
+    constexpr int LPR = C / 4;     // lanes per grid point when a tile is fetched in 16-byte pieces
+    constexpr int NP = C / 8;      // such pieces per lane and tile
+    constexpr int TS = KSU <= 16 ? 16 : 32;
+    static_assert(C == 32 || C == 64, "32 or 64 channels");
+    static_assert(KSU % 4 == 0 && KSU >= 4 && KSU <= 32, "4 .. 32 steps in fours");
     __shared__ __attribute__((aligned(16))) float xs[4][32 * PX];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -404,11 +419,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     const unsigned WT = (unsigned)(r + 31) / 32;
     const unsigned stride = gridDim.x * 4;
 
-    float wreg0[32], wreg1[32];  // W[c = kh*32 + kk][o = cb*32 + tk], cb = 0, 1
+    float wreg0[KL], wreg1[KL];  // W[c = kh*KL + kk][o = cb*32 + tk], cb = 0, 1
 #pragma unroll
-    for (int kk = 0; kk < 32; ++kk) {
-        wreg0[kk] = Wkn[(kh * 32 + kk) * C + tk];
-        wreg1[kk] = Wkn[(kh * 32 + kk) * C + 32 + tk];
+    for (int kk = 0; kk < KL; ++kk) {
+        wreg0[kk] = Wkn[(kh * KL + kk) * C + tk];
+        wreg1[kk] = NCB == 2 ? Wkn[(kh * KL + kk) * C + (NCB - 1) * 32 + tk] : 0.f;
     }
     // bias in accumulator layout (element 4q + e of half cb belongs to channel cb*32 + 8q + 4kh + e): the C operand
     // of a pair's first MFMAs
@@ -417,7 +432,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     for (int q = 0; q < 4; ++q) {
         const float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
         const float4 b0 = bias ? *reinterpret_cast<const float4*>(bias + 8 * q + 4 * kh) : z;
-        const float4 b1 = bias ? *reinterpret_cast<const float4*>(bias + 32 + 8 * q + 4 * kh) : z;
+        const float4 b1 = (bias && NCB == 2) ? *reinterpret_cast<const float4*>(bias + (NCB - 1) * 32 + 8 * q + 4 * kh) : z;
         bo0[4 * q + 0] = b0.x; bo0[4 * q + 1] = b0.y; bo0[4 * q + 2] = b0.z; bo0[4 * q + 3] = b0.w;
         bo1[4 * q + 0] = b1.x; bo1[4 * q + 1] = b1.y; bo1[4 * q + 2] = b1.z; bo1[4 * q + 3] = b1.w;
     }
@@ -429,22 +444,26 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     float* const xw = xs[wave];
 
     // (named registers and macros: a register array that lives across the loop ends up in scratch memory)
-    // piece I of a tile is row (lane + 64 I) / 16, channels 4 (lane % 16) ..; rows past the end of the grid row
-    // read its last point
+    // piece I of a tile is grid point (lane + 64 I) / LPR, channels 4 (lane % LPR) ..; points past the end of the
+    // grid row read its last point
     float4 s0, s1, s2, s3, s4, s5, s6, s7;
 #define SPGT_X_PIECE(BASE_, W0_, I_) \
-    (*reinterpret_cast<const float4*>((BASE_) + (uint32_t)(min((W0_) + ((lane + 64 * (I_)) >> 4), r - 1) * C + 4 * (lane & 15))))
+    (*reinterpret_cast<const float4*>((BASE_) + (uint32_t)(min((W0_) + ((lane + 64 * (I_)) / LPR), r - 1) * C + 4 * (lane % LPR))))
 #define SPGT_LOAD_X_TILE(T_)                                                                        \
     {                                                                                               \
         const unsigned row_ = (T_) / WT;                                                            \
         const int w0_ = (int)((T_) - row_ * WT) * 32;                                               \
         const float* xb_ = x + (int64_t)row_ * r * C;                                               \
         s0 = SPGT_X_PIECE(xb_, w0_, 0); s1 = SPGT_X_PIECE(xb_, w0_, 1); s2 = SPGT_X_PIECE(xb_, w0_, 2); \
-        s3 = SPGT_X_PIECE(xb_, w0_, 3); s4 = SPGT_X_PIECE(xb_, w0_, 4); s5 = SPGT_X_PIECE(xb_, w0_, 5); \
-        s6 = SPGT_X_PIECE(xb_, w0_, 6); s7 = SPGT_X_PIECE(xb_, w0_, 7);                             \
+        s3 = SPGT_X_PIECE(xb_, w0_, 3);                                                             \
+        if (NP == 8) {                                                                              \
+            s4 = SPGT_X_PIECE(xb_, w0_, 4); s5 = SPGT_X_PIECE(xb_, w0_, 5);                         \
+            s6 = SPGT_X_PIECE(xb_, w0_, 6); s7 = SPGT_X_PIECE(xb_, w0_, 7);                         \
+        }                                                                                           \
     }
 #define SPGT_STORE_X_PIECE(I_, V_) \
-    *reinterpret_cast<float4*>(xw + ((lane + 64 * (I_)) >> 4) * PX + 4 * (lane & 15)) = V_;
+    *reinterpret_cast<float4*>(xw + ((lane + 64 * (I_)) / LPR) * PX + 4 * (lane % LPR)) = V_;
+    s4 = s5 = s6 = s7 = make_float4(0.f, 0.f, 0.f, 0.f);
     unsigned t = blockIdx.x * 4 + wave;
     if (t < pairs) SPGT_LOAD_X_TILE(t)
     for (; t < pairs; t += stride) {
@@ -453,55 +472,57 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         const unsigned n = row / (unsigned)r;
         const unsigned h = row - n * (unsigned)r;
         SPGT_STORE_X_PIECE(0, s0) SPGT_STORE_X_PIECE(1, s1) SPGT_STORE_X_PIECE(2, s2) SPGT_STORE_X_PIECE(3, s3)
-        SPGT_STORE_X_PIECE(4, s4) SPGT_STORE_X_PIECE(5, s5) SPGT_STORE_X_PIECE(6, s6) SPGT_STORE_X_PIECE(7, s7)
+        if (NP == 8) {
+            SPGT_STORE_X_PIECE(4, s4) SPGT_STORE_X_PIECE(5, s5) SPGT_STORE_X_PIECE(6, s6) SPGT_STORE_X_PIECE(7, s7)
+        }
         const float* ub = U + ((int64_t)n * m2 * r + h) * C;  // U[n][0][h][0]
         float ureg0[KSU], ureg1[KSU];
 #pragma unroll
         for (int kk = 0; kk < KSU; ++kk) {
             ureg0[kk] = ub[uoff[kk]];
-            ureg1[kk] = ub[uoff[kk] + 32u];
+            ureg1[kk] = NCB == 2 ? ub[uoff[kk] + (uint32_t)((NCB - 1) * 32)] : 0.f;
         }
-        // the operand table holds 16 steps per tile; points past the row's end take the last point's entries
-        const float* tb = tabA + (int64_t)wt * (16 * 64);
+        // the operand table holds TS steps per tile; points past the row's end take the last point's entries
+        const float* tb = tabA + (int64_t)wt * (TS * 64);
         const uint32_t tl = (uint32_t)(kh * 32 + min(tk, r - 1 - wt * 32));
         float ta[KSU];
 #pragma unroll
         for (int kk = 0; kk < KSU; ++kk) ta[kk] = tb[tl + (uint32_t)(kk * 64)];
         SPGT_LOAD_X_TILE(min(t + stride, pairs - 1))  // after the last pair: loaded again, not used
-        const float* xr = xw + tk * PX + kh * 32;
-        float4 xv[8];
+        const float* xr = xw + tk * PX + kh * KL;
+        float4 xv[NP];
 #pragma unroll
-        for (int g = 0; g < 8; ++g) xv[g] = *reinterpret_cast<const float4*>(xr + 4 * g);
+        for (int g = 0; g < NP; ++g) xv[g] = *reinterpret_cast<const float4*>(xr + 4 * g);
         __builtin_amdgcn_sched_barrier(0);
         v16f acc0 = bo0, acc1 = bo1;
 #pragma unroll
-        for (int g = 0; g < 8; ++g) {
+        for (int g = 0; g < NP; ++g) {
             acc0 = mfma32(wreg0[4 * g + 0], xv[g].x, acc0);
-            acc1 = mfma32(wreg1[4 * g + 0], xv[g].x, acc1);
+            if (NCB == 2) acc1 = mfma32(wreg1[4 * g + 0], xv[g].x, acc1);
             acc0 = mfma32(wreg0[4 * g + 1], xv[g].y, acc0);
-            acc1 = mfma32(wreg1[4 * g + 1], xv[g].y, acc1);
+            if (NCB == 2) acc1 = mfma32(wreg1[4 * g + 1], xv[g].y, acc1);
             acc0 = mfma32(wreg0[4 * g + 2], xv[g].z, acc0);
-            acc1 = mfma32(wreg1[4 * g + 2], xv[g].z, acc1);
+            if (NCB == 2) acc1 = mfma32(wreg1[4 * g + 2], xv[g].z, acc1);
             acc0 = mfma32(wreg0[4 * g + 3], xv[g].w, acc0);
-            acc1 = mfma32(wreg1[4 * g + 3], xv[g].w, acc1);
+            if (NCB == 2) acc1 = mfma32(wreg1[4 * g + 3], xv[g].w, acc1);
         }
 #pragma unroll
         for (int kk = 0; kk < KSU; ++kk) {
             acc0 = mfma32(ureg0[kk], ta[kk], acc0);
-            acc1 = mfma32(ureg1[kk], ta[kk], acc1);
+            if (NCB == 2) acc1 = mfma32(ureg1[kk], ta[kk], acc1);
         }
         // acc{cb}[4q + e] = out[w][o = cb*32 + 8q + 4kh + e] before the activation
         float y[32];
 #pragma unroll
         for (int q = 0; q < 16; ++q) y[q] = acc0[q], y[16 + q] = acc1[q];
 #pragma unroll
-        for (int q = 0; q < 32; ++q) {
+        for (int q = 0; q < 16 * NCB; ++q) {
             if (ACT == SPGT_ACT_RELU) y[q] = fmaxf(y[q], 0.f);
             if (ACT == SPGT_ACT_SILU) y[q] = y[q] * __builtin_amdgcn_rcpf(1.f + __expf(-y[q]));
         }
         float* const op = out + ((int64_t)row * r + min(wt * 32 + tk, r - 1)) * C + 4 * kh;
 #pragma unroll
-        for (int q = 0; q < 8; ++q)
+        for (int q = 0; q < 4 * NCB; ++q)
             *reinterpret_cast<float4*>(op + 8 * q) = make_float4(y[4 * q], y[4 * q + 1], y[4 * q + 2], y[4 * q + 3]);
     }
 #undef SPGT_LOAD_X_TILE
@@ -520,9 +541,10 @@ int dft_rows_check(const char* who, const void* a, const void* tab, const void* 
     if (!a || !tab || !b) return fail(SPGT_ERR_INVALID_ARGUMENT, "truncated_dft_rows: null pointer argument");
     if (rows <= 0 || r <= 0) return fail(SPGT_ERR_INVALID_ARGUMENT, "truncated_dft_rows: rows and r must be positive");
     if (C <= 0 || C % 32 != 0) return fail(SPGT_ERR_INVALID_ARGUMENT, "truncated_dft_rows: channels must be a multiple of 32");
-    if (m2 <= 0 || m2 > 32 || (m2 & 1))
-        return fail(SPGT_ERR_INVALID_ARGUMENT, "truncated_dft_rows: 2*modes must be even and at most 32");
-    if (r > 1024) return fail(SPGT_ERR_INVALID_ARGUMENT, "truncated_dft_rows: r exceeds 1024");
+    if (m2 <= 0 || m2 > 64 || (m2 & 1))
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "truncated_dft_rows: 2*modes must be even and at most 64");
+    if (r > (m2 > 32 ? 512 : 1024))
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "truncated_dft_rows: r exceeds 1024 (512 when 2*modes > 32)");
     if (ceil_div(rows * (C / 32), (int64_t)4) > INT32_MAX)
         return fail(SPGT_ERR_INVALID_ARGUMENT, "truncated_dft_rows: too many rows");
     if (!aligned4(a) || !aligned16(tab) || !aligned4(b))
@@ -532,26 +554,42 @@ int dft_rows_check(const char* who, const void* a, const void* tab, const void* 
     return SPGT_OK;
 }
 
+template <typename K>
+void allow_lds(K kernel, size_t lds) {
+    if (lds > 64 * 1024)
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  (int)lds);
+}
+
 }  // namespace
 
 extern "C" int spgt_truncated_dft_rows_supported(int r, int channels, int modes) {
-    return (r > 0 && r <= 1024 && channels > 0 && channels % 32 == 0 && modes > 0 && 2 * modes <= 32) ? 1 : 0;
+    return (r > 0 && channels > 0 && channels % 32 == 0 && modes > 0 && 2 * modes <= 64 &&
+            r <= (2 * modes > 32 ? 512 : 1024)) ? 1 : 0;
 }
 
 extern "C" int spgt_truncated_dft_rows_forward(const float* x, const float* table, float* Y, int64_t rows, int r,
                                                int channels, int modes, int planar, hipStream_t stream) {
     const int m2 = 2 * modes;
     if (int rc = dft_rows_check("truncated_dft_rows_forward", x, table, Y, rows, r, channels, m2)) return rc;
-    const size_t lds = (size_t)2 * ((r + 1) / 2) * 32 * sizeof(float);
-    auto kernel = channels == 64 ? dft_rows_forward_k<64> : (channels == 32 ? dft_rows_forward_k<32> : dft_rows_forward_k<0>);
-    if (lds > 64 * 1024)
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                  (int)lds);
-    // workgroups loop over (row, channel block) items: about two per CU, so the table is staged few times
-    const unsigned grid = (unsigned)std::min<int64_t>(ceil_div(rows * (channels / 32), (int64_t)4), 2 * device_cu_count());
     if (planar && rows % r != 0)
         return fail(SPGT_ERR_INVALID_ARGUMENT, "truncated_dft_rows_forward: planar output needs rows = N * r");
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), lds, stream, x, table, Y, rows, r, channels, m2, planar);
+    const int mb = m2 > 32 ? 2 : 1;
+    const size_t lds = (size_t)2 * ((r + 1) / 2) * 32 * mb * sizeof(float);
+    // workgroups loop over (row, channel block) items: about two per CU, so the table is staged few times
+    const unsigned grid = (unsigned)std::min<int64_t>(ceil_div(rows * (channels / 32), (int64_t)4), 2 * device_cu_count());
+#define SPGT_DFT_FWD(CT, MB)                                                                                    \
+    {                                                                                                           \
+        allow_lds(dft_rows_forward_k<CT, MB>, lds);                                                             \
+        hipLaunchKernelGGL((dft_rows_forward_k<CT, MB>), dim3(grid), dim3(256), lds, stream, x, table, Y, rows, r, \
+                           channels, m2, planar);                                                               \
+    }
+    if (mb == 1) {
+        if (channels == 64) SPGT_DFT_FWD(64, 1) else if (channels == 32) SPGT_DFT_FWD(32, 1) else SPGT_DFT_FWD(0, 1)
+    } else {
+        if (channels == 64) SPGT_DFT_FWD(64, 2) else if (channels == 32) SPGT_DFT_FWD(32, 2) else SPGT_DFT_FWD(0, 2)
+    }
+#undef SPGT_DFT_FWD
     return check_launch("truncated_dft_rows_forward");
 }
 
@@ -559,21 +597,25 @@ extern "C" int spgt_truncated_dft_rows_inverse(const float* U, const float* tabl
                                                int channels, int modes, int planar, hipStream_t stream) {
     const int m2 = 2 * modes;
     if (int rc = dft_rows_check("truncated_dft_rows_inverse", U, table, y, rows, r, channels, m2)) return rc;
-    const size_t lds = (size_t)((r + 31) / 32) * 32 * (m2 + 1) * sizeof(float);
-    auto kernel = dft_rows_inverse_k;
-    if (lds > 64 * 1024)
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                  (int)lds);
-    const unsigned grid = (unsigned)std::min<int64_t>(ceil_div(rows * (channels / 32), (int64_t)4), 2 * device_cu_count());
     if (planar && rows % r != 0)
         return fail(SPGT_ERR_INVALID_ARGUMENT, "truncated_dft_rows_inverse: planar input needs rows = N * r");
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), lds, stream, U, table, y, rows, r, channels, m2, planar);
+    const size_t lds = (size_t)((r + 31) / 32) * 32 * (m2 + 1) * sizeof(float);
+    const unsigned grid = (unsigned)std::min<int64_t>(ceil_div(rows * (channels / 32), (int64_t)4), 2 * device_cu_count());
+    if (m2 <= 32) {
+        allow_lds(dft_rows_inverse_k<16>, lds);
+        hipLaunchKernelGGL(dft_rows_inverse_k<16>, dim3(grid), dim3(256), lds, stream, U, table, y, rows, r, channels, m2,
+                           planar);
+    } else {
+        allow_lds(dft_rows_inverse_k<32>, lds);
+        hipLaunchKernelGGL(dft_rows_inverse_k<32>, dim3(grid), dim3(256), lds, stream, U, table, y, rows, r, channels, m2,
+                           planar);
+    }
     return check_launch("truncated_dft_rows_inverse");
 }
 
 extern "C" int spgt_spectral_modes_middle_supported(int r, int Cin, int Cout, int modes) {
     return (r > 0 && r <= 4096 && Cin > 0 && Cin <= kMidC && Cout > 0 && Cout <= kMidC && modes > 0 &&
-            2 * modes <= 32 && 2 * modes <= r) ? 1 : 0;
+            2 * modes <= 64 && 2 * modes <= r) ? 1 : 0;
 }
 
 extern "C" size_t spgt_spectral_modes_middle_workspace_bytes(int N, int Cout, int modes) {
@@ -590,7 +632,7 @@ extern "C" int spgt_spectral_modes_middle(const float* Y, const float* table_h, 
     if (N <= 0 || N > 65535) return fail(SPGT_ERR_INVALID_ARGUMENT, "spectral_modes_middle: N must be 1..65535");
     if (!spgt_spectral_modes_middle_supported(r, Cin, Cout, modes))
         return fail(SPGT_ERR_INVALID_ARGUMENT,
-                    "spectral_modes_middle: needs Cin, Cout <= 64, 2*modes <= min(32, r), r <= 4096");
+                    "spectral_modes_middle: needs Cin, Cout <= 64, 2*modes <= min(64, r), r <= 4096");
     if (workspace_bytes < spgt_spectral_modes_middle_workspace_bytes(N, Cout, modes))
         return fail(SPGT_ERR_WORKSPACE, "spectral_modes_middle: workspace too small");
     if (!aligned4(Y) || !aligned4(U) || !aligned8(table_h) || !aligned8(table_h_inverse) || !aligned8(weight_1) ||
@@ -605,18 +647,24 @@ extern "C" int spgt_spectral_modes_middle(const float* Y, const float* table_h, 
     hipLaunchKernelGGL(spectral_rows_contract_k, dim3(modes, N, ceil_div(m2, kMidRows)), dim3(256), lds1, stream, Y,
                        reinterpret_cast<const float2*>(table_h), reinterpret_cast<const float2*>(weight_1),
                        reinterpret_cast<const float2*>(weight_2), O, r, Cin, Cout, modes);
-    // about three workgroups per CU for the expansion
-    const int chunks = std::max(1, std::min(ceil_div(r, 4), ceil_div(3 * device_cu_count(), modes * N)));
+    // about three workgroups per CU for the expansion; a chunk's table rows must fit 64 KiB of LDS
+    int chunks = std::max(1, std::min(ceil_div(r, 4), ceil_div(3 * device_cu_count(), modes * N)));
+    chunks = std::max(chunks, ceil_div(r * m2 * (int)sizeof(float2), 64 * 1024));
     const int rows_per_wg = ceil_div(r, chunks);
     const size_t lds2 = (size_t)rows_per_wg * m2 * sizeof(float2);
-    hipLaunchKernelGGL(spectral_rows_expand_k, dim3(modes, N, ceil_div(r, rows_per_wg)), dim3(256), lds2, stream, O,
-                       reinterpret_cast<const float2*>(table_h_inverse), U, r, Cout, modes, rows_per_wg);
+    const dim3 grid2(modes, N, ceil_div(r, rows_per_wg));
+    if (m2 <= 32)
+        hipLaunchKernelGGL(spectral_rows_expand_k<32>, grid2, dim3(256), lds2, stream, O,
+                           reinterpret_cast<const float2*>(table_h_inverse), U, r, Cout, modes, rows_per_wg);
+    else
+        hipLaunchKernelGGL(spectral_rows_expand_k<64>, grid2, dim3(256), lds2, stream, O,
+                           reinterpret_cast<const float2*>(table_h_inverse), U, r, Cout, modes, rows_per_wg);
     return check_launch("spectral_modes_middle");
 }
 
 extern "C" int spgt_spectral_inverse_linear_supported(int r, int in_features, int out_features, int modes) {
-    return (r > 0 && r <= 1024 && in_features == 64 && out_features == 64 && modes > 0 && 2 * modes <= 32 &&
-            2 * modes <= r) ? 1 : 0;
+    return (r > 0 && r <= 1024 && in_features == out_features && (in_features == 32 || in_features == 64) &&
+            modes > 0 && 2 * modes <= 64 && 2 * modes <= r) ? 1 : 0;
 }
 
 extern "C" int spgt_spectral_inverse_linear(const float* U, const float* table_operand, const float* x,
@@ -625,7 +673,8 @@ extern "C" int spgt_spectral_inverse_linear(const float* U, const float* table_o
     if (!U || !table_operand || !x || !weight_kn || !out)
         return fail(SPGT_ERR_INVALID_ARGUMENT, "spectral_inverse_linear: null pointer argument");
     if (!spgt_spectral_inverse_linear_supported(r, channels, channels, modes))
-        return fail(SPGT_ERR_INVALID_ARGUMENT, "spectral_inverse_linear: needs 64 channels, 2*modes <= min(32, r), r <= 1024");
+        return fail(SPGT_ERR_INVALID_ARGUMENT,
+                    "spectral_inverse_linear: needs 32 or 64 channels, 2*modes <= min(64, r), r <= 1024");
     if (rows <= 0 || rows % r != 0 || rows > INT32_MAX)
         return fail(SPGT_ERR_INVALID_ARGUMENT, "spectral_inverse_linear: rows must be a positive multiple of r");
     if (activation != SPGT_ACT_NONE && activation != SPGT_ACT_RELU && activation != SPGT_ACT_SILU)
@@ -639,17 +688,22 @@ extern "C" int spgt_spectral_inverse_linear(const float* U, const float* table_o
     if (pairs > (int64_t)INT32_MAX - 4096)
         return fail(SPGT_ERR_INVALID_ARGUMENT, "spectral_inverse_linear: more than 2^31 tiles of 32 grid points");
     const dim3 grid((unsigned)std::min<int64_t>(ceil_div(pairs, (int64_t)4), (int64_t)device_cu_count()));
-#define SPGT_SIL_LAUNCH(ACT, KSU)                                                                                 \
-    hipLaunchKernelGGL((spectral_inverse_linear_k<ACT, KSU>), grid, dim3(256), 0, stream, U, table_operand, x, \
+#define SPGT_SIL_LAUNCH(ACT, KSU, C)                                                                               \
+    hipLaunchKernelGGL((spectral_inverse_linear_k<ACT, KSU, C>), grid, dim3(256), 0, stream, U, table_operand, x, \
                        weight_kn, bias, out, r, 2 * modes, (unsigned)pairs)
-#define SPGT_SIL_STEPS(ACT)                         \
-    if (modes <= 4) SPGT_SIL_LAUNCH(ACT, 4);        \
-    else if (modes <= 8) SPGT_SIL_LAUNCH(ACT, 8);   \
-    else if (modes <= 12) SPGT_SIL_LAUNCH(ACT, 12); \
-    else SPGT_SIL_LAUNCH(ACT, 16)
-    if (activation == SPGT_ACT_RELU) { SPGT_SIL_STEPS(SPGT_ACT_RELU); }
-    else if (activation == SPGT_ACT_SILU) { SPGT_SIL_STEPS(SPGT_ACT_SILU); }
-    else { SPGT_SIL_STEPS(SPGT_ACT_NONE); }
+#define SPGT_SIL_STEPS(ACT, C)                         \
+    if (modes <= 4) SPGT_SIL_LAUNCH(ACT, 4, C);        \
+    else if (modes <= 8) SPGT_SIL_LAUNCH(ACT, 8, C);   \
+    else if (modes <= 12) SPGT_SIL_LAUNCH(ACT, 12, C); \
+    else if (modes <= 16) SPGT_SIL_LAUNCH(ACT, 16, C); \
+    else if (modes <= 24) SPGT_SIL_LAUNCH(ACT, 24, C); \
+    else SPGT_SIL_LAUNCH(ACT, 32, C)
+#define SPGT_SIL_ACT(C)                                                        \
+    if (activation == SPGT_ACT_RELU) { SPGT_SIL_STEPS(SPGT_ACT_RELU, C); }     \
+    else if (activation == SPGT_ACT_SILU) { SPGT_SIL_STEPS(SPGT_ACT_SILU, C); } \
+    else { SPGT_SIL_STEPS(SPGT_ACT_NONE, C); }
+    if (channels == 64) { SPGT_SIL_ACT(64) } else { SPGT_SIL_ACT(32) }
+#undef SPGT_SIL_ACT
 #undef SPGT_SIL_STEPS
 #undef SPGT_SIL_LAUNCH
     return check_launch("spectral_inverse_linear");

@@ -163,12 +163,13 @@ def _truncated_dft_rows_supported(r: int, channels: int, modes: int) -> bool:
 
 def pad_dft_table(table: Tensor, inverse: bool) -> Tensor:
     """The [r, 2m] twiddle table in the zero-padded layout the row kernels keep in LDS:
-    [2*ceil(r/2), 32] for the forward kernel, [32*ceil(r/32), 2m + 1] for the inverse one."""
+    [2*ceil(r/2), 32] (64 columns when 2m > 32) for the forward kernel, [32*ceil(r/32), 2m + 1] for the inverse
+    one."""
     r, m2 = table.shape
     if inverse:
         out = table.new_zeros(((r + 31) // 32 * 32, m2 + 1))
     else:
-        out = table.new_zeros(((r + 1) // 2 * 2, 32))
+        out = table.new_zeros(((r + 1) // 2 * 2, 32 if m2 <= 32 else 64))
     out[:r, :m2] = table
     return out
 
@@ -195,8 +196,8 @@ def _truncated_dft_rows(src: Tensor, table: Tensor, inverse: bool, planar: bool 
     require_gpu_f32("src", src)
     require_gpu_f32("table", table)
     r, m2 = table.shape
-    if m2 > 32 or m2 % 2:
-        raise ValueError("the table must have an even number of at most 32 columns")
+    if m2 > 64 or m2 % 2:
+        raise ValueError("the table must have an even number of at most 64 columns")
     padded = _padded(table, inverse)
     if inverse:
         if planar:
@@ -455,14 +456,15 @@ def _spectral_inverse_linear(U: Tensor, table_operand: Tensor, X: Tensor, weight
     modes = U.shape[1] // 2
     if tuple(weight_kn.shape) != (C, C):
         raise ValueError("weight_kn must be [C, C]")
-    if tuple(table_operand.shape) != ((r + 31) // 32, 16, 64):
-        raise ValueError("table_operand must be [ceil(r/32), 16, 64]")
+    steps = 16 if modes <= 16 else 32
+    if tuple(table_operand.shape) != ((r + 31) // 32, steps, 64):
+        raise ValueError(f"table_operand must be [ceil(r/32), {steps}, 64]")
     if bias is not None:
         require_gpu_f32("bias", bias)
         if bias.numel() != C:
             raise ValueError(f"bias has {bias.numel()} elements, expected {C}")
     if not _spectral_inverse_linear_supported(r, C, C, modes):
-        raise ValueError("spectral_inverse_linear: needs 64 channels, 2*modes <= min(32, r), r <= 1024")
+        raise ValueError("spectral_inverse_linear: needs 32 or 64 channels, 2*modes <= min(64, r), r <= 1024")
     out = torch.empty_like(X)
     if X.numel() == 0:
         return out
@@ -641,20 +643,22 @@ def spectral_inverse_linear_supported(r: int, cin: int, cout: int, modes: int) -
 
 
 def inverse_table_operand(table: Tensor) -> Tensor:
-    """The inverse row-DFT table [r, 2m] in the order the fused kernel's lanes read it: [ceil(r/32), 16, 64] with
-    entry (t, kk, l) = table[32 t + l % 32, 2 kk + l // 32], zero outside the table."""
+    """The inverse row-DFT table [r, 2m] in the order the fused kernel's lanes read it: [ceil(r/32), steps, 64]
+    with entry (t, kk, l) = table[32 t + l % 32, 2 kk + l // 32], zero outside the table; steps = 16 for
+    m <= 16, else 32."""
     r, m2 = table.shape
     wt = (r + 31) // 32
-    full = torch.zeros(wt * 32, 32, dtype=table.dtype, device=table.device)
+    steps = 16 if m2 <= 32 else 32
+    full = torch.zeros(wt * 32, 2 * steps, dtype=table.dtype, device=table.device)
     full[:r, :m2] = table
     # [t, w', kk, kh] -> [t, kk, kh, w'] -> lanes l = kh*32 + w'
-    return full.view(wt, 32, 16, 2).permute(0, 2, 3, 1).reshape(wt, 16, 64).contiguous()
+    return full.view(wt, 32, steps, 2).permute(0, 2, 3, 1).reshape(wt, steps, 64).contiguous()
 
 
 def spectral_inverse_linear(U: Tensor, table_operand: Tensor, X: Tensor, weight_kn: Tensor, bias, activation) -> Tensor:
     """The end of Sp_SpectralConv2D.forward in one pass: act(X @ weight_kn + bias + y) with y the inverse DFT
     along w of the planar spectrum U [N, 2m, r, C] (what truncated_dft_rows_inverse(U, table, planar=True)
-    returns); X [N, r, r, C], 64 channels (inference only)."""
+    returns); X [N, r, r, C], 32 or 64 channels (inference only)."""
     return dexts.spectral_inverse_linear(U.detach(), table_operand, X.detach(), weight_kn,
                                          None if bias is None else bias.detach(), activation)
 

@@ -224,23 +224,24 @@ class Sp_SpectralConv2D(nn.Module):
         N, r, _, cin = X.size()
         m, cout = self.mode, self.out_dim
         needs_graph = torch.is_grad_enabled() and (X.requires_grad or self.fourier_weight[0].requires_grad)
-        if (self.use_truncated_dft and not needs_graph and truncated_dft.supported(r, m) and
-                fused_linear_usable(X, self.residual_layer)):
-            # only the retained modes are ever computed: no FFT, no transposes, no full-size spectrum;
-            # the residual Linear, the add and the activation are one kernel
+        truncated = self.use_truncated_dft and not needs_graph and truncated_dft.supported(r, m)
+        if (truncated and self.droprate == 0 and truncated_dft.fused_tail_supported(r, cin, cout, m) and
+                gpu_inference(X, *self.residual_layer.parameters())):
+            # only the retained modes are ever computed: no FFT, no transposes, no full-size spectrum; the
+            # inverse transform along w, the residual Linear, the add and the activation are one kernel
+            return truncated_dft.spectral_modes_apply_linear(
+                X.contiguous(), self.fourier_weight[0], self.fourier_weight[1], m,
+                linear_weight_kn(self.residual_layer), self.residual_layer.bias,
+                activation_name(self.activation_layer))
+        if truncated and fused_linear_usable(X, self.residual_layer):
             X0 = X.contiguous()
-            if self.droprate == 0 and truncated_dft.fused_tail_supported(r, cin, cout, m):
-                # ... and the inverse transform along w happens inside that kernel too
-                return truncated_dft.spectral_modes_apply_linear(
-                    X0, self.fourier_weight[0], self.fourier_weight[1], m, linear_weight_kn(self.residual_layer),
-                    self.residual_layer.bias, activation_name(self.activation_layer))
             Y = truncated_dft.spectral_modes_apply(always_dropout(X0, self.droprate), self.fourier_weight[0],
                                                    self.fourier_weight[1], m)
             return fused_linear(X0, linear_weight_kn(self.residual_layer), self.residual_layer.bias,
                                 activation_name(self.activation_layer), Y)
         res = self.residual_layer(X)
         X = always_dropout(X, self.droprate)
-        if self.use_truncated_dft and not needs_graph and truncated_dft.supported(r, m):
+        if truncated:
             Y = truncated_dft.spectral_modes_apply(X.contiguous(), self.fourier_weight[0], self.fourier_weight[1], m)
             return self.activation_layer(Y + res)
         X = batched_transpose(X, [N], [r, r], [cin])  # -> [N, in_dim, r, r]

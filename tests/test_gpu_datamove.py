@@ -208,7 +208,8 @@ def test_spectral_modes_compact_vs_einsum(gpu, N, Cin, Cout, m):
 
 
 @pytest.mark.parametrize("N,r,Cin,Cout,m", [(2, 9, 6, 4, 3), (8, 141, 64, 64, 12), (4, 211, 64, 64, 12), (3, 16, 8, 8, 8),
-                                             (2, 30, 5, 7, 15)])
+                                             (2, 30, 5, 7, 15), (1, 421, 32, 32, 21), (1, 512, 32, 32, 23),
+                                             (2, 211, 64, 64, 15), (1, 70, 64, 32, 32), (2, 141, 32, 32, 12)])
 def test_truncated_dft_spectral_layer_vs_oracle(gpu, N, r, Cin, Cout, m):
     """The DFT-as-matrix-product route of the spectral layer against the oracle's rfft2 / irfft2 route (fp64)."""
     from spgt_amd.network import truncated_dft as T
@@ -412,7 +413,9 @@ def test_bilinear_resample_pre_bias(gpu, src_nhwc, dst_nhwc):
     assert (got - want).abs().max().item() <= 1e-5 * max(1.0, want.abs().max().item())
 
 
-@pytest.mark.parametrize("rows,r,C,m", [(3, 211, 64, 12), (5, 16, 32, 8), (2, 33, 96, 16), (1, 7, 32, 3), (844, 211, 64, 12)])
+@pytest.mark.parametrize("rows,r,C,m", [(3, 211, 64, 12), (5, 16, 32, 8), (2, 33, 96, 16), (1, 7, 32, 3), (844, 211, 64, 12),
+                                        (3, 421, 32, 21), (2, 512, 64, 23), (2, 65, 96, 32), (5, 35, 32, 17),
+                                        (2, 511, 32, 24)])
 def test_truncated_dft_rows_against_float64(gpu, rows, r, C, m):
     """Both row kernels against float64 matrix products with the same tables, and the forward one against
     torch.fft.rfft on the CPU (network/sp_layer.py:136-141 keeps columns kw < m of the ortho-normalised rfft2)."""
@@ -438,12 +441,16 @@ def test_truncated_dft_rows_against_float64(gpu, rows, r, C, m):
 def test_truncated_dft_rows_rejects(gpu):
     from spgt_amd._lib import SpgtError
     assert not dm.truncated_dft_rows_supported(211, 48, 12)
-    assert not dm.truncated_dft_rows_supported(211, 64, 17)
+    assert dm.truncated_dft_rows_supported(211, 64, 17) and dm.truncated_dft_rows_supported(512, 64, 32)
+    assert not dm.truncated_dft_rows_supported(211, 64, 33) and not dm.truncated_dft_rows_supported(513, 64, 17)
+    assert dm.truncated_dft_rows_supported(1024, 64, 16) and not dm.truncated_dft_rows_supported(1025, 64, 16)
     with pytest.raises(SpgtError):
         dm.truncated_dft_rows_forward(rnd(2, 9, 48, seed=1).to(gpu), rnd(9, 8, seed=2).to(gpu))
 
 
-@pytest.mark.parametrize("N,r,cin,cout,m", [(2, 211, 64, 64, 12), (1, 21, 32, 32, 4), (3, 16, 64, 32, 8), (2, 33, 24, 40, 16)])
+@pytest.mark.parametrize("N,r,cin,cout,m", [(2, 211, 64, 64, 12), (1, 21, 32, 32, 4), (3, 16, 64, 32, 8), (2, 33, 24, 40, 16),
+                                            (1, 421, 32, 32, 21), (1, 512, 64, 64, 23), (2, 64, 17, 9, 32),
+                                            (1, 1500, 8, 8, 20)])
 def test_spectral_modes_middle_against_float64(gpu, N, r, cin, cout, m):
     """DFT along h onto the kept rows, complex contraction, inverse DFT along h (network/sp_layer.py:136-151
     restricted to the kept modes) against the same three products in float64."""
@@ -529,18 +536,21 @@ def test_denormalize_boundary_rejects_bad_shapes(gpu):
 
 
 
-@pytest.mark.parametrize("N,r,m", [(1, 33, 4), (2, 64, 12), (4, 211, 12), (2, 141, 16), (1, 32, 16), (1, 40, 6),
-                                   (2, 7, 3), (3, 5, 1), (1, 97, 9)])
+@pytest.mark.parametrize("N,r,m,C", [(1, 33, 4, 64), (2, 64, 12, 64), (4, 211, 12, 64), (2, 141, 16, 64), (1, 32, 16, 64),
+                                     (1, 40, 6, 64), (2, 7, 3, 64), (3, 5, 1, 64), (1, 97, 9, 64), (1, 421, 21, 64),
+                                     (1, 512, 23, 64), (1, 64, 32, 64), (2, 45, 17, 64), (1, 100, 25, 64),
+                                     (2, 141, 12, 32), (1, 421, 21, 32), (1, 512, 23, 32), (2, 7, 3, 32),
+                                     (1, 33, 16, 32), (1, 70, 32, 32), (3, 40, 6, 32)])
 @pytest.mark.parametrize("act", [None, "relu", "silu"])
-def test_spectral_inverse_linear_matches_separate_kernels(gpu, N, r, m, act):
+def test_spectral_inverse_linear_matches_separate_kernels(gpu, N, r, m, C, act):
     """The fused end of the spectral layer against its parts: truncated_dft_rows_inverse + fused_linear with the
     transform's result as residual (which are tested against the FFT route and a float64 product themselves).
     Tolerance 2e-6 of the output scale: the fused kernel adds the spectral term in the accumulator, the parts
     round it to fp32 in memory first."""
     from spgt_amd.extension.bind.linear import fused_linear
     from spgt_amd.network.truncated_dft import dft_tables
-    C = 64
-    assert dm.spectral_inverse_linear_supported(r, C, C, m) and not dm.spectral_inverse_linear_supported(r, 32, 32, m)
+    assert dm.spectral_inverse_linear_supported(r, C, C, m) and not dm.spectral_inverse_linear_supported(r, 96, 96, m)
+    assert not dm.spectral_inverse_linear_supported(r, 32, 64, m)
     g = torch.Generator().manual_seed(N * 1000 + r + m)
     x = torch.randn(N, r, r, C, generator=g).to(gpu)
     U = torch.randn(N, 2 * m, r, C, generator=g).to(gpu)
@@ -549,14 +559,18 @@ def test_spectral_inverse_linear_matches_separate_kernels(gpu, N, r, m, act):
     _, _, _, fwi = dft_tables(r, m, gpu)
     got = dm.spectral_inverse_linear(U, dm.inverse_table_operand(fwi), x, w, b, act)
     y = dm.truncated_dft_rows_inverse(U, fwi, planar=True)
-    want = fused_linear(x, w, b, act or "none", y)
+    activate = {None: lambda t: t, "relu": torch.relu, "silu": torch.nn.functional.silu}[act]
+    parts = (lambda bias: fused_linear(x, w, bias, act or "none", y)) if C == 64 else \
+        (lambda bias: activate(x @ w + (0 if bias is None else bias) + y))
+    want = parts(b)
     assert got.shape == want.shape
-    assert (got - want).abs().max().item() <= 2e-6 * max(1.0, want.abs().max().item())
+    tol = 2e-6 if C == 64 else 1e-5  # the library product behind the 32-channel comparison may not be plain fp32
+    assert (got - want).abs().max().item() <= tol * max(1.0, want.abs().max().item())
     # and against float64 arithmetic
     y64 = torch.einsum("wj,njho->nhwo", fwi.double(), U.double())
     z = x.double() @ w.double() + b.double() + y64
     z = torch.relu(z) if act == "relu" else (z * torch.sigmoid(z) if act == "silu" else z)
     assert (got.double() - z).abs().max().item() <= 1e-5 * max(1.0, z.abs().max().item())
     no_bias = dm.spectral_inverse_linear(U, dm.inverse_table_operand(fwi), x, w, None, act)
-    want_nb = fused_linear(x, w, None, act or "none", y)
-    assert (no_bias - want_nb).abs().max().item() <= 2e-6 * max(1.0, want_nb.abs().max().item())
+    want_nb = parts(None)
+    assert (no_bias - want_nb).abs().max().item() <= tol * max(1.0, want_nb.abs().max().item())

@@ -135,6 +135,55 @@ def test_full_model_vs_oracle_mid_size(gpu, r, ra):
     assert rel_l2(got.cpu().double(), want) < TOL
 
 
+def test_full_model_reference_yaml_defaults(gpu):
+    """The reference's own default configuration (config/darcy_config.yaml with config_accessor.py:15-40 applied:
+    R = 421, subsample_node 3 -> r = 141, subsample_attn 6 -> r_attn = 71, 6 encoder layers, spectral width 32,
+    ceil(sqrt(141)) = 12 modes), drop rates 0, random init, against the oracle in fp64."""
+    torch.manual_seed(5)
+    r, ra = 141, 71
+    cfg = dict(
+        drop_module=0.0, boundary_condition="dirichlet", target_normalizer=SM.UnitNormalizer(),
+        resolution_size=O.resolution_sizes(r, ra), dim_node=1, dim_hidden=128, drop_downscaler=0.0,
+        acti_downscaler="relu", num_encoder_layer=6, num_head=4, dim_position=2, attn_norm_eps=1e-6,
+        drop_encoder_attn=0.0, drop_encoder_attn_fc=0.0, attn_xavier=0.01, attn_diagonal=0.01, attn_symmetric=False,
+        dim_encoder_ffn=256, drop_encoder_ffn=0.0, acti_encoder_ffn="relu", drop_upscaler=0.0, acti_upscaler="silu",
+        num_decoder_layer=2, dim_target=1, dim_spatial_hidden=32, num_frequence_mode=12, drop_decoder_layer=0.0,
+        acti_decoder_layer="silu")
+    m = SM.Sp_GalerkinTransformer2D(cfg)
+    sd = {k: v.clone() for k, v in m.state_dict().items()}
+    x = torch.randn(2, r, r, 1, generator=torch.Generator().manual_seed(6))
+    lin = lambda n: torch.linspace(0, 1, n)
+    mesh = lambda n: torch.stack(torch.meshgrid(lin(n), lin(n), indexing="ij"), dim=-1)[None].repeat(2, 1, 1, 1)
+    pos, grid = mesh(ra), mesh(r)
+    po = {k: (v.double().t() if k.rsplit(".", 1)[-1] in ("weight_Q", "weight_K", "weight_V") else v.double())
+          for k, v in sd.items()}
+    want = O.galerkin_transformer_2d(po, cfg, x.double(), pos.double(), grid.double(), weight_layout="sp")
+    m = m.to(gpu).eval()
+    with torch.no_grad():
+        got = m(x.to(gpu), pos.to(gpu), grid.to(gpu))
+    assert rel_l2(got.cpu().double(), want) < TOL
+
+
+@pytest.mark.parametrize("N,r,width,modes", [(1, 421, 32, 21), (1, 512, 32, 23), (2, 211, 64, 15), (2, 141, 32, 12)])
+@pytest.mark.parametrize("truncated", [True, False])
+def test_spectral_conv_reference_default_modes(gpu, N, r, width, modes, truncated):
+    """Sp_SpectralConv2D at the mode counts config_accessor.py:39 derives (ceil(sqrt(r)): 21 at r = 421, 23 at 512,
+    15 at 211, 12 at 141) and the yaml's width 32, both routes, against the oracle's rfft2 / irfft2 in fp64."""
+    torch.manual_seed(7)
+    layer = L.Sp_SpectralConv2D(width, width, modes, 0.0, "silu")
+    with torch.no_grad():
+        for w in layer.fourier_weight:
+            w.copy_(torch.randn(w.shape) / width)
+    sd = {k: v.clone().double() for k, v in layer.state_dict().items()}
+    x = torch.randn(N, r, r, width, generator=torch.Generator().manual_seed(8))
+    want = O.spectral_conv2d(sd, x.double(), modes, "silu", weight_layout="sp")
+    layer = layer.to(gpu).eval()
+    layer.use_truncated_dft = truncated
+    with torch.no_grad():
+        got = layer(x.to(gpu))
+    assert max_rel(got.cpu().double(), want) < TOL
+
+
 def test_deferred_upsampling_matches_module_order(gpu):
     """The decoder's input layer in front of the up-scaler's last interpolation (a Linear over the channels commutes
     with it) against the reference's order of the same modules (network/model.py:59-64, network/sp_model.py:60):
