@@ -575,14 +575,11 @@ struct FusedPlan {
 constexpr int kU1 = 4;  // 16 tokens per unrolled group in pass 1
 constexpr int kU2 = 2;  // 32 tokens per unrolled group in pass 2
 
-// Workgroups per pass: three per compute unit.  Measured on MI355X (256 CUs) at
-// B=8, S=44521: counts that are whole multiples of the CU count (512, 768, 1024)
-// beat those in between by 3-10 %, and 768 is the fastest of them.
-#ifdef SPGT_TUNING
-int g_target_wg1 = 0, g_target_wg2 = 0;
-#else
-constexpr int g_target_wg1 = 0, g_target_wg2 = 0;
-#endif
+// Workgroups of the 256-thread plans: three per compute unit in the K/V pass, four in the Q pass.  Measured on
+// MI355X (256 CUs) at B=8, S=44521 with inputs and outputs that change from call to call: counts that are whole
+// multiples of the CU count beat those in between by 3-10 %; the Q pass takes 77 / 74.6 us with 768 / 1024
+// workgroups without position channels and 90 / 83 us with them (512: 94 us, 1280: 97 us, 1536: 89 us).
+constexpr int g_target_wg1 = 0;
 
 // Long sequences give every wave of a 1024-thread workgroup (4 heads x 4 sub-ranges) enough tokens: one
 // workgroup per CU then, whose four tiles per head are summed in LDS before they go to memory.
@@ -603,7 +600,7 @@ FusedPlan make_plan(int B, int S, int H) {
     const int dflt = 3 * cus;
     FusedPlan p;
     const int g1 = 4 * kU1, g2 = 16 * kU2;
-    const int t2 = g_target_wg2 > 0 ? g_target_wg2 : dflt;
+    const int t2 = 4 * cus;
     const int per_bh2 = std::max(1, t2 / bg);
     p.tpc2 = std::max(g2, ceil_div(ceil_div(S, per_bh2), g2) * g2);
     p.nchunk2 = ceil_div(S, p.tpc2);

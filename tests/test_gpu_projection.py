@@ -18,7 +18,9 @@ def rnd(*shape, seed=0):
 
 @pytest.mark.parametrize("dp", [0, 2])
 @pytest.mark.parametrize("B,S,Dm", [(1, 1, 128), (2, 50, 128), (1, 777, 128), (3, 4099, 128), (2, 130, 256),
-                                    (2, 97, 384), (1, 333, 512)])
+                                    (2, 97, 384), (1, 333, 512),
+                                    # long inputs: ragged last tiles, many short sequences, one long sequence
+                                    (3, 30011, 128), (1024, 65, 128), (1100, 64, 128), (1, 65537, 128)])
 def test_projection_vs_oracle(gpu, dp, B, S, Dm):
     H = Dm // 32
     x, W, b = rnd(B, S, Dm, seed=1), rnd(Dm, Dm, seed=2) / Dm ** 0.5, rnd(Dm, seed=3)
@@ -34,7 +36,9 @@ def test_projection_vs_oracle(gpu, dp, B, S, Dm):
 
 @pytest.mark.parametrize("dp", [0, 2])
 @pytest.mark.parametrize("B,S,Dm", [(1, 1, 128), (2, 50, 128), (1, 777, 128), (3, 4099, 128), (2, 130, 256),
-                                    (2, 97, 384), (1, 333, 512)])
+                                    (2, 97, 384), (1, 333, 512),
+                                    # long inputs: ragged last tiles, many short sequences, one long sequence
+                                    (3, 30011, 128), (1024, 65, 128), (1100, 64, 128), (1, 65537, 128)])
 def test_projection_layernorm_vs_oracle(gpu, dp, B, S, Dm):
     H = Dm // 32
     x, W, b = rnd(B, S, Dm, seed=5), rnd(Dm, Dm, seed=6) / Dm ** 0.5, rnd(Dm, seed=7)
@@ -60,6 +64,16 @@ def test_projection_identity_weight_is_exact(gpu):
     got = ga.multihead_projection_with_position_rrc_cuda(
         x.to(gpu), torch.eye(Dm, device=gpu), torch.zeros(Dm, device=gpu), torch.zeros(B, S, 0, device=gpu), H, 32, 0)
     assert torch.equal(got.cpu(), x.view(B, S, H, 32).permute(0, 2, 3, 1))
+
+
+def test_projection_identity_weight_is_exact_on_long_inputs(gpu):
+    B, S, Dm, H = 5, 20001, 128, 4
+    x = rnd(B, S, Dm, seed=14)
+    pos = torch.rand(B, S, 2, generator=torch.Generator().manual_seed(15))
+    got = ga.multihead_projection_with_position_rrc_cuda(
+        x.to(gpu), torch.eye(Dm, device=gpu), torch.zeros(Dm, device=gpu), pos.to(gpu), H, 32, 2)
+    assert torch.equal(got[:, :, 2:].cpu(), x.view(B, S, H, 32).permute(0, 2, 3, 1))
+    assert torch.equal(got[:, :, :2].cpu(), pos.transpose(1, 2)[:, None].expand(B, H, 2, S))
 
 
 def test_layernorm_constant_rows_give_bias(gpu):
