@@ -293,9 +293,10 @@ def fno_stack_bench(dev, with_cpu):
     return res
 
 
-def kernel_rooflines(dev):
+def kernel_rooflines(dev, use_graph=True):
     """Every operator of the path at its benchmark shape: algorithmic bytes (or flops), time from HIP events on the
-    launch stream, and the fraction of the bounding peak (HBM 8 TB/s; fp32 MFMA 157.3 TFLOP/s)."""
+    launch stream, and the fraction of the bounding peak (HBM 8 TB/s; fp32 MFMA 157.3 TFLOP/s).  use_graph=False
+    launches eagerly (for runs under a profiler, which then sees plain dispatches)."""
     import torch
     from spgt_amd.extension.bind import datamove as dm
     from spgt_amd.extension.bind import galerkin_attention as ga
@@ -308,6 +309,8 @@ def kernel_rooflines(dev):
         torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         try:
+            if not use_graph:
+                raise RuntimeError("eager launches requested")
             side = torch.cuda.Stream()
             side.wait_stream(torch.cuda.current_stream())
             with torch.cuda.stream(side):
@@ -493,7 +496,14 @@ def main():
     torch.cuda.set_device(dev)
 
     if args.only == "kernels":
-        print(json.dumps({"kernel_rooflines": kernel_rooflines(dev)}))
+        if args.calibrate_copy:
+            src = torch.empty(256 * 1024 * 1024 // 4, device=dev).normal_()
+            dst = torch.empty_like(src)
+            for _ in range(5):
+                dst.copy_(src)  # reads 256 MiB, writes 256 MiB
+            torch.cuda.synchronize()
+            del src, dst
+        print(json.dumps({"kernel_rooflines": kernel_rooflines(dev, use_graph=False)}))
         return
     if args.only == "darcy":
         print(json.dumps({"darcy_inference": darcy_bench(dev, with_cpu=False, steps=max(1, min(args.steps, 20)),
