@@ -38,15 +38,20 @@ Operator-level layouts (what the reference's CUDA extension returns):
   op_transpose_scatter_dual .... extension/bind/datamove.cu:46-64
   op_spectral_conv2d_sp ........ network/sp_layer.py:125-156
 
-Pinning status (see tests/test_oracle_*.py and tests/golden/):
-  * arithmetic pieces are pinned by closed forms, brute-force loops on tiny
-    inputs and library identities;
-  * the composition of modules (concat orders, channel splits, boundary
-    handling) is pinned by golden vectors written from the reference's own
-    network/layer.py and network/model.py by tests/golden/make_golden.py;
-  * third-party arithmetic below torch (FFT, BLAS, convolution) is whatever
-    the installed torch build provides: parity unpinned against the
-    reference's PyTorch 2.1 / CUDA 11.8 stack, which is not available.
+Pinning status: every function here has a CPU-side check in tests/ that does not retype its formula.
+  * golden vectors written from the reference's own network/layer.py and network/model.py by
+    tests/golden/make_golden.py (tests/test_oracle_golden.py): project_heads, project_layernorm_heads,
+    galerkin_attention (the attention's three static pieces), attention_module, encoder_layer (and through it
+    feed_forward, _act), spectral_conv2d, op_spectral_conv2d_sp, down_scaler, up_scaler (and through them conv_block,
+    _interp), galerkin_transformer_2d (and through it encoder_mixer, decoder_regressor, _with_position);
+  * closed forms, brute-force loops on tiny inputs and library identities (tests/test_oracle_closed_forms.py):
+    galerkin_attention, project_heads, project_layernorm_heads, complex_mode_product, spectral_conv2d,
+    bilinear_align_corners, resolution_sizes and every op_* layout function;
+  * tests/test_oracle_pins.py: attention_core_token_major and attention_ktv (reference golden vectors and a
+    three-loop product), the invsigma orientation of op_projection_layernorm_rrc with a non-symmetric weight,
+    gauss_inverse_transform by hand, galerkin_transformer_2d with a normalizer's mean and std.
+  The library routines below torch (FFT, GEMM, convolution) are taken as given: they are the routines the
+  reference itself calls.
 """
 import math
 
