@@ -391,7 +391,7 @@ int spgt_linear_forward(const float* x, int64_t ldx, const float* weight_kn, con
                         int64_t out_plane_stride, int64_t tokens, int in_features, int out_features,
                         spgt_stream_t stream);
 
-/* 1 when spgt_ffn_scalar_forward has a kernel for this shape (in_features 64 or 128,
+/* 1 when spgt_ffn_scalar_forward has a kernel for this shape (in_features 32, 64 or 128,
  * hidden_features 128 or 256), else 0. */
 int spgt_ffn_scalar_supported(int in_features, int hidden_features);
 

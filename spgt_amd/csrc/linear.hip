@@ -1281,7 +1281,8 @@ extern "C" int spgt_linear_forward(const float* x, int64_t ldx, const float* wei
 }
 
 extern "C" int spgt_ffn_scalar_supported(int in_features, int hidden_features) {
-    return ((in_features == 64 || in_features == 128) && (hidden_features == 128 || hidden_features == 256)) ? 1 : 0;
+    return ((in_features == 32 || in_features == 64 || in_features == 128) &&
+            (hidden_features == 128 || hidden_features == 256)) ? 1 : 0;
 }
 
 extern "C" int spgt_ffn_scalar_forward(const float* x, int64_t ldx, const float* weight1_kn, const float* bias1,
@@ -1292,7 +1293,7 @@ extern "C" int spgt_ffn_scalar_forward(const float* x, int64_t ldx, const float*
     if (tokens < 0) return fail(SPGT_ERR_INVALID_ARGUMENT, "ffn_scalar_forward: negative token count");
     if (!spgt_ffn_scalar_supported(in_features, hidden_features))
         return fail(SPGT_ERR_INVALID_ARGUMENT,
-                    "ffn_scalar_forward: in_features must be 64 or 128 and hidden_features 128 or 256");
+                    "ffn_scalar_forward: in_features must be 32, 64 or 128 and hidden_features 128 or 256");
     if (activation != SPGT_ACT_NONE && activation != SPGT_ACT_RELU && activation != SPGT_ACT_SILU)
         return fail(SPGT_ERR_INVALID_ARGUMENT, "ffn_scalar_forward: unknown activation");
     if (ldx < in_features || (ldx & 3) || !aligned16(x) || !aligned4(out) || !aligned4(weight1_kn) ||
@@ -1302,8 +1303,9 @@ extern "C" int spgt_ffn_scalar_forward(const float* x, int64_t ldx, const float*
     if (tokens == 0) return SPGT_OK;
 #define SPGT_FFN(KV, CB) \
     launch_ffn_scalar<KV, CB>(x, ldx, weight1_kn, bias1, weight2, bias2, activation, out, tokens, stream)
-    if (in_features == 64) { if (hidden_features == 128) SPGT_FFN(64, 1); else SPGT_FFN(64, 2); }
-    else                   { if (hidden_features == 128) SPGT_FFN(128, 1); else SPGT_FFN(128, 2); }
+    if (in_features == 32)      { if (hidden_features == 128) SPGT_FFN(32, 1); else SPGT_FFN(32, 2); }
+    else if (in_features == 64) { if (hidden_features == 128) SPGT_FFN(64, 1); else SPGT_FFN(64, 2); }
+    else                        { if (hidden_features == 128) SPGT_FFN(128, 1); else SPGT_FFN(128, 2); }
 #undef SPGT_FFN
     return check_launch("ffn_scalar_forward");
 }

@@ -156,7 +156,7 @@ def test_linear_errors(gpu):
     assert out.shape == (0, 128)
 
 
-@pytest.mark.parametrize("K,HID", [(64, 256), (64, 128), (128, 256), (128, 128)])
+@pytest.mark.parametrize("K,HID", [(64, 256), (64, 128), (128, 256), (128, 128), (32, 128), (32, 256)])
 @pytest.mark.parametrize("T", [1, 45, 5000])
 @pytest.mark.parametrize("act", ["relu", "silu"])
 def test_ffn_scalar(gpu, K, HID, T, act):
