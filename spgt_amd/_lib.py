@@ -119,6 +119,17 @@ def load():
     return _lib
 
 
+def open_library(path: str):
+    """A handle to a build of the library at `path` with every entry point's signature set; not cached and not
+    used by the operators (tests compare builds with it)."""
+    lib = ctypes.CDLL(path)
+    for name, (restype, argtypes) in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = restype
+        fn.argtypes = argtypes
+    return lib
+
+
 def last_error() -> str:
     return load().spgt_last_error().decode("utf-8", "replace")
 

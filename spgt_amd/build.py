@@ -11,6 +11,10 @@ import sys
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC_DIR = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "libspgt_hip.so")
+# The same library with the hand-written MFMA statements of linear.hip replaced by the compiler's intrinsic:
+# test infrastructure (tests compare the two bit for bit), never loaded by the package.
+CHECK_LIB_PATH = os.path.join(PKG_DIR, "libspgt_hip_mfma_check.so")
+CHECK_SOURCE, CHECK_DEFINE = "linear.hip", "-DSPGT_MFMA_BUILTIN=1"
 
 SOURCES = [
     "spgt_host.cpp",
@@ -60,29 +64,33 @@ def build(verbose: bool = False, incremental: bool = False, jobs: int = 8) -> st
         # hipcc's host pass does not know the device-only feature name and says so.
         return "\n".join(l for l in text.splitlines() if "not a recognized feature" not in l)
 
-    def compile_one(name):
+    def compile_one(job):
+        name, defines, suffix = job
         src = os.path.join(CSRC_DIR, name)
-        obj = os.path.join(obj_dir, name + ".o")
+        obj = os.path.join(obj_dir, name + suffix + ".o")
         if incremental and os.path.exists(obj) and os.path.getmtime(obj) > max(os.path.getmtime(src), hdr_mtime):
             return obj, ""
-        cmd = [hipcc, *flags, "-x", "hip", "-c", src, "-o", obj]
+        cmd = [hipcc, *flags, *defines, "-x", "hip", "-c", src, "-o", obj]
         proc = subprocess.run(cmd, cwd=CSRC_DIR, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
         if proc.returncode != 0:
             raise RuntimeError("hipcc failed:\n" + " ".join(cmd) + "\n" + clean(proc.stdout))
         return obj, clean(proc.stdout)
 
+    work = [(name, [], "") for name in SOURCES] + [(CHECK_SOURCE, [CHECK_DEFINE], ".builtin")]
     with ThreadPoolExecutor(max_workers=max(1, jobs)) as pool:
-        results = list(pool.map(compile_one, SOURCES))
-    objs = [o for o, _ in results]
+        results = list(pool.map(compile_one, work))
+    objs = [o for o, _ in results[:-1]]
+    check_objs = [results[-1][0] if name == CHECK_SOURCE else o for name, o in zip(SOURCES, objs)]
     log = "\n".join(t for _, t in results if t.strip())
-    tmp = LIB_PATH + ".tmp"
-    cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", tmp]
-    proc = subprocess.run(cmd, cwd=CSRC_DIR, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    if proc.returncode != 0:
-        raise RuntimeError("link failed:\n" + " ".join(cmd) + "\n" + clean(proc.stdout))
+    for path, members in ((LIB_PATH, objs), (CHECK_LIB_PATH, check_objs)):
+        tmp = path + ".tmp"
+        cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *members, "-o", tmp]
+        proc = subprocess.run(cmd, cwd=CSRC_DIR, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+        if proc.returncode != 0:
+            raise RuntimeError("link failed:\n" + " ".join(cmd) + "\n" + clean(proc.stdout))
+        os.replace(tmp, path)
     if verbose and log.strip():
         print(log)
-    os.replace(tmp, LIB_PATH)
     return LIB_PATH
 
 

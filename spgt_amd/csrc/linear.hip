@@ -622,6 +622,21 @@ __global__ __launch_bounds__(256) void ffn_scalar_k(
 // cycles per instruction measured).  The compiler does not see an MFMA in these statements, so the wait states
 // it would insert are written out: two before (operand just written by a vector instruction), and
 // mfma_acc_done() before the accumulator is read (an MFMA of 16 passes needs 18 after it).
+// With SPGT_MFMA_BUILTIN the same helpers are the compiler's intrinsic (which it schedules and protects itself):
+// the build makes a second library from that form, and a test compares the two bit for bit, so that a compiler
+// change that breaks the hand-counted wait states shows up as a failing test.
+#ifdef SPGT_MFMA_BUILTIN
+__device__ __forceinline__ void mfma32_acc_first(v16f& acc, float w, float x) {
+    v16f zero;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) zero[i] = 0.f;
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(w, x, zero, 0, 0, 0);
+}
+__device__ __forceinline__ void mfma32_acc(v16f& acc, float w, float x) {
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(w, x, acc, 0, 0, 0);
+}
+__device__ __forceinline__ void mfma_acc_done(v16f&) {}
+#else
 __device__ __forceinline__ void mfma32_acc_first(v16f& acc, float w, float x) {
     asm volatile("s_nop 1\n\tv_mfma_f32_32x32x2_f32 %0, %1, %2, 0" : "=a"(acc) : "a"(w), "v"(x));
 }
@@ -629,6 +644,7 @@ __device__ __forceinline__ void mfma32_acc(v16f& acc, float w, float x) {
     asm volatile("s_nop 1\n\tv_mfma_f32_32x32x2_f32 %0, %1, %2, %0" : "+a"(acc) : "a"(w), "v"(x));
 }
 __device__ __forceinline__ void mfma_acc_done(v16f& acc) { asm volatile("s_nop 15\n\ts_nop 7" : "+a"(acc)); }
+#endif
 
 // The tail of an encoder layer after the attention core, one launch per layer
 // (Sp_EncoderLayer.forward, network/sp_layer.py:97-103, with the attention's fc_layer, :75, and
@@ -909,12 +925,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 }
 
 // The weight operand in a vector register, the accumulator in accumulation registers.
+#ifdef SPGT_MFMA_BUILTIN
+__device__ __forceinline__ void mfma32_accv_first(v16f& acc, float w, float x) { mfma32_acc_first(acc, w, x); }
+__device__ __forceinline__ void mfma32_accv(v16f& acc, float w, float x) { mfma32_acc(acc, w, x); }
+#else
 __device__ __forceinline__ void mfma32_accv_first(v16f& acc, float w, float x) {
     asm volatile("s_nop 1\n\tv_mfma_f32_32x32x2_f32 %0, %1, %2, 0" : "=a"(acc) : "v"(w), "v"(x));
 }
 __device__ __forceinline__ void mfma32_accv(v16f& acc, float w, float x) {
     asm volatile("s_nop 1\n\tv_mfma_f32_32x32x2_f32 %0, %1, %2, %0" : "+a"(acc) : "v"(w), "v"(x));
 }
+#endif
 
 // Wide linear layers on long inputs with every weight resident (the structure of encoder_tail_k):
 //   out[t, n] = act(x[t, :] . W[:, n] + bias[n]),  in_features 128, out_features 128*NCB,

@@ -245,3 +245,45 @@ def test_linear_long_inputs_wide_output_without_planes_or_bias(gpu, act):
     assert got.shape == (T, 384)
     assert (got.double() - want).abs().max().item() <= 1e-5 * max(1.0, want.abs().max().item())
     assert torch.equal(got, fused_linear(x, w, None, act))
+
+
+def test_hand_written_mfma_statements_match_the_compilers_intrinsic(gpu):
+    """linear_resident_k and encoder_tail_k issue their MFMAs as assembly statements with hand-counted wait states,
+    which the compiler's hazard recognizer does not see.  The build makes a second library in which the same
+    helpers are the compiler's intrinsic; the two must agree bit for bit on the kernels that use them (same
+    instruction, same operands, same order), so a toolchain change that breaks the hand-written form fails here."""
+    import os
+    from spgt_amd import _lib, build
+    from spgt_amd.extension.bind.linear import fused_encoder_tail, fused_encoder_tail_folded, fused_linear
+    assert os.path.exists(build.CHECK_LIB_PATH), "build the library with `python -m spgt_amd.build`"
+    main, check = _lib.load(), _lib.open_library(build.CHECK_LIB_PATH)
+
+    def on(lib, fn):
+        _lib._lib = lib
+        try:
+            return fn()
+        finally:
+            _lib._lib = main
+
+    g = torch.Generator().manual_seed(2024)
+    T = 70001
+    x = torch.randn(T, 128, generator=g).to(gpu)
+    w = (torch.randn(128, 384, generator=g) / 128 ** 0.5).to(gpu)
+    b = torch.randn(384, generator=g).to(gpu)
+    for act in ("none", "silu"):
+        for planes in (1, 3):
+            call = lambda: fused_linear(x, w, b, act, planes=planes)  # 128 -> 384 on a long input: linear_resident_k
+            assert torch.equal(on(main, call), on(check, call))
+    for K1 in (128, 136):
+        a = torch.randn(T, K1, generator=g).to(gpu)
+        wfc, bfc = (torch.randn(K1, 128, generator=g) / K1 ** 0.5).to(gpu), torch.randn(128, generator=g).to(gpu)
+        w1, b1 = (torch.randn(128, 256, generator=g) / 128 ** 0.5).to(gpu), torch.randn(256, generator=g).to(gpu)
+        w2, b2 = (torch.randn(256, 128, generator=g) / 16.0).to(gpu), torch.randn(128, generator=g).to(gpu)
+        call = lambda: fused_encoder_tail(a, x, wfc, bfc, w1, b1, w2, b2, "silu")
+        assert torch.equal(on(main, call), on(check, call))
+    B, S = 3, 23333
+    q, xr = torch.randn(B, S, 128, generator=g).to(gpu), torch.randn(B, S, 128, generator=g).to(gpu)
+    pos = torch.rand(B, S, 2, generator=g).to(gpu)
+    ffc, fpos = (torch.randn(B, 128, 128, generator=g) / 11.0).to(gpu), torch.randn(B, 2, 128, generator=g).to(gpu)
+    call = lambda: fused_encoder_tail_folded(q, pos, xr, ffc, fpos, bfc, w1, b1, w2, b2, "relu")
+    assert torch.equal(on(main, call), on(check, call))
