@@ -298,9 +298,10 @@ template <int D>
 __global__ __launch_bounds__(256) void qm_apply_fm(const float* __restrict__ Q, const float* __restrict__ M,
                                                    float* __restrict__ out, int S, int tokens_per_chunk) {
     constexpr int DP = D - 32;
-    // D == 34: a wave stages the 64 x 34 output rows of a unit in its own LDS slice and writes them
-    // out as one contiguous 8704-byte run (rows of 136 bytes would otherwise go out in 8-byte pieces).
-    constexpr int kStagePitch = 36;
+    // D == 34: a wave stages the 64 x 34 output rows of a unit in its own LDS slice, laid out as they are in
+    // memory, and copies the contiguous 8704-byte run with 16-byte accesses (rows of 136 bytes would otherwise
+    // go out in 8-byte pieces); the run starts at a multiple of 8 bytes only (S * 136 bytes per (batch, head)).
+    constexpr int kStagePitch = 34;
     __shared__ __attribute__((aligned(16))) float stage_all[DP == 2 ? 4 * 64 * kStagePitch : 4];
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
@@ -446,12 +447,16 @@ __global__ __launch_bounds__(256) void qm_apply_fm(const float* __restrict__ Q, 
             // the wave's own LDS slice: program order is enough, no barrier
             const int ntok = min(64, s1 - sb);
             float* dst = ob + (int64_t)sb * D;
-            constexpr int R2 = D / 2;  // float2 per token row
-            for (int e = lane; e < ntok * R2; e += 64) {
-                const int tok = e / R2;
-                const int c2 = e - tok * R2;
-                const float2 v = *reinterpret_cast<const float2*>(stage + tok * kStagePitch + 2 * c2);
-                st_stream<true>(reinterpret_cast<float2*>(dst + (int64_t)tok * D + 2 * c2), v);
+            typedef v4f v4f_a8 __attribute__((aligned(8)));
+            const int n4 = ntok * D / 4;  // whole 16-byte pieces of the run
+            for (int e = lane; e < n4; e += 64) {
+                const v4f v = *reinterpret_cast<const v4f_a8*>(stage + 4 * e);
+                __builtin_nontemporal_store(v, reinterpret_cast<v4f_a8*>(dst + 4 * e));
+            }
+            if ((ntok * D) & 2) {  // an odd number of tokens leaves one 8-byte piece
+                if (lane == 0)
+                    st_stream<true>(reinterpret_cast<float2*>(dst + 4 * n4),
+                                    *reinterpret_cast<const float2*>(stage + 4 * n4));
             }
         }
     };
