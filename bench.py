@@ -577,7 +577,7 @@ def main():
     q_bytes = 2 * B * H * 32 * S * 4
     qd = dist([st[2] for st in stages])
     roofline = {
-        "bound": "hbm", "kernel": "ktv_ln_partial_tm<0,4>", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
+        "bound": "hbm", "kernel": "ktv_ln_partial_tm<0,4,4>", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
         "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": recorded_kv_pass_traffic(),
         "traffic_source": "recorded: rocprofv3 FETCH_SIZE + WRITE_SIZE summary under profiles/ for this kernel and "
                           "shape (counters need runs of their own), not a reading of this run",
