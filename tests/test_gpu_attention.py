@@ -43,7 +43,10 @@ def fused_reference(q, k, v, pos, gK, bK, gV, bV, eps, H, dp, dtype=torch.float6
 
 
 @pytest.mark.parametrize("dp", [0, 2])
-@pytest.mark.parametrize("B,S,H", [(1, 1, 4), (2, 50, 4), (1, 777, 4), (3, 4099, 4), (2, 1000, 8)])
+@pytest.mark.parametrize("B,S,H", [(1, 1, 4), (2, 50, 4), (1, 777, 4), (3, 4099, 4), (2, 1000, 8),
+                                   # long sequences: the K/V pass runs 1024-thread workgroups whose four token
+                                   # sub-ranges per head meet in LDS; ragged last chunks, two head groups
+                                   (2, 150001, 4), (1, 140003, 8)])
 def test_fused_attention_vs_oracle(gpu, dp, B, S, H):
     C = H * 32
     q, k, v = rnd(B, S, C, seed=1), rnd(B, S, C, seed=2) * 1.7 + 0.3, rnd(B, S, C, seed=3) * 0.6 - 0.2

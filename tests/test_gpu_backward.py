@@ -16,7 +16,10 @@ def rnd(*shape, seed=0):
 
 
 @pytest.mark.parametrize("d", [32, 34])
-@pytest.mark.parametrize("B,H,S", [(1, 1, 1), (2, 4, 50), (1, 3, 777), (2, 2, 4099)])
+@pytest.mark.parametrize("B,H,S", [(1, 1, 1), (2, 4, 50), (1, 3, 777), (2, 2, 4099),
+                                   # chunks of several 128-token blocks per wave, ragged tails: (8, 4, 20011) gives a
+                                   # wave two blocks, the benchmark shape four
+                                   (8, 4, 20011), (8, 4, 44521)])
 def test_attention_backward(gpu, d, B, H, S):
     Q, K, V, G = rnd(B, H, d, S, seed=1), rnd(B, H, d, S, seed=2), rnd(B, H, d, S, seed=3), rnd(B, H, S, d, seed=4)
     q, k, v = (t.double().requires_grad_(True) for t in (Q, K, V))
