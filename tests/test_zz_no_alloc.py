@@ -48,12 +48,15 @@ def _call(lib, static, q, k, v, pos, aff, eps, B, S, H, dp):
     return out, ktv
 
 
+# two calls in a row, the second smaller than the first; the second pair starts on the long-sequence plan of the
+# K/V pass (1024-thread workgroups) and falls back to the short one
+@pytest.mark.parametrize("calls", [[(3, 6007), (2, 1531)], [(2, 150001), (1, 9001)]])
 @pytest.mark.parametrize("dp", [0, 2])
-def test_static_scratch_entry_point_matches_workspace_entry_point(gpu, dp):
+def test_static_scratch_entry_point_matches_workspace_entry_point(gpu, dp, calls):
     lib = _lib.load()
     H, eps = 4, 1e-6
     assert lib.spgt_galerkin_attention_fused_static_max_bytes() == 16 << 20
-    for call, (B, S) in enumerate([(3, 6007), (2, 1531)]):  # second call smaller than the first
+    for call, (B, S) in enumerate(calls):
         print(f"static scratch: call {call} B={B} S={S} dp={dp}", flush=True)
         (q, k, v, pos), aff = _inputs(B, S, H, 100 + 10 * call, gpu)
         assert lib.spgt_galerkin_attention_fused_workspace_bytes(B, S, H, dp) <= 16 << 20
