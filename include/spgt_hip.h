@@ -131,10 +131,13 @@ int spgt_galerkin_attention_fused_forward(const float* Q, const float* K, const 
  * of spgt_galerkin_attention_fused_static_max_bytes() bytes (16 MiB) that is part of the library's
  * code object: every GPU the library runs on holds one copy until the process ends.  The call
  * allocates and frees nothing; a shape whose spgt_galerkin_attention_fused_workspace_bytes exceeds
- * the array is rejected with SPGT_ERR_WORKSPACE (B=8, S=44521, H=4 needs 12.6 MB).  All calls on
+ * the array is rejected with SPGT_ERR_WORKSPACE (B=8, S=44521, H=4 needs 4.2 MB).  All calls on
  * one GPU share that GPU's array: calls that overlap in time on one GPU (two streams, two threads)
- * race and must be serialised by the caller.  Arguments and results otherwise as
- * spgt_galerkin_attention_fused_forward (Q and out are required). */
+ * race and must be serialised by the caller.  The first call on a GPU does that GPU's one-time
+ * set-up on the host (hipGetSymbolAddress of the array, which may load the code object, and the
+ * K/V pass's dynamic-LDS attribute; both checked, SPGT_ERR_LAUNCH on failure): make one call on
+ * each GPU before capturing a graph or entering a section that must not allocate.  Arguments and
+ * results otherwise as spgt_galerkin_attention_fused_forward (Q and out are required). */
 size_t spgt_galerkin_attention_fused_static_max_bytes(void);
 int spgt_galerkin_attention_fused_forward_static(const float* Q, const float* K, const float* V,
                                                  int64_t ld_in, const float* position,
@@ -466,6 +469,21 @@ typedef struct {
  * weight as nine [Cin, Cout] taps), and the modules refresh all of them from the parameters with this call
  * at the start of a forward, so that a parameter changed in place by any means is never served stale. */
 int spgt_strided_copy_batch(const spgt_copy_desc* descs, int count, spgt_stream_t stream);
+
+/* Weight and bias gradients of y = x W + b from dL/dy on token-major operands: what the reference's
+ * projection backward computes with a library GEMM on the transposed input and a library reduction
+ * (extension/bind/galerkin_attention.cu:41-46).
+ *   x    : [tokens, in_features], row stride ldx floats (batch entry b at x + b * x_batch_stride; 0 = shared)
+ *   grad : [tokens, out_features], row stride ldg floats (batch entry b at grad + b * grad_batch_stride)
+ *   out  : per batch entry in_features * out_features + out_features floats, packed one after the other:
+ *          dW [in_features, out_features] row-major (dW[k][n] = sum_t x[t][k] grad[t][n]) followed by
+ *          db [out_features] (sum over the tokens)
+ * The sum over the tokens is split over at most 256 chunks whose partial results go to the workspace and
+ * are added in a fixed order: results are identical from run to run.  out_features must be a multiple of 4. */
+size_t spgt_linear_weight_grad_workspace_bytes(int64_t tokens, int in_features, int out_features, int batch);
+int spgt_linear_weight_grad(const float* x, int64_t ldx, int64_t x_batch_stride, const float* grad, int64_t ldg,
+                            int64_t grad_batch_stride, float* out, void* workspace, size_t workspace_bytes,
+                            int64_t tokens, int in_features, int out_features, int batch, spgt_stream_t stream);
 
 /* Instrumented variant of spgt_galerkin_attention_fused_forward for benchmarks (no reference
  * counterpart): enqueues the call `iterations` times back to back (no synchronisation between

@@ -281,9 +281,10 @@ def resolution_sizes(r_large, r_small):
     down/up sampling; mid = round(r_large * f) - 1 with f = sqrt(r_small/r_large)
     rounded to 4 decimals and then up to a multiple of 0.005 in the reference's
     particular way (which looks at the last printed digit)."""
-    factor = round(float(np.sqrt(r_small / r_large)), 4)
-    last_digit = float(repr(factor)[-1])
-    factor = round(factor, 3)
+    # np.sqrt returns a numpy scalar, whose round() is numpy's (scale, round half to even, unscale), not Python's
+    factor = np.sqrt(r_small / r_large).round(4)
+    last_digit = float(repr(float(factor))[-1])
+    factor = float(factor.round(3))
     if last_digit < 5:
         factor += 5.0e-3
     factor = int(factor / 5.0e-3 + 0.5) * 5.0e-3

@@ -24,7 +24,7 @@ SOURCES = [
     "splitk_gemm.hip",
     "projection.hip",
     "datamove.hip",
-    "spectral.hip", "spectral_dft.hip", "linear.hip",
+    "spectral.hip", "spectral_dft.hip", "linear.hip", "linear_backward.hip",
 ]
 
 # Packed fp32 VALU forms (v_pk_*_f32) are switched off for all device code.

@@ -243,14 +243,41 @@ __global__ __launch_bounds__(256) void layernorm_heads_backward_k(
     }
 }
 
-// out[c] = sum_blocks part[block][c], blocks in increasing order.  grid ceil(C/256), block 256.
-__global__ __launch_bounds__(256) void column_sum_k(const float* __restrict__ part, float* __restrict__ out, int C,
-                                                    int nblock) {
-    const int c = blockIdx.x * 256 + threadIdx.x;
-    if (c >= C) return;
+// out[c] = sum_blocks part[block][c] in a fixed order: sixteen interleaved chains (block = q, q + 16, ...), each
+// summed in increasing block order with eight loads in flight, then combined by a fixed binary tree.  (One thread
+// per column walking all blocks took 235 us for the 4096 blocks of 65 536 tokens: one dependent load at a time.)
+// grid ceil(C/64), block 1024 = 64 columns x 16 chains.
+__global__ __launch_bounds__(1024) void column_sum_k(const float* __restrict__ part, float* __restrict__ out, int C,
+                                                     int nblock) {
+    __shared__ float sm[16][64];
+    const int q = threadIdx.x >> 6;
+    const int c = blockIdx.x * 64 + (threadIdx.x & 63);
     float s = 0.f;
-    for (int b = 0; b < nblock; ++b) s += part[(int64_t)b * C + c];
-    out[c] = s;
+    if (c < C) {
+        const float* src = part + c;
+        for (int b0 = q; b0 < nblock; b0 += 16 * 8) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int b = b0 + 16 * u;
+                v[u] = b < nblock ? src[(int64_t)b * C] : 0.f;
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) s += v[u];
+        }
+    }
+    sm[q][threadIdx.x & 63] = s;
+    __syncthreads();
+    if (q == 0 && c < C) {
+        float t[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) t[i] = sm[i][threadIdx.x & 63];
+#pragma unroll
+        for (int w = 8; w >= 1; w /= 2)
+#pragma unroll
+            for (int i = 0; i < w; ++i) t[i] += t[i + w];
+        out[c] = t[0];
+    }
 }
 
 }  // namespace spgt
@@ -391,7 +418,7 @@ extern "C" int spgt_layernorm_heads_backward(const float* pre_ln, const float* g
     float* bpart = gpart + (size_t)nblock * C;
     hipLaunchKernelGGL(layernorm_heads_backward_k, dim3(nb, num_head / 4), dim3(256), 0, stream, pre_ln, grad_ln,
                        ln_weight, norm_eps, grad_pre_ln, gpart, bpart, tokens, num_head, tpb);
-    hipLaunchKernelGGL(column_sum_k, dim3(ceil_div(C, 256)), dim3(256), 0, stream, gpart, grad_ln_weight, C, nb);
-    hipLaunchKernelGGL(column_sum_k, dim3(ceil_div(C, 256)), dim3(256), 0, stream, bpart, grad_ln_bias, C, nb);
+    hipLaunchKernelGGL(column_sum_k, dim3(ceil_div(C, 64)), dim3(1024), 0, stream, gpart, grad_ln_weight, C, nb);
+    hipLaunchKernelGGL(column_sum_k, dim3(ceil_div(C, 64)), dim3(1024), 0, stream, bpart, grad_ln_bias, C, nb);
     return check_launch("layernorm_heads_backward");
 }

@@ -26,7 +26,7 @@
 #include <vector>
 
 // Size of the device array behind spgt_galerkin_attention_fused_forward_static (16 MiB: the headline shape
-// B=8, S=44521, H=4 needs 12.6 MB of partial tiles).
+// B=8, S=44521, H=4 needs 4.2 MB of partial tiles, one per 1024-thread workgroup and head).
 #ifndef SPGT_STATIC_SCRATCH_BYTES
 #define SPGT_STATIC_SCRATCH_BYTES (16u << 20)
 #endif
@@ -642,6 +642,29 @@ extern "C" size_t spgt_galerkin_attention_fused_workspace_bytes(int B, int S, in
 
 namespace {
 
+constexpr int kMaxDevices = 64;
+std::atomic<int> g_sub_lds_allowed[kMaxDevices];
+
+// The long-sequence K/V pass asks for 64 KiB (72 KiB with position channels) of dynamic LDS, which a kernel
+// must be allowed once per device.  Done on a device's first call (not a stream operation: callers that
+// capture graphs make one call outside the capture first); a failure is reported, not ignored.
+int allow_sub_range_lds() {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
+        return fail(SPGT_ERR_LAUNCH, "galerkin_attention_fused: no current device");
+    if (g_sub_lds_allowed[dev].load(std::memory_order_acquire)) return SPGT_OK;
+    const hipError_t e0 = hipFuncSetAttribute(reinterpret_cast<const void*>(&ktv_ln_partial_tm<0, kU1, kSub>),
+                                              hipFuncAttributeMaxDynamicSharedMemorySize,
+                                              (int)(kSub * 4 * 32 * 32 * sizeof(float)));
+    const hipError_t e2 = hipFuncSetAttribute(reinterpret_cast<const void*>(&ktv_ln_partial_tm<2, kU1, kSub>),
+                                              hipFuncAttributeMaxDynamicSharedMemorySize,
+                                              (int)(kSub * 4 * 34 * 34 * sizeof(float)));
+    if (e0 != hipSuccess || e2 != hipSuccess)
+        return fail(SPGT_ERR_LAUNCH, "galerkin_attention_fused: the K/V pass was refused its dynamic LDS size");
+    g_sub_lds_allowed[dev].store(1, std::memory_order_release);
+    return SPGT_OK;
+}
+
 // Validates, then enqueues the three launches.  With `ev` (4 events) an event
 // is recorded before the first launch (unless record_first is false: the caller
 // has recorded it already) and after each launch.
@@ -687,18 +710,11 @@ int fused_forward_impl(
     if (p.nsub > 1) {
         const dim3 block_sub(256 * kSub);
         const size_t lds = (size_t)kSub * 4 * D * D * sizeof(float);
+        if (int rc = allow_sub_range_lds()) return rc;
         if (dp == 0) {
-            static const hipError_t attr0 = hipFuncSetAttribute(
-                reinterpret_cast<const void*>(&ktv_ln_partial_tm<0, kU1, kSub>),
-                hipFuncAttributeMaxDynamicSharedMemorySize, (int)(kSub * 4 * 32 * 32 * sizeof(float)));
-            (void)attr0;
             hipLaunchKernelGGL((ktv_ln_partial_tm<0, kU1, kSub>), grid1, block_sub, lds, stream, K, V, pos, ln_weight_K,
                                ln_bias_K, ln_weight_V, ln_bias_V, norm_eps, partial, S, H, ld_in, p.tpc1);
         } else {
-            static const hipError_t attr2 = hipFuncSetAttribute(
-                reinterpret_cast<const void*>(&ktv_ln_partial_tm<2, kU1, kSub>),
-                hipFuncAttributeMaxDynamicSharedMemorySize, (int)(kSub * 4 * 34 * 34 * sizeof(float)));
-            (void)attr2;
             hipLaunchKernelGGL((ktv_ln_partial_tm<2, kU1, kSub>), grid1, block_sub, lds, stream, K, V, pos, ln_weight_K,
                                ln_bias_K, ln_weight_V, ln_bias_V, norm_eps, partial, S, H, ld_in, p.tpc1);
         }
@@ -745,15 +761,14 @@ constexpr size_t kStaticScratchBytes = SPGT_STATIC_SCRATCH_BYTES;
 // One copy per GPU the library's code object is loaded on, held until the process ends.
 static __device__ __align__(256) float scratch[kStaticScratchBytes / sizeof(float)];
 
-constexpr int kMaxDevices = 64;
-std::atomic<float*> g_scratch_ptr[kMaxDevices];
+std::atomic<float*> g_scratch_ptr[64];
 
 // Device address of `scratch` on the current device (looked up once per device), or null with the
 // error recorded.  The array's name is only a host-side handle for this lookup; every launch and
 // copy uses the pointer returned here.
 float* static_scratch_ptr() {
     int dev = -1;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) {
         (void)fail(SPGT_ERR_LAUNCH, "galerkin_attention_fused_static: no current device");
         return nullptr;
     }
@@ -793,6 +808,7 @@ extern "C" int spgt_galerkin_attention_fused_forward_static(
                     "spgt_galerkin_attention_fused_forward with a caller workspace");
     float* ws = static_scratch_ptr();
     if (!ws) return SPGT_ERR_LAUNCH;
+    if (int rc = allow_sub_range_lds()) return rc;  // with the lookup above: all one-time set-up of a device
     // Every partial tile the reduction reads is written by the K/V pass of the same call, so nothing
     // in the array has to start at zero.
     return fused_forward_impl(Q, K, V, ld_in, position, ln_weight_K, ln_bias_K, ln_weight_V, ln_bias_V, norm_eps,

@@ -1,0 +1,182 @@
+// Weight and bias gradients of a token-major Linear y = x W + b:
+//   dW[k][n] = sum_t x[t][k] g[t][n]        db[n] = sum_t g[t][n]
+// (reference: extension/bind/galerkin_attention.cu:41-46, where the two are a library GEMM on the
+// transposed input and a library reduction).  The contraction runs over the tokens, tens of thousands
+// to millions of them, against 128 x 128 results: a split over token chunks, each chunk's [K, N] tile
+// accumulated in MFMA registers straight from global memory (both operands are read with lanes along
+// the feature axis, 128-byte runs; no transpose of x is ever formed), then one deterministic
+// second-stage sum over the chunks (tile_reduce), bias gradient included.
+#include "spgt_device.h"
+#include "spgt_host.h"
+#include "spgt_kernels.h"
+
+namespace spgt {
+
+// partial[batch][chunk][k * N + n] = sum over the chunk's tokens of x[t][k] * g[t][n]
+// partial[batch][chunk][K * N + n] = sum over the chunk's tokens of g[t][n]
+// grid (nchunk, batch * nstrip, ceil(K / 128)), block 256: wave w takes rows k in [32 (4 z + w), +32) of the strip
+// of NT * 32 columns.  MFMA 32x32x2 step kk contracts tokens 2 kk and 2 kk + 1 of the chunk (lane half = token),
+// A = x[t][k0 + lane % 32], B = g[t][n0 + 32 nt + lane % 32].  Operand batches of BK steps are requested one
+// batch ahead of the MFMAs that consume them.
+template <int NT>
+__global__ __launch_bounds__(256) void xtg_partial_k(const float* __restrict__ X, int64_t ldx, int64_t x_batch,
+                                                     const float* __restrict__ G, int64_t ldg, int64_t g_batch,
+                                                     float* __restrict__ partial, int64_t T, int K, int N,
+                                                     int tokens_per_chunk, int nstrip) {
+    constexpr int BK = 8;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int tk = lane & 31;
+    const int kh = lane >> 5;
+    const int chunk = blockIdx.x;
+    const int nchunk = gridDim.x;
+    const int b = blockIdx.y / nstrip;
+    const int strip = blockIdx.y - b * nstrip;
+    const int k0 = (blockIdx.z * 4 + wave) * 32;
+    const int n0 = strip * NT * 32;
+    const int E = K * N + N;
+    if (k0 >= K) return;  // whole wave: no barrier follows
+    const int64_t t0 = (int64_t)chunk * tokens_per_chunk;
+    const int64_t t1 = min(T, t0 + tokens_per_chunk);
+    const int steps = (int)((t1 - t0 + 1) / 2);
+    // clamped feature indices: rows past K and columns past N read valid memory and are masked to zero
+    const bool kok = k0 + tk < K;
+    const float* xp = X + b * x_batch + t0 * ldx + min(k0 + tk, K - 1);
+    const float* gp = G + b * g_batch + t0 * ldg;
+    uint32_t goff[NT];
+    bool nok[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        nok[nt] = n0 + 32 * nt + tk < N;
+        goff[nt] = (uint32_t)min(n0 + 32 * nt + tk, N - 1);
+    }
+    v16f acc[NT];
+    float colsum[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        colsum[nt] = 0.f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[nt][r] = 0.f;
+    }
+    const int last = (int)(t1 - t0) - 1;  // last valid token of the chunk, relative
+    float xa[BK], ga[NT][BK], xb[BK], gb[NT][BK];
+    auto fetch = [&](float (&xv)[BK], float (&gv)[NT][BK], int batch) {
+#pragma unroll
+        for (int u = 0; u < BK; ++u) {
+            const int rel = 2 * (batch * BK + u) + kh;
+            const bool ok = rel <= last;
+            const int64_t tr = ok ? rel : last;
+            const float xval = xp[tr * ldx];
+            xv[u] = (ok && kok) ? xval : 0.f;
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                const float gval = gp[tr * ldg + goff[nt]];
+                gv[nt][u] = (ok && nok[nt]) ? gval : 0.f;
+            }
+        }
+    };
+    auto multiply = [&](const float (&xv)[BK], const float (&gv)[NT][BK]) {
+#pragma unroll
+        for (int u = 0; u < BK; ++u)
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                acc[nt] = mfma32(xv[u], gv[nt][u], acc[nt]);
+                colsum[nt] += gv[nt][u];
+            }
+    };
+    const int nbatch = (steps + BK - 1) / BK;  // steps past the chunk's end contribute zeros
+    if (nbatch > 0) fetch(xa, ga, 0);
+    for (int bt = 0; bt < nbatch; bt += 2) {
+        if (bt + 1 < nbatch) fetch(xb, gb, bt + 1);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(xa, ga);
+        __builtin_amdgcn_sched_barrier(0);
+        if (bt + 2 < nbatch) fetch(xa, ga, bt + 2);
+        __builtin_amdgcn_sched_barrier(0);
+        if (bt + 1 < nbatch) multiply(xb, gb);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    float* out = partial + ((int64_t)b * nchunk + chunk) * E;
+    // acc[nt][r] = dW[k0 + 8 (r / 4) + 4 kh + r % 4][n0 + 32 nt + tk]
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        if (nok[nt]) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int k = k0 + 8 * (r >> 2) + 4 * kh + (r & 3);
+                if (k < K) out[(int64_t)k * N + n0 + 32 * nt + tk] = acc[nt][r];
+            }
+        }
+        // bias gradient: the two token halves of a column meet; written once per strip, by the wave of rows 0..31
+        const float cs = colsum[nt] + __shfl_xor(colsum[nt], 32, 64);
+        if (k0 == 0 && kh == 0 && nok[nt]) out[(int64_t)K * N + n0 + 32 * nt + tk] = cs;
+    }
+}
+
+}  // namespace spgt
+
+using namespace spgt;
+
+namespace {
+
+struct WgradPlan {
+    int nt, nstrip, kz, tpc, nchunk;
+};
+
+WgradPlan wgrad_plan(int64_t T, int K, int N, int batch) {
+    WgradPlan p;
+    p.nt = N >= 128 ? 4 : (N > 32 ? 2 : 1);
+    p.nstrip = ceil_div(N, p.nt * 32);
+    p.kz = ceil_div(K, 128);
+    // about two workgroups per compute unit, at most as many chunks as tile_reduce sums, at least 64 tokens each
+    const int per = std::max(1, 2 * device_cu_count() / std::max(1, batch * p.nstrip * p.kz));
+    int64_t nchunk = std::min<int64_t>(std::min(per, kReduceChains * kReduceMaxPerChain), std::max<int64_t>(1, T / 64));
+    int64_t tpc = ceil_div(ceil_div(T, nchunk), (int64_t)16) * 16;
+    p.tpc = (int)tpc;
+    p.nchunk = (int)ceil_div(T, tpc);
+    return p;
+}
+
+}  // namespace
+
+extern "C" size_t spgt_linear_weight_grad_workspace_bytes(int64_t tokens, int in_features, int out_features,
+                                                          int batch) {
+    if (tokens <= 0 || in_features <= 0 || out_features <= 0 || batch <= 0 || out_features % 4 != 0) return 0;
+    if (tokens > ((int64_t)1 << 31) - 1024 || (int64_t)in_features * out_features + out_features > INT32_MAX) return 0;
+    const WgradPlan p = wgrad_plan(tokens, in_features, out_features, batch);
+    return (size_t)batch * p.nchunk * ((size_t)in_features * out_features + out_features) * sizeof(float);
+}
+
+extern "C" int spgt_linear_weight_grad(const float* x, int64_t ldx, int64_t x_batch_stride, const float* grad,
+                                       int64_t ldg, int64_t grad_batch_stride, float* out, void* workspace,
+                                       size_t workspace_bytes, int64_t tokens, int in_features, int out_features,
+                                       int batch, hipStream_t stream) {
+    if (!x || !grad || !out || !workspace)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "linear_weight_grad: null pointer argument");
+    const size_t need = spgt_linear_weight_grad_workspace_bytes(tokens, in_features, out_features, batch);
+    if (need == 0)
+        return fail(SPGT_ERR_INVALID_ARGUMENT,
+                    "linear_weight_grad: sizes must be positive, out_features a multiple of 4, tokens below 2^31");
+    if (ldx < in_features || ldg < out_features)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "linear_weight_grad: row strides shorter than the rows");
+    const int64_t E = (int64_t)in_features * out_features + out_features;
+    if (workspace_bytes < need || !aligned16(workspace))
+        return fail(SPGT_ERR_WORKSPACE, "linear_weight_grad: workspace missing, misaligned or too small");
+    if (!aligned4(x) || !aligned4(grad) || !aligned16(out))
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "linear_weight_grad: out must be 16-byte aligned");
+    const WgradPlan p = wgrad_plan(tokens, in_features, out_features, batch);
+    if ((int64_t)batch * p.nstrip > 65535 || p.kz > 65535)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "linear_weight_grad: too many column strips or row blocks");
+    float* partial = static_cast<float*>(workspace);
+    const dim3 grid(p.nchunk, batch * p.nstrip, p.kz);
+#define SPGT_XTG(NT)                                                                                               \
+    hipLaunchKernelGGL((xtg_partial_k<NT>), grid, dim3(256), 0, stream, x, ldx, x_batch_stride, grad, ldg,         \
+                       grad_batch_stride, partial, tokens, in_features, out_features, p.tpc, p.nstrip)
+    if (p.nt == 4) SPGT_XTG(4);
+    else if (p.nt == 2) SPGT_XTG(2);
+    else SPGT_XTG(1);
+#undef SPGT_XTG
+    hipLaunchKernelGGL(tile_reduce, dim3(ceil_div((int)E, 256), batch), dim3(1024), 0, stream, partial, out, (int)E,
+                       p.nchunk, 1.0f);
+    return check_launch("linear_weight_grad");
+}

@@ -13,6 +13,7 @@ from torch import Tensor
 
 from ... import _lib
 from ..._lib import check, ptr, require_gpu_f32, stream_of, workspace
+from .linear import linear_weight_grad
 
 GEMM_ORDER = {"RRR": 0, "RRC": 1, "RCR": 2, "RCC": 3, "CRR": 4, "CRC": 5, "CCR": 6, "CCC": 7}
 
@@ -132,12 +133,11 @@ def _heads_feature_to_token_major(src: Tensor, batch: int, num_head: int, dim_po
 
 
 def _linear_backward(grad_tm: Tensor, input: Tensor, weight: Tensor):
-    """Gradients of y = x @ W + b given dL/dy token-major: library GEMMs, as in the reference's
-    extension/bind/galerkin_attention.cu:41-46."""
-    dm = weight.shape[0]
+    """Gradients of y = x @ W + b given dL/dy token-major (reference: extension/bind/galerkin_attention.cu:41-46):
+    dX by a library GEMM, dW and db by this package's split-over-tokens kernel."""
     grad_input = torch.matmul(grad_tm, weight.t())
-    grad_bias = grad_tm.sum(dim=(0, 1))
-    grad_weight = torch.matmul(input.reshape(-1, dm).t(), grad_tm.reshape(-1, dm))
+    # x^T g over hundreds of thousands of tokens and the column sums of g: one pass, fixed summation order
+    grad_weight, grad_bias = linear_weight_grad(input, grad_tm)
     return grad_input, grad_weight, grad_bias
 
 

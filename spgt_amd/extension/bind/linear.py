@@ -198,3 +198,24 @@ def fused_encoder_tail_folded(q: Tensor, position, x: Tensor, folded_fc: Tensor,
             ptr(fc_bias), ptr(ffn1_weight_kn), ptr(ffn1_bias), ptr(ffn2_weight_kn), ptr(ffn2_bias),
             ACTIVATIONS[activation], ptr(out), B, S, dp, D, F, stream_of(x)))
     return out
+
+
+def linear_weight_grad(x: Tensor, grad: Tensor):
+    """(dW [in, out], db [out]) of y = x @ W + b from dL/dy: dW = x^T grad and db = column sums of grad over all
+    leading dimensions, in one pass over x and grad with a fixed summation order (reference:
+    extension/bind/galerkin_attention.cu:41-46).  x [..., in], grad [..., out], out a multiple of 4."""
+    K, N = x.shape[-1], grad.shape[-1]
+    xr, T, ldx = _rows("x", x, K)
+    gr, Tg, ldg = _rows("grad", grad, N)
+    if T != Tg:
+        raise ValueError(f"x has {T} rows and grad {Tg}")
+    lib = _lib.load()
+    nbytes = lib.spgt_linear_weight_grad_workspace_bytes(T, K, N, 1)
+    if nbytes == 0:
+        raise ValueError(f"unsupported weight-gradient shape: tokens={T} in={K} out={N} (out must be a multiple of 4)")
+    ws = _lib.workspace(nbytes, xr)
+    out = torch.empty(K * N + N, dtype=torch.float32, device=xr.device)
+    with torch.cuda.device(xr.device):
+        check(lib.spgt_linear_weight_grad(ptr(xr), ldx, 0, ptr(gr), ldg, 0, ptr(out), ptr(ws), ws.numel(), T, K, N, 1,
+                                          stream_of(xr)))
+    return out[:K * N].view(K, N), out[K * N:]

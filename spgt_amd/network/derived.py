@@ -26,14 +26,24 @@ _tls = threading.local()
 _generation = [0]
 
 
-class _Entry:
-    __slots__ = ("dst", "srcs", "ptrs", "descs")
+def _signature(shape, copies: List[Copy]) -> tuple:
+    """What a derived tensor was built from: the storage address, dtype, device and strided view of every
+    source as the spec names them now.  A parameter object that was replaced (load_state_dict(assign=True),
+    `lin.weight = nn.Parameter(...)`, parametrizations) or whose strides changed gives another signature."""
+    return (tuple(shape),) + tuple(
+        (src.data_ptr(), src.dtype, src.device, soff, tuple(size), tuple(sstr), doff, tuple(dstr))
+        for src, soff, size, sstr, doff, dstr in copies)
 
-    def __init__(self, shape, copies: List[Copy]) -> None:
+
+class _Entry:
+    __slots__ = ("dst", "spec", "sig", "descs", "stamp")
+
+    def __init__(self, spec, shape, copies: List[Copy], sig) -> None:
         device = copies[0][0].device
         self.dst = torch.empty(shape, dtype=torch.float32, device=device)
-        self.srcs = [c[0] for c in copies]
-        self.ptrs = tuple(s.data_ptr() for s in self.srcs)
+        self.spec = spec
+        self.sig = sig
+        self.stamp = -1
         self.descs = []
         for src, soff, size, sstr, doff, dstr in copies:
             if src.dtype != torch.float32 or src.device != device:
@@ -47,10 +57,9 @@ class _Entry:
             self.descs.append(d)
 
     def valid(self) -> bool:
-        for s, p in zip(self.srcs, self.ptrs):
-            if s.data_ptr() != p:
-                return False
-        return True
+        """True when the spec, consulted now, still names the sources this entry copies from.  The spec
+        re-resolves the parameters through their modules, so a replaced parameter is seen."""
+        return _signature(*self.spec()) == self.sig
 
 
 def _launch(descs: Sequence, device) -> None:
@@ -64,22 +73,28 @@ def _launch(descs: Sequence, device) -> None:
 
 def derived(module: nn.Module, name: str, spec: Callable[[], Tuple[Sequence[int], List[Copy]]]) -> Tensor:
     """The derived tensor `name` of `module`, up to date with its sources.  `spec()` gives its shape and the
-    strided copies that fill it; it is consulted when the tensor does not exist yet or a source has moved."""
+    strided copies that fill it, and must look the parameters up through their modules every time it is called
+    (it is kept and consulted again by every later refresh, to see parameters that were replaced)."""
     table = module.__dict__.setdefault("_spgt_derived", {})
     ent = table.get(name)
-    if ent is None or not ent.valid():
-        shape, copies = spec()
-        ent = _Entry(shape, copies)
+    active = getattr(_tls, "active", False)
+    if ent is not None and active and ent.stamp == getattr(_tls, "forward_id", -2):
+        return ent.dst  # checked and rewritten by the refresh that opened this forward
+    shape, copies = spec()
+    sig = _signature(shape, copies)
+    if ent is None or ent.sig != sig:
+        ent = _Entry(spec, shape, copies, sig)
         table[name] = ent
         _generation[0] += 1
         _launch(ent.descs, ent.dst.device)
-    elif not getattr(_tls, "active", False):
+    elif not active:
         _launch(ent.descs, ent.dst.device)  # no forward-level refresh is covering this request
     return ent.dst
 
 
 def refresh(root: nn.Module) -> None:
-    """Rewrites every derived tensor under `root` from its sources, in one launch per 64 copies."""
+    """Rewrites every derived tensor under `root` from its sources, in one launch per 64 copies.  Entries
+    whose sources are no longer the ones they were built from are dropped; their next request rebuilds them."""
     cache = root.__dict__.get("_spgt_refresh")
     if cache is None or cache[0] != _generation[0]:
         entries = [e for m in root.modules() for e in m.__dict__.get("_spgt_derived", {}).values()]
@@ -89,7 +104,7 @@ def refresh(root: nn.Module) -> None:
     if not entries:
         return
     if not all(e.valid() for e in entries):
-        # a source moved (new storage, another device): drop those tensors, their next request rebuilds them
+        # a source moved (new parameter object, new storage, other strides, another device)
         for m in root.modules():
             table = m.__dict__.get("_spgt_derived")
             if table:
@@ -98,6 +113,12 @@ def refresh(root: nn.Module) -> None:
         _generation[0] += 1
         return refresh(root)
     _launch(descs, entries[0].dst.device)
+    stamp = getattr(_tls, "forward_id", -2)
+    for e in entries:
+        e.stamp = stamp
+
+
+_forward_counter = [0]
 
 
 def refreshes_derived(forward):
@@ -109,11 +130,14 @@ def refreshes_derived(forward):
         if getattr(_tls, "active", False):
             return forward(self, *args, **kwargs)
         _tls.active = True
+        _forward_counter[0] += 1
+        _tls.forward_id = _forward_counter[0]
         try:
             refresh(self)
             return forward(self, *args, **kwargs)
         finally:
             _tls.active = False
+            _tls.forward_id = -2
 
     return wrapper
 

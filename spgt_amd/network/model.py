@@ -15,6 +15,26 @@ from .derived import derived, refreshes_derived
 from .layer import ConvResBlock2D, activation_name, always_dropout, gpu_inference, make_activation
 
 
+def get_resolution_size(r_large: int, r_small: int):
+    """The five grid sizes (fine, mid, attention, mid, fine) of the two down- and two up-sampling steps
+    around the encoder, as the reference derives them (common/trivial.py:78-96): the side ratio of one step,
+    sqrt(r_small / r_large), is rounded to four decimals and then to a multiple of 0.005, upwards when the last
+    digit the rounded number prints with is below 5 (whatever decimal place that digit stands in: the reference
+    reads it off the printed number, and configurations depend on that), and r_mid = round(r_large * ratio) - 1.
+    (211, 71) -> 122, (141, 71) -> 99, (421, 71) -> 172, (512, 256) -> 363."""
+    import numpy as np
+    # The reference rounds numpy scalars (np.sqrt's result), and round() of a numpy scalar scales, rounds half to
+    # even and unscales, which differs from Python's exactly-rounded round() on ties such as 0.5825 and 0.4975
+    # ((56, 19) -> 31, (198, 49) -> 98): numpy's rounding is used here for that reason.
+    step = 5.0e-3
+    ratio = np.round(np.sqrt(r_small / r_large), 4)
+    last_printed_digit = int(repr(float(ratio))[-1])
+    coarse = float(np.round(ratio, 3)) + (step if last_printed_digit < 5 else 0.0)
+    r_mid = round(r_large * (int(coarse / step + 0.5) * step)) - 1
+    fine, mid, small = (r_large, r_large), (r_mid, r_mid), (r_small, r_small)
+    return (fine, mid, small, mid, fine)
+
+
 def resample(X: Tensor, size) -> Tensor:
     """Bilinear, align_corners=True, on [N, C, H, W]."""
     if torch.is_grad_enabled() and X.requires_grad:
@@ -109,9 +129,15 @@ class UpScaler2D(nn.Module):
         w = self.conv.conv_layer.weight
         if w.stride(2) != 3 * w.stride(3):  # the nine taps are walked as one axis
             return w.detach().permute(1, 2, 3, 0).reshape(w.size(1), 9 * w.size(0)).contiguous()
-        cout, cin = w.size(0), w.size(1)
-        return derived(self, "tap_weight_kn", lambda: (
-            (cin, 9 * cout), [(w, 0, (cin, 9, cout), (w.stride(1), w.stride(3), w.stride(0)), 0, (9 * cout, cout, 1))]))
+        conv = self.conv.conv_layer
+
+        def spec():  # looks the weight up on every call: the parameter may be replaced
+            w = conv.weight
+            cout, cin = w.size(0), w.size(1)
+            return (cin, 9 * cout), [(w, 0, (cin, 9, cout), (w.stride(1), w.stride(3), w.stride(0)), 0,
+                                      (9 * cout, cout, 1))]
+
+        return derived(self, "tap_weight_kn", spec)
 
     def _mixes_before_resampling(self, X: Tensor) -> bool:
         """True when interpolate -> conv3x3 -> activations is computed as GEMM at the low resolution + gather:

@@ -47,9 +47,6 @@ class Sp_GalerkinAttention(nn.Module):
             # the reference's position kernel is written for two coordinates and skips the case of none
             # (extension/native/multihead_dim32.cu:6-22, 593-598); any other value corrupts memory there
             raise ValueError(f"dim_position must be 0 or 2 (got {dim_position})")
-        if dim_hidden > 512:
-            raise ValueError(f"dim_hidden must be 128, 256, 384 or 512 (got {dim_hidden}): the projection operators "
-                             "keep a head's weight columns in registers")
         self.dim_hidden = dim_hidden
         self.num_head = num_head
         self.dim_head = dim_hidden // num_head
@@ -110,7 +107,22 @@ class Sp_GalerkinAttention(nn.Module):
         """The attention core before fc_layer: [N, seqlen, num_head * (dim_position + dim_head)]."""
         N, seqlen, C = Q.size()
         H, dp = self.num_head, self.dim_position
-        if self._needs_graph(Q, K, V):
+        if self._needs_graph(Q, K, V) and C > 512:
+            # wider than the projection operators serve (they keep a head's weight columns in registers, up to
+            # dim_hidden 512): library GEMM and LayerNorm under autograd, laid out as the attention operator reads
+            def wide(x, w, b, ln_w=None, ln_b=None):
+                y = torch.addmm(b, x.reshape(N * seqlen, C), w).view(N, seqlen, H, self.dim_head)
+                if ln_w is not None:
+                    y = F.layer_norm(y, [self.dim_head], None, None, self.norm_eps) * ln_w + ln_b
+                if dp:
+                    y = torch.cat([position.unsqueeze(2).expand(N, seqlen, H, dp), y], dim=-1)
+                return y.permute(0, 2, 3, 1).contiguous()  # [N, H, dp + dim_head, seqlen]
+
+            X = multihead_galerkin_attention_cccr_cuda(
+                wide(Q, self.weight_Q, self.bias_Q), wide(K, self.weight_K, self.bias_K, self.ln_weight_K, self.ln_bias_K),
+                wide(V, self.weight_V, self.bias_V, self.ln_weight_V, self.ln_bias_V))
+            X = X.transpose(1, 2).contiguous().view(N, seqlen, H * (dp + self.dim_head))
+        elif self._needs_graph(Q, K, V):
             q = multihead_projection_with_position_rrc_cuda(Q, self.weight_Q, self.bias_Q, position, H, self.dim_head, dp)
             k = multihead_projection_layernorm_with_position_rrc_cuda(
                 K, self.weight_K, self.bias_K, self.ln_weight_K, self.ln_bias_K, position, self.norm_eps, H,

@@ -62,9 +62,10 @@ class Sp_DecoderRegressor(nn.Module):
     def _split_weight_kn(self, dim_x: int):
         """spatial_fc_layer.weight as ([dim_x, C], [dim_position, C]): the hidden-feature and the grid columns,
         transposed; derived tensors, rewritten from the parameter at the start of every inference forward."""
-        w = self.spatial_fc_layer.weight
-        return (derived(self, f"fc_hidden_kn_{dim_x}", lambda: transposed_2d(w, slice(0, dim_x))),
-                derived(self, f"fc_grid_kn_{dim_x}", lambda: transposed_2d(w, slice(dim_x, w.size(1)))))
+        lin = self.spatial_fc_layer  # the specs look the weight up on every call: the parameter may be replaced
+        return (derived(self, f"fc_hidden_kn_{dim_x}", lambda: transposed_2d(lin.weight, slice(0, dim_x))),
+                derived(self, f"fc_grid_kn_{dim_x}",
+                        lambda: transposed_2d(lin.weight, slice(dim_x, lin.weight.size(1)))))
 
     def accepts_low_resolution(self, X: Tensor, grid: Tensor) -> bool:
         """True when forward(X, grid, resample_to=size) is available for a channels-last X."""

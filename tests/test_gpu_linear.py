@@ -287,3 +287,45 @@ def test_hand_written_mfma_statements_match_the_compilers_intrinsic(gpu):
     ffc, fpos = (torch.randn(B, 128, 128, generator=g) / 11.0).to(gpu), torch.randn(B, 2, 128, generator=g).to(gpu)
     call = lambda: fused_encoder_tail_folded(q, pos, xr, ffc, fpos, bfc, w1, b1, w2, b2, "relu")
     assert torch.equal(on(main, call), on(check, call))
+
+
+@pytest.mark.parametrize("K,N", [(128, 128), (136, 128), (128, 256), (256, 128), (70, 36), (32, 4), (128, 384)])
+@pytest.mark.parametrize("T", [1, 63, 1000, 65536 + 3])
+def test_linear_weight_grad(gpu, K, N, T):
+    """dW = x^T g and db = column sums of g (the reference's projection backward, galerkin_attention.cu:41-46)
+    against float64 products; ragged sizes, a strided x, and bit-identical reruns."""
+    from spgt_amd.extension.bind.linear import linear_weight_grad
+    gen = torch.Generator().manual_seed(K * 7 + N * 3 + T)
+    xfull = torch.randn(T, K + 8, generator=gen)
+    x, g = xfull[:, :K], torch.randn(T, N, generator=gen)
+    xg = xfull.to(gpu)[:, :K]  # row stride K + 8
+    dW, db = linear_weight_grad(xg, g.to(gpu))
+    want_w, want_b = x.double().t() @ g.double(), g.double().sum(0)
+    assert dW.shape == (K, N) and db.shape == (N,)
+    scale = max(1.0, T ** 0.5)
+    assert (dW.cpu().double() - want_w).abs().max() < 2e-5 * scale
+    assert (db.cpu().double() - want_b).abs().max() < 2e-5 * scale
+    dW2, db2 = linear_weight_grad(xg.contiguous(), g.to(gpu))
+    assert torch.equal(dW, dW2) and torch.equal(db, db2)
+
+
+def test_linear_weight_grad_batched_through_the_c_abi(gpu):
+    """Three gradient planes against one input in one call (the packed Q | K | V projection's backward)."""
+    import ctypes
+    from spgt_amd import _lib
+    lib = _lib.load()
+    T, K, N = 5000, 128, 128
+    gen = torch.Generator().manual_seed(5)
+    x, g = torch.randn(T, K, generator=gen), torch.randn(3, T, N, generator=gen)
+    xd, gd = x.to(gpu), g.to(gpu)
+    out = torch.empty(3, K * N + N, device=gpu)
+    nws = lib.spgt_linear_weight_grad_workspace_bytes(T, K, N, 3)
+    ws = torch.empty(nws, dtype=torch.uint8, device=gpu)
+    p = lambda t: ctypes.c_void_p(t.data_ptr())
+    _lib.check(lib.spgt_linear_weight_grad(p(xd), K, 0, p(gd), N, T * N, p(out), p(ws), nws, T, K, N, 3,
+                                           ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
+    torch.cuda.synchronize()
+    for j in range(3):
+        assert (out[j, :K * N].view(K, N).cpu().double() - x.double().t() @ g[j].double()).abs().max() < 2e-3
+        assert (out[j, K * N:].cpu().double() - g[j].double().sum(0)).abs().max() < 2e-3
+    assert lib.spgt_linear_weight_grad_workspace_bytes(T, K, 126, 1) == 0

@@ -164,6 +164,29 @@ def test_resolution_sizes_known_answers(r_large, r_small, r_mid):
     assert rs == ((r_large,) * 2, (r_mid,) * 2, (r_small,) * 2, (r_mid,) * 2, (r_large,) * 2)
 
 
+# Ties of the two roundings, where round() of the numpy scalar the reference holds (scale, round half to even,
+# unscale: sqrt(19/56) -> 0.5825 -> 0.582) and Python's exactly-rounded round() of a float (-> 0.583) part ways:
+# the expected values follow numpy's, i.e. what common/trivial.py:84-89 computes on np.sqrt's result.
+@pytest.mark.parametrize("r_large,r_small,r_mid", [
+    (56, 19, 31), (67, 66, 65), (112, 38, 64), (198, 49, 98), (202, 50, 100), (295, 73, 147), (299, 74, 149),
+    (303, 75, 151)])
+def test_resolution_sizes_follow_numpy_scalar_rounding(r_large, r_small, r_mid):
+    assert O.resolution_sizes(r_large, r_small)[1] == (r_mid, r_mid)
+
+
+def test_product_resolution_rule_matches_the_oracle():
+    """spgt_amd.network.model.get_resolution_size (what a user builds cfg['resolution_size'] with) against the
+    oracle over every fine size up to 1300 and a sweep of attention sizes, and on the known answers."""
+    from spgt_amd.network.model import get_resolution_size
+    for r_large, r_small, r_mid in ((211, 71, 122), (141, 71, 99), (421, 71, 172), (512, 256, 363), (56, 19, 31)):
+        assert get_resolution_size(r_large, r_small)[1] == (r_mid, r_mid)
+    for r_large in range(4, 1300):
+        for r_small in range(2, r_large + 1, max(1, r_large // 29)):
+            got = get_resolution_size(r_large, r_small)
+            assert tuple(map(tuple, got)) == tuple(map(tuple, O.resolution_sizes(r_large, r_small))), (r_large, r_small)
+            assert all(isinstance(v, int) for pair in got for v in pair)
+
+
 def test_datamove_ops():
     x = rnd(2, 3, 4, 5, seed=19)
     y = O.op_batched_transpose(x, [2], [3, 4], [5])

@@ -78,3 +78,27 @@ def test_static_scratch_entry_point_rejects_oversized_shapes(gpu):
     p = ctypes.c_void_p(t.data_ptr())
     rc = lib.spgt_galerkin_attention_fused_forward_static(p, p, p, 128, None, p, p, p, p, 1e-6, p, p, B, S, H, 0, None)
     assert rc == -2 and "static" in _lib.last_error()
+
+
+def test_static_scratch_entry_point_leaves_device_memory_alone(gpu):
+    """After a GPU's first call (one-time set-up: symbol lookup, kernel attribute) the entry point must neither
+    take nor give back device memory: free memory as the driver reports it, and torch's own allocator statistics,
+    are the same before and after calls on both plans of the K/V pass."""
+    lib = _lib.load()
+    H, eps = 4, 1e-6
+    p = lambda t: ctypes.c_void_p(t.data_ptr())
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    for dp, (B, S) in ((0, (2, 150001)), (2, (2, 150001)), (2, (3, 6007))):
+        D = dp + 32
+        (q, k, v, pos), aff = _inputs(B, S, H, 300, gpu)
+        out = torch.empty(B, S, H * D, device=gpu)
+        ktv = torch.empty(B, H, D, D, device=gpu)
+        args = (p(q), p(k), p(v), H * 32, p(pos) if dp else None, p(aff[0]), p(aff[1]), p(aff[2]), p(aff[3]), eps,
+                p(out), p(ktv), B, S, H, dp, stream)
+        _lib.check(lib.spgt_galerkin_attention_fused_forward_static(*args))  # first call of this kind
+        torch.cuda.synchronize()
+        free0, reserved0 = torch.cuda.mem_get_info()[0], torch.cuda.memory_reserved()
+        for _ in range(3):
+            _lib.check(lib.spgt_galerkin_attention_fused_forward_static(*args))
+        torch.cuda.synchronize()
+        assert torch.cuda.mem_get_info()[0] == free0 and torch.cuda.memory_reserved() == reserved0
