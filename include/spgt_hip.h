@@ -246,24 +246,25 @@ int spgt_truncated_dft_rows_forward(const float* x, const float* table, float* Y
 int spgt_truncated_dft_rows_inverse(const float* U, const float* table, float* y, int64_t rows, int r,
                                     int channels, int modes, int planar, spgt_stream_t stream);
 
-/* 1 when spgt_spectral_inverse_linear serves this shape (32 or 64 channels in and out,
- * 2*modes <= min(64, r), r <= 1024). */
+/* 1 when spgt_spectral_inverse_linear serves this shape ((in, out) features 32 -> 32, 64 -> 64, 64 -> 32,
+ * 128 -> 32 or 128 -> 64; 2*modes <= min(64, r), r <= 1024). */
 int spgt_spectral_inverse_linear_supported(int r, int in_features, int out_features, int modes);
 
 /* The end of Sp_SpectralConv2D.forward (network/sp_layer.py:132, 149-155) in one pass:
  *   out[row, w, o] = activation(sum_c x[row, w, c] * weight_kn[c, o] + bias[o] + sum_j table[w, j] * U[row, o, j])
  * = the residual Linear, the w-direction of irfft2 for the retained modes (spgt_truncated_dft_rows_inverse),
  * their sum and the activation, without the inverse transform's result going to memory.
- * U planar [N, 2*modes, r, channels] as spgt_spectral_modes_middle writes it; x, out [rows = N*r, r, channels];
- * weight_kn [channels, channels] (the transpose of nn.Linear.weight); bias [channels] or null;
+ * U planar [N, 2*modes, r, out_features] as spgt_spectral_modes_middle writes it; x [rows = N*r, r, in_features];
+ * out [rows, r, out_features]; weight_kn [in_features, out_features] (the transpose of nn.Linear.weight); bias
+ * [out_features] or null;
  * table_operand [ceil(r/32), steps, 64], steps = 16 for modes <= 16, else 32: entry (t, kk, l) =
  * table[32 t + l % 32, 2 kk + l / 32] of the inverse table above, zero where the row is >= r or the column
  * >= 2*modes. */
 int spgt_spectral_inverse_linear(const float* U, const float* table_operand, const float* x, const float* weight_kn,
-                                 const float* bias, int activation, float* out, int64_t rows, int r, int channels,
-                                 int modes, spgt_stream_t stream);
+                                 const float* bias, int activation, float* out, int64_t rows, int r,
+                                 int in_features, int out_features, int modes, spgt_stream_t stream);
 
-/* 1 when spgt_spectral_modes_middle serves this shape (Cin, Cout <= 64, 2*modes <= min(64, r),
+/* 1 when spgt_spectral_modes_middle serves this shape (Cin <= 128, Cout <= 64, 2*modes <= min(64, r),
  * r <= 4096). */
 int spgt_spectral_modes_middle_supported(int r, int Cin, int Cout, int modes);
 

@@ -56,7 +56,7 @@ SIGNATURES = {
     "spgt_bias_activation_nchw": (_i, [_p, _p, _i, _i, _i64, _i, _i, _p]),
     "spgt_denormalize_boundary": (_i, [_p, _p, _p, _i, _p, _i, _i, _i, _i, _i, _p]),
     "spgt_spectral_inverse_linear_supported": (_i, [_i, _i, _i, _i]),
-    "spgt_spectral_inverse_linear": (_i, [_p, _p, _p, _p, _p, _i, _p, _i64, _i, _i, _i, _p]),
+    "spgt_spectral_inverse_linear": (_i, [_p, _p, _p, _p, _p, _i, _p, _i64, _i, _i, _i, _i, _p]),
     "spgt_truncated_dft_rows_supported": (_i, [_i, _i, _i]),
     "spgt_truncated_dft_rows_forward": (_i, [_p, _p, _p, _i64, _i, _i, _i, _i, _p]),
     "spgt_truncated_dft_rows_inverse": (_i, [_p, _p, _p, _i64, _i, _i, _i, _i, _p]),

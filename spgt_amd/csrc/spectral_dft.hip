@@ -224,19 +224,23 @@ __global__ __launch_bounds__(256) void dft_rows_inverse_k(const float* __restric
 // Lanes run along channels, so every global access is a 256-byte run; twiddle factors sit in LDS and
 // are wave-uniform.  All loads of a phase are in flight together (the data is a few MB: the kernels
 // are bound by memory round trips, not bandwidth), and every sum runs in a fixed order.
-constexpr int kMidC = 64;     // channels per operand (lanes)
+constexpr int kMidC = 64;     // output channels (lanes of the contraction's result)
 constexpr int kMidRows = 3;   // kept rows kh per workgroup of the first kernel
-constexpr int kMidHB = 32;    // grid rows h fetched per batch
+constexpr int kMidHB = 32;    // grid rows h fetched per batch (per channel of a lane)
 
 // grid (m, N, ceil(2m / kMidRows)), block 256.  O [N][m][2m][Cout] complex.
+// CPL: input channels per lane (Cin <= 64 CPL): a lane forms Z for channels lane, lane + 64, ...
+template <int CPL>
 __global__ __launch_bounds__(256) void spectral_rows_contract_k(
     const float* __restrict__ Y, const float2* __restrict__ G, const float2* __restrict__ W1,
     const float2* __restrict__ W2, float2* __restrict__ O, int r, int Cin, int Cout, int m) {
+    constexpr int MC = 64 * CPL;
+    constexpr int HB = kMidHB / CPL;
     extern __shared__ float2 lds[];
-    // [tab: kMidRows x r][part: 4 x kMidRows x 64]; part doubles as the per-c-quarter partial O
+    // [tab: kMidRows x r][part: 4 x kMidRows x MC]; part doubles as the per-c-quarter partial O
     float2* tab = lds;
-    float2 (*part)[kMidRows][kMidC] = reinterpret_cast<float2 (*)[kMidRows][kMidC]>(lds + kMidRows * r);
-    __shared__ float2 Zs[kMidRows][kMidC];
+    float2 (*part)[kMidRows][MC] = reinterpret_cast<float2 (*)[kMidRows][MC]>(lds + kMidRows * r);
+    __shared__ float2 Zs[kMidRows][MC];
     const int m2 = 2 * m;
     const int kw = blockIdx.x;
     const int64_t n = blockIdx.y;
@@ -249,79 +253,104 @@ __global__ __launch_bounds__(256) void spectral_rows_contract_k(
     }
     __syncthreads();
 
-    // Z = G Y: wave hq sums its quarter of h for the workgroup's rows; lane = input channel
+    // Z = G Y: wave hq sums its quarter of h for the workgroup's rows; lane = input channel (+ 64 j)
     {
         const int hlen = (r + 3) / 4;
         const int h0 = wave * hlen;
         const int h1 = min(r, h0 + hlen);
-        const float* yre = Y + ((n * m2 + 2 * kw) * r) * (int64_t)Cin + lane;
+        const float* yre = Y + ((n * m2 + 2 * kw) * r) * (int64_t)Cin;
         const float* yim = yre + (int64_t)r * Cin;
-        const bool cok = lane < Cin;
-        float2 acc[kMidRows];
+        int cj[CPL];
+        bool cok[CPL];
 #pragma unroll
-        for (int q = 0; q < kMidRows; ++q) acc[q] = make_float2(0.f, 0.f);
-        for (int hb = h0; hb < h1; hb += kMidHB) {
-            float a[kMidHB], b[kMidHB];
+        for (int j = 0; j < CPL; ++j) {
+            cok[j] = lane + 64 * j < Cin;
+            cj[j] = min(lane + 64 * j, Cin - 1);
+        }
+        float2 acc[kMidRows][CPL];
 #pragma unroll
-            for (int u = 0; u < kMidHB; ++u) {
+        for (int q = 0; q < kMidRows; ++q)
+#pragma unroll
+            for (int j = 0; j < CPL; ++j) acc[q][j] = make_float2(0.f, 0.f);
+        for (int hb = h0; hb < h1; hb += HB) {
+            float a[CPL][HB], b[CPL][HB];
+#pragma unroll
+            for (int u = 0; u < HB; ++u) {
                 const int h = min(hb + u, h1 - 1);
-                a[u] = cok ? yre[(int64_t)h * Cin] : 0.f;
-                b[u] = cok ? yim[(int64_t)h * Cin] : 0.f;
+#pragma unroll
+                for (int j = 0; j < CPL; ++j) {
+                    const float av = yre[(int64_t)h * Cin + cj[j]], bv = yim[(int64_t)h * Cin + cj[j]];
+                    a[j][u] = cok[j] ? av : 0.f;
+                    b[j][u] = cok[j] ? bv : 0.f;
+                }
             }
 #pragma unroll
-            for (int u = 0; u < kMidHB; ++u) {
+            for (int u = 0; u < HB; ++u) {
                 if (hb + u < h1) {
 #pragma unroll
                     for (int q = 0; q < kMidRows; ++q) {
                         const float2 g = tab[q * r + hb + u];
-                        acc[q].x = fmaf(g.x, a[u], acc[q].x);
-                        acc[q].x = fmaf(-g.y, b[u], acc[q].x);
-                        acc[q].y = fmaf(g.x, b[u], acc[q].y);
-                        acc[q].y = fmaf(g.y, a[u], acc[q].y);
+#pragma unroll
+                        for (int j = 0; j < CPL; ++j) {
+                            acc[q][j].x = fmaf(g.x, a[j][u], acc[q][j].x);
+                            acc[q][j].x = fmaf(-g.y, b[j][u], acc[q][j].x);
+                            acc[q][j].y = fmaf(g.x, b[j][u], acc[q][j].y);
+                            acc[q][j].y = fmaf(g.y, a[j][u], acc[q][j].y);
+                        }
                     }
                 }
             }
         }
 #pragma unroll
-        for (int q = 0; q < kMidRows; ++q) part[wave][q][lane] = acc[q];
+        for (int q = 0; q < kMidRows; ++q)
+#pragma unroll
+            for (int j = 0; j < CPL; ++j) part[wave][q][lane + 64 * j] = acc[q][j];
     }
     __syncthreads();
-    for (int e = threadIdx.x; e < kMidRows * kMidC; e += 256) {
-        const int q = e / kMidC, c = e % kMidC;
+    for (int e = threadIdx.x; e < kMidRows * MC; e += 256) {
+        const int q = e / MC, c = e % MC;
         const float2 p0 = part[0][q][c], p1 = part[1][q][c], p2 = part[2][q][c], p3 = part[3][q][c];
         Zs[q][c] = make_float2((p0.x + p1.x) + (p2.x + p3.x), (p0.y + p1.y) + (p2.y + p3.y));
     }
     __syncthreads();
 
-    // O = Z . W: wave w takes input channels [16w, 16w+16) of every row; lane = output channel
+    // O = Z . W: wave w takes input channels [w MC/4, (w + 1) MC/4) of every row, sixteen at a time; lane = output
+    // channel
     {
-        constexpr int CQ = kMidC / 4;
+        constexpr int CQ = MC / 4;
         const bool ook = lane < Cout;
-        float2 wv[kMidRows][CQ];
+        float2 o[kMidRows];
 #pragma unroll
-        for (int q = 0; q < kMidRows; ++q) {
-            const int kh = min(kh0 + q, m2 - 1);
-            const float2* Wm = (kh < m ? W1 + ((int64_t)kh * m + kw) * Cin * Cout
-                                       : W2 + ((int64_t)(kh - m) * m + kw) * Cin * Cout) + lane;
+        for (int q = 0; q < kMidRows; ++q) o[q] = make_float2(0.f, 0.f);
 #pragma unroll
-            for (int u = 0; u < CQ; ++u) {
-                const int c = wave * CQ + u;
-                wv[q][u] = (ook && c < Cin) ? Wm[(int64_t)c * Cout] : make_float2(0.f, 0.f);
+        for (int c0 = 0; c0 < CQ; c0 += 16) {
+            float2 wv[kMidRows][16];
+#pragma unroll
+            for (int q = 0; q < kMidRows; ++q) {
+                const int kh = min(kh0 + q, m2 - 1);
+                const float2* Wm = (kh < m ? W1 + ((int64_t)kh * m + kw) * Cin * Cout
+                                           : W2 + ((int64_t)(kh - m) * m + kw) * Cin * Cout) + min(lane, Cout - 1);
+#pragma unroll
+                for (int u = 0; u < 16; ++u) {
+                    const int c = wave * CQ + c0 + u;
+                    const float2 wval = Wm[(int64_t)min(c, Cin - 1) * Cout];
+                    wv[q][u] = (ook && c < Cin) ? wval : make_float2(0.f, 0.f);
+                }
+            }
+#pragma unroll
+            for (int q = 0; q < kMidRows; ++q) {
+#pragma unroll
+                for (int u = 0; u < 16; ++u) {
+                    const float2 z = Zs[q][wave * CQ + c0 + u];
+                    o[q].x = fmaf(z.x, wv[q][u].x, o[q].x);
+                    o[q].x = fmaf(-z.y, wv[q][u].y, o[q].x);
+                    o[q].y = fmaf(z.y, wv[q][u].x, o[q].y);
+                    o[q].y = fmaf(z.x, wv[q][u].y, o[q].y);
+                }
             }
         }
 #pragma unroll
-        for (int q = 0; q < kMidRows; ++q) {
-            float2 o = make_float2(0.f, 0.f);
-#pragma unroll
-            for (int u = 0; u < CQ; ++u) {
-                const float2 z = Zs[q][wave * CQ + u];
-                o.x = fmaf(z.x, wv[q][u].x, o.x);
-                o.x = fmaf(-z.y, wv[q][u].y, o.x);
-                o.y = fmaf(z.y, wv[q][u].x, o.y);
-                o.y = fmaf(z.x, wv[q][u].y, o.y);
-            }
-            part[wave][q][lane] = o;
-        }
+        for (int q = 0; q < kMidRows; ++q) part[wave][q][lane] = o[q];
     }
     __syncthreads();
     for (int e = threadIdx.x; e < kMidRows * kMidC; e += 256) {
@@ -379,7 +408,8 @@ __global__ __launch_bounds__(256) void spectral_rows_expand_k(
 // The end of Sp_SpectralConv2D.forward (network/sp_layer.py:132, 149-155) in one pass over the grid:
 //   out[row, w, o] = act( sum_c x[row, w, c] W[c, o] + bias[o] + sum_j table[w, j] U[row, o, j] )
 // i.e. the residual Linear, the inverse DFT along w of the retained modes, their sum and the activation;
-// the inverse transform's result never goes to memory.  C = 32 or 64 channels in and out, planar U [N][2m][r][C].
+// the inverse transform's result never goes to memory.  CIN = 32, 64 or 128 channels in, COUT = 32 or 64 out,
+// planar U [N][2m][r][COUT].
 // Both terms are MFMA products with output channels along the accumulator's registers and grid points along
 // its lanes (so a lane stores 16-byte pieces of its grid point's row): A = W resp. U in registers,
 // B = x tile (from a wave-private LDS tile, 16-byte reads, lane (w, kh) takes channels kh*C/2 + kk) resp.
@@ -396,22 +426,24 @@ __global__ __launch_bounds__(256) void spectral_rows_expand_k(
 // its own values to its address.
 // KSU: MFMA steps of the inverse transform, modes rounded up (the table entries of the steps past the modes are
 // zero); a template parameter so that neither the loads nor the MFMAs sit behind branches.  TS: steps per tile in
-// the operand table.  C: channels in and out, 32 or 64; a lane's contraction channels are kh * C/2 + kk.
-// grid (min(ceil(pairs / 4), CUs)), block 256.
-template <int ACT, int KSU, int C>
+// the operand table.  CIN: input channels of the Linear (32, 64 or 128; a lane's contraction channels are
+// kh * CIN/2 + kk), COUT: channels of U and of the result (32 or 64).
+// grid (min(ceil(pairs / 4), CUs)), block 256, dynamic LDS 4 * 32 * (CIN + 4) floats.
+template <int ACT, int KSU, int CIN, int COUT>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void spectral_inverse_linear_k(
     const float* __restrict__ U, const float* __restrict__ tabA, const float* __restrict__ x,
     const float* __restrict__ Wkn, const float* __restrict__ bias, float* __restrict__ out, int r, int m2,
     unsigned pairs) {
-    constexpr int PX = C + 4;
-    constexpr int NCB = C / 32;    // blocks of 32 output channels, one accumulator chain each
-    constexpr int KL = C / 2;      // contraction channels of the Linear per lane (MFMA steps)
-    constexpr int LPR = C / 4;     // lanes per grid point when a tile is fetched in 16-byte pieces
-    constexpr int NP = C / 8;      // such pieces per lane and tile
+    constexpr int PX = CIN + 4;
+    constexpr int NCB = COUT / 32;   // blocks of 32 output channels, one accumulator chain each
+    constexpr int KL = CIN / 2;      // contraction channels of the Linear per lane (MFMA steps)
+    constexpr int LPR = CIN / 4;     // lanes per grid point when a tile is fetched in 16-byte pieces
+    constexpr int NP = CIN / 8;      // such pieces per lane and tile
     constexpr int TS = KSU <= 16 ? 16 : 32;
-    static_assert(C == 32 || C == 64, "32 or 64 channels");
+    static_assert(CIN == 32 || CIN == 64 || CIN == 128, "32, 64 or 128 input channels");
+    static_assert(COUT == 32 || COUT == 64, "32 or 64 output channels");
     static_assert(KSU % 4 == 0 && KSU >= 4 && KSU <= 32, "4 .. 32 steps in fours");
-    __shared__ __attribute__((aligned(16))) float xs[4][32 * PX];
+    extern __shared__ __attribute__((aligned(16))) float xs_all[];  // [4 waves][32 * PX]
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int tk = lane & 31;
@@ -422,8 +454,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     float wreg0[KL], wreg1[KL];  // W[c = kh*KL + kk][o = cb*32 + tk], cb = 0, 1
 #pragma unroll
     for (int kk = 0; kk < KL; ++kk) {
-        wreg0[kk] = Wkn[(kh * KL + kk) * C + tk];
-        wreg1[kk] = NCB == 2 ? Wkn[(kh * KL + kk) * C + (NCB - 1) * 32 + tk] : 0.f;
+        wreg0[kk] = Wkn[(kh * KL + kk) * COUT + tk];
+        wreg1[kk] = NCB == 2 ? Wkn[(kh * KL + kk) * COUT + (NCB - 1) * 32 + tk] : 0.f;
     }
     // bias in accumulator layout (element 4q + e of half cb belongs to channel cb*32 + 8q + 4kh + e): the C operand
     // of a pair's first MFMAs
@@ -440,30 +472,36 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     // (finite values that meet zero table entries)
     uint32_t uoff[KSU];
 #pragma unroll
-    for (int kk = 0; kk < KSU; ++kk) uoff[kk] = (uint32_t)min(2 * kk + kh, m2 - 1) * (uint32_t)(r * C) + (uint32_t)tk;
-    float* const xw = xs[wave];
+    for (int kk = 0; kk < KSU; ++kk) uoff[kk] = (uint32_t)min(2 * kk + kh, m2 - 1) * (uint32_t)(r * COUT) + (uint32_t)tk;
+    float* const xw = xs_all + wave * (32 * PX);
 
     // (named registers and macros: a register array that lives across the loop ends up in scratch memory)
     // piece I of a tile is grid point (lane + 64 I) / LPR, channels 4 (lane % LPR) ..; points past the end of the
     // grid row read its last point
-    float4 s0, s1, s2, s3, s4, s5, s6, s7;
+    float4 s0, s1, s2, s3, s4, s5, s6, s7, s8, s9, s10, s11, s12, s13, s14, s15;
 #define SPGT_X_PIECE(BASE_, W0_, I_) \
-    (*reinterpret_cast<const float4*>((BASE_) + (uint32_t)(min((W0_) + ((lane + 64 * (I_)) / LPR), r - 1) * C + 4 * (lane % LPR))))
+    (*reinterpret_cast<const float4*>((BASE_) + (uint32_t)(min((W0_) + ((lane + 64 * (I_)) / LPR), r - 1) * CIN + 4 * (lane % LPR))))
 #define SPGT_LOAD_X_TILE(T_)                                                                        \
     {                                                                                               \
         const unsigned row_ = (T_) / WT;                                                            \
         const int w0_ = (int)((T_) - row_ * WT) * 32;                                               \
-        const float* xb_ = x + (int64_t)row_ * r * C;                                               \
+        const float* xb_ = x + (int64_t)row_ * r * CIN;                                             \
         s0 = SPGT_X_PIECE(xb_, w0_, 0); s1 = SPGT_X_PIECE(xb_, w0_, 1); s2 = SPGT_X_PIECE(xb_, w0_, 2); \
         s3 = SPGT_X_PIECE(xb_, w0_, 3);                                                             \
-        if (NP == 8) {                                                                              \
+        if (NP >= 8) {                                                                              \
             s4 = SPGT_X_PIECE(xb_, w0_, 4); s5 = SPGT_X_PIECE(xb_, w0_, 5);                         \
             s6 = SPGT_X_PIECE(xb_, w0_, 6); s7 = SPGT_X_PIECE(xb_, w0_, 7);                         \
+        }                                                                                           \
+        if (NP >= 16) {                                                                             \
+            s8 = SPGT_X_PIECE(xb_, w0_, 8); s9 = SPGT_X_PIECE(xb_, w0_, 9);                         \
+            s10 = SPGT_X_PIECE(xb_, w0_, 10); s11 = SPGT_X_PIECE(xb_, w0_, 11);                     \
+            s12 = SPGT_X_PIECE(xb_, w0_, 12); s13 = SPGT_X_PIECE(xb_, w0_, 13);                     \
+            s14 = SPGT_X_PIECE(xb_, w0_, 14); s15 = SPGT_X_PIECE(xb_, w0_, 15);                     \
         }                                                                                           \
     }
 #define SPGT_STORE_X_PIECE(I_, V_) \
     *reinterpret_cast<float4*>(xw + ((lane + 64 * (I_)) / LPR) * PX + 4 * (lane % LPR)) = V_;
-    s4 = s5 = s6 = s7 = make_float4(0.f, 0.f, 0.f, 0.f);
+    s4 = s5 = s6 = s7 = s8 = s9 = s10 = s11 = s12 = s13 = s14 = s15 = make_float4(0.f, 0.f, 0.f, 0.f);
     unsigned t = blockIdx.x * 4 + wave;
     if (t < pairs) SPGT_LOAD_X_TILE(t)
     for (; t < pairs; t += stride) {
@@ -472,10 +510,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         const unsigned n = row / (unsigned)r;
         const unsigned h = row - n * (unsigned)r;
         SPGT_STORE_X_PIECE(0, s0) SPGT_STORE_X_PIECE(1, s1) SPGT_STORE_X_PIECE(2, s2) SPGT_STORE_X_PIECE(3, s3)
-        if (NP == 8) {
+        if (NP >= 8) {
             SPGT_STORE_X_PIECE(4, s4) SPGT_STORE_X_PIECE(5, s5) SPGT_STORE_X_PIECE(6, s6) SPGT_STORE_X_PIECE(7, s7)
         }
-        const float* ub = U + ((int64_t)n * m2 * r + h) * C;  // U[n][0][h][0]
+        if (NP >= 16) {
+            SPGT_STORE_X_PIECE(8, s8) SPGT_STORE_X_PIECE(9, s9) SPGT_STORE_X_PIECE(10, s10) SPGT_STORE_X_PIECE(11, s11)
+            SPGT_STORE_X_PIECE(12, s12) SPGT_STORE_X_PIECE(13, s13) SPGT_STORE_X_PIECE(14, s14) SPGT_STORE_X_PIECE(15, s15)
+        }
+        const float* ub = U + ((int64_t)n * m2 * r + h) * COUT;  // U[n][0][h][0]
         float ureg0[KSU], ureg1[KSU];
 #pragma unroll
         for (int kk = 0; kk < KSU; ++kk) {
@@ -520,7 +562,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
             if (ACT == SPGT_ACT_RELU) y[q] = fmaxf(y[q], 0.f);
             if (ACT == SPGT_ACT_SILU) y[q] = y[q] * __builtin_amdgcn_rcpf(1.f + __expf(-y[q]));
         }
-        float* const op = out + ((int64_t)row * r + min(wt * 32 + tk, r - 1)) * C + 4 * kh;
+        float* const op = out + ((int64_t)row * r + min(wt * 32 + tk, r - 1)) * COUT + 4 * kh;
 #pragma unroll
         for (int q = 0; q < 4 * NCB; ++q)
             *reinterpret_cast<float4*>(op + 8 * q) = make_float4(y[4 * q], y[4 * q + 1], y[4 * q + 2], y[4 * q + 3]);
@@ -585,9 +627,11 @@ extern "C" int spgt_truncated_dft_rows_forward(const float* x, const float* tabl
                            channels, m2, planar);                                                               \
     }
     if (mb == 1) {
-        if (channels == 64) SPGT_DFT_FWD(64, 1) else if (channels == 32) SPGT_DFT_FWD(32, 1) else SPGT_DFT_FWD(0, 1)
+        if (channels == 64) SPGT_DFT_FWD(64, 1) else if (channels == 32) SPGT_DFT_FWD(32, 1)
+        else if (channels == 128) SPGT_DFT_FWD(128, 1) else SPGT_DFT_FWD(0, 1)
     } else {
-        if (channels == 64) SPGT_DFT_FWD(64, 2) else if (channels == 32) SPGT_DFT_FWD(32, 2) else SPGT_DFT_FWD(0, 2)
+        if (channels == 64) SPGT_DFT_FWD(64, 2) else if (channels == 32) SPGT_DFT_FWD(32, 2)
+        else if (channels == 128) SPGT_DFT_FWD(128, 2) else SPGT_DFT_FWD(0, 2)
     }
 #undef SPGT_DFT_FWD
     return check_launch("truncated_dft_rows_forward");
@@ -614,7 +658,7 @@ extern "C" int spgt_truncated_dft_rows_inverse(const float* U, const float* tabl
 }
 
 extern "C" int spgt_spectral_modes_middle_supported(int r, int Cin, int Cout, int modes) {
-    return (r > 0 && r <= 4096 && Cin > 0 && Cin <= kMidC && Cout > 0 && Cout <= kMidC && modes > 0 &&
+    return (r > 0 && r <= 4096 && Cin > 0 && Cin <= 2 * kMidC && Cout > 0 && Cout <= kMidC && modes > 0 &&
             2 * modes <= 64 && 2 * modes <= r) ? 1 : 0;
 }
 
@@ -632,7 +676,7 @@ extern "C" int spgt_spectral_modes_middle(const float* Y, const float* table_h, 
     if (N <= 0 || N > 65535) return fail(SPGT_ERR_INVALID_ARGUMENT, "spectral_modes_middle: N must be 1..65535");
     if (!spgt_spectral_modes_middle_supported(r, Cin, Cout, modes))
         return fail(SPGT_ERR_INVALID_ARGUMENT,
-                    "spectral_modes_middle: needs Cin, Cout <= 64, 2*modes <= min(64, r), r <= 4096");
+                    "spectral_modes_middle: needs Cin <= 128, Cout <= 64, 2*modes <= min(64, r), r <= 4096");
     if (workspace_bytes < spgt_spectral_modes_middle_workspace_bytes(N, Cout, modes))
         return fail(SPGT_ERR_WORKSPACE, "spectral_modes_middle: workspace too small");
     if (!aligned4(Y) || !aligned4(U) || !aligned8(table_h) || !aligned8(table_h_inverse) || !aligned8(weight_1) ||
@@ -640,13 +684,18 @@ extern "C" int spgt_spectral_modes_middle(const float* Y, const float* table_h, 
         return fail(SPGT_ERR_INVALID_ARGUMENT, "spectral_modes_middle: complex operands must be 8-byte aligned");
     const int m2 = 2 * modes;
     float2* O = reinterpret_cast<float2*>(workspace);
-    const size_t lds1 = ((size_t)kMidRows * r + 4 * kMidRows * kMidC) * sizeof(float2);
-    static const hipError_t opt_in = hipFuncSetAttribute(reinterpret_cast<const void*>(spectral_rows_contract_k),
-                                                         hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
-    (void)opt_in;
-    hipLaunchKernelGGL(spectral_rows_contract_k, dim3(modes, N, ceil_div(m2, kMidRows)), dim3(256), lds1, stream, Y,
-                       reinterpret_cast<const float2*>(table_h), reinterpret_cast<const float2*>(weight_1),
-                       reinterpret_cast<const float2*>(weight_2), O, r, Cin, Cout, modes);
+    const int cpl = Cin > kMidC ? 2 : 1;
+    const size_t lds1 = ((size_t)kMidRows * r + 4 * kMidRows * kMidC * cpl) * sizeof(float2);
+    const dim3 grid1(modes, N, ceil_div(m2, kMidRows));
+#define SPGT_MID_CONTRACT(CPL)                                                                                       \
+    {                                                                                                                \
+        allow_lds(spectral_rows_contract_k<CPL>, lds1);                                                              \
+        hipLaunchKernelGGL(spectral_rows_contract_k<CPL>, grid1, dim3(256), lds1, stream, Y,                         \
+                           reinterpret_cast<const float2*>(table_h), reinterpret_cast<const float2*>(weight_1),      \
+                           reinterpret_cast<const float2*>(weight_2), O, r, Cin, Cout, modes);                       \
+    }
+    if (cpl == 1) SPGT_MID_CONTRACT(1) else SPGT_MID_CONTRACT(2)
+#undef SPGT_MID_CONTRACT
     // about three workgroups per CU for the expansion; a chunk's table rows must fit 64 KiB of LDS
     int chunks = std::max(1, std::min(ceil_div(r, 4), ceil_div(3 * device_cu_count(), modes * N)));
     chunks = std::max(chunks, ceil_div(r * m2 * (int)sizeof(float2), 64 * 1024));
@@ -663,18 +712,61 @@ extern "C" int spgt_spectral_modes_middle(const float* Y, const float* table_h, 
 }
 
 extern "C" int spgt_spectral_inverse_linear_supported(int r, int in_features, int out_features, int modes) {
-    return (r > 0 && r <= 1024 && in_features == out_features && (in_features == 32 || in_features == 64) &&
-            modes > 0 && 2 * modes <= 64 && 2 * modes <= r) ? 1 : 0;
+    const bool pair = (in_features == out_features && (in_features == 32 || in_features == 64)) ||
+                      (in_features == 64 && out_features == 32) ||
+                      (in_features == 128 && (out_features == 32 || out_features == 64));
+    return (r > 0 && r <= 1024 && pair && modes > 0 && 2 * modes <= 64 && 2 * modes <= r) ? 1 : 0;
 }
+
+namespace {
+
+template <int ACT, int CIN, int COUT>
+int launch_inverse_linear(const float* U, const float* table_operand, const float* x, const float* weight_kn,
+                          const float* bias, float* out, int r, int modes, int64_t pairs, hipStream_t stream) {
+    const dim3 grid((unsigned)std::min<int64_t>(ceil_div(pairs, (int64_t)4), (int64_t)device_cu_count()));
+    const size_t lds = (size_t)4 * 32 * (CIN + 4) * sizeof(float);
+#define SPGT_SIL_LAUNCH(KSU)                                                                                        \
+    {                                                                                                               \
+        if (lds > 64 * 1024 &&                                                                                      \
+            hipFuncSetAttribute(reinterpret_cast<const void*>(spectral_inverse_linear_k<ACT, KSU, CIN, COUT>),      \
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)               \
+            return fail(SPGT_ERR_LAUNCH, "spectral_inverse_linear: the kernel was refused its dynamic LDS size");    \
+        hipLaunchKernelGGL((spectral_inverse_linear_k<ACT, KSU, CIN, COUT>), grid, dim3(256), lds, stream, U,       \
+                           table_operand, x, weight_kn, bias, out, r, 2 * modes, (unsigned)pairs);                  \
+    }
+    if (modes <= 4) SPGT_SIL_LAUNCH(4)
+    else if (modes <= 8) SPGT_SIL_LAUNCH(8)
+    else if (modes <= 12) SPGT_SIL_LAUNCH(12)
+    else if (modes <= 16) SPGT_SIL_LAUNCH(16)
+    else if (modes <= 24) SPGT_SIL_LAUNCH(24)
+    else SPGT_SIL_LAUNCH(32)
+#undef SPGT_SIL_LAUNCH
+    return SPGT_OK;
+}
+
+template <int CIN, int COUT>
+int launch_inverse_linear_act(int activation, const float* U, const float* table_operand, const float* x,
+                              const float* weight_kn, const float* bias, float* out, int r, int modes, int64_t pairs,
+                              hipStream_t stream) {
+    if (activation == SPGT_ACT_RELU)
+        return launch_inverse_linear<SPGT_ACT_RELU, CIN, COUT>(U, table_operand, x, weight_kn, bias, out, r, modes, pairs, stream);
+    if (activation == SPGT_ACT_SILU)
+        return launch_inverse_linear<SPGT_ACT_SILU, CIN, COUT>(U, table_operand, x, weight_kn, bias, out, r, modes, pairs, stream);
+    return launch_inverse_linear<SPGT_ACT_NONE, CIN, COUT>(U, table_operand, x, weight_kn, bias, out, r, modes, pairs, stream);
+}
+
+}  // namespace
 
 extern "C" int spgt_spectral_inverse_linear(const float* U, const float* table_operand, const float* x,
                                             const float* weight_kn, const float* bias, int activation, float* out,
-                                            int64_t rows, int r, int channels, int modes, hipStream_t stream) {
+                                            int64_t rows, int r, int in_features, int out_features, int modes,
+                                            hipStream_t stream) {
     if (!U || !table_operand || !x || !weight_kn || !out)
         return fail(SPGT_ERR_INVALID_ARGUMENT, "spectral_inverse_linear: null pointer argument");
-    if (!spgt_spectral_inverse_linear_supported(r, channels, channels, modes))
+    if (!spgt_spectral_inverse_linear_supported(r, in_features, out_features, modes))
         return fail(SPGT_ERR_INVALID_ARGUMENT,
-                    "spectral_inverse_linear: needs 32 or 64 channels, 2*modes <= min(64, r), r <= 1024");
+                    "spectral_inverse_linear: needs (in, out) features in {32->32, 64->64, 64->32, 128->32, 128->64}, "
+                    "2*modes <= min(64, r), r <= 1024");
     if (rows <= 0 || rows % r != 0 || rows > INT32_MAX)
         return fail(SPGT_ERR_INVALID_ARGUMENT, "spectral_inverse_linear: rows must be a positive multiple of r");
     if (activation != SPGT_ACT_NONE && activation != SPGT_ACT_RELU && activation != SPGT_ACT_SILU)
@@ -687,24 +779,16 @@ extern "C" int spgt_spectral_inverse_linear(const float* U, const float* table_o
     const int64_t pairs = (int64_t)rows * ((r + 31) / 32);
     if (pairs > (int64_t)INT32_MAX - 4096)
         return fail(SPGT_ERR_INVALID_ARGUMENT, "spectral_inverse_linear: more than 2^31 tiles of 32 grid points");
-    const dim3 grid((unsigned)std::min<int64_t>(ceil_div(pairs, (int64_t)4), (int64_t)device_cu_count()));
-#define SPGT_SIL_LAUNCH(ACT, KSU, C)                                                                               \
-    hipLaunchKernelGGL((spectral_inverse_linear_k<ACT, KSU, C>), grid, dim3(256), 0, stream, U, table_operand, x, \
-                       weight_kn, bias, out, r, 2 * modes, (unsigned)pairs)
-#define SPGT_SIL_STEPS(ACT, C)                         \
-    if (modes <= 4) SPGT_SIL_LAUNCH(ACT, 4, C);        \
-    else if (modes <= 8) SPGT_SIL_LAUNCH(ACT, 8, C);   \
-    else if (modes <= 12) SPGT_SIL_LAUNCH(ACT, 12, C); \
-    else if (modes <= 16) SPGT_SIL_LAUNCH(ACT, 16, C); \
-    else if (modes <= 24) SPGT_SIL_LAUNCH(ACT, 24, C); \
-    else SPGT_SIL_LAUNCH(ACT, 32, C)
-#define SPGT_SIL_ACT(C)                                                        \
-    if (activation == SPGT_ACT_RELU) { SPGT_SIL_STEPS(SPGT_ACT_RELU, C); }     \
-    else if (activation == SPGT_ACT_SILU) { SPGT_SIL_STEPS(SPGT_ACT_SILU, C); } \
-    else { SPGT_SIL_STEPS(SPGT_ACT_NONE, C); }
-    if (channels == 64) { SPGT_SIL_ACT(64) } else { SPGT_SIL_ACT(32) }
-#undef SPGT_SIL_ACT
-#undef SPGT_SIL_STEPS
-#undef SPGT_SIL_LAUNCH
+    int rc;
+#define SPGT_SIL_SHAPE(CIN, COUT)                                                                                 \
+    rc = launch_inverse_linear_act<CIN, COUT>(activation, U, table_operand, x, weight_kn, bias, out, r, modes, pairs, \
+                                              stream)
+    if (in_features == 32) SPGT_SIL_SHAPE(32, 32);
+    else if (in_features == 64 && out_features == 64) SPGT_SIL_SHAPE(64, 64);
+    else if (in_features == 64) SPGT_SIL_SHAPE(64, 32);
+    else if (out_features == 32) SPGT_SIL_SHAPE(128, 32);
+    else SPGT_SIL_SHAPE(128, 64);
+#undef SPGT_SIL_SHAPE
+    if (rc != SPGT_OK) return rc;
     return check_launch("spectral_inverse_linear");
 }

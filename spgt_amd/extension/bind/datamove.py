@@ -443,35 +443,38 @@ def _spectral_inverse_linear_supported(r: int, cin: int, cout: int, modes: int) 
 
 
 def _spectral_inverse_linear(U: Tensor, table_operand: Tensor, X: Tensor, weight_kn: Tensor, bias, activation) -> Tensor:
-    """act(X @ weight_kn + bias + inverse row DFT of U): U planar [N, 2m, r, C], X [N, r, r, C] -> [N, r, r, C]."""
+    """act(X @ weight_kn + bias + inverse row DFT of U): U planar [N, 2m, r, Cout], X [N, r, r, Cin],
+    weight_kn [Cin, Cout] -> [N, r, r, Cout]."""
     for name, t in (("U", U), ("table_operand", table_operand), ("X", X), ("weight_kn", weight_kn)):
         require_gpu_f32(name, t)
     if activation not in _ACT:
         raise ValueError("activation must be None, 'none', 'relu' or 'silu'")
     if X.dim() != 4 or X.shape[1] != X.shape[2]:
-        raise ValueError("X must be [N, r, r, C]")
-    N, r, _, C = X.shape
-    if U.dim() != 4 or U.shape[0] != N or U.shape[2] != r or U.shape[3] != C or U.shape[1] % 2:
-        raise ValueError("U must be planar [N, 2*modes, r, C]")
+        raise ValueError("X must be [N, r, r, Cin]")
+    N, r, _, cin = X.shape
+    if weight_kn.dim() != 2 or weight_kn.shape[0] != cin:
+        raise ValueError("weight_kn must be [Cin, Cout]")
+    cout = weight_kn.shape[1]
+    if U.dim() != 4 or U.shape[0] != N or U.shape[2] != r or U.shape[3] != cout or U.shape[1] % 2:
+        raise ValueError("U must be planar [N, 2*modes, r, Cout]")
     modes = U.shape[1] // 2
-    if tuple(weight_kn.shape) != (C, C):
-        raise ValueError("weight_kn must be [C, C]")
     steps = 16 if modes <= 16 else 32
     if tuple(table_operand.shape) != ((r + 31) // 32, steps, 64):
         raise ValueError(f"table_operand must be [ceil(r/32), {steps}, 64]")
     if bias is not None:
         require_gpu_f32("bias", bias)
-        if bias.numel() != C:
-            raise ValueError(f"bias has {bias.numel()} elements, expected {C}")
-    if not _spectral_inverse_linear_supported(r, C, C, modes):
-        raise ValueError("spectral_inverse_linear: needs 32 or 64 channels, 2*modes <= min(64, r), r <= 1024")
-    out = torch.empty_like(X)
+        if bias.numel() != cout:
+            raise ValueError(f"bias has {bias.numel()} elements, expected {cout}")
+    if not _spectral_inverse_linear_supported(r, cin, cout, modes):
+        raise ValueError("spectral_inverse_linear: needs (Cin, Cout) in {32->32, 64->64, 64->32, 128->32, 128->64}, "
+                         "2*modes <= min(64, r), r <= 1024")
+    out = torch.empty((N, r, r, cout), dtype=X.dtype, device=X.device)
     if X.numel() == 0:
         return out
     with torch.cuda.device(X.device):
         check(_lib.load().spgt_spectral_inverse_linear(ptr(U), ptr(table_operand), ptr(X), ptr(weight_kn),
                                                        ptr(bias) if bias is not None else None, _ACT[activation],
-                                                       ptr(out), N * r, r, C, modes, stream_of(X)))
+                                                       ptr(out), N * r, r, cin, cout, modes, stream_of(X)))
     return out
 
 

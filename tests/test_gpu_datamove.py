@@ -450,7 +450,8 @@ def test_truncated_dft_rows_rejects(gpu):
 
 @pytest.mark.parametrize("N,r,cin,cout,m", [(2, 211, 64, 64, 12), (1, 21, 32, 32, 4), (3, 16, 64, 32, 8), (2, 33, 24, 40, 16),
                                             (1, 421, 32, 32, 21), (1, 512, 64, 64, 23), (2, 64, 17, 9, 32),
-                                            (1, 1500, 8, 8, 20)])
+                                            (1, 1500, 8, 8, 20), (2, 128, 128, 32, 12), (1, 256, 128, 32, 16),
+                                            (1, 512, 128, 64, 23), (2, 37, 100, 24, 9), (1, 45, 65, 64, 7)])
 def test_spectral_modes_middle_against_float64(gpu, N, r, cin, cout, m):
     """DFT along h onto the kept rows, complex contraction, inverse DFT along h (network/sp_layer.py:136-151
     restricted to the kept modes) against the same three products in float64."""
@@ -574,3 +575,27 @@ def test_spectral_inverse_linear_matches_separate_kernels(gpu, N, r, m, C, act):
     no_bias = dm.spectral_inverse_linear(U, dm.inverse_table_operand(fwi), x, w, None, act)
     want_nb = parts(None)
     assert (no_bias - want_nb).abs().max().item() <= tol * max(1.0, want_nb.abs().max().item())
+
+
+@pytest.mark.parametrize("N,r,m", [(1, 33, 4), (4, 128, 12), (2, 256, 16), (1, 512, 23), (2, 7, 3), (1, 100, 25), (1, 70, 32)])
+@pytest.mark.parametrize("cin,cout", [(128, 32), (128, 64), (64, 32)])
+@pytest.mark.parametrize("act", [None, "silu"])
+def test_spectral_inverse_linear_unequal_widths(gpu, N, r, m, cin, cout, act):
+    """The same kernel with more input than output channels (the reference's own spectral-layer benchmark is
+    128 -> 32, evaluate/sp_fno2d.py:12-14) against float64 arithmetic, with and without bias."""
+    from spgt_amd.network.truncated_dft import dft_tables
+    assert dm.spectral_inverse_linear_supported(r, cin, cout, m)
+    assert not dm.spectral_inverse_linear_supported(r, 32, 128, m)
+    g = torch.Generator().manual_seed(N * 977 + r + m + cin + cout)
+    x = torch.randn(N, r, r, cin, generator=g).to(gpu)
+    U = torch.randn(N, 2 * m, r, cout, generator=g).to(gpu)
+    w = (torch.randn(cin, cout, generator=g) / cin ** 0.5).to(gpu)
+    b = torch.randn(cout, generator=g).to(gpu)
+    _, _, _, fwi = dft_tables(r, m, gpu)
+    y64 = torch.einsum("wj,njho->nhwo", fwi.double(), U.double())
+    for bias in (b, None):
+        got = dm.spectral_inverse_linear(U, dm.inverse_table_operand(fwi), x, w, bias, act)
+        z = x.double() @ w.double() + (0 if bias is None else bias.double()) + y64
+        z = z * torch.sigmoid(z) if act == "silu" else z
+        assert got.shape == (N, r, r, cout)
+        assert (got.double() - z).abs().max().item() <= 1e-5 * max(1.0, z.abs().max().item())

@@ -184,6 +184,29 @@ def test_spectral_conv_reference_default_modes(gpu, N, r, width, modes, truncate
     assert max_rel(got.cpu().double(), want) < TOL
 
 
+@pytest.mark.parametrize("N,r,cin,cout,modes", [(4, 256, 128, 32, 16), (2, 128, 128, 32, 12), (1, 512, 128, 32, 23),
+                                                (2, 77, 128, 64, 9), (2, 50, 64, 32, 8)])
+def test_spectral_conv_unequal_widths_take_the_fused_route(gpu, N, r, cin, cout, modes):
+    """Sp_SpectralConv2D with in_dim != out_dim at the reference's own benchmark shape (evaluate/sp_fno2d.py:12-26:
+    B = 4, 128 -> 32, modes ceil(sqrt(r))): the three-launch truncated-DFT route must serve it (no library GEMM or
+    FFT behind it), and agree with the oracle's rfft2 / irfft2 in fp64."""
+    from spgt_amd.network import truncated_dft
+    torch.manual_seed(17)
+    layer = L.Sp_SpectralConv2D(cin, cout, modes, 0.0, "silu")
+    with torch.no_grad():
+        for w in layer.fourier_weight:
+            w.copy_(torch.randn(w.shape) / cin)
+    sd = {k: v.clone().double() for k, v in layer.state_dict().items()}
+    x = torch.randn(N, r, r, cin, generator=torch.Generator().manual_seed(18))
+    want = O.spectral_conv2d(sd, x.double(), modes, "silu", weight_layout="sp")
+    assert truncated_dft.fused_tail_supported(r, cin, cout, modes)
+    layer = layer.to(gpu).eval()
+    with torch.no_grad():
+        got = layer(x.to(gpu))
+    assert got.shape == (N, r, r, cout)
+    assert max_rel(got.cpu().double(), want) < TOL
+
+
 def test_deferred_upsampling_matches_module_order(gpu):
     """The decoder's input layer in front of the up-scaler's last interpolation (a Linear over the channels commutes
     with it) against the reference's order of the same modules (network/model.py:59-64, network/sp_model.py:60):
