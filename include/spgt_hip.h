@@ -125,6 +125,26 @@ int spgt_galerkin_attention_fused_forward(const float* Q, const float* K, const 
                                           size_t workspace_bytes, int B, int S, int H, int dp,
                                           spgt_stream_t stream);
 
+/* Backward of spgt_galerkin_attention_fused_forward on the same token-major operands: the reference's
+ * multihead_galerkin_attention_cccr_backward (extension/bind/galerkin_attention.cu:126-173) together with the
+ * LayerNorm backward of its two projection+LayerNorm operators (extension/native/multihead_dim32.cu:148-271),
+ * from the plain projections x@W+b as the forward takes them.
+ *   grad_out : [B, S, H*(dp+32)] gradient of the forward's `out`
+ *   Q, K, V, position, ln_*, norm_eps : the forward's inputs; ktv : the forward's K'^T V' / S
+ *   grad_Q, grad_K, grad_V : [B, S, H*32] with row stride ld_out floats: gradients of the plain projections
+ *                            (the LayerNorm backward of K and V is applied; position gets no gradient)
+ *   grad_ln  : [4, H*32]: gradients of ln_weight_K, ln_bias_K, ln_weight_V, ln_bias_V
+ * Two passes over the sequence (Q~^T G / S as partial tiles summed in a fixed order; then one stream over
+ * K, V and grad_out that writes the three gradients), LayerNorm statistics recomputed in registers. */
+size_t spgt_galerkin_attention_fused_backward_workspace_bytes(int B, int S, int H, int dp);
+int spgt_galerkin_attention_fused_backward(const float* grad_out, const float* Q, const float* K, const float* V,
+                                           int64_t ld_in, const float* position, const float* ln_weight_K,
+                                           const float* ln_bias_K, const float* ln_weight_V,
+                                           const float* ln_bias_V, float norm_eps, const float* ktv,
+                                           float* grad_Q, float* grad_K, float* grad_V, int64_t ld_out,
+                                           float* grad_ln, void* workspace, size_t workspace_bytes, int B, int S,
+                                           int H, int dp, spgt_stream_t stream);
+
 /* spgt_galerkin_attention_fused_forward for callers that cannot allocate device memory or hand in
  * a workspace (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).
  * It has no counterpart in the reference.  The partial tiles of the K/V pass go to a device array

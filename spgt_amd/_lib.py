@@ -34,6 +34,9 @@ SIGNATURES = {
     "spgt_galerkin_attention_fused_workspace_bytes": (_sz, [_i, _i, _i, _i]),
     "spgt_galerkin_attention_fused_forward": (
         _i, [_p, _p, _p, _i64, _p, _p, _p, _p, _p, _f, _p, _p, _p, _sz, _i, _i, _i, _i, _p]),
+    "spgt_galerkin_attention_fused_backward_workspace_bytes": (_sz, [_i, _i, _i, _i]),
+    "spgt_galerkin_attention_fused_backward": (
+        _i, [_p, _p, _p, _p, _i64, _p, _p, _p, _p, _p, _f, _p, _p, _p, _p, _i64, _p, _p, _sz, _i, _i, _i, _i, _p]),
     "spgt_galerkin_attention_fused_static_max_bytes": (_sz, []),
     "spgt_galerkin_attention_fused_forward_static": (
         _i, [_p, _p, _p, _i64, _p, _p, _p, _p, _p, _f, _p, _p, _i, _i, _i, _i, _p]),

@@ -19,6 +19,7 @@ CHECK_SOURCE, CHECK_DEFINE = "linear.hip", "-DSPGT_MFMA_BUILTIN=1"
 SOURCES = [
     "spgt_host.cpp",
     "attn_fused.hip",
+    "attn_fused_backward.hip",
     "attn_fm.hip",
     "attn_backward.hip",
     "splitk_gemm.hip",

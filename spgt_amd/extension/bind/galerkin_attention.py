@@ -279,6 +279,51 @@ def _attention_fused_forward(QKV_or_Q, K, V, position, ln_weight_K, ln_bias_K, l
     return (out, ktv) if return_ktv else out
 
 
+def _attention_fused_backward(grad_out, Q, K, V, position, ln_weight_K, ln_bias_K, ln_weight_V, ln_bias_V,
+                              norm_eps: float, ktv, num_head: int, dim_position: int):
+    """Backward of _attention_fused_forward on the same operands: grad_out [B, S, H*(dp+32)] ->
+    (dQ, dK, dV [B, S, H*32] w.r.t. the plain projections, d ln_weight_K, d ln_bias_K, d ln_weight_V, d ln_bias_V
+    [H, 32]) (reference: extension/bind/galerkin_attention.cu:126-173, extension/native/multihead_dim32.cu:148-271)."""
+    H = num_head
+    D = dim_position + 32
+    B, S, _ = Q.shape
+    ld = Q.stride(1)
+    for name, t in (("Q", Q), ("K", K), ("V", V)):
+        require_gpu_f32(name, t, contiguous=False)
+        if tuple(t.shape) != (B, S, H * 32) or t.stride(2) != 1 or t.stride(1) != ld or (B > 1 and t.stride(0) != S * ld):
+            raise ValueError(f"{name}: Q, K, V must share shape [B, S, {H * 32}] and strides [S*ld, ld, 1]")
+    grad_out = grad_out.contiguous()
+    require_gpu_f32("grad_out", grad_out)
+    if tuple(grad_out.shape) != (B, S, H * D):
+        raise ValueError(f"grad_out has shape {tuple(grad_out.shape)}, expected {(B, S, H * D)}")
+    require_gpu_f32("ktv", ktv)
+    if tuple(ktv.shape) != (B, H, D, D):
+        raise ValueError(f"ktv has shape {tuple(ktv.shape)}, expected {(B, H, D, D)}")
+    for name, t in (("ln_weight_K", ln_weight_K), ("ln_bias_K", ln_bias_K), ("ln_weight_V", ln_weight_V),
+                    ("ln_bias_V", ln_bias_V)):
+        require_gpu_f32(name, t)
+        if t.numel() != H * 32:
+            raise ValueError(f"{name} must have {H * 32} elements")
+    if dim_position == 2:
+        require_gpu_f32("position", position)
+        if tuple(position.shape) != (B, S, 2):
+            raise ValueError(f"position must be [{B}, {S}, 2]")
+    lib = _lib.load()
+    nbytes = lib.spgt_galerkin_attention_fused_backward_workspace_bytes(B, S, H, dim_position)
+    if nbytes == 0:
+        raise ValueError("unsupported shape: num_head must be a multiple of 4, dim_position 0 or 2")
+    ws = workspace(nbytes, Q)
+    grads = torch.empty((3, B, S, H * 32), dtype=torch.float32, device=Q.device)
+    grad_ln = torch.empty((4, H, 32), dtype=torch.float32, device=Q.device)
+    with torch.cuda.device(Q.device):
+        check(lib.spgt_galerkin_attention_fused_backward(
+            ptr(grad_out), ptr(Q), ptr(K), ptr(V), ld, ptr(position) if dim_position == 2 else None,
+            ptr(ln_weight_K), ptr(ln_bias_K), ptr(ln_weight_V), ptr(ln_bias_V), float(norm_eps), ptr(ktv),
+            ptr(grads[0]), ptr(grads[1]), ptr(grads[2]), H * 32, ptr(grad_ln), ptr(ws), ws.numel(), B, S, H,
+            dim_position, stream_of(Q)))
+    return grads[0], grads[1], grads[2], grad_ln[0], grad_ln[1], grad_ln[2], grad_ln[3]
+
+
 def _attention_ktv_forward(K, V, position, ln_weight_K, ln_bias_K, ln_weight_V, ln_bias_V, norm_eps: float,
                            num_head: int, dim_position: int):
     """K'^T V' / S [B, H, d, d] of the fused attention core (K/V pass and tile reduction, no pass over Q):
@@ -384,6 +429,7 @@ gexts = SimpleNamespace(
     multihead_galerkin_attention_cccr_forward=_attention_cccr_forward,
     batched_skinny_gemm=_batched_skinny_gemm,
     galerkin_attention_fused_forward=_attention_fused_forward,
+    galerkin_attention_fused_backward=_attention_fused_backward,
 )
 
 
@@ -488,11 +534,41 @@ def fold_ktv_into_fc(ktv: Tensor, fc_weight_kn: Tensor, dim_position: int):
     return gexts.fold_ktv_into_fc(ktv, fc_weight_kn, dim_position)
 
 
+class Galerkin_Attention_Fused_Function(torch.autograd.Function):
+    """The fused token-major attention core with its backward (no counterpart as one operator in the reference,
+    whose autograd functions are the three above; this one computes what their composition computes, starting
+    from the plain projections)."""
+
+    @staticmethod
+    def forward(ctx: Any, Q: Tensor, K: Tensor, V: Tensor, position, lnwK: Tensor, lnbK: Tensor, lnwV: Tensor,
+                lnbV: Tensor, norm_eps: float, num_head: int, dim_position: int):
+        out, ktv = gexts.galerkin_attention_fused_forward(Q, K, V, position, lnwK, lnbK, lnwV, lnbV, norm_eps,
+                                                          num_head, dim_position, True)
+        ctx.save_for_backward(Q, K, V, position if dim_position == 2 else None, lnwK, lnbK, lnwV, lnbV, ktv)
+        ctx.args = (float(norm_eps), int(num_head), int(dim_position))
+        return out
+
+    @staticmethod
+    def backward(ctx: Any, grad_out: Tensor):
+        Q, K, V, position, lnwK, lnbK, lnwV, lnbV, ktv = ctx.saved_tensors
+        norm_eps, num_head, dim_position = ctx.args
+        dQ, dK, dV, dgK, dbK, dgV, dbV = gexts.galerkin_attention_fused_backward(
+            grad_out, Q, K, V, position, lnwK, lnbK, lnwV, lnbV, norm_eps, ktv, num_head, dim_position)
+        shape = lnwK.shape
+        return (dQ, dK, dV, None, dgK.view(shape), dbK.view(shape), dgV.view(shape), dbV.view(shape), None, None, None)
+
+
 def galerkin_attention_fused(Q: Tensor, K: Tensor, V: Tensor, position, ln_weight_K: Tensor, ln_bias_K: Tensor,
                              ln_weight_V: Tensor, ln_bias_V: Tensor, norm_eps: float, num_head: int,
                              dim_position: int, return_ktv: bool = False):
-    """LayerNorm(K), LayerNorm(V), K'^T V'/S and Q' (K'^T V'/S) in one call on
-    token-major projections (inference only: no autograd graph is recorded)."""
+    """LayerNorm(K), LayerNorm(V), K'^T V'/S and Q' (K'^T V'/S) in one call on token-major projections.
+    Differentiable w.r.t. Q, K, V and the four LayerNorm parameters (not w.r.t. position); with return_ktv the
+    call is inference-only and also returns K'^T V'/S."""
+    needs_graph = torch.is_grad_enabled() and any(
+        t.requires_grad for t in (Q, K, V, ln_weight_K, ln_bias_K, ln_weight_V, ln_bias_V))
+    if needs_graph and not return_ktv:
+        return Galerkin_Attention_Fused_Function.apply(Q, K, V, position, ln_weight_K, ln_bias_K, ln_weight_V,
+                                                       ln_bias_V, norm_eps, num_head, dim_position)
     return gexts.galerkin_attention_fused_forward(
         Q, K, V, position, ln_weight_K, ln_bias_K, ln_weight_V, ln_bias_V, norm_eps, num_head, dim_position,
         return_ktv)

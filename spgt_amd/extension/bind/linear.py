@@ -219,3 +219,24 @@ def linear_weight_grad(x: Tensor, grad: Tensor):
         check(lib.spgt_linear_weight_grad(ptr(xr), ldx, 0, ptr(gr), ldg, 0, ptr(out), ptr(ws), ws.numel(), T, K, N, 1,
                                           stream_of(xr)))
     return out[:K * N].view(K, N), out[K * N:]
+
+
+def linear_weight_grad_batched(x: Tensor, grads: Tensor):
+    """The same for several gradient planes against one input in one call: x [..., in], grads [P, ..., out]
+    (contiguous planes) -> (dW [P, in, out], db [P, out]).  The backward of a packed projection such as
+    [W_Q | W_K | W_V], whose three outputs are separate planes."""
+    K, N, P = x.shape[-1], grads.shape[-1], grads.shape[0]
+    xr, T, ldx = _rows("x", x, K)
+    require_gpu_f32("grads", grads)
+    if grads.numel() != P * T * N:
+        raise ValueError(f"grads has {grads.numel()} elements, expected {P} planes of {T} x {N}")
+    lib = _lib.load()
+    nbytes = lib.spgt_linear_weight_grad_workspace_bytes(T, K, N, P)
+    if nbytes == 0:
+        raise ValueError(f"unsupported weight-gradient shape: tokens={T} in={K} out={N} (out must be a multiple of 4)")
+    ws = _lib.workspace(nbytes, xr)
+    out = torch.empty((P, K * N + N), dtype=torch.float32, device=xr.device)
+    with torch.cuda.device(xr.device):
+        check(lib.spgt_linear_weight_grad(ptr(xr), ldx, 0, ptr(grads), N, T * N, ptr(out), ptr(ws), ws.numel(), T, K, N,
+                                          P, stream_of(xr)))
+    return out[:, :K * N].view(P, K, N), out[:, K * N:]

@@ -32,13 +32,48 @@ from ..extension.bind.galerkin_attention import (fold_ktv_into_fc, galerkin_atte
                                                  multihead_projection_with_position_rrc_cuda)
 from . import truncated_dft
 from ..extension.bind.linear import (encoder_tail_supported, fused_encoder_tail, fused_encoder_tail_folded,
-                                     fused_linear, linear_supported)
+                                     fused_linear, linear_supported, linear_weight_grad_batched)
 from .derived import derived, refreshes_derived
 from .layer import (FeedForward, activation_name, always_dropout, fused_linear_usable, gpu_inference,
                     linear_weight_kn, make_activation)
 
 
+class _PackedProjectionFunction(torch.autograd.Function):
+    """x -> (x W_Q + b_Q, x W_K + b_K, x W_V + b_V) as three contiguous planes: one launch of the fused linear
+    kernel over [W_Q | W_K | W_V] forward; backward dX by three chained launches of the same kernel on the
+    transposed weights and (dW, db) of all three by one pass over x and the three gradient planes."""
+
+    @staticmethod
+    def forward(ctx, x, wq, wk, wv, bq, bk, bv, packed_w, packed_b):
+        N, S, C = x.shape
+        ctx.save_for_backward(x, wq, wk, wv)
+        out = fused_linear(x.reshape(N * S, C), packed_w, packed_b, planes=3).view(3, N, S, C)
+        return out[0], out[1], out[2]
+
+    @staticmethod
+    def backward(ctx, dq, dk, dv):
+        x, wq, wk, wv = ctx.saved_tensors
+        N, S, C = x.shape
+        if dq.data_ptr() + 4 * dq.numel() == dk.data_ptr() and dk.data_ptr() + 4 * dk.numel() == dv.data_ptr() and \
+                dq.is_contiguous() and dk.is_contiguous() and dv.is_contiguous():
+            # the attention backward hands over the three planes of one buffer: no copy
+            grads = torch.as_strided(dq, (3, N * S, C), (N * S * C, C, 1))
+        else:
+            grads = torch.stack([dq.reshape(N * S, C), dk.reshape(N * S, C), dv.reshape(N * S, C)])
+        dx = None
+        if ctx.needs_input_grad[0]:
+            for g, w in zip(grads, (wq, wk, wv)):
+                dx = fused_linear(g, w.t().contiguous(), None, "none", dx)  # dx += g @ w^T
+            dx = dx.view(N, S, C)
+        dW, db = linear_weight_grad_batched(x.reshape(N * S, C), grads)
+        return dx, dW[0], dW[1], dW[2], db[0], db[1], db[2], None, None
+
+
 class Sp_GalerkinAttention(nn.Module):
+    # under autograd: the fused token-major core with its own backward (True) or the reference's sequence of three
+    # feature-major operators (False)
+    fused_training = True
+
     def __init__(self, dim_hidden, num_head, dim_position, norm_eps, attn_droprate, fc_droprate, xavier, diagonal,
                  symmetric) -> None:
         super().__init__()
@@ -122,6 +157,15 @@ class Sp_GalerkinAttention(nn.Module):
                 wide(Q, self.weight_Q, self.bias_Q), wide(K, self.weight_K, self.bias_K, self.ln_weight_K, self.ln_bias_K),
                 wide(V, self.weight_V, self.bias_V, self.ln_weight_V, self.ln_bias_V))
             X = X.transpose(1, 2).contiguous().view(N, seqlen, H * (dp + self.dim_head))
+        elif self._needs_graph(Q, K, V) and self.fused_training and Q is K and K is V and linear_supported(C, 3 * C) \
+                and linear_supported(C, C) and Q.is_cuda and Q.dtype == torch.float32:
+            # training on the token-major path: packed projection, then the fused core, both with their own backward
+            w, b = self._packed_qkv()
+            q, k, v = _PackedProjectionFunction.apply(Q.contiguous(), self.weight_Q, self.weight_K, self.weight_V,
+                                                      self.bias_Q, self.bias_K, self.bias_V, w, b)
+            pos = position.contiguous() if dp else None
+            X = galerkin_attention_fused(q, k, v, pos, self.ln_weight_K, self.ln_bias_K, self.ln_weight_V,
+                                         self.ln_bias_V, self.norm_eps, H, dp)
         elif self._needs_graph(Q, K, V):
             q = multihead_projection_with_position_rrc_cuda(Q, self.weight_Q, self.bias_Q, position, H, self.dim_head, dp)
             k = multihead_projection_layernorm_with_position_rrc_cuda(

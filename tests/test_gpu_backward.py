@@ -98,12 +98,16 @@ def test_heads_feature_to_token_major(gpu):
 
 
 @pytest.mark.parametrize("dp", [0, 2])
-def test_attention_module_trains_like_the_oracle(gpu, dp):
-    """Sp_GalerkinAttention under autograd (operator sequence + the three backwards) against autograd
+@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("B,S", [(2, 150), (3, 2501)])
+def test_attention_module_trains_like_the_oracle(gpu, dp, fused, B, S):
+    """Sp_GalerkinAttention under autograd, on the fused token-major path (packed projection + fused core, each
+    with its own backward) and on the reference's operator sequence with its three backwards, against autograd
     through the oracle's plain-PyTorch restatement, for the input and every parameter."""
     torch.manual_seed(5)
-    B, S, H = 2, 150, 4
+    H = 4
     m = L.Sp_GalerkinAttention(128, H, dp, 1e-6, 0.0, 0.0, 0.7, 0.01, False)
+    m.fused_training = fused
     with torch.no_grad():
         for prm in m.parameters():
             prm.add_(0.1 * torch.randn_like(prm))
@@ -120,3 +124,63 @@ def test_attention_module_trains_like_the_oracle(gpu, dp):
     assert max_rel(xg.grad.cpu().double(), xo.grad) < TOL
     for name, prm in m.named_parameters():
         assert max_rel(prm.grad.cpu().double(), po[name].grad) < TOL, name
+
+
+@pytest.mark.parametrize("dp", [0, 2])
+@pytest.mark.parametrize("B,H,S", [(1, 4, 1), (2, 4, 50), (1, 8, 777), (2, 4, 4099), (3, 4, 20011), (8, 4, 44521)])
+def test_fused_attention_backward(gpu, dp, B, H, S):
+    """galerkin_attention_fused under autograd (token-major forward + its two-pass backward) against autograd
+    through the oracle's attention core in float64: gradients of the plain projections q, k, v and of the four
+    LayerNorm parameters, one of them zero; ragged sequence lengths up to the benchmark shape."""
+    q, k, v = rnd(B, S, H * 32, seed=21), rnd(B, S, H * 32, seed=22) * 1.3 + 0.2, rnd(B, S, H * 32, seed=23)
+    pos = torch.rand(B, S, dp, generator=torch.Generator().manual_seed(24))
+    aff = [1 + 0.3 * rnd(H, 32, seed=25), 0.2 * rnd(H, 32, seed=26), 1 + 0.3 * rnd(H, 32, seed=27), 0.2 * rnd(H, 32, seed=28)]
+    aff[0][1, 5] = 0.0
+    G = rnd(B, S, H * (dp + 32), seed=29)
+    if S > 10000:  # the float64 oracle on one batch entry, the kernel on all of them
+        sl = slice(B - 1, B)
+    else:
+        sl = slice(0, B)
+    leaves = [t[sl].double().requires_grad_(True) for t in (q, k, v)] + [t.double().requires_grad_(True) for t in aff]
+    O.attention_core_token_major(leaves[0], leaves[1], leaves[2], pos[sl].double(), *leaves[3:], 1e-6, H).backward(G[sl].double())
+    dl = [t.to(gpu).requires_grad_(True) for t in (q, k, v)] + [t.to(gpu).requires_grad_(True) for t in aff]
+    out = ga.galerkin_attention_fused(dl[0], dl[1], dl[2], pos.to(gpu) if dp else None, *dl[3:], 1e-6, H, dp)
+    out.backward(G.to(gpu))
+    for i, name in enumerate(("dq", "dk", "dv")):
+        assert max_rel(dl[i].grad[sl].cpu().double(), leaves[i].grad) < TOL, name
+    if sl == slice(0, B):
+        for i, name in zip(range(3, 7), ("dgammaK", "dbetaK", "dgammaV", "dbetaV")):
+            assert dl[i].grad.shape == (H, 32)
+            assert max_rel(dl[i].grad.cpu().double(), leaves[i].grad) < TOL, name
+    # a second run gives the same bits (fixed summation order)
+    grads1 = [t.grad.clone() for t in dl]
+    for t in dl:
+        t.grad = None
+    ga.galerkin_attention_fused(dl[0], dl[1], dl[2], pos.to(gpu) if dp else None, *dl[3:], 1e-6, H, dp).backward(G.to(gpu))
+    assert all(torch.equal(a, t.grad) for a, t in zip(grads1, dl))
+
+
+def test_fused_attention_backward_layernorm_parameters_at_full_size(gpu):
+    """d gamma / d beta at B=8, S=44521 against float64 sums formed on the GPU from the same definitions
+    (dy * x_hat and dy summed over all tokens), where the float64 CPU oracle would take minutes."""
+    B, S, H, dp = 8, 44521, 4, 2
+    q, k, v = rnd(B, S, H * 32, seed=31).to(gpu), (rnd(B, S, H * 32, seed=32) * 1.3 + 0.2).to(gpu), rnd(B, S, H * 32, seed=33).to(gpu)
+    pos = torch.rand(B, S, dp, generator=torch.Generator().manual_seed(34)).to(gpu)
+    aff = [(1 + 0.3 * rnd(H, 32, seed=35)).to(gpu), (0.2 * rnd(H, 32, seed=36)).to(gpu),
+           (1 + 0.3 * rnd(H, 32, seed=37)).to(gpu), (0.2 * rnd(H, 32, seed=38)).to(gpu)]
+    G = rnd(B, S, H * (dp + 32), seed=39).to(gpu)
+    dl = [t.clone().requires_grad_(True) for t in (q, k, v)] + [t.clone().requires_grad_(True) for t in aff]
+    ga.galerkin_attention_fused(dl[0], dl[1], dl[2], pos, *dl[3:], 1e-6, H, dp).backward(G)
+    # the same function in float64 torch ops on the GPU, differentiated by autograd
+    ref = [t.double().requires_grad_(True) for t in (q, k, v)] + [t.double().requires_grad_(True) for t in aff]
+
+    def heads(x, gamma=None, beta=None):
+        x = x.view(B, S, H, 32)
+        if gamma is not None:
+            x = torch.nn.functional.layer_norm(x, [32], None, None, 1e-6) * gamma + beta
+        return torch.cat([pos.double().unsqueeze(2).expand(B, S, H, dp), x], -1).transpose(1, 2)  # [B, H, S, D]
+    Qh, Kh, Vh = heads(ref[0]), heads(ref[1], ref[3], ref[4]), heads(ref[2], ref[5], ref[6])
+    out = Qh @ (Kh.transpose(-2, -1) @ Vh / S)
+    out.transpose(1, 2).reshape(B, S, H * (dp + 32)).backward(G.double())
+    for i, name in enumerate(("dq", "dk", "dv", "dgammaK", "dbetaK", "dgammaV", "dbetaV")):
+        assert max_rel(dl[i].grad.double(), ref[i].grad) < TOL, name
