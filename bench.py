@@ -419,6 +419,20 @@ def kernel_rooflines(dev, use_graph=True):
     hbm("attention_fused_dp0", 4 * B * S * 128 * 4, fused(0))
     hbm("attention_fused_dp2", (3 * 128 + 136 + 2 * 2) * B * S * 4, fused(2))
 
+    # backward of the fused core: grad_out, q, k, v read, dq, dk, dv written (each counted once; the kernel
+    # reads grad_out twice), LayerNorm backward of K and V included
+    def fused_bwd(dp):
+        def make():
+            q, k, v = rn(B, S, 128), rn(B, S, 128), rn(B, S, 128)
+            pos = ru(B, S, 2) if dp else None
+            G = rn(B, S, H * (32 + dp))
+            ktv = rn(B, H, 32 + dp, 32 + dp)
+            return lambda: ga.gexts.galerkin_attention_fused_backward(G, q, k, v, pos, one, zero, one, zero, 1e-6, ktv,
+                                                                      H, dp)
+        return make
+    hbm("attention_fused_backward_dp0", 7 * B * S * 128 * 4, fused_bwd(0))
+    hbm("attention_fused_backward_dp2", (6 * 128 + 136 + 2) * B * S * 4, fused_bwd(2))
+
     def projection(layernorm, dp):
         def make():
             x, pos = rn(B, S, 128), ru(B, S, 2)[..., :dp]
@@ -555,6 +569,12 @@ def kernel_rooflines(dev, use_graph=True):
         # an encoder layer after the attention core in one launch (output projection 136 -> 128, residuals, FFN 256)
         mfma(f"encoder_tail_136_128_256_T{tag}", 2 * T * (136 * 128 + 2 * 128 * 256), T * (136 + 256) * 4,
              lin(136, lambda x, res: ln.fused_encoder_tail(x, res, wfc, bias, w4, b4, w5, bias, "silu"), True))
+    # weight + bias gradient of a Linear from token-major x and dL/dy (one pass over both, fixed summation order)
+    for T, tag in ((B * S, "356k"), (4 * 128 * 128, "65k")):
+        def make_wgrad():
+            x, gy = rn(T, 128), rn(T, 128)
+            return lambda: ln.linear_weight_grad(x, gy)
+        mfma(f"linear_weight_grad_128x128_T{tag}", 2 * T * 128 * 128, T * 256 * 4, make_wgrad)
     Tf = 4 * 211 * 211
     w6, b6 = rn(64, 64) / 8.0, rn(64)
     w7, b7, w8, b8 = rn(64, 256) / 8.0, rn(256), rn(1, 256) / 16.0, rn(1)

@@ -19,7 +19,7 @@ namespace spgt {
 // A = x[t][k0 + lane % 32], B = g[t][n0 + 32 nt + lane % 32].  Operand batches of BK steps are requested one
 // batch ahead of the MFMAs that consume them.
 template <int NT>
-__global__ __launch_bounds__(256) void xtg_partial_k(const float* __restrict__ X, int64_t ldx, int64_t x_batch,
+__global__ __launch_bounds__(256, 2) void xtg_partial_k(const float* __restrict__ X, int64_t ldx, int64_t x_batch,
                                                      const float* __restrict__ G, int64_t ldg, int64_t g_batch,
                                                      float* __restrict__ partial, int64_t T, int K, int N,
                                                      int tokens_per_chunk, int nstrip) {
@@ -60,40 +60,40 @@ __global__ __launch_bounds__(256) void xtg_partial_k(const float* __restrict__ X
     }
     const int last = (int)(t1 - t0) - 1;  // last valid token of the chunk, relative
     float xa[BK], ga[NT][BK], xb[BK], gb[NT][BK];
+    // fetch only requests (clamped addresses); the masks are applied when the values are used, so that a batch's
+    // loads stay in flight under the previous batch's MFMAs
     auto fetch = [&](float (&xv)[BK], float (&gv)[NT][BK], int batch) {
 #pragma unroll
         for (int u = 0; u < BK; ++u) {
-            const int rel = 2 * (batch * BK + u) + kh;
-            const bool ok = rel <= last;
-            const int64_t tr = ok ? rel : last;
-            const float xval = xp[tr * ldx];
-            xv[u] = (ok && kok) ? xval : 0.f;
+            const int64_t tr = min(2 * (batch * BK + u) + kh, last);
+            xv[u] = xp[tr * ldx];
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-                const float gval = gp[tr * ldg + goff[nt]];
-                gv[nt][u] = (ok && nok[nt]) ? gval : 0.f;
-            }
+            for (int nt = 0; nt < NT; ++nt) gv[nt][u] = gp[tr * ldg + goff[nt]];
         }
     };
-    auto multiply = [&](const float (&xv)[BK], const float (&gv)[NT][BK]) {
+    auto multiply = [&](const float (&xv)[BK], const float (&gv)[NT][BK], int batch) {
 #pragma unroll
-        for (int u = 0; u < BK; ++u)
+        for (int u = 0; u < BK; ++u) {
+            const bool ok = 2 * (batch * BK + u) + kh <= last;
+            const float xm = (ok && kok) ? xv[u] : 0.f;
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
-                acc[nt] = mfma32(xv[u], gv[nt][u], acc[nt]);
-                colsum[nt] += gv[nt][u];
+                const float gm = (ok && nok[nt]) ? gv[nt][u] : 0.f;
+                acc[nt] = mfma32(xm, gm, acc[nt]);
+                colsum[nt] += gm;
             }
+        }
     };
     const int nbatch = (steps + BK - 1) / BK;  // steps past the chunk's end contribute zeros
     if (nbatch > 0) fetch(xa, ga, 0);
     for (int bt = 0; bt < nbatch; bt += 2) {
         if (bt + 1 < nbatch) fetch(xb, gb, bt + 1);
         __builtin_amdgcn_sched_barrier(0);
-        multiply(xa, ga);
+        multiply(xa, ga, bt);
         __builtin_amdgcn_sched_barrier(0);
         if (bt + 2 < nbatch) fetch(xa, ga, bt + 2);
         __builtin_amdgcn_sched_barrier(0);
-        if (bt + 1 < nbatch) multiply(xb, gb);
+        if (bt + 1 < nbatch) multiply(xb, gb, bt + 1);
         __builtin_amdgcn_sched_barrier(0);
     }
     float* out = partial + ((int64_t)b * nchunk + chunk) * E;

@@ -12,7 +12,8 @@ import torch.nn.functional as F
 from torch import Tensor, nn
 
 from ..extension.bind.datamove import bias_activation_nchw_
-from ..extension.bind.linear import ffn_scalar_supported, fused_ffn_scalar, fused_linear, linear_supported
+from ..extension.bind.linear import (ffn_scalar_supported, fused_ffn_scalar, fused_linear, linear_supported,
+                                     linear_weight_grad)
 from .derived import derived, refreshes_derived, transposed_2d
 
 
@@ -41,6 +42,48 @@ def fused_linear_usable(X: Tensor, *linears: nn.Linear) -> bool:
     """gpu_inference, and the fused linear kernel has a variant for every layer's shape."""
     return (gpu_inference(X, *[p for l in linears for p in l.parameters()]) and
             all(linear_supported(l.in_features, l.out_features) for l in linears))
+
+
+class _LinearFunction(torch.autograd.Function):
+    """x @ W^T + b (+ residual) for an nn.Linear's parameters, forward and backward on this package's kernels:
+    the fused linear kernel forward and for dX = g @ W, and one pass over x and g for dW = g^T x and db (the
+    library's GEMM for that product, whose contraction runs over all tokens, takes 250 us at 65k tokens)."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias, weight_kn, residual):
+        ctx.save_for_backward(x, weight)
+        ctx.has_bias, ctx.has_residual = bias is not None, residual is not None
+        return fused_linear(x, weight_kn, bias, "none", residual)
+
+    @staticmethod
+    def backward(ctx, g):
+        x, weight = ctx.saved_tensors
+        g = g.contiguous()
+        dx = None
+        if ctx.needs_input_grad[0]:
+            w = weight.detach()
+            # g @ W: the fused kernel where it has a variant for [out -> in], else the library's GEMM
+            dx = (fused_linear(g, w.contiguous(), None, "none") if linear_supported(w.shape[0], w.shape[1])
+                  else torch.matmul(g, w))
+        dw = db = None
+        if ctx.needs_input_grad[1] or (ctx.has_bias and ctx.needs_input_grad[2]):
+            dw_kn, db = linear_weight_grad(x, g)
+            dw = dw_kn.t()
+            if not ctx.has_bias:
+                db = None
+        return dx, dw, db, None, (g if ctx.has_residual else None)
+
+
+def linear_trainable(X: Tensor, lin: nn.Linear) -> bool:
+    """True when linear_train serves lin(X): fp32 on a GPU, the fused linear kernel has a variant for the forward
+    product, and the weight gradient's row length is a multiple of 4."""
+    return (X.is_cuda and X.dtype == torch.float32 and lin.weight.dtype == torch.float32 and
+            linear_supported(lin.in_features, lin.out_features) and lin.out_features % 4 == 0)
+
+
+def linear_train(X: Tensor, lin: nn.Linear, residual: Tensor = None) -> Tensor:
+    """lin(X) (+ residual) with an autograd graph, on this package's kernels (see _LinearFunction)."""
+    return _LinearFunction.apply(X, lin.weight, lin.bias, linear_weight_kn(lin), residual)
 
 
 def always_dropout(X: Tensor, p: float) -> Tensor:
@@ -102,5 +145,12 @@ class FeedForward(nn.Module):
             H = fused_linear(X, linear_weight_kn(self.layer1), self.layer1.bias, activation_name(self.activation_layer))
             Y = fused_linear(H, linear_weight_kn(self.layer2), self.layer2.bias, "none", residual)
             return always_dropout(Y, self.droprate)
+        if linear_trainable(X, self.layer1) and linear_trainable(X, self.layer2):
+            # under autograd: the same kernels, with the weight gradients by this package's pass over the tokens
+            Hd = self.activation_layer(linear_train(X, self.layer1))
+            if self.droprate == 0:
+                return linear_train(Hd, self.layer2, residual)
+            Y = always_dropout(linear_train(Hd, self.layer2), self.droprate)
+            return Y if residual is None else residual + Y
         Y = always_dropout(self.layer2(self.activation_layer(self.layer1(X))), self.droprate)
         return Y if residual is None else residual + Y

@@ -35,7 +35,7 @@ from ..extension.bind.linear import (encoder_tail_supported, fused_encoder_tail,
                                      fused_linear, linear_supported, linear_weight_grad_batched)
 from .derived import derived, refreshes_derived
 from .layer import (FeedForward, activation_name, always_dropout, fused_linear_usable, gpu_inference,
-                    linear_weight_kn, make_activation)
+                    linear_train, linear_trainable, linear_weight_kn, make_activation)
 
 
 class _PackedProjectionFunction(torch.autograd.Function):
@@ -214,6 +214,11 @@ class Sp_GalerkinAttention(nn.Module):
         if fused_linear_usable(X, self.fc_layer) and (residual is None or self.fc_droprate == 0):
             Y = fused_linear(X, linear_weight_kn(self.fc_layer), self.fc_layer.bias, "none", residual)
             return always_dropout(Y, self.fc_droprate)
+        if linear_trainable(X, self.fc_layer):
+            if self.fc_droprate == 0:
+                return linear_train(X, self.fc_layer, residual)
+            Y = always_dropout(linear_train(X, self.fc_layer), self.fc_droprate)
+            return Y if residual is None else residual + Y
         Y = always_dropout(self.fc_layer(X), self.fc_droprate)
         return Y if residual is None else residual + Y
 

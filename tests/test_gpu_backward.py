@@ -184,3 +184,33 @@ def test_fused_attention_backward_layernorm_parameters_at_full_size(gpu):
     out.transpose(1, 2).reshape(B, S, H * (dp + 32)).backward(G.double())
     for i, name in enumerate(("dq", "dk", "dv", "dgammaK", "dbetaK", "dgammaV", "dbetaV")):
         assert max_rel(dl[i].grad.double(), ref[i].grad) < TOL, name
+
+
+@pytest.mark.parametrize("dp,act", [(0, "silu"), (2, "relu")])
+def test_encoder_layer_trains_like_the_oracle(gpu, dp, act):
+    """A whole Sp_EncoderLayer under autograd (packed projection, fused attention core, output projection and
+    feed-forward net, each with this package's backward) against autograd through the oracle in float64: the
+    gradient of the input and of every parameter."""
+    torch.manual_seed(7)
+    B, S, H = 2, 1333, 4
+    m = L.Sp_EncoderLayer(128, H, dp, 1e-6, 0.0, 0.0, 0.7, 0.01, False, 256, 0.0, act)
+    with torch.no_grad():
+        for prm in m.parameters():
+            prm.add_(0.05 * torch.randn_like(prm))
+    x = rnd(B, S, 128, seed=41)
+    pos = torch.rand(B, S, dp, generator=torch.Generator().manual_seed(42))
+    G = rnd(B, S, 128, seed=43)
+    po = {k: v.detach().double().clone().requires_grad_(True) for k, v in m.state_dict().items()}
+    xo = x.double().requires_grad_(True)
+    transposed = {k: (v.t() if k.rsplit(".", 1)[-1] in ("weight_Q", "weight_K", "weight_V") else v) for k, v in po.items()}
+    O.encoder_layer(transposed, xo, pos.double(), H, 1e-6, act).backward(G.double())
+    m = m.to(gpu)
+    xg = x.to(gpu).requires_grad_(True)
+    out = m(xg, pos.to(gpu))
+    out.backward(G.to(gpu))
+    with torch.no_grad():
+        assert max_rel(out.detach().cpu().double(), O.encoder_layer(transposed, xo, pos.double(), H, 1e-6, act).detach()) < TOL
+    assert max_rel(xg.grad.cpu().double(), xo.grad) < TOL
+    for name, prm in m.named_parameters():
+        assert prm.grad is not None, name
+        assert max_rel(prm.grad.cpu().double(), po[name].grad) < TOL, name
