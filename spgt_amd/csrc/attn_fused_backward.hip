@@ -18,28 +18,45 @@
 #include "spgt_host.h"
 #include "spgt_kernels.h"
 
+// Cache policy of the touch-once streams: q (pass 1) and k, v (pass 2) are read once, grad_out is read by both
+// passes (182 MB at B=8, S=44521: it can stay in the 256 MB last-level cache between them if the other streams
+// do not displace it).
+#ifndef SPGT_BWD_NT_Q
+#define SPGT_BWD_NT_Q true
+#endif
+#ifndef SPGT_BWD_NT_KV
+#define SPGT_BWD_NT_KV true
+#endif
+
 namespace spgt {
 
 // Pass 1: partial[b][h][chunk] = sum over the chunk's tokens of Q~[s]^T G[s]  (D x D, row-major; the dp x dp
 // corner is not needed by pass 2 and is written as zero).
-// grid (nchunk, H/4, B), block 256: wave = head.  Lane l: token slot t = l/16, feature pair p = l%16; a 16x16x4
-// MFMA contracts the four token slots: A = q[2p + ta], B = G[2p + tb].
-template <int DP, int U>
-__global__ __launch_bounds__(256) void qtg_partial_tm(const float* __restrict__ Q, int64_t ld,
-                                                      const float* __restrict__ pos, const float* __restrict__ G,
-                                                      float* __restrict__ partial, int S, int H,
-                                                      int tokens_per_chunk) {
+// grid (nchunk, H/4, B), block 256 * NSUB: wave w handles head 4 blockIdx.y + w % 4 on the sub-range w / 4 of the
+// workgroup's chunk; with NSUB > 1 the sub-ranges' tiles meet in LDS and the workgroup writes their sum (sub-ranges
+// in increasing order), as in the forward's K/V pass: one 1024-thread workgroup per CU on long sequences.
+// Lane l: token slot t = l/16, feature pair p = l%16; a 16x16x4 MFMA contracts the four token slots:
+// A = q[2p + ta], B = G[2p + tb].
+template <int DP, int U, int NSUB>
+__global__ __launch_bounds__(256 * NSUB) void qtg_partial_tm(const float* __restrict__ Q, int64_t ld,
+                                                             const float* __restrict__ pos,
+                                                             const float* __restrict__ G,
+                                                             float* __restrict__ partial, int S, int H,
+                                                             int tokens_per_chunk) {
     constexpr int D = DP + 32;
+    extern __shared__ __attribute__((aligned(16))) float sub_tiles[];  // NSUB > 1: [NSUB][4 heads][D * D]
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    const int wave = (threadIdx.x >> 6) & 3;
+    const int sub = threadIdx.x >> 8;
     const int h = blockIdx.y * 4 + wave;
     const int b = blockIdx.z;
     const int chunk = blockIdx.x;
     const int nchunk = gridDim.x;
     const int t = lane >> 4;
     const int p = lane & 15;
-    const int s0 = min(S, chunk * tokens_per_chunk);
-    const int s1 = min(S, s0 + tokens_per_chunk);
+    const int sub_len = tokens_per_chunk / NSUB;
+    const int s0 = min(S, chunk * tokens_per_chunk + sub * sub_len);
+    const int s1 = min(S, s0 + sub_len);
     const int64_t ldg = (int64_t)H * D;
     const float* qb = Q + ((int64_t)b * S + s0) * ld + h * 32 + 2 * p;
     const float* gb = G + ((int64_t)b * S + s0) * ldg + h * D;
@@ -56,7 +73,7 @@ __global__ __launch_bounds__(256) void qtg_partial_tm(const float* __restrict__ 
 
     auto load_unit = [&](int rel) {
         Unit u;
-        u.q = *reinterpret_cast<const float2*>(qb + (int64_t)rel * ld);
+        u.q = ld_stream<SPGT_BWD_NT_Q>(reinterpret_cast<const float2*>(qb + (int64_t)rel * ld));
         const float* gr = gb + (int64_t)rel * ldg;
         u.g = *reinterpret_cast<const float2*>(gr + DP + 2 * p);
         if (DP == 2) {
@@ -115,7 +132,8 @@ __global__ __launch_bounds__(256) void qtg_partial_tm(const float* __restrict__ 
         }
     }
     // acc[ta][tb][r] = N[DP + 2 (4 t + r) + ta][DP + 2 p + tb]
-    float* tile = partial + (((int64_t)b * H + h) * nchunk + chunk) * (D * D);
+    float* tile = NSUB > 1 ? sub_tiles + (sub * 4 + wave) * (D * D)
+                           : partial + (((int64_t)b * H + h) * nchunk + chunk) * (D * D);
 #pragma unroll
     for (int ta = 0; ta < 2; ++ta)
 #pragma unroll
@@ -141,6 +159,22 @@ __global__ __launch_bounds__(256) void qtg_partial_tm(const float* __restrict__ 
             if (p == 0) {
                 tile[0] = 0.f; tile[1] = 0.f; tile[D] = 0.f; tile[D + 1] = 0.f;
             }
+        }
+    }
+    if constexpr (NSUB > 1) {
+        __syncthreads();
+        constexpr int E4 = D * D / 4;  // float4 per tile
+        for (int e = threadIdx.x; e < 4 * E4; e += 256 * NSUB) {
+            const int hh = e / E4;
+            const int r4 = e - hh * E4;
+            float4 sum = *reinterpret_cast<const float4*>(sub_tiles + hh * (D * D) + 4 * r4);
+#pragma unroll
+            for (int q = 1; q < NSUB; ++q) {
+                const float4 v = *reinterpret_cast<const float4*>(sub_tiles + (q * 4 + hh) * (D * D) + 4 * r4);
+                sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
+            }
+            float* dst = partial + (((int64_t)b * H + blockIdx.y * 4 + hh) * nchunk + chunk) * (D * D) + 4 * r4;
+            *reinterpret_cast<float4*>(dst) = sum;
         }
     }
 }
@@ -223,10 +257,10 @@ __global__ __launch_bounds__(256) void attn_bwd_apply_tm(
         const float* kp = kbase + (int64_t)s * ld;
         const float* vp = vbase + (int64_t)s * ld;
         const float* gp = gbase + (int64_t)s * ldg + DP + 4 * g;
-        u.k0 = *reinterpret_cast<const float4*>(kp);
-        u.k1 = *reinterpret_cast<const float4*>(kp + 16);
-        u.v0 = *reinterpret_cast<const float4*>(vp);
-        u.v1 = *reinterpret_cast<const float4*>(vp + 16);
+        u.k0 = ld_stream<SPGT_BWD_NT_KV>(reinterpret_cast<const float4*>(kp));
+        u.k1 = ld_stream<SPGT_BWD_NT_KV>(reinterpret_cast<const float4*>(kp + 16));
+        u.v0 = ld_stream<SPGT_BWD_NT_KV>(reinterpret_cast<const float4*>(vp));
+        u.v1 = ld_stream<SPGT_BWD_NT_KV>(reinterpret_cast<const float4*>(vp + 16));
         u.g0 = *reinterpret_cast<const float2*>(gp);       // rows of 34 floats: 8-byte pieces
         u.g1 = *reinterpret_cast<const float2*>(gp + 2);
         u.g2 = *reinterpret_cast<const float2*>(gp + 16);
@@ -403,8 +437,11 @@ namespace {
 
 size_t round256(size_t x) { return (x + 255) & ~(size_t)255; }
 
+constexpr int kBwdSub = 4;           // token sub-ranges per 1024-thread workgroup of pass 1 on long sequences
+constexpr int kBwdSubMinTokens = 256;  // per wave
+
 struct FusedBwdPlan {
-    int tpc1, nchunk1, tpc2, nchunk2;
+    int nsub, tpc1, nchunk1, tpc2, nchunk2;
     size_t off_n, off_gpart, bytes;
 };
 
@@ -417,7 +454,15 @@ FusedBwdPlan fused_bwd_plan(int B, int S, int H, int dp) {
     // chunks as tile_reduce sums
     const int t1 = S / std::max(1, 3 * cus / bg) < 128 ? cus : 3 * cus;
     const int per1 = std::min(kReduceChains * kReduceMaxPerChain, std::max(1, t1 / bg));
+    p.nsub = 1;
     p.tpc1 = std::max(16, ceil_div(ceil_div(S, per1), 16) * 16);
+    // long sequences: one workgroup of kBwdSub x 4 waves per CU, whose sub-range tiles are summed in LDS
+    const int gs = 16 * kBwdSub;
+    const int tpc_sub = std::max(gs, ceil_div(ceil_div(S, std::max(1, cus / bg)), gs) * gs);
+    if (tpc_sub / kBwdSub >= kBwdSubMinTokens && ceil_div(S, tpc_sub) <= kReduceChains * kReduceMaxPerChain) {
+        p.nsub = kBwdSub;
+        p.tpc1 = tpc_sub;
+    }
     p.nchunk1 = ceil_div(S, p.tpc1);
     // pass 2: two workgroups per CU
     const int per2 = std::max(1, 2 * cus / bg);
@@ -472,10 +517,24 @@ extern "C" int spgt_galerkin_attention_fused_backward(
     float* gpart = reinterpret_cast<float*>(ws + p.off_gpart);
     const float* pos = position ? position : K;  // never dereferenced when dp == 0
     const dim3 grid1(p.nchunk1, H / 4, B), grid2(p.nchunk2, H / 4, B);
-    if (dp == 0)
-        hipLaunchKernelGGL((qtg_partial_tm<0, 4>), grid1, dim3(256), 0, stream, Q, ld_in, pos, grad_out, partial, S, H, p.tpc1);
-    else
-        hipLaunchKernelGGL((qtg_partial_tm<2, 4>), grid1, dim3(256), 0, stream, Q, ld_in, pos, grad_out, partial, S, H, p.tpc1);
+    if (p.nsub > 1) {
+        const size_t lds = (size_t)kBwdSub * 4 * D * D * sizeof(float);
+        const void* fn = dp == 0 ? reinterpret_cast<const void*>(&qtg_partial_tm<0, 4, kBwdSub>)
+                                 : reinterpret_cast<const void*>(&qtg_partial_tm<2, 4, kBwdSub>);
+        if (lds > 64 * 1024 &&
+            hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+            return fail(SPGT_ERR_LAUNCH, "galerkin_attention_fused_backward: pass 1 was refused its dynamic LDS size");
+        if (dp == 0)
+            hipLaunchKernelGGL((qtg_partial_tm<0, 4, kBwdSub>), grid1, dim3(256 * kBwdSub), lds, stream, Q, ld_in, pos,
+                               grad_out, partial, S, H, p.tpc1);
+        else
+            hipLaunchKernelGGL((qtg_partial_tm<2, 4, kBwdSub>), grid1, dim3(256 * kBwdSub), lds, stream, Q, ld_in, pos,
+                               grad_out, partial, S, H, p.tpc1);
+    } else if (dp == 0) {
+        hipLaunchKernelGGL((qtg_partial_tm<0, 4, 1>), grid1, dim3(256), 0, stream, Q, ld_in, pos, grad_out, partial, S, H, p.tpc1);
+    } else {
+        hipLaunchKernelGGL((qtg_partial_tm<2, 4, 1>), grid1, dim3(256), 0, stream, Q, ld_in, pos, grad_out, partial, S, H, p.tpc1);
+    }
     hipLaunchKernelGGL(tile_reduce, dim3(ceil_div(D * D, 256), B * H), dim3(1024), 0, stream, partial, nmat, D * D,
                        p.nchunk1, 1.0f / (float)S);
     if (dp == 0)
