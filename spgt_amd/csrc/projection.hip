@@ -28,6 +28,16 @@ namespace spgt {
 #define SPGT_PROJ_TILE 32
 #endif
 constexpr int kProjTile = SPGT_PROJ_TILE;  // tokens per tile (64 = two interleaved sub-tiles: 159 us against 150 us at B=8, S=44521)
+// Results are collected per wave in LDS for kProjStage tiles (96 tokens of each of the wave's 32 feature rows) and
+// leave as 384-byte runs per row, two rows per store instruction: rows of [D, S] start at arbitrary 4-byte offsets
+// when S is odd, so every piece of a row touches a partial cache line at either end, and with 128-byte pieces (one
+// tile at a time, straight from the accumulators) the kernel wrote 1.43 times its output.  0 = store every tile
+// straight from the accumulators.
+#ifndef SPGT_PROJ_STAGE
+#define SPGT_PROJ_STAGE 3
+#endif
+constexpr int kProjStage = SPGT_PROJ_STAGE;
+constexpr int kProjStagePitch = 32 * (kProjStage > 0 ? kProjStage : 1) + 4;  // floats per staged row (16-byte rows)
 
 // grid (nchunk, H/4, B), block 256.  KC = dim_hidden / 128.
 template <int KC, int DP, bool LN>
@@ -39,9 +49,11 @@ __global__ __launch_bounds__(256) void projection_rrc_k(
     constexpr int D = DP + 32;
     constexpr int PITCH = K + 1;
     constexpr int TT = KC <= 2 ? kProjTile : 32;  // tokens per tile (wide inputs: the staging registers decide)
-    extern __shared__ float xs[];  // [TT][PITCH]
+    extern __shared__ __attribute__((aligned(16))) float xs[];  // [TT][PITCH], then [4 waves][32][kProjStagePitch]
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
+    constexpr int XS_WORDS = (TT * PITCH + 3) / 4 * 4;
+    float* const os = xs + XS_WORDS + wave * (32 * kProjStagePitch);  // this wave's staged rows
     const int h = blockIdx.y * 4 + wave;
     const int b = blockIdx.z;
     const int tk = lane & 31;
@@ -159,12 +171,45 @@ __global__ __launch_bounds__(256) void projection_rrc_k(
                 for (int r = 0; r < 16; ++r) y[r] = fmaf(y[r] * rstd, greg[r], oreg[r]);
                 if (kh == 0 && s < s_end) invsigma[((int64_t)b * H + h) * S + s] = rstd;
             }
-            if (s < s_end) {
+            if (kProjStage == 0) {
+                if (s < s_end) {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const int i = 8 * (r >> 2) + 4 * kh + (r & 3);
+                        ob[(int64_t)(DP + i) * S + s] = y[r];
+                    }
+                }
+            } else {
+                // into the wave's LDS rows; they leave when kProjStage tiles are there or the chunk ends
+                const int slot = ((s0 - s_begin) / 32 + tb) % kProjStage;
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int i = 8 * (r >> 2) + 4 * kh + (r & 3);
-                    ob[(int64_t)(DP + i) * S + s] = y[r];
+                    os[i * kProjStagePitch + slot * 32 + tk] = y[r];
                 }
+                const bool last_tile = s0 + (tb + 1) * 32 >= s_end;
+                if (slot == kProjStage - 1 || last_tile) {
+                    const int w0 = s0 + tb * 32 - slot * 32;      // first token of the staged window
+                    const int nvalid = min(s_end - w0, (slot + 1) * 32);
+                    // lane (tk, kh): tokens 4 tk .. 4 tk + 3 of row 2 q + kh; 4-byte aligned 16-byte stores
+                    const int t4 = 4 * tk;  // lanes past the window (tk >= 8 kProjStage) read its last piece and store nothing
+                    const int t4r = min(t4, 32 * kProjStage - 4);
+#pragma unroll
+                    for (int q = 0; q < 16; ++q) {
+                        const int i = 2 * q + kh;
+                        const float4 v = *reinterpret_cast<const float4*>(os + i * kProjStagePitch + t4r);
+                        float* dst = ob + (int64_t)(DP + i) * S + w0 + t4;
+                        if (t4 + 3 < nvalid) {
+                            *reinterpret_cast<v4f_a4*>(dst) = v4f{v.x, v.y, v.z, v.w};
+                        } else if (t4 < nvalid) {
+                            dst[0] = v.x;
+                            if (t4 + 1 < nvalid) dst[1] = v.y;
+                            if (t4 + 2 < nvalid) dst[2] = v.z;
+                        }
+                    }
+                }
+            }
+            if (s < s_end) {
                 if (DP == 2) ob[(int64_t)kh * S + s] = pos[((int64_t)b * S + s) * 2 + kh];
             }
         }
@@ -179,7 +224,7 @@ void launch_projection(const float* x, const float* W, const float* bias, const 
                        hipStream_t stream) {
     constexpr int K = 128 * KC;
     constexpr int TT = KC <= 2 ? kProjTile : 32;
-    const size_t lds = (size_t)TT * (K + 1) * sizeof(float);
+    const size_t lds = ((size_t)(TT * (K + 1) + 3) / 4 * 4 + (kProjStage > 0 ? 4 * 32 * kProjStagePitch : 0)) * sizeof(float);
     // about two workgroups per CU; chunks are whole tiles
     const int per_b = std::max(1, 2 * device_cu_count() / std::max(1, B * (H / 4)));
     const int tpc = std::max(TT, ceil_div(ceil_div(S, per_b), TT) * TT);
