@@ -300,6 +300,14 @@ class Sp_SpectralConv2D(nn.Module):
                                                    self.fourier_weight[1], m)
             return fused_linear(X0, linear_weight_kn(self.residual_layer), self.residual_layer.bias,
                                 activation_name(self.activation_layer), Y)
+        if (needs_graph and self.use_truncated_dft and self.droprate == 0 and X.is_cuda and X.dtype == torch.float32
+                and truncated_dft.supported(r, m) and truncated_dft.spectral_linear_trainable(r, cin, cout, m)):
+            # training on the truncated-DFT route: the layer's linear part (residual Linear + spectral term) is one
+            # autograd function whose backward runs the adjoint stages on the same kernels
+            lin = self.residual_layer
+            pre = truncated_dft.spectral_linear_train(X.contiguous(), self.fourier_weight[0], self.fourier_weight[1], m,
+                                                      lin.weight, lin.bias, linear_weight_kn(lin))
+            return self.activation_layer(pre)
         res = self.residual_layer(X)
         X = always_dropout(X, self.droprate)
         if truncated:

@@ -24,6 +24,7 @@ from typing import Dict, Tuple
 import torch
 from torch import Tensor
 
+from ..extension.bind.linear import fused_linear, linear_supported, linear_weight_grad
 from ..extension.bind.datamove import (inverse_table_operand, spectral_inverse_linear,
                                        spectral_inverse_linear_supported, spectral_modes_compact, spectral_modes_middle,
                                        spectral_modes_middle_supported, truncated_dft_rows_forward,
@@ -78,12 +79,93 @@ def spectral_modes_apply_linear(x: Tensor, weight_1: Tensor, weight_2: Tensor, m
     spectral layer after dropout; requires fused_tail_supported."""
     N, r, _, cin = x.shape
     fw, gh, ghi, fwi = dft_tables(r, m, x.device)
-    key = (r, m, str(x.device))
-    if key not in _OPERAND_TABLES:
-        _OPERAND_TABLES[key] = inverse_table_operand(fwi)
     yp = truncated_dft_rows_forward(x, fw, planar=True)             # [N, 2m, r, Cin]
     up = spectral_modes_middle(yp, gh, ghi, weight_1, weight_2)     # [N, 2m, r, Cout]
-    return spectral_inverse_linear(up, _OPERAND_TABLES[key], x, linear_weight_kn, linear_bias, activation)
+    return spectral_inverse_linear(up, _operand_table(r, m, x.device), x, linear_weight_kn, linear_bias, activation)
+
+
+def _operand_table(r: int, m: int, device) -> Tensor:
+    key = (r, m, str(device))
+    if key not in _OPERAND_TABLES:
+        _OPERAND_TABLES[key] = inverse_table_operand(dft_tables(r, m, device)[3])
+    return _OPERAND_TABLES[key]
+
+
+class _SpectralLinearFunction(torch.autograd.Function):
+    """x @ W_lin^T + b + irfft2(W_f . truncate(rfft2(x))) on the truncated-DFT route, with its backward on the same
+    kernels.  Every stage is linear, so the backward runs the adjoint stages in reverse: the inverse row transform's
+    adjoint is a forward row transform with the inverse table, the forward one's an inverse row transform with the
+    forward table, and the adjoint of the complex-linear middle (DFT along h, channel contraction, inverse DFT
+    along h) is the same kernel with conjugate-transposed tables and weights.  The Fourier weights' gradient,
+    dW[kh, kw, c, o] = sum_n conj(Z[n, kh, c, kw]) dO[n, kh, o, kw], is formed from the retained modes (a few MB)
+    by library products."""
+
+    @staticmethod
+    def forward(ctx, x, weight_1, weight_2, lin_weight, lin_bias, lin_weight_kn, m):
+        N, r, _, cin = x.shape
+        fw, gh, ghi, _ = dft_tables(r, m, x.device)
+        yp = truncated_dft_rows_forward(x, fw, planar=True)                         # [N, 2m, r, Cin]
+        up = spectral_modes_middle(yp, gh, ghi, weight_1, weight_2)                 # [N, 2m, r, Cout]
+        out = spectral_inverse_linear(up, _operand_table(r, m, x.device), x, lin_weight_kn, lin_bias, None)
+        ctx.save_for_backward(x, weight_1, weight_2, lin_weight, yp)
+        ctx.m, ctx.has_bias = m, lin_bias is not None
+        return out
+
+    @staticmethod
+    def backward(ctx, g):
+        x, weight_1, weight_2, lin_weight, yp = ctx.saved_tensors
+        m = ctx.m
+        g = g.contiguous()
+        N, r, _, cout = g.shape
+        cin = x.shape[-1]
+        fw, gh, ghi, fwi = dft_tables(r, m, x.device)
+        ghi_h = ghi.conj().t().contiguous()                                         # [2m, r]
+        dup = truncated_dft_rows_forward(g, fwi, planar=True)                       # [N, 2m, r, Cout] = Fi^T g
+        dx = None
+        if ctx.needs_input_grad[0]:
+            gh_h = gh.conj().t().contiguous()                                       # [r, 2m]
+            conj_t = lambda w: torch.view_as_real(torch.view_as_complex(w).conj().transpose(2, 3).contiguous())
+            w1h, w2h = conj_t(weight_1.detach()), conj_t(weight_2.detach())         # [m, m, Cout, Cin, 2]
+            if cin <= 64:
+                dyp = spectral_modes_middle(dup, ghi_h, gh_h, w1h, w2h)             # [N, 2m, r, Cin]
+            else:  # the middle kernel writes at most 64 channels per call
+                dyp = torch.cat([spectral_modes_middle(dup, ghi_h, gh_h, w1h[:, :, :, c0:c0 + 64].contiguous(),
+                                                       w2h[:, :, :, c0:c0 + 64].contiguous())
+                                 for c0 in range(0, cin, 64)], dim=3)
+            dx = truncated_dft_rows_inverse(dyp, fw, planar=True)                   # [N, r, r, Cin]
+            g2, w = g.view(-1, cout), lin_weight.detach()
+            if linear_supported(cout, cin):
+                dx = fused_linear(g2, w.contiguous(), None, "none", dx.view(-1, cin)).view(N, r, r, cin)
+            else:
+                dx = dx + torch.matmul(g2, w).view(N, r, r, cin)
+        dw_lin = db = dw1 = dw2 = None
+        if ctx.needs_input_grad[3] or (ctx.has_bias and ctx.needs_input_grad[4]):
+            dw_kn, db = linear_weight_grad(x.view(-1, cin), g.view(-1, cout))
+            dw_lin = dw_kn.t()
+            if not ctx.has_bias:
+                db = None
+        if ctx.needs_input_grad[1] or ctx.needs_input_grad[2]:
+            yc = torch.complex(yp[:, 0::2], yp[:, 1::2])                            # [N, kw, h, Cin]
+            z = torch.einsum("kh,nwhc->nkwc", gh, yc)                               # [N, 2m, kw, Cin]
+            duc = torch.complex(dup[:, 0::2], dup[:, 1::2])                         # [N, kw, h, Cout]
+            do = torch.einsum("kh,nwho->nkwo", ghi_h, duc)                          # [N, 2m, kw, Cout]
+            dw = torch.view_as_real(torch.einsum("nkwc,nkwo->kwco", z.conj(), do))  # [2m, kw, Cin, Cout, 2]
+            dw1, dw2 = dw[:m], dw[m:]
+        return dx, dw1, dw2, dw_lin, db, None, None
+
+
+def spectral_linear_trainable(r: int, cin: int, cout: int, m: int) -> bool:
+    """True when spectral_linear_train serves this shape: the three-launch route forward, and for the backward a
+    row-transform variant for both widths and a weight-gradient row length that is a multiple of 4."""
+    return (fused_tail_supported(r, cin, cout, m) and truncated_dft_rows_supported(r, cout, m) and
+            spectral_modes_middle_supported(r, cout, min(cin, 64), m) and cout % 4 == 0)
+
+
+def spectral_linear_train(x: Tensor, weight_1: Tensor, weight_2: Tensor, m: int, lin_weight: Tensor, lin_bias,
+                          lin_weight_kn: Tensor) -> Tensor:
+    """x @ lin_weight^T + lin_bias + irfft2(W . truncate(rfft2(x))) for x [N, r, r, Cin], with an autograd graph
+    (see _SpectralLinearFunction); requires spectral_linear_trainable."""
+    return _SpectralLinearFunction.apply(x, weight_1, weight_2, lin_weight, lin_bias, lin_weight_kn, m)
 
 
 def spectral_modes_apply(x: Tensor, weight_1: Tensor, weight_2: Tensor, m: int) -> Tensor:

@@ -214,3 +214,34 @@ def test_encoder_layer_trains_like_the_oracle(gpu, dp, act):
     for name, prm in m.named_parameters():
         assert prm.grad is not None, name
         assert max_rel(prm.grad.cpu().double(), po[name].grad) < TOL, name
+
+
+@pytest.mark.parametrize("N,r,cin,cout,m,act", [(2, 33, 64, 64, 5, "silu"), (2, 40, 128, 32, 6, "silu"),
+                                                (1, 64, 32, 32, 8, "relu"), (2, 21, 128, 64, 4, "silu"),
+                                                (1, 141, 64, 32, 12, "silu")])
+def test_spectral_conv_trains_like_the_oracle(gpu, N, r, cin, cout, m, act):
+    """Sp_SpectralConv2D under autograd on the truncated-DFT route (forward and adjoint stages on the same kernels)
+    against autograd through the oracle's rfft2 / irfft2 restatement in float64: the gradient of the input, of
+    both Fourier weights and of the residual Linear."""
+    from spgt_amd.network import truncated_dft
+    torch.manual_seed(23)
+    layer = L.Sp_SpectralConv2D(cin, cout, m, 0.0, act)
+    with torch.no_grad():
+        for w in layer.fourier_weight:
+            w.copy_(torch.randn(w.shape) / cin)
+    x = rnd(N, r, r, cin, seed=51)
+    G = rnd(N, r, r, cout, seed=52)
+    po = {k: v.detach().double().clone().requires_grad_(True) for k, v in layer.state_dict().items()}
+    xo = x.double().requires_grad_(True)
+    want = O.spectral_conv2d(po, xo, m, act, weight_layout="sp")
+    want.backward(G.double())
+    assert truncated_dft.spectral_linear_trainable(r, cin, cout, m)
+    layer = layer.to(gpu)
+    xg = x.to(gpu).requires_grad_(True)
+    got = layer(xg)
+    got.backward(G.to(gpu))
+    assert max_rel(got.detach().cpu().double(), want.detach()) < TOL
+    assert max_rel(xg.grad.cpu().double(), xo.grad) < TOL
+    for name, prm in layer.named_parameters():
+        assert prm.grad is not None, name
+        assert max_rel(prm.grad.cpu().double(), po[name].grad) < TOL, name
