@@ -380,12 +380,19 @@ def kernel_rooflines(dev, use_graph=True):
 
     rot = Rotation(dev, use_graph)
     rows = {}
+    # eager runs (under a profiler): one fill kernel before every row, so that a trace can be cut into rows
+    marker = None if use_graph else torch.zeros(64, dtype=torch.int16, device=dev)  # no other int16 fill in the run
+
+    def mark():
+        if marker is not None:
+            marker.fill_(len(rows))
 
     def common(r):
         return {"us": round(r["t"] * 1e6, 2), "us_one_set": round(r["t_one"] * 1e6, 2), "operand_sets": r["sets"],
                 "bytes_between_reuse": int(r["between"]), "timing": r["mode"]}
 
     def hbm(name, nbytes, make, traffic=None):
+        mark()
         r = rot.run(make, traffic if traffic is not None else nbytes)
         row = common(r)
         ok = r["between"] >= ROTATE_BYTES
@@ -396,6 +403,7 @@ def kernel_rooflines(dev, use_graph=True):
         rows[name] = row
 
     def mfma(name, flops, nbytes, make):
+        mark()
         r = rot.run(make, nbytes)
         row = common(r)
         row.update({"flops": int(flops), "TFLOP/s": round(flops / r["t"] / 1e12, 2),
