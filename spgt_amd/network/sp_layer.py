@@ -54,8 +54,11 @@ class _PackedProjectionFunction(torch.autograd.Function):
     def backward(ctx, dq, dk, dv):
         x, wq, wk, wv = ctx.saved_tensors
         N, S, C = x.shape
-        if dq.data_ptr() + 4 * dq.numel() == dk.data_ptr() and dk.data_ptr() + 4 * dk.numel() == dv.data_ptr() and \
-                dq.is_contiguous() and dk.is_contiguous() and dv.is_contiguous():
+        planes = (dq, dk, dv)
+        same_buffer = (all(t.is_contiguous() and t.dtype == torch.float32 for t in planes) and
+                       len({t.untyped_storage().data_ptr() for t in planes}) == 1 and
+                       dk.data_ptr() - dq.data_ptr() == 4 * dq.numel() == dv.data_ptr() - dk.data_ptr())
+        if same_buffer:
             # the attention backward hands over the three planes of one buffer: no copy
             grads = torch.as_strided(dq, (3, N * S, C), (N * S * C, C, 1))
         else:

@@ -245,3 +245,28 @@ def test_spectral_conv_trains_like_the_oracle(gpu, N, r, cin, cout, m, act):
     for name, prm in layer.named_parameters():
         assert prm.grad is not None, name
         assert max_rel(prm.grad.cpu().double(), po[name].grad) < TOL, name
+
+
+def test_packed_projection_function_with_separate_gradient_tensors(gpu):
+    """The packed Q | K | V projection's backward when its three gradients are separate allocations (the attention
+    backward hands it three planes of one buffer, which takes the no-copy branch): against torch's own autograd."""
+    from spgt_amd.network.sp_layer import _PackedProjectionFunction
+    torch.manual_seed(3)
+    N, S, C = 2, 777, 128
+    x = torch.randn(N, S, C, device=gpu, requires_grad=True)
+    ws = [(torch.randn(C, C, device=gpu) / C ** 0.5).requires_grad_(True) for _ in range(3)]
+    bs = [torch.randn(C, device=gpu).requires_grad_(True) for _ in range(3)]
+    packed_w = torch.cat([w.detach() for w in ws], dim=1).contiguous()
+    packed_b = torch.cat([b.detach() for b in bs]).contiguous()
+    outs = _PackedProjectionFunction.apply(x, *ws, *bs, packed_w, packed_b)
+    gs = [torch.randn(N, S, C, device=gpu) for _ in range(3)]
+    got = torch.autograd.grad(outs, [x, *ws, *bs], gs)
+    x2 = x.detach().double().requires_grad_(True)
+    ws2 = [w.detach().double().requires_grad_(True) for w in ws]
+    bs2 = [b.detach().double().requires_grad_(True) for b in bs]
+    ref_outs = [x2 @ w + b for w, b in zip(ws2, bs2)]
+    want = torch.autograd.grad(ref_outs, [x2, *ws2, *bs2], [g.double() for g in gs])
+    for o, r in zip(outs, ref_outs):
+        assert max_rel(o.detach().double().cpu(), r.detach().cpu()) < TOL
+    for g, w in zip(got, want):
+        assert max_rel(g.double().cpu(), w.cpu()) < TOL
