@@ -44,16 +44,32 @@ def fused_linear_usable(X: Tensor, *linears: nn.Linear) -> bool:
             all(linear_supported(l.in_features, l.out_features) for l in linears))
 
 
+def _weight_and_bias_grad(x: Tensor, g: Tensor, has_bias: bool):
+    """(dW [out, in], db [out] or None) of y = x @ W^T + b from g = dL/dy: one pass over x and g with a fixed
+    summation order.  The pass writes rows of out features, which must be a multiple of 4; a Linear with a narrow
+    output (the regression head's 128 -> 1) is served with the roles swapped, dW = g^T x."""
+    out_f, in_f = g.shape[-1], x.shape[-1]
+    if out_f % 4 == 0:
+        dw_kn, db = linear_weight_grad(x, g)
+        return dw_kn.t(), (db if has_bias else None)
+    dw, _ = linear_weight_grad(g, x)  # [out, in]
+    return dw, (g.reshape(-1, out_f).sum(0) if has_bias else None)
+
+
 class _LinearFunction(torch.autograd.Function):
     """x @ W^T + b (+ residual) for an nn.Linear's parameters, forward and backward on this package's kernels:
-    the fused linear kernel forward and for dX = g @ W, and one pass over x and g for dW = g^T x and db (the
-    library's GEMM for that product, whose contraction runs over all tokens, takes 250 us at 65k tokens)."""
+    the fused linear kernel forward and for dX = g @ W where it has a variant for the shape (the library's GEMM
+    otherwise), and one pass over x and g for dW = g^T x and db (the library's GEMM for that product, whose
+    contraction runs over all tokens, takes 250 us at 65k tokens)."""
 
     @staticmethod
     def forward(ctx, x, weight, bias, weight_kn, residual):
         ctx.save_for_backward(x, weight)
         ctx.has_bias, ctx.has_residual = bias is not None, residual is not None
-        return fused_linear(x, weight_kn, bias, "none", residual)
+        if weight_kn is not None:
+            return fused_linear(x, weight_kn, bias, "none", residual)
+        y = F.linear(x, weight, bias)
+        return y if residual is None else y + residual
 
     @staticmethod
     def backward(ctx, g):
@@ -67,23 +83,49 @@ class _LinearFunction(torch.autograd.Function):
                   else torch.matmul(g, w))
         dw = db = None
         if ctx.needs_input_grad[1] or (ctx.has_bias and ctx.needs_input_grad[2]):
-            dw_kn, db = linear_weight_grad(x, g)
-            dw = dw_kn.t()
-            if not ctx.has_bias:
-                db = None
+            dw, db = _weight_and_bias_grad(x, g, ctx.has_bias)
         return dx, dw, db, None, (g if ctx.has_residual else None)
 
 
 def linear_trainable(X: Tensor, lin: nn.Linear) -> bool:
-    """True when linear_train serves lin(X): fp32 on a GPU, the fused linear kernel has a variant for the forward
-    product, and the weight gradient's row length is a multiple of 4."""
+    """True when linear_train serves lin(X): fp32 on a GPU and a row length the weight-gradient pass can write
+    (out_features, or else in_features, a multiple of 4)."""
     return (X.is_cuda and X.dtype == torch.float32 and lin.weight.dtype == torch.float32 and
-            linear_supported(lin.in_features, lin.out_features) and lin.out_features % 4 == 0)
+            (lin.out_features % 4 == 0 or lin.in_features % 4 == 0))
 
 
 def linear_train(X: Tensor, lin: nn.Linear, residual: Tensor = None) -> Tensor:
     """lin(X) (+ residual) with an autograd graph, on this package's kernels (see _LinearFunction)."""
-    return _LinearFunction.apply(X, lin.weight, lin.bias, linear_weight_kn(lin), residual)
+    kn = linear_weight_kn(lin) if linear_supported(lin.in_features, lin.out_features) else None
+    return _LinearFunction.apply(X, lin.weight, lin.bias, kn, residual)
+
+
+class _SplitLinearFunction(torch.autograd.Function):
+    """Linear(cat([x, extra], -1)) without the concatenation, for up to four extra columns (the decoder's input
+    layer on hidden features and grid coordinates): forward = the fused linear kernel with the extra columns as a
+    rank-r update in its epilogue; backward: dX = g @ W[:, :in_x] by the library's GEMM, the two column blocks of
+    dW and db by this package's pass over the tokens."""
+
+    @staticmethod
+    def forward(ctx, x, extra, weight, bias, weight_x_kn, weight_extra_kn):
+        ctx.save_for_backward(x, extra, weight)
+        ctx.has_bias = bias is not None
+        return fused_linear(x, weight_x_kn, bias, "none", x_extra=extra, weight_extra_kn=weight_extra_kn)
+
+    @staticmethod
+    def backward(ctx, g):
+        x, extra, weight = ctx.saved_tensors
+        g = g.contiguous()
+        in_x = x.shape[-1]
+        w = weight.detach()
+        dx = torch.matmul(g, w[:, :in_x]) if ctx.needs_input_grad[0] else None
+        dextra = torch.matmul(g, w[:, in_x:]) if ctx.needs_input_grad[1] else None
+        dw = db = None
+        if ctx.needs_input_grad[2] or (ctx.has_bias and ctx.needs_input_grad[3]):
+            dwx, db = _weight_and_bias_grad(x, g, ctx.has_bias)
+            dwe, _ = _weight_and_bias_grad(extra, g, False)
+            dw = torch.cat([dwx, dwe], dim=1)
+        return dx, dextra, dw, db, None, None
 
 
 def always_dropout(X: Tensor, p: float) -> Tensor:

@@ -11,7 +11,7 @@ from torch import Tensor, nn
 from ..extension.bind.datamove import bilinear_nhwc_affine, denormalize_boundary
 from ..extension.bind.linear import fused_linear, linear_supported
 from .derived import derived, refreshes_derived, transposed_2d
-from .layer import FeedForward, always_dropout, gpu_inference
+from .layer import FeedForward, _SplitLinearFunction, always_dropout, gpu_inference
 from .model import DownScaler2D, UpScaler2D
 from .sp_layer import Sp_EncoderLayer, Sp_SpectralConv2D
 
@@ -93,6 +93,12 @@ class Sp_DecoderRegressor(nn.Module):
             # the GEMM runs over the hidden features; the grid columns are a rank-2 update in its epilogue
             w_x, w_grid = self._split_weight_kn(dim_x)
             X = fused_linear(X, w_x, self.spatial_fc_layer.bias, "none", x_extra=grid, weight_extra_kn=w_grid)
+        elif (X.is_cuda and X.dtype == torch.float32 and grid is not None and grid.is_cuda and
+                grid.dtype == torch.float32 and W.dtype == torch.float32 and linear_supported(dim_x, W.size(0)) and
+                0 < W.size(1) - dim_x <= 4 and grid.size(-1) == W.size(1) - dim_x and W.size(0) % 4 == 0):
+            # under autograd: the same kernel forward, weight gradients by this package's pass over the tokens
+            w_x, w_grid = self._split_weight_kn(dim_x)
+            X = _SplitLinearFunction.apply(X.contiguous(), grid.contiguous(), W, self.spatial_fc_layer.bias, w_x, w_grid)
         else:
             X = F.linear(X, W[:, :dim_x], self.spatial_fc_layer.bias) + F.linear(grid, W[:, dim_x:])
         for layer in self.layers:

@@ -247,6 +247,59 @@ def test_spectral_conv_trains_like_the_oracle(gpu, N, r, cin, cout, m, act):
         assert max_rel(prm.grad.cpu().double(), po[name].grad) < TOL, name
 
 
+@pytest.mark.parametrize("N,r,dim_x,hidden,m", [(2, 33, 128, 32, 5), (1, 40, 64, 64, 6)])
+def test_decoder_regressor_trains_like_the_oracle(gpu, N, r, dim_x, hidden, m):
+    """Sp_DecoderRegressor under autograd (input layer on hidden features and grid columns without a concatenation,
+    spectral layers on the truncated-DFT route, regression head with one output feature) against autograd through
+    the oracle in float64: output, gradient of the hidden features and of every parameter."""
+    from spgt_amd.network import sp_model as M
+    torch.manual_seed(29)
+    dec = M.Sp_DecoderRegressor(2, dim_x, 1, 2, hidden, m, 0.0, "silu")
+    with torch.no_grad():
+        for layer in dec.layers:
+            for w in layer.fourier_weight:
+                w.copy_(torch.randn(w.shape) / hidden)
+    x = rnd(N, r, r, dim_x, seed=61)
+    grid = rnd(N, r, r, 2, seed=62)
+    G = rnd(N, r, r, 1, seed=63)
+    po = {k: v.detach().double().clone().requires_grad_(True) for k, v in dec.state_dict().items()}
+    xo = x.double().requires_grad_(True)
+    want = O.decoder_regressor(po, xo, grid.double(), 2, m, "silu", weight_layout="sp")
+    want.backward(G.double())
+    dec = dec.to(gpu)
+    xg = x.to(gpu).requires_grad_(True)
+    got = dec(xg, grid.to(gpu))
+    got.backward(G.to(gpu))
+    assert max_rel(got.detach().cpu().double(), want.detach()) < TOL
+    assert max_rel(xg.grad.cpu().double(), xo.grad) < TOL
+    for name, prm in dec.named_parameters():
+        assert prm.grad is not None, name
+        assert max_rel(prm.grad.cpu().double(), po[name].grad) < TOL, name
+
+
+@pytest.mark.parametrize("in_f,hid,out_f", [(32, 128, 1), (128, 256, 128), (36, 40, 3)])
+def test_feed_forward_trains_like_the_oracle(gpu, in_f, hid, out_f):
+    """FeedForward under autograd, including a head with one output feature (weight gradient with the roles of
+    input and gradient swapped) and widths no kernel here serves (torch throughout)."""
+    from spgt_amd.network.layer import FeedForward
+    torch.manual_seed(31)
+    ffn = FeedForward(in_f, out_f, hid, 0.0, "silu")
+    x = rnd(3, 1201, in_f, seed=71)
+    G = rnd(3, 1201, out_f, seed=72)
+    po = {k: v.detach().double().clone().requires_grad_(True) for k, v in ffn.state_dict().items()}
+    xo = x.double().requires_grad_(True)
+    want = O.feed_forward(po, xo, "silu")
+    want.backward(G.double())
+    ffn = ffn.to(gpu)
+    xg = x.to(gpu).requires_grad_(True)
+    got = ffn(xg)
+    got.backward(G.to(gpu))
+    assert max_rel(got.detach().cpu().double(), want.detach()) < TOL
+    assert max_rel(xg.grad.cpu().double(), xo.grad) < TOL
+    for name, prm in ffn.named_parameters():
+        assert max_rel(prm.grad.cpu().double(), po[name].grad) < TOL, name
+
+
 def test_packed_projection_function_with_separate_gradient_tensors(gpu):
     """The packed Q | K | V projection's backward when its three gradients are separate allocations (the attention
     backward hands it three planes of one buffer, which takes the no-copy branch): against torch's own autograd."""
