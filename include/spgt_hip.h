@@ -325,6 +325,16 @@ int spgt_bilinear_resample(const float* src, const float* pre_bias, float* dst, 
                            int pre_activation, int pre_activation_count, int post_activation,
                            spgt_stream_t stream);
 
+/* Backward of the resampling: the adjoint of F.interpolate(mode='bilinear', align_corners=True) from
+ * [H_in, W_in] to [H_out, W_out], grad_in[i] = sum over the outputs o that read source i of weight(o, i) *
+ * grad_out[o], gathered per source position in a fixed order (no atomic additions).  The reference leaves this
+ * step to autograd of F.interpolate in DownScaler2D / UpScaler2D (network/model.py:30-38, 59-64).  Both tensors
+ * have the same layout: SPGT_LAYOUT_NCHW (grad_out [N, C, H_out, W_out], grad_in [N, C, H_in, W_in]) or
+ * SPGT_LAYOUT_NHWC (grad_out [N, H_out, W_out, C], grad_in [N, H_in, W_in, C]; C a multiple of 4, 16-byte
+ * aligned).  Every element of grad_in is written. */
+int spgt_bilinear_adjoint(const float* grad_out, float* grad_in, int N, int C, int H_in, int W_in, int H_out,
+                          int W_out, int layout, spgt_stream_t stream);
+
 /* UpScaler2D's last F.interpolate (network/model.py:63-64) on a channels-last source together with the grid
  * columns' share of the decoder's input layer Linear(cat([X, grid])) (network/sp_model.py:60, 118):
  *   dst[n, y, x, c] = bilinear(src)[n, y, x, c] + sum_e extra[n, y, x, e] * w_extra[e, c]

@@ -54,6 +54,7 @@ SIGNATURES = {
     "spgt_bilinear_align_corners_nhwc": (_i, [_p, _p, _i, _i, _i, _i, _i, _i, _p]),
     "spgt_bilinear_resample": (_i, [_p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p]),
     "spgt_bilinear_nhwc_affine": (_i, [_p, _p, _i, _i, _i, _i, _i, _i, _p, _p, _i, _p]),
+    "spgt_bilinear_adjoint": (_i, [_p, _p, _i, _i, _i, _i, _i, _i, _i, _p]),
     "spgt_upsample_conv3x3_gather": (_i, [_p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p]),
     "spgt_bilinear_resample_concat": (_i, [_p, _p, _p, _p, _i, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p]),
     "spgt_bias_activation_nchw": (_i, [_p, _p, _i, _i, _i64, _i, _i, _p]),

@@ -718,6 +718,120 @@ __global__ __launch_bounds__(256) void bilinear_nhwc_affine_k(const float* __res
     }
 }
 
+// ---- adjoint of the resampling (its backward) -------------------------------------------------------------------
+// The resampling is linear in its source, out[o] = sum over i of A[o][i] in[i] per axis with at most two non-zero
+// weights per output, so the gradient of the source is grad_in[i] = sum over o of A[o][i] grad_out[o].  The reference
+// leaves this to autograd of F.interpolate (network/model.py:30-38, 59-64), whose backward scatters with atomic
+// additions; here every source position gathers from the few outputs that touch it, in a fixed order.
+
+// Weight with which output index o reads source index i: both taps count (at the last source index they coincide).
+__device__ __forceinline__ float adjoint_weight(float scale, int o, int i, int in_size) {
+    const ResampleTap t = resample_tap(scale, o, in_size);
+    return (t.i1 == i ? t.l0 : 0.f) + (t.i1 + t.ip == i ? t.l1 : 0.f);
+}
+
+__device__ __forceinline__ bool adjoint_touches(float scale, int o, int i, int in_size) {
+    const ResampleTap t = resample_tap(scale, o, in_size);
+    return t.i1 == i || t.i1 + t.ip == i;
+}
+
+// The outputs that touch source index i: first source index scale * o in (i - 1, i + 1).  The bounds are estimated
+// in floating point and then widened while the neighbouring output still touches i, with the forward's own
+// arithmetic, so that no contribution is lost to rounding; an output inside the range that does not touch i has
+// weight zero.  lo > hi when no output reads i (down-sampling by more than two).
+struct AdjointRange {
+    int lo, hi;
+};
+__device__ __forceinline__ AdjointRange adjoint_range(float scale, int i, int in_size, int out_size) {
+    AdjointRange r;
+    if (!(scale > 0.f)) {
+        r.lo = 0, r.hi = out_size - 1;
+        return r;
+    }
+    const float inv = 1.0f / scale;
+    r.lo = min(max((int)ceilf(((float)i - 1.f) * inv), 0), out_size - 1);
+    r.hi = max(min((int)floorf(((float)i + 1.f) * inv), out_size - 1), 0);
+    while (r.lo > 0 && adjoint_touches(scale, r.lo - 1, i, in_size)) --r.lo;
+    while (r.hi < out_size - 1 && adjoint_touches(scale, r.hi + 1, i, in_size)) ++r.hi;
+    return r;
+}
+
+// Channels-last on both sides: grad_out [N, Hout, Wout, C] -> grad_in [N, Hin, Win, C], C a multiple of 4.  A thread
+// makes 4 channels of one source pixel; the lanes of a pixel read 16-byte pieces of one 4*C-byte run.  G outputs
+// of a row are requested together (indices past the range repeat its last one with weight zero).
+// grid: ceil(N*Hin*Win*C/4 / 256) rounded up to a multiple of 8, block 256.
+template <int G>
+__global__ __launch_bounds__(256) void bilinear_adjoint_nhwc_k(const float* __restrict__ gout,
+                                                               float* __restrict__ gin, int C4, int Hin, int Win,
+                                                               int Hout, int Wout, float hscale, float wscale,
+                                                               unsigned items) {
+    const unsigned f = (unsigned)xcd_contiguous_tile() * 256u + threadIdx.x;
+    if (f >= items) return;
+    const int q = (int)(f % (unsigned)C4);
+    const unsigned pix = f / (unsigned)C4;
+    const int x = (int)(pix % (unsigned)Win);
+    const unsigned line = pix / (unsigned)Win;
+    const int y = (int)(line % (unsigned)Hin);
+    const int64_t n = line / (unsigned)Hin;
+    const int64_t C = 4 * (int64_t)C4;
+    const AdjointRange ry = adjoint_range(hscale, y, Hin, Hout), rx = adjoint_range(wscale, x, Win, Wout);
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int oy = ry.lo; oy <= ry.hi; ++oy) {
+        const float hw = adjoint_weight(hscale, oy, y, Hin);
+        const float* row = gout + ((n * Hout + oy) * (int64_t)Wout) * C + 4 * q;
+        for (int ox0 = rx.lo; ox0 <= rx.hi; ox0 += G) {
+            float4 v[G];
+            float w[G];
+#pragma unroll
+            for (int j = 0; j < G; ++j) {
+                v[j] = *reinterpret_cast<const float4*>(row + (int64_t)min(ox0 + j, rx.hi) * C);
+                w[j] = ox0 + j <= rx.hi ? hw * adjoint_weight(wscale, ox0 + j, x, Win) : 0.f;
+            }
+#pragma unroll
+            for (int j = 0; j < G; ++j) {
+                acc.x = fmaf(w[j], v[j].x, acc.x), acc.y = fmaf(w[j], v[j].y, acc.y);
+                acc.z = fmaf(w[j], v[j].z, acc.z), acc.w = fmaf(w[j], v[j].w, acc.w);
+            }
+        }
+    }
+    *reinterpret_cast<float4*>(gin + (int64_t)pix * C + 4 * q) = acc;
+}
+
+// Planes on both sides: grad_out [planes, Hout, Wout] -> grad_in [planes, Hin, Win].  A thread makes one source
+// position of 4 consecutive planes at a time; lanes run along the source row.
+// grid (ceil(Win/64), ceil(Hin/4), ceil(planes/4) or fewer), block (64, 4).
+__global__ __launch_bounds__(256) void bilinear_adjoint_planes_k(const float* __restrict__ gout,
+                                                                 float* __restrict__ gin, int planes, int Hin,
+                                                                 int Win, int Hout, int Wout, float hscale,
+                                                                 float wscale) {
+    const int x = blockIdx.x * 64 + threadIdx.x;
+    const int y = blockIdx.y * 4 + threadIdx.y;
+    if (x >= Win || y >= Hin) return;
+    const AdjointRange ry = adjoint_range(hscale, y, Hin, Hout), rx = adjoint_range(wscale, x, Win, Wout);
+    const int64_t oplane = (int64_t)Hout * Wout;
+    for (int64_t p0 = (int64_t)blockIdx.z * 4; p0 < planes; p0 += (int64_t)gridDim.z * 4) {
+        float acc[4] = {0.f, 0.f, 0.f, 0.f};
+        const float* base[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) base[j] = gout + min(p0 + j, (int64_t)planes - 1) * oplane;  // repeats, unwritten
+        for (int oy = ry.lo; oy <= ry.hi; ++oy) {
+            const float hw = adjoint_weight(hscale, oy, y, Hin);
+            for (int ox = rx.lo; ox <= rx.hi; ++ox) {
+                const float w = hw * adjoint_weight(wscale, ox, x, Win);
+                const int64_t o = (int64_t)oy * Wout + ox;
+                float v[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) v[j] = base[j][o];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[j] = fmaf(w, v[j], acc[j]);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if (p0 + j < planes) gin[((p0 + j) * Hin + y) * Win + x] = acc[j];
+    }
+}
+
 // UpScaler2D's interpolate -> conv3x3(padding 1) -> bias -> activation(s) (network/model.py:59-62) with the channel
 // mixing done before the interpolation.  Both steps are linear, so
 //   conv(interp(X))[y, x, co] = sum over the 9 taps (ky, kx) of interp(Z_t)[y + ky - 1, x + kx - 1, co],
@@ -1136,6 +1250,45 @@ extern "C" int spgt_bilinear_nhwc_affine(const float* src, float* dst, int N, in
     hipLaunchKernelGGL(spgt::bilinear_nhwc_affine_k, dim3((unsigned)blocks), dim3(256), 0, stream, src, dst, C / 4,
                        H_in, W_in, H_out, W_out, hscale, wscale, extra, w_extra, n_extra, (unsigned)items);
     return check_launch("bilinear_nhwc_affine");
+}
+
+extern "C" int spgt_bilinear_adjoint(const float* grad_out, float* grad_in, int N, int C, int H_in, int W_in,
+                                     int H_out, int W_out, int layout, hipStream_t stream) {
+    if (!grad_out || !grad_in) return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear_adjoint: null pointer argument");
+    if (N <= 0 || C <= 0 || H_in <= 0 || W_in <= 0 || H_out <= 0 || W_out <= 0)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear_adjoint: sizes must be positive");
+    if (H_in > (1 << 23) || W_in > (1 << 23) || H_out > (1 << 23) || W_out > (1 << 23))
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear_adjoint: image sides above 2^23");
+    const float hscale = H_out > 1 ? (float)(H_in - 1) / (float)(H_out - 1) : 0.f;
+    const float wscale = W_out > 1 ? (float)(W_in - 1) / (float)(W_out - 1) : 0.f;
+    if (layout == SPGT_LAYOUT_NHWC) {
+        if (C % 4 != 0 || !aligned16(grad_out) || !aligned16(grad_in))
+            return fail(SPGT_ERR_INVALID_ARGUMENT,
+                        "bilinear_adjoint: channels-last needs C a multiple of 4 and 16-byte aligned tensors");
+        const int64_t items = (int64_t)N * H_in * W_in * (C / 4);
+        if (items > (int64_t)INT32_MAX - 2048 || (int64_t)N * H_out * W_out * (C / 4) > (int64_t)INT32_MAX)
+            return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear_adjoint: more than 2^33 elements on one side");
+        const int64_t blocks = ceil_div(ceil_div(items, (int64_t)256), (int64_t)8) * 8;
+        // an up-sampling's sources are each read by three or four outputs of a row, a down-sampling's by one or two
+        if (wscale < 1.f)
+            hipLaunchKernelGGL(spgt::bilinear_adjoint_nhwc_k<4>, dim3((unsigned)blocks), dim3(256), 0, stream, grad_out,
+                               grad_in, C / 4, H_in, W_in, H_out, W_out, hscale, wscale, (unsigned)items);
+        else
+            hipLaunchKernelGGL(spgt::bilinear_adjoint_nhwc_k<2>, dim3((unsigned)blocks), dim3(256), 0, stream, grad_out,
+                               grad_in, C / 4, H_in, W_in, H_out, W_out, hscale, wscale, (unsigned)items);
+    } else if (layout == SPGT_LAYOUT_NCHW) {
+        const int64_t planes = (int64_t)N * C;
+        if (planes > INT32_MAX || !aligned4(grad_out) || !aligned4(grad_in))
+            return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear_adjoint: more than 2^31 planes, or misaligned tensors");
+        if (ceil_div(H_in, 4) > 65535)
+            return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear_adjoint: H_in above 262140");
+        const dim3 grid(ceil_div(W_in, 64), ceil_div(H_in, 4), (unsigned)std::min<int64_t>(ceil_div(planes, (int64_t)4), 4096));
+        hipLaunchKernelGGL(spgt::bilinear_adjoint_planes_k, grid, dim3(64, 4), 0, stream, grad_out, grad_in, (int)planes,
+                           H_in, W_in, H_out, W_out, hscale, wscale);
+    } else {
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear_adjoint: layout must be NCHW or NHWC (both tensors alike)");
+    }
+    return check_launch("bilinear_adjoint");
 }
 
 extern "C" int spgt_bilinear_resample(const float* src, const float* pre_bias, float* dst, int N, int C, int H_in,

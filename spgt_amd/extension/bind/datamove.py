@@ -157,6 +157,32 @@ def _bilinear_align_corners_nhwc(X: Tensor, size) -> Tensor:
     return out
 
 
+def _bilinear_adjoint(grad: Tensor, in_size, nhwc: bool = False) -> Tensor:
+    """The gradient of the source of a bilinear align_corners resampling from in_size = (H_in, W_in) to grad's
+    size: grad [N, C, H_out, W_out] -> [N, C, H_in, W_in], or with nhwc both tensors channels-last
+    ([N, H, W, C], C a multiple of 4).  A gather per source position in a fixed order."""
+    require_gpu_f32("grad", grad)
+    if grad.dim() != 4:
+        raise ValueError("grad must have four dimensions")
+    H_in, W_in = (in_size, in_size) if isinstance(in_size, int) else tuple(in_size)
+    if nhwc:
+        N, H_out, W_out, C = grad.shape
+        if C % 4:
+            raise ValueError("the channel count must be a multiple of 4")
+        out = torch.empty((N, H_in, W_in, C), dtype=grad.dtype, device=grad.device)
+    else:
+        N, C, H_out, W_out = grad.shape
+        out = torch.empty((N, C, H_in, W_in), dtype=grad.dtype, device=grad.device)
+    if out.numel() == 0:
+        return out
+    if grad.numel() == 0:
+        return out.zero_()
+    with torch.cuda.device(grad.device):
+        check(_lib.load().spgt_bilinear_adjoint(ptr(grad), ptr(out), N, C, H_in, W_in, H_out, W_out, 1 if nhwc else 0,
+                                                stream_of(grad)))
+    return out
+
+
 def _truncated_dft_rows_supported(r: int, channels: int, modes: int) -> bool:
     return bool(_lib.load().spgt_truncated_dft_rows_supported(int(r), int(channels), int(modes)))
 
@@ -525,6 +551,7 @@ dexts = SimpleNamespace(
     spectral_mode_contract=_spectral_mode_contract,
     spectral_modes_compact=_spectral_modes_compact,
     bilinear_align_corners=_bilinear_align_corners,
+    bilinear_adjoint=_bilinear_adjoint,
 )
 
 
@@ -606,6 +633,70 @@ def bilinear_align_corners(X: Tensor, size) -> Tensor:
 def bilinear_align_corners_nhwc(X: Tensor, size) -> Tensor:
     """F.interpolate(X, size, mode='bilinear', align_corners=True).permute(0, 2, 3, 1), contiguous (inference only)."""
     return dexts.bilinear_align_corners_nhwc(X.detach(), size)
+
+
+def _pair(size):
+    return (size, size) if isinstance(size, int) else tuple(size)
+
+
+class Bilinear_Function(torch.autograd.Function):
+    """F.interpolate(X, size, mode='bilinear', align_corners=True) on [N, C, H, W]; backward = bilinear_adjoint."""
+
+    @staticmethod
+    def forward(ctx: Any, X: Tensor, size):
+        ctx.in_size = tuple(X.shape[-2:])
+        return dexts.bilinear_align_corners(X.contiguous(), _pair(size))
+
+    @staticmethod
+    def backward(ctx: Any, grad_out: Tensor):
+        return dexts.bilinear_adjoint(grad_out.contiguous(), ctx.in_size, False), None
+
+
+class Bilinear_To_Nhwc_Function(torch.autograd.Function):
+    """The same from [N, C, H, W] to channels-last [N, H', W', C].  The backward gathers channels-last (C a multiple
+    of 4) and hands the gradient back as the [N, C, H, W] view of that tensor."""
+
+    @staticmethod
+    def forward(ctx: Any, X: Tensor, size):
+        ctx.in_size = tuple(X.shape[-2:])
+        return dexts.bilinear_align_corners_nhwc(X.contiguous(), _pair(size))
+
+    @staticmethod
+    def backward(ctx: Any, grad_out: Tensor):
+        return dexts.bilinear_adjoint(grad_out.contiguous(), ctx.in_size, True).permute(0, 3, 1, 2), None
+
+
+class Bilinear_Nhwc_Function(torch.autograd.Function):
+    """The same with channels-last tensors on both sides, [N, H, W, C] -> [N, H', W', C], C a multiple of 4."""
+
+    @staticmethod
+    def forward(ctx: Any, X: Tensor, size):
+        ctx.in_size = tuple(X.shape[1:3])
+        return dexts.bilinear_nhwc_affine(X.contiguous(), _pair(size))
+
+    @staticmethod
+    def backward(ctx: Any, grad_out: Tensor):
+        return dexts.bilinear_adjoint(grad_out.contiguous(), ctx.in_size, True), None
+
+
+def bilinear_adjoint(grad: Tensor, in_size, nhwc: bool = False) -> Tensor:
+    """Gradient of the source of a bilinear align_corners resampling from in_size to grad's size."""
+    return dexts.bilinear_adjoint(grad.detach(), in_size, nhwc)
+
+
+def bilinear_train(X: Tensor, size) -> Tensor:
+    """F.interpolate(X, size, mode='bilinear', align_corners=True) on [N, C, H, W] with an autograd graph."""
+    return Bilinear_Function.apply(X, size)
+
+
+def bilinear_to_nhwc_train(X: Tensor, size) -> Tensor:
+    """interpolate(X).permute(0, 2, 3, 1), contiguous, with an autograd graph; X [N, C, H, W], C a multiple of 4."""
+    return Bilinear_To_Nhwc_Function.apply(X, size)
+
+
+def bilinear_nhwc_train(X: Tensor, size) -> Tensor:
+    """Channels-last interpolate, [N, H, W, C] -> [N, H', W', C], with an autograd graph; C a multiple of 4."""
+    return Bilinear_Nhwc_Function.apply(X, size)
 
 
 def bilinear_resample(X: Tensor, size, src_nhwc: bool = False, dst_nhwc: bool = False, pre_activation=None,

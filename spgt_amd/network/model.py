@@ -8,6 +8,7 @@ import torch.nn.functional as F
 from torch import Tensor, nn
 
 from ..extension.bind.datamove import (bilinear_align_corners, bilinear_align_corners_nhwc, bilinear_nhwc_affine,
+                                       bilinear_nhwc_train, bilinear_to_nhwc_train, bilinear_train,
                                        bilinear_resample, bilinear_resample_concat, conv3x3_resample,
                                        conv3x3_resample_supported, upsample_conv3x3_gather)
 from ..extension.bind.linear import fused_linear, linear_supported
@@ -35,17 +36,33 @@ def get_resolution_size(r_large: int, r_small: int):
     return (fine, mid, small, mid, fine)
 
 
+def _channels_last_memory(X: Tensor) -> bool:
+    """True for an [N, C, H, W] tensor that is a permuted view of a contiguous [N, H, W, C] one."""
+    return X.dim() == 4 and not X.is_contiguous() and X.permute(0, 2, 3, 1).is_contiguous()
+
+
 def resample(X: Tensor, size) -> Tensor:
-    """Bilinear, align_corners=True, on [N, C, H, W]."""
+    """Bilinear, align_corners=True, on [N, C, H, W].  A channels-last input gives a channels-last result, as
+    F.interpolate does."""
     if torch.is_grad_enabled() and X.requires_grad:
-        return F.interpolate(X, size=tuple(size), mode="bilinear", align_corners=True)
+        if not (X.is_cuda and X.dtype == torch.float32 and X.dim() == 4):
+            return F.interpolate(X, size=tuple(size), mode="bilinear", align_corners=True)
+        if _channels_last_memory(X) and X.size(1) % 4 == 0:
+            return bilinear_nhwc_train(X.permute(0, 2, 3, 1), tuple(size)).permute(0, 3, 1, 2)
+        return bilinear_train(X, tuple(size))
     return bilinear_align_corners(X.contiguous(), tuple(size))
 
 
 def resample_to_nhwc(X: Tensor, size) -> Tensor:
     """Bilinear, align_corners=True, [N, C, H, W] -> [N, H', W', C] (contiguous)."""
     if torch.is_grad_enabled() and X.requires_grad:
-        return F.interpolate(X, size=tuple(size), mode="bilinear", align_corners=True).permute(0, 2, 3, 1)
+        if not (X.is_cuda and X.dtype == torch.float32 and X.dim() == 4):
+            return F.interpolate(X, size=tuple(size), mode="bilinear", align_corners=True).permute(0, 2, 3, 1)
+        if X.size(1) % 4 != 0:
+            return bilinear_train(X, tuple(size)).permute(0, 2, 3, 1)
+        if _channels_last_memory(X):
+            return bilinear_nhwc_train(X.permute(0, 2, 3, 1), tuple(size))
+        return bilinear_to_nhwc_train(X, tuple(size))
     return bilinear_align_corners_nhwc(X.contiguous(), tuple(size))
 
 

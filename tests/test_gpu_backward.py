@@ -277,6 +277,38 @@ def test_decoder_regressor_trains_like_the_oracle(gpu, N, r, dim_x, hidden, m):
         assert max_rel(prm.grad.cpu().double(), po[name].grad) < TOL, name
 
 
+@pytest.mark.parametrize("r,r_attn,dim", [(41, 21, 32), (64, 32, 48)])
+def test_scalers_train_like_the_oracle(gpu, r, r_attn, dim):
+    """DownScaler2D and UpScaler2D under autograd (resamplings forward and backward on this package's kernels, in
+    the planes and the channels-last layouts) against autograd through the oracle in float64."""
+    from spgt_amd.network import model as M
+    torch.manual_seed(37)
+    sizes = M.get_resolution_size(r, r_attn)
+    for kind in ("down", "up"):
+        if kind == "down":
+            mod = M.DownScaler2D(sizes, 1, dim, 0.0, "relu")
+            x = rnd(2, r, r, 1, seed=81)
+            fn = O.down_scaler
+            G = rnd(2, r_attn, r_attn, dim, seed=82)
+        else:
+            mod = M.UpScaler2D(sizes, dim, dim, 0.0, "silu")
+            x = rnd(2, r_attn, r_attn, dim, seed=83)
+            fn = O.up_scaler
+            G = rnd(2, r, r, dim, seed=84)
+        po = {k: v.detach().double().clone().requires_grad_(True) for k, v in mod.state_dict().items()}
+        xo = x.double().requires_grad_(True)
+        want = fn(po, xo, sizes, "relu" if kind == "down" else "silu")
+        want.backward(G.double())
+        mod = mod.to(gpu)
+        xg = x.to(gpu).requires_grad_(True)
+        got = mod(xg)
+        got.backward(G.to(gpu))
+        assert max_rel(got.detach().cpu().double(), want.detach()) < TOL, kind
+        assert max_rel(xg.grad.cpu().double(), xo.grad) < TOL, kind
+        for name, prm in mod.named_parameters():
+            assert max_rel(prm.grad.cpu().double(), po[name].grad) < TOL, (kind, name)
+
+
 @pytest.mark.parametrize("in_f,hid,out_f", [(32, 128, 1), (128, 256, 128), (36, 40, 3)])
 def test_feed_forward_trains_like_the_oracle(gpu, in_f, hid, out_f):
     """FeedForward under autograd, including a head with one output feature (weight gradient with the roles of

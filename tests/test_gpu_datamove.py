@@ -177,6 +177,57 @@ def test_bilinear_vs_oracle(gpu, shape, size):
     assert max_rel(got.cpu(), lib) < 1e-4
 
 
+@pytest.mark.parametrize("shape,size", [((2, 4, 7, 9), (7, 9)), ((2, 4, 7, 9), (4, 5)), ((2, 4, 7, 9), (13, 17)),
+                                        ((1, 4, 5, 5), (1, 1)), ((1, 8, 1, 1), (3, 4)), ((2, 128, 71, 71), (122, 122)),
+                                        ((2, 128, 122, 122), (71, 71)), ((1, 4, 2, 300), (5, 301)),
+                                        ((1, 4, 40, 33), (9, 7)), ((1, 12, 9, 7), (40, 33)), ((3, 5, 17, 12), (25, 30))])
+def test_bilinear_adjoint_vs_oracle(gpu, shape, size):
+    """The resampling's backward (both layouts, and the three autograd functions built on it) against autograd
+    through the oracle's restatement in float64; up- and down-sampling, by more than two (sources no output reads),
+    single rows and single outputs.  The source coordinates are formed in float32 as in the forward, which
+    bounds the agreement with float64 at a few 1e-6 relative to the largest value."""
+    x = rnd(*shape, seed=16)
+    g = rnd(*shape[:2], *size, seed=17)
+    xo = x.double().requires_grad_(True)
+    O.bilinear_align_corners(xo, size).backward(g.double())
+    want = xo.grad
+    got = dm.bilinear_adjoint(g.to(gpu), shape[-2:])
+    assert got.shape == want.shape
+    assert max_rel(got.cpu().double(), want) < 5e-5
+    xg = x.to(gpu).requires_grad_(True)
+    dm.bilinear_train(xg, size).backward(g.to(gpu))
+    assert max_rel(xg.grad.cpu().double(), want) < 5e-5
+    if shape[1] % 4 == 0:
+        got = dm.bilinear_adjoint(g.permute(0, 2, 3, 1).contiguous().to(gpu), shape[-2:], nhwc=True)
+        assert max_rel(got.permute(0, 3, 1, 2).cpu().double(), want) < 5e-5
+        xg = x.to(gpu).requires_grad_(True)
+        y = dm.bilinear_to_nhwc_train(xg, size)
+        assert max_rel(y.detach().permute(0, 3, 1, 2).cpu().double(), O.bilinear_align_corners(x.double(), size)) < 5e-5
+        y.backward(g.permute(0, 2, 3, 1).to(gpu))
+        assert max_rel(xg.grad.cpu().double(), want) < 5e-5
+        xg = x.permute(0, 2, 3, 1).contiguous().to(gpu).requires_grad_(True)
+        y = dm.bilinear_nhwc_train(xg, size)
+        assert max_rel(y.detach().permute(0, 3, 1, 2).cpu().double(), O.bilinear_align_corners(x.double(), size)) < 5e-5
+        y.backward(g.permute(0, 2, 3, 1).contiguous().to(gpu))
+        assert max_rel(xg.grad.permute(0, 3, 1, 2).cpu().double(), want) < 5e-5
+
+
+@pytest.mark.parametrize("hw,size", [((257, 257), (363, 363)), ((363, 363), (512, 512)), ((512, 512), (363, 363)),
+                                      ((363, 363), (257, 257))])
+def test_bilinear_adjoint_inner_product_at_the_model_sizes(gpu, hw, size):
+    """<A x, g> = <x, A^T g> for the four resamplings of the r = 512 model with 128 channels, both layouts; the
+    column sums of A^T g also equal those of g (the weights of an output sum to one)."""
+    torch.manual_seed(5)
+    x = torch.randn(2, 128, *hw, device=gpu)
+    g = torch.randn(2, 128, *size, device=gpu)
+    lhs = (dm.bilinear_align_corners(x, size).double() * g.double()).sum().item()
+    a = dm.bilinear_adjoint(g, hw)
+    assert abs((x.double() * a.double()).sum().item() - lhs) < 1e-6 * x.numel() ** 0.5 * 10
+    assert max_rel(a.double().sum((2, 3)).cpu(), g.double().sum((2, 3)).cpu()) < 1e-6
+    b = dm.bilinear_adjoint(g.permute(0, 2, 3, 1).contiguous(), hw, nhwc=True)
+    assert max_rel(b.permute(0, 3, 1, 2).cpu(), a.cpu()) < 1e-6
+
+
 def test_bilinear_closed_forms(gpu):
     x = rnd(2, 3, 7, 9, seed=15).to(gpu)
     assert torch.equal(dm.bilinear_align_corners(x, (7, 9)), x)  # identity when sizes agree
