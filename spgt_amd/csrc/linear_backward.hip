@@ -113,6 +113,140 @@ __global__ __launch_bounds__(256, 2) void xtg_partial_k(const float* __restrict_
     }
 }
 
+// The same partial sums for 128 x 128 blocks of dW with 16-byte loads: a wave takes every fourth pair of the
+// chunk's tokens and holds the whole block, 16 accumulators of 32 x 32.  Lane (i = lane % 32, h = lane / 32) loads
+// x[t + h][k0 + 4 i .. 4 i + 3] and g[t + h][n0 + 4 i .. 4 i + 3]; register a of the x piece against register b of
+// the g piece is one MFMA 32x32x2 whose row index i stands for feature k0 + 4 i + a and whose column index j for
+// n0 + 4 j + b, so the features never have to be rearranged: two load instructions feed 16 MFMAs (the kernel
+// above issues five loads for four).  The four waves' blocks are summed through LDS in a fixed order.
+// grid (nchunk, batch * nstrip, K / 128), block 256, one workgroup per compute unit (512 registers per lane).
+// Requires K and N multiples of 128, ldx and ldg multiples of 4, 16-byte aligned x and g.
+__global__ __launch_bounds__(256, 1) void xtg_partial_wide_k(const float* __restrict__ X, int64_t ldx, int64_t x_batch,
+                                                             const float* __restrict__ G, int64_t ldg,
+                                                             int64_t g_batch, float* __restrict__ partial, int64_t T,
+                                                             int K, int N, int tokens_per_chunk, int nstrip) {
+    constexpr int D = 4;  // steps of operands in flight ahead of the MFMAs
+    __shared__ float4 tile[16 * 4 * 64];  // [a][b][r / 4][lane]: one wave's block, 64 KB
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int tk = lane & 31;
+    const int kh = lane >> 5;
+    const int chunk = blockIdx.x;
+    const int nchunk = gridDim.x;
+    const int b = blockIdx.y / nstrip;
+    const int strip = blockIdx.y - b * nstrip;
+    const int k0 = blockIdx.z * 128;
+    const int n0 = strip * 128;
+    const int E = K * N + N;
+    const int64_t t0 = (int64_t)chunk * tokens_per_chunk;
+    const int64_t t1 = min(T, t0 + tokens_per_chunk);
+    const int last = (int)(t1 - t0) - 1;
+    const int pairs = (last + 2) / 2;            // token pairs of the chunk
+    const int steps = (pairs - wave + 3) / 4;    // pairs wave, wave + 4, ... of them
+    const float* xp = X + b * x_batch + t0 * ldx + k0 + 4 * tk;
+    const float* gp = G + b * g_batch + t0 * ldg + n0 + 4 * tk;
+    v16f acc[4][4];
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[a][c][r] = 0.f;
+    float colsum[4] = {0.f, 0.f, 0.f, 0.f};
+    float4 xq[D], gq[D];
+    auto issue = [&](int slot, int s) {
+        const int64_t tr = min(2 * (4 * s + wave) + kh, last);  // past the end: a valid row, masked when used
+        xq[slot] = *reinterpret_cast<const float4*>(xp + tr * ldx);
+        gq[slot] = *reinterpret_cast<const float4*>(gp + tr * ldg);
+    };
+    auto use = [&](int slot, int s) {
+        const bool ok = 2 * (4 * s + wave) + kh <= last;
+        const float xr[4] = {ok ? xq[slot].x : 0.f, ok ? xq[slot].y : 0.f, ok ? xq[slot].z : 0.f, ok ? xq[slot].w : 0.f};
+        const float gr[4] = {ok ? gq[slot].x : 0.f, ok ? gq[slot].y : 0.f, ok ? gq[slot].z : 0.f, ok ? gq[slot].w : 0.f};
+#pragma unroll
+        for (int a = 0; a < 4; ++a)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) acc[a][c] = mfma32(xr[a], gr[c], acc[a][c]);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) colsum[c] += gr[c];
+    };
+    if (last >= 0) {
+#pragma unroll
+        for (int d = 0; d < D; ++d) {
+            issue(d, d);  // in the loop's own order, so that the loop waits for the oldest step only
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        for (int s = 0; s < steps; s += D) {
+#pragma unroll
+            for (int d = 0; d < D; ++d) {
+                use(d, s + d);  // a step past the wave's last contributes zeros
+                __builtin_amdgcn_sched_barrier(0);
+                issue(d, s + d + D);  // stays D - 1 steps of MFMAs ahead of its use
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    }
+    float* out = partial + ((int64_t)b * nchunk + chunk) * E;
+    // bias gradient: the two token halves of a column meet, then the four waves in a fixed order
+    float* colsm = reinterpret_cast<float*>(tile);  // [4][128], before the blocks need the space
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        const float cs = colsum[c] + __shfl_xor(colsum[c], 32, 64);
+        if (kh == 0) colsm[wave * 128 + 4 * tk + c] = cs;
+    }
+    __syncthreads();
+    if (wave == 1 && k0 == 0) {
+        for (int n = lane; n < 128; n += 64)
+            out[(int64_t)K * N + n0 + n] = (colsm[n] + colsm[128 + n]) + (colsm[256 + n] + colsm[384 + n]);
+    }
+    __syncthreads();
+    // the waves' blocks: wave 3 -> LDS, wave 2 adds and writes, wave 1 adds and writes, wave 0 adds and stores
+#pragma unroll 1
+    for (int turn = 3; turn >= 0; --turn) {
+        if (wave == turn) {
+            if (turn < 3) {
+#pragma unroll
+                for (int a = 0; a < 4; ++a) {
+                    float4 v[16];  // a row group's sixteen pieces are requested before the first is used
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) v[i] = tile[(a * 16 + i) * 64 + lane];
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int c = 0; c < 4; ++c)
+#pragma unroll
+                        for (int r4 = 0; r4 < 4; ++r4) {
+                            const float4 w = v[c * 4 + r4];
+                            acc[a][c][4 * r4] += w.x, acc[a][c][4 * r4 + 1] += w.y;
+                            acc[a][c][4 * r4 + 2] += w.z, acc[a][c][4 * r4 + 3] += w.w;
+                        }
+                }
+            }
+            if (turn > 0) {
+#pragma unroll
+                for (int a = 0; a < 4; ++a)
+#pragma unroll
+                    for (int c = 0; c < 4; ++c)
+#pragma unroll
+                        for (int r4 = 0; r4 < 4; ++r4)
+                            tile[((a * 4 + c) * 4 + r4) * 64 + lane] = make_float4(
+                                acc[a][c][4 * r4], acc[a][c][4 * r4 + 1], acc[a][c][4 * r4 + 2], acc[a][c][4 * r4 + 3]);
+            }
+        }
+        if (turn > 0) __syncthreads();
+    }
+    if (wave == 0) {
+        // acc[a][c][r] = dW[k0 + 4 (8 (r / 4) + 4 kh + r % 4) + a][n0 + 4 tk + c]
+#pragma unroll
+        for (int a = 0; a < 4; ++a)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int k = k0 + 4 * (8 * (r >> 2) + 4 * kh + (r & 3)) + a;
+                *reinterpret_cast<float4*>(out + (int64_t)k * N + n0 + 4 * tk) =
+                    make_float4(acc[a][0][r], acc[a][1][r], acc[a][2][r], acc[a][3][r]);
+            }
+    }
+}
+
 }  // namespace spgt
 
 using namespace spgt;
@@ -121,15 +255,21 @@ namespace {
 
 struct WgradPlan {
     int nt, nstrip, kz, tpc, nchunk;
+    bool wide;
 };
 
+// The plan depends on the sizes only (the workspace query has nothing else): the wide kernel serves K and N
+// multiples of 128 and is chosen then; a call whose strides or alignment do not fit it runs the kernel above on
+// the same chunks.
 WgradPlan wgrad_plan(int64_t T, int K, int N, int batch) {
     WgradPlan p;
+    p.wide = K % 128 == 0 && N % 128 == 0;
     p.nt = N >= 128 ? 4 : (N > 32 ? 2 : 1);
     p.nstrip = ceil_div(N, p.nt * 32);
     p.kz = ceil_div(K, 128);
-    // about two workgroups per compute unit, at most as many chunks as tile_reduce sums, at least 64 tokens each
-    const int per = std::max(1, 2 * device_cu_count() / std::max(1, batch * p.nstrip * p.kz));
+    // about two workgroups per compute unit (one for the wide kernel, whose waves hold 512 registers), at most
+    // as many chunks as tile_reduce sums, at least 64 tokens each
+    const int per = std::max(1, (p.wide ? 1 : 2) * device_cu_count() / std::max(1, batch * p.nstrip * p.kz));
     int64_t nchunk = std::min<int64_t>(std::min(per, kReduceChains * kReduceMaxPerChain), std::max<int64_t>(1, T / 64));
     int64_t tpc = ceil_div(ceil_div(T, nchunk), (int64_t)16) * 16;
     p.tpc = (int)tpc;
@@ -172,7 +312,12 @@ extern "C" int spgt_linear_weight_grad(const float* x, int64_t ldx, int64_t x_ba
 #define SPGT_XTG(NT)                                                                                               \
     hipLaunchKernelGGL((xtg_partial_k<NT>), grid, dim3(256), 0, stream, x, ldx, x_batch_stride, grad, ldg,         \
                        grad_batch_stride, partial, tokens, in_features, out_features, p.tpc, p.nstrip)
-    if (p.nt == 4) SPGT_XTG(4);
+    const bool wide_ok = p.wide && ldx % 4 == 0 && ldg % 4 == 0 && x_batch_stride % 4 == 0 &&
+                         grad_batch_stride % 4 == 0 && aligned16(x) && aligned16(grad);
+    if (wide_ok)
+        hipLaunchKernelGGL(xtg_partial_wide_k, grid, dim3(256), 0, stream, x, ldx, x_batch_stride, grad, ldg,
+                           grad_batch_stride, partial, tokens, in_features, out_features, p.tpc, p.nstrip);
+    else if (p.nt == 4) SPGT_XTG(4);
     else if (p.nt == 2) SPGT_XTG(2);
     else SPGT_XTG(1);
 #undef SPGT_XTG
