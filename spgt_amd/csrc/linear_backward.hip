@@ -119,8 +119,9 @@ __global__ __launch_bounds__(256, 2) void xtg_partial_k(const float* __restrict_
 // the g piece is one MFMA 32x32x2 whose row index i stands for feature k0 + 4 i + a and whose column index j for
 // n0 + 4 j + b, so the features never have to be rearranged: two load instructions feed 16 MFMAs (the kernel
 // above issues five loads for four).  The four waves' blocks are summed through LDS in a fixed order.
-// grid (nchunk, batch * nstrip, K / 128), block 256, one workgroup per compute unit (512 registers per lane).
-// Requires K and N multiples of 128, ldx and ldg multiples of 4, 16-byte aligned x and g.
+// grid (nchunk, batch * nstrip, ceil(K / 128)), block 256, one workgroup per compute unit (512 registers per lane).
+// Requires N a multiple of 128, K a multiple of 4 and at least 128 (the rows of the last block past K are read from
+// the row's last piece, used as zeros and not stored), ldx and ldg multiples of 4, 16-byte aligned x and g.
 __global__ __launch_bounds__(256, 1) void xtg_partial_wide_k(const float* __restrict__ X, int64_t ldx, int64_t x_batch,
                                                              const float* __restrict__ G, int64_t ldg,
                                                              int64_t g_batch, float* __restrict__ partial, int64_t T,
@@ -143,7 +144,8 @@ __global__ __launch_bounds__(256, 1) void xtg_partial_wide_k(const float* __rest
     const int last = (int)(t1 - t0) - 1;
     const int pairs = (last + 2) / 2;            // token pairs of the chunk
     const int steps = (pairs - wave + 3) / 4;    // pairs wave, wave + 4, ... of them
-    const float* xp = X + b * x_batch + t0 * ldx + k0 + 4 * tk;
+    const bool kok = k0 + 4 * tk < K;  // K is a multiple of 4: a piece lies inside the row or past it
+    const float* xp = X + b * x_batch + t0 * ldx + min(k0 + 4 * tk, K - 4);
     const float* gp = G + b * g_batch + t0 * ldg + n0 + 4 * tk;
     v16f acc[4][4];
 #pragma unroll
@@ -161,7 +163,9 @@ __global__ __launch_bounds__(256, 1) void xtg_partial_wide_k(const float* __rest
     };
     auto use = [&](int slot, int s) {
         const bool ok = 2 * (4 * s + wave) + kh <= last;
-        const float xr[4] = {ok ? xq[slot].x : 0.f, ok ? xq[slot].y : 0.f, ok ? xq[slot].z : 0.f, ok ? xq[slot].w : 0.f};
+        const bool xok = ok && kok;
+        const float xr[4] = {xok ? xq[slot].x : 0.f, xok ? xq[slot].y : 0.f, xok ? xq[slot].z : 0.f,
+                             xok ? xq[slot].w : 0.f};
         const float gr[4] = {ok ? gq[slot].x : 0.f, ok ? gq[slot].y : 0.f, ok ? gq[slot].z : 0.f, ok ? gq[slot].w : 0.f};
 #pragma unroll
         for (int a = 0; a < 4; ++a)
@@ -241,8 +245,9 @@ __global__ __launch_bounds__(256, 1) void xtg_partial_wide_k(const float* __rest
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int k = k0 + 4 * (8 * (r >> 2) + 4 * kh + (r & 3)) + a;
-                *reinterpret_cast<float4*>(out + (int64_t)k * N + n0 + 4 * tk) =
-                    make_float4(acc[a][0][r], acc[a][1][r], acc[a][2][r], acc[a][3][r]);
+                if (k < K)
+                    *reinterpret_cast<float4*>(out + (int64_t)k * N + n0 + 4 * tk) =
+                        make_float4(acc[a][0][r], acc[a][1][r], acc[a][2][r], acc[a][3][r]);
             }
     }
 }
@@ -258,12 +263,12 @@ struct WgradPlan {
     bool wide;
 };
 
-// The plan depends on the sizes only (the workspace query has nothing else): the wide kernel serves K and N
-// multiples of 128 and is chosen then; a call whose strides or alignment do not fit it runs the kernel above on
-// the same chunks.
+// The plan depends on the sizes only (the workspace query has nothing else): the wide kernel serves N a multiple
+// of 128 with K a multiple of 4 from 128 up and is chosen then; a call whose strides or alignment do not fit it
+// runs the kernel above on the same chunks.
 WgradPlan wgrad_plan(int64_t T, int K, int N, int batch) {
     WgradPlan p;
-    p.wide = K % 128 == 0 && N % 128 == 0;
+    p.wide = K % 4 == 0 && K >= 128 && N % 128 == 0;
     p.nt = N >= 128 ? 4 : (N > 32 ? 2 : 1);
     p.nstrip = ceil_div(N, p.nt * 32);
     p.kz = ceil_div(K, 128);
