@@ -546,6 +546,11 @@ def kernel_rooflines(dev, use_graph=True):
         low64, grid2, wg = rn(4, 122, 122, 64), rn(4, 211, 211, 2), rn(2, 64)
         return lambda: dm.bilinear_nhwc_affine(low64, (211, 211), grid2, wg)
     hbm("bilinear_122_to_211_nhwc_plus_grid_columns", 4 * 4 * (64 * (211 * 211 + 122 * 122) + 2 * 211 * 211), make_affine)
+    # the resampling's backward (a gather per source position), planes and channels-last
+    hbm("bilinear_adjoint_122_to_211_planes", bil(211, 122),
+        resample((4, 128, 122, 122), lambda t: dm.bilinear_adjoint(t, (211, 211))))
+    hbm("bilinear_adjoint_211_to_122_nhwc", bil(122, 211),
+        resample((4, 211, 211, 128), lambda t: dm.bilinear_adjoint(t, (122, 122), nhwc=True)))
     hbm("bias_silu2_nchw_to_nhwc_122", 2 * 4 * 128 * 122 * 122 * 4,
         resample((4, 128, 122, 122), lambda t: dm.bilinear_resample(t, (122, 122), dst_nhwc=True, pre_bias=cb,
                                                                      pre_activation="silu", pre_count=2)))
