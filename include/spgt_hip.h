@@ -484,6 +484,30 @@ int spgt_encoder_tail_folded_forward(const float* q, int64_t ld_q, const float* 
                                      float* out, int B, int64_t S, int dp, int dim_hidden, int ffn_hidden,
                                      spgt_stream_t stream);
 
+/* The same two launches with the reference's dropouts applied inside them: Sp_GalerkinAttention drops the output
+ * of fc_layer (network/sp_layer.py:76) and FeedForward its own output (network/layer.py:173), both with
+ * F.dropout's default training=True, i.e. also in inference, before the residual is added.
+ *   y1 = x + dropout(fc output, fc_droprate)      out = y1 + dropout(ffn output, ffn_droprate)
+ * The keep decision of an element is a hash of (seed, site, token, column); kept values are scaled by
+ * 1 / (1 - rate).  seed points to two 32-bit words in device memory (8-byte aligned): read by the kernel, so a
+ * captured graph that refills them with a generator kernel draws new masks on every replay.  Rates in [0, 1);
+ * with both 0 the calls are spgt_encoder_tail_forward / spgt_encoder_tail_folded_forward and seed may be null.
+ * The masks are this library's own: they follow the reference's distribution, not torch's random stream. */
+int spgt_encoder_tail_forward_dropout(const float* attn_out, int64_t ld_attn, const float* x,
+                                      const float* fc_weight_kn, const float* fc_bias,
+                                      const float* ffn1_weight_kn, const float* ffn1_bias,
+                                      const float* ffn2_weight_kn, const float* ffn2_bias, int activation,
+                                      float* out, int64_t tokens, int attn_features, int dim_hidden, int ffn_hidden,
+                                      const uint32_t* seed, float fc_droprate, float ffn_droprate,
+                                      spgt_stream_t stream);
+int spgt_encoder_tail_folded_forward_dropout(const float* q, int64_t ld_q, const float* position, const float* x,
+                                             const float* folded_fc, const float* folded_pos, const float* fc_bias,
+                                             const float* ffn1_weight_kn, const float* ffn1_bias,
+                                             const float* ffn2_weight_kn, const float* ffn2_bias, int activation,
+                                             float* out, int B, int64_t S, int dp, int dim_hidden, int ffn_hidden,
+                                             const uint32_t* seed, float fc_droprate, float ffn_droprate,
+                                             spgt_stream_t stream);
+
 /* One strided copy: dst[i0*dst_stride[0] + i1*dst_stride[1] + i2*dst_stride[2]] =
  * src[i0*src_stride[0] + i1*src_stride[1] + i2*src_stride[2]] for i_k < size[k]; 32-bit words, strides in words. */
 typedef struct {

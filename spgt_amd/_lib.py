@@ -76,11 +76,15 @@ SIGNATURES = {
     "spgt_ffn_scalar_forward": (_i, [_p, _i64, _p, _p, _p, _p, _i, _p, _i64, _i, _i, _p]),
     "spgt_encoder_tail_supported": (_i, [_i, _i, _i]),
     "spgt_encoder_tail_forward": (_i, [_p, _i64, _p, _p, _p, _p, _p, _p, _p, _i, _p, _i64, _i, _i, _i, _p]),
+    "spgt_encoder_tail_forward_dropout": (
+        _i, [_p, _i64, _p, _p, _p, _p, _p, _p, _p, _i, _p, _i64, _i, _i, _i, _p, _f, _f, _p]),
     "spgt_galerkin_attention_ktv_forward": (
         _i, [_p, _p, _i64, _p, _p, _p, _p, _p, _f, _p, _p, _sz, _i, _i, _i, _i, _p]),
     "spgt_fold_ktv_into_fc": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _p]),
     "spgt_encoder_tail_folded_forward": (
         _i, [_p, _i64, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _p, _i, _i64, _i, _i, _i, _p]),
+    "spgt_encoder_tail_folded_forward_dropout": (
+        _i, [_p, _i64, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _p, _i, _i64, _i, _i, _i, _p, _f, _f, _p]),
     "spgt_strided_copy_batch": (_i, [_p, _i, _p]),
     "spgt_linear_weight_grad_workspace_bytes": (_sz, [_i64, _i, _i, _i]),
     "spgt_linear_weight_grad": (_i, [_p, _i64, _i64, _p, _i64, _i64, _p, _p, _sz, _i64, _i, _i, _i, _p]),

@@ -669,12 +669,43 @@ __device__ __forceinline__ void mfma_acc_done(v16f& acc) { asm volatile("s_nop 1
 // [B][2][128], meet the token's position pos [T][2] as a rank-2 update of y1 (no Wpos: no position columns).
 // Tiles then never straddle two of the B sequences of S tokens, a workgroup takes consecutive tiles (so that
 // the sequence, and with it the resident fc weights, changes at most a few times), and T = B * S.
-template <int K1, bool FOLD>
+// DROP: the reference's two dropouts of an encoder layer (always on, also in inference: F.dropout's default,
+// network/sp_layer.py:76 and network/layer.py:173) applied where their operands are formed,
+//   y1 = x + dropout(a @ Wfc + bfc, p_fc)        out = y1 + dropout(act(..) @ W2 + b2, p_ffn)
+// with the keep decision of element (token t, column n) a hash of (seed, site, t, n): an integer mixer of the
+// token's base value plus a per-column constant, compared with p * 2^32.  The seed is read from device memory, so
+// that a captured graph whose seed tensor is refilled by a generator kernel draws new masks on every replay.
+__device__ __forceinline__ uint32_t dropout_mix(uint32_t h) {
+    h ^= h >> 16;
+    h *= 0x21f0aaadu;
+    h ^= h >> 15;
+    h *= 0x735a2d97u;
+    h ^= h >> 15;
+    return h;
+}
+struct DropoutSite {
+    uint32_t base, threshold;
+    float scale;
+};
+__device__ __forceinline__ DropoutSite dropout_site(const uint32_t* seed, uint32_t site, int64_t t, float p) {
+    DropoutSite d;
+    const uint32_t lo = (uint32_t)t, hi = (uint32_t)((uint64_t)t >> 32);
+    d.base = dropout_mix(dropout_mix(seed[0] ^ (lo * 0x9e3779b1u)) ^ seed[1] ^ (hi * 0x85ebca77u) ^ (site * 0xc2b2ae3du));
+    d.threshold = p <= 0.f ? 0u : (uint32_t)fminf(p * 4294967296.0f, 4294967040.0f);
+    d.scale = p <= 0.f ? 1.f : 1.f / (1.f - p);
+    return d;
+}
+__device__ __forceinline__ float dropout_apply(const DropoutSite& d, int n, float v) {
+    return dropout_mix(d.base + (uint32_t)n * 0x27d4eb2fu) >= d.threshold ? v * d.scale : 0.f;
+}
+
+template <int K1, bool FOLD, bool DROP>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void encoder_tail_k(
     const float* __restrict__ a, int64_t lda, const float* __restrict__ x, const float* __restrict__ Wfc,
     const float* __restrict__ bfc, const float* __restrict__ W1, const float* __restrict__ b1,
     const float* __restrict__ W2, const float* __restrict__ b2, int act, float* __restrict__ out, int64_t T,
-    const float* __restrict__ Wpos, const float* __restrict__ pos, int64_t S) {
+    const float* __restrict__ Wpos, const float* __restrict__ pos, int64_t S, const uint32_t* __restrict__ seed,
+    float p_fc, float p_ffn) {
     static_assert(!FOLD || K1 == 128, "the folded form reads the projected Q");
     constexpr int D = 128, F = 256, TT = 32;
     constexpr int PA = K1 + 4, PY = D + 4, PH = F + 4;
@@ -781,6 +812,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         const int64_t t = tile_t0(tile) + tk;
         const bool tok = t < tile_end(tile);
         const bool more = tile + step < limit;
+        DropoutSite site_fc, site_ffn;
+        if (DROP) {
+            site_fc = dropout_site(seed, 0u, t, p_fc);
+            site_ffn = dropout_site(seed, 1u, t, p_ffn);
+        }
         if (FOLD && tile_seq(tile) != cur_b) {
             // another sequence: its fc weights into the registers, its position rows into LDS (last read before
             // the barrier that ended the previous tile)
@@ -819,15 +855,30 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
             for (int q = 0; q < 4; ++q) {
                 const float4 bq = *reinterpret_cast<const float4*>(bias_s + n0 + 4 * kh + 8 * q);
                 float4 y;
-                y.x = (acc[0][4 * q + 0] + acc[1][4 * q + 0]) + bq.x + xq[q].x;
-                y.y = (acc[0][4 * q + 1] + acc[1][4 * q + 1]) + bq.y + xq[q].y;
-                y.z = (acc[0][4 * q + 2] + acc[1][4 * q + 2]) + bq.z + xq[q].z;
-                y.w = (acc[0][4 * q + 3] + acc[1][4 * q + 3]) + bq.w + xq[q].w;
+                if (!DROP) {
+                    y.x = (acc[0][4 * q + 0] + acc[1][4 * q + 0]) + bq.x + xq[q].x;
+                    y.y = (acc[0][4 * q + 1] + acc[1][4 * q + 1]) + bq.y + xq[q].y;
+                    y.z = (acc[0][4 * q + 2] + acc[1][4 * q + 2]) + bq.z + xq[q].z;
+                    y.w = (acc[0][4 * q + 3] + acc[1][4 * q + 3]) + bq.w + xq[q].w;
+                } else {
+                    y.x = (acc[0][4 * q + 0] + acc[1][4 * q + 0]) + bq.x;
+                    y.y = (acc[0][4 * q + 1] + acc[1][4 * q + 1]) + bq.y;
+                    y.z = (acc[0][4 * q + 2] + acc[1][4 * q + 2]) + bq.z;
+                    y.w = (acc[0][4 * q + 3] + acc[1][4 * q + 3]) + bq.w;
+                }
                 if (FOLD && Wpos) {
                     const float4 w0 = *reinterpret_cast<const float4*>(posw_s + n0 + 4 * kh + 8 * q);
                     const float4 w1 = *reinterpret_cast<const float4*>(posw_s + D + n0 + 4 * kh + 8 * q);
                     y.x += pq.x * w0.x + pq.y * w1.x; y.y += pq.x * w0.y + pq.y * w1.y;
                     y.z += pq.x * w0.z + pq.y * w1.z; y.w += pq.x * w0.w + pq.y * w1.w;
+                }
+                if (DROP) {
+                    // the whole output of fc_layer (bias and position rows included) is what the reference drops
+                    const int n = n0 + 4 * kh + 8 * q;
+                    y.x = dropout_apply(site_fc, n + 0, y.x) + xq[q].x;
+                    y.y = dropout_apply(site_fc, n + 1, y.y) + xq[q].y;
+                    y.z = dropout_apply(site_fc, n + 2, y.z) + xq[q].z;
+                    y.w = dropout_apply(site_fc, n + 3, y.w) + xq[q].w;
                 }
                 *reinterpret_cast<float4*>(bufY + tk * PY + n0 + 8 * q + 4 * kh) = y;
             }
@@ -912,10 +963,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                     const float4 bq = *reinterpret_cast<const float4*>(bias_s + 384 + n0 + 4 * kh + 8 * q);
                     const float4 y1 = *reinterpret_cast<const float4*>(bufY + tk * PY + n0 + 8 * q + 4 * kh);
                     float4 o;
-                    o.x = (acc[0][4 * q + 0] + acc[1][4 * q + 0]) + bq.x + y1.x;
-                    o.y = (acc[0][4 * q + 1] + acc[1][4 * q + 1]) + bq.y + y1.y;
-                    o.z = (acc[0][4 * q + 2] + acc[1][4 * q + 2]) + bq.z + y1.z;
-                    o.w = (acc[0][4 * q + 3] + acc[1][4 * q + 3]) + bq.w + y1.w;
+                    if (!DROP) {
+                        o.x = (acc[0][4 * q + 0] + acc[1][4 * q + 0]) + bq.x + y1.x;
+                        o.y = (acc[0][4 * q + 1] + acc[1][4 * q + 1]) + bq.y + y1.y;
+                        o.z = (acc[0][4 * q + 2] + acc[1][4 * q + 2]) + bq.z + y1.z;
+                        o.w = (acc[0][4 * q + 3] + acc[1][4 * q + 3]) + bq.w + y1.w;
+                    } else {
+                        const int n = n0 + 4 * kh + 8 * q;
+                        o.x = dropout_apply(site_ffn, n + 0, (acc[0][4 * q + 0] + acc[1][4 * q + 0]) + bq.x) + y1.x;
+                        o.y = dropout_apply(site_ffn, n + 1, (acc[0][4 * q + 1] + acc[1][4 * q + 1]) + bq.y) + y1.y;
+                        o.z = dropout_apply(site_ffn, n + 2, (acc[0][4 * q + 2] + acc[1][4 * q + 2]) + bq.z) + y1.z;
+                        o.w = dropout_apply(site_ffn, n + 3, (acc[0][4 * q + 3] + acc[1][4 * q + 3]) + bq.w) + y1.w;
+                    }
                     *reinterpret_cast<float4*>(out + t * D + n0 + 4 * kh + 8 * q) = o;
                 }
             }
@@ -1331,13 +1390,29 @@ extern "C" int spgt_ffn_scalar_forward(const float* x, int64_t ldx, const float*
     return check_launch("ffn_scalar_forward");
 }
 
-extern "C" int spgt_encoder_tail_folded_forward(const float* q, int64_t ld_q, const float* position, const float* x,
-                                                const float* folded_fc, const float* folded_pos,
-                                                const float* fc_bias, const float* ffn1_weight_kn,
-                                                const float* ffn1_bias, const float* ffn2_weight_kn,
-                                                const float* ffn2_bias, int activation, float* out, int B,
-                                                int64_t S, int dp, int dim_hidden, int ffn_hidden,
-                                                hipStream_t stream) {
+namespace {
+
+// One-time (per process) permission for a kernel to use more than 64 KB of dynamic LDS.
+template <class K>
+void allow_tail_lds(K kernel) {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+}
+
+int dropout_args_ok(const uint32_t* seed, float p_fc, float p_ffn) {
+    if (!(p_fc >= 0.f && p_fc < 1.f) || !(p_ffn >= 0.f && p_ffn < 1.f))
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "encoder_tail dropout: drop rates must lie in [0, 1)");
+    if ((p_fc > 0.f || p_ffn > 0.f) && (!seed || !aligned8(seed)))
+        return fail(SPGT_ERR_INVALID_ARGUMENT,
+                    "encoder_tail dropout: drop rates above 0 need an 8-byte aligned seed (two 32-bit words) in device memory");
+    return SPGT_OK;
+}
+
+int encoder_tail_folded_common(const float* q, int64_t ld_q, const float* position, const float* x,
+                               const float* folded_fc, const float* folded_pos, const float* fc_bias,
+                               const float* ffn1_weight_kn, const float* ffn1_bias, const float* ffn2_weight_kn,
+                               const float* ffn2_bias, int activation, float* out, int B, int64_t S, int dp,
+                               int dim_hidden, int ffn_hidden, const uint32_t* seed, float p_fc, float p_ffn,
+                               hipStream_t stream) {
     if (!q || !x || !folded_fc || !fc_bias || !ffn1_weight_kn || !ffn1_bias || !ffn2_weight_kn || !ffn2_bias || !out)
         return fail(SPGT_ERR_INVALID_ARGUMENT, "encoder_tail_folded_forward: null pointer argument");
     if ((dp != 0 && dp != 2) || (dp == 2 && (!position || !folded_pos)))
@@ -1360,25 +1435,58 @@ extern "C" int spgt_encoder_tail_folded_forward(const float* q, int64_t ld_q, co
     const int64_t per_wg = ceil_div(tiles, (int64_t)device_cu_count());
     const unsigned grid = (unsigned)ceil_div(tiles, per_wg);
     const size_t lds = std::max<size_t>(((size_t)32 * (128 + 4 + 132 + 260) + 512 + 256) * sizeof(float), 84 * 1024);
-    static const hipError_t opt = hipFuncSetAttribute(reinterpret_cast<const void*>(encoder_tail_k<128, true>),
-                                                      hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
-    (void)opt;
-    hipLaunchKernelGGL((encoder_tail_k<128, true>), dim3(grid), dim3(256), lds, stream, q, ld_q, x, folded_fc, fc_bias,
-                       ffn1_weight_kn, ffn1_bias, ffn2_weight_kn, ffn2_bias, activation, out, (int64_t)B * S,
-                       dp == 2 ? folded_pos : nullptr, position, S);
+    static const bool once = (allow_tail_lds(encoder_tail_k<128, true, false>), allow_tail_lds(encoder_tail_k<128, true, true>), true);
+    (void)once;
+    if (p_fc > 0.f || p_ffn > 0.f)
+        hipLaunchKernelGGL((encoder_tail_k<128, true, true>), dim3(grid), dim3(256), lds, stream, q, ld_q, x, folded_fc,
+                           fc_bias, ffn1_weight_kn, ffn1_bias, ffn2_weight_kn, ffn2_bias, activation, out, (int64_t)B * S,
+                           dp == 2 ? folded_pos : nullptr, position, S, seed, p_fc, p_ffn);
+    else
+        hipLaunchKernelGGL((encoder_tail_k<128, true, false>), dim3(grid), dim3(256), lds, stream, q, ld_q, x, folded_fc,
+                           fc_bias, ffn1_weight_kn, ffn1_bias, ffn2_weight_kn, ffn2_bias, activation, out, (int64_t)B * S,
+                           dp == 2 ? folded_pos : nullptr, position, S, nullptr, 0.f, 0.f);
     return check_launch("encoder_tail_folded_forward");
+}
+
+}  // namespace
+
+extern "C" int spgt_encoder_tail_folded_forward(const float* q, int64_t ld_q, const float* position, const float* x,
+                                                const float* folded_fc, const float* folded_pos,
+                                                const float* fc_bias, const float* ffn1_weight_kn,
+                                                const float* ffn1_bias, const float* ffn2_weight_kn,
+                                                const float* ffn2_bias, int activation, float* out, int B,
+                                                int64_t S, int dp, int dim_hidden, int ffn_hidden,
+                                                hipStream_t stream) {
+    return encoder_tail_folded_common(q, ld_q, position, x, folded_fc, folded_pos, fc_bias, ffn1_weight_kn, ffn1_bias,
+                                      ffn2_weight_kn, ffn2_bias, activation, out, B, S, dp, dim_hidden, ffn_hidden,
+                                      nullptr, 0.f, 0.f, stream);
+}
+
+extern "C" int spgt_encoder_tail_folded_forward_dropout(const float* q, int64_t ld_q, const float* position,
+                                                        const float* x, const float* folded_fc, const float* folded_pos,
+                                                        const float* fc_bias, const float* ffn1_weight_kn,
+                                                        const float* ffn1_bias, const float* ffn2_weight_kn,
+                                                        const float* ffn2_bias, int activation, float* out, int B,
+                                                        int64_t S, int dp, int dim_hidden, int ffn_hidden,
+                                                        const uint32_t* seed, float fc_droprate, float ffn_droprate,
+                                                        hipStream_t stream) {
+    if (int rc = dropout_args_ok(seed, fc_droprate, ffn_droprate)) return rc;
+    return encoder_tail_folded_common(q, ld_q, position, x, folded_fc, folded_pos, fc_bias, ffn1_weight_kn, ffn1_bias,
+                                      ffn2_weight_kn, ffn2_bias, activation, out, B, S, dp, dim_hidden, ffn_hidden, seed,
+                                      fc_droprate, ffn_droprate, stream);
 }
 
 extern "C" int spgt_encoder_tail_supported(int attn_features, int dim_hidden, int ffn_hidden) {
     return ((attn_features == 128 || attn_features == 136) && dim_hidden == 128 && ffn_hidden == 256) ? 1 : 0;
 }
 
-extern "C" int spgt_encoder_tail_forward(const float* attn_out, int64_t ld_attn, const float* x,
-                                         const float* fc_weight_kn, const float* fc_bias,
-                                         const float* ffn1_weight_kn, const float* ffn1_bias,
-                                         const float* ffn2_weight_kn, const float* ffn2_bias, int activation,
-                                         float* out, int64_t tokens, int attn_features, int dim_hidden,
-                                         int ffn_hidden, hipStream_t stream) {
+namespace {
+
+int encoder_tail_common(const float* attn_out, int64_t ld_attn, const float* x, const float* fc_weight_kn,
+                        const float* fc_bias, const float* ffn1_weight_kn, const float* ffn1_bias,
+                        const float* ffn2_weight_kn, const float* ffn2_bias, int activation, float* out, int64_t tokens,
+                        int attn_features, int dim_hidden, int ffn_hidden, const uint32_t* seed, float p_fc,
+                        float p_ffn, hipStream_t stream) {
     if (!attn_out || !x || !fc_weight_kn || !fc_bias || !ffn1_weight_kn || !ffn1_bias || !ffn2_weight_kn ||
         !ffn2_bias || !out)
         return fail(SPGT_ERR_INVALID_ARGUMENT, "encoder_tail_forward: null pointer argument");
@@ -1402,19 +1510,45 @@ extern "C" int spgt_encoder_tail_forward(const float* attn_out, int64_t ld_attn,
     // attention tile + y1 + hidden tile + biases; at least half of the CU's LDS (one workgroup per CU anyway:
     // a wave uses most of its SIMD's registers)
     const size_t lds = std::max<size_t>(((size_t)32 * ((size_t)attn_features + 4 + 132 + 260) + 512 + 256) * sizeof(float), 84 * 1024);
-    static const hipError_t opt136 = hipFuncSetAttribute(reinterpret_cast<const void*>(encoder_tail_k<136, false>),
-                                                         hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
-    static const hipError_t opt128 = hipFuncSetAttribute(reinterpret_cast<const void*>(encoder_tail_k<128, false>),
-                                                         hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
-    (void)opt136;
-    (void)opt128;
-    if (attn_features == 136)
-        hipLaunchKernelGGL((encoder_tail_k<136, false>), dim3(grid), dim3(256), lds, stream, attn_out, ld_attn, x,
-                           fc_weight_kn, fc_bias, ffn1_weight_kn, ffn1_bias, ffn2_weight_kn, ffn2_bias, activation, out,
-                           tokens, nullptr, nullptr, (int64_t)0);
-    else
-        hipLaunchKernelGGL((encoder_tail_k<128, false>), dim3(grid), dim3(256), lds, stream, attn_out, ld_attn, x,
-                           fc_weight_kn, fc_bias, ffn1_weight_kn, ffn1_bias, ffn2_weight_kn, ffn2_bias, activation, out,
-                           tokens, nullptr, nullptr, (int64_t)0);
+    static const bool once = (allow_tail_lds(encoder_tail_k<136, false, false>), allow_tail_lds(encoder_tail_k<128, false, false>),
+                              allow_tail_lds(encoder_tail_k<136, false, true>), allow_tail_lds(encoder_tail_k<128, false, true>), true);
+    (void)once;
+    const bool drop = p_fc > 0.f || p_ffn > 0.f;
+#define SPGT_TAIL(K1, DROPF)                                                                                          \
+    hipLaunchKernelGGL((encoder_tail_k<K1, false, DROPF>), dim3(grid), dim3(256), lds, stream, attn_out, ld_attn, x,   \
+                       fc_weight_kn, fc_bias, ffn1_weight_kn, ffn1_bias, ffn2_weight_kn, ffn2_bias, activation, out,   \
+                       tokens, nullptr, nullptr, (int64_t)0, drop ? seed : nullptr, p_fc, p_ffn)
+    if (attn_features == 136) {
+        if (drop) SPGT_TAIL(136, true); else SPGT_TAIL(136, false);
+    } else {
+        if (drop) SPGT_TAIL(128, true); else SPGT_TAIL(128, false);
+    }
+#undef SPGT_TAIL
     return check_launch("encoder_tail_forward");
+}
+
+}  // namespace
+
+extern "C" int spgt_encoder_tail_forward(const float* attn_out, int64_t ld_attn, const float* x,
+                                         const float* fc_weight_kn, const float* fc_bias,
+                                         const float* ffn1_weight_kn, const float* ffn1_bias,
+                                         const float* ffn2_weight_kn, const float* ffn2_bias, int activation,
+                                         float* out, int64_t tokens, int attn_features, int dim_hidden,
+                                         int ffn_hidden, hipStream_t stream) {
+    return encoder_tail_common(attn_out, ld_attn, x, fc_weight_kn, fc_bias, ffn1_weight_kn, ffn1_bias, ffn2_weight_kn,
+                               ffn2_bias, activation, out, tokens, attn_features, dim_hidden, ffn_hidden, nullptr, 0.f,
+                               0.f, stream);
+}
+
+extern "C" int spgt_encoder_tail_forward_dropout(const float* attn_out, int64_t ld_attn, const float* x,
+                                                 const float* fc_weight_kn, const float* fc_bias,
+                                                 const float* ffn1_weight_kn, const float* ffn1_bias,
+                                                 const float* ffn2_weight_kn, const float* ffn2_bias, int activation,
+                                                 float* out, int64_t tokens, int attn_features, int dim_hidden,
+                                                 int ffn_hidden, const uint32_t* seed, float fc_droprate,
+                                                 float ffn_droprate, hipStream_t stream) {
+    if (int rc = dropout_args_ok(seed, fc_droprate, ffn_droprate)) return rc;
+    return encoder_tail_common(attn_out, ld_attn, x, fc_weight_kn, fc_bias, ffn1_weight_kn, ffn1_bias, ffn2_weight_kn,
+                               ffn2_bias, activation, out, tokens, attn_features, dim_hidden, ffn_hidden, seed,
+                               fc_droprate, ffn_droprate, stream);
 }

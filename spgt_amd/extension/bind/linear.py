@@ -128,11 +128,35 @@ def encoder_tail_supported(attn_features: int, dim_hidden: int, ffn_hidden: int)
     return bool(_lib.load().spgt_encoder_tail_supported(int(attn_features), int(dim_hidden), int(ffn_hidden)))
 
 
+def dropout_seed(device) -> Tensor:
+    """Two 32-bit words from torch's generator of `device`, in device memory, for the kernels that apply dropout
+    themselves.  Drawn by a generator kernel: torch.manual_seed governs it, and inside a captured graph every
+    replay draws new words."""
+    return torch.randint(0, 2 ** 31 - 1, (2,), dtype=torch.int32, device=device)
+
+
+def _dropout_args(x: Tensor, fc_droprate: float, ffn_droprate: float, seed):
+    fc_droprate, ffn_droprate = float(fc_droprate), float(ffn_droprate)
+    if not (0.0 <= fc_droprate < 1.0 and 0.0 <= ffn_droprate < 1.0):
+        raise ValueError("drop rates must lie in [0, 1)")
+    if fc_droprate == 0.0 and ffn_droprate == 0.0:
+        return 0.0, 0.0, None
+    if seed is None:
+        seed = dropout_seed(x.device)
+    if not (seed.is_cuda and seed.device == x.device and seed.dtype == torch.int32 and seed.numel() >= 2 and
+            seed.is_contiguous()):
+        raise ValueError("seed must be a contiguous int32 tensor of two words on x's device")
+    return fc_droprate, ffn_droprate, seed
+
+
 def fused_encoder_tail(attn_out: Tensor, x: Tensor, fc_weight_kn: Tensor, fc_bias: Tensor, ffn1_weight_kn: Tensor,
-                       ffn1_bias: Tensor, ffn2_weight_kn: Tensor, ffn2_bias: Tensor, activation: str) -> Tensor:
+                       ffn1_bias: Tensor, ffn2_weight_kn: Tensor, ffn2_bias: Tensor, activation: str,
+                       fc_droprate: float = 0.0, ffn_droprate: float = 0.0, seed: Optional[Tensor] = None) -> Tensor:
     """y1 = x + attn_out @ fc_weight_kn + fc_bias;  returns y1 + act(y1 @ ffn1_weight_kn + ffn1_bias) @ ffn2_weight_kn
     + ffn2_bias: the attention's output projection, both residual adds and the feed-forward net of an encoder layer
-    in one kernel.  attn_out [..., K1], x [..., D]; weights [in, out] contiguous."""
+    in one kernel.  attn_out [..., K1], x [..., D]; weights [in, out] contiguous.
+    With drop rates above 0 the two terms added to the residual stream are dropped first, as the reference's
+    F.dropout calls do (masks from this library's own generator, seeded by `seed` or by dropout_seed)."""
     if activation not in ACTIVATIONS:
         raise ValueError(f"activation must be one of {sorted(ACTIVATIONS)}")
     for name, w in (("fc_weight_kn", fc_weight_kn), ("fc_bias", fc_bias), ("ffn1_weight_kn", ffn1_weight_kn),
@@ -151,16 +175,24 @@ def fused_encoder_tail(attn_out: Tensor, x: Tensor, fc_weight_kn: Tensor, fc_bia
     out = torch.empty_like(x)
     if T == 0:
         return out
+    fc_droprate, ffn_droprate, seed = _dropout_args(x, fc_droprate, ffn_droprate, seed)
     with torch.cuda.device(x.device):
-        check(_lib.load().spgt_encoder_tail_forward(
-            ptr(ar), lda, ptr(x), ptr(fc_weight_kn), ptr(fc_bias), ptr(ffn1_weight_kn), ptr(ffn1_bias),
-            ptr(ffn2_weight_kn), ptr(ffn2_bias), ACTIVATIONS[activation], ptr(out), T, K1, D, F, stream_of(x)))
+        if seed is None:
+            check(_lib.load().spgt_encoder_tail_forward(
+                ptr(ar), lda, ptr(x), ptr(fc_weight_kn), ptr(fc_bias), ptr(ffn1_weight_kn), ptr(ffn1_bias),
+                ptr(ffn2_weight_kn), ptr(ffn2_bias), ACTIVATIONS[activation], ptr(out), T, K1, D, F, stream_of(x)))
+        else:
+            check(_lib.load().spgt_encoder_tail_forward_dropout(
+                ptr(ar), lda, ptr(x), ptr(fc_weight_kn), ptr(fc_bias), ptr(ffn1_weight_kn), ptr(ffn1_bias),
+                ptr(ffn2_weight_kn), ptr(ffn2_bias), ACTIVATIONS[activation], ptr(out), T, K1, D, F, ptr(seed),
+                fc_droprate, ffn_droprate, stream_of(x)))
     return out
 
 
 def fused_encoder_tail_folded(q: Tensor, position, x: Tensor, folded_fc: Tensor, folded_pos, fc_bias: Tensor,
                               ffn1_weight_kn: Tensor, ffn1_bias: Tensor, ffn2_weight_kn: Tensor, ffn2_bias: Tensor,
-                              activation: str) -> Tensor:
+                              activation: str, fc_droprate: float = 0.0, ffn_droprate: float = 0.0,
+                              seed: Optional[Tensor] = None) -> Tensor:
     """fused_encoder_tail with the attention's last product folded into the output projection (see
     galerkin_attention.fold_ktv_into_fc): y1 = x + q @ folded_fc[b] + position @ folded_pos[b] + fc_bias, then the
     feed-forward net.  q [B, S, 128] (the projected Q; a column slice of the packed projection is fine),
@@ -192,11 +224,18 @@ def fused_encoder_tail_folded(q: Tensor, position, x: Tensor, folded_fc: Tensor,
     out = torch.empty_like(x)
     if out.numel() == 0:
         return out
+    fc_droprate, ffn_droprate, seed = _dropout_args(x, fc_droprate, ffn_droprate, seed)
     with torch.cuda.device(x.device):
-        check(_lib.load().spgt_encoder_tail_folded_forward(
-            ptr(q), ld, ptr(position) if dp else None, ptr(x), ptr(folded_fc), ptr(folded_pos) if dp else None,
-            ptr(fc_bias), ptr(ffn1_weight_kn), ptr(ffn1_bias), ptr(ffn2_weight_kn), ptr(ffn2_bias),
-            ACTIVATIONS[activation], ptr(out), B, S, dp, D, F, stream_of(x)))
+        if seed is None:
+            check(_lib.load().spgt_encoder_tail_folded_forward(
+                ptr(q), ld, ptr(position) if dp else None, ptr(x), ptr(folded_fc), ptr(folded_pos) if dp else None,
+                ptr(fc_bias), ptr(ffn1_weight_kn), ptr(ffn1_bias), ptr(ffn2_weight_kn), ptr(ffn2_bias),
+                ACTIVATIONS[activation], ptr(out), B, S, dp, D, F, stream_of(x)))
+        else:
+            check(_lib.load().spgt_encoder_tail_folded_forward_dropout(
+                ptr(q), ld, ptr(position) if dp else None, ptr(x), ptr(folded_fc), ptr(folded_pos) if dp else None,
+                ptr(fc_bias), ptr(ffn1_weight_kn), ptr(ffn1_bias), ptr(ffn2_weight_kn), ptr(ffn2_bias),
+                ACTIVATIONS[activation], ptr(out), B, S, dp, D, F, ptr(seed), fc_droprate, ffn_droprate, stream_of(x)))
     return out
 
 

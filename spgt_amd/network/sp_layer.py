@@ -246,10 +246,13 @@ class Sp_EncoderLayer(nn.Module):
     @refreshes_derived
     def forward(self, X: Tensor, position: Tensor) -> Tensor:
         att, ffn = self.attention_layer, self.ffn_layer
-        if (att.fc_droprate == 0 and ffn.droprate == 0 and gpu_inference(X, *self.parameters()) and
+        if (0 <= att.fc_droprate < 1 and 0 <= ffn.droprate < 1 and gpu_inference(X, *self.parameters()) and
                 encoder_tail_supported(att.fc_layer.in_features, att.fc_layer.out_features, ffn.layer1.out_features)
                 and ffn.layer2.out_features == att.fc_layer.out_features):
-            # output projection, both residual adds and the feed-forward net in one launch
+            # output projection, both residual adds and the feed-forward net in one launch; the layer's two
+            # dropouts (always on in the reference, network/sp_layer.py:76 and network/layer.py:173) are applied
+            # inside it when their rates are not zero
+            drop = dict(fc_droprate=att.fc_droprate, ffn_droprate=ffn.droprate)
             fold = (X.numel() // X.size(-1) >= self.fold_attention_min_tokens if self.fold_attention is None
                     else self.fold_attention)
             if fold and att.dim_head == 32 and att.num_head * 32 == X.size(-1) == 128 and X.dim() == 3:
@@ -258,11 +261,11 @@ class Sp_EncoderLayer(nn.Module):
                 return fused_encoder_tail_folded(q, pos, X.contiguous(), folded_fc, folded_pos, att.fc_layer.bias,
                                                  linear_weight_kn(ffn.layer1), ffn.layer1.bias,
                                                  linear_weight_kn(ffn.layer2), ffn.layer2.bias,
-                                                 activation_name(ffn.activation_layer))
+                                                 activation_name(ffn.activation_layer), **drop)
             A = att.attend(X, X, X, position)
             return fused_encoder_tail(A, X.contiguous(), linear_weight_kn(att.fc_layer), att.fc_layer.bias,
                                       linear_weight_kn(ffn.layer1), ffn.layer1.bias, linear_weight_kn(ffn.layer2),
-                                      ffn.layer2.bias, activation_name(ffn.activation_layer))
+                                      ffn.layer2.bias, activation_name(ffn.activation_layer), **drop)
         X = self.attention_layer(X, X, X, position, residual=X)
         return self.ffn_layer(X, residual=X)
 

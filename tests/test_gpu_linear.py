@@ -209,6 +209,82 @@ def test_encoder_tail(gpu, K1, T, act):
     assert got.shape == want.shape
     assert (got - want).abs().max().item() <= 2e-5 * max(1.0, want.abs().max().item())
 
+@pytest.mark.parametrize("variant", ["plain136", "plain128", "folded"])
+def test_encoder_tail_dropout(gpu, variant):
+    """The tail's two dropouts (the reference's always-on F.dropout of fc_layer's and of the feed-forward net's
+    output, network/sp_layer.py:76 and network/layer.py:173).  The masks are the library's own, so the test is of
+    their properties: every element of the dropped term is either 0 or the undropped value / (1 - p); the kept
+    fraction is 1 - p overall, per column and per token; neighbouring columns, neighbouring tokens and the two sites
+    are uncorrelated; one seed repeats, another differs; rate 0 is the kernel without dropout, bit for bit."""
+    from spgt_amd.extension.bind.linear import fused_encoder_tail, fused_encoder_tail_folded
+    g = torch.Generator().manual_seed(11)
+    B, S = 3, 3333
+    T, p = B * S, 0.3
+    K1 = 136 if variant == "plain136" else 128
+    x = torch.randn(B, S, 128, generator=g).to(gpu)
+    bfc = torch.randn(128, generator=g).to(gpu)
+    w1, b1 = (torch.randn(128, 256, generator=g) / 128 ** 0.5).to(gpu), torch.randn(256, generator=g).to(gpu)
+    w2, b2 = (torch.randn(256, 128, generator=g) / 16.0).to(gpu), torch.randn(128, generator=g).to(gpu)
+    if variant == "folded":
+        q = torch.randn(B, S, 128, generator=g).to(gpu)
+        pos = torch.rand(B, S, 2, generator=g).to(gpu)
+        ffc = (torch.randn(B, 128, 128, generator=g) / 11.0).to(gpu)
+        fpos = torch.randn(B, 2, 128, generator=g).to(gpu)
+        run = lambda w2_, b2_, **kw: fused_encoder_tail_folded(q, pos, x, ffc, fpos, bfc, w1, b1, w2_, b2_, "silu", **kw)
+    else:
+        a = torch.randn(B, S, K1, generator=g).to(gpu)
+        wfc = (torch.randn(K1, 128, generator=g) / K1 ** 0.5).to(gpu)
+        run = lambda w2_, b2_, **kw: fused_encoder_tail(a, x, wfc, bfc, w1, b1, w2_, b2_, "silu", **kw)
+    z2, zb = torch.zeros_like(w2), torch.zeros_like(b2)
+    seed = torch.tensor([12345, 678], dtype=torch.int32, device=gpu)
+    seed2 = torch.tensor([12346, 678], dtype=torch.int32, device=gpu)
+    y1 = run(z2, zb)                     # x + fc
+    full = run(w2, b2)                   # y1 + ffn
+    assert torch.equal(run(w2, b2, fc_droprate=0.0, ffn_droprate=0.0, seed=seed), full)
+
+    def check_site(dropped, base, term, what):
+        """dropped = base + mask * term / (1 - p); returns the mask [T, 128]."""
+        d = (dropped - base).reshape(T, 128).double()
+        t = term.reshape(T, 128).double() / (1 - p)
+        tol = 2e-5 * max(1.0, t.abs().max().item())
+        # (the kernel with dropout adds the residual after the position rows, the one without before them: `base`
+        # may differ from the kernel's own value in the last bit, so "dropped" is |d| < tol rather than d == 0)
+        keep = d.abs() > 0.5 * t.abs()
+        clear = t.abs() > 10 * tol          # elements whose term tells the two cases apart: all but a handful
+        assert clear.float().mean().item() > 0.995, what
+        assert ((d - t).abs()[keep & clear] < tol).all(), what
+        assert (d.abs()[~keep & clear] < tol).all(), what
+        keep = keep | ~clear                # (counted as kept: at most 0.5 % of the elements)
+        frac = keep.float().mean().item()
+        assert frac == pytest.approx(1 - p, abs=3e-3), what
+        assert (keep.float().mean(0) - (1 - p)).abs().max().item() < 0.03, what            # per column, 10k tokens
+        per_token = keep.float().mean(1)
+        assert per_token.std().item() == pytest.approx((p * (1 - p) / 128) ** 0.5, rel=0.1), what
+        assert (keep[:, 1:] & keep[:, :-1]).float().mean().item() == pytest.approx((1 - p) ** 2, abs=4e-3), what
+        assert (keep[1:] & keep[:-1]).float().mean().item() == pytest.approx((1 - p) ** 2, abs=4e-3), what
+        return keep
+
+    # the fc site alone (feed-forward weights zero: out = y1)
+    d_fc = run(z2, zb, fc_droprate=p, seed=seed)
+    m_fc = check_site(d_fc, x, y1 - x, "fc site")
+    assert torch.equal(d_fc, run(z2, zb, fc_droprate=p, seed=seed))
+    m_other = check_site(run(z2, zb, fc_droprate=p, seed=seed2), x, y1 - x, "fc site, another seed")
+    assert (m_fc != m_other).float().mean().item() == pytest.approx(2 * p * (1 - p), abs=5e-3)
+    # the feed-forward site alone
+    d_ffn = run(w2, b2, ffn_droprate=p, seed=seed)
+    m_ffn = check_site(d_ffn, y1, full - y1, "ffn site")
+    assert (m_fc & m_ffn).float().mean().item() == pytest.approx((1 - p) ** 2, abs=4e-3)
+    # both: a seed is drawn when none is given, and two calls differ
+    o1, o2 = run(w2, b2, fc_droprate=p, ffn_droprate=p), run(w2, b2, fc_droprate=p, ffn_droprate=p)
+    assert not torch.equal(o1, o2) and torch.isfinite(o1).all()
+    torch.manual_seed(5)
+    o3 = run(w2, b2, fc_droprate=p, ffn_droprate=p)
+    torch.manual_seed(5)
+    assert torch.equal(o3, run(w2, b2, fc_droprate=p, ffn_droprate=p))
+    with pytest.raises(Exception):
+        run(w2, b2, fc_droprate=1.0)
+
+
 @pytest.mark.parametrize("K1", [128, 136])
 @pytest.mark.parametrize("T", [8192 + 5, 70001])
 def test_encoder_tail_many_tiles(gpu, K1, T):

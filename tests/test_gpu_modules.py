@@ -273,6 +273,59 @@ def test_encoder_layer_folded_attention(gpu, dp, B, S):
     assert rel_l2(got.cpu(), want.cpu()) < 1e-5 and max_rel(got.cpu(), want.cpu()) < 1e-4
 
 
+@pytest.mark.parametrize("fold", [False, True])
+def test_encoder_layer_with_drop_rates_stays_fused(gpu, fold):
+    """With the reference's drop rates (always on, F.dropout's default) the layer still runs as one launch after the
+    attention core, with the two dropouts inside it.  A dropout only on fc_layer's output enters the layer's first
+    residual sum linearly, so with the feed-forward net's second layer zeroed the mean over many draws is the layer
+    without dropout; draws differ, torch.manual_seed repeats them, and a captured graph draws new masks on every
+    replay."""
+    torch.manual_seed(9)
+    B, S = 2, 600
+    layer = L.Sp_EncoderLayer(128, 4, 2, 1e-6, 0.0, 0.25, 0.5, 0.01, False, 256, 0.0, "relu").to(gpu).eval()
+    layer.fold_attention = fold
+    with torch.no_grad():
+        layer.ffn_layer.layer2.weight.zero_()
+        layer.ffn_layer.layer2.bias.zero_()
+    x = torch.randn(B, S, 128, device=gpu)
+    pos = torch.rand(B, S, 2, device=gpu)
+    with torch.no_grad():
+        layer.attention_layer.fc_droprate = 0.0
+        want = layer(x, pos)
+        layer.attention_layer.fc_droprate = 0.25
+        n = 400
+        acc = torch.zeros_like(want, dtype=torch.float64)
+        for _ in range(n):
+            acc += layer(x, pos)
+        mean = (acc / n).float()
+        # element-wise standard error of the mean: |term| sqrt(p / (1 - p) / n) = 0.029 |term|
+        term = (want - x).abs()
+        assert ((mean - want).abs() <= 0.029 * 6 * term + 1e-5).all()
+        torch.manual_seed(3)
+        a = layer(x, pos)
+        b = layer(x, pos)
+        torch.manual_seed(3)
+        assert torch.equal(a, layer(x, pos)) and not torch.equal(a, b)
+        layer.ffn_layer.droprate = 0.25
+        c = layer(x, pos)
+        assert torch.isfinite(c).all() and not torch.equal(c, a)
+        # a captured forward: the seed words are drawn by a generator kernel inside the graph
+        stream = torch.cuda.Stream()
+        stream.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(stream):
+            layer(x, pos)
+        torch.cuda.current_stream().wait_stream(stream)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            out = layer(x, pos)
+        outs = []
+        for _ in range(3):
+            graph.replay()
+            torch.cuda.synchronize()
+            outs.append(out.clone())
+        assert not torch.equal(outs[0], outs[1]) and not torch.equal(outs[1], outs[2])
+
+
 def test_graphed_inference_replays_match_eager(gpu):
     """A HIP-graph capture of the whole forward: every replay, with eager work and synchronisation between
     replays and with fresh inputs, reproduces the eager forward.  The convolution library picks algorithms
