@@ -382,6 +382,25 @@ int spgt_conv3x3_resample(const float* x, const float* weight, const float* bias
                           int Cout, int H_in, int W_in, int H_out, int W_out, int pre_activation,
                           int post_activation, spgt_stream_t stream);
 
+/* The three down-scaler kernels with ConvResBlock2D's dropout inside them (conv -> dropout -> activation,
+ * network/layer.py:7-24; F.dropout's default training=True keeps it on in inference too): the sum of convolution and
+ * bias is dropped before the first activation, with one decision per convolution output (n, c, y, x), the same for
+ * every resampled pixel that reads it.  seed: two 32-bit words in device memory (8-byte aligned), read by the
+ * kernel (see spgt_encoder_tail_forward_dropout); droprate in [0, 1), 0 = the call without dropout (seed may be
+ * null).  spgt_bilinear_resample_concat_dropout drops the samples of the sources flagged in pre_flags.  The masks
+ * are this library's own: the reference's distribution, not torch's random stream. */
+int spgt_bias_activation_nchw_dropout(float* x, const float* bias, int N, int C, int64_t HW, int activation,
+                                      int activation_count, const uint32_t* seed, float droprate,
+                                      spgt_stream_t stream);
+int spgt_conv3x3_resample_dropout(const float* x, const float* weight, const float* bias, float* out, int N, int Cin,
+                                  int Cout, int H_in, int W_in, int H_out, int W_out, int pre_activation,
+                                  int post_activation, const uint32_t* seed, float droprate, spgt_stream_t stream);
+int spgt_bilinear_resample_concat_dropout(const float* const* srcs, const float* const* pre_biases, const int* channels,
+                                          const int* pre_flags, int n_src, float* dst, int N, int H_in, int W_in,
+                                          int H_out, int W_out, int pre_activation, int pre_activation_count,
+                                          int post_activation, const uint32_t* seed, float droprate,
+                                          spgt_stream_t stream);
+
 /* The tail of ConvResBlock2D (network/layer.py:7-24) after a bias-free convolution, and the
  * scaler's own activation where it follows directly (network/model.py:61-62), in place:
  * x[n, c, :] = activation^activation_count(x[n, c, :] + bias[c]) on x [N, C, HW]; bias may be null,

@@ -57,7 +57,10 @@ SIGNATURES = {
     "spgt_bilinear_adjoint": (_i, [_p, _p, _i, _i, _i, _i, _i, _i, _i, _p]),
     "spgt_upsample_conv3x3_gather": (_i, [_p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p]),
     "spgt_bilinear_resample_concat": (_i, [_p, _p, _p, _p, _i, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p]),
+    "spgt_bilinear_resample_concat_dropout": (
+        _i, [_p, _p, _p, _p, _i, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p, _f, _p]),
     "spgt_bias_activation_nchw": (_i, [_p, _p, _i, _i, _i64, _i, _i, _p]),
+    "spgt_bias_activation_nchw_dropout": (_i, [_p, _p, _i, _i, _i64, _i, _i, _p, _f, _p]),
     "spgt_denormalize_boundary": (_i, [_p, _p, _p, _i, _p, _i, _i, _i, _i, _i, _p]),
     "spgt_spectral_inverse_linear_supported": (_i, [_i, _i, _i, _i]),
     "spgt_spectral_inverse_linear": (_i, [_p, _p, _p, _p, _p, _i, _p, _i64, _i, _i, _i, _i, _p]),
@@ -69,6 +72,7 @@ SIGNATURES = {
     "spgt_spectral_modes_middle": (_i, [_p, _p, _p, _p, _p, _p, _p, _sz, _i, _i, _i, _i, _i, _p]),
     "spgt_conv3x3_resample_supported": (_i, [_i]),
     "spgt_conv3x3_resample": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p]),
+    "spgt_conv3x3_resample_dropout": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p, _f, _p]),
     "spgt_linear_supported": (_i, [_i, _i]),
     "spgt_linear_forward": (_i, [_p, _i64, _p, _p, _p, _i64, _i, _i, _p, _i64, _p, _i, _p, _i64, _i, _i64, _i64, _i, _i,
                                  _p]),
@@ -171,3 +175,10 @@ def stream_of(t: torch.Tensor):
 def workspace(nbytes: int, like: torch.Tensor) -> torch.Tensor:
     """Scratch from torch's caching allocator on `like`'s device (at least 16 bytes)."""
     return torch.empty(max(int(nbytes), 16), dtype=torch.uint8, device=like.device)
+
+
+def dropout_seed(device):
+    """Two 32-bit words from torch's generator of `device`, in device memory, for the kernels that apply dropout
+    themselves.  Drawn by a generator kernel: torch.manual_seed governs it, and inside a captured graph every
+    replay draws new words."""
+    return torch.randint(0, 2 ** 31 - 1, (2,), dtype=torch.int32, device=device)

@@ -672,33 +672,7 @@ __device__ __forceinline__ void mfma_acc_done(v16f& acc) { asm volatile("s_nop 1
 // DROP: the reference's two dropouts of an encoder layer (always on, also in inference: F.dropout's default,
 // network/sp_layer.py:76 and network/layer.py:173) applied where their operands are formed,
 //   y1 = x + dropout(a @ Wfc + bfc, p_fc)        out = y1 + dropout(act(..) @ W2 + b2, p_ffn)
-// with the keep decision of element (token t, column n) a hash of (seed, site, t, n): an integer mixer of the
-// token's base value plus a per-column constant, compared with p * 2^32.  The seed is read from device memory, so
-// that a captured graph whose seed tensor is refilled by a generator kernel draws new masks on every replay.
-__device__ __forceinline__ uint32_t dropout_mix(uint32_t h) {
-    h ^= h >> 16;
-    h *= 0x21f0aaadu;
-    h ^= h >> 15;
-    h *= 0x735a2d97u;
-    h ^= h >> 15;
-    return h;
-}
-struct DropoutSite {
-    uint32_t base, threshold;
-    float scale;
-};
-__device__ __forceinline__ DropoutSite dropout_site(const uint32_t* seed, uint32_t site, int64_t t, float p) {
-    DropoutSite d;
-    const uint32_t lo = (uint32_t)t, hi = (uint32_t)((uint64_t)t >> 32);
-    d.base = dropout_mix(dropout_mix(seed[0] ^ (lo * 0x9e3779b1u)) ^ seed[1] ^ (hi * 0x85ebca77u) ^ (site * 0xc2b2ae3du));
-    d.threshold = p <= 0.f ? 0u : (uint32_t)fminf(p * 4294967296.0f, 4294967040.0f);
-    d.scale = p <= 0.f ? 1.f : 1.f / (1.f - p);
-    return d;
-}
-__device__ __forceinline__ float dropout_apply(const DropoutSite& d, int n, float v) {
-    return dropout_mix(d.base + (uint32_t)n * 0x27d4eb2fu) >= d.threshold ? v * d.scale : 0.f;
-}
-
+// with the keep decision of element (token t, column n) a hash of (seed, site, t, n) (dropout_site, dropout_apply).
 template <int K1, bool FOLD, bool DROP>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void encoder_tail_k(
     const float* __restrict__ a, int64_t lda, const float* __restrict__ x, const float* __restrict__ Wfc,
@@ -814,8 +788,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         const bool more = tile + step < limit;
         DropoutSite site_fc, site_ffn;
         if (DROP) {
-            site_fc = dropout_site(seed, 0u, t, p_fc);
-            site_ffn = dropout_site(seed, 1u, t, p_ffn);
+            site_fc = dropout_site(seed, kDropSiteFc, t, p_fc);
+            site_ffn = dropout_site(seed, kDropSiteFfn, t, p_ffn);
         }
         if (FOLD && tile_seq(tile) != cur_b) {
             // another sequence: its fc weights into the registers, its position rows into LDS (last read before

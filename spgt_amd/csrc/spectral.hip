@@ -279,6 +279,13 @@ struct ResampleAct {
     int pre, pre_n, post;
 };
 
+// Dropout of the source samples (ConvResBlock2D's conv -> dropout -> activation, network/layer.py:7-24, always on
+// in the reference): seed = two words in device memory, null for none; see dropout_site in spgt_device.h.
+struct DropArgs {
+    const uint32_t* seed;
+    float p;
+};
+
 // act applied `count` times to every element of v, with the choice of activation made once for all of them: the
 // element-wise form puts a branch tree between the loads of successive samples, which then go out a few at a time.
 template <int N>
@@ -541,7 +548,8 @@ struct ResampleSources {
 // grid: tiles = N * Hout * ceil(Wout/32), rounded up to a multiple of 8; block 256.
 __global__ __launch_bounds__(256) void bilinear_concat_to_nhwc_k(ResampleSources S, float* __restrict__ dst, int C,
                                                                  int Hin, int Win, int Hout, int Wout, float hscale,
-                                                                 float wscale, ResampleAct act, int xtiles, int tiles) {
+                                                                 float wscale, ResampleAct act, int xtiles, int tiles,
+                                                                 DropArgs drop) {
     __shared__ float4 tile[32 * 33];
     const int logical = xcd_contiguous_tile();
     if (logical >= tiles) return;
@@ -577,6 +585,16 @@ __global__ __launch_bounds__(256) void bilinear_concat_to_nhwc_k(ResampleSources
                 const float pb = (pre[k] && b) ? b[ch - lo] : 0.f;
 #pragma unroll
                 for (int j = 0; j < 4; ++j) u[4 * k + j] = t[4 * k + j] + pb;
+                if (drop.seed && pre[k]) {
+                    // a flagged source is a convolution output before its dropout: one decision per source sample,
+                    // the same for every output that reads it
+                    const DropoutSite ds = dropout_site(drop.seed, kDropSiteConcat, n * (hi - lo) + (ch - lo), drop.p);
+                    const uint32_t e = (uint32_t)off;
+                    u[4 * k] = dropout_apply(ds, e, u[4 * k]);
+                    u[4 * k + 1] = dropout_apply(ds, e + (uint32_t)tw.ip, u[4 * k + 1]);
+                    u[4 * k + 2] = dropout_apply(ds, e + (uint32_t)(th.ip * Win), u[4 * k + 2]);
+                    u[4 * k + 3] = dropout_apply(ds, e + (uint32_t)(th.ip * Win + tw.ip), u[4 * k + 3]);
+                }
             }
             if (S.pre_mask) {
                 act_many<16>(u, act.pre, act.pre_n);
@@ -929,7 +947,7 @@ __global__ __launch_bounds__(256) void conv3x3_resample_k(const float* __restric
                                                           const float* __restrict__ weight,
                                                           const float* __restrict__ bias, float* __restrict__ out,
                                                           int Cout, int H, int W, int Hout, int Wout, float hscale,
-                                                          float wscale, ResampleAct act) {
+                                                          float wscale, ResampleAct act, DropArgs drop) {
     const int ox = blockIdx.x * 64 + threadIdx.x;
     const int oy = blockIdx.y;
     const int64_t n = blockIdx.z;
@@ -982,6 +1000,16 @@ __global__ __launch_bounds__(256) void conv3x3_resample_k(const float* __restric
                 }
         // at the last row / column (hp or wp = 0) the second sample is the first one again
         float t[4] = {v00, wp ? v01 : v00, hp ? v10 : v00, hp ? (wp ? v11 : v10) : (wp ? v01 : v00)};
+        if (drop.seed) {
+            // the block's dropout sits between its convolution and its activation: one decision per convolution
+            // output (n, c, y, x), the same for every resampled pixel that reads it
+            const DropoutSite ds = dropout_site(drop.seed, kDropSiteConvResample, n * Cout + c, drop.p);
+            const uint32_t e = (uint32_t)(h1 * W + w1);
+            t[0] = dropout_apply(ds, e, t[0]);
+            t[1] = dropout_apply(ds, e + (uint32_t)wp, t[1]);
+            t[2] = dropout_apply(ds, e + (uint32_t)(hp * W), t[2]);
+            t[3] = dropout_apply(ds, e + (uint32_t)(hp * W + wp), t[3]);
+        }
         const float no_bias[1] = {0.f};  // the bias is in the convolution sums already
         float v[1];
         blend_many<true, 1>(t, no_bias, w0l, w1l, h0l, h1l, act, v);
@@ -992,15 +1020,21 @@ __global__ __launch_bounds__(256) void conv3x3_resample_k(const float* __restric
 // x[n, c, :] = act^count(x[n, c, :] + bias[c]) in place on [planes = N*C, HW]: the bias add and the
 // activation(s) that follow a bias-free convolution.  grid (chunks, planes), block 256.
 __global__ __launch_bounds__(256) void bias_activation_nchw_k(float* __restrict__ x, const float* __restrict__ bias,
-                                                              int C, int64_t HW, int act, int count) {
+                                                              int C, int64_t HW, int act, int count, DropArgs drop) {
     const int64_t pl = blockIdx.y;
     const float b = bias ? bias[pl % C] : 0.f;
     float* row = x + pl * HW;
     const int64_t stride = (int64_t)gridDim.x * 256;
+    DropoutSite ds;
+    if (drop.seed) ds = dropout_site(drop.seed, kDropSiteBiasAct, pl, drop.p);
     for (int64_t e0 = (int64_t)blockIdx.x * 256 + threadIdx.x; e0 < HW; e0 += 4 * stride) {
         float v[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) v[j] = row[min(e0 + j * stride, HW - 1)] + b;  // past the end: read, not written
+        if (drop.seed) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) v[j] = dropout_apply(ds, (uint32_t)min(e0 + j * stride, HW - 1), v[j]);
+        }
         act_many<4>(v, act, count);
 #pragma unroll
         for (int j = 0; j < 4; ++j)
@@ -1176,10 +1210,22 @@ extern "C" int spgt_bilinear_align_corners_nhwc(const float* src, float* dst, in
                            SPGT_LAYOUT_NHWC, ResampleAct{SPGT_ACT_NONE, 0, SPGT_ACT_NONE}, stream);
 }
 
-extern "C" int spgt_bilinear_resample_concat(const float* const* srcs, const float* const* pre_biases,
-                                             const int* channels, const int* pre_flags, int n_src, float* dst, int N,
-                                             int H_in, int W_in, int H_out, int W_out, int pre_activation,
-                                             int pre_activation_count, int post_activation, hipStream_t stream) {
+namespace {
+
+// seed / rate of the entry points that drop: rate 0 means none (seed may then be null)
+int drop_args(const uint32_t* seed, float droprate, spgt::DropArgs* out) {
+    if (!(droprate >= 0.f && droprate < 1.f)) return fail(SPGT_ERR_INVALID_ARGUMENT, "dropout: the rate must lie in [0, 1)");
+    if (droprate > 0.f && (!seed || !aligned8(seed)))
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "dropout: a rate above 0 needs an 8-byte aligned seed (two 32-bit words) in device memory");
+    out->seed = droprate > 0.f ? seed : nullptr;
+    out->p = droprate;
+    return SPGT_OK;
+}
+
+int resample_concat_common(const float* const* srcs, const float* const* pre_biases, const int* channels,
+                           const int* pre_flags, int n_src, float* dst, int N, int H_in, int W_in, int H_out, int W_out,
+                           int pre_activation, int pre_activation_count, int post_activation, spgt::DropArgs drop,
+                           hipStream_t stream) {
     if (!srcs || !channels || !dst) return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear_resample_concat: null pointer argument");
     if (n_src < 1 || n_src > 4) return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear_resample_concat: 1 to 4 sources");
     if (N <= 0 || H_in <= 0 || W_in <= 0 || H_out <= 0 || W_out <= 0)
@@ -1218,9 +1264,32 @@ extern "C" int spgt_bilinear_resample_concat(const float* const* srcs, const flo
     const float wscale = W_out > 1 ? (float)(W_in - 1) / (float)(W_out - 1) : 0.f;
     const ResampleSources S{src[0], src[1], src[2], src[3], bias[0], bias[1], bias[2], bias[3],
                             first[1], first[2], first[3], mask};
+    if ((int64_t)H_in * W_in > UINT32_MAX) return fail(SPGT_ERR_INVALID_ARGUMENT, "bilinear_resample_concat: source planes above 2^32 samples");
     hipLaunchKernelGGL(spgt::bilinear_concat_to_nhwc_k, dim3((unsigned)(ceil_div(tiles, (int64_t)8) * 8)), dim3(256), 0,
-                       stream, S, dst, (int)C, H_in, W_in, H_out, W_out, hscale, wscale, act, xtiles, (int)tiles);
+                       stream, S, dst, (int)C, H_in, W_in, H_out, W_out, hscale, wscale, act, xtiles, (int)tiles, drop);
     return check_launch("bilinear_resample_concat");
+}
+
+}  // namespace
+
+extern "C" int spgt_bilinear_resample_concat(const float* const* srcs, const float* const* pre_biases,
+                                             const int* channels, const int* pre_flags, int n_src, float* dst, int N,
+                                             int H_in, int W_in, int H_out, int W_out, int pre_activation,
+                                             int pre_activation_count, int post_activation, hipStream_t stream) {
+    return resample_concat_common(srcs, pre_biases, channels, pre_flags, n_src, dst, N, H_in, W_in, H_out, W_out,
+                                  pre_activation, pre_activation_count, post_activation, spgt::DropArgs{nullptr, 0.f},
+                                  stream);
+}
+
+extern "C" int spgt_bilinear_resample_concat_dropout(const float* const* srcs, const float* const* pre_biases,
+                                                     const int* channels, const int* pre_flags, int n_src, float* dst,
+                                                     int N, int H_in, int W_in, int H_out, int W_out,
+                                                     int pre_activation, int pre_activation_count, int post_activation,
+                                                     const uint32_t* seed, float droprate, hipStream_t stream) {
+    spgt::DropArgs drop;
+    if (int rc = drop_args(seed, droprate, &drop)) return rc;
+    return resample_concat_common(srcs, pre_biases, channels, pre_flags, n_src, dst, N, H_in, W_in, H_out, W_out,
+                                  pre_activation, pre_activation_count, post_activation, drop, stream);
 }
 
 extern "C" int spgt_upsample_conv3x3_gather(const float* Z, const float* bias, float* dst, int N, int C, int H_in,
@@ -1371,8 +1440,10 @@ extern "C" int spgt_denormalize_boundary(const float* x, const float* scale, con
     return check_launch("denormalize_boundary");
 }
 
-extern "C" int spgt_bias_activation_nchw(float* x, const float* bias, int N, int C, int64_t HW, int activation,
-                                         int activation_count, hipStream_t stream) {
+namespace {
+
+int bias_activation_common(float* x, const float* bias, int N, int C, int64_t HW, int activation, int activation_count,
+                           spgt::DropArgs drop, hipStream_t stream) {
     if (!x) return fail(SPGT_ERR_INVALID_ARGUMENT, "bias_activation_nchw: null pointer argument");
     if (N <= 0 || C <= 0 || HW <= 0) return fail(SPGT_ERR_INVALID_ARGUMENT, "bias_activation_nchw: sizes must be positive");
     if ((int64_t)N * C > 65535) return fail(SPGT_ERR_INVALID_ARGUMENT, "bias_activation_nchw: N*C exceeds 65535");
@@ -1381,16 +1452,34 @@ extern "C" int spgt_bias_activation_nchw(float* x, const float* bias, int N, int
     if (!aligned4(x) || (bias && !aligned4(bias)))
         return fail(SPGT_ERR_INVALID_ARGUMENT, "bias_activation_nchw: operands must be 4-byte aligned");
     const int chunks = (int)std::min<int64_t>(ceil_div(HW, (int64_t)1024), 64);
+    if (HW > UINT32_MAX) return fail(SPGT_ERR_INVALID_ARGUMENT, "bias_activation_nchw: planes above 2^32 elements");
     hipLaunchKernelGGL(bias_activation_nchw_k, dim3(chunks, N * C), dim3(256), 0, stream, x, bias, C, HW, activation,
-                       activation == SPGT_ACT_NONE ? 0 : activation_count);
+                       activation == SPGT_ACT_NONE ? 0 : activation_count, drop);
     return check_launch("bias_activation_nchw");
+}
+
+}  // namespace
+
+extern "C" int spgt_bias_activation_nchw(float* x, const float* bias, int N, int C, int64_t HW, int activation,
+                                         int activation_count, hipStream_t stream) {
+    return bias_activation_common(x, bias, N, C, HW, activation, activation_count, spgt::DropArgs{nullptr, 0.f}, stream);
+}
+
+extern "C" int spgt_bias_activation_nchw_dropout(float* x, const float* bias, int N, int C, int64_t HW, int activation,
+                                                 int activation_count, const uint32_t* seed, float droprate,
+                                                 hipStream_t stream) {
+    spgt::DropArgs drop;
+    if (int rc = drop_args(seed, droprate, &drop)) return rc;
+    return bias_activation_common(x, bias, N, C, HW, activation, activation_count, drop, stream);
 }
 
 extern "C" int spgt_conv3x3_resample_supported(int Cin) { return (Cin >= 1 && Cin <= 4) ? 1 : 0; }
 
-extern "C" int spgt_conv3x3_resample(const float* x, const float* weight, const float* bias, float* out, int N,
-                                     int Cin, int Cout, int H_in, int W_in, int H_out, int W_out, int pre_activation,
-                                     int post_activation, hipStream_t stream) {
+namespace {
+
+int conv3x3_resample_common(const float* x, const float* weight, const float* bias, float* out, int N, int Cin, int Cout,
+                            int H_in, int W_in, int H_out, int W_out, int pre_activation, int post_activation,
+                            spgt::DropArgs drop, hipStream_t stream) {
     if (!x || !weight || !out) return fail(SPGT_ERR_INVALID_ARGUMENT, "conv3x3_resample: null pointer argument");
     if (N <= 0 || Cout <= 0 || H_in <= 0 || W_in <= 0 || H_out <= 0 || W_out <= 0)
         return fail(SPGT_ERR_INVALID_ARGUMENT, "conv3x3_resample: sizes must be positive");
@@ -1409,7 +1498,8 @@ extern "C" int spgt_conv3x3_resample(const float* x, const float* weight, const 
     if (lds > 64 * 1024) return fail(SPGT_ERR_INVALID_ARGUMENT, "conv3x3_resample: too many output channels");
 #define SPGT_CONV(CI)                                                                                                \
     hipLaunchKernelGGL(conv3x3_resample_k<CI>, grid, block, lds, stream, x, weight, bias, out, Cout, H_in, W_in,      \
-                       H_out, W_out, hscale, wscale, act)
+                       H_out, W_out, hscale, wscale, act, drop)
+    if ((int64_t)H_in * W_in > UINT32_MAX) return fail(SPGT_ERR_INVALID_ARGUMENT, "conv3x3_resample: planes above 2^32 samples");
     switch (Cin) {
         case 1: SPGT_CONV(1); break;
         case 2: SPGT_CONV(2); break;
@@ -1418,4 +1508,23 @@ extern "C" int spgt_conv3x3_resample(const float* x, const float* weight, const 
     }
 #undef SPGT_CONV
     return check_launch("conv3x3_resample");
+}
+
+}  // namespace
+
+extern "C" int spgt_conv3x3_resample(const float* x, const float* weight, const float* bias, float* out, int N,
+                                     int Cin, int Cout, int H_in, int W_in, int H_out, int W_out, int pre_activation,
+                                     int post_activation, hipStream_t stream) {
+    return conv3x3_resample_common(x, weight, bias, out, N, Cin, Cout, H_in, W_in, H_out, W_out, pre_activation,
+                                   post_activation, spgt::DropArgs{nullptr, 0.f}, stream);
+}
+
+extern "C" int spgt_conv3x3_resample_dropout(const float* x, const float* weight, const float* bias, float* out, int N,
+                                             int Cin, int Cout, int H_in, int W_in, int H_out, int W_out,
+                                             int pre_activation, int post_activation, const uint32_t* seed,
+                                             float droprate, hipStream_t stream) {
+    spgt::DropArgs drop;
+    if (int rc = drop_args(seed, droprate, &drop)) return rc;
+    return conv3x3_resample_common(x, weight, bias, out, N, Cin, Cout, H_in, W_in, H_out, W_out, pre_activation,
+                                   post_activation, drop, stream);
 }

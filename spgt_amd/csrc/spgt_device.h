@@ -203,6 +203,41 @@ __device__ __forceinline__ void zero_window_row_remainders(float2* __restrict__ 
     }
 }
 
+// Dropout inside a kernel (the reference's F.dropout calls, on by default also in inference): the keep decision of
+// element (row, column) of a site is an integer hash of (seed, site, row, column) compared with p * 2^32; kept values
+// are scaled by 1 / (1 - p).  A row is a token of a [T, C] tensor or a plane (n, c) of an NCHW one, the column the
+// position inside it; the row's base value is mixed once, an element costs one more mix.  The two seed words are read
+// from device memory, so that a captured graph whose seed tensor is refilled by a generator kernel draws new masks
+// on every replay.
+__device__ __forceinline__ uint32_t dropout_mix(uint32_t h) {
+    h ^= h >> 16;
+    h *= 0x21f0aaadu;
+    h ^= h >> 15;
+    h *= 0x735a2d97u;
+    h ^= h >> 15;
+    return h;
+}
+struct DropoutSite {
+    uint32_t base, threshold;
+    float scale;
+};
+__device__ __forceinline__ uint32_t dropout_threshold(float p) {
+    return p <= 0.f ? 0u : (uint32_t)fminf(p * 4294967296.0f, 4294967040.0f);
+}
+__device__ __forceinline__ DropoutSite dropout_site(const uint32_t* seed, uint32_t site, int64_t row, float p) {
+    DropoutSite d;
+    const uint32_t lo = (uint32_t)row, hi = (uint32_t)((uint64_t)row >> 32);
+    d.base = dropout_mix(dropout_mix(seed[0] ^ (lo * 0x9e3779b1u)) ^ seed[1] ^ (hi * 0x85ebca77u) ^ (site * 0xc2b2ae3du));
+    d.threshold = dropout_threshold(p);
+    d.scale = p <= 0.f ? 1.f : 1.f / (1.f - p);
+    return d;
+}
+__device__ __forceinline__ float dropout_apply(const DropoutSite& d, uint32_t column, float v) {
+    return dropout_mix(d.base + column * 0x27d4eb2fu) >= d.threshold ? v * d.scale : 0.f;
+}
+// Site numbers of the kernels that drop (distinct, so that one seed may serve a whole forward).
+enum { kDropSiteFc = 0, kDropSiteFfn = 1, kDropSiteBiasAct = 2, kDropSiteConvResample = 3, kDropSiteConcat = 4 };
+
 __host__ __device__ __forceinline__ int ceil_div(int a, int b) { return (a + b - 1) / b; }
 __host__ __device__ __forceinline__ int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 

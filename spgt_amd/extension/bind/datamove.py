@@ -15,7 +15,7 @@ import torch
 from torch import Tensor
 
 from ... import _lib
-from ..._lib import check, ptr, require_gpu_f32, stream_of, workspace
+from ..._lib import check, dropout_seed, ptr, require_gpu_f32, stream_of, workspace
 
 
 # --------------------------------------------------------------------------- #
@@ -325,11 +325,27 @@ def _bilinear_resample(X: Tensor, size, src_nhwc: bool = False, dst_nhwc: bool =
     return out
 
 
+def _drop_seed(device, droprate: float, seed):
+    """(rate, seed tensor or None): a seed is drawn when the rate is not zero and none was given."""
+    droprate = float(droprate)
+    if not 0.0 <= droprate < 1.0:
+        raise ValueError("the drop rate must lie in [0, 1)")
+    if droprate == 0.0:
+        return 0.0, None
+    if seed is None:
+        seed = dropout_seed(device)
+    if not (seed.is_cuda and seed.device == device and seed.dtype == torch.int32 and seed.numel() >= 2 and
+            seed.is_contiguous()):
+        raise ValueError("seed must be a contiguous int32 tensor of two words on the operands' device")
+    return droprate, seed
+
+
 def _bilinear_resample_concat(sources, size, pre_biases=None, pre_flags=None, pre_activation=None,
-                              pre_count: int = 1, post_activation=None) -> Tensor:
+                              pre_count: int = 1, post_activation=None, pre_droprate: float = 0.0, seed=None) -> Tensor:
     """post(interpolate(cat(sources, dim=1))) into channels-last without the concatenated tensor: sources are 1 to 4
     NCHW tensors [N, C_s, H, W] whose channel counts add up to a multiple of 4.  Where pre_flags[s] is set, source s
-    first gets pre_biases[s] (or nothing, if None) added and pre_activation applied pre_count times."""
+    first gets pre_biases[s] (or nothing, if None) added, is dropped at pre_droprate (ConvResBlock2D's dropout,
+    between the convolution and its activation) and has pre_activation applied pre_count times."""
     n = len(sources)
     if not 1 <= n <= 4:
         raise ValueError("1 to 4 sources")
@@ -360,10 +376,16 @@ def _bilinear_resample_concat(sources, size, pre_biases=None, pre_flags=None, pr
     chans = (ctypes.c_int * n)(*[int(X.shape[1]) for X in sources])
     flags = (ctypes.c_int * n)(*pre_flags)
     npre = int(pre_count) if _ACT[pre_activation] else 0
+    pre_droprate, seed = _drop_seed(out.device, pre_droprate if any(pre_flags) else 0.0, seed)
     with torch.cuda.device(out.device):
-        check(_lib.load().spgt_bilinear_resample_concat(srcs, biases, chans, flags, n, ptr(out), N, H_in, W_in, H_out,
-                                                        W_out, _ACT[pre_activation], npre, _ACT[post_activation],
-                                                        stream_of(out)))
+        if seed is None:
+            check(_lib.load().spgt_bilinear_resample_concat(srcs, biases, chans, flags, n, ptr(out), N, H_in, W_in,
+                                                            H_out, W_out, _ACT[pre_activation], npre,
+                                                            _ACT[post_activation], stream_of(out)))
+        else:
+            check(_lib.load().spgt_bilinear_resample_concat_dropout(
+                srcs, biases, chans, flags, n, ptr(out), N, H_in, W_in, H_out, W_out, _ACT[pre_activation], npre,
+                _ACT[post_activation], ptr(seed), pre_droprate, stream_of(out)))
     return out
 
 
@@ -421,8 +443,8 @@ def _bilinear_nhwc_affine(X: Tensor, size, extra: Tensor = None, weight_extra_kn
     return out
 
 
-def _bias_activation_nchw_(X: Tensor, bias, activation=None, count: int = 1) -> Tensor:
-    """In place on X [N, C, ...]: X = activation^count(X + bias[c]); returns X."""
+def _bias_activation_nchw_(X: Tensor, bias, activation=None, count: int = 1, droprate: float = 0.0, seed=None) -> Tensor:
+    """In place on X [N, C, ...]: X = activation^count(dropout(X + bias[c], droprate)); returns X."""
     require_gpu_f32("X", X)
     if X.dim() < 2:
         raise ValueError("X needs at least two dimensions")
@@ -436,9 +458,15 @@ def _bias_activation_nchw_(X: Tensor, bias, activation=None, count: int = 1) -> 
             raise ValueError(f"bias has {bias.numel()} elements, expected {C}")
     if X.numel() == 0:
         return X
+    droprate, seed = _drop_seed(X.device, droprate, seed)
     with torch.cuda.device(X.device):
-        check(_lib.load().spgt_bias_activation_nchw(ptr(X), ptr(bias) if bias is not None else None, N, C, HW,
-                                                    _ACT[activation], int(count), stream_of(X)))
+        if seed is None:
+            check(_lib.load().spgt_bias_activation_nchw(ptr(X), ptr(bias) if bias is not None else None, N, C, HW,
+                                                        _ACT[activation], int(count), stream_of(X)))
+        else:
+            check(_lib.load().spgt_bias_activation_nchw_dropout(ptr(X), ptr(bias) if bias is not None else None, N, C,
+                                                                HW, _ACT[activation], int(count), ptr(seed), droprate,
+                                                                stream_of(X)))
     return X
 
 
@@ -504,9 +532,10 @@ def _spectral_inverse_linear(U: Tensor, table_operand: Tensor, X: Tensor, weight
     return out
 
 
-def _conv3x3_resample(X: Tensor, weight: Tensor, bias, size, pre_activation=None, post_activation=None) -> Tensor:
-    """post(interpolate(pre(conv3x3(X, weight, padding=1) + bias))) for X [N, H, W, Cin] channels-last with
-    Cin <= 4: [N, Cout, H', W'] without the full-resolution convolution output ever being stored."""
+def _conv3x3_resample(X: Tensor, weight: Tensor, bias, size, pre_activation=None, post_activation=None,
+                      droprate: float = 0.0, seed=None) -> Tensor:
+    """post(interpolate(pre(dropout(conv3x3(X, weight, padding=1) + bias, droprate)))) for X [N, H, W, Cin]
+    channels-last with Cin <= 4: [N, Cout, H', W'] without the full-resolution convolution output ever being stored."""
     require_gpu_f32("X", X)
     require_gpu_f32("weight", weight)
     if X.dim() != 4 or weight.dim() != 4 or tuple(weight.shape[2:]) != (3, 3) or weight.shape[1] != X.shape[3]:
@@ -523,10 +552,17 @@ def _conv3x3_resample(X: Tensor, weight: Tensor, bias, size, pre_activation=None
     out = torch.empty((N, Cout, H_out, W_out), dtype=X.dtype, device=X.device)
     if out.numel() == 0:
         return out
+    droprate, seed = _drop_seed(X.device, droprate, seed)
     with torch.cuda.device(X.device):
-        check(_lib.load().spgt_conv3x3_resample(ptr(X), ptr(weight), ptr(bias) if bias is not None else None, ptr(out),
-                                                N, Cin, Cout, H, W, H_out, W_out, _ACT[pre_activation],
-                                                _ACT[post_activation], stream_of(X)))
+        if seed is None:
+            check(_lib.load().spgt_conv3x3_resample(ptr(X), ptr(weight), ptr(bias) if bias is not None else None,
+                                                    ptr(out), N, Cin, Cout, H, W, H_out, W_out, _ACT[pre_activation],
+                                                    _ACT[post_activation], stream_of(X)))
+        else:
+            check(_lib.load().spgt_conv3x3_resample_dropout(ptr(X), ptr(weight), ptr(bias) if bias is not None else None,
+                                                            ptr(out), N, Cin, Cout, H, W, H_out, W_out,
+                                                            _ACT[pre_activation], _ACT[post_activation], ptr(seed),
+                                                            droprate, stream_of(X)))
     return out
 
 
@@ -707,12 +743,12 @@ def bilinear_resample(X: Tensor, size, src_nhwc: bool = False, dst_nhwc: bool = 
 
 
 def bilinear_resample_concat(sources, size, pre_biases=None, pre_flags=None, pre_activation=None, pre_count: int = 1,
-                             post_activation=None) -> Tensor:
+                             post_activation=None, pre_droprate: float = 0.0, seed=None) -> Tensor:
     """post(interpolate(cat(sources, dim=1))) into channels-last, the concatenation never stored (inference only)."""
     return dexts.bilinear_resample_concat([X.detach() for X in sources], size,
                                           None if pre_biases is None else [None if b is None else b.detach()
                                                                            for b in pre_biases],
-                                          pre_flags, pre_activation, pre_count, post_activation)
+                                          pre_flags, pre_activation, pre_count, post_activation, pre_droprate, seed)
 
 
 def upsample_conv3x3_gather(Z: Tensor, bias, size, activation=None, count: int = 1) -> Tensor:
@@ -726,9 +762,9 @@ def bilinear_nhwc_affine(X: Tensor, size, extra: Tensor = None, weight_extra_kn:
                                       None if weight_extra_kn is None else weight_extra_kn.detach())
 
 
-def bias_activation_nchw_(X: Tensor, bias, activation=None, count: int = 1) -> Tensor:
-    """In place: X = activation^count(X + bias[c]) on [N, C, ...] (inference only)."""
-    return dexts.bias_activation_nchw_(X, None if bias is None else bias.detach(), activation, count)
+def bias_activation_nchw_(X: Tensor, bias, activation=None, count: int = 1, droprate: float = 0.0, seed=None) -> Tensor:
+    """In place: X = activation^count(dropout(X + bias[c], droprate)) on [N, C, ...] (inference only)."""
+    return dexts.bias_activation_nchw_(X, None if bias is None else bias.detach(), activation, count, droprate, seed)
 
 
 def spectral_inverse_linear_supported(r: int, cin: int, cout: int, modes: int) -> bool:
@@ -797,8 +833,9 @@ def conv3x3_resample_supported(cin: int) -> bool:
     return bool(_lib.load().spgt_conv3x3_resample_supported(int(cin)))
 
 
-def conv3x3_resample(X: Tensor, weight: Tensor, bias, size, pre_activation=None, post_activation=None) -> Tensor:
-    """3x3 convolution (padding 1) of a channels-last input with few channels, bias, activation, bilinear
+def conv3x3_resample(X: Tensor, weight: Tensor, bias, size, pre_activation=None, post_activation=None,
+                     droprate: float = 0.0, seed=None) -> Tensor:
+    """3x3 convolution (padding 1) of a channels-last input with few channels, bias, dropout, activation, bilinear
     align_corners resampling and a second activation in one pass: [N, H, W, Cin] -> [N, Cout, H', W'] (inference only)."""
     return dexts.conv3x3_resample(X.detach(), weight.detach(), None if bias is None else bias.detach(), size,
-                                  pre_activation, post_activation)
+                                  pre_activation, post_activation, droprate, seed)

@@ -12,7 +12,7 @@ import torch
 from torch import Tensor
 
 from ... import _lib
-from ..._lib import check, ptr, require_gpu_f32, stream_of
+from ..._lib import check, dropout_seed, ptr, require_gpu_f32, stream_of
 
 ACTIVATIONS = {"none": 0, "relu": 1, "silu": 2}
 RES_NONE, RES_BEFORE_ACT, RES_AFTER_ACT = 0, 1, 2
@@ -126,13 +126,6 @@ def fused_ffn_scalar(x: Tensor, weight1_kn: Tensor, bias1: Optional[Tensor], wei
 def encoder_tail_supported(attn_features: int, dim_hidden: int, ffn_hidden: int) -> bool:
     """True when fused_encoder_tail has a kernel for this shape."""
     return bool(_lib.load().spgt_encoder_tail_supported(int(attn_features), int(dim_hidden), int(ffn_hidden)))
-
-
-def dropout_seed(device) -> Tensor:
-    """Two 32-bit words from torch's generator of `device`, in device memory, for the kernels that apply dropout
-    themselves.  Drawn by a generator kernel: torch.manual_seed governs it, and inside a captured graph every
-    replay draws new words."""
-    return torch.randint(0, 2 ** 31 - 1, (2,), dtype=torch.int32, device=device)
 
 
 def _dropout_args(x: Tensor, fc_droprate: float, ffn_droprate: float, seed):

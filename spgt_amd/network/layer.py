@@ -142,8 +142,9 @@ class ConvResBlock2D(nn.Module):
         self.activation_layer = make_activation(activation)
 
     def fusable(self, X: Tensor) -> bool:
-        """Inference without dropout: the bias and the activation can ride in the caller's next kernel."""
-        return self.droprate == 0 and gpu_inference(X, *self.parameters())
+        """Inference: the bias, the dropout (the reference's F.dropout, on by default in inference too) and the
+        activation can ride in the caller's next kernel."""
+        return 0 <= self.droprate < 1 and gpu_inference(X, *self.parameters())
 
     def conv_raw(self, X: Tensor) -> Tensor:
         """The convolution without its bias (to be added by the kernel that consumes the result)."""
@@ -155,7 +156,7 @@ class ConvResBlock2D(nn.Module):
         """conv -> dropout -> activation, the activation applied 1 + extra_activations times."""
         if self.fusable(X):
             return bias_activation_nchw_(self.conv_raw(X), self.conv_layer.bias, activation_name(self.activation_layer),
-                                         1 + extra_activations)
+                                         1 + extra_activations, droprate=self.droprate)
         X = self.activation_layer(always_dropout(self.conv_layer(X), self.droprate))
         for _ in range(extra_activations):
             X = self.activation_layer(X)

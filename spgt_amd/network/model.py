@@ -98,8 +98,9 @@ class DownScaler2D(nn.Module):
             # few input channels: convolution, bias, activation, resampling and the scaler's activation in one
             # pass straight from the channels-last input; the full-resolution convolution output is never stored
             X = conv3x3_resample(X.contiguous(), c0.weight, c0.bias, self.resolution_size[1],
-                                 pre_activation=activation_name(self.conv0.activation_layer), post_activation=act)
-        elif fused and self.conv0.fusable(X):
+                                 pre_activation=activation_name(self.conv0.activation_layer), post_activation=act,
+                                 droprate=self.conv0.droprate)
+        elif fused and self.conv0.fusable(X) and self.conv0.droprate == 0:
             X = nhwc_to_nchw(X)
             # conv0's bias and activation, the resampling and the scaler's activation in one pass
             X = bilinear_resample(self.conv0.conv_raw(X), self.resolution_size[1], pre_bias=self.conv0.conv_layer.bias,
@@ -115,7 +116,8 @@ class DownScaler2D(nn.Module):
             return bilinear_resample_concat(
                 [X1, X2, self.conv3.conv_raw(X2)], self.resolution_size[2],
                 pre_biases=[None, None, self.conv3.conv_layer.bias], pre_flags=[0, 0, 1],
-                pre_activation=activation_name(self.conv3.activation_layer), post_activation=act)
+                pre_activation=activation_name(self.conv3.activation_layer), post_activation=act,
+                pre_droprate=self.conv3.droprate)
         X3 = self.conv3(X2)
         X = torch.cat([X1, X2, X3], dim=1)
         # the activation commutes with the permute, so the second resampling can write channels-last directly
@@ -136,8 +138,8 @@ class UpScaler2D(nn.Module):
 
     def can_defer_last_resample(self, X: Tensor) -> bool:
         """True when forward(X, defer_last_resample=True) is available: fused inference with one kind of activation."""
-        return (gpu_inference(X, *self.parameters()) and self.droprate == 0 and self.conv.fusable(X) and
-                type(self.conv.activation_layer) is type(self.activation_layer))
+        return (gpu_inference(X, *self.parameters()) and self.droprate == 0 and self.conv.droprate == 0 and
+                self.conv.fusable(X) and type(self.conv.activation_layer) is type(self.activation_layer))
 
     def _tap_weight_kn(self) -> Tensor:
         """The convolution's weight as [Cin, 9 * Cout], column (3 ky + kx) * Cout + co: the nine per-tap 1x1

@@ -228,6 +228,72 @@ def test_bilinear_adjoint_inner_product_at_the_model_sizes(gpu, hw, size):
     assert max_rel(b.permute(0, 3, 1, 2).cpu(), a.cpu()) < 1e-6
 
 
+def _kept_fraction_ok(keep, p, n_rows_tol=0.04):
+    assert keep.float().mean().item() == pytest.approx(1 - p, abs=4e-3)
+    flat = keep.reshape(-1, keep.shape[-1])
+    assert (flat[:, 1:] & flat[:, :-1]).float().mean().item() == pytest.approx((1 - p) ** 2, abs=6e-3)
+    assert (flat[1:] & flat[:-1]).float().mean().item() == pytest.approx((1 - p) ** 2, abs=6e-3)
+
+
+def test_down_scaler_kernels_with_dropout(gpu):
+    """ConvResBlock2D's dropout (conv -> dropout -> activation, network/layer.py:7-24, on in inference too) inside
+    the three kernels that consume a convolution's sums.  The masks are the library's own, so the test is of their
+    properties: a dropped sum is 0 and a kept one is scaled by 1 / (1 - p); kept fractions and neighbour
+    correlations fit independent draws; one seed repeats and another differs; and a resampling reads the same
+    decision for a source sample from every output that touches it (the resampled result equals the resampling of
+    the same-size result under the same seed)."""
+    g = torch.Generator().manual_seed(21)
+    p = 0.3
+    seed = torch.tensor([77, 99], dtype=torch.int32, device=gpu)
+    seed2 = torch.tensor([78, 99], dtype=torch.int32, device=gpu)
+    # bias + dropout + activation in place
+    x = torch.randn(3, 20, 37, 41, generator=g).to(gpu)
+    b = torch.randn(20, generator=g).to(gpu)
+    plain = dm.bias_activation_nchw_(x.clone(), b, None)
+    d = dm.bias_activation_nchw_(x.clone(), b, None, droprate=p, seed=seed)
+    keep = d != 0
+    assert torch.equal(d[keep], (plain / (1 - p))[keep]) or max_rel(d[keep].cpu(), (plain / (1 - p))[keep].cpu()) < 1e-6
+    _kept_fraction_ok(keep, p)
+    assert torch.equal(d, dm.bias_activation_nchw_(x.clone(), b, None, droprate=p, seed=seed))
+    other = dm.bias_activation_nchw_(x.clone(), b, None, droprate=p, seed=seed2) != 0
+    assert (keep != other).float().mean().item() == pytest.approx(2 * p * (1 - p), abs=6e-3)
+    assert torch.equal(dm.bias_activation_nchw_(x.clone(), b, "relu", 2, droprate=p, seed=seed), torch.relu(d))
+    assert not torch.equal(dm.bias_activation_nchw_(x.clone(), b, None, droprate=p),
+                           dm.bias_activation_nchw_(x.clone(), b, None, droprate=p))
+    # conv3x3 + bias + dropout + activation + resampling
+    xi = torch.randn(2, 45, 52, 1, generator=g).to(gpu)
+    w = torch.randn(24, 1, 3, 3, generator=g).to(gpu)
+    cb = torch.randn(24, generator=g).to(gpu)
+    same = dm.conv3x3_resample(xi, w, cb, (45, 52))
+    same_d = dm.conv3x3_resample(xi, w, cb, (45, 52), droprate=p, seed=seed)
+    keep = same_d != 0
+    assert max_rel(same_d[keep].cpu(), (same / (1 - p))[keep].cpu()) < 1e-6
+    _kept_fraction_ok(keep, p)
+    for size in ((31, 29), (70, 81)):
+        pre = dm.conv3x3_resample(xi, w, cb, (45, 52), pre_activation="silu", droprate=p, seed=seed)
+        got = dm.conv3x3_resample(xi, w, cb, size, pre_activation="silu", post_activation="relu", droprate=p, seed=seed)
+        want = torch.relu(dm.bilinear_align_corners(pre, size))
+        assert max_rel(got.cpu(), want.cpu()) < 1e-5
+    # concatenation whose last source is a convolution's sums without bias, dropout and activation
+    x1, x2 = torch.randn(2, 8, 33, 35, generator=g).to(gpu), torch.randn(2, 8, 33, 35, generator=g).to(gpu)
+    raw = torch.randn(2, 12, 33, 35, generator=g).to(gpu)
+    b3 = torch.randn(12, generator=g).to(gpu)
+    kw = dict(pre_biases=[None, None, b3], pre_flags=[0, 0, 1])
+    same = dm.bilinear_resample_concat([x1, x2, raw], (33, 35), **kw)
+    same_d = dm.bilinear_resample_concat([x1, x2, raw], (33, 35), pre_droprate=p, seed=seed, **kw)
+    assert torch.equal(same_d[..., :16], same[..., :16])
+    keep = same_d[..., 16:] != 0
+    assert max_rel(same_d[..., 16:][keep].cpu(), (same[..., 16:] / (1 - p))[keep].cpu()) < 1e-6
+    _kept_fraction_ok(keep.permute(0, 3, 1, 2), p)
+    pre = dm.bilinear_resample_concat([x1, x2, raw], (33, 35), pre_activation="silu", pre_droprate=p, seed=seed, **kw)
+    got = dm.bilinear_resample_concat([x1, x2, raw], (20, 23), pre_activation="silu", post_activation="relu",
+                                      pre_droprate=p, seed=seed, **kw)
+    want = torch.relu(dm.bilinear_align_corners(pre.permute(0, 3, 1, 2).contiguous(), (20, 23))).permute(0, 2, 3, 1)
+    assert max_rel(got.cpu(), want.cpu()) < 1e-5
+    with pytest.raises(Exception):
+        dm.bias_activation_nchw_(x.clone(), b, None, droprate=1.5)
+
+
 def test_bilinear_closed_forms(gpu):
     x = rnd(2, 3, 7, 9, seed=15).to(gpu)
     assert torch.equal(dm.bilinear_align_corners(x, (7, 9)), x)  # identity when sizes agree

@@ -326,6 +326,41 @@ def test_encoder_layer_with_drop_rates_stays_fused(gpu, fold):
         assert not torch.equal(outs[0], outs[1]) and not torch.equal(outs[1], outs[2])
 
 
+def test_model_with_the_reference_drop_rates(gpu):
+    """The whole model with the yaml's drop rates (0.05 on the down-scaler's blocks, on fc_layer's output and on the
+    feed-forward nets; the reference's dropouts are on in inference): the forward runs on the fused kernels with
+    their own masks.  Two forwards differ, torch.manual_seed repeats one (up to the convolution library's own
+    run-to-run rounding), and the mean over many forwards agrees with the mean over as many forwards of the same
+    model on the route that calls torch's F.dropout (taken when gradients are enabled) as well as two such means
+    agree with each other."""
+    p, i, _, meta = load_golden("galerkin_transformer_2d")
+    cfgd = dict(model_cfg(meta), drop_downscaler=0.05, drop_encoder_attn_fc=0.05, drop_encoder_ffn=0.05)
+    md = load_into(SM.Sp_GalerkinTransformer2D(cfgd), p, gpu)
+    x, pos, grid = i["x"].to(gpu), i["position"].to(gpu), i["grid"].to(gpu)
+    n = 300
+
+    def mean_of(fn):
+        acc = None
+        for _ in range(n):
+            y = fn().detach().double()
+            acc = y if acc is None else acc + y
+        return (acc / n).cpu()
+
+    with torch.no_grad():
+        torch.manual_seed(1)
+        a = md(x, pos, grid)
+        b = md(x, pos, grid)
+        torch.manual_seed(1)
+        again = md(x, pos, grid)
+        assert rel_l2(again.cpu(), a.cpu()) < 1e-5 and rel_l2(b.cpu(), a.cpu()) > 1e-4
+        fused = mean_of(lambda: md(x, pos, grid))
+    with torch.enable_grad():
+        ref1 = mean_of(lambda: md(x, pos, grid))
+        ref2 = mean_of(lambda: md(x, pos, grid))
+    noise = rel_l2(ref1, ref2)
+    assert rel_l2(fused, ref1) < 2.0 * noise + 1e-3, (rel_l2(fused, ref1), noise)
+
+
 def test_graphed_inference_replays_match_eager(gpu):
     """A HIP-graph capture of the whole forward: every replay, with eager work and synchronisation between
     replays and with fresh inputs, reproduces the eager forward.  The convolution library picks algorithms
