@@ -521,8 +521,7 @@ extern "C" int spgt_galerkin_attention_fused_backward(
         const size_t lds = (size_t)kBwdSub * 4 * D * D * sizeof(float);
         const void* fn = dp == 0 ? reinterpret_cast<const void*>(&qtg_partial_tm<0, 4, kBwdSub>)
                                  : reinterpret_cast<const void*>(&qtg_partial_tm<2, 4, kBwdSub>);
-        if (lds > 64 * 1024 &&
-            hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+        if (!allow_dynamic_lds(fn, lds))
             return fail(SPGT_ERR_LAUNCH, "galerkin_attention_fused_backward: pass 1 was refused its dynamic LDS size");
         if (dp == 0)
             hipLaunchKernelGGL((qtg_partial_tm<0, 4, kBwdSub>), grid1, dim3(256 * kBwdSub), lds, stream, Q, ld_in, pos,

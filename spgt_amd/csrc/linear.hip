@@ -1164,9 +1164,6 @@ void launch_linear(const float* x, int64_t ldx, const float* W, const float* bia
     const int gy = N / (32 * NCB);
     const int64_t tiles = ceil_div(T, (int64_t)TT);
     auto kernel = linear_tm_k<K, NCB, RES>;
-    static const hipError_t lds_opt_in = hipFuncSetAttribute(
-        reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
-    (void)lds_opt_in;
     const int tpw = pick_tiles_per_wg(tiles, gy, device_cu_count());
     const int total_wgs = (int)(ceil_div(tiles, (int64_t)tpw) * gy);
     // More than two workgroups per CU run in rounds of two (see pick_tiles_per_wg): asking for more
@@ -1174,6 +1171,7 @@ void launch_linear(const float* x, int64_t ldx, const float* W, const float* bia
     size_t lds_request = lds;
     if (total_wgs > 2 * device_cu_count()) lds_request = std::max<size_t>(lds, 72 * 1024);
     const dim3 grid((unsigned)(ceil_div(total_wgs, 8) * 8));  // whole rounds over the 8 XCDs
+    (void)allow_dynamic_lds(kernel, lds_request);
     hipLaunchKernelGGL(kernel, grid, dim3(256), lds_request, stream, x, ldx, W, N, bias, res, ldr, res_mode, act, x2, ldx2, W2,
                        r2, out, ldo, plane_cols, plane_stride, T, tpw, gy, total_wgs);
 }
@@ -1187,9 +1185,7 @@ void launch_linear_ws(const float* x, int64_t ldx, const float* W, const float* 
     // at least half of the CU's LDS so that no second workgroup joins
     const size_t lds = std::max<size_t>(LinearWs<K>::lds_bytes, 84 * 1024);
     auto kernel = linear_ws_k<K, RES, ACT>;
-    static const hipError_t lds_opt_in = hipFuncSetAttribute(
-        reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-    (void)lds_opt_in;
+    (void)allow_dynamic_lds(kernel, lds);
     hipLaunchKernelGGL(kernel, dim3(slots * gy), dim3(512), lds, stream, x, ldx, W, N, bias, res, ldr, res_mode, out,
                        ldo, plane_cols, plane_stride, T, gy);
 }
@@ -1213,9 +1209,7 @@ void launch_linear_resident(const float* x, int64_t ldx, const float* W, const f
 #define SPGT_RES_LAUNCH(ACT)                                                                                  \
     {                                                                                                         \
         auto kernel = linear_resident_k<NCB, ACT>;                                                            \
-        static const hipError_t lds_opt_in = hipFuncSetAttribute(                                             \
-            reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);    \
-        (void)lds_opt_in;                                                                                     \
+        (void)allow_dynamic_lds(kernel, lds);                                                                 \
         hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), lds, stream, x, ldx, W, bias, out, ldo, plane_cols, \
                            plane_stride, T);                                                                  \
     }
@@ -1366,12 +1360,6 @@ extern "C" int spgt_ffn_scalar_forward(const float* x, int64_t ldx, const float*
 
 namespace {
 
-// One-time (per process) permission for a kernel to use more than 64 KB of dynamic LDS.
-template <class K>
-void allow_tail_lds(K kernel) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
-}
-
 int dropout_args_ok(const uint32_t* seed, float p_fc, float p_ffn) {
     if (!(p_fc >= 0.f && p_fc < 1.f) || !(p_ffn >= 0.f && p_ffn < 1.f))
         return fail(SPGT_ERR_INVALID_ARGUMENT, "encoder_tail dropout: drop rates must lie in [0, 1)");
@@ -1409,8 +1397,8 @@ int encoder_tail_folded_common(const float* q, int64_t ld_q, const float* positi
     const int64_t per_wg = ceil_div(tiles, (int64_t)device_cu_count());
     const unsigned grid = (unsigned)ceil_div(tiles, per_wg);
     const size_t lds = std::max<size_t>(((size_t)32 * (128 + 4 + 132 + 260) + 512 + 256) * sizeof(float), 84 * 1024);
-    static const bool once = (allow_tail_lds(encoder_tail_k<128, true, false>), allow_tail_lds(encoder_tail_k<128, true, true>), true);
-    (void)once;
+    if (p_fc > 0.f || p_ffn > 0.f) (void)allow_dynamic_lds(encoder_tail_k<128, true, true>, lds);
+    else (void)allow_dynamic_lds(encoder_tail_k<128, true, false>, lds);
     if (p_fc > 0.f || p_ffn > 0.f)
         hipLaunchKernelGGL((encoder_tail_k<128, true, true>), dim3(grid), dim3(256), lds, stream, q, ld_q, x, folded_fc,
                            fc_bias, ffn1_weight_kn, ffn1_bias, ffn2_weight_kn, ffn2_bias, activation, out, (int64_t)B * S,
@@ -1484,18 +1472,16 @@ int encoder_tail_common(const float* attn_out, int64_t ld_attn, const float* x, 
     // attention tile + y1 + hidden tile + biases; at least half of the CU's LDS (one workgroup per CU anyway:
     // a wave uses most of its SIMD's registers)
     const size_t lds = std::max<size_t>(((size_t)32 * ((size_t)attn_features + 4 + 132 + 260) + 512 + 256) * sizeof(float), 84 * 1024);
-    static const bool once = (allow_tail_lds(encoder_tail_k<136, false, false>), allow_tail_lds(encoder_tail_k<128, false, false>),
-                              allow_tail_lds(encoder_tail_k<136, false, true>), allow_tail_lds(encoder_tail_k<128, false, true>), true);
-    (void)once;
     const bool drop = p_fc > 0.f || p_ffn > 0.f;
 #define SPGT_TAIL(K1, DROPF)                                                                                          \
+    (void)allow_dynamic_lds(encoder_tail_k<K1, false, DROPF>, lds);                                                    \
     hipLaunchKernelGGL((encoder_tail_k<K1, false, DROPF>), dim3(grid), dim3(256), lds, stream, attn_out, ld_attn, x,   \
                        fc_weight_kn, fc_bias, ffn1_weight_kn, ffn1_bias, ffn2_weight_kn, ffn2_bias, activation, out,   \
                        tokens, nullptr, nullptr, (int64_t)0, drop ? seed : nullptr, p_fc, p_ffn)
     if (attn_features == 136) {
-        if (drop) SPGT_TAIL(136, true); else SPGT_TAIL(136, false);
+        if (drop) { SPGT_TAIL(136, true); } else { SPGT_TAIL(136, false); }
     } else {
-        if (drop) SPGT_TAIL(128, true); else SPGT_TAIL(128, false);
+        if (drop) { SPGT_TAIL(128, true); } else { SPGT_TAIL(128, false); }
     }
 #undef SPGT_TAIL
     return check_launch("encoder_tail_forward");

@@ -230,9 +230,7 @@ void launch_projection(const float* x, const float* W, const float* bias, const 
     const int tpc = std::max(TT, ceil_div(ceil_div(S, per_b), TT) * TT);
     const dim3 grid(ceil_div(S, tpc), H / 4, B);
     auto kernel = projection_rrc_k<KC, DP, LN>;
-    if (lds > 64 * 1024)
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                  (int)lds);
+    (void)allow_dynamic_lds(kernel, lds);
     hipLaunchKernelGGL(kernel, grid, dim3(256), lds, stream, x, W, bias, lnw, lnb, pos, out, invsigma, S, H, eps, tpc);
 }
 

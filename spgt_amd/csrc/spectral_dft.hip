@@ -598,9 +598,7 @@ int dft_rows_check(const char* who, const void* a, const void* tab, const void* 
 
 template <typename K>
 void allow_lds(K kernel, size_t lds) {
-    if (lds > 64 * 1024)
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                  (int)lds);
+    (void)allow_dynamic_lds(kernel, lds);
 }
 
 }  // namespace
@@ -727,9 +725,7 @@ int launch_inverse_linear(const float* U, const float* table_operand, const floa
     const size_t lds = (size_t)4 * 32 * (CIN + 4) * sizeof(float);
 #define SPGT_SIL_LAUNCH(KSU)                                                                                        \
     {                                                                                                               \
-        if (lds > 64 * 1024 &&                                                                                      \
-            hipFuncSetAttribute(reinterpret_cast<const void*>(spectral_inverse_linear_k<ACT, KSU, CIN, COUT>),      \
-                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)               \
+        if (!allow_dynamic_lds(spectral_inverse_linear_k<ACT, KSU, CIN, COUT>, lds))                                \
             return fail(SPGT_ERR_LAUNCH, "spectral_inverse_linear: the kernel was refused its dynamic LDS size");    \
         hipLaunchKernelGGL((spectral_inverse_linear_k<ACT, KSU, CIN, COUT>), grid, dim3(256), lds, stream, U,       \
                            table_operand, x, weight_kn, bias, out, r, 2 * modes, (unsigned)pairs);                  \

@@ -2,8 +2,10 @@
 #include "spgt_host.h"
 
 #include <atomic>
+#include <mutex>
 #include <stdio.h>
 #include <string.h>
+#include <vector>
 
 namespace spgt {
 
@@ -33,6 +35,33 @@ int device_cu_count() {
         cached[dev].store(n, std::memory_order_relaxed);
     }
     return n;
+}
+
+bool allow_dynamic_lds(const void* fn, size_t bytes) {
+    if (bytes <= 64 * 1024) return true;
+    struct Granted {
+        int dev;
+        const void* fn;
+        size_t bytes;
+    };
+    static std::mutex mu;
+    static std::vector<Granted> granted;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return false;
+    std::lock_guard<std::mutex> lock(mu);
+    for (Granted& g : granted)
+        if (g.dev == dev && g.fn == fn) {
+            if (g.bytes >= bytes) return true;
+            if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes) != hipSuccess) return false;
+            g.bytes = bytes;
+            return true;
+        }
+    if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+    }
+    granted.push_back(Granted{dev, fn, bytes});
+    return true;
 }
 
 }  // namespace spgt
