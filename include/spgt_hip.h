@@ -559,6 +559,14 @@ int spgt_linear_weight_grad(const float* x, int64_t ldx, int64_t x_batch_stride,
                             int64_t grad_batch_stride, float* out, void* workspace, size_t workspace_bytes,
                             int64_t tokens, int in_features, int out_features, int batch, spgt_stream_t stream);
 
+/* out = residual + dropout(y, droprate) on [rows, cols] row-major (cols a multiple of 4; residual may be null; out
+ * may be y): the reference's F.dropout followed by the residual add (network/sp_layer.py:76, 100-103;
+ * network/layer.py:173) in one pass.  Keep decisions: a hash of (seed, site, row, column), kept values scaled by
+ * 1 / (1 - droprate); seed = two 32-bit words in device memory.  The same call on dL/dout with the forward's seed
+ * and site and no residual is the dropout's backward.  The masks are this library's own. */
+int spgt_dropout_add(const float* y, const float* residual, float* out, int64_t rows, int cols,
+                     const uint32_t* seed, float droprate, int site, spgt_stream_t stream);
+
 /* Instrumented variant of spgt_galerkin_attention_fused_forward for benchmarks (no reference
  * counterpart): enqueues the call `iterations` times back to back (no synchronisation between
  * them, as a caller's loop would), iteration i reading the input set i % n_sets and writing the

@@ -92,6 +92,7 @@ SIGNATURES = {
     "spgt_strided_copy_batch": (_i, [_p, _i, _p]),
     "spgt_linear_weight_grad_workspace_bytes": (_sz, [_i64, _i, _i, _i]),
     "spgt_linear_weight_grad": (_i, [_p, _i64, _i64, _p, _i64, _i64, _p, _p, _sz, _i64, _i, _i, _i, _p]),
+    "spgt_dropout_add": (_i, [_p, _p, _p, _i64, _i, _p, _f, _i, _p]),
     "spgt_galerkin_attention_fused_profile": (
         _i, [_p, _p, _p, _p, _i, _i64, _p, _p, _p, _p, _p, _f, _p, _p, _sz, _i, _i, _i, _i, _p, _i,
              ctypes.POINTER(ctypes.c_float)]),

@@ -252,6 +252,29 @@ __global__ __launch_bounds__(256, 1) void xtg_partial_wide_k(const float* __rest
     }
 }
 
+// out = residual + dropout(y) on [rows, cols] (cols a multiple of 4; residual may be null): the reference's
+// F.dropout followed by the residual add (network/sp_layer.py:76, 100-103; network/layer.py:173) in one pass, with
+// the keep decisions of dropout_site / dropout_apply (spgt_device.h).  The same call on a gradient with the
+// forward's seed is the backward of the dropout.  A thread takes 16-byte pieces, grid-stride.
+__global__ __launch_bounds__(256) void dropout_add_k(const float* __restrict__ y, const float* __restrict__ residual,
+                                                     float* __restrict__ out, int64_t pieces, int cols4,
+                                                     const uint32_t* __restrict__ seed, float p, uint32_t site) {
+    const int64_t stride = (int64_t)gridDim.x * 256;
+    for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < pieces; e += stride) {
+        const int64_t row = e / cols4;
+        const uint32_t col = 4u * (uint32_t)(e - row * cols4);
+        const DropoutSite ds = dropout_site(seed, site, row, p);
+        const float4 v = reinterpret_cast<const float4*>(y)[e];
+        float4 o = make_float4(dropout_apply(ds, col, v.x), dropout_apply(ds, col + 1, v.y),
+                               dropout_apply(ds, col + 2, v.z), dropout_apply(ds, col + 3, v.w));
+        if (residual) {
+            const float4 r = reinterpret_cast<const float4*>(residual)[e];
+            o.x += r.x, o.y += r.y, o.z += r.z, o.w += r.w;
+        }
+        reinterpret_cast<float4*>(out)[e] = o;
+    }
+}
+
 }  // namespace spgt
 
 using namespace spgt;
@@ -329,4 +352,20 @@ extern "C" int spgt_linear_weight_grad(const float* x, int64_t ldx, int64_t x_ba
     hipLaunchKernelGGL(tile_reduce, dim3(ceil_div((int)E, 256), batch), dim3(1024), 0, stream, partial, out, (int)E,
                        p.nchunk, 1.0f);
     return check_launch("linear_weight_grad");
+}
+
+extern "C" int spgt_dropout_add(const float* y, const float* residual, float* out, int64_t rows, int cols,
+                                const uint32_t* seed, float droprate, int site, hipStream_t stream) {
+    if (!y || !out || !seed) return fail(SPGT_ERR_INVALID_ARGUMENT, "dropout_add: null pointer argument");
+    if (rows < 0 || cols <= 0 || cols % 4 != 0)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "dropout_add: cols must be a positive multiple of 4");
+    if (!(droprate >= 0.f && droprate < 1.f)) return fail(SPGT_ERR_INVALID_ARGUMENT, "dropout_add: the rate must lie in [0, 1)");
+    if (!aligned16(y) || !aligned16(out) || (residual && !aligned16(residual)) || !aligned8(seed))
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "dropout_add: tensors must be 16-byte aligned, the seed 8-byte aligned");
+    if (rows == 0) return SPGT_OK;
+    const int64_t pieces = rows * (cols / 4);
+    const unsigned grid = (unsigned)std::min<int64_t>(ceil_div(pieces, (int64_t)256), (int64_t)16 * device_cu_count());
+    hipLaunchKernelGGL(dropout_add_k, dim3(grid), dim3(256), 0, stream, y, residual, out, pieces, cols / 4, seed, droprate,
+                       (uint32_t)site);
+    return check_launch("dropout_add");
 }

@@ -272,3 +272,26 @@ def linear_weight_grad_batched(x: Tensor, grads: Tensor):
         check(lib.spgt_linear_weight_grad(ptr(xr), ldx, 0, ptr(grads), N, T * N, ptr(out), ptr(ws), ws.numel(), T, K, N,
                                           P, stream_of(xr)))
     return out[:, :K * N].view(P, K, N), out[:, K * N:]
+
+
+def dropout_add(y: Tensor, residual: Optional[Tensor], droprate: float, seed: Tensor, site: int = 5) -> Tensor:
+    """residual + dropout(y, droprate) (or dropout(y) alone) on [..., C], C a multiple of 4, in one pass with the
+    library's own masks: a hash of (seed, site, row, column).  Called on a gradient with the forward's seed it is
+    the dropout's backward.  seed: two int32 words on y's device (_lib.dropout_seed)."""
+    require_gpu_f32("y", y)
+    C = y.shape[-1]
+    if C % 4:
+        raise ValueError("the last dimension must be a multiple of 4")
+    if residual is not None:
+        require_gpu_f32("residual", residual)
+        if residual.shape != y.shape:
+            raise ValueError("residual must have y's shape")
+    if not (seed.is_cuda and seed.device == y.device and seed.dtype == torch.int32 and seed.numel() >= 2):
+        raise ValueError("seed must be an int32 tensor of two words on y's device")
+    out = torch.empty_like(y)
+    if y.numel() == 0:
+        return out
+    with torch.cuda.device(y.device):
+        check(_lib.load().spgt_dropout_add(ptr(y), ptr(residual) if residual is not None else None, ptr(out),
+                                           y.numel() // C, C, ptr(seed), float(droprate), int(site), stream_of(y)))
+    return out

@@ -12,7 +12,8 @@ import torch.nn.functional as F
 from torch import Tensor, nn
 
 from ..extension.bind.datamove import bias_activation_nchw_
-from ..extension.bind.linear import (ffn_scalar_supported, fused_ffn_scalar, fused_linear, linear_supported,
+from .._lib import dropout_seed
+from ..extension.bind.linear import (dropout_add, ffn_scalar_supported, fused_ffn_scalar, fused_linear, linear_supported,
                                      linear_weight_grad)
 from .derived import derived, refreshes_derived, transposed_2d
 
@@ -132,6 +133,31 @@ def always_dropout(X: Tensor, p: float) -> Tensor:
     return F.dropout(X, p=p) if p > 0 else X
 
 
+class _DropoutAddFunction(torch.autograd.Function):
+    """residual + dropout(y) in one pass; the backward regenerates the mask from the saved seed words."""
+
+    @staticmethod
+    def forward(ctx, y, residual, p):
+        seed = dropout_seed(y.device)
+        ctx.seed, ctx.p, ctx.has_residual = seed, p, residual is not None
+        return dropout_add(y.contiguous(), None if residual is None else residual.contiguous(), p, seed)
+
+    @staticmethod
+    def backward(ctx, g):
+        dy = dropout_add(g.contiguous(), None, ctx.p, ctx.seed) if ctx.needs_input_grad[0] else None
+        return dy, (g if ctx.has_residual else None), None
+
+
+def always_dropout_add(Y: Tensor, residual: Tensor, p: float) -> Tensor:
+    """residual + F.dropout(Y, p) (the dropout always on, as in the reference), or the dropout alone without a
+    residual.  On the GPU in fp32 it is one kernel with the library's own masks, forward and backward."""
+    if p > 0 and Y.is_cuda and Y.dtype == torch.float32 and Y.shape[-1] % 4 == 0 and 0 < p < 1 and (
+            residual is None or (residual.is_cuda and residual.dtype == torch.float32 and residual.shape == Y.shape)):
+        return _DropoutAddFunction.apply(Y, residual, p)
+    Y = always_dropout(Y, p)
+    return Y if residual is None else residual + Y
+
+
 class ConvResBlock2D(nn.Module):
     """conv3x3 -> dropout -> activation on [N, C, H, W]."""
 
@@ -193,7 +219,6 @@ class FeedForward(nn.Module):
             Hd = self.activation_layer(linear_train(X, self.layer1))
             if self.droprate == 0:
                 return linear_train(Hd, self.layer2, residual)
-            Y = always_dropout(linear_train(Hd, self.layer2), self.droprate)
-            return Y if residual is None else residual + Y
+            return always_dropout_add(linear_train(Hd, self.layer2), residual, self.droprate)
         Y = always_dropout(self.layer2(self.activation_layer(self.layer1(X))), self.droprate)
         return Y if residual is None else residual + Y

@@ -34,7 +34,7 @@ from . import truncated_dft
 from ..extension.bind.linear import (encoder_tail_supported, fused_encoder_tail, fused_encoder_tail_folded,
                                      fused_linear, linear_supported, linear_weight_grad_batched)
 from .derived import derived, refreshes_derived
-from .layer import (FeedForward, activation_name, always_dropout, fused_linear_usable, gpu_inference,
+from .layer import (FeedForward, activation_name, always_dropout, always_dropout_add, fused_linear_usable, gpu_inference,
                     linear_train, linear_trainable, linear_weight_kn, make_activation)
 
 
@@ -220,8 +220,7 @@ class Sp_GalerkinAttention(nn.Module):
         if linear_trainable(X, self.fc_layer):
             if self.fc_droprate == 0:
                 return linear_train(X, self.fc_layer, residual)
-            Y = always_dropout(linear_train(X, self.fc_layer), self.fc_droprate)
-            return Y if residual is None else residual + Y
+            return always_dropout_add(linear_train(X, self.fc_layer), residual, self.fc_droprate)
         Y = always_dropout(self.fc_layer(X), self.fc_droprate)
         return Y if residual is None else residual + Y
 

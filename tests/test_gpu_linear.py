@@ -406,3 +406,41 @@ def test_linear_weight_grad_batched_through_the_c_abi(gpu):
         assert (out[j, :K * N].view(K, N).cpu().double() - x.double().t() @ g[j].double()).abs().max() < 2e-3
         assert (out[j, K * N:].cpu().double() - g[j].double().sum(0)).abs().max() < 2e-3
     assert lib.spgt_linear_weight_grad_workspace_bytes(T, K, 126, 1) == 0
+
+
+def test_dropout_add_and_its_backward(gpu):
+    """residual + dropout(y) in one pass (the reference's F.dropout + residual add, network/sp_layer.py:76, 100-103,
+    network/layer.py:173) with the library's own masks: kept values scaled by 1 / (1 - p), dropped ones leave the
+    residual untouched, the kept fraction fits, another seed gives another mask; the autograd function's gradient of
+    y carries the forward's mask and the residual's gradient is the incoming one."""
+    from spgt_amd._lib import dropout_seed
+    from spgt_amd.extension.bind.linear import dropout_add
+    from spgt_amd.network.layer import always_dropout_add
+    g = torch.Generator().manual_seed(3)
+    p = 0.2
+    y = torch.randn(5, 1000, 128, generator=g).to(gpu)
+    r = torch.randn(5, 1000, 128, generator=g).to(gpu)
+    seed = torch.tensor([5, 6], dtype=torch.int32, device=gpu)
+    d = dropout_add(y, None, p, seed)
+    keep = d != 0
+    assert torch.equal(d[keep], (y * (1.0 / (1.0 - p)))[keep])
+    assert keep.float().mean().item() == pytest.approx(1 - p, abs=3e-3)
+    assert (keep[..., 1:] & keep[..., :-1]).float().mean().item() == pytest.approx((1 - p) ** 2, abs=4e-3)
+    assert (keep[:, 1:] & keep[:, :-1]).float().mean().item() == pytest.approx((1 - p) ** 2, abs=4e-3)
+    o = dropout_add(y, r, p, seed)
+    assert torch.equal(o[~keep], r[~keep]) and torch.equal(o, d + r)
+    other = dropout_add(y, None, p, torch.tensor([5, 7], dtype=torch.int32, device=gpu)) != 0
+    assert (keep != other).float().mean().item() == pytest.approx(2 * p * (1 - p), abs=4e-3)
+    assert (keep != (dropout_add(y, None, p, seed, site=6) != 0)).float().mean().item() == pytest.approx(
+        2 * p * (1 - p), abs=4e-3)
+    yg, rg = y.clone().requires_grad_(True), r.clone().requires_grad_(True)
+    out = always_dropout_add(yg, rg, p)
+    go = torch.randn(5, 1000, 128, generator=g).to(gpu)
+    out.backward(go)
+    kept = (out.detach() - r) != 0
+    assert torch.equal(rg.grad, go)
+    assert torch.equal(yg.grad[kept], (go * (1.0 / (1.0 - p)))[kept]) and (yg.grad[~kept] == 0).all()
+    assert kept.float().mean().item() == pytest.approx(1 - p, abs=3e-3)
+    alone = always_dropout_add(yg, None, p)
+    assert alone.shape == y.shape and not torch.equal(alone, always_dropout_add(yg, None, p))
+    assert torch.equal(always_dropout_add(y, r, 0.0), y + r)
