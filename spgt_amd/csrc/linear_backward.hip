@@ -18,7 +18,9 @@ namespace spgt {
 // of NT * 32 columns.  MFMA 32x32x2 step kk contracts tokens 2 kk and 2 kk + 1 of the chunk (lane half = token),
 // A = x[t][k0 + lane % 32], B = g[t][n0 + 32 nt + lane % 32].  Operand batches of BK steps are requested one
 // batch ahead of the MFMAs that consume them.
-template <int NT>
+// TSPLIT (for K <= 32, where three of the four waves would have no rows): the four waves take the same 32 rows and
+// a quarter of the chunk's tokens each, and their tiles are added through LDS in a fixed order.
+template <int NT, bool TSPLIT>
 __global__ __launch_bounds__(256, 2) void xtg_partial_k(const float* __restrict__ X, int64_t ldx, int64_t x_batch,
                                                      const float* __restrict__ G, int64_t ldg, int64_t g_batch,
                                                      float* __restrict__ partial, int64_t T, int K, int N,
@@ -32,12 +34,15 @@ __global__ __launch_bounds__(256, 2) void xtg_partial_k(const float* __restrict_
     const int nchunk = gridDim.x;
     const int b = blockIdx.y / nstrip;
     const int strip = blockIdx.y - b * nstrip;
-    const int k0 = (blockIdx.z * 4 + wave) * 32;
+    const int k0 = TSPLIT ? 0 : (blockIdx.z * 4 + wave) * 32;
     const int n0 = strip * NT * 32;
     const int E = K * N + N;
-    if (k0 >= K) return;  // whole wave: no barrier follows
-    const int64_t t0 = (int64_t)chunk * tokens_per_chunk;
-    const int64_t t1 = min(T, t0 + tokens_per_chunk);
+    if (!TSPLIT && k0 >= K) return;  // whole wave: no barrier follows
+    const int64_t c0 = (int64_t)chunk * tokens_per_chunk;
+    const int64_t c1 = min(T, c0 + tokens_per_chunk);
+    const int64_t quarter = TSPLIT ? (tokens_per_chunk / 4) : 0;  // tokens_per_chunk is a multiple of 16
+    const int64_t t0 = TSPLIT ? min(c1, c0 + wave * quarter) : c0;
+    const int64_t t1 = TSPLIT ? min(c1, t0 + quarter) : c1;
     const int steps = (int)((t1 - t0 + 1) / 2);
     // clamped feature indices: rows past K and columns past N read valid memory and are masked to zero
     const bool kok = k0 + tk < K;
@@ -97,6 +102,28 @@ __global__ __launch_bounds__(256, 2) void xtg_partial_k(const float* __restrict_
         __builtin_amdgcn_sched_barrier(0);
     }
     float* out = partial + ((int64_t)b * nchunk + chunk) * E;
+    if constexpr (TSPLIT) {
+        // the four waves' tiles and column sums: waves 1..3 to LDS, wave 0 adds them in order
+        __shared__ float red[3][NT * 17 * 64];
+        if (wave > 0) {
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) red[wave - 1][(nt * 17 + r) * 64 + lane] = acc[nt][r];
+                red[wave - 1][(nt * 17 + 16) * 64 + lane] = colsum[nt];
+            }
+        }
+        __syncthreads();
+        if (wave > 0) return;
+#pragma unroll
+        for (int w = 0; w < 3; ++w)
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[nt][r] += red[w][(nt * 17 + r) * 64 + lane];
+                colsum[nt] += red[w][(nt * 17 + 16) * 64 + lane];
+            }
+    }
     // acc[nt][r] = dW[k0 + 8 (r / 4) + 4 kh + r % 4][n0 + 32 nt + tk]
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
@@ -338,16 +365,20 @@ extern "C" int spgt_linear_weight_grad(const float* x, int64_t ldx, int64_t x_ba
     float* partial = static_cast<float*>(workspace);
     const dim3 grid(p.nchunk, batch * p.nstrip, p.kz);
 #define SPGT_XTG(NT)                                                                                               \
-    hipLaunchKernelGGL((xtg_partial_k<NT>), grid, dim3(256), 0, stream, x, ldx, x_batch_stride, grad, ldg,         \
-                       grad_batch_stride, partial, tokens, in_features, out_features, p.tpc, p.nstrip)
+    if (in_features <= 32)                                                                                         \
+        hipLaunchKernelGGL((xtg_partial_k<NT, true>), grid, dim3(256), 0, stream, x, ldx, x_batch_stride, grad, ldg, \
+                           grad_batch_stride, partial, tokens, in_features, out_features, p.tpc, p.nstrip);        \
+    else                                                                                                           \
+        hipLaunchKernelGGL((xtg_partial_k<NT, false>), grid, dim3(256), 0, stream, x, ldx, x_batch_stride, grad, ldg, \
+                           grad_batch_stride, partial, tokens, in_features, out_features, p.tpc, p.nstrip)
     const bool wide_ok = p.wide && ldx % 4 == 0 && ldg % 4 == 0 && x_batch_stride % 4 == 0 &&
                          grad_batch_stride % 4 == 0 && aligned16(x) && aligned16(grad);
     if (wide_ok)
         hipLaunchKernelGGL(xtg_partial_wide_k, grid, dim3(256), 0, stream, x, ldx, x_batch_stride, grad, ldg,
                            grad_batch_stride, partial, tokens, in_features, out_features, p.tpc, p.nstrip);
-    else if (p.nt == 4) SPGT_XTG(4);
-    else if (p.nt == 2) SPGT_XTG(2);
-    else SPGT_XTG(1);
+    else if (p.nt == 4) { SPGT_XTG(4); }
+    else if (p.nt == 2) { SPGT_XTG(2); }
+    else { SPGT_XTG(1); }
 #undef SPGT_XTG
     hipLaunchKernelGGL(tile_reduce, dim3(ceil_div((int)E, 256), batch), dim3(1024), 0, stream, partial, out, (int)E,
                        p.nchunk, 1.0f);

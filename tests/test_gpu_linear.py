@@ -366,7 +366,7 @@ def test_hand_written_mfma_statements_match_the_compilers_intrinsic(gpu):
 
 
 @pytest.mark.parametrize("K,N", [(128, 128), (136, 128), (128, 256), (256, 128), (70, 36), (32, 4), (128, 384), (200, 128),
-                                 (132, 256)])
+                                 (132, 256), (1, 128), (20, 128), (32, 64)])
 @pytest.mark.parametrize("T", [1, 63, 1000, 65536 + 3])
 def test_linear_weight_grad(gpu, K, N, T):
     """dW = x^T g and db = column sums of g (the reference's projection backward, galerkin_attention.cu:41-46)
