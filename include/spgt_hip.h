@@ -370,6 +370,14 @@ int spgt_upsample_conv3x3_gather(const float* Z, const float* bias, float* dst, 
                                  int H_out, int W_out, int activation, int activation_count,
                                  spgt_stream_t stream);
 
+/* Backward of spgt_upsample_conv3x3_gather without bias and activation: the gradient of the per-tap products,
+ * dZ [N, H_in, W_in, 9, C] from grad [N, H_out, W_out, C] (the adjoint of shift + align_corners interpolation per tap,
+ * gathered per low-resolution pixel in a fixed order).  With it UpScaler2D's interpolate -> conv3x3
+ * (network/model.py:59-62) trains as a Linear on the low-resolution tokens plus this pair of kernels; the reference
+ * leaves the step to autograd of F.interpolate and the convolution library.  C a multiple of 4, 16-byte aligned. */
+int spgt_upsample_conv3x3_gather_adjoint(const float* grad, float* dZ, int N, int C, int H_in, int W_in, int H_out,
+                                         int W_out, spgt_stream_t stream);
+
 /* 1 when spgt_conv3x3_resample serves this number of input channels (1..4), else 0. */
 int spgt_conv3x3_resample_supported(int Cin);
 

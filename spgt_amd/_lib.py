@@ -56,6 +56,7 @@ SIGNATURES = {
     "spgt_bilinear_nhwc_affine": (_i, [_p, _p, _i, _i, _i, _i, _i, _i, _p, _p, _i, _p]),
     "spgt_bilinear_adjoint": (_i, [_p, _p, _i, _i, _i, _i, _i, _i, _i, _p]),
     "spgt_upsample_conv3x3_gather": (_i, [_p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p]),
+    "spgt_upsample_conv3x3_gather_adjoint": (_i, [_p, _p, _i, _i, _i, _i, _i, _i, _p]),
     "spgt_bilinear_resample_concat": (_i, [_p, _p, _p, _p, _i, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p]),
     "spgt_bilinear_resample_concat_dropout": (
         _i, [_p, _p, _p, _p, _i, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p, _f, _p]),

@@ -934,6 +934,63 @@ __global__ __launch_bounds__(256) void upsample_conv3x3_gather_k(const float* __
     *reinterpret_cast<float4*>(dst + (int64_t)pixel * C + 4 * q) = make_float4(acc[0], acc[1], acc[2], acc[3]);
 }
 
+// The adjoint of upsample_conv3x3_gather_k without bias and activation (its backward): the gradient of the per-tap
+// products, dZ[n, yl, xl, t, c] = sum over the output pixels (oy, ox) whose tap t = (ky, kx) reads the interpolated
+// image at (qy, qx) = (oy + ky - 1, ox + kx - 1) inside the image, of weight(qy -> yl) weight(qx -> xl) g[n, oy, ox, c],
+// with the weights of the resampling's adjoint (adjoint_weight).  A thread makes 4 channels of all nine taps of one
+// low-resolution pixel: it walks the window of output pixels one wider than the range of interpolated positions
+// that touch the pixel and adds each value into the taps that reach a touching position from it; fixed order.
+// g [N, Hout, Wout, C], dZ [N, Hin, Win, 9, C].  grid: ceil(N*Hin*Win*C/4 / 256) rounded up to a multiple of 8.
+__global__ __launch_bounds__(256) void upsample_conv3x3_gather_adjoint_k(const float* __restrict__ g,
+                                                                         float* __restrict__ dZ, int C4, int Hin,
+                                                                         int Win, int Hout, int Wout, float hscale,
+                                                                         float wscale, unsigned items) {
+    const unsigned f = (unsigned)xcd_contiguous_tile() * 256u + threadIdx.x;
+    if (f >= items) return;
+    const int q = (int)(f % (unsigned)C4);
+    const unsigned pix = f / (unsigned)C4;
+    const int xl = (int)(pix % (unsigned)Win);
+    const unsigned line = pix / (unsigned)Win;
+    const int yl = (int)(line % (unsigned)Hin);
+    const int64_t n = line / (unsigned)Hin;
+    const int64_t C = 4 * (int64_t)C4;
+    const AdjointRange ry = adjoint_range(hscale, yl, Hin, Hout), rx = adjoint_range(wscale, xl, Win, Wout);
+    float4 acc[9];
+#pragma unroll
+    for (int t = 0; t < 9; ++t) acc[t] = make_float4(0.f, 0.f, 0.f, 0.f);
+    const int y0 = max(ry.lo - 1, 0), y1 = min(ry.hi + 1, Hout - 1);
+    const int x0 = max(rx.lo - 1, 0), x1 = min(rx.hi + 1, Wout - 1);
+    for (int oy = y0; oy <= y1; ++oy) {
+        float hwk[3];
+#pragma unroll
+        for (int ky = 0; ky < 3; ++ky) {
+            const int qy = oy + ky - 1;
+            hwk[ky] = (qy >= 0 && qy < Hout) ? adjoint_weight(hscale, qy, yl, Hin) : 0.f;
+        }
+        const float* row = g + ((n * Hout + oy) * (int64_t)Wout) * C + 4 * q;
+        for (int ox = x0; ox <= x1; ++ox) {
+            float wwk[3];
+#pragma unroll
+            for (int kx = 0; kx < 3; ++kx) {
+                const int qx = ox + kx - 1;
+                wwk[kx] = (qx >= 0 && qx < Wout) ? adjoint_weight(wscale, qx, xl, Win) : 0.f;
+            }
+            const float4 v = *reinterpret_cast<const float4*>(row + (int64_t)ox * C);
+#pragma unroll
+            for (int ky = 0; ky < 3; ++ky)
+#pragma unroll
+                for (int kx = 0; kx < 3; ++kx) {
+                    const float w = hwk[ky] * wwk[kx];
+                    float4& a = acc[3 * ky + kx];
+                    a.x = fmaf(w, v.x, a.x), a.y = fmaf(w, v.y, a.y), a.z = fmaf(w, v.z, a.z), a.w = fmaf(w, v.w, a.w);
+                }
+        }
+    }
+    float* dst = dZ + (int64_t)pix * 9 * C + 4 * q;
+#pragma unroll
+    for (int t = 0; t < 9; ++t) *reinterpret_cast<float4*>(dst + t * C) = acc[t];
+}
+
 // DownScaler2D's first stage in one pass for a few input channels (network/model.py:30-33:
 // conv0 = ConvResBlock2D(in_dim, out_dim, 3x3, padding 1), interpolate to resolution_size[1],
 // activation): out[n, c, oy, ox] = post(bilinear(pre(conv3x3(x)[n, c] + bias[c]))).  The four
@@ -1313,6 +1370,27 @@ extern "C" int spgt_upsample_conv3x3_gather(const float* Z, const float* bias, f
                        C / 4, H_in, W_in, H_out, W_out, hscale, wscale, activation,
                        activation == SPGT_ACT_NONE ? 0 : activation_count, (unsigned)items);
     return check_launch("upsample_conv3x3_gather");
+}
+
+extern "C" int spgt_upsample_conv3x3_gather_adjoint(const float* grad, float* dZ, int N, int C, int H_in, int W_in,
+                                                    int H_out, int W_out, hipStream_t stream) {
+    if (!grad || !dZ) return fail(SPGT_ERR_INVALID_ARGUMENT, "upsample_conv3x3_gather_adjoint: null pointer argument");
+    if (N <= 0 || C <= 0 || H_in <= 0 || W_in <= 0 || H_out <= 0 || W_out <= 0)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "upsample_conv3x3_gather_adjoint: sizes must be positive");
+    if (C % 4 != 0) return fail(SPGT_ERR_INVALID_ARGUMENT, "upsample_conv3x3_gather_adjoint: C must be a multiple of 4");
+    if (!aligned16(grad) || !aligned16(dZ))
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "upsample_conv3x3_gather_adjoint: operands must be 16-byte aligned");
+    if (H_in > (1 << 23) || W_in > (1 << 23) || H_out > (1 << 23) || W_out > (1 << 23))
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "upsample_conv3x3_gather_adjoint: image sides above 2^23");
+    const int64_t items = (int64_t)N * H_in * W_in * (C / 4);
+    if (items > (int64_t)INT32_MAX - 2048 || (int64_t)N * H_out * W_out * (C / 4) > (int64_t)INT32_MAX)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "upsample_conv3x3_gather_adjoint: more than 2^33 elements on one side");
+    const int64_t blocks = ceil_div(ceil_div(items, (int64_t)256), (int64_t)8) * 8;
+    const float hscale = H_out > 1 ? (float)(H_in - 1) / (float)(H_out - 1) : 0.f;
+    const float wscale = W_out > 1 ? (float)(W_in - 1) / (float)(W_out - 1) : 0.f;
+    hipLaunchKernelGGL(spgt::upsample_conv3x3_gather_adjoint_k, dim3((unsigned)blocks), dim3(256), 0, stream, grad, dZ,
+                       C / 4, H_in, W_in, H_out, W_out, hscale, wscale, (unsigned)items);
+    return check_launch("upsample_conv3x3_gather_adjoint");
 }
 
 extern "C" int spgt_bilinear_nhwc_affine(const float* src, float* dst, int N, int C, int H_in, int W_in, int H_out,

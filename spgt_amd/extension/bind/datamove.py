@@ -415,6 +415,27 @@ def _upsample_conv3x3_gather(Z: Tensor, bias, size, activation=None, count: int 
     return out
 
 
+def _upsample_conv3x3_gather_adjoint(grad: Tensor, in_size) -> Tensor:
+    """The gradient of the per-tap products of upsample_conv3x3_gather (no bias, no activation): grad
+    [N, H', W', C] -> dZ [N, H, W, 9, C] with in_size = (H, W); C a multiple of 4."""
+    require_gpu_f32("grad", grad)
+    if grad.dim() != 4:
+        raise ValueError("grad must be [N, H', W', C]")
+    N, H_out, W_out, C = grad.shape
+    if C % 4:
+        raise ValueError("the channel count must be a multiple of 4")
+    H_in, W_in = (in_size, in_size) if isinstance(in_size, int) else tuple(in_size)
+    out = torch.empty((N, H_in, W_in, 9, C), dtype=grad.dtype, device=grad.device)
+    if out.numel() == 0:
+        return out
+    if grad.numel() == 0:
+        return out.zero_()
+    with torch.cuda.device(grad.device):
+        check(_lib.load().spgt_upsample_conv3x3_gather_adjoint(ptr(grad), ptr(out), N, C, H_in, W_in, H_out, W_out,
+                                                               stream_of(grad)))
+    return out
+
+
 def _bilinear_nhwc_affine(X: Tensor, size, extra: Tensor = None, weight_extra_kn: Tensor = None) -> Tensor:
     """Channels-last bilinear align_corners resampling X [N, H, W, C] -> [N, H', W', C] (C a multiple of 4), plus
     extra @ weight_extra_kn for extra [N, H', W', E] and weight_extra_kn [E, C], E <= 4: the few columns that a
@@ -588,6 +609,7 @@ dexts = SimpleNamespace(
     spectral_modes_compact=_spectral_modes_compact,
     bilinear_align_corners=_bilinear_align_corners,
     bilinear_adjoint=_bilinear_adjoint,
+    upsample_conv3x3_gather_adjoint=_upsample_conv3x3_gather_adjoint,
 )
 
 
@@ -717,6 +739,34 @@ class Bilinear_Nhwc_Function(torch.autograd.Function):
     @staticmethod
     def backward(ctx: Any, grad_out: Tensor):
         return dexts.bilinear_adjoint(grad_out.contiguous(), ctx.in_size, True), None
+
+
+class Upsample_Conv3x3_Gather_Function(torch.autograd.Function):
+    """conv3x3(interpolate(X)) + bias from the per-tap products Z [N, H, W, 9, C] of X at low resolution, no
+    activation; backward: the gather's adjoint for Z, a sum over the pixels for the bias."""
+
+    @staticmethod
+    def forward(ctx: Any, Z: Tensor, bias, size):
+        ctx.in_size = tuple(Z.shape[1:3])
+        ctx.has_bias = bias is not None
+        return dexts.upsample_conv3x3_gather(Z.contiguous(), bias, _pair(size), None, 0)
+
+    @staticmethod
+    def backward(ctx: Any, grad_out: Tensor):
+        g = grad_out.contiguous()
+        dZ = dexts.upsample_conv3x3_gather_adjoint(g, ctx.in_size) if ctx.needs_input_grad[0] else None
+        db = g.sum((0, 1, 2)) if ctx.has_bias and ctx.needs_input_grad[1] else None
+        return dZ, db, None
+
+
+def upsample_conv3x3_gather_train(Z: Tensor, bias, size) -> Tensor:
+    """conv3x3(interpolate(X)) + bias from the per-tap products Z of X, with an autograd graph (no activation)."""
+    return Upsample_Conv3x3_Gather_Function.apply(Z, bias, size)
+
+
+def upsample_conv3x3_gather_adjoint(grad: Tensor, in_size) -> Tensor:
+    """Gradient of the per-tap products of upsample_conv3x3_gather from the gradient of its (unactivated) result."""
+    return dexts.upsample_conv3x3_gather_adjoint(grad.detach(), in_size)
 
 
 def bilinear_adjoint(grad: Tensor, in_size, nhwc: bool = False) -> Tensor:

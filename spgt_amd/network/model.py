@@ -10,10 +10,11 @@ from torch import Tensor, nn
 from ..extension.bind.datamove import (bilinear_align_corners, bilinear_align_corners_nhwc, bilinear_nhwc_affine,
                                        bilinear_nhwc_train, bilinear_to_nhwc_train, bilinear_train,
                                        bilinear_resample, bilinear_resample_concat, conv3x3_resample,
-                                       conv3x3_resample_supported, upsample_conv3x3_gather)
+                                       conv3x3_resample_supported, upsample_conv3x3_gather,
+                                       upsample_conv3x3_gather_train)
 from ..extension.bind.linear import fused_linear, linear_supported
 from .derived import derived, refreshes_derived
-from .layer import ConvResBlock2D, activation_name, always_dropout, gpu_inference, make_activation
+from .layer import ConvResBlock2D, _LinearFunction, activation_name, always_dropout, gpu_inference, make_activation
 
 
 def get_resolution_size(r_large: int, r_small: int):
@@ -169,6 +170,19 @@ class UpScaler2D(nn.Module):
                 c.out_channels % 4 == 0 and linear_supported(c.in_channels, 9 * c.out_channels) and
                 size[0] * size[1] >= 2 * X.size(1) * X.size(2))
 
+    def _trains_mixing_before_resampling(self, X: Tensor) -> bool:
+        """True when the training route can take interpolate -> conv3x3 as Linear + gather (see forward)."""
+        c = self.conv.conv_layer
+        size = self.resolution_size[3]
+        size = (size, size) if isinstance(size, int) else tuple(size)
+        return (torch.is_grad_enabled() and X.is_cuda and X.dtype == torch.float32 and X.dim() == 4 and
+                c.weight.dtype == torch.float32 and c.kernel_size == (3, 3) and c.padding == (1, 1) and
+                c.stride == (1, 1) and c.dilation == (1, 1) and c.groups == 1 and c.padding_mode == "zeros" and
+                c.out_channels % 4 == 0 and linear_supported(c.in_channels, 9 * c.out_channels) and
+                size[0] * size[1] >= 2 * X.size(1) * X.size(2) and
+                # the adjoint walks the outputs around a source pixel: bounded up-sampling only
+                size[0] <= 3 * X.size(1) and size[1] <= 3 * X.size(2))
+
     def _mid_resolution_nhwc(self, X: Tensor) -> Tensor:
         """interpolate -> conv -> activation -> activation as [N, r_mid, r_mid, out_dim] channels-last."""
         N, H, W, C = X.shape
@@ -204,6 +218,19 @@ class UpScaler2D(nn.Module):
             else:
                 X = self.activation_layer(self.conv(X))
             return bilinear_resample(X, self.resolution_size[4], dst_nhwc=True)
+        if self._trains_mixing_before_resampling(X):
+            # under autograd the same reordering: the convolution's channel mixing as a Linear on the low-resolution
+            # tokens (forward, dX and dW on this package's kernels), then the nine-tap gather, whose backward is
+            # its adjoint; the library convolution (forward, data and weight gradient) and the first
+            # interpolation do not run
+            N, H, W, C = X.shape
+            c = self.conv.conv_layer
+            w_taps = c.weight.permute(2, 3, 0, 1).reshape(9 * c.out_channels, c.in_channels)  # rows (ky, kx, co)
+            Z = _LinearFunction.apply(X.reshape(N * H * W, C), w_taps, None, self._tap_weight_kn(), None)
+            Y = upsample_conv3x3_gather_train(Z.view(N, H, W, 9, c.out_channels), c.bias, self.resolution_size[3])
+            Y = self.conv.activation_layer(always_dropout(Y, self.conv.droprate))
+            Y = self.activation_layer(always_dropout(Y, self.droprate))
+            return bilinear_nhwc_train(Y, tuple(self.resolution_size[4]))
         X = resample(X.permute(0, 3, 1, 2), self.resolution_size[3])
         X = self.activation_layer(always_dropout(self.conv(X), self.droprate))
         return resample_to_nhwc(X, self.resolution_size[4])

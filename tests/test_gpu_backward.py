@@ -277,10 +277,11 @@ def test_decoder_regressor_trains_like_the_oracle(gpu, N, r, dim_x, hidden, m):
         assert max_rel(prm.grad.cpu().double(), po[name].grad) < TOL, name
 
 
-@pytest.mark.parametrize("r,r_attn,dim", [(41, 21, 32), (64, 32, 48)])
+@pytest.mark.parametrize("r,r_attn,dim", [(41, 21, 32), (64, 32, 48), (41, 21, 128)])
 def test_scalers_train_like_the_oracle(gpu, r, r_attn, dim):
     """DownScaler2D and UpScaler2D under autograd (resamplings forward and backward on this package's kernels, in
-    the planes and the channels-last layouts) against autograd through the oracle in float64."""
+    the planes and the channels-last layouts; at 128 channels the up-scaler's interpolate -> conv3x3 as a Linear on the
+    low-resolution tokens plus the nine-tap gather and its adjoint) against autograd through the oracle in float64."""
     from spgt_amd.network import model as M
     torch.manual_seed(37)
     sizes = M.get_resolution_size(r, r_attn)

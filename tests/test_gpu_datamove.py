@@ -294,6 +294,34 @@ def test_down_scaler_kernels_with_dropout(gpu):
         dm.bias_activation_nchw_(x.clone(), b, None, droprate=1.5)
 
 
+@pytest.mark.parametrize("N,hw,size,C", [(2, (9, 7), (13, 11), 8), (1, (21, 21), (29, 29), 128), (2, (5, 6), (5, 6), 4),
+                                          (1, (4, 4), (12, 11), 12), (1, (7, 1), (9, 1), 4)])
+def test_upsample_conv3x3_gather_adjoint(gpu, N, hw, size, C):
+    """The backward of the nine-tap gather (UpScaler2D's interpolate -> conv3x3 as a Linear on the low-resolution
+    tokens followed by a gather, network/model.py:59-62): against autograd in float64 through the oracle's
+    resampling and torch's convolution on per-tap identity weights, and as an autograd function with its bias."""
+    g = torch.Generator().manual_seed(31)
+    Z = torch.randn(N, *hw, 9, C, generator=g)
+    G = torch.randn(N, *size, C, generator=g)
+    bias = torch.randn(C, generator=g)
+    # oracle: out[n, y, x, c] = sum over taps of interp(Z_t)[y + ky - 1, x + kx - 1, c] (zero outside) + bias
+    Zo = Z.double().requires_grad_(True)
+    bo = bias.double().requires_grad_(True)
+    up = O.bilinear_align_corners(Zo.permute(0, 3, 4, 1, 2).reshape(N, 9 * C, *hw), size).view(N, 9, C, *size)
+    pad = torch.nn.functional.pad(up, (1, 1, 1, 1))
+    want = sum(pad[:, 3 * ky + kx, :, ky:ky + size[0], kx:kx + size[1]] for ky in range(3) for kx in range(3))
+    want = want.permute(0, 2, 3, 1) + bo
+    want.backward(G.double())
+    Zg = Z.to(gpu).requires_grad_(True)
+    bg = bias.to(gpu).requires_grad_(True)
+    got = dm.upsample_conv3x3_gather_train(Zg, bg, size)
+    assert max_rel(got.detach().cpu().double(), want.detach()) < 5e-5
+    got.backward(G.to(gpu))
+    assert max_rel(Zg.grad.cpu().double(), Zo.grad) < 5e-5
+    assert max_rel(bg.grad.cpu().double(), bo.grad) < 5e-5
+    assert torch.equal(dm.upsample_conv3x3_gather_adjoint(G.to(gpu), hw), Zg.grad)
+
+
 def test_bilinear_closed_forms(gpu):
     x = rnd(2, 3, 7, 9, seed=15).to(gpu)
     assert torch.equal(dm.bilinear_align_corners(x, (7, 9)), x)  # identity when sizes agree
