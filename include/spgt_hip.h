@@ -409,6 +409,20 @@ int spgt_bilinear_resample_concat_dropout(const float* const* srcs, const float*
                                           int post_activation, const uint32_t* seed, float droprate,
                                           spgt_stream_t stream);
 
+/* Backward of spgt_conv3x3_resample (its _dropout form with a seed) without post activation, for an input that
+ * needs no gradient (DownScaler2D's first stage on the model's input field, network/model.py:30-33): the gradients
+ * of the convolution's weight and bias from grad = dL/dP, P [N, Cout, H_out, W_out] = bilinear(pre(dropout(conv3x3(x)
+ * + bias))).  The full-resolution chain is formed again from x, weight, bias and the forward's seed; nothing of it
+ * was stored.  out [Cout][R], R = 4 * ceil((1 + 9 * Cin) / 4): per output channel the bias gradient, then the
+ * weight gradient [Cin][3][3], then padding.  The reference leaves this step to autograd (library convolution,
+ * dropout, activation and F.interpolate backward).  workspace: spgt_conv3x3_resample_backward_workspace_bytes
+ * (0 = unsupported shape), 16-byte aligned. */
+size_t spgt_conv3x3_resample_backward_workspace_bytes(int N, int Cin, int Cout, int H_in);
+int spgt_conv3x3_resample_backward(const float* x, const float* weight, const float* bias, const float* grad,
+                                   float* out, void* workspace, size_t workspace_bytes, int N, int Cin, int Cout,
+                                   int H_in, int W_in, int H_out, int W_out, int pre_activation, const uint32_t* seed,
+                                   float droprate, spgt_stream_t stream);
+
 /* The tail of ConvResBlock2D (network/layer.py:7-24) after a bias-free convolution, and the
  * scaler's own activation where it follows directly (network/model.py:61-62), in place:
  * x[n, c, :] = activation^activation_count(x[n, c, :] + bias[c]) on x [N, C, HW]; bias may be null,

@@ -10,6 +10,7 @@
 //       network/model.py:30, 36, 59, 63
 #include "spgt_device.h"
 #include "spgt_host.h"
+#include "spgt_kernels.h"
 
 // complex elements a zero-fill block writes, roughly (tuned on MI355X)
 #ifndef SPGT_ROWS_NB
@@ -1074,6 +1075,102 @@ __global__ __launch_bounds__(256) void conv3x3_resample_k(const float* __restric
     }
 }
 
+// Backward of conv3x3_resample_k for an input that needs no gradient (the model's input field): the gradients of
+// the convolution's weight and bias from the gradient of P = bilinear(pre(dropout(conv3x3(x) + bias))) (no post
+// activation).  Nothing of the full-resolution chain was stored by the forward, so every source position (y, x)
+// of a plane (n, c) is formed again: z = conv + bias, the dropout decision of the forward's seed, the derivative
+// of the pre activation at the dropped value, and the resampling's adjoint gathered from the gradient plane
+// (adjoint_range / adjoint_weight); gz = adjoint * act' * keep-scale then meets the 3x3 patch:
+//   db[c] += gz,   dW[c][ci][ky][kx] += gz * x[n, y + ky - 1, x + kx - 1, ci].
+// A workgroup takes one output channel and a run of image rows (rows of all images counted through), a wave a
+// row at a time, lanes along x; per-thread sums are reduced over the workgroup in a fixed order and written as one
+// record of R = 4 ceil((1 + 9 CIN) / 4) floats, [db, dW...]; tile_reduce adds the records of the runs.
+// x [N, H, W, CIN] channels-last, grad [N, Cout, Hout, Wout], partial [runs][Cout][R].
+// grid (runs, Cout), block (64, 4).
+template <int CIN>
+__global__ __launch_bounds__(256) void conv3x3_resample_backward_k(const float* __restrict__ x,
+                                                                   const float* __restrict__ weight,
+                                                                   const float* __restrict__ bias,
+                                                                   const float* __restrict__ grad,
+                                                                   float* __restrict__ partial, int N, int Cout, int H,
+                                                                   int W, int Hout, int Wout, float hscale, float wscale,
+                                                                   int pre_act, DropArgs drop, int rows_per_run) {
+    constexpr int NV = 1 + 9 * CIN;
+    constexpr int R = (NV + 3) / 4 * 4;
+    const int c = blockIdx.y;
+    const int run = blockIdx.x;
+    const int lane = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.y);
+    float wreg[9 * CIN];
+#pragma unroll
+    for (int k = 0; k < 9 * CIN; ++k) wreg[k] = weight[(int64_t)c * 9 * CIN + k];
+    const float b = bias ? bias[c] : 0.f;
+    float acc[NV];
+#pragma unroll
+    for (int k = 0; k < NV; ++k) acc[k] = 0.f;
+    const int64_t total_rows = (int64_t)N * H;
+    const int64_t g0 = (int64_t)run * rows_per_run, g1 = min(total_rows, g0 + rows_per_run);
+    for (int64_t gr = g0 + wave; gr < g1; gr += 4) {
+        const int64_t n = gr / H;
+        const int y = (int)(gr - n * H);
+        const AdjointRange ry = adjoint_range(hscale, y, H, Hout);
+        DropoutSite ds;
+        if (drop.seed) ds = dropout_site(drop.seed, kDropSiteConvResample, n * Cout + c, drop.p);
+        const float* gplane = grad + (n * Cout + c) * (int64_t)Hout * Wout;
+        for (int xx = lane; xx < W; xx += 64) {
+            const AdjointRange rx = adjoint_range(wscale, xx, W, Wout);
+            float gsum = 0.f;
+            for (int oy = ry.lo; oy <= ry.hi; ++oy) {
+                const float hw = adjoint_weight(hscale, oy, y, H);
+                for (int ox = rx.lo; ox <= rx.hi; ++ox)
+                    gsum = fmaf(hw * adjoint_weight(wscale, ox, xx, W), gplane[(int64_t)oy * Wout + ox], gsum);
+            }
+            float patch[9 * CIN];
+#pragma unroll
+            for (int ky = 0; ky < 3; ++ky)
+#pragma unroll
+                for (int kx = 0; kx < 3; ++kx) {
+                    const int yy = y + ky - 1, xq = xx + kx - 1;
+                    const bool in = yy >= 0 && yy < H && xq >= 0 && xq < W;
+                    const float* px = x + ((n * H + min(max(yy, 0), H - 1)) * (int64_t)W + min(max(xq, 0), W - 1)) * CIN;
+#pragma unroll
+                    for (int ci = 0; ci < CIN; ++ci) patch[ci * 9 + ky * 3 + kx] = in ? px[ci] : 0.f;
+                }
+            float z = b;
+#pragma unroll
+            for (int k = 0; k < 9 * CIN; ++k) z = fmaf(wreg[k], patch[k], z);
+            const bool keep = !drop.seed || dropout_keep(ds, (uint32_t)(y * W + xx));
+            const float keep_scale = !keep ? 0.f : (drop.seed ? ds.scale : 1.f);
+            const float zd = z * keep_scale;
+            float d = 1.f;
+            if (pre_act == SPGT_ACT_RELU) {
+                d = zd > 0.f ? 1.f : 0.f;
+            } else if (pre_act == SPGT_ACT_SILU) {
+                const float sg = __builtin_amdgcn_rcpf(1.f + __expf(-zd));
+                d = sg * (1.f + zd * (1.f - sg));
+            }
+            const float gz = gsum * d * keep_scale;
+            acc[0] += gz;
+#pragma unroll
+            for (int k = 0; k < 9 * CIN; ++k) acc[1 + k] = fmaf(gz, patch[k], acc[1 + k]);
+        }
+    }
+    // lanes of a wave, then the four waves, in a fixed order
+    __shared__ float red[4][R];
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+        float v = acc[k];
+#pragma unroll
+        for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, 64);
+        if (lane == 0) red[wave][k] = v;
+    }
+    __syncthreads();
+    const int tid = threadIdx.y * 64 + threadIdx.x;
+    if (tid < R)
+        partial[((int64_t)run * Cout + c) * R + tid] =
+            tid < NV ? (red[0][tid] + red[1][tid]) + (red[2][tid] + red[3][tid]) : 0.f;
+}
+
 // x[n, c, :] = act^count(x[n, c, :] + bias[c]) in place on [planes = N*C, HW]: the bias add and the
 // activation(s) that follow a bias-free convolution.  grid (chunks, planes), block 256.
 __global__ __launch_bounds__(256) void bias_activation_nchw_k(float* __restrict__ x, const float* __restrict__ bias,
@@ -1605,4 +1702,71 @@ extern "C" int spgt_conv3x3_resample_dropout(const float* x, const float* weight
     if (int rc = drop_args(seed, droprate, &drop)) return rc;
     return conv3x3_resample_common(x, weight, bias, out, N, Cin, Cout, H_in, W_in, H_out, W_out, pre_activation,
                                    post_activation, drop, stream);
+}
+
+namespace {
+
+struct ConvBackwardPlan {
+    int record, rows_per_run, runs;
+};
+
+ConvBackwardPlan conv_backward_plan(int N, int Cin, int H_in) {
+    ConvBackwardPlan p;
+    p.record = (1 + 9 * Cin + 3) / 4 * 4;
+    const int64_t rows = (int64_t)N * H_in;
+    // as many runs of rows as tile_reduce sums, at least four rows (one per wave) each
+    const int64_t runs = std::max<int64_t>(1, std::min<int64_t>(kReduceChains * kReduceMaxPerChain, rows / 4));
+    p.rows_per_run = (int)ceil_div(rows, runs);
+    p.runs = (int)ceil_div(rows, (int64_t)p.rows_per_run);
+    return p;
+}
+
+}  // namespace
+
+extern "C" size_t spgt_conv3x3_resample_backward_workspace_bytes(int N, int Cin, int Cout, int H_in) {
+    if (N <= 0 || Cout <= 0 || H_in <= 0 || !spgt_conv3x3_resample_supported(Cin)) return 0;
+    const ConvBackwardPlan p = conv_backward_plan(N, Cin, H_in);
+    return (size_t)p.runs * Cout * p.record * sizeof(float);
+}
+
+extern "C" int spgt_conv3x3_resample_backward(const float* x, const float* weight, const float* bias, const float* grad,
+                                              float* out, void* workspace, size_t workspace_bytes, int N, int Cin,
+                                              int Cout, int H_in, int W_in, int H_out, int W_out, int pre_activation,
+                                              const uint32_t* seed, float droprate, hipStream_t stream) {
+    if (!x || !weight || !grad || !out || !workspace)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "conv3x3_resample_backward: null pointer argument");
+    if (N <= 0 || Cout <= 0 || H_in <= 0 || W_in <= 0 || H_out <= 0 || W_out <= 0)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "conv3x3_resample_backward: sizes must be positive");
+    if (!spgt_conv3x3_resample_supported(Cin))
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "conv3x3_resample_backward: 1 to 4 input channels");
+    if (!act_known(pre_activation)) return fail(SPGT_ERR_INVALID_ARGUMENT, "conv3x3_resample_backward: unknown activation");
+    if (Cout > 65535 || (int64_t)H_in * W_in > UINT32_MAX || H_in > (1 << 23) || W_in > (1 << 23) ||
+        H_out > (1 << 23) || W_out > (1 << 23))
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "conv3x3_resample_backward: more than 65535 output channels or too large an image");
+    spgt::DropArgs drop;
+    if (int rc = drop_args(seed, droprate, &drop)) return rc;
+    const size_t need = spgt_conv3x3_resample_backward_workspace_bytes(N, Cin, Cout, H_in);
+    if (workspace_bytes < need || !aligned16(workspace))
+        return fail(SPGT_ERR_WORKSPACE, "conv3x3_resample_backward: workspace missing, misaligned or too small");
+    if (!aligned4(x) || !aligned4(weight) || !aligned4(grad) || !aligned16(out) || (bias && !aligned4(bias)))
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "conv3x3_resample_backward: out must be 16-byte aligned");
+    const ConvBackwardPlan p = conv_backward_plan(N, Cin, H_in);
+    const int64_t E = (int64_t)Cout * p.record;
+    if (E > INT32_MAX) return fail(SPGT_ERR_INVALID_ARGUMENT, "conv3x3_resample_backward: too many output channels");
+    const float hscale = H_out > 1 ? (float)(H_in - 1) / (float)(H_out - 1) : 0.f;
+    const float wscale = W_out > 1 ? (float)(W_in - 1) / (float)(W_out - 1) : 0.f;
+    float* partial = static_cast<float*>(workspace);
+    const dim3 grid(p.runs, Cout), block(64, 4);
+#define SPGT_CONVB(CI)                                                                                             \
+    hipLaunchKernelGGL(conv3x3_resample_backward_k<CI>, grid, block, 0, stream, x, weight, bias, grad, partial, N, \
+                       Cout, H_in, W_in, H_out, W_out, hscale, wscale, pre_activation, drop, p.rows_per_run)
+    switch (Cin) {
+        case 1: SPGT_CONVB(1); break;
+        case 2: SPGT_CONVB(2); break;
+        case 3: SPGT_CONVB(3); break;
+        default: SPGT_CONVB(4); break;
+    }
+#undef SPGT_CONVB
+    hipLaunchKernelGGL(tile_reduce, dim3(ceil_div((int)E, 256), 1), dim3(1024), 0, stream, partial, out, (int)E, p.runs, 1.0f);
+    return check_launch("conv3x3_resample_backward");
 }

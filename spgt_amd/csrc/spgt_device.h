@@ -232,8 +232,11 @@ __device__ __forceinline__ DropoutSite dropout_site(const uint32_t* seed, uint32
     d.scale = p <= 0.f ? 1.f : 1.f / (1.f - p);
     return d;
 }
+__device__ __forceinline__ bool dropout_keep(const DropoutSite& d, uint32_t column) {
+    return dropout_mix(d.base + column * 0x27d4eb2fu) >= d.threshold;
+}
 __device__ __forceinline__ float dropout_apply(const DropoutSite& d, uint32_t column, float v) {
-    return dropout_mix(d.base + column * 0x27d4eb2fu) >= d.threshold ? v * d.scale : 0.f;
+    return dropout_keep(d, column) ? v * d.scale : 0.f;
 }
 // Site numbers of the kernels that drop (distinct, so that one seed may serve a whole forward).
 enum { kDropSiteFc = 0, kDropSiteFfn = 1, kDropSiteBiasAct = 2, kDropSiteConvResample = 3, kDropSiteConcat = 4 };

@@ -587,8 +587,46 @@ def _conv3x3_resample(X: Tensor, weight: Tensor, bias, size, pre_activation=None
     return out
 
 
+def _conv3x3_resample_backward(X: Tensor, weight: Tensor, bias, grad: Tensor, pre_activation=None,
+                               droprate: float = 0.0, seed=None):
+    """(dW [Cout, Cin, 3, 3], db [Cout]) of P = interpolate(pre(dropout(conv3x3(X, weight, padding=1) + bias)))
+    from grad = dL/dP [N, Cout, H', W'], for X [N, H, W, Cin] (Cin <= 4) that needs no gradient.  The
+    full-resolution chain is formed again from X, the weights and the forward's seed."""
+    require_gpu_f32("X", X)
+    require_gpu_f32("weight", weight)
+    require_gpu_f32("grad", grad)
+    if X.dim() != 4 or weight.dim() != 4 or tuple(weight.shape[2:]) != (3, 3) or weight.shape[1] != X.shape[3]:
+        raise ValueError("X must be [N, H, W, Cin] and weight [Cout, Cin, 3, 3]")
+    if pre_activation not in _ACT:
+        raise ValueError("activation must be None, 'none', 'relu' or 'silu'")
+    N, H, W, Cin = X.shape
+    Cout = weight.shape[0]
+    if grad.dim() != 4 or grad.shape[0] != N or grad.shape[1] != Cout:
+        raise ValueError("grad must be [N, Cout, H', W']")
+    if bias is not None:
+        require_gpu_f32("bias", bias)
+    if droprate > 0 and seed is None:
+        raise ValueError("the backward needs the forward's seed")
+    droprate, seed = _drop_seed(X.device, droprate, seed)
+    H_out, W_out = grad.shape[2:]
+    lib = _lib.load()
+    nbytes = lib.spgt_conv3x3_resample_backward_workspace_bytes(N, Cin, Cout, H)
+    if nbytes == 0:
+        raise ValueError(f"unsupported shape: N={N} Cin={Cin} Cout={Cout} H={H}")
+    ws = workspace(nbytes, X)
+    R = (1 + 9 * Cin + 3) // 4 * 4
+    out = torch.empty((Cout, R), dtype=torch.float32, device=X.device)
+    with torch.cuda.device(X.device):
+        check(lib.spgt_conv3x3_resample_backward(ptr(X), ptr(weight), ptr(bias) if bias is not None else None, ptr(grad),
+                                                 ptr(out), ptr(ws), ws.numel(), N, Cin, Cout, H, W, H_out, W_out,
+                                                 _ACT[pre_activation], ptr(seed) if seed is not None else None, droprate,
+                                                 stream_of(X)))
+    return out[:, 1:1 + 9 * Cin].reshape(Cout, Cin, 3, 3), out[:, 0]
+
+
 dexts = SimpleNamespace(
     conv3x3_resample=_conv3x3_resample,
+    conv3x3_resample_backward=_conv3x3_resample_backward,
     spectral_inverse_linear_supported=_spectral_inverse_linear_supported,
     spectral_inverse_linear=_spectral_inverse_linear,
     denormalize_boundary=_denormalize_boundary,
@@ -767,6 +805,35 @@ def upsample_conv3x3_gather_train(Z: Tensor, bias, size) -> Tensor:
 def upsample_conv3x3_gather_adjoint(grad: Tensor, in_size) -> Tensor:
     """Gradient of the per-tap products of upsample_conv3x3_gather from the gradient of its (unactivated) result."""
     return dexts.upsample_conv3x3_gather_adjoint(grad.detach(), in_size)
+
+
+class Conv3x3_Resample_Function(torch.autograd.Function):
+    """interpolate(pre(dropout(conv3x3(X) + bias))) for a channels-last X [N, H, W, Cin <= 4] that needs no gradient
+    (the down-scaler's first stage on the model's input): one kernel forward, one backward that forms the
+    full-resolution chain again instead of storing it."""
+
+    @staticmethod
+    def forward(ctx: Any, X: Tensor, weight: Tensor, bias, size, pre_activation, droprate: float):
+        seed = dropout_seed(X.device) if droprate > 0 else None
+        ctx.save_for_backward(X, weight, bias if bias is not None else weight.new_empty(0))
+        ctx.has_bias, ctx.pre, ctx.droprate, ctx.seed = bias is not None, pre_activation, droprate, seed
+        return dexts.conv3x3_resample(X.contiguous(), weight.contiguous(), bias, _pair(size), pre_activation, None,
+                                      droprate, seed)
+
+    @staticmethod
+    def backward(ctx: Any, grad_out: Tensor):
+        X, weight, bias = ctx.saved_tensors
+        dW, db = dexts.conv3x3_resample_backward(X.contiguous(), weight.contiguous(), bias if ctx.has_bias else None,
+                                                 grad_out.contiguous(), ctx.pre, ctx.droprate, ctx.seed)
+        return None, dW, (db if ctx.has_bias else None), None, None, None
+
+
+def conv3x3_resample_train(X: Tensor, weight: Tensor, bias, size, pre_activation=None, droprate: float = 0.0) -> Tensor:
+    """interpolate(pre(dropout(conv3x3(X) + bias))) with an autograd graph for the weight and the bias; X itself
+    must not need a gradient."""
+    if X.requires_grad:
+        raise ValueError("conv3x3_resample_train has no gradient for its input")
+    return Conv3x3_Resample_Function.apply(X, weight, bias, size, pre_activation, float(droprate))
 
 
 def bilinear_adjoint(grad: Tensor, in_size, nhwc: bool = False) -> Tensor:

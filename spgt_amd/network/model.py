@@ -10,6 +10,7 @@ from torch import Tensor, nn
 from ..extension.bind.datamove import (bilinear_align_corners, bilinear_align_corners_nhwc, bilinear_nhwc_affine,
                                        bilinear_nhwc_train, bilinear_to_nhwc_train, bilinear_train,
                                        bilinear_resample, bilinear_resample_concat, conv3x3_resample,
+                                       conv3x3_resample_train,
                                        conv3x3_resample_supported, upsample_conv3x3_gather,
                                        upsample_conv3x3_gather_train)
 from ..extension.bind.linear import fused_linear, linear_supported
@@ -106,6 +107,15 @@ class DownScaler2D(nn.Module):
             # conv0's bias and activation, the resampling and the scaler's activation in one pass
             X = bilinear_resample(self.conv0.conv_raw(X), self.resolution_size[1], pre_bias=self.conv0.conv_layer.bias,
                                   pre_activation=activation_name(self.conv0.activation_layer), post_activation=act)
+        elif (torch.is_grad_enabled() and not X.requires_grad and X.is_cuda and X.dtype == torch.float32 and
+                X.dim() == 4 and c0.weight.dtype == torch.float32 and conv3x3_resample_supported(X.size(-1)) and
+                c0.kernel_size == (3, 3) and c0.padding == (1, 1) and c0.stride == (1, 1) and c0.dilation == (1, 1) and
+                c0.groups == 1 and c0.padding_mode == "zeros" and 0 <= self.conv0.droprate < 1):
+            # training on the model's input field: the same single pass forward, and a backward that forms the
+            # full-resolution convolution, dropout and activation again instead of storing them
+            X = self.activation_layer(conv3x3_resample_train(
+                X, c0.weight, c0.bias, self.resolution_size[1], activation_name(self.conv0.activation_layer),
+                self.conv0.droprate))
         else:
             X = self.activation_layer(resample(self.conv0(nhwc_to_nchw(X)), self.resolution_size[1]))
         X1 = self.conv1(X)

@@ -322,6 +322,48 @@ def test_upsample_conv3x3_gather_adjoint(gpu, N, hw, size, C):
     assert torch.equal(dm.upsample_conv3x3_gather_adjoint(G.to(gpu), hw), Zg.grad)
 
 
+@pytest.mark.parametrize("Cin,Cout,hw,size,act,p", [(1, 24, (45, 52), (31, 37), "relu", 0.0),
+                                                     (1, 128, (41, 41), (29, 29), "relu", 0.25),
+                                                     (3, 10, (20, 33), (27, 40), "silu", 0.25),
+                                                     (4, 6, (9, 8), (9, 8), None, 0.0), (2, 5, (12, 70), (5, 23), "silu", 0.0)])
+def test_conv3x3_resample_backward(gpu, Cin, Cout, hw, size, act, p):
+    """Weight and bias gradients of the down-scaler's first stage (conv3x3 -> dropout -> activation -> interpolate,
+    network/model.py:30-33 with network/layer.py:7-24) from the kernel that forms the full-resolution chain again,
+    against autograd in float64 through torch's convolution, the forward's own dropout mask (read off a same-size
+    forward with the same seed) and the oracle's resampling."""
+    g = torch.Generator().manual_seed(41)
+    N = 2
+    x = torch.randn(N, *hw, Cin, generator=g)
+    w = torch.randn(Cout, Cin, 3, 3, generator=g) / 3.0
+    b = torch.randn(Cout, generator=g)
+    G = torch.randn(N, Cout, *size, generator=g)
+    seed = torch.tensor([4242, 17], dtype=torch.int32, device=gpu)
+    xg, wg, bg = x.to(gpu), w.to(gpu), b.to(gpu)
+    wo, bo = w.double().requires_grad_(True), b.double().requires_grad_(True)
+    z = torch.nn.functional.conv2d(x.double().permute(0, 3, 1, 2), wo, bo, padding=1)
+    if p > 0:
+        plain = dm.conv3x3_resample(xg, wg, bg, hw)
+        dropped = dm.conv3x3_resample(xg, wg, bg, hw, droprate=p, seed=seed)
+        mask = ((dropped != 0) | (plain == 0)).cpu().double()
+        assert mask.mean().item() == pytest.approx(1 - p, abs=0.02)
+        z = z * mask / (1 - p)
+    a = z if act is None else (torch.relu(z) if act == "relu" else torch.nn.functional.silu(z))
+    want = O.bilinear_align_corners(a, size)
+    want.backward(G.double())
+    got = dm.conv3x3_resample(xg, wg, bg, size, pre_activation=act, droprate=p, seed=seed if p > 0 else None)
+    assert max_rel(got.cpu().double(), want.detach()) < 5e-5
+    dW, db = dm.dexts.conv3x3_resample_backward(xg, wg, bg, G.to(gpu), act, p, seed if p > 0 else None)
+    assert max_rel(dW.cpu().double(), wo.grad) < 1e-4
+    assert max_rel(db.cpu().double(), bo.grad) < 1e-4
+    # the autograd function (its own seed): gradients exist, and without dropout they are the ones above
+    wt, bt = wg.clone().requires_grad_(True), bg.clone().requires_grad_(True)
+    out = dm.conv3x3_resample_train(xg, wt, bt, size, act, p)
+    out.backward(G.to(gpu))
+    assert wt.grad.shape == w.shape and bt.grad.shape == b.shape
+    if p == 0:
+        assert torch.equal(wt.grad, dW) and torch.equal(bt.grad, db)
+
+
 def test_bilinear_closed_forms(gpu):
     x = rnd(2, 3, 7, 9, seed=15).to(gpu)
     assert torch.equal(dm.bilinear_align_corners(x, (7, 9)), x)  # identity when sizes agree
