@@ -417,7 +417,7 @@ int spgt_bilinear_resample_concat_dropout(const float* const* srcs, const float*
  * weight gradient [Cin][3][3], then padding.  The reference leaves this step to autograd (library convolution,
  * dropout, activation and F.interpolate backward).  workspace: spgt_conv3x3_resample_backward_workspace_bytes
  * (0 = unsupported shape), 16-byte aligned. */
-size_t spgt_conv3x3_resample_backward_workspace_bytes(int N, int Cin, int Cout, int H_in);
+size_t spgt_conv3x3_resample_backward_workspace_bytes(int N, int Cin, int Cout, int H_in, int W_in);
 int spgt_conv3x3_resample_backward(const float* x, const float* weight, const float* bias, const float* grad,
                                    float* out, void* workspace, size_t workspace_bytes, int N, int Cin, int Cout,
                                    int H_in, int W_in, int H_out, int W_out, int pre_activation, const uint32_t* seed,

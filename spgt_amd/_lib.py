@@ -74,7 +74,7 @@ SIGNATURES = {
     "spgt_conv3x3_resample_supported": (_i, [_i]),
     "spgt_conv3x3_resample": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p]),
     "spgt_conv3x3_resample_dropout": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p, _f, _p]),
-    "spgt_conv3x3_resample_backward_workspace_bytes": (_sz, [_i, _i, _i, _i]),
+    "spgt_conv3x3_resample_backward_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
     "spgt_conv3x3_resample_backward": (
         _i, [_p, _p, _p, _p, _p, _p, _sz, _i, _i, _i, _i, _i, _i, _i, _i, _p, _f, _p]),
     "spgt_linear_supported": (_i, [_i, _i]),

@@ -1171,6 +1171,137 @@ __global__ __launch_bounds__(256) void conv3x3_resample_backward_k(const float* 
             tid < NV ? (red[0][tid] + red[1][tid]) + (red[2][tid] + red[3][tid]) : 0.f;
 }
 
+// The adjoint's geometry along one axis as a table, for resamplings that do not enlarge (scale >= 1: a source
+// index is read by at most three outputs): entry i = (first output lo, weights of outputs lo, lo + 1, lo + 2; zero
+// where the output does not read i).  grid (ceil(in_size / 256)), block 256.
+__global__ __launch_bounds__(256) void adjoint_table_k(float scale, int in_size, int out_size, float4* __restrict__ table) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= in_size) return;
+    AdjointRange r = adjoint_range(scale, i, in_size, out_size);
+    // outputs at the range's start that touch i with weight zero are skipped: with scale >= 1 the source positions
+    // of the outputs are at least one apart, so at most three of them lie within one of i
+    while (r.lo < r.hi && adjoint_weight(scale, r.lo, i, in_size) == 0.f) ++r.lo;
+    float w[3];
+#pragma unroll
+    for (int k = 0; k < 3; ++k) w[k] = (r.lo + k <= r.hi) ? adjoint_weight(scale, r.lo + k, i, in_size) : 0.f;
+    table[i] = make_float4(__int_as_float(max(r.lo, 0)), w[0], w[1], w[2]);
+}
+
+// conv3x3_resample_backward_k with the adjoint's geometry read from adjoint_table_k's tables (rows: ytab, columns:
+// xtab) instead of being formed per position and channel, and CG output channels per workgroup, which share a
+// position's input patch, its nine gather weights and offsets.  Records as in conv3x3_resample_backward_k.
+// grid (runs, ceil(Cout / CG)), block (64, 4).
+template <int CIN, int CG>
+__global__ __launch_bounds__(256) void conv3x3_resample_backward_tab_k(
+    const float* __restrict__ x, const float* __restrict__ weight, const float* __restrict__ bias,
+    const float* __restrict__ grad, float* __restrict__ partial, int N, int Cout, int H, int W, int Hout, int Wout,
+    const float4* __restrict__ ytab, const float4* __restrict__ xtab, int pre_act, DropArgs drop, int rows_per_run) {
+    constexpr int NV = 1 + 9 * CIN;
+    constexpr int R = (NV + 3) / 4 * 4;
+    const int c0 = blockIdx.y * CG;
+    const int run = blockIdx.x;
+    const int lane = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.y);
+    float wreg[CG][9 * CIN], breg[CG], acc[CG][NV];
+#pragma unroll
+    for (int j = 0; j < CG; ++j) {
+        const int c = min(c0 + j, Cout - 1);  // channels past the end repeat the last and are not written
+#pragma unroll
+        for (int k = 0; k < 9 * CIN; ++k) wreg[j][k] = weight[(int64_t)c * 9 * CIN + k];
+        breg[j] = bias ? bias[c] : 0.f;
+#pragma unroll
+        for (int k = 0; k < NV; ++k) acc[j][k] = 0.f;
+    }
+    const int64_t total_rows = (int64_t)N * H;
+    const int64_t g0 = (int64_t)run * rows_per_run, g1 = min(total_rows, g0 + rows_per_run);
+    const int64_t oplane = (int64_t)Hout * Wout;
+    for (int64_t gr = g0 + wave; gr < g1; gr += 4) {
+        const int64_t n = gr / H;
+        const int y = (int)(gr - n * H);
+        const float4 ty = ytab[y];
+        const int ylo = __float_as_int(ty.x);
+        const float hw[3] = {ty.y, ty.z, ty.w};
+        int yoff[3];
+#pragma unroll
+        for (int a = 0; a < 3; ++a) yoff[a] = min(ylo + a, Hout - 1) * Wout;
+        DropoutSite ds[CG];
+        if (drop.seed) {
+#pragma unroll
+            for (int j = 0; j < CG; ++j)
+                ds[j] = dropout_site(drop.seed, kDropSiteConvResample, n * Cout + min(c0 + j, Cout - 1), drop.p);
+        }
+        const float* gimg = grad + (n * Cout + c0) * oplane;
+        for (int xx = lane; xx < W; xx += 64) {
+            const float4 tx = xtab[xx];
+            const int xlo = __float_as_int(tx.x);
+            const float ww[3] = {tx.y, tx.z, tx.w};
+            float wgt[9];
+            int off[9];
+#pragma unroll
+            for (int a = 0; a < 3; ++a)
+#pragma unroll
+                for (int e = 0; e < 3; ++e) {
+                    wgt[3 * a + e] = hw[a] * ww[e];
+                    off[3 * a + e] = yoff[a] + min(xlo + e, Wout - 1);
+                }
+            float patch[9 * CIN];
+#pragma unroll
+            for (int ky = 0; ky < 3; ++ky)
+#pragma unroll
+                for (int kx = 0; kx < 3; ++kx) {
+                    const int yy = y + ky - 1, xq = xx + kx - 1;
+                    const bool in = yy >= 0 && yy < H && xq >= 0 && xq < W;
+                    const float* px = x + ((n * H + min(max(yy, 0), H - 1)) * (int64_t)W + min(max(xq, 0), W - 1)) * CIN;
+#pragma unroll
+                    for (int ci = 0; ci < CIN; ++ci) patch[ci * 9 + ky * 3 + kx] = in ? px[ci] : 0.f;
+                }
+            const uint32_t e = (uint32_t)(y * W + xx);
+#pragma unroll
+            for (int j = 0; j < CG; ++j) {
+                const float* gp = gimg + min(j, Cout - 1 - c0) * oplane;
+                float gsum = 0.f;
+#pragma unroll
+                for (int t = 0; t < 9; ++t) gsum = fmaf(wgt[t], gp[off[t]], gsum);
+                float z = breg[j];
+#pragma unroll
+                for (int k = 0; k < 9 * CIN; ++k) z = fmaf(wreg[j][k], patch[k], z);
+                const bool keep = !drop.seed || dropout_keep(ds[j], e);
+                const float keep_scale = !keep ? 0.f : (drop.seed ? ds[j].scale : 1.f);
+                const float zd = z * keep_scale;
+                float d = 1.f;
+                if (pre_act == SPGT_ACT_RELU) {
+                    d = zd > 0.f ? 1.f : 0.f;
+                } else if (pre_act == SPGT_ACT_SILU) {
+                    const float sg = __builtin_amdgcn_rcpf(1.f + __expf(-zd));
+                    d = sg * (1.f + zd * (1.f - sg));
+                }
+                const float gz = gsum * d * keep_scale;
+                acc[j][0] += gz;
+#pragma unroll
+                for (int k = 0; k < 9 * CIN; ++k) acc[j][1 + k] = fmaf(gz, patch[k], acc[j][1 + k]);
+            }
+        }
+    }
+    __shared__ float red[4][CG * R];
+#pragma unroll
+    for (int j = 0; j < CG; ++j)
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            float v = acc[j][k];
+#pragma unroll
+            for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, 64);
+            if (lane == 0) red[wave][j * R + k] = v;
+        }
+    __syncthreads();
+    const int tid = threadIdx.y * 64 + threadIdx.x;
+    for (int i = tid; i < CG * R; i += 256) {
+        const int j = i / R, k = i - j * R;
+        if (c0 + j < Cout)
+            partial[((int64_t)run * Cout + c0 + j) * R + k] =
+                k < NV ? (red[0][i] + red[1][i]) + (red[2][i] + red[3][i]) : 0.f;
+    }
+}
+
 // x[n, c, :] = act^count(x[n, c, :] + bias[c]) in place on [planes = N*C, HW]: the bias add and the
 // activation(s) that follow a bias-free convolution.  grid (chunks, planes), block 256.
 __global__ __launch_bounds__(256) void bias_activation_nchw_k(float* __restrict__ x, const float* __restrict__ bias,
@@ -1723,10 +1854,11 @@ ConvBackwardPlan conv_backward_plan(int N, int Cin, int H_in) {
 
 }  // namespace
 
-extern "C" size_t spgt_conv3x3_resample_backward_workspace_bytes(int N, int Cin, int Cout, int H_in) {
-    if (N <= 0 || Cout <= 0 || H_in <= 0 || !spgt_conv3x3_resample_supported(Cin)) return 0;
+extern "C" size_t spgt_conv3x3_resample_backward_workspace_bytes(int N, int Cin, int Cout, int H_in, int W_in) {
+    if (N <= 0 || Cout <= 0 || H_in <= 0 || W_in <= 0 || !spgt_conv3x3_resample_supported(Cin)) return 0;
     const ConvBackwardPlan p = conv_backward_plan(N, Cin, H_in);
-    return (size_t)p.runs * Cout * p.record * sizeof(float);
+    // the records of the runs, then the two geometry tables (16 bytes per row and per column)
+    return (size_t)p.runs * Cout * p.record * sizeof(float) + ((size_t)H_in + W_in) * sizeof(float4);
 }
 
 extern "C" int spgt_conv3x3_resample_backward(const float* x, const float* weight, const float* bias, const float* grad,
@@ -1745,7 +1877,7 @@ extern "C" int spgt_conv3x3_resample_backward(const float* x, const float* weigh
         return fail(SPGT_ERR_INVALID_ARGUMENT, "conv3x3_resample_backward: more than 65535 output channels or too large an image");
     spgt::DropArgs drop;
     if (int rc = drop_args(seed, droprate, &drop)) return rc;
-    const size_t need = spgt_conv3x3_resample_backward_workspace_bytes(N, Cin, Cout, H_in);
+    const size_t need = spgt_conv3x3_resample_backward_workspace_bytes(N, Cin, Cout, H_in, W_in);
     if (workspace_bytes < need || !aligned16(workspace))
         return fail(SPGT_ERR_WORKSPACE, "conv3x3_resample_backward: workspace missing, misaligned or too small");
     if (!aligned4(x) || !aligned4(weight) || !aligned4(grad) || !aligned16(out) || (bias && !aligned4(bias)))
@@ -1757,16 +1889,36 @@ extern "C" int spgt_conv3x3_resample_backward(const float* x, const float* weigh
     const float wscale = W_out > 1 ? (float)(W_in - 1) / (float)(W_out - 1) : 0.f;
     float* partial = static_cast<float*>(workspace);
     const dim3 grid(p.runs, Cout), block(64, 4);
+    if (hscale >= 1.f && wscale >= 1.f) {
+        // not an enlargement: at most three outputs read a source index along an axis, and their weights come from
+        // two small tables made first
+        float4* ytab = reinterpret_cast<float4*>(partial + (size_t)p.runs * Cout * p.record);
+        float4* xtab = ytab + H_in;
+        hipLaunchKernelGGL(adjoint_table_k, dim3(ceil_div(H_in, 256)), dim3(256), 0, stream, hscale, H_in, H_out, ytab);
+        hipLaunchKernelGGL(adjoint_table_k, dim3(ceil_div(W_in, 256)), dim3(256), 0, stream, wscale, W_in, W_out, xtab);
+#define SPGT_CONVT(CI, CGR)                                                                                          \
+    hipLaunchKernelGGL((conv3x3_resample_backward_tab_k<CI, CGR>), dim3(p.runs, ceil_div(Cout, CGR)), block, 0, stream, \
+                       x, weight, bias, grad, partial, N, Cout, H_in, W_in, H_out, W_out, ytab, xtab, pre_activation,   \
+                       drop, p.rows_per_run)
+        switch (Cin) {
+            case 1: SPGT_CONVT(1, 4); break;
+            case 2: SPGT_CONVT(2, 2); break;
+            case 3: SPGT_CONVT(3, 2); break;
+            default: SPGT_CONVT(4, 1); break;
+        }
+#undef SPGT_CONVT
+    } else {
 #define SPGT_CONVB(CI)                                                                                             \
     hipLaunchKernelGGL(conv3x3_resample_backward_k<CI>, grid, block, 0, stream, x, weight, bias, grad, partial, N, \
                        Cout, H_in, W_in, H_out, W_out, hscale, wscale, pre_activation, drop, p.rows_per_run)
-    switch (Cin) {
-        case 1: SPGT_CONVB(1); break;
-        case 2: SPGT_CONVB(2); break;
-        case 3: SPGT_CONVB(3); break;
-        default: SPGT_CONVB(4); break;
-    }
+        switch (Cin) {
+            case 1: SPGT_CONVB(1); break;
+            case 2: SPGT_CONVB(2); break;
+            case 3: SPGT_CONVB(3); break;
+            default: SPGT_CONVB(4); break;
+        }
 #undef SPGT_CONVB
+    }
     hipLaunchKernelGGL(tile_reduce, dim3(ceil_div((int)E, 256), 1), dim3(1024), 0, stream, partial, out, (int)E, p.runs, 1.0f);
     return check_launch("conv3x3_resample_backward");
 }

@@ -610,7 +610,7 @@ def _conv3x3_resample_backward(X: Tensor, weight: Tensor, bias, grad: Tensor, pr
     droprate, seed = _drop_seed(X.device, droprate, seed)
     H_out, W_out = grad.shape[2:]
     lib = _lib.load()
-    nbytes = lib.spgt_conv3x3_resample_backward_workspace_bytes(N, Cin, Cout, H)
+    nbytes = lib.spgt_conv3x3_resample_backward_workspace_bytes(N, Cin, Cout, H, W)
     if nbytes == 0:
         raise ValueError(f"unsupported shape: N={N} Cin={Cin} Cout={Cout} H={H}")
     ws = workspace(nbytes, X)
