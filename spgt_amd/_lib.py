@@ -174,7 +174,29 @@ def ptr(t: torch.Tensor):
 
 
 def stream_of(t: torch.Tensor):
-    return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+    """torch's current stream on t's device, as the raw handle the C ABI takes."""
+    index = t.device.index
+    return ctypes.c_void_p(torch._C._cuda_getCurrentRawStream(torch.cuda.current_device() if index is None else index))
+
+
+class _NoGuard:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_GUARD = _NoGuard()
+
+
+def device_guard(device):
+    """`with device_guard(t.device):` makes t's device current for the launch inside, like torch.cuda.device, and
+    costs nothing when it is current already."""
+    index = device.index
+    if index is None or index == torch.cuda.current_device():
+        return _NO_GUARD
+    return torch.cuda.device(device)
 
 
 def workspace(nbytes: int, like: torch.Tensor) -> torch.Tensor:

@@ -32,7 +32,7 @@ def _batched_transpose(src: Tensor, batch_list: List[int], M_list: List[int], N_
     out = torch.empty(list(batch_list) + list(N_list) + list(M_list), dtype=src.dtype, device=src.device)
     if src.numel() == 0:
         return out
-    with torch.cuda.device(src.device):
+    with _lib.device_guard(src.device):
         check(_lib.load().spgt_batched_transpose(ptr(src), ptr(out), b, M, N, stream_of(src)))
     return out
 
@@ -48,7 +48,7 @@ def _transpose_gather_dual(src: Tensor, dim_list: List[int], H_all: int, W_all: 
     shape = [H_low, W_low] + list(dim_list)
     out1 = torch.empty(shape, dtype=src.dtype, device=src.device)
     out2 = torch.empty(shape, dtype=src.dtype, device=src.device)
-    with torch.cuda.device(src.device):
+    with _lib.device_guard(src.device):
         check(_lib.load().spgt_transpose_gather_dual(
             ptr(src), ptr(out1), ptr(out2), dim, H_all, W_all, H_low, W_low, H_base_1, W_base_1, H_base_2, W_base_2,
             stream_of(src)))
@@ -66,7 +66,7 @@ def _transpose_scatter_dual(src1: Tensor, src2: Tensor, dim_list: List[int], H_a
         if t.numel() != H_low * W_low * dim:
             raise ValueError(f"{name} has {t.numel()} elements, expected {H_low}x{W_low}x{dim}")
     out = torch.empty(list(dim_list) + [H_all, W_all], dtype=src1.dtype, device=src1.device)
-    with torch.cuda.device(src1.device):
+    with _lib.device_guard(src1.device):
         check(_lib.load().spgt_transpose_scatter_dual(
             ptr(src1), ptr(src2), ptr(out), dim, H_all, W_all, H_low, W_low, H_base_1, W_base_1, H_base_2, W_base_2,
             stream_of(src1)))
@@ -93,7 +93,7 @@ def _spectral_mode_contract(X_ft: Tensor, weight_1: Tensor, weight_2: Tensor, H_
     if ws[1].shape[3] != Cout:
         raise ValueError("weight_1 and weight_2 disagree on Cout")
     out = torch.empty((N, Cout, H_all, W_all), dtype=torch.complex64, device=X_ft.device)
-    with torch.cuda.device(X_ft.device):
+    with _lib.device_guard(X_ft.device):
         check(_lib.load().spgt_spectral_mode_contract(
             ptr(X_ft), ptr(ws[0]), ptr(ws[1]), ptr(out), N, Cin, Cout, H_all, W_all, H_low, W_low, H_base_1,
             W_base_1, H_base_2, W_base_2, stream_of(X_ft)))
@@ -117,7 +117,7 @@ def _spectral_modes_compact(Z: Tensor, weight_1: Tensor, weight_2: Tensor) -> Te
     if tuple(Z.shape) != (N, 2 * m_h, Cin, m_w):
         raise ValueError(f"Z has shape {tuple(Z.shape)}, expected {(N, 2 * m_h, Cin, m_w)}")
     out = torch.empty((N, 2 * m_h, Cout, m_w), dtype=torch.complex64, device=Z.device)
-    with torch.cuda.device(Z.device):
+    with _lib.device_guard(Z.device):
         check(_lib.load().spgt_spectral_modes_compact(ptr(Z), ptr(ws[0]), ptr(ws[1]), ptr(out), N, Cin, Cout, m_h,
                                                       m_w, stream_of(Z)))
     return out
@@ -135,7 +135,7 @@ def _bilinear_align_corners(X: Tensor, size) -> Tensor:
     planes = prod(lead)
     if planes == 0:
         return out
-    with torch.cuda.device(X.device):
+    with _lib.device_guard(X.device):
         check(_lib.load().spgt_bilinear_align_corners(ptr(X), ptr(out), planes, H_in, W_in, H_out, W_out,
                                                        stream_of(X)))
     return out
@@ -151,7 +151,7 @@ def _bilinear_align_corners_nhwc(X: Tensor, size) -> Tensor:
     out = torch.empty((N, H_out, W_out, C), dtype=X.dtype, device=X.device)
     if out.numel() == 0:
         return out
-    with torch.cuda.device(X.device):
+    with _lib.device_guard(X.device):
         check(_lib.load().spgt_bilinear_align_corners_nhwc(ptr(X), ptr(out), N, C, H_in, W_in, H_out, W_out,
                                                             stream_of(X)))
     return out
@@ -177,7 +177,7 @@ def _bilinear_adjoint(grad: Tensor, in_size, nhwc: bool = False) -> Tensor:
         return out
     if grad.numel() == 0:
         return out.zero_()
-    with torch.cuda.device(grad.device):
+    with _lib.device_guard(grad.device):
         check(_lib.load().spgt_bilinear_adjoint(ptr(grad), ptr(out), N, C, H_in, W_in, H_out, W_out, 1 if nhwc else 0,
                                                 stream_of(grad)))
     return out
@@ -252,7 +252,7 @@ def _truncated_dft_rows(src: Tensor, table: Tensor, inverse: bool, planar: bool 
     if rows == 0:
         return out
     fn = _lib.load().spgt_truncated_dft_rows_inverse if inverse else _lib.load().spgt_truncated_dft_rows_forward
-    with torch.cuda.device(src.device):
+    with _lib.device_guard(src.device):
         check(fn(ptr(src), ptr(padded), ptr(out), rows, r, C, m2 // 2, int(planar), stream_of(src)))
     return out
 
@@ -282,7 +282,7 @@ def _spectral_modes_middle(Y: Tensor, table_h: Tensor, table_h_inverse: Tensor, 
         return U
     lib = _lib.load()
     ws = workspace(lib.spgt_spectral_modes_middle_workspace_bytes(N, cout, m), Y)
-    with torch.cuda.device(Y.device):
+    with _lib.device_guard(Y.device):
         check(lib.spgt_spectral_modes_middle(ptr(Y), ptr(table_h), ptr(table_h_inverse), ptr(weight_1), ptr(weight_2),
                                              ptr(U), ptr(ws), ws.numel(), N, r, cin, cout, m, stream_of(Y)))
     return U
@@ -318,7 +318,7 @@ def _bilinear_resample(X: Tensor, size, src_nhwc: bool = False, dst_nhwc: bool =
         require_gpu_f32("pre_bias", pre_bias)
         if pre_bias.numel() != C:
             raise ValueError(f"pre_bias has {pre_bias.numel()} elements, expected {C}")
-    with torch.cuda.device(X.device):
+    with _lib.device_guard(X.device):
         check(_lib.load().spgt_bilinear_resample(ptr(X), ptr(pre_bias) if pre_bias is not None else None, ptr(out), N, C, H_in, W_in, H_out, W_out, int(src_nhwc),
                                                  int(dst_nhwc), _ACT[pre_activation], npre, _ACT[post_activation],
                                                  stream_of(X)))
@@ -377,7 +377,7 @@ def _bilinear_resample_concat(sources, size, pre_biases=None, pre_flags=None, pr
     flags = (ctypes.c_int * n)(*pre_flags)
     npre = int(pre_count) if _ACT[pre_activation] else 0
     pre_droprate, seed = _drop_seed(out.device, pre_droprate if any(pre_flags) else 0.0, seed)
-    with torch.cuda.device(out.device):
+    with _lib.device_guard(out.device):
         if seed is None:
             check(_lib.load().spgt_bilinear_resample_concat(srcs, biases, chans, flags, n, ptr(out), N, H_in, W_in,
                                                             H_out, W_out, _ACT[pre_activation], npre,
@@ -408,7 +408,7 @@ def _upsample_conv3x3_gather(Z: Tensor, bias, size, activation=None, count: int 
     out = torch.empty((N, H_out, W_out, C), dtype=Z.dtype, device=Z.device)
     if out.numel() == 0:
         return out
-    with torch.cuda.device(Z.device):
+    with _lib.device_guard(Z.device):
         check(_lib.load().spgt_upsample_conv3x3_gather(ptr(Z), ptr(bias) if bias is not None else None, ptr(out), N, C,
                                                        H_in, W_in, H_out, W_out, _ACT[activation], int(count),
                                                        stream_of(Z)))
@@ -430,7 +430,7 @@ def _upsample_conv3x3_gather_adjoint(grad: Tensor, in_size) -> Tensor:
         return out
     if grad.numel() == 0:
         return out.zero_()
-    with torch.cuda.device(grad.device):
+    with _lib.device_guard(grad.device):
         check(_lib.load().spgt_upsample_conv3x3_gather_adjoint(ptr(grad), ptr(out), N, C, H_in, W_in, H_out, W_out,
                                                                stream_of(grad)))
     return out
@@ -457,7 +457,7 @@ def _bilinear_nhwc_affine(X: Tensor, size, extra: Tensor = None, weight_extra_kn
     out = torch.empty((N, H_out, W_out, C), dtype=X.dtype, device=X.device)
     if out.numel() == 0:
         return out
-    with torch.cuda.device(X.device):
+    with _lib.device_guard(X.device):
         check(_lib.load().spgt_bilinear_nhwc_affine(ptr(X), ptr(out), N, C, H_in, W_in, H_out, W_out,
                                                     ptr(extra) if E else None, ptr(weight_extra_kn) if E else None, E,
                                                     stream_of(X)))
@@ -480,7 +480,7 @@ def _bias_activation_nchw_(X: Tensor, bias, activation=None, count: int = 1, dro
     if X.numel() == 0:
         return X
     droprate, seed = _drop_seed(X.device, droprate, seed)
-    with torch.cuda.device(X.device):
+    with _lib.device_guard(X.device):
         if seed is None:
             check(_lib.load().spgt_bias_activation_nchw(ptr(X), ptr(bias) if bias is not None else None, N, C, HW,
                                                         _ACT[activation], int(count), stream_of(X)))
@@ -507,7 +507,7 @@ def _denormalize_boundary(X: Tensor, scale: Tensor, shift: Tensor, zero_boundary
     out = torch.empty_like(X)
     if X.numel() == 0:
         return out
-    with torch.cuda.device(X.device):
+    with _lib.device_guard(X.device):
         check(_lib.load().spgt_denormalize_boundary(ptr(X), ptr(scale), ptr(shift), int(scale.numel() > 1), ptr(out),
                                                     N, H, W, C, int(bool(zero_boundary)), stream_of(X)))
     return out
@@ -546,7 +546,7 @@ def _spectral_inverse_linear(U: Tensor, table_operand: Tensor, X: Tensor, weight
     out = torch.empty((N, r, r, cout), dtype=X.dtype, device=X.device)
     if X.numel() == 0:
         return out
-    with torch.cuda.device(X.device):
+    with _lib.device_guard(X.device):
         check(_lib.load().spgt_spectral_inverse_linear(ptr(U), ptr(table_operand), ptr(X), ptr(weight_kn),
                                                        ptr(bias) if bias is not None else None, _ACT[activation],
                                                        ptr(out), N * r, r, cin, cout, modes, stream_of(X)))
@@ -574,7 +574,7 @@ def _conv3x3_resample(X: Tensor, weight: Tensor, bias, size, pre_activation=None
     if out.numel() == 0:
         return out
     droprate, seed = _drop_seed(X.device, droprate, seed)
-    with torch.cuda.device(X.device):
+    with _lib.device_guard(X.device):
         if seed is None:
             check(_lib.load().spgt_conv3x3_resample(ptr(X), ptr(weight), ptr(bias) if bias is not None else None,
                                                     ptr(out), N, Cin, Cout, H, W, H_out, W_out, _ACT[pre_activation],
@@ -616,7 +616,7 @@ def _conv3x3_resample_backward(X: Tensor, weight: Tensor, bias, grad: Tensor, pr
     ws = workspace(nbytes, X)
     R = (1 + 9 * Cin + 3) // 4 * 4
     out = torch.empty((Cout, R), dtype=torch.float32, device=X.device)
-    with torch.cuda.device(X.device):
+    with _lib.device_guard(X.device):
         check(lib.spgt_conv3x3_resample_backward(ptr(X), ptr(weight), ptr(bias) if bias is not None else None, ptr(grad),
                                                  ptr(out), ptr(ws), ws.numel(), N, Cin, Cout, H, W, H_out, W_out,
                                                  _ACT[pre_activation], ptr(seed) if seed is not None else None, droprate,

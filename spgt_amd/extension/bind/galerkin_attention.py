@@ -44,7 +44,7 @@ def _projection_forward(input: Tensor, weight: Tensor, bias: Tensor, position: T
     (reference: extension/bind/galerkin_attention.cu:9-24)."""
     _check_projection_args(input, weight, bias, position, seqlen, dim_hidden, num_head, dim_head, dim_position, batch)
     out = torch.empty((batch, num_head, dim_position + dim_head, seqlen), dtype=input.dtype, device=input.device)
-    with torch.cuda.device(input.device):
+    with _lib.device_guard(input.device):
         check(_lib.load().spgt_multihead_projection_with_position_rrc_forward(
             ptr(input), ptr(weight), ptr(bias), ptr(position) if dim_position else None, ptr(out), seqlen, dim_hidden,
             num_head, dim_head, dim_position, batch, stream_of(input)))
@@ -63,7 +63,7 @@ def _projection_layernorm_forward(input: Tensor, weight: Tensor, bias: Tensor, l
         raise ValueError("LayerNorm weight and bias must be [num_head, dim_head]")
     hat_ln = torch.empty((batch, num_head, dim_position + dim_head, seqlen), dtype=input.dtype, device=input.device)
     invsigma = torch.empty((batch, num_head, seqlen), dtype=input.dtype, device=input.device)
-    with torch.cuda.device(input.device):
+    with _lib.device_guard(input.device):
         check(_lib.load().spgt_multihead_projection_layernorm_with_position_rrc_forward(
             ptr(input), ptr(weight), ptr(bias), ptr(lnw), ptr(lnb), float(norm_eps),
             ptr(position) if dim_position else None, ptr(hat_ln), ptr(invsigma), seqlen, dim_hidden, num_head,
@@ -86,7 +86,7 @@ def _attention_cccr_forward(Q: Tensor, K: Tensor, V: Tensor, batch: int, num_hea
         raise ValueError(f"unsupported attention shape: batch={batch} num_head={num_head} d_posk={d_posk} "
                          f"seqlen={seqlen} (d_posk must be 32 or 34)")
     ws = workspace(nbytes, Q)
-    with torch.cuda.device(Q.device):
+    with _lib.device_guard(Q.device):
         check(lib.spgt_galerkin_attention_cccr_forward(
             ptr(Q), ptr(K), ptr(V), ptr(out), ptr(ws), ws.numel(), batch, num_head, d_posk, seqlen, stream_of(Q)))
     return out
@@ -110,7 +110,7 @@ def _attention_cccr_backward(grad_out: Tensor, Q: Tensor, K: Tensor, V: Tensor, 
     if nbytes == 0:
         raise ValueError("unsupported attention shape (d_posk must be 32 or 34)")
     ws = workspace(nbytes, Q)
-    with torch.cuda.device(Q.device):
+    with _lib.device_guard(Q.device):
         check(lib.spgt_galerkin_attention_cccr_backward(
             ptr(grad_out), ptr(Q), ptr(K), ptr(V), ptr(dQ), ptr(dK), ptr(dV), ptr(ws), ws.numel(), batch, num_head,
             d_posk, seqlen, stream_of(Q)))
@@ -126,7 +126,7 @@ def _heads_feature_to_token_major(src: Tensor, batch: int, num_head: int, dim_po
     if tuple(src.shape) != (batch, num_head, dim_position + dim_head, seqlen):
         raise ValueError(f"src has shape {tuple(src.shape)}")
     dst = torch.empty((batch, seqlen, num_head * dim_head), dtype=src.dtype, device=src.device)
-    with torch.cuda.device(src.device):
+    with _lib.device_guard(src.device):
         check(_lib.load().spgt_heads_feature_to_token_major(ptr(src), ptr(dst), batch, num_head, dim_position,
                                                             dim_head, seqlen, stream_of(src)))
     return dst
@@ -197,7 +197,7 @@ def _projection_layernorm_backward(grad_ln: Tensor, input: Tensor, weight: Tenso
     grad_lnw = torch.empty((num_head, dim_head), dtype=pre.dtype, device=pre.device)
     grad_lnb = torch.empty((num_head, dim_head), dtype=pre.dtype, device=pre.device)
     ws = workspace(lib.spgt_layernorm_heads_backward_workspace_bytes(tokens, num_head), pre)
-    with torch.cuda.device(pre.device):
+    with _lib.device_guard(pre.device):
         check(lib.spgt_layernorm_heads_backward(
             ptr(pre), ptr(g), ptr(lnw), float(norm_eps), ptr(grad_pre), ptr(grad_lnw), ptr(grad_lnb), ptr(ws),
             ws.numel(), tokens, num_head, stream_of(pre)))
@@ -225,7 +225,7 @@ def _batched_skinny_gemm(A: Tensor, B: Tensor, alpha: float) -> Tensor:
         return C.zero_()
     lib = _lib.load()
     ws = workspace(lib.spgt_batched_skinny_gemm_workspace_bytes(M, N, K, batch), A)
-    with torch.cuda.device(A.device):
+    with _lib.device_guard(A.device):
         check(lib.spgt_batched_skinny_gemm(
             ptr(A), ptr(B), ptr(C), float(alpha), M, N, K, M * K, K * N, M * N, GEMM_ORDER["RRR"], batch,
             ptr(ws), ws.numel(), stream_of(A)))
@@ -271,7 +271,7 @@ def _attention_fused_forward(QKV_or_Q, K, V, position, ln_weight_K, ln_bias_K, l
     ktv = torch.empty((B, H, D, D), dtype=torch.float32, device=Q.device)
     ws = workspace(lib.spgt_galerkin_attention_fused_workspace_bytes(B, S, H, dim_position), Q)
     pos_ptr = ptr(position) if dim_position == 2 else None
-    with torch.cuda.device(Q.device):
+    with _lib.device_guard(Q.device):
         check(lib.spgt_galerkin_attention_fused_forward(
             ptr(Q), ptr(K), ptr(V), ld, pos_ptr, ptr(ln_weight_K), ptr(ln_bias_K), ptr(ln_weight_V),
             ptr(ln_bias_V), float(norm_eps), ptr(out), ptr(ktv), ptr(ws), ws.numel(), B, S, H, dim_position,
@@ -315,7 +315,7 @@ def _attention_fused_backward(grad_out, Q, K, V, position, ln_weight_K, ln_bias_
     ws = workspace(nbytes, Q)
     grads = torch.empty((3, B, S, H * 32), dtype=torch.float32, device=Q.device)
     grad_ln = torch.empty((4, H, 32), dtype=torch.float32, device=Q.device)
-    with torch.cuda.device(Q.device):
+    with _lib.device_guard(Q.device):
         check(lib.spgt_galerkin_attention_fused_backward(
             ptr(grad_out), ptr(Q), ptr(K), ptr(V), ld, ptr(position) if dim_position == 2 else None,
             ptr(ln_weight_K), ptr(ln_bias_K), ptr(ln_weight_V), ptr(ln_bias_V), float(norm_eps), ptr(ktv),
@@ -356,7 +356,7 @@ def _attention_ktv_forward(K, V, position, ln_weight_K, ln_bias_K, ln_weight_V, 
     lib = _lib.load()
     ktv = torch.empty((B, H, D, D), dtype=torch.float32, device=K.device)
     ws = workspace(lib.spgt_galerkin_attention_fused_workspace_bytes(B, S, H, dim_position), K)
-    with torch.cuda.device(K.device):
+    with _lib.device_guard(K.device):
         check(lib.spgt_galerkin_attention_ktv_forward(
             ptr(K), ptr(V), ld, ptr(position) if dim_position == 2 else None, ptr(ln_weight_K), ptr(ln_bias_K),
             ptr(ln_weight_V), ptr(ln_bias_V), float(norm_eps), ptr(ktv), ptr(ws), ws.numel(), B, S, H, dim_position,
@@ -377,7 +377,7 @@ def _fold_ktv_into_fc(ktv, fc_weight_kn, dim_position: int):
     N = fc_weight_kn.shape[1]
     folded = torch.empty((B, H * 32, N), dtype=torch.float32, device=ktv.device)
     folded_pos = torch.empty((B, dim_position, N), dtype=torch.float32, device=ktv.device) if dim_position else None
-    with torch.cuda.device(ktv.device):
+    with _lib.device_guard(ktv.device):
         check(_lib.load().spgt_fold_ktv_into_fc(ptr(ktv), ptr(fc_weight_kn), ptr(folded),
                                                 ptr(folded_pos) if folded_pos is not None else None, B, H,
                                                 dim_position, N, stream_of(ktv)))
@@ -407,7 +407,7 @@ def _attention_fused_profile(input_sets, position, ln_weight_K, ln_bias_K, ln_we
     arrs = [(ctypes.c_void_p * n)(*[trip[j].data_ptr() for trip in input_sets]) for j in range(3)]
     out_arr = (ctypes.c_void_p * n)(*[o.data_ptr() for o in outs])
     stage = (ctypes.c_float * (3 * int(iterations)))()
-    with torch.cuda.device(Q0.device):
+    with _lib.device_guard(Q0.device):
         check(lib.spgt_galerkin_attention_fused_profile(
             arrs[0], arrs[1], arrs[2], out_arr, n, Q0.stride(1), ptr(position) if dim_position == 2 else None,
             ptr(ln_weight_K), ptr(ln_bias_K), ptr(ln_weight_V), ptr(ln_bias_V), float(norm_eps), ptr(ktv),

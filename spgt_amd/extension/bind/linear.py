@@ -79,7 +79,7 @@ def fused_linear(x: Tensor, weight_kn: Tensor, bias: Optional[Tensor] = None, ac
         xe, we, ldxe = x_extra.contiguous(), weight_extra_kn, ne
     if T == 0:
         return out
-    with torch.cuda.device(x.device):
+    with _lib.device_guard(x.device):
         check(_lib.load().spgt_linear_forward(
             ptr(xr), ldx, ptr(weight_kn), ptr(bias) if bias is not None else None,
             ptr(rr) if rr is not None else None, ldr, mode, ACTIVATIONS[activation],
@@ -116,7 +116,7 @@ def fused_ffn_scalar(x: Tensor, weight1_kn: Tensor, bias1: Optional[Tensor], wei
     out = torch.empty(list(x.shape[:-1]) + [1], dtype=x.dtype, device=x.device)
     if T == 0:
         return out
-    with torch.cuda.device(x.device):
+    with _lib.device_guard(x.device):
         check(_lib.load().spgt_ffn_scalar_forward(
             ptr(xr), ldx, ptr(weight1_kn), ptr(bias1) if bias1 is not None else None, ptr(weight2),
             ptr(bias2) if bias2 is not None else None, ACTIVATIONS[activation], ptr(out), T, K, HID, stream_of(x)))
@@ -169,7 +169,7 @@ def fused_encoder_tail(attn_out: Tensor, x: Tensor, fc_weight_kn: Tensor, fc_bia
     if T == 0:
         return out
     fc_droprate, ffn_droprate, seed = _dropout_args(x, fc_droprate, ffn_droprate, seed)
-    with torch.cuda.device(x.device):
+    with _lib.device_guard(x.device):
         if seed is None:
             check(_lib.load().spgt_encoder_tail_forward(
                 ptr(ar), lda, ptr(x), ptr(fc_weight_kn), ptr(fc_bias), ptr(ffn1_weight_kn), ptr(ffn1_bias),
@@ -218,7 +218,7 @@ def fused_encoder_tail_folded(q: Tensor, position, x: Tensor, folded_fc: Tensor,
     if out.numel() == 0:
         return out
     fc_droprate, ffn_droprate, seed = _dropout_args(x, fc_droprate, ffn_droprate, seed)
-    with torch.cuda.device(x.device):
+    with _lib.device_guard(x.device):
         if seed is None:
             check(_lib.load().spgt_encoder_tail_folded_forward(
                 ptr(q), ld, ptr(position) if dp else None, ptr(x), ptr(folded_fc), ptr(folded_pos) if dp else None,
@@ -247,7 +247,7 @@ def linear_weight_grad(x: Tensor, grad: Tensor):
         raise ValueError(f"unsupported weight-gradient shape: tokens={T} in={K} out={N} (out must be a multiple of 4)")
     ws = _lib.workspace(nbytes, xr)
     out = torch.empty(K * N + N, dtype=torch.float32, device=xr.device)
-    with torch.cuda.device(xr.device):
+    with _lib.device_guard(xr.device):
         check(lib.spgt_linear_weight_grad(ptr(xr), ldx, 0, ptr(gr), ldg, 0, ptr(out), ptr(ws), ws.numel(), T, K, N, 1,
                                           stream_of(xr)))
     return out[:K * N].view(K, N), out[K * N:]
@@ -268,7 +268,7 @@ def linear_weight_grad_batched(x: Tensor, grads: Tensor):
         raise ValueError(f"unsupported weight-gradient shape: tokens={T} in={K} out={N} (out must be a multiple of 4)")
     ws = _lib.workspace(nbytes, xr)
     out = torch.empty((P, K * N + N), dtype=torch.float32, device=xr.device)
-    with torch.cuda.device(xr.device):
+    with _lib.device_guard(xr.device):
         check(lib.spgt_linear_weight_grad(ptr(xr), ldx, 0, ptr(grads), N, T * N, ptr(out), ptr(ws), ws.numel(), T, K, N,
                                           P, stream_of(xr)))
     return out[:, :K * N].view(P, K, N), out[:, K * N:]
@@ -291,7 +291,7 @@ def dropout_add(y: Tensor, residual: Optional[Tensor], droprate: float, seed: Te
     out = torch.empty_like(y)
     if y.numel() == 0:
         return out
-    with torch.cuda.device(y.device):
+    with _lib.device_guard(y.device):
         check(_lib.load().spgt_dropout_add(ptr(y), ptr(residual) if residual is not None else None, ptr(out),
                                            y.numel() // C, C, ptr(seed), float(droprate), int(site), stream_of(y)))
     return out

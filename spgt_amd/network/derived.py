@@ -66,7 +66,7 @@ def _launch(descs: Sequence, device) -> None:
     if not descs:
         return
     arr = (_lib.CopyDesc * len(descs))(*descs)
-    with torch.cuda.device(device):
+    with _lib.device_guard(device):
         _lib.check(_lib.load().spgt_strided_copy_batch(
             arr, len(descs), torch.cuda.current_stream(device).cuda_stream))
 

@@ -32,17 +32,33 @@ def linear_weight_kn(lin: nn.Linear) -> Tensor:
     return derived(lin, "weight_kn", lambda: transposed_2d(lin.weight))
 
 
-def gpu_inference(X: Tensor, *params: Tensor) -> bool:
-    """fp32 on a GPU with nothing to differentiate: the case the fused inference kernels serve."""
+def _any_requires_grad(sources) -> bool:
+    for src in sources:
+        if src is None:
+            continue
+        if isinstance(src, Tensor):
+            if src.requires_grad:
+                return True
+        elif isinstance(src, nn.Module):
+            if any(p.requires_grad for p in src.parameters()):
+                return True
+        elif _any_requires_grad(src):
+            return True
+    return False
+
+
+def gpu_inference(X: Tensor, *sources) -> bool:
+    """fp32 on a GPU with nothing to differentiate: the case the fused inference kernels serve.  sources: tensors,
+    modules (their parameters) or sequences of those; they are only looked at while gradients are enabled, so that
+    a forward under torch.no_grad() does not walk the module tree."""
     if not X.is_cuda or X.dtype != torch.float32:
         return False
-    return not (torch.is_grad_enabled() and (X.requires_grad or any(p.requires_grad for p in params)))
+    return not (torch.is_grad_enabled() and (X.requires_grad or _any_requires_grad(sources)))
 
 
 def fused_linear_usable(X: Tensor, *linears: nn.Linear) -> bool:
     """gpu_inference, and the fused linear kernel has a variant for every layer's shape."""
-    return (gpu_inference(X, *[p for l in linears for p in l.parameters()]) and
-            all(linear_supported(l.in_features, l.out_features) for l in linears))
+    return gpu_inference(X, *linears) and all(linear_supported(l.in_features, l.out_features) for l in linears)
 
 
 def _weight_and_bias_grad(x: Tensor, g: Tensor, has_bias: bool):
@@ -170,7 +186,7 @@ class ConvResBlock2D(nn.Module):
     def fusable(self, X: Tensor) -> bool:
         """Inference: the bias, the dropout (the reference's F.dropout, on by default in inference too) and the
         activation can ride in the caller's next kernel."""
-        return 0 <= self.droprate < 1 and gpu_inference(X, *self.parameters())
+        return 0 <= self.droprate < 1 and gpu_inference(X, self)
 
     def conv_raw(self, X: Tensor) -> Tensor:
         """The convolution without its bias (to be added by the kernel that consumes the result)."""
@@ -203,7 +219,7 @@ class FeedForward(nn.Module):
     def forward(self, X: Tensor, residual: Tensor = None) -> Tensor:
         """ffn(X), or residual + ffn(X) when a residual is given."""
         if (self.layer2.out_features == 1 and residual is None and
-                gpu_inference(X, *self.parameters()) and
+                gpu_inference(X, self) and
                 ffn_scalar_supported(self.layer1.in_features, self.layer1.out_features)):
             # single output feature: both layers in one kernel, the hidden activations stay in registers
             Y = fused_ffn_scalar(X, linear_weight_kn(self.layer1), self.layer1.bias, self.layer2.weight.detach(),

@@ -92,7 +92,7 @@ class DownScaler2D(nn.Module):
         self.activation_layer = make_activation(activation)
 
     def forward(self, X: Tensor) -> Tensor:
-        fused = gpu_inference(X, *self.parameters())
+        fused = gpu_inference(X, self)
         act = activation_name(self.activation_layer)
         c0 = self.conv0.conv_layer
         if (fused and self.conv0.fusable(X) and conv3x3_resample_supported(X.size(-1)) and c0.kernel_size == (3, 3) and
@@ -149,7 +149,7 @@ class UpScaler2D(nn.Module):
 
     def can_defer_last_resample(self, X: Tensor) -> bool:
         """True when forward(X, defer_last_resample=True) is available: fused inference with one kind of activation."""
-        return (gpu_inference(X, *self.parameters()) and self.droprate == 0 and self.conv.droprate == 0 and
+        return (gpu_inference(X, self) and self.droprate == 0 and self.conv.droprate == 0 and
                 self.conv.fusable(X) and type(self.conv.activation_layer) is type(self.activation_layer))
 
     def _tap_weight_kn(self) -> Tensor:
@@ -218,7 +218,7 @@ class UpScaler2D(nn.Module):
             Y = self.conv.conv_raw(X)
             return bilinear_resample(Y, tuple(Y.shape[-2:]), dst_nhwc=True, pre_bias=self.conv.conv_layer.bias,
                                      pre_activation=activation_name(self.activation_layer), pre_count=2)
-        if gpu_inference(X, *self.parameters()) and self.droprate == 0:
+        if gpu_inference(X, self) and self.droprate == 0:
             # channels-last in, NCHW out for the convolution; the block's bias and activation and the
             # scaler's own activation are one in-place pass (an upsampling reads every source sample
             # several times, so they are not applied inside it); the second resampling writes channels-last

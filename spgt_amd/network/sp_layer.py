@@ -245,7 +245,7 @@ class Sp_EncoderLayer(nn.Module):
     @refreshes_derived
     def forward(self, X: Tensor, position: Tensor) -> Tensor:
         att, ffn = self.attention_layer, self.ffn_layer
-        if (0 <= att.fc_droprate < 1 and 0 <= ffn.droprate < 1 and gpu_inference(X, *self.parameters()) and
+        if (0 <= att.fc_droprate < 1 and 0 <= ffn.droprate < 1 and gpu_inference(X, self) and
                 encoder_tail_supported(att.fc_layer.in_features, att.fc_layer.out_features, ffn.layer1.out_features)
                 and ffn.layer2.out_features == att.fc_layer.out_features):
             # output projection, both residual adds and the feed-forward net in one launch; the layer's two
@@ -292,7 +292,7 @@ class Sp_SpectralConv2D(nn.Module):
         needs_graph = torch.is_grad_enabled() and (X.requires_grad or self.fourier_weight[0].requires_grad)
         truncated = self.use_truncated_dft and not needs_graph and truncated_dft.supported(r, m)
         if (truncated and self.droprate == 0 and truncated_dft.fused_tail_supported(r, cin, cout, m) and
-                gpu_inference(X, *self.residual_layer.parameters())):
+                gpu_inference(X, self.residual_layer)):
             # only the retained modes are ever computed: no FFT, no transposes, no full-size spectrum; the
             # inverse transform along w, the residual Linear, the add and the activation are one kernel
             return truncated_dft.spectral_modes_apply_linear(
