@@ -331,8 +331,9 @@ def test_model_with_the_reference_drop_rates(gpu):
     feed-forward nets; the reference's dropouts are on in inference): the forward runs on the fused kernels with
     their own masks.  Two forwards differ, torch.manual_seed repeats one (up to the convolution library's own
     run-to-run rounding), and the mean over many forwards agrees with the mean over as many forwards of the same
-    model on the route that calls torch's F.dropout (taken when gradients are enabled) as well as two such means
-    agree with each other."""
+    model on the route taken when gradients are enabled (other kernels, other launches, torch's F.dropout in the
+    down-scaler's convolution blocks, separate dropout passes with seeds of their own elsewhere) as well as two such
+    means agree with each other.  The masks' own properties are tested kernel by kernel."""
     p, i, _, meta = load_golden("galerkin_transformer_2d")
     cfgd = dict(model_cfg(meta), drop_downscaler=0.05, drop_encoder_attn_fc=0.05, drop_encoder_ffn=0.05)
     md = load_into(SM.Sp_GalerkinTransformer2D(cfgd), p, gpu)
