@@ -2,9 +2,10 @@
 
 Same function names, argument order and result layouts as the reference's
 extension/bind/datamove.py:68-87 (python surface) and
-extension/bind/datamove.cu:66-70 (the `dexts` module surface), plus two
+extension/bind/datamove.cu:66-70 (the `dexts` module surface), plus the
 operators the reference leaves to library calls: the fused spectral-mode
-contraction and bilinear resampling.  Tensors must be contiguous and on a GPU.
+contraction, the truncated-DFT stages, bilinear resampling (with its backward)
+and the scalers' fused forms.  Tensors must be contiguous and on a GPU.
 """
 import ctypes
 from math import prod

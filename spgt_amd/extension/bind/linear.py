@@ -1,10 +1,12 @@
-"""Fused token-major linear layer, backed by libspgt_hip.so (inference only).
+"""Fused token-major linear layers, backed by libspgt_hip.so.
 
 The reference's modules call nn.Linear and then separate elementwise kernels for
 the activation and the residual add (network/layer.py:155-174,
 network/sp_layer.py:75, 97-103 and 132, 155, network/sp_model.py:60, 63); here the three
-are one kernel.  There is no autograd: modules use it under torch.no_grad() and
-fall back to their nn.Linear graph when gradients are required.
+are one kernel (fused_linear, fused_ffn_scalar, fused_encoder_tail).  These functions build no
+autograd graph themselves: the modules call them under torch.no_grad() and, when gradients are
+required, through autograd functions (network/layer.py) whose backward uses linear_weight_grad
+(dW, db in one pass over the tokens) and dropout_add from this file.
 """
 from typing import Optional
 

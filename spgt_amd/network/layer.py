@@ -3,9 +3,10 @@ convolution block and the two-layer feed-forward net.  Parameter names and
 shapes match the reference's network/layer.py:7-24 (ConvResBlock2D) and
 :155-174 (FeedForward) so that its checkpoints load unchanged.
 
-As in the reference, `F.dropout` is applied with its default training=True
-whenever the drop rate is non-zero, also under model.eval(); run with drop
-rates of 0 for deterministic inference.
+As in the reference, dropout is applied whenever the drop rate is non-zero,
+also under model.eval() (the reference calls `F.dropout` with its default
+training=True); run with drop rates of 0 for deterministic inference.  On the
+GPU the fused kernels apply it themselves, with the library's own masks.
 """
 import torch
 import torch.nn.functional as F

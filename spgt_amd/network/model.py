@@ -1,7 +1,11 @@
-"""Down- and up-scalers around the encoder: 3x3 convolutions (library) with
-bilinear align_corners resampling (this package's HIP kernel when no autograd
-graph is needed).  Structure, parameter names and shapes follow the
-reference's network/model.py:7-39 (DownScaler2D) and :42-65 (UpScaler2D).
+"""Down- and up-scalers around the encoder: 3x3 convolutions with bilinear
+align_corners resampling.  Inference fuses them into this package's kernels
+where it can (the down-scaler's three middle convolutions stay with the
+library); under autograd the resamplings, the down-scaler's first stage and
+the up-scaler's convolution (as a Linear on the low-resolution tokens plus a
+gather) run on this package's kernels forward and backward.  Structure,
+parameter names and shapes follow the reference's network/model.py:7-39
+(DownScaler2D) and :42-65 (UpScaler2D).
 """
 import torch
 import torch.nn.functional as F
