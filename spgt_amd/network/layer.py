@@ -78,31 +78,48 @@ class _LinearFunction(torch.autograd.Function):
     """x @ W^T + b (+ residual) for an nn.Linear's parameters, forward and backward on this package's kernels:
     the fused linear kernel forward and for dX = g @ W where it has a variant for the shape (the library's GEMM
     otherwise), and one pass over x and g for dW = g^T x and db (the library's GEMM for that product, whose
-    contraction runs over all tokens, takes 250 us at 65k tokens)."""
+    contraction runs over all tokens, takes 250 us at 65k tokens).
+    relu: the result is relu(x @ W^T + b), formed in the forward kernel's epilogue; the backward masks the incoming
+    gradient with the saved result.  with_identity: x is handed on as a second result, for a caller that also adds
+    it as a residual further on: that residual's gradient then arrives here and rides in the dX product."""
 
     @staticmethod
-    def forward(ctx, x, weight, bias, weight_kn, residual):
-        ctx.save_for_backward(x, weight)
-        ctx.has_bias, ctx.has_residual = bias is not None, residual is not None
+    def forward(ctx, x, weight, bias, weight_kn, residual, relu=False, with_identity=False):
+        ctx.has_bias, ctx.has_residual, ctx.relu, ctx.with_identity = bias is not None, residual is not None, relu, with_identity
         if weight_kn is not None:
-            return fused_linear(x, weight_kn, bias, "none", residual)
-        y = F.linear(x, weight, bias)
-        return y if residual is None else y + residual
+            y = fused_linear(x, weight_kn, bias, "relu" if relu else "none", residual)
+        else:
+            y = F.linear(x, weight, bias)
+            if residual is not None:
+                y = y + residual
+            if relu:
+                y = torch.relu_(y)
+        ctx.save_for_backward(x, weight, *([y] if relu else []))
+        return (y, x.view_as(x)) if with_identity else y
 
     @staticmethod
-    def backward(ctx, g):
-        x, weight = ctx.saved_tensors
+    def backward(ctx, g, g_identity=None):
+        x, weight = ctx.saved_tensors[:2]
         g = g.contiguous()
+        if ctx.relu:
+            g = torch.ops.aten.threshold_backward(g, ctx.saved_tensors[2], 0)
         dx = None
         if ctx.needs_input_grad[0]:
             w = weight.detach()
+            gi = None if g_identity is None else g_identity.reshape(-1, x.shape[-1]).contiguous()
             # g @ W: the fused kernel where it has a variant for [out -> in], else the library's GEMM
-            dx = (fused_linear(g, w.contiguous(), None, "none") if linear_supported(w.shape[0], w.shape[1])
-                  else torch.matmul(g, w))
+            if linear_supported(w.shape[0], w.shape[1]):
+                dx = fused_linear(g.reshape(-1, w.shape[0]), w.contiguous(), None, "none", gi).view(x.shape)
+            else:
+                dx = torch.matmul(g, w)
+                if gi is not None:
+                    dx = dx + gi.view(x.shape)
+        elif g_identity is not None:
+            dx = g_identity
         dw = db = None
         if ctx.needs_input_grad[1] or (ctx.has_bias and ctx.needs_input_grad[2]):
             dw, db = _weight_and_bias_grad(x, g, ctx.has_bias)
-        return dx, dw, db, None, (g if ctx.has_residual else None)
+        return dx, dw, db, None, (g if ctx.has_residual else None), None, None
 
 
 def linear_trainable(X: Tensor, lin: nn.Linear) -> bool:
@@ -112,10 +129,11 @@ def linear_trainable(X: Tensor, lin: nn.Linear) -> bool:
             (lin.out_features % 4 == 0 or lin.in_features % 4 == 0))
 
 
-def linear_train(X: Tensor, lin: nn.Linear, residual: Tensor = None) -> Tensor:
-    """lin(X) (+ residual) with an autograd graph, on this package's kernels (see _LinearFunction)."""
+def linear_train(X: Tensor, lin: nn.Linear, residual: Tensor = None, relu: bool = False, with_identity: bool = False):
+    """lin(X) (+ residual), or relu of it, with an autograd graph, on this package's kernels (see _LinearFunction);
+    with_identity: (result, X handed on for use as a residual further on)."""
     kn = linear_weight_kn(lin) if linear_supported(lin.in_features, lin.out_features) else None
-    return _LinearFunction.apply(X, lin.weight, lin.bias, kn, residual)
+    return _LinearFunction.apply(X, lin.weight, lin.bias, kn, residual, relu, with_identity)
 
 
 class _SplitLinearFunction(torch.autograd.Function):
@@ -233,7 +251,13 @@ class FeedForward(nn.Module):
             return always_dropout(Y, self.droprate)
         if linear_trainable(X, self.layer1) and linear_trainable(X, self.layer2):
             # under autograd: the same kernels, with the weight gradients by this package's pass over the tokens
-            Hd = self.activation_layer(linear_train(X, self.layer1))
+            relu = isinstance(self.activation_layer, nn.ReLU)
+            identity = residual is X and X.is_contiguous()
+            Hd = linear_train(X, self.layer1, None, relu, identity)
+            if identity:
+                Hd, residual = Hd
+            if not relu:
+                Hd = self.activation_layer(Hd)
             if self.droprate == 0:
                 return linear_train(Hd, self.layer2, residual)
             return always_dropout_add(linear_train(Hd, self.layer2), residual, self.droprate)

@@ -48,10 +48,12 @@ class _PackedProjectionFunction(torch.autograd.Function):
         N, S, C = x.shape
         ctx.save_for_backward(x, wq, wk, wv)
         out = fused_linear(x.reshape(N * S, C), packed_w, packed_b, planes=3).view(3, N, S, C)
-        return out[0], out[1], out[2]
+        # the fourth result is x itself: a caller that also adds x as a residual takes it from here, so that the
+        # residual's gradient arrives in this backward and rides in the dX product instead of a separate add
+        return out[0], out[1], out[2], x.view_as(x)
 
     @staticmethod
-    def backward(ctx, dq, dk, dv):
+    def backward(ctx, dq, dk, dv, dres):
         x, wq, wk, wv = ctx.saved_tensors
         N, S, C = x.shape
         planes = (dq, dk, dv)
@@ -65,6 +67,7 @@ class _PackedProjectionFunction(torch.autograd.Function):
             grads = torch.stack([dq.reshape(N * S, C), dk.reshape(N * S, C), dv.reshape(N * S, C)])
         dx = None
         if ctx.needs_input_grad[0]:
+            dx = None if dres is None else dres.reshape(N * S, C).contiguous()
             for g, w in zip(grads, (wq, wk, wv)):
                 dx = fused_linear(g, w.t().contiguous(), None, "none", dx)  # dx += g @ w^T
             dx = dx.view(N, S, C)
@@ -139,10 +142,18 @@ class Sp_GalerkinAttention(nn.Module):
     def forward(self, Q: Tensor, K: Tensor, V: Tensor, position: Tensor, residual: Tensor = None) -> Tensor:
         """Q, K, V [N, seqlen, dim_hidden], position [N, seqlen, dim_position] -> [N, seqlen, dim_hidden];
         with `residual` the result is residual + attention(Q, K, V)."""
-        return self.project(self.attend(Q, K, V, position), residual)
+        X, identity = self._attend(Q, K, V, position)
+        if identity is not None and residual is Q:
+            residual = identity  # Q as the packed projection's autograd function handed it on (see there)
+        return self.project(X, residual)
 
     def attend(self, Q: Tensor, K: Tensor, V: Tensor, position: Tensor) -> Tensor:
         """The attention core before fc_layer: [N, seqlen, num_head * (dim_position + dim_head)]."""
+        return self._attend(Q, K, V, position)[0]
+
+    def _attend(self, Q: Tensor, K: Tensor, V: Tensor, position: Tensor):
+        """(attend(...), Q as an output of the training route's packed projection or None)."""
+        identity = None
         N, seqlen, C = Q.size()
         H, dp = self.num_head, self.dim_position
         if self._needs_graph(Q, K, V) and C > 512:
@@ -164,8 +175,10 @@ class Sp_GalerkinAttention(nn.Module):
                 and linear_supported(C, C) and Q.is_cuda and Q.dtype == torch.float32:
             # training on the token-major path: packed projection, then the fused core, both with their own backward
             w, b = self._packed_qkv()
-            q, k, v = _PackedProjectionFunction.apply(Q.contiguous(), self.weight_Q, self.weight_K, self.weight_V,
-                                                      self.bias_Q, self.bias_K, self.bias_V, w, b)
+            q, k, v, ident = _PackedProjectionFunction.apply(Q.contiguous(), self.weight_Q, self.weight_K,
+                                                             self.weight_V, self.bias_Q, self.bias_K, self.bias_V, w, b)
+            if Q.is_contiguous():
+                identity = ident
             pos = position.contiguous() if dp else None
             X = galerkin_attention_fused(q, k, v, pos, self.ln_weight_K, self.ln_bias_K, self.ln_weight_V,
                                          self.ln_bias_V, self.norm_eps, H, dp)
@@ -195,7 +208,7 @@ class Sp_GalerkinAttention(nn.Module):
             pos = position.contiguous() if dp else None
             X = galerkin_attention_fused(q, k, v, pos, self.ln_weight_K.detach(), self.ln_bias_K.detach(),
                                          self.ln_weight_V.detach(), self.ln_bias_V.detach(), self.norm_eps, H, dp)
-        return X
+        return X, identity
 
     def folded_projection(self, X: Tensor, position: Tensor):
         """(q, position, folded_fc, folded_pos) for fused_encoder_tail_folded: self-attention on X whose last

@@ -345,12 +345,13 @@ def test_packed_projection_function_with_separate_gradient_tensors(gpu):
     packed_w = torch.cat([w.detach() for w in ws], dim=1).contiguous()
     packed_b = torch.cat([b.detach() for b in bs]).contiguous()
     outs = _PackedProjectionFunction.apply(x, *ws, *bs, packed_w, packed_b)
-    gs = [torch.randn(N, S, C, device=gpu) for _ in range(3)]
+    assert len(outs) == 4 and torch.equal(outs[3], x)  # the input handed on for a residual add further on
+    gs = [torch.randn(N, S, C, device=gpu) for _ in range(4)]
     got = torch.autograd.grad(outs, [x, *ws, *bs], gs)
     x2 = x.detach().double().requires_grad_(True)
     ws2 = [w.detach().double().requires_grad_(True) for w in ws]
     bs2 = [b.detach().double().requires_grad_(True) for b in bs]
-    ref_outs = [x2 @ w + b for w, b in zip(ws2, bs2)]
+    ref_outs = [x2 @ w + b for w, b in zip(ws2, bs2)] + [x2 * 1.0]
     want = torch.autograd.grad(ref_outs, [x2, *ws2, *bs2], [g.double() for g in gs])
     for o, r in zip(outs, ref_outs):
         assert max_rel(o.detach().double().cpu(), r.detach().cpu()) < TOL
