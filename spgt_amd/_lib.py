@@ -204,8 +204,35 @@ def workspace(nbytes: int, like: torch.Tensor) -> torch.Tensor:
     return torch.empty(max(int(nbytes), 16), dtype=torch.uint8, device=like.device)
 
 
+_seed_tls = threading.local()
+_SEED_POOL_WORDS = 128
+
+
+class seed_scope:
+    """Within this context (one model forward), dropout_seed hands out consecutive word pairs of one drawn
+    pool instead of launching a generator kernel per call.  The pool never outlives the context: a forward
+    captured into a graph draws its pool inside the capture, so every replay gets new words."""
+
+    def __enter__(self):
+        self.outer = getattr(_seed_tls, "pool", None), getattr(_seed_tls, "used", 0), getattr(_seed_tls, "on", False)
+        _seed_tls.pool, _seed_tls.used, _seed_tls.on = None, 0, True
+        return self
+
+    def __exit__(self, *exc):
+        _seed_tls.pool, _seed_tls.used, _seed_tls.on = self.outer
+        return False
+
+
 def dropout_seed(device):
     """Two 32-bit words from torch's generator of `device`, in device memory, for the kernels that apply dropout
     themselves.  Drawn by a generator kernel: torch.manual_seed governs it, and inside a captured graph every
-    replay draws new words."""
-    return torch.randint(0, 2 ** 31 - 1, (2,), dtype=torch.int32, device=device)
+    replay draws new words.  Every call gives a different pair."""
+    if not getattr(_seed_tls, "on", False):
+        return torch.randint(0, 2 ** 31 - 1, (2,), dtype=torch.int32, device=device)
+    device = torch.device(device)
+    pool, used = _seed_tls.pool, _seed_tls.used
+    if pool is None or pool.device != device or used + 2 > pool.numel():
+        pool, used = torch.randint(0, 2 ** 31 - 1, (_SEED_POOL_WORDS,), dtype=torch.int32, device=device), 0
+        _seed_tls.pool = pool
+    _seed_tls.used = used + 2
+    return pool[used:used + 2]

@@ -134,7 +134,8 @@ def refreshes_derived(forward):
         _tls.forward_id = _forward_counter[0]
         try:
             refresh(self)
-            return forward(self, *args, **kwargs)
+            with _lib.seed_scope():
+                return forward(self, *args, **kwargs)
         finally:
             _tls.active = False
             _tls.forward_id = -2

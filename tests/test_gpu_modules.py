@@ -273,6 +273,25 @@ def test_encoder_layer_folded_attention(gpu, dp, B, S):
     assert rel_l2(got.cpu(), want.cpu()) < 1e-5 and max_rel(got.cpu(), want.cpu()) < 1e-4
 
 
+def test_dropout_seeds_of_one_forward_come_from_one_draw(gpu):
+    """Inside a forward every dropout site gets its own word pair out of one generator call; outside, each
+    call draws its own.  torch.manual_seed governs both."""
+    from spgt_amd import _lib
+
+    torch.manual_seed(5)
+    with _lib.seed_scope():
+        a, b = _lib.dropout_seed(gpu), _lib.dropout_seed(gpu)
+        assert a.untyped_storage().data_ptr() == b.untyped_storage().data_ptr()
+        assert a.data_ptr() + 8 == b.data_ptr() and a.numel() == b.numel() == 2
+        pairs = [tuple(_lib.dropout_seed(gpu).tolist()) for _ in range(70)]  # runs past one pool
+        assert len(set(pairs + [tuple(a.tolist()), tuple(b.tolist())])) == 72
+    c = _lib.dropout_seed(gpu)
+    assert c.numel() == 2 and c.untyped_storage().data_ptr() != a.untyped_storage().data_ptr()
+    torch.manual_seed(5)
+    with _lib.seed_scope():
+        assert torch.equal(_lib.dropout_seed(gpu), a)
+
+
 @pytest.mark.parametrize("fold", [False, True])
 def test_encoder_layer_with_drop_rates_stays_fused(gpu, fold):
     """With the reference's drop rates (always on, F.dropout's default) the layer still runs as one launch after the
