@@ -150,6 +150,145 @@ __global__ __launch_bounds__(256) void dft_rows_forward_k(const float* __restric
     }
 }
 
+// The forward transform for 32 < 2m <= 64 table columns, with the grid row folded onto itself first:
+// cos(2 pi kw (r - w) / r) = cos(2 pi kw w / r) and sin(..(r - w)..) = -sin(..w..), so with
+//   xe[f] = x[f] + x[r - f],  xo[f] = x[f] - x[r - f]      f = 1 .. ceil(r/2) - 1
+// (f = 0 and, for even r, f = r/2 stand alone) the real columns are sums of xe against the cosines and the
+// imaginary columns sums of xo against the sines over F = floor(r/2) + 1 folded points: half the contraction
+// length, one 32-column block each, i.e. half the MFMAs of the unfolded form with two column blocks.
+// The LDS copy of the table holds row f as [32 real entries | 32 imaginary entries]; the real entries of the
+// points that stand alone are halved (their xe is formed as x[f] + x[f]).  Sums run in a fixed order.
+// V channels per lane (C % (32 V) == 0): a lane loads V consecutive channels of its grid point at once (a wave
+// issues a quarter of the load instructions at V = 4, which is what bounds the V = 1 form at 128 channels) and
+// component e of the piece feeds accumulator e, whose lane tk stands for channel V tk + e; one table entry from
+// LDS serves the V MFMAs of a step.  V = 4 keeps 128 accumulator registers: one wave per SIMD.
+// grid (workgroups), block 256, dynamic LDS 2 * ceil(F/2) * 64 floats; tab as for dft_rows_forward_k<CT, 2>.
+template <int V>
+struct FoldPiece;
+template <>
+struct FoldPiece<1> { typedef float type; };
+template <>
+struct FoldPiece<2> { typedef float2 type; };
+template <>
+struct FoldPiece<4> { typedef float4 type; };
+__device__ __forceinline__ float fold_get(float v, int) { return v; }
+__device__ __forceinline__ float fold_get(const float2& v, int e) { return e == 0 ? v.x : v.y; }
+__device__ __forceinline__ float fold_get(const float4& v, int e) { return e == 0 ? v.x : e == 1 ? v.y : e == 2 ? v.z : v.w; }
+
+template <int CT, int V>
+__global__ __launch_bounds__(256) void dft_rows_forward_fold_k(const float* __restrict__ x,
+                                                               const float* __restrict__ tab, float* __restrict__ Y,
+                                                               int64_t rows, int r, int C_, int m2, int planar) {
+    typedef typename FoldPiece<V>::type piece_t;
+    extern __shared__ float ts[];
+    const int C = CT ? CT : C_;
+    const int F = r / 2 + 1;
+    const int KHf = (F + 1) / 2;  // MFMA steps: two folded points each
+    for (int e = threadIdx.x; e < 2 * KHf * 64; e += 256) {
+        const int f = e >> 6, col = e & 63, kw = col & 31, part = col >> 5;
+        float v = (f < F && 2 * kw + part < m2) ? tab[(int64_t)f * 64 + 2 * kw + part] : 0.f;
+        if (part == 0 && (f == 0 || 2 * f == r)) v *= 0.5f;
+        ts[e] = v;
+    }
+    __syncthreads();
+    const int lane = threadIdx.x & 63;
+    const int tk = lane & 31;
+    const int kh = lane >> 5;
+    const int CB = C / (32 * V);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    constexpr int BK = V == 1 ? 16 : 8;
+    const int nb = (KHf + BK - 1) / BK;
+    for (int64_t gw = (int64_t)blockIdx.x * 4 + wave; gw < rows * CB; gw += (int64_t)gridDim.x * 4) {
+        const int64_t row = gw / CB;
+        const int cb = (int)(gw % CB);
+        const float* base = x + row * (int64_t)r * C + cb * (32 * V) + tk * V;
+        piece_t a0[BK], b0[BK], a1[BK], b1[BK];
+        v16f acc_re[V], acc_im[V];
+#pragma unroll
+        for (int e = 0; e < V; ++e)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc_re[e][i] = acc_im[e][i] = 0.f;
+        // steps past the last folded point read that point again (against zero table rows); the partner of
+        // point 0 is point 0 itself
+#define SPGT_FOLD_FETCH(AV, BV, B)                                                                   \
+        _Pragma("unroll") for (int u = 0; u < BK; ++u) {                                              \
+            const int f = min(2 * ((B) * BK + u) + kh, F - 1);                                        \
+            AV[u] = *reinterpret_cast<const piece_t*>(base + (uint32_t)(f * C));                      \
+            BV[u] = *reinterpret_cast<const piece_t*>(base + (uint32_t)((f == 0 ? 0 : r - f) * C));   \
+        }
+#define SPGT_FOLD_MUL(AV, BV, B)                                                                      \
+        _Pragma("unroll") for (int u = 0; u < BK; ++u) {                                              \
+            const int kk = (B) * BK + u;                                                              \
+            if (kk < KHf) {                                                                           \
+                const float* tr = ts + (2 * kk + kh) * 64 + tk;                                       \
+                const float tre = tr[0], tim = tr[32];                                                \
+                _Pragma("unroll") for (int e = 0; e < V; ++e) {                                       \
+                    const float av = fold_get(AV[u], e), bv = fold_get(BV[u], e);                     \
+                    acc_re[e] = mfma32(tre, av + bv, acc_re[e]);                                      \
+                    acc_im[e] = mfma32(tim, av - bv, acc_im[e]);                                      \
+                }                                                                                     \
+            }                                                                                         \
+        }
+        SPGT_FOLD_FETCH(a0, b0, 0)
+        for (int b = 0; b < nb; b += 2) {
+            if (b + 1 < nb) { SPGT_FOLD_FETCH(a1, b1, b + 1) }
+            __builtin_amdgcn_sched_barrier(0);
+            SPGT_FOLD_MUL(a0, b0, b)
+            __builtin_amdgcn_sched_barrier(0);
+            if (b + 2 < nb) { SPGT_FOLD_FETCH(a0, b0, b + 2) }
+            __builtin_amdgcn_sched_barrier(0);
+            if (b + 1 < nb) { SPGT_FOLD_MUL(a1, b1, b + 1) }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#undef SPGT_FOLD_FETCH
+#undef SPGT_FOLD_MUL
+        // acc_re[e][4q + i] = Re Y[c = cb*32V + V tk + e][kw = 8q + 4kh + i], acc_im the imaginary part:
+        // columns 2kw, 2kw + 1
+        if (planar) {
+            const int64_t n = row / r;
+            const int64_t h = row - n * r;
+            float* yp = Y + (n * m2 * r + h) * (int64_t)C + cb * (32 * V) + tk * V;
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int j = 2 * (8 * q + 4 * kh + i);
+                    if (j < m2) {
+                        float* pre = yp + (int64_t)j * r * C;
+                        float* pim = yp + (int64_t)(j + 1) * r * C;
+                        if (V == 4) {
+                            *reinterpret_cast<float4*>(pre) = make_float4(acc_re[0][4 * q + i], acc_re[1 % V][4 * q + i],
+                                                                          acc_re[2 % V][4 * q + i], acc_re[3 % V][4 * q + i]);
+                            *reinterpret_cast<float4*>(pim) = make_float4(acc_im[0][4 * q + i], acc_im[1 % V][4 * q + i],
+                                                                          acc_im[2 % V][4 * q + i], acc_im[3 % V][4 * q + i]);
+                        } else if (V == 2) {
+                            *reinterpret_cast<float2*>(pre) = make_float2(acc_re[0][4 * q + i], acc_re[1 % V][4 * q + i]);
+                            *reinterpret_cast<float2*>(pim) = make_float2(acc_im[0][4 * q + i], acc_im[1 % V][4 * q + i]);
+                        } else {
+                            pre[0] = acc_re[0][4 * q + i];
+                            pim[0] = acc_im[0][4 * q + i];
+                        }
+                    }
+                }
+        } else {
+#pragma unroll
+            for (int e = 0; e < V; ++e) {
+                float* yr = Y + (row * C + cb * (32 * V) + tk * V + e) * (int64_t)m2;
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int j = 2 * (8 * q + 4 * kh + i);
+                        if (j < m2) {
+                            yr[j] = acc_re[e][4 * q + i];
+                            yr[j + 1] = acc_im[e][4 * q + i];
+                        }
+                    }
+            }
+        }
+    }
+}
+
 // grid (workgroups), block 256; waves stride over the (row, channel block) items.
 // tab [32*ceil(r/32)][m2 + 1]: row w holds the m2 table entries of grid point w, zero elsewhere.
 // U [rows][C][m2] (or planar [rows/r][m2][r][C]) -> y [rows][r][C].  KMAX >= m2 / 2: MFMA steps held in registers.
@@ -363,31 +502,36 @@ __global__ __launch_bounds__(256) void spectral_rows_contract_k(
     }
 }
 
-// grid (m, N, chunks of h), block 256.  Wave w of a workgroup takes rows h = h0 + w, h0 + w + 4, ...
+// grid (m, N, chunks of h), block 256.  LPR = 64: wave w of a workgroup takes rows h = h0 + w, h0 + w + 4, ...
+// with a lane per output channel; LPR = 32 (Cout <= 32): each half of a wave takes a row of its own.
 // KHMAX >= 2m: kept rows held in registers.
-template <int KHMAX>
+template <int KHMAX, int LPR>
 __global__ __launch_bounds__(256) void spectral_rows_expand_k(
     const float2* __restrict__ O, const float2* __restrict__ Gi, float* __restrict__ U, int r, int Cout, int m,
     int rows_per_wg) {
     extern __shared__ float2 lds[];  // Gi rows of the chunk: [rows_per_wg][2m]
+    constexpr int RPW = 64 / LPR;    // rows a wave works on at a time
     const int m2 = 2 * m;
     const int kw = blockIdx.x;
     const int64_t n = blockIdx.y;
     const int h0 = blockIdx.z * rows_per_wg;
     const int h1 = min(r, h0 + rows_per_wg);
     const int lane = threadIdx.x & 63;
+    const int o = lane % LPR;
+    const int sub = lane / LPR;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     for (int e = threadIdx.x; e < (h1 - h0) * m2; e += 256) lds[e] = Gi[(int64_t)h0 * m2 + e];
     // the mode's O[kh][o] for all kept rows stays in registers
     float2 ov[KHMAX];
-    const float2* Om = O + ((n * m + kw) * m2) * (int64_t)Cout + lane;
+    const float2* Om = O + ((n * m + kw) * m2) * (int64_t)Cout + o;
 #pragma unroll
-    for (int kh = 0; kh < KHMAX; ++kh) ov[kh] = (kh < m2 && lane < Cout) ? Om[(int64_t)kh * Cout] : make_float2(0.f, 0.f);
+    for (int kh = 0; kh < KHMAX; ++kh) ov[kh] = (kh < m2 && o < Cout) ? Om[(int64_t)kh * Cout] : make_float2(0.f, 0.f);
     __syncthreads();
-    float* ure = U + ((n * m2 + 2 * kw) * r) * (int64_t)Cout + lane;
+    float* ure = U + ((n * m2 + 2 * kw) * r) * (int64_t)Cout + o;
     float* uim = ure + (int64_t)r * Cout;
-    for (int h = h0 + wave; h < h1; h += 4) {
-        const float2* g = lds + (h - h0) * m2;
+    for (int hb = h0 + wave * RPW; hb < h1; hb += 4 * RPW) {
+        const int h = hb + sub;
+        const float2* g = lds + (min(h, h1 - 1) - h0) * m2;
         float2 acc = make_float2(0.f, 0.f);
 #pragma unroll
         for (int kh = 0; kh < KHMAX; ++kh) {
@@ -398,7 +542,7 @@ __global__ __launch_bounds__(256) void spectral_rows_expand_k(
                 acc.y = fmaf(g[kh].y, ov[kh].x, acc.y);
             }
         }
-        if (lane < Cout) {
+        if (o < Cout && h < h1) {
             ure[(int64_t)h * Cout] = acc.x;
             uim[(int64_t)h * Cout] = acc.y;
         }
@@ -628,8 +772,27 @@ extern "C" int spgt_truncated_dft_rows_forward(const float* x, const float* tabl
         if (channels == 64) SPGT_DFT_FWD(64, 1) else if (channels == 32) SPGT_DFT_FWD(32, 1)
         else if (channels == 128) SPGT_DFT_FWD(128, 1) else SPGT_DFT_FWD(0, 1)
     } else {
-        if (channels == 64) SPGT_DFT_FWD(64, 2) else if (channels == 32) SPGT_DFT_FWD(32, 2)
-        else if (channels == 128) SPGT_DFT_FWD(128, 2) else SPGT_DFT_FWD(0, 2)
+        const size_t lds_fold = (size_t)2 * ((r / 2 + 2) / 2) * 64 * sizeof(float);
+        // the widest pieces the alignment of x and the channel count allow
+        const bool planar_ok16 = !planar || aligned16(Y), planar_ok8 = !planar || aligned8(Y);
+        const int v = (channels % 128 == 0 && aligned16(x) && planar_ok16) ? 4
+                      : (channels % 64 == 0 && aligned8(x) && planar_ok8) ? 2 : 1;
+        const unsigned grid_fold = (unsigned)std::min<int64_t>(ceil_div(rows * (channels / (32 * v)), (int64_t)4),
+                                                               (v == 4 ? 1 : 2) * device_cu_count());
+#define SPGT_DFT_FOLD(CT, V)                                                                                    \
+    {                                                                                                           \
+        allow_lds(dft_rows_forward_fold_k<CT, V>, lds_fold);                                                    \
+        hipLaunchKernelGGL((dft_rows_forward_fold_k<CT, V>), dim3(grid_fold), dim3(256), lds_fold, stream, x,   \
+                           table, Y, rows, r, channels, m2, planar);                                            \
+    }
+        if (v == 4) {
+            if (channels == 128) SPGT_DFT_FOLD(128, 4) else SPGT_DFT_FOLD(0, 4)
+        } else if (v == 2) {
+            if (channels == 64) SPGT_DFT_FOLD(64, 2) else SPGT_DFT_FOLD(0, 2)
+        } else {
+            if (channels == 32) SPGT_DFT_FOLD(32, 1) else SPGT_DFT_FOLD(0, 1)
+        }
+#undef SPGT_DFT_FOLD
     }
 #undef SPGT_DFT_FWD
     return check_launch("truncated_dft_rows_forward");
@@ -700,12 +863,15 @@ extern "C" int spgt_spectral_modes_middle(const float* Y, const float* table_h, 
     const int rows_per_wg = ceil_div(r, chunks);
     const size_t lds2 = (size_t)rows_per_wg * m2 * sizeof(float2);
     const dim3 grid2(modes, N, ceil_div(r, rows_per_wg));
-    if (m2 <= 32)
-        hipLaunchKernelGGL(spectral_rows_expand_k<32>, grid2, dim3(256), lds2, stream, O,
-                           reinterpret_cast<const float2*>(table_h_inverse), U, r, Cout, modes, rows_per_wg);
-    else
-        hipLaunchKernelGGL(spectral_rows_expand_k<64>, grid2, dim3(256), lds2, stream, O,
-                           reinterpret_cast<const float2*>(table_h_inverse), U, r, Cout, modes, rows_per_wg);
+#define SPGT_MID_EXPAND(KHMAX, LPR)                                                                                  \
+    hipLaunchKernelGGL((spectral_rows_expand_k<KHMAX, LPR>), grid2, dim3(256), lds2, stream, O,                      \
+                       reinterpret_cast<const float2*>(table_h_inverse), U, r, Cout, modes, rows_per_wg)
+    if (m2 <= 32) {
+        if (Cout <= 32) SPGT_MID_EXPAND(32, 32); else SPGT_MID_EXPAND(32, 64);
+    } else {
+        if (Cout <= 32) SPGT_MID_EXPAND(64, 32); else SPGT_MID_EXPAND(64, 64);
+    }
+#undef SPGT_MID_EXPAND
     return check_launch("spectral_modes_middle");
 }
 
