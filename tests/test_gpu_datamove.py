@@ -602,7 +602,8 @@ def test_bilinear_resample_pre_bias(gpu, src_nhwc, dst_nhwc):
 
 @pytest.mark.parametrize("rows,r,C,m", [(3, 211, 64, 12), (5, 16, 32, 8), (2, 33, 96, 16), (1, 7, 32, 3), (844, 211, 64, 12),
                                         (3, 421, 32, 21), (2, 512, 64, 23), (2, 65, 96, 32), (5, 35, 32, 17),
-                                        (2, 511, 32, 24)])
+                                        (2, 511, 32, 24), (2, 100, 128, 20), (2, 101, 256, 19), (3, 34, 192, 17),
+                                        (2, 40, 128, 20)])
 def test_truncated_dft_rows_against_float64(gpu, rows, r, C, m):
     """Both row kernels against float64 matrix products with the same tables, and the forward one against
     torch.fft.rfft on the CPU (network/sp_layer.py:136-141 keeps columns kw < m of the ortho-normalised rfft2)."""
@@ -658,17 +659,19 @@ def test_spectral_modes_middle_against_float64(gpu, N, r, cin, cout, m):
     assert (got - want).abs().max().item() <= 1e-5 * max(1.0, want.abs().max().item())
 
 
-def test_truncated_dft_rows_planar_layout(gpu):
-    """planar=True is the interleaved result with the mode axis moved ahead of the grid row."""
+@pytest.mark.parametrize("r,C,m", [(33, 64, 8), (70, 128, 20), (45, 64, 18), (35, 32, 17), (64, 256, 32)])
+def test_truncated_dft_rows_planar_layout(gpu, r, C, m):
+    """planar=True is the interleaved result with the mode axis moved ahead of the grid row (also for more than
+    16 modes, where the forward kernel folds the grid row and loads several channels per lane)."""
     from spgt_amd.network.truncated_dft import dft_tables
-    fw, _, _, fwi = dft_tables(33, 8, "cpu")
-    x = rnd(2, 33, 33, 64, seed=91).to(gpu)
-    a = dm.truncated_dft_rows_forward(x.view(66, 33, 64), fw.to(gpu)).view(2, 33, 64, 16)
+    fw, _, _, fwi = dft_tables(r, m, "cpu")
+    x = rnd(2, r, r, C, seed=91).to(gpu)
+    a = dm.truncated_dft_rows_forward(x.view(2 * r, r, C), fw.to(gpu)).view(2, r, C, 2 * m)
     b = dm.truncated_dft_rows_forward(x, fw.to(gpu), planar=True)
     assert torch.equal(b, a.permute(0, 3, 1, 2).contiguous())
-    u = rnd(2, 16, 33, 64, seed=92).to(gpu)
+    u = rnd(2, 2 * m, r, C, seed=92).to(gpu)
     c = dm.truncated_dft_rows_inverse(u, fwi.to(gpu), planar=True)
-    d = dm.truncated_dft_rows_inverse(u.permute(0, 2, 3, 1).contiguous().view(66, 64, 16), fwi.to(gpu)).view(2, 33, 33, 64)
+    d = dm.truncated_dft_rows_inverse(u.permute(0, 2, 3, 1).contiguous().view(2 * r, C, 2 * m), fwi.to(gpu)).view(2, r, r, C)
     assert torch.equal(c, d)
 
 
