@@ -562,10 +562,12 @@ __global__ __launch_bounds__(256) void spectral_rows_expand_k(
 // One wave per SIMD (waves that share a SIMD's matrix pipe run their MFMAs at about half the rate of a lone
 // wave; with four waves per SIMD and a wave per half of the channels this pass took 44 us at [4, 211, 211, 64],
 // with two fatter waves 43-51 us, with one 34 us): a wave makes all channels of a 32-point tile (for C = 64 two
-// independent accumulator chains off the same x and table operands), and walks the (grid row, tile) pairs of the
-// whole input 4 * gridDim.x apart.  Per pair: the parked x rows go to the wave's LDS tile; this pair's U and table entries and the next
-// pair's x rows are requested (wave-uniform base + 32-bit lane offsets, computed once for U); then the 64 MFMAs
-// of the Linear, the MFMAs of the inverse transform, activation and stores.  Stores are unconditional: points
+// independent accumulator chains off the same x and table operands), and takes a run of consecutive (grid row,
+// tile) pairs (the runs of the 4 * gridDim.x waves differ by at most one pair), so that a row's U is fetched once
+// per run and row.  Per pair: the parked x rows go to the wave's LDS tile; U when the row changes, this pair's
+// table entries and the next pair's x rows are requested (wave-uniform base + 32-bit lane offsets, computed once
+// for U); then the 64 MFMAs of the Linear, the MFMAs of the inverse transform, activation and stores.  Stores
+// are unconditional: points
 // past the end of a grid row are computed from the row's last point and that point's table entries, and write
 // its own values to its address.
 // KSU: MFMA steps of the inverse transform, modes rounded up (the table entries of the steps past the modes are
@@ -593,7 +595,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     const int tk = lane & 31;
     const int kh = lane >> 5;
     const unsigned WT = (unsigned)(r + 31) / 32;
-    const unsigned stride = gridDim.x * 4;
 
     float wreg0[KL], wreg1[KL];  // W[c = kh*KL + kk][o = cb*32 + tk], cb = 0, 1
 #pragma unroll
@@ -646,13 +647,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 #define SPGT_STORE_X_PIECE(I_, V_) \
     *reinterpret_cast<float4*>(xw + ((lane + 64 * (I_)) / LPR) * PX + 4 * (lane % LPR)) = V_;
     s4 = s5 = s6 = s7 = s8 = s9 = s10 = s11 = s12 = s13 = s14 = s15 = make_float4(0.f, 0.f, 0.f, 0.f);
-    unsigned t = blockIdx.x * 4 + wave;
-    if (t < pairs) SPGT_LOAD_X_TILE(t)
-    for (; t < pairs; t += stride) {
+    // a wave takes a run of consecutive pairs (runs differ by at most one pair): the tiles of a grid row follow
+    // each other, and the row's U stays in registers until the row changes
+    const unsigned waves = gridDim.x * 4, wi = blockIdx.x * 4 + wave;
+    const unsigned per = pairs / waves, extra = pairs % waves;
+    unsigned t = wi * per + min(wi, extra);
+    const unsigned t_end = t + per + (wi < extra ? 1u : 0u);
+    typedef float vKf __attribute__((ext_vector_type(KSU)));
+    vKf ureg0, ureg1;
+    unsigned u_row = ~0u;
+    if (t < t_end) SPGT_LOAD_X_TILE(t)
+    for (; t < t_end; ++t) {
         const unsigned row = t / WT;
         const int wt = (int)(t - row * WT);
-        const unsigned n = row / (unsigned)r;
-        const unsigned h = row - n * (unsigned)r;
         SPGT_STORE_X_PIECE(0, s0) SPGT_STORE_X_PIECE(1, s1) SPGT_STORE_X_PIECE(2, s2) SPGT_STORE_X_PIECE(3, s3)
         if (NP >= 8) {
             SPGT_STORE_X_PIECE(4, s4) SPGT_STORE_X_PIECE(5, s5) SPGT_STORE_X_PIECE(6, s6) SPGT_STORE_X_PIECE(7, s7)
@@ -661,12 +668,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
             SPGT_STORE_X_PIECE(8, s8) SPGT_STORE_X_PIECE(9, s9) SPGT_STORE_X_PIECE(10, s10) SPGT_STORE_X_PIECE(11, s11)
             SPGT_STORE_X_PIECE(12, s12) SPGT_STORE_X_PIECE(13, s13) SPGT_STORE_X_PIECE(14, s14) SPGT_STORE_X_PIECE(15, s15)
         }
-        const float* ub = U + ((int64_t)n * m2 * r + h) * COUT;  // U[n][0][h][0]
-        float ureg0[KSU], ureg1[KSU];
+        // (the widest shape has no registers to spare for that and fetches U for every pair)
+        constexpr bool KEEP_U = !(KSU == 32 && CIN == 128 && COUT == 64);
+        if (!KEEP_U || row != u_row) {
+            u_row = row;
+            const unsigned n = row / (unsigned)r;
+            const unsigned h = row - n * (unsigned)r;
+            const float* ub = U + ((int64_t)n * m2 * r + h) * COUT;  // U[n][0][h][0]
 #pragma unroll
-        for (int kk = 0; kk < KSU; ++kk) {
-            ureg0[kk] = ub[uoff[kk]];
-            ureg1[kk] = NCB == 2 ? ub[uoff[kk] + (uint32_t)((NCB - 1) * 32)] : 0.f;
+            for (int kk = 0; kk < KSU; ++kk) {
+                ureg0[kk] = ub[uoff[kk]];
+                ureg1[kk] = NCB == 2 ? ub[uoff[kk] + (uint32_t)((NCB - 1) * 32)] : 0.f;
+            }
         }
         // the operand table holds TS steps per tile; points past the row's end take the last point's entries
         const float* tb = tabA + (int64_t)wt * (TS * 64);
@@ -674,7 +687,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         float ta[KSU];
 #pragma unroll
         for (int kk = 0; kk < KSU; ++kk) ta[kk] = tb[tl + (uint32_t)(kk * 64)];
-        SPGT_LOAD_X_TILE(min(t + stride, pairs - 1))  // after the last pair: loaded again, not used
+        SPGT_LOAD_X_TILE(min(t + 1, t_end - 1))  // after the last pair: loaded again, not used
         const float* xr = xw + tk * PX + kh * KL;
         float4 xv[NP];
 #pragma unroll
