@@ -24,10 +24,6 @@
 
 namespace spgt {
 
-#ifndef SPGT_PROJ_TILE
-#define SPGT_PROJ_TILE 32
-#endif
-constexpr int kProjTile = SPGT_PROJ_TILE;  // tokens per tile (64 = two interleaved sub-tiles: 159 us against 150 us at B=8, S=44521)
 // Results are collected per wave in LDS for kProjStage tiles (96 tokens of each of the wave's 32 feature rows) and
 // leave as 384-byte runs per row, two rows per store instruction: rows of [D, S] start at arbitrary 4-byte offsets
 // when S is odd, so every piece of a row touches a partial cache line at either end, and with 128-byte pieces (one
@@ -39,20 +35,27 @@ constexpr int kProjTile = SPGT_PROJ_TILE;  // tokens per tile (64 = two interlea
 constexpr int kProjStage = SPGT_PROJ_STAGE;
 constexpr int kProjStagePitch = 32 * (kProjStage > 0 ? kProjStage : 1) + 4;  // floats per staged row (16-byte rows)
 
-// grid (nchunk, H/4, B), block 256.  KC = dim_hidden / 128.
+// grid (nchunk, H/4, B), block 256; at 128 input features two workgroups share a CU, and one fills its LDS tile
+// and drains its staged rows while the other multiplies (one workgroup per CU with two alternating LDS tiles:
+// 160-176 us against 130-145 us at B=8, S=44521).  KC = dim_hidden / 128.
+// Lane (token tk, half kh) takes k = kh K/2 + j for MFMA j: four consecutive MFMAs' x operands are one 16-byte LDS
+// read, and with rows K + 4 words apart those reads and the 16-byte writes of the incoming tile are free of bank
+// conflicts.  Two accumulator chains alternate over groups of four k-steps, so that no MFMA waits for the one
+// before it.
 template <int KC, int DP, bool LN>
-__global__ __launch_bounds__(256) void projection_rrc_k(
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(KC == 1 ? 2 : 1))) void projection_rrc_k(
     const float* __restrict__ x, const float* __restrict__ W, const float* __restrict__ bias,
     const float* __restrict__ lnw, const float* __restrict__ lnb, const float* __restrict__ pos,
     float* __restrict__ out, float* __restrict__ invsigma, int S, int H, float eps, int tokens_per_chunk) {
     constexpr int K = 128 * KC;
     constexpr int D = DP + 32;
-    constexpr int PITCH = K + 1;
-    constexpr int TT = KC <= 2 ? kProjTile : 32;  // tokens per tile (wide inputs: the staging registers decide)
+    constexpr int PITCH = K + 4;
+    constexpr int TT = 32;  // tokens per tile
+    constexpr int TB = 1;
     extern __shared__ __attribute__((aligned(16))) float xs[];  // [TT][PITCH], then [4 waves][32][kProjStagePitch]
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    constexpr int XS_WORDS = (TT * PITCH + 3) / 4 * 4;
+    constexpr int XS_WORDS = TT * PITCH;
     float* const os = xs + XS_WORDS + wave * (32 * kProjStagePitch);  // this wave's staged rows
     const int h = blockIdx.y * 4 + wave;
     const int b = blockIdx.z;
@@ -61,10 +64,10 @@ __global__ __launch_bounds__(256) void projection_rrc_k(
     const int s_begin = blockIdx.x * tokens_per_chunk;
     const int s_end = min(S, s_begin + tokens_per_chunk);
 
-    // A operand: W[2kk + kh][h*32 + tk]
+    // A operand: W[kh K/2 + kk][h*32 + tk]
     float wreg[K / 2];
 #pragma unroll
-    for (int kk = 0; kk < K / 2; ++kk) wreg[kk] = W[(int64_t)(2 * kk + kh) * K + h * 32 + tk];
+    for (int kk = 0; kk < K / 2; ++kk) wreg[kk] = W[(int64_t)(kh * (K / 2) + kk) * K + h * 32 + tk];
     // accumulator element r holds feature i(r) = 8*(r/4) + 4*kh + r%4
     float breg[16], greg[16], oreg[16];
 #pragma unroll
@@ -98,53 +101,55 @@ __global__ __launch_bounds__(256) void projection_rrc_k(
             const int e = threadIdx.x + 256 * i;
             const int row = e / (K / 4);
             const int c4 = e % (K / 4);
-            float* d = xs + row * PITCH + 4 * c4;
-            d[0] = stage[i].x; d[1] = stage[i].y; d[2] = stage[i].z; d[3] = stage[i].w;
+            *reinterpret_cast<float4*>(xs + row * PITCH + 4 * c4) = stage[i];
         }
     };
 
-    if (s_begin < s_end) load_tile(s_begin);
-    for (int s0 = s_begin; s0 < s_end; s0 += TT) {
-        __syncthreads();  // previous tile fully consumed
+    if (s_begin < s_end) {
+        load_tile(s_begin);
         store_tile();
-        __syncthreads();
-        if (s0 + TT < s_end) load_tile(s0 + TT);
-        // TB = TT / 32 sub-tiles of 32 tokens share the weight operand: TB independent accumulator chains, whose
-        // MFMAs alternate, so that none waits for its predecessor's result
-        constexpr int TB = TT / 32;
+        if (s_begin + TT < s_end) load_tile(s_begin + TT);
+    }
+    __syncthreads();
+    for (int s0 = s_begin; s0 < s_end; s0 += TT) {
         v16f accs[TB];
-#pragma unroll
-        for (int tb = 0; tb < TB; ++tb)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) accs[tb][r] = 0.f;
         {
-            const float* xr = xs + tk * PITCH + kh;
-            // LDS reads for the next batch of MFMAs are issued before the current batch, so their
-            // latency hides behind the matrix pipe
-            constexpr int BK = 16 / TB;
-            constexpr int NB = K / 2 / BK;
-            float xv[2][TB][BK];
+            const float* xr = xs + tk * PITCH + kh * (K / 2);
+            // operands are read from LDS a batch of four groups (sixteen k-steps) ahead of their MFMAs
+            constexpr int NG = K / 8, GB = 4;
+            v16f acc0, acc1;
 #pragma unroll
-            for (int tb = 0; tb < TB; ++tb)
+            for (int r = 0; r < 16; ++r) acc0[r] = acc1[r] = 0.f;
+            float4 xv[2][GB];
 #pragma unroll
-                for (int j = 0; j < BK; ++j) xv[0][tb][j] = xr[tb * 32 * PITCH + 2 * j];
+            for (int g = 0; g < GB; ++g) xv[0][g] = *reinterpret_cast<const float4*>(xr + 4 * g);
 #pragma unroll
-            for (int bt = 0; bt < NB; ++bt) {
-                if (bt + 1 < NB) {
+            for (int g0 = 0; g0 < NG; g0 += GB) {
+                if (g0 + GB < NG) {
 #pragma unroll
-                    for (int tb = 0; tb < TB; ++tb)
-#pragma unroll
-                        for (int j = 0; j < BK; ++j)
-                            xv[(bt + 1) & 1][tb][j] = xr[tb * 32 * PITCH + 2 * ((bt + 1) * BK + j)];
+                    for (int g = 0; g < GB; ++g)
+                        xv[((g0 / GB) + 1) & 1][g] = *reinterpret_cast<const float4*>(xr + 4 * (g0 + GB + g));
                 }
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int j = 0; j < BK; ++j)
-#pragma unroll
-                    for (int tb = 0; tb < TB; ++tb)
-                        accs[tb] = mfma32(wreg[bt * BK + j], xv[bt & 1][tb][j], accs[tb]);
+                for (int g = 0; g < GB; ++g) {
+                    const float4 v = xv[(g0 / GB) & 1][g];
+                    if (g & 1) {
+                        acc1 = mfma32(wreg[4 * (g0 + g) + 0], v.x, acc1);
+                        acc1 = mfma32(wreg[4 * (g0 + g) + 1], v.y, acc1);
+                        acc1 = mfma32(wreg[4 * (g0 + g) + 2], v.z, acc1);
+                        acc1 = mfma32(wreg[4 * (g0 + g) + 3], v.w, acc1);
+                    } else {
+                        acc0 = mfma32(wreg[4 * (g0 + g) + 0], v.x, acc0);
+                        acc0 = mfma32(wreg[4 * (g0 + g) + 1], v.y, acc0);
+                        acc0 = mfma32(wreg[4 * (g0 + g) + 2], v.z, acc0);
+                        acc0 = mfma32(wreg[4 * (g0 + g) + 3], v.w, acc0);
+                    }
+                }
                 __builtin_amdgcn_sched_barrier(0);
             }
+#pragma unroll
+            for (int r = 0; r < 16; ++r) accs[0][r] = acc0[r] + acc1[r];
         }
 #pragma unroll
         for (int tb = 0; tb < TB; ++tb) {
@@ -213,6 +218,12 @@ __global__ __launch_bounds__(256) void projection_rrc_k(
                 if (DP == 2) ob[(int64_t)kh * S + s] = pos[((int64_t)b * S + s) * 2 + kh];
             }
         }
+        __syncthreads();  // the tile has been read by every wave
+        if (s0 + TT < s_end) {
+            store_tile();
+            if (s0 + 2 * TT < s_end) load_tile(s0 + 2 * TT);
+        }
+        __syncthreads();
     }
 }
 
@@ -223,8 +234,8 @@ void launch_projection(const float* x, const float* W, const float* bias, const 
                        const float* pos, float* out, float* invsigma, int B, int S, int H, float eps,
                        hipStream_t stream) {
     constexpr int K = 128 * KC;
-    constexpr int TT = KC <= 2 ? kProjTile : 32;
-    const size_t lds = ((size_t)(TT * (K + 1) + 3) / 4 * 4 + (kProjStage > 0 ? 4 * 32 * kProjStagePitch : 0)) * sizeof(float);
+    constexpr int TT = 32;
+    const size_t lds = ((size_t)TT * (K + 4) + (kProjStage > 0 ? 4 * 32 * kProjStagePitch : 0)) * sizeof(float);
     // about two workgroups per CU; chunks are whole tiles
     const int per_b = std::max(1, 2 * device_cu_count() / std::max(1, B * (H / 4)));
     const int tpc = std::max(TT, ceil_div(ceil_div(S, per_b), TT) * TT);
