@@ -25,7 +25,7 @@ namespace spgt {
 // tab [2*ceil(r/2)][32 MB]: row w holds the m2 table entries of grid point w, zero elsewhere.
 // Y [rows][C][m2], or planar [rows/r][m2][r][C].  CT = C when known at compile time (row offsets
 // become immediates), 0 = any C.  MB = blocks of 32 table columns (m2 <= 32 MB): one accumulator per block,
-// all fed by the same x operand.
+// all fed by the same x operand (the host launches MB = 1; more than 32 columns go to dft_rows_forward_fold_k).
 template <int CT, int MB>
 __global__ __launch_bounds__(256) void dft_rows_forward_k(const float* __restrict__ x, const float* __restrict__ tab,
                                                           float* __restrict__ Y, int64_t rows, int r, int C_, int m2,
