@@ -90,6 +90,11 @@ __global__ __launch_bounds__(256 * NSUB) void ktv_ln_partial_tm(
     float* __restrict__ partial, int S, int H, int64_t ld, int tokens_per_chunk) {
     constexpr int D = DP + 32;
     extern __shared__ __attribute__((aligned(16))) float sub_tiles[];  // NSUB > 1: [NSUB][4 heads][D * D]
+    // DP == 2: the positions of a group of 4*U tokens are 8*U consecutive floats, fetched by one load instruction
+    // per group (a float per lane) and handed to the lanes that need them through this wave-private stage, one
+    // token slot's U positions side by side: a load of its own per unit would be a third more vector memory
+    // instructions than the K and V loads, for 1.5 % more bytes.
+    __shared__ __attribute__((aligned(16))) float pos_stage[DP == 2 ? 4 * NSUB * 8 * U : 4];
     const int lane = threadIdx.x & 63;
     const int wave = (threadIdx.x >> 6) & 3;
     const int sub = threadIdx.x >> 8;
@@ -123,14 +128,17 @@ __global__ __launch_bounds__(256 * NSUB) void ktv_ln_partial_tm(
     float kp[2][2] = {{0.f, 0.f}, {0.f, 0.f}};  // sum yK[ta] * pos[a]
     float pv[2][2] = {{0.f, 0.f}, {0.f, 0.f}};  // sum pos[a] * yV[tb]
     float pp[3] = {0.f, 0.f, 0.f};              // sum p0p0, p0p1, p1p1
+    // The position block is the same for every head: where the heads' tiles meet in LDS (NSUB > 1) only the first
+    // head's waves form it, and the other heads' tiles take it from there when the workgroup writes them out.
+    const bool pp_here = NSUB == 1 || wave == 0;
 
     // `rel` is the token index relative to the chunk start.
-    auto load_unit = [&](const float* kg, const float* vg, const float* pg, uint32_t rel) {
+    auto load_unit = [&](const float* kg, const float* vg, const float* pg, uint32_t rel, bool with_pos) {
         KtvUnit<DP> u;
         const uint32_t off = rel * uld + (uint32_t)f;
         u.k = ld_stream<SPGT_NT_P1LD>(reinterpret_cast<const float2*>(kg + off));
         u.v = ld_stream<SPGT_NT_P1LD>(reinterpret_cast<const float2*>(vg + off));
-        if (DP == 2) u.p = *reinterpret_cast<const float2*>(pg + rel * 2u);
+        if (DP == 2 && with_pos) u.p = *reinterpret_cast<const float2*>(pg + rel * 2u);
         else u.p = make_float2(0.f, 0.f);
         return u;
     };
@@ -156,9 +164,11 @@ __global__ __launch_bounds__(256 * NSUB) void ktv_ln_partial_tm(
             pv[0][1] = fmaf(pz.x, yv.y, pv[0][1]);
             pv[1][0] = fmaf(pz.y, yv.x, pv[1][0]);
             pv[1][1] = fmaf(pz.y, yv.y, pv[1][1]);
-            pp[0] = fmaf(pz.x, pz.x, pp[0]);
-            pp[1] = fmaf(pz.x, pz.y, pp[1]);
-            pp[2] = fmaf(pz.y, pz.y, pp[2]);
+            if (pp_here) {
+                pp[0] = fmaf(pz.x, pz.x, pp[0]);
+                pp[1] = fmaf(pz.x, pz.y, pp[1]);
+                pp[2] = fmaf(pz.y, pz.y, pp[2]);
+            }
         }
     };
 
@@ -170,19 +180,36 @@ __global__ __launch_bounds__(256 * NSUB) void ktv_ln_partial_tm(
     const int len = s1 - s0;
     const int nfull = len / G;
     KtvUnit<DP> bufA[U], bufB[U];
-    auto load_group = [&](KtvUnit<DP>(&buf)[U], int g) {  // g is clamped to the full groups
+    float prawA = 0.f, prawB = 0.f;  // DP == 2: float (lane % (8 U)) of the group's positions
+    static_assert(DP == 0 || 8 * U <= 64, "a group's positions are one float per lane");
+    // where that float goes in the stage: token 4u + ts, component c -> [ts][u][c]
+    const int pl = lane % (8 * U);
+    const int pdst = ((pl >> 1) & 3) * (2 * U) + (pl >> 3) * 2 + (pl & 1);
+    float* const pstage = pos_stage + (sub * 4 + wave) * (8 * U);
+    auto load_group = [&](KtvUnit<DP>(&buf)[U], float& praw, int g) {  // g is clamped to the full groups
         const int64_t go = (int64_t)min(g, nfull - 1) * G;
         const float* kg = kchunk + go * ld;
         const float* vg = vchunk + go * ld;
         const float* pg = pchunk + go * 2;
 #pragma unroll
-        for (int u = 0; u < U; ++u) buf[u] = load_unit(kg, vg, pg, (uint32_t)(4 * u + t));
+        for (int u = 0; u < U; ++u) buf[u] = load_unit(kg, vg, pg, (uint32_t)(4 * u + t), false);
+        if (DP == 2) praw = pg[pl];
     };
     // A full group normalises its 2*U (token, tensor) pairs in lock-step; each
     // value sees the same operations in the same order as in ln_pair.
-    auto compute_full = [&](const KtvUnit<DP>(&buf)[U]) {
+    auto compute_full = [&](const KtvUnit<DP>(&buf)[U], float praw) {
         constexpr int N = 2 * U;
         float x0[N], x1[N], red[N];
+        float pzs[2 * U];  // this lane's token slot: positions of units 0 .. U-1
+        if (DP == 2) {
+            // (the stage is the wave's own: LDS operations of one wave complete in order, no barrier)
+            pstage[pdst] = praw;
+#pragma unroll
+            for (int i = 0; i < 2 * U; i += 4) {
+                const float4 q = *reinterpret_cast<const float4*>(pstage + t * (2 * U) + i);
+                pzs[i] = q.x; pzs[i + 1] = q.y; pzs[i + 2] = q.z; pzs[i + 3] = q.w;
+            }
+        }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             x0[2 * u] = buf[u].k.x;
@@ -216,7 +243,7 @@ __global__ __launch_bounds__(256 * NSUB) void ktv_ln_partial_tm(
             acc[1][0] = mfma16(yk1, yv0, acc[1][0]);
             acc[1][1] = mfma16(yk1, yv1, acc[1][1]);
             if (DP == 2) {
-                const float2 pz = buf[u].p;
+                const float2 pz = make_float2(pzs[2 * u], pzs[2 * u + 1]);
                 kp[0][0] = fmaf(yk0, pz.x, kp[0][0]);
                 kp[0][1] = fmaf(yk0, pz.y, kp[0][1]);
                 kp[1][0] = fmaf(yk1, pz.x, kp[1][0]);
@@ -225,32 +252,37 @@ __global__ __launch_bounds__(256 * NSUB) void ktv_ln_partial_tm(
                 pv[0][1] = fmaf(pz.x, yv1, pv[0][1]);
                 pv[1][0] = fmaf(pz.y, yv0, pv[1][0]);
                 pv[1][1] = fmaf(pz.y, yv1, pv[1][1]);
-                pp[0] = fmaf(pz.x, pz.x, pp[0]);
-                pp[1] = fmaf(pz.x, pz.y, pp[1]);
-                pp[2] = fmaf(pz.y, pz.y, pp[2]);
+            }
+        }
+        if (DP == 2 && pp_here) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                pp[0] = fmaf(pzs[2 * u], pzs[2 * u], pp[0]);
+                pp[1] = fmaf(pzs[2 * u], pzs[2 * u + 1], pp[1]);
+                pp[2] = fmaf(pzs[2 * u + 1], pzs[2 * u + 1], pp[2]);
             }
         }
     };
     if (nfull > 0) {
-        load_group(bufA, 0);
+        load_group(bufA, prawA, 0);
         int g = 0;
         for (; g + 2 <= nfull; g += 2) {
-            load_group(bufB, g + 1);
+            load_group(bufB, prawB, g + 1);
             __builtin_amdgcn_sched_barrier(0);  // keep the prefetch ahead of the arithmetic
-            compute_full(bufA);
+            compute_full(bufA, prawA);
             __builtin_amdgcn_sched_barrier(0);
-            load_group(bufA, g + 2);
+            load_group(bufA, prawA, g + 2);
             __builtin_amdgcn_sched_barrier(0);
-            compute_full(bufB);
+            compute_full(bufB, prawB);
             __builtin_amdgcn_sched_barrier(0);
         }
-        if (g < nfull) compute_full(bufA);
+        if (g < nfull) compute_full(bufA, prawA);
     }
     if (nfull * G < len) {
         const int rel0 = nfull * G + t;
 #pragma unroll
         for (int u = 0; u < U; ++u)
-            bufA[u] = load_unit(kchunk, vchunk, pchunk, (uint32_t)min(rel0 + 4 * u, len - 1));
+            bufA[u] = load_unit(kchunk, vchunk, pchunk, (uint32_t)min(rel0 + 4 * u, len - 1), true);
 #pragma unroll
         for (int u = 0; u < U; ++u) compute_unit(bufA[u], (rel0 + 4 * u) < len);
     }
@@ -314,6 +346,17 @@ __global__ __launch_bounds__(256 * NSUB) void ktv_ln_partial_tm(
             for (int q = 1; q < NSUB; ++q) {
                 const float4 v = *reinterpret_cast<const float4*>(sub_tiles + (q * 4 + hh) * (D * D) + 4 * r4);
                 sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
+            }
+            if (DP == 2 && hh != 0 && (r4 == 0 || r4 == D / 4)) {
+                // the position block M[0..1][0..1] (floats 0, 1, D, D + 1 of the tile) as the first head has it
+                float4 z = *reinterpret_cast<const float4*>(sub_tiles + 4 * r4);
+#pragma unroll
+                for (int q = 1; q < NSUB; ++q) {
+                    const float4 v = *reinterpret_cast<const float4*>(sub_tiles + (q * 4) * (D * D) + 4 * r4);
+                    z.x += v.x; z.y += v.y; z.z += v.z; z.w += v.w;
+                }
+                if (r4 == 0) { sum.x = z.x; sum.y = z.y; }
+                else { sum.z = z.z; sum.w = z.w; }
             }
             float* dst = partial + (((int64_t)b * H + blockIdx.y * 4 + hh) * nchunk + chunk) * (D * D) + 4 * r4;
             st_stream<SPGT_NT_TILE>(reinterpret_cast<float4*>(dst), sum);

@@ -62,7 +62,7 @@ __global__ __launch_bounds__(256 * NSUB) void qtg_partial_tm(const float* __rest
     const float* gb = G + ((int64_t)b * S + s0) * ldg + h * D;
     const float* pb = pos + ((int64_t)b * S + s0) * 2;
 
-    struct Unit { float2 q, g, gp, ps; };
+    struct Unit { float2 q, g; };
     v4f acc[2][2];
 #pragma unroll
     for (int i = 0; i < 2; ++i)
@@ -71,32 +71,36 @@ __global__ __launch_bounds__(256 * NSUB) void qtg_partial_tm(const float* __rest
     float qgp[2][2] = {{0.f, 0.f}, {0.f, 0.f}};  // sum q[ta] * G[position column a]
     float pg[2][2] = {{0.f, 0.f}, {0.f, 0.f}};   // sum pos[a] * G[feature tb]
 
+    // DP == 2: a group of 4*U tokens needs 8*U position floats and 8*U floats of G's position columns.  One load
+    // instruction per group fetches both (lanes 0-31 a position float, lanes 32-63 a float of G) and a
+    // wave-private LDS stage hands each token slot its U pairs of either kind, side by side; loads of their own
+    // per unit would double the vector memory instructions of the pass for 3 % more bytes.
+    static_assert(DP == 0 || 8 * U == 32, "a group's position floats fill half a wave");
+    __shared__ __attribute__((aligned(16))) float pair_stage[DP == 2 ? 4 * NSUB * 16 * U : 4];
+    float* const pstage = pair_stage + (sub * 4 + wave) * (16 * U);
+    const int pkind = lane >> 5;                 // 0: position, 1: G's position columns
+    const int ptok = (lane & 31) >> 1;           // token of the group
+    const int pc = lane & 1;
+    const int pdst = (ptok & 3) * (4 * U) + pkind * (2 * U) + (ptok >> 2) * 2 + pc;  // [slot][kind][unit][c]
+
     auto load_unit = [&](int rel) {
         Unit u;
         u.q = ld_stream<SPGT_BWD_NT_Q>(reinterpret_cast<const float2*>(qb + (int64_t)rel * ld));
-        const float* gr = gb + (int64_t)rel * ldg;
-        u.g = *reinterpret_cast<const float2*>(gr + DP + 2 * p);
-        if (DP == 2) {
-            u.gp = *reinterpret_cast<const float2*>(gr);
-            u.ps = *reinterpret_cast<const float2*>(pb + (int64_t)rel * 2);
-        } else {
-            u.gp = make_float2(0.f, 0.f);
-            u.ps = make_float2(0.f, 0.f);
-        }
+        u.g = *reinterpret_cast<const float2*>(gb + (int64_t)rel * ldg + DP + 2 * p);
         return u;
     };
-    auto compute_unit = [&](const Unit& u, bool valid) {
+    auto compute_unit = [&](const Unit& u, float2 ps, float2 gp, bool valid) {
         const float q0 = valid ? u.q.x : 0.f, q1 = valid ? u.q.y : 0.f;
         acc[0][0] = mfma16(q0, u.g.x, acc[0][0]);
         acc[0][1] = mfma16(q0, u.g.y, acc[0][1]);
         acc[1][0] = mfma16(q1, u.g.x, acc[1][0]);
         acc[1][1] = mfma16(q1, u.g.y, acc[1][1]);
         if (DP == 2) {
-            const float p0 = valid ? u.ps.x : 0.f, p1 = valid ? u.ps.y : 0.f;
-            qgp[0][0] = fmaf(q0, u.gp.x, qgp[0][0]);
-            qgp[0][1] = fmaf(q0, u.gp.y, qgp[0][1]);
-            qgp[1][0] = fmaf(q1, u.gp.x, qgp[1][0]);
-            qgp[1][1] = fmaf(q1, u.gp.y, qgp[1][1]);
+            const float p0 = valid ? ps.x : 0.f, p1 = valid ? ps.y : 0.f;
+            qgp[0][0] = fmaf(q0, gp.x, qgp[0][0]);
+            qgp[0][1] = fmaf(q0, gp.y, qgp[0][1]);
+            qgp[1][0] = fmaf(q1, gp.x, qgp[1][0]);
+            qgp[1][1] = fmaf(q1, gp.y, qgp[1][1]);
             pg[0][0] = fmaf(p0, u.g.x, pg[0][0]);
             pg[0][1] = fmaf(p0, u.g.y, pg[0][1]);
             pg[1][0] = fmaf(p1, u.g.x, pg[1][0]);
@@ -108,26 +112,47 @@ __global__ __launch_bounds__(256 * NSUB) void qtg_partial_tm(const float* __rest
     const int len = s1 - s0;
     const int ngroup = (len + GT - 1) / GT;
     Unit bufA[U], bufB[U];
-    auto load_group = [&](Unit(&buf)[U], int g) {
-        const int base = min(g, ngroup - 1) * GT + t;
+    float prawA = 0.f, prawB = 0.f;
+    auto load_group = [&](Unit(&buf)[U], float& praw, int g) {
+        const int gbase = min(g, ngroup - 1) * GT;
+        const int base = gbase + t;
 #pragma unroll
         for (int u = 0; u < U; ++u) buf[u] = load_unit(min(base + 4 * u, len - 1));
+        if (DP == 2) {
+            const int64_t rel = min(gbase + ptok, len - 1);
+            praw = pkind == 0 ? pb[rel * 2 + pc] : gb[rel * ldg + pc];
+        }
     };
-    auto compute_group = [&](const Unit(&buf)[U], int g) {
+    auto compute_group = [&](const Unit(&buf)[U], float praw, int g) {
         const int base = g * GT + t;
+        float pairs[4 * U];  // this lane's token slot: positions of units 0 .. U-1, then G's position columns
+        if (DP == 2) {
+            // (the stage is the wave's own: LDS operations of one wave complete in order, no barrier)
+            pstage[pdst] = praw;
 #pragma unroll
-        for (int u = 0; u < U; ++u) compute_unit(buf[u], base + 4 * u < len);
+            for (int i = 0; i < 4 * U; i += 4) {
+                const float4 v = *reinterpret_cast<const float4*>(pstage + t * (4 * U) + i);
+                pairs[i] = v.x; pairs[i + 1] = v.y; pairs[i + 2] = v.z; pairs[i + 3] = v.w;
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4 * U; ++i) pairs[i] = 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            compute_unit(buf[u], make_float2(pairs[2 * u], pairs[2 * u + 1]),
+                         make_float2(pairs[2 * U + 2 * u], pairs[2 * U + 2 * u + 1]), base + 4 * u < len);
     };
     if (ngroup > 0) {
-        load_group(bufA, 0);
+        load_group(bufA, prawA, 0);
         for (int g = 0; g < ngroup; g += 2) {
-            load_group(bufB, g + 1);
+            load_group(bufB, prawB, g + 1);
             __builtin_amdgcn_sched_barrier(0);
-            compute_group(bufA, g);
+            compute_group(bufA, prawA, g);
             __builtin_amdgcn_sched_barrier(0);
-            load_group(bufA, g + 2);
+            load_group(bufA, prawA, g + 2);
             __builtin_amdgcn_sched_barrier(0);
-            if (g + 1 < ngroup) compute_group(bufB, g + 1);
+            if (g + 1 < ngroup) compute_group(bufB, prawB, g + 1);
             __builtin_amdgcn_sched_barrier(0);
         }
     }
