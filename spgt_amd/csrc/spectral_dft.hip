@@ -719,10 +719,28 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
             if (ACT == SPGT_ACT_RELU) y[q] = fmaxf(y[q], 0.f);
             if (ACT == SPGT_ACT_SILU) y[q] = y[q] * __builtin_amdgcn_rcpf(1.f + __expf(-y[q]));
         }
-        float* const op = out + ((int64_t)row * r + min(wt * 32 + tk, r - 1)) * COUT + 4 * kh;
+        // Through the wave's LDS tile (its x rows are in registers since before the MFMAs) the results leave as
+        // whole rows: a lane's accumulator holds 16-byte pieces 32 bytes apart in its grid point's row, and stores
+        // of those touch 32 cache lines per instruction; as rows, a store instruction writes 1 KB in one run
+        // (33-34 -> 32 us at [8, 141, 141, 64] and [4, 211, 211, 64], non-temporal form; as plain stores the row
+        // form was slower than the pieces).  Grid points past the row's end hold the last point's values and go to
+        // its address.
+        constexpr int PO = COUT + 4;
+        constexpr int LPO = COUT / 4;  // lanes per output row
 #pragma unroll
         for (int q = 0; q < 4 * NCB; ++q)
-            *reinterpret_cast<float4*>(op + 8 * q) = make_float4(y[4 * q], y[4 * q + 1], y[4 * q + 2], y[4 * q + 3]);
+            *reinterpret_cast<float4*>(xw + tk * PO + 4 * kh + 8 * q) =
+                make_float4(y[4 * q], y[4 * q + 1], y[4 * q + 2], y[4 * q + 3]);
+        float4 rows[4 * NCB];
+#pragma unroll
+        for (int i = 0; i < 4 * NCB; ++i)
+            rows[i] = *reinterpret_cast<const float4*>(xw + ((lane + 64 * i) / LPO) * PO + 4 * (lane % LPO));
+        float* const orow = out + (int64_t)row * r * COUT + 4 * (lane % LPO);
+#pragma unroll
+        for (int i = 0; i < 4 * NCB; ++i) {
+            const int pnt = min(wt * 32 + (lane + 64 * i) / LPO, r - 1);
+            st_stream<true>(reinterpret_cast<float4*>(orow + (uint32_t)(pnt * COUT)), rows[i]);
+        }
     }
 #undef SPGT_LOAD_X_TILE
 #undef SPGT_X_PIECE
