@@ -212,8 +212,9 @@ int check_windows(const char* who, int dim, int H_all, int W_all, int H_low, int
     if (hb1 < 0 || hb2 < 0 || wb1 < 0 || wb2 < 0 || hb1 + H_low > H_all || hb2 + H_low > H_all ||
         wb1 + W_low > W_all || wb2 + W_low > W_all)
         return fail(SPGT_ERR_INVALID_ARGUMENT, "transpose_gather/scatter_dual: a window leaves the [H_all, W_all] plane");
-    if ((size_t)W_low * 65 * 8 * 2 > 64 * 1024)
-        return fail(SPGT_ERR_INVALID_ARGUMENT, "transpose_gather/scatter_dual: W_low above 63 is not supported");
+    // the scatter kernel keeps two windows' rows of 64 planes in LDS (W_low * 65 * 8 bytes each) out of 160 KiB
+    if ((size_t)W_low * 65 * 8 * 2 > 160 * 1024)
+        return fail(SPGT_ERR_INVALID_ARGUMENT, "transpose_gather/scatter_dual: W_low above 157 is not supported");
     if (H_all > 65535 || H_low > 65535)
         return fail(SPGT_ERR_INVALID_ARGUMENT, "transpose_gather/scatter_dual: H_all exceeds 65535");
     (void)who;
@@ -254,7 +255,10 @@ extern "C" int spgt_transpose_gather_dual(const float* src, float* out1, float* 
         return fail(SPGT_ERR_INVALID_ARGUMENT, "transpose_gather_dual: complex operands must be 8-byte aligned");
     Windows win{{H_base_1, H_base_2}, {W_base_1, W_base_2}};
     const dim3 grid(ceil_div(dim, 64), H_low, 2);
-    hipLaunchKernelGGL(transpose_gather_dual_k, grid, dim3(256), (size_t)W_low * 65 * 8, stream,
+    const size_t lds = (size_t)W_low * 65 * 8;
+    if (lds > 64 * 1024 && !allow_dynamic_lds(reinterpret_cast<const void*>(transpose_gather_dual_k), lds))
+        return fail(SPGT_ERR_LAUNCH, "transpose_gather_dual: the kernel was refused its dynamic LDS size");
+    hipLaunchKernelGGL(transpose_gather_dual_k, grid, dim3(256), lds, stream,
                        reinterpret_cast<const uint64_t*>(src), reinterpret_cast<uint64_t*>(out1),
                        reinterpret_cast<uint64_t*>(out2), dim, H_all, W_all, H_low, W_low, win);
     return check_launch("transpose_gather_dual");
@@ -277,7 +281,10 @@ extern "C" int spgt_transpose_scatter_dual(const float* src1, const float* src2,
     const int64_t nB = (int64_t)dim * chunks;
     if (nA + nB >= ((int64_t)1 << 31))
         return fail(SPGT_ERR_INVALID_ARGUMENT, "transpose_scatter_dual: too many planes for one launch");
-    hipLaunchKernelGGL(transpose_scatter_dual_k, dim3((unsigned)(nA + nB)), dim3(256), (size_t)W_low * 65 * 8 * 2, stream,
+    const size_t lds = (size_t)W_low * 65 * 8 * 2;
+    if (lds > 64 * 1024 && !allow_dynamic_lds(reinterpret_cast<const void*>(transpose_scatter_dual_k), lds))
+        return fail(SPGT_ERR_LAUNCH, "transpose_scatter_dual: the kernel was refused its dynamic LDS size");
+    hipLaunchKernelGGL(transpose_scatter_dual_k, dim3((unsigned)(nA + nB)), dim3(256), lds, stream,
                        reinterpret_cast<const uint64_t*>(src1), reinterpret_cast<const uint64_t*>(src2),
                        reinterpret_cast<uint64_t*>(out), dim, H_all, W_all, H_low, W_low, win, spans, (int)nA,
                        std::max(1, chunks));

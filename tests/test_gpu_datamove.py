@@ -53,6 +53,8 @@ GATHER_CASES = [
     ([8, 64], 141, 71, 12, 12, 0, 0, 129, 0),
     ([3, 65], 20, 11, 5, 7, 2, 1, 15, 4),
     ([4, 32], 8, 5, 5, 5, 0, 0, 3, 0),  # overlapping windows
+    ([2, 70], 12, 160, 3, 100, 0, 2, 9, 60),   # wide windows: more than 64 KiB of LDS
+    ([1, 5], 7, 157, 2, 157, 0, 0, 5, 0),      # the widest window
 ]
 
 
